@@ -1,0 +1,192 @@
+// C ABI: library set-up, GGUF block dequantisation, resident matrices and the GEMV entry points.
+#include <cstring>
+#include <vector>
+
+#include "context.h"
+
+using namespace esp;
+
+extern "C" {
+
+int esp_init(void) { return ensure_init(); }
+
+int esp_device_info(char *name, size_t name_capacity, int *compute_units, size_t *hbm_bytes) {
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    const Context &c = context();
+    if (name && name_capacity) {
+        std::strncpy(name, c.props.gcnArchName, name_capacity - 1);
+        name[name_capacity - 1] = 0;
+    }
+    if (compute_units) *compute_units = c.props.multiProcessorCount;
+    if (hbm_bytes) *hbm_bytes = c.props.totalGlobalMem;
+    return ESP_OK;
+}
+
+size_t esp_format_bytes(int format, size_t elements) {
+    if (!format_supported(format) || elements % format_block_elems(format) != 0) return 0;
+    return format_bytes(format, elements);
+}
+
+int esp_dequantize(int format, const void *blocks, size_t elements, float *out) {
+    if (!format_supported(format)) return fail(ESP_ERR_UNSUPPORTED, "dequantize: unknown format %d", format);
+    if (elements % format_block_elems(format) != 0)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "dequantize: %zu elements is not a whole number of blocks", elements);
+    if (elements == 0) return ESP_OK;
+    if (!blocks || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "dequantize: null pointer");
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    const size_t bytes = format_bytes(format, elements);
+    uint8_t *d_blocks = nullptr;
+    float *d_out = nullptr;
+    if ((rc = device_alloc(&d_blocks, bytes)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_out, elements)) != ESP_OK) { (void)hipFree(d_blocks); return rc; }
+    hipError_t e = hipMemcpyAsync(d_blocks, blocks, bytes, hipMemcpyHostToDevice, c.stream);
+    if (e == hipSuccess) e = launch_dequant(format, d_blocks, elements, d_out, c.stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(out, d_out, elements * sizeof(float), hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+    (void)hipFree(d_blocks);
+    (void)hipFree(d_out);
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "dequantize");
+}
+
+ESPMatrix *esp_matrix_create(int format, const void *gguf_blocks, int rows, int cols) {
+    DeviceMatrix m;
+    if (matrix_upload(format, gguf_blocks, rows, cols, &m) != ESP_OK) return nullptr;
+    ESPMatrix *h = new ESPMatrix();
+    h->m = m;
+    return h;
+}
+
+void esp_matrix_free(ESPMatrix *matrix) {
+    if (!matrix) return;
+    matrix_release(&matrix->m);
+    delete matrix;
+}
+
+size_t esp_matrix_bytes(const ESPMatrix *matrix) { return matrix ? matrix->m.bytes() : 0; }
+
+int esp_matrix_dequantize(const ESPMatrix *matrix, float *out) {
+    if (!matrix || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "matrix_dequantize: null pointer");
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    const size_t elems = (size_t)matrix->m.rows * matrix->m.cols;
+    float *d_out = nullptr;
+    if ((rc = device_alloc(&d_out, elems)) != ESP_OK) return rc;
+    hipError_t e = launch_dequant_matrix(matrix->m, d_out, c.stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(out, d_out, elems * sizeof(float), hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+    (void)hipFree(d_out);
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "matrix_dequantize");
+}
+
+int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y, const float *residual) {
+    if (!matrix || !x_f16 || !y) return fail(ESP_ERR_INVALID_ARGUMENT, "gemv: null pointer");
+    if (batch <= 0) return fail(ESP_ERR_INVALID_ARGUMENT, "gemv: batch %d", batch);
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    const DeviceMatrix &m = matrix->m;
+    const size_t nx = (size_t)batch * m.cols, ny = (size_t)batch * m.rows;
+    uint16_t *d_x = nullptr;
+    float *d_y = nullptr, *d_res = nullptr;
+    if ((rc = device_alloc(&d_x, nx)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_y, ny)) != ESP_OK) { (void)hipFree(d_x); return rc; }
+    if (residual && (rc = device_alloc(&d_res, ny)) != ESP_OK) { (void)hipFree(d_x); (void)hipFree(d_y); return rc; }
+    hipError_t e = hipMemcpyAsync(d_x, x_f16, nx * 2, hipMemcpyHostToDevice, c.stream);
+    if (e == hipSuccess && residual) e = hipMemcpyAsync(d_res, residual, ny * 4, hipMemcpyHostToDevice, c.stream);
+    if (e == hipSuccess) {
+        GemvParams p;
+        p.w = m; p.x = d_x; p.y = d_y; p.residual = d_res; p.batch = batch;
+        p.epilogue = residual ? EPI_ADD_RESIDUAL : EPI_STORE_F32;
+        e = launch_gemv(p, c.stream);
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(y, d_y, ny * 4, hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+    (void)hipFree(d_x); (void)hipFree(d_y);
+    if (d_res) (void)hipFree(d_res);
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "gemv");
+}
+
+int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int rotate,
+                  double *mean_us, double *best_us) {
+    if (!matrix || batch <= 0 || iters <= 0 || warmup < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "gemv_time: bad argument");
+    if (rotate < 1) rotate = 1;
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    const DeviceMatrix &m = matrix->m;
+    const size_t nx = (size_t)batch * m.cols, ny = (size_t)batch * m.rows;
+    const size_t qs_bytes = (size_t)m.rows * m.qs_row_bytes, sc_count = m.scales ? (size_t)m.rows * (m.cols / 32) : 0;
+
+    std::vector<DeviceMatrix> copies(rotate, m);
+    uint16_t *d_x = nullptr;
+    float *d_y = nullptr;
+    std::vector<hipEvent_t> marks;
+    hipError_t e = hipSuccess;
+    rc = ESP_OK;
+    for (int i = 1; i < rotate && rc == ESP_OK; i++) {
+        copies[i].qs = nullptr; copies[i].scales = nullptr;
+        rc = device_alloc(&copies[i].qs, qs_bytes);
+        if (rc == ESP_OK && sc_count) rc = device_alloc(&copies[i].scales, sc_count);
+        if (rc == ESP_OK) e = hipMemcpyAsync(copies[i].qs, m.qs, qs_bytes, hipMemcpyDeviceToDevice, c.stream);
+        if (rc == ESP_OK && e == hipSuccess && sc_count)
+            e = hipMemcpyAsync(copies[i].scales, m.scales, sc_count * 2, hipMemcpyDeviceToDevice, c.stream);
+        if (e != hipSuccess) rc = fail_hip(e, "gemv_time copy");
+    }
+    if (rc == ESP_OK) rc = device_alloc(&d_x, nx);
+    if (rc == ESP_OK) rc = device_alloc(&d_y, ny);
+    if (rc == ESP_OK) {
+        // activations ~ small deterministic values; the kernel's timing does not depend on them
+        std::vector<uint16_t> hx(nx);
+        for (size_t i = 0; i < nx; i++) hx[i] = (uint16_t)(0x3000u + (i * 37u) % 0x0C00u);
+        e = hipMemcpyAsync(d_x, hx.data(), nx * 2, hipMemcpyHostToDevice, c.stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+        if (e != hipSuccess) rc = fail_hip(e, "gemv_time upload");
+    }
+    if (rc == ESP_OK) {
+        GemvParams p;
+        p.x = d_x; p.y = d_y; p.batch = batch; p.epilogue = EPI_STORE_F32;
+        for (int i = 0; i < warmup && e == hipSuccess; i++) { p.w = copies[i % rotate]; e = launch_gemv(p, c.stream); }
+        // mean: `iters` launches queued back to back between two events
+        marks.resize(iters + 3, nullptr);
+        for (auto &ev : marks) if (e == hipSuccess) e = hipEventCreate(&ev);
+        hipEvent_t t0 = marks[iters + 1], t1 = marks[iters + 2];
+        if (e == hipSuccess) e = hipEventRecord(t0, c.stream);
+        for (int i = 0; i < iters && e == hipSuccess; i++) {
+            p.w = copies[(warmup + i) % rotate];
+            e = launch_gemv(p, c.stream);
+        }
+        if (e == hipSuccess) e = hipEventRecord(t1, c.stream);
+        // best: every launch bracketed by its own events
+        if (e == hipSuccess) e = hipEventRecord(marks[0], c.stream);
+        for (int i = 0; i < iters && e == hipSuccess; i++) {
+            p.w = copies[(warmup + i) % rotate];
+            e = launch_gemv(p, c.stream);
+            if (e == hipSuccess) e = hipEventRecord(marks[i + 1], c.stream);
+        }
+        if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+        if (e == hipSuccess) {
+            float total_ms = 0.0f;
+            e = hipEventElapsedTime(&total_ms, t0, t1);
+            double best = 1e30;
+            for (int i = 0; i < iters && e == hipSuccess; i++) {
+                float ms = 0.0f;
+                e = hipEventElapsedTime(&ms, marks[i], marks[i + 1]);
+                if (ms * 1e3 < best) best = ms * 1e3;
+            }
+            if (mean_us) *mean_us = (double)total_ms * 1e3 / iters;
+            if (best_us) *best_us = best;
+        }
+        if (e != hipSuccess) rc = fail_hip(e, "gemv_time");
+    }
+    for (auto ev : marks) if (ev) (void)hipEventDestroy(ev);
+    for (int i = 1; i < rotate; i++) { if (copies[i].qs) (void)hipFree(copies[i].qs); if (copies[i].scales) (void)hipFree(copies[i].scales); }
+    if (d_x) (void)hipFree(d_x);
+    if (d_y) (void)hipFree(d_y);
+    return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,74 @@
+// Shared declarations for the HIP side of the library (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace esp {
+
+// GGUF tensor type ids (public ggml numbering) for the formats this library runs.
+enum Format : int { FMT_F32 = 0, FMT_F16 = 1, FMT_Q4_0 = 2, FMT_Q8_0 = 8, FMT_Q4_K = 12 };
+
+inline bool format_supported(int f) {
+    return f == FMT_F32 || f == FMT_F16 || f == FMT_Q4_0 || f == FMT_Q8_0 || f == FMT_Q4_K;
+}
+// elements per quantisation block and bytes per block in the GGUF file layout
+inline int format_block_elems(int f) { return f == FMT_Q4_K ? 256 : (f == FMT_Q8_0 || f == FMT_Q4_0) ? 32 : 1; }
+inline int format_block_bytes(int f) {
+    switch (f) {
+    case FMT_F32: return 4;
+    case FMT_F16: return 2;
+    case FMT_Q4_0: return 18;
+    case FMT_Q8_0: return 34;
+    case FMT_Q4_K: return 144;
+    default: return 0;
+    }
+}
+inline size_t format_bytes(int f, size_t elems) { return elems / format_block_elems(f) * format_block_bytes(f); }
+
+// A weight matrix resident in HBM, laid out for the GEMV kernels.
+//   Q4_K : `qs` holds the GGUF 144-byte super-blocks unchanged, row-major (16-byte aligned rows).
+//   Q8_0 : split planes — `qs` = int8 quants [rows][cols], `scales` = fp16 d [rows][cols/32].
+//   Q4_0 : split planes — `qs` = packed nibbles [rows][cols/2] (16 bytes per block, GGUF nibble
+//          order), `scales` = fp16 d [rows][cols/32].
+//   F16  : `qs` = fp16 values [rows][cols].
+// The split planes carry exactly the bits of the GGUF blocks (34 / 18 bytes per 32 weights); they
+// exist because 34- and 18-byte blocks cannot be read with aligned 128-bit loads.
+struct DeviceMatrix {
+    int format = 0;
+    int rows = 0, cols = 0;
+    uint8_t *qs = nullptr;
+    uint16_t *scales = nullptr;
+    size_t qs_row_bytes = 0;
+    size_t bytes() const {  // algorithmic bytes: what one GEMV must read
+        return (size_t)rows * qs_row_bytes + (scales ? (size_t)rows * (cols / 32) * 2 : 0);
+    }
+};
+
+// GEMV epilogues (what happens to the fp32 row sums)
+enum Epilogue : int {
+    EPI_STORE_F32 = 0,     // y[b][r] = acc
+    EPI_ADD_RESIDUAL = 1,  // y[b][r] = residual[b][r] + acc
+};
+
+struct GemvParams {
+    DeviceMatrix w;
+    const uint16_t *x = nullptr;  // fp16 activations [batch][cols]
+    float *y = nullptr;           // fp32 out [batch][rows]
+    const float *residual = nullptr;
+    int batch = 1;
+    int epilogue = EPI_STORE_F32;
+};
+
+// kernels/gemv.hip
+hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
+// kernels/dequant.hip — GGUF-layout blocks -> fp32, bit-exact to the block definitions
+hipError_t launch_dequant(int format, const uint8_t *blocks, size_t elems, float *out, hipStream_t stream);
+// GGUF-layout blocks -> DeviceMatrix planes (device to device)
+hipError_t launch_repack(int format, const uint8_t *blocks, int rows, int cols, const DeviceMatrix &dst,
+                         hipStream_t stream);
+// DeviceMatrix -> fp32 [rows][cols] (used to check the planes carry the same bits)
+hipError_t launch_dequant_matrix(const DeviceMatrix &m, float *out, hipStream_t stream);
+
+}  // namespace esp

@@ -1,0 +1,169 @@
+// GGUF block dequantisation to fp32 and the upload-time re-layout of Q8_0 / Q4_0 into planes.
+//
+// Stands in for the absent Edgerunner package's DequantDispatcher.dequantize(tensor:device:)
+// (call sites: Sources/EspressoGGUF/GGUFModelLoader.swift:359-372).  Results are bit-exact to the
+// public ggml block definitions: every product is rounded to fp32 before the next operation
+// (__fmul_rn / __fsub_rn are never contracted into a fused multiply-add).
+#include "../common.h"
+
+namespace esp {
+namespace {
+
+__device__ __forceinline__ float half_at(const uint8_t *p) {
+    uint16_t bits = (uint16_t)(p[0] | (p[1] << 8));
+    return (float)__builtin_bit_cast(_Float16, bits);
+}
+
+// one thread per element, blocks addressed in the GGUF byte layout
+__global__ void dequant_q8_0_kernel(const uint8_t *blocks, size_t elems, float *out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= elems) return;
+    const uint8_t *blk = blocks + (i >> 5) * 34;
+    float d = half_at(blk);
+    int q = (int8_t)blk[2 + (i & 31)];
+    out[i] = __fmul_rn((float)q, d);
+}
+
+__global__ void dequant_q4_0_kernel(const uint8_t *blocks, size_t elems, float *out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= elems) return;
+    const uint8_t *blk = blocks + (i >> 5) * 18;
+    float d = half_at(blk);
+    int j = (int)(i & 31);
+    uint8_t byte = blk[2 + (j & 15)];
+    int n = j < 16 ? (byte & 0x0F) : (byte >> 4);
+    out[i] = __fmul_rn((float)(n - 8), d);
+}
+
+__device__ __forceinline__ void q4k_scale_min(int j, const uint8_t *s, int &sc, int &m) {
+    if (j < 4) {
+        sc = s[j] & 63;
+        m = s[j + 4] & 63;
+    } else {
+        sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4);
+        m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+    }
+}
+
+__global__ void dequant_q4_k_kernel(const uint8_t *blocks, size_t elems, float *out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= elems) return;
+    const uint8_t *blk = blocks + (i >> 8) * 144;
+    int e = (int)(i & 255);
+    int sub = e >> 5, l = e & 31, chunk = sub >> 1;
+    float d = half_at(blk), dmin = half_at(blk + 2);
+    int sc, m;
+    q4k_scale_min(sub, blk + 4, sc, m);
+    uint8_t byte = blk[16 + chunk * 32 + l];
+    int n = (sub & 1) ? (byte >> 4) : (byte & 0x0F);
+    float d1 = __fmul_rn(d, (float)sc);
+    float m1 = __fmul_rn(dmin, (float)m);
+    out[i] = __fsub_rn(__fmul_rn(d1, (float)n), m1);
+}
+
+__global__ void dequant_f16_kernel(const uint8_t *blocks, size_t elems, float *out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= elems) return;
+    out[i] = half_at(blocks + 2 * i);
+}
+
+__global__ void copy_f32_kernel(const uint8_t *blocks, size_t elems, float *out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= elems) return;
+    out[i] = reinterpret_cast<const float *>(blocks)[i];
+}
+
+// GGUF 34-byte Q8_0 / 18-byte Q4_0 blocks -> (quant plane, scale plane).  One thread per block.
+__global__ void repack_q8_0_kernel(const uint8_t *blocks, size_t nblocks, uint8_t *qs, uint16_t *scales) {
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const uint8_t *blk = blocks + b * 34;
+    scales[b] = (uint16_t)(blk[0] | (blk[1] << 8));
+    for (int j = 0; j < 32; j++) qs[b * 32 + j] = blk[2 + j];
+}
+
+__global__ void repack_q4_0_kernel(const uint8_t *blocks, size_t nblocks, uint8_t *qs, uint16_t *scales) {
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const uint8_t *blk = blocks + b * 18;
+    scales[b] = (uint16_t)(blk[0] | (blk[1] << 8));
+    for (int j = 0; j < 16; j++) qs[b * 16 + j] = blk[2 + j];
+}
+
+// plane layouts -> fp32, same arithmetic as the block kernels
+__global__ void dequant_planes_q8_0_kernel(const uint8_t *qs, const uint16_t *scales, size_t elems, float *out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= elems) return;
+    float d = (float)__builtin_bit_cast(_Float16, scales[i >> 5]);
+    out[i] = __fmul_rn((float)(int8_t)qs[i], d);
+}
+
+__global__ void dequant_planes_q4_0_kernel(const uint8_t *qs, const uint16_t *scales, size_t elems, float *out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= elems) return;
+    float d = (float)__builtin_bit_cast(_Float16, scales[i >> 5]);
+    int j = (int)(i & 31);
+    uint8_t byte = qs[(i >> 5) * 16 + (j & 15)];
+    int n = j < 16 ? (byte & 0x0F) : (byte >> 4);
+    out[i] = __fmul_rn((float)(n - 8), d);
+}
+
+inline dim3 grid_for(size_t n, int threads) { return dim3((unsigned)((n + threads - 1) / threads)); }
+
+}  // namespace
+
+hipError_t launch_dequant(int format, const uint8_t *blocks, size_t elems, float *out, hipStream_t stream) {
+    if (!blocks || !out) return hipErrorInvalidValue;
+    if (elems == 0) return hipSuccess;
+    if (elems % format_block_elems(format) != 0) return hipErrorInvalidValue;
+    const int t = 256;
+    switch (format) {
+    case FMT_Q8_0: hipLaunchKernelGGL(dequant_q8_0_kernel, grid_for(elems, t), dim3(t), 0, stream, blocks, elems, out); break;
+    case FMT_Q4_0: hipLaunchKernelGGL(dequant_q4_0_kernel, grid_for(elems, t), dim3(t), 0, stream, blocks, elems, out); break;
+    case FMT_Q4_K: hipLaunchKernelGGL(dequant_q4_k_kernel, grid_for(elems, t), dim3(t), 0, stream, blocks, elems, out); break;
+    case FMT_F16: hipLaunchKernelGGL(dequant_f16_kernel, grid_for(elems, t), dim3(t), 0, stream, blocks, elems, out); break;
+    case FMT_F32: hipLaunchKernelGGL(copy_f32_kernel, grid_for(elems, t), dim3(t), 0, stream, blocks, elems, out); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_repack(int format, const uint8_t *blocks, int rows, int cols, const DeviceMatrix &dst,
+                         hipStream_t stream) {
+    if (!blocks || !dst.qs || rows <= 0 || cols <= 0) return hipErrorInvalidValue;
+    const size_t elems = (size_t)rows * cols;
+    const int t = 256;
+    switch (format) {
+    case FMT_Q8_0:
+        hipLaunchKernelGGL(repack_q8_0_kernel, grid_for(elems / 32, t), dim3(t), 0, stream, blocks, elems / 32, dst.qs, dst.scales);
+        break;
+    case FMT_Q4_0:
+        hipLaunchKernelGGL(repack_q4_0_kernel, grid_for(elems / 32, t), dim3(t), 0, stream, blocks, elems / 32, dst.qs, dst.scales);
+        break;
+    case FMT_Q4_K:
+    case FMT_F16:
+    case FMT_F32: {
+        hipError_t e = hipMemcpyAsync(dst.qs, blocks, format_bytes(format, elems), hipMemcpyDeviceToDevice, stream);
+        if (e != hipSuccess) return e;
+        break;
+    }
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dequant_matrix(const DeviceMatrix &m, float *out, hipStream_t stream) {
+    const size_t elems = (size_t)m.rows * m.cols;
+    const int t = 256;
+    switch (m.format) {
+    case FMT_Q8_0:
+        hipLaunchKernelGGL(dequant_planes_q8_0_kernel, grid_for(elems, t), dim3(t), 0, stream, m.qs, m.scales, elems, out);
+        return hipGetLastError();
+    case FMT_Q4_0:
+        hipLaunchKernelGGL(dequant_planes_q4_0_kernel, grid_for(elems, t), dim3(t), 0, stream, m.qs, m.scales, elems, out);
+        return hipGetLastError();
+    default: return launch_dequant(m.format, m.qs, elems, out, stream);
+    }
+}
+
+}  // namespace esp

@@ -1,0 +1,86 @@
+"""numpy-facing wrappers over the C ABI's GGUF-block and GEMV entry points."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def init() -> None:
+    _lib.check(_lib.load_library().esp_init())
+
+
+def device_info() -> dict:
+    L = _lib.load_library()
+    name = C.create_string_buffer(128)
+    cus, hbm = C.c_int(0), C.c_size_t(0)
+    _lib.check(L.esp_device_info(name, 128, C.byref(cus), C.byref(hbm)))
+    return {"name": name.value.decode(), "compute_units": cus.value, "hbm_bytes": hbm.value}
+
+
+def format_bytes(fmt: int, elements: int) -> int:
+    return int(_lib.load_library().esp_format_bytes(fmt, elements))
+
+
+def dequantize(fmt: int, blocks: np.ndarray, elements: int) -> np.ndarray:
+    """DequantDispatcher.dequantize: GGUF-layout blocks -> fp32 (decoded on the GPU)."""
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    out = np.empty(elements, dtype=np.float32)
+    _lib.check(_lib.load_library().esp_dequantize(fmt, _ptr(blocks), elements, _ptr(out)))
+    return out
+
+
+class Matrix:
+    """A [rows, cols] weight resident in HBM in the GEMV kernels' layout."""
+
+    def __init__(self, fmt: int, blocks: np.ndarray, rows: int, cols: int):
+        L = _lib.load_library()
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        expected = L.esp_format_bytes(fmt, rows * cols)
+        if expected == 0 or blocks.size != expected:
+            raise ValueError(f"{blocks.size} bytes given, format {fmt} needs {expected} for {rows}x{cols}")
+        self._h = L.esp_matrix_create(fmt, _ptr(blocks), rows, cols)
+        if not self._h:
+            raise _lib.EspressoError(-1, _lib.last_error())
+        self.format, self.rows, self.cols = fmt, rows, cols
+
+    def close(self) -> None:
+        if self._h:
+            _lib.load_library().esp_matrix_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def bytes(self) -> int:
+        return int(_lib.load_library().esp_matrix_bytes(self._h))
+
+    def dequantize(self) -> np.ndarray:
+        out = np.empty(self.rows * self.cols, dtype=np.float32)
+        _lib.check(_lib.load_library().esp_matrix_dequantize(self._h, _ptr(out)))
+        return out.reshape(self.rows, self.cols)
+
+    def gemv(self, x_f16: np.ndarray, residual: np.ndarray | None = None) -> np.ndarray:
+        x = np.ascontiguousarray(x_f16, dtype=np.float16).reshape(-1, self.cols)
+        batch = x.shape[0]
+        y = np.empty((batch, self.rows), dtype=np.float32)
+        res = None
+        if residual is not None:
+            res = np.ascontiguousarray(residual, dtype=np.float32).reshape(batch, self.rows)
+        _lib.check(_lib.load_library().esp_gemv(self._h, _ptr(x), batch, _ptr(y), _ptr(res) if res is not None else None))
+        return y
+
+    def time_gemv(self, batch: int = 1, warmup: int = 10, iters: int = 50, rotate: int = 1) -> dict:
+        mean, best = C.c_double(0), C.c_double(0)
+        _lib.check(_lib.load_library().esp_gemv_time(self._h, batch, warmup, iters, rotate, C.byref(mean), C.byref(best)))
+        return {"mean_us": mean.value, "best_us": best.value}
