@@ -34,6 +34,7 @@ def load_library() -> C.CDLL:
         _build.build()
     lib = C.CDLL(path)
     _declare(lib)
+    _declare_llama(lib)
     _LIB = lib
     return lib
 
@@ -69,3 +70,53 @@ def _declare(L: C.CDLL) -> None:
     L.esp_gemv.argtypes = [vp, vp, i32, vp, vp]
     L.esp_gemv_time.restype = i32
     L.esp_gemv_time.argtypes = [vp, i32, i32, i32, i32, dp, dp]
+
+
+class LlamaConfigStruct(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layer", "n_head", "n_kv_head", "d_model", "head_dim", "hidden_dim", "vocab", "max_seq")] + \
+               [("norm_eps", C.c_float), ("rope_theta", C.c_float), ("eos_token", C.c_int32), ("kv_format", C.c_int32),
+                ("max_sequences", C.c_int32)]
+
+
+class GenerationStatsStruct(C.Structure):
+    _fields_ = [("generated", C.c_int32), ("prefill_ms", C.c_double), ("decode_ms", C.c_double),
+                ("first_token_latency_ms", C.c_double), ("tokens_per_second", C.c_double)]
+
+
+class TwoTokenStatsStruct(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("passes", "committed_total", "accepted_total", "reference_passes",
+                                         "reference_committed_total", "reference_accepted_total")]
+
+
+def _declare_llama(L: C.CDLL) -> None:
+    vp, sz, i32 = C.c_void_p, C.c_size_t, C.c_int
+    L.esp_llama_create.restype = vp
+    L.esp_llama_create.argtypes = [C.POINTER(LlamaConfigStruct)]
+    L.esp_llama_free.argtypes = [vp]
+    L.esp_llama_set_weight.restype = i32
+    L.esp_llama_set_weight.argtypes = [vp, i32, i32, i32, vp, sz]
+    L.esp_llama_finalize.restype = i32
+    L.esp_llama_finalize.argtypes = [vp]
+    L.esp_llama_weight_bytes.restype = sz
+    L.esp_llama_weight_bytes.argtypes = [vp]
+    L.esp_llama_reset.restype = i32
+    L.esp_llama_reset.argtypes = [vp]
+    L.esp_llama_prefill.restype = i32
+    L.esp_llama_prefill.argtypes = [vp, i32, vp, i32]
+    L.esp_llama_advance.restype = i32
+    L.esp_llama_advance.argtypes = [vp, i32, C.c_uint32]
+    L.esp_llama_select_greedy_token.restype = i32
+    L.esp_llama_select_greedy_token.argtypes = [vp, i32, C.POINTER(C.c_uint32)]
+    L.esp_llama_visible_token_count.restype = i32
+    L.esp_llama_visible_token_count.argtypes = [vp, i32]
+    L.esp_llama_set_visible_token_count.restype = i32
+    L.esp_llama_set_visible_token_count.argtypes = [vp, i32, i32]
+    L.esp_llama_read_last_hidden.restype = i32
+    L.esp_llama_read_last_hidden.argtypes = [vp, i32, vp]
+    L.esp_llama_read_logits.restype = i32
+    L.esp_llama_read_logits.argtypes = [vp, i32, vp]
+    L.esp_llama_generate.restype = i32
+    L.esp_llama_generate.argtypes = [vp, vp, i32, i32, vp, C.POINTER(i32), C.POINTER(GenerationStatsStruct), vp]
+    L.esp_llama_generate_two_token.restype = i32
+    L.esp_llama_generate_two_token.argtypes = [vp, vp, vp, i32, i32, i32, vp, C.POINTER(i32),
+                                               C.POINTER(GenerationStatsStruct), C.POINTER(TwoTokenStatsStruct)]

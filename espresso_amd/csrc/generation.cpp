@@ -1,0 +1,148 @@
+#include "generation.h"
+
+#include <chrono>
+
+namespace esp {
+namespace {
+using Clock = std::chrono::steady_clock;
+double ms_since(Clock::time_point t0) { return std::chrono::duration<double, std::milli>(Clock::now() - t0).count(); }
+}  // namespace
+
+int generate_greedy(LlamaRuntime &rt, const uint32_t *prompt, int prompt_count, int max_tokens,
+                    std::vector<uint32_t> *out, GenerationTiming *timing) {
+    out->clear();
+    const LlamaConfig &c = rt.config();
+    if (prompt_count <= 0 || !prompt) return fail(ESP_ERR_INVALID_ARGUMENT, "Prompt tokens must not be empty");       // (:6200-6202)
+    if (max_tokens < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "maxTokens must be >= 0");                               // (:1411-1413)
+    if (prompt_count >= c.max_seq) return fail(ESP_ERR_OUT_OF_RANGE, "prompt of %d tokens does not fit context %d", prompt_count, c.max_seq);
+    const int eff = max_tokens < c.max_seq - prompt_count ? max_tokens : c.max_seq - prompt_count;
+    auto t_prefill = Clock::now();
+    int rc = rt.prefill(0, prompt, prompt_count);
+    if (rc != ESP_OK) return rc;
+    if (timing) timing->prefill_ms = ms_since(t_prefill);
+
+    auto t_start = Clock::now(), t_emit = t_start;
+    int all = prompt_count;
+    while ((int)out->size() < eff) {
+        uint32_t next = 0;
+        if ((rc = rt.select_greedy(0, &next)) != ESP_OK) return rc;
+        auto now = Clock::now();
+        if (timing) {
+            if (out->empty()) timing->first_token_latency_ms = std::chrono::duration<double, std::milli>(now - t_start).count();
+            timing->token_latencies_ms.push_back(std::chrono::duration<double, std::milli>(now - t_emit).count());
+        }
+        out->push_back(next);
+        if (c.eos_token >= 0 && next == (uint32_t)c.eos_token) break;   // EOS is appended, then the loop ends (:6385-6388)
+        all++;
+        if ((int)out->size() >= eff || all >= c.max_seq) break;         // (:6407)
+        if ((rc = rt.advance(0, next)) != ESP_OK) return rc;            // position all - 1 (:6411)
+        t_emit = now;
+    }
+    if (timing) timing->decode_ms = ms_since(t_start);
+    return ESP_OK;
+}
+
+int generate_two_token(LlamaRuntime &full, LlamaRuntime &draft, const uint32_t *prompt, int prompt_count,
+                       int max_tokens, bool reference_accounting, std::vector<uint32_t> *out,
+                       TwoTokenStats *stats, GenerationTiming *timing) {
+    out->clear();
+    TwoTokenStats st;
+    const LlamaConfig &c = full.config();
+    if (prompt_count <= 0 || !prompt) return fail(ESP_ERR_INVALID_ARGUMENT, "Prompt tokens must not be empty");   // (:6021-6023)
+    if (max_tokens < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "maxTokens must be >= 0");
+    if (draft.config().vocab != c.vocab)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "draft vocab %d does not match target vocab %d", draft.config().vocab, c.vocab);  // (:5375-5379)
+    if (prompt_count >= c.max_seq || prompt_count >= draft.config().max_seq)
+        return fail(ESP_ERR_OUT_OF_RANGE, "prompt of %d tokens does not fit the context", prompt_count);
+    const int max_seq = c.max_seq < draft.config().max_seq ? c.max_seq : draft.config().max_seq;
+    const int eff = max_tokens < max_seq - prompt_count ? max_tokens : max_seq - prompt_count;
+    const int eos = c.eos_token;
+
+    auto t_prefill = Clock::now();
+    int rc;
+    if ((rc = full.prefill(0, prompt, prompt_count)) != ESP_OK) return rc;
+    if ((rc = draft.prefill(0, prompt, prompt_count)) != ESP_OK) return rc;
+    if (timing) timing->prefill_ms = ms_since(t_prefill);
+    auto t_start = Clock::now(), t_emit = t_start;
+    auto emit = [&](uint32_t tok) {
+        auto now = Clock::now();
+        if (timing) {
+            if (out->empty()) timing->first_token_latency_ms = std::chrono::duration<double, std::milli>(now - t_start).count();
+            timing->token_latencies_ms.push_back(std::chrono::duration<double, std::milli>(now - t_emit).count());
+        }
+        t_emit = now;
+        out->push_back(tok);
+    };
+    auto finish = [&]() {
+        const int after_first = (int)out->size() - 1;
+        if (after_first > 0) {
+            st.reference_passes = (after_first + 1) / 2;
+            st.reference_committed_total = after_first;
+        }
+        if (!reference_accounting) st.reference_accepted_total = -1;
+        if (stats) *stats = st;
+        if (timing) timing->decode_ms = ms_since(t_start);
+        return ESP_OK;
+    };
+    if (eff <= 0) return finish();
+
+    // the first token comes from the prefilled state (:6069-6087)
+    uint32_t current = 0;
+    if ((rc = full.select_greedy(0, &current)) != ESP_OK) return rc;
+    emit(current);
+    int all = prompt_count + 1;
+    if ((eos >= 0 && current == (uint32_t)eos) || (int)out->size() >= eff || all >= max_seq) return finish();
+
+    // Invariant: `current` is the last emitted token; neither model has consumed it yet.
+    while ((int)out->size() < eff && all < max_seq) {
+        st.passes++;
+        uint32_t proposed = 0;
+        if ((rc = draft.advance(0, current)) != ESP_OK) return rc;
+        if ((rc = draft.select_greedy(0, &proposed)) != ESP_OK) return rc;
+
+        const int pos = full.visible(0);                       // == all - 1
+        const bool can_two = eff - (int)out->size() >= 2 && all + 1 < max_seq;
+        StepRows rows{};
+        rows.count = can_two ? 2 : 1;
+        rows.token[0] = (int)current; rows.pos[0] = pos; rows.seq[0] = 0;
+        rows.token[1] = (int)proposed; rows.pos[1] = pos + 1; rows.seq[1] = 0;
+        uint32_t exact[2] = {0, 0};
+        if ((rc = full.forward_rows(rows)) != ESP_OK) return rc;
+        if ((rc = full.head_rows(rows.count, exact)) != ESP_OK) return rc;
+
+        // row 0 is always exact: keep its KV column and emit the token that follows it
+        full.set_visible(0, pos + 1);
+        emit(exact[0]);
+        all++;
+        st.committed_total++;
+        if (reference_accounting && proposed == exact[0]) st.reference_accepted_total++;
+        const bool accepted = can_two && proposed == exact[0];
+        if ((eos >= 0 && exact[0] == (uint32_t)eos) || (int)out->size() >= eff || all >= max_seq) {
+            if ((rc = full.keep_row(0, 0)) != ESP_OK) return rc;
+            break;
+        }
+        if (!accepted) {
+            if ((rc = full.keep_row(0, 0)) != ESP_OK) return rc;
+            current = exact[0];
+            continue;
+        }
+        // the proposal was right: row 1 ran on the exact token, so its column and its successor stand
+        st.accepted_total++;
+        st.committed_total++;
+        full.set_visible(0, pos + 2);
+        if ((rc = full.keep_row(1, 0)) != ESP_OK) return rc;
+        if ((rc = draft.advance(0, proposed)) != ESP_OK) return rc;
+        if (reference_accounting) {
+            uint32_t p1 = 0;
+            if ((rc = draft.select_greedy(0, &p1)) != ESP_OK) return rc;
+            if (p1 == exact[1]) st.reference_accepted_total++;
+        }
+        emit(exact[1]);
+        all++;
+        current = exact[1];
+        if (eos >= 0 && exact[1] == (uint32_t)eos) break;
+    }
+    return finish();
+}
+
+}  // namespace esp

@@ -1,0 +1,56 @@
+// Argument blocks and launchers of the per-token kernels (kernels/decode_ops.hip).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace esp {
+
+constexpr int kMaxStepRows = 16;
+
+// The rows (tokens) of one step, passed by value so that no host-to-device copy is needed.
+struct StepRows {
+    int count;
+    int token[kMaxStepRows];
+    int pos[kMaxStepRows];
+    int seq[kMaxStepRows];
+};
+
+struct QkvPostArgs {
+    const float *qkv;      // [rows][attnDim + 2 kvDim] in the fused matrix's row order
+    const float *q_norm;   // [head_dim] or null
+    const float *k_norm;   // [head_dim] or null
+    float norm_eps;
+    int n_head, n_kv_head, head_dim, max_seq;
+    const float *rope_cos;  // [max_seq][head_dim/2]
+    const float *rope_sin;
+    const int *pos;         // [rows]
+    const int *seq;         // [rows]
+    float *q_out;           // [rows][attnDim]
+    void *k_cache;          // this layer: [seq][kvDim][max_seq]
+    void *v_cache;          // this layer: [seq][max_seq][kvDim]
+    size_t cache_seq_stride;  // elements per sequence (kvDim * max_seq)
+};
+
+struct AttentionArgs {
+    const float *q;         // [rows][attnDim]
+    const void *k_cache;
+    const void *v_cache;
+    size_t cache_seq_stride;
+    int n_head, n_kv_head, head_dim, max_seq;
+    const int *pos;
+    const int *seq;
+    uint16_t *ctx_f16;      // [rows][attnDim]
+};
+
+hipError_t launch_embed(const void *table, bool table_is_f16, const int *tokens, int rows, int d, float *hidden, hipStream_t s);
+hipError_t launch_rmsnorm(const float *x, const float *w, float eps, int rows, int d, uint16_t *out_f16,
+                          unsigned long long *argmax_cells, hipStream_t s);
+hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStream_t s);
+hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
+hipError_t launch_swiglu(const float *gu, int rows, int hidden, uint16_t *act_f16, hipStream_t s);
+hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_token, float *out_value, hipStream_t s);
+hipError_t launch_set_rows(const StepRows &rows, int *tokens, int *pos, int *seq, hipStream_t s);
+hipError_t launch_copy_rows(const float *src, float *dst, int rows, int d, hipStream_t s);
+
+}  // namespace esp

@@ -1,0 +1,403 @@
+#include "llama_runtime.h"
+
+#include <cmath>
+#include <cstring>
+
+namespace esp {
+namespace {
+
+// fp16 bits -> float on the host (weights arrive as raw bytes)
+float half_to_float_host(uint16_t h) {
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu, mant = h & 0x3FFu, f;
+    if (exp == 0) {
+        if (mant == 0) f = sign;
+        else {
+            int e = -1;
+            do { mant <<= 1; e++; } while ((mant & 0x400u) == 0);
+            f = sign | ((uint32_t)(127 - 15 - e) << 23) | ((mant & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) f = sign | 0x7F800000u | (mant << 13);
+    else f = sign | ((exp + 112u) << 23) | (mant << 13);
+    float out;
+    std::memcpy(&out, &f, 4);
+    return out;
+}
+
+template <typename T>
+void free_device(T *&p) {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+}
+
+}  // namespace
+
+int LlamaRuntime::create(const LlamaConfig &c, LlamaRuntime **out) {
+    *out = nullptr;
+    // validateRuntimeConfig (RealModelInferenceEngine.swift:7615-7634)
+    if (c.n_layer <= 0 || c.n_head <= 0 || c.n_kv_head <= 0 || c.d_model <= 0 || c.head_dim <= 0 ||
+        c.hidden_dim <= 0 || c.vocab <= 0 || c.max_seq <= 0)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "llama config: every dimension must be positive");
+    if (c.n_head % c.n_kv_head != 0)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "llama config: nHead %d is not a multiple of nKVHead %d", c.n_head, c.n_kv_head);
+    if (c.head_dim % 2 != 0) return fail(ESP_ERR_INVALID_ARGUMENT, "llama config: headDim %d must be even", c.head_dim);
+    if (c.kv_format != FMT_F32 && c.kv_format != FMT_F16)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "llama config: KV cache format must be f32 or f16");
+    if (c.max_sequences < 1 || c.max_sequences > kMaxStepRows)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "llama config: max_sequences must be 1..%d", kMaxStepRows);
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    LlamaRuntime *rt = new LlamaRuntime();
+    rt->c_ = c;
+    rt->h_layers_.resize(c.n_layer);
+    rt->visible_.assign(c.max_sequences, 0);
+    *out = rt;
+    return ESP_OK;
+}
+
+LlamaRuntime::~LlamaRuntime() {
+    free_device(embedding_);
+    free_device(final_norm_);
+    matrix_release(&lm_head_);
+    for (Layer &L : layers_) {
+        free_device(L.rms_att); free_device(L.rms_ffn); free_device(L.q_norm); free_device(L.k_norm);
+        matrix_release(&L.wqkv); matrix_release(&L.wo); matrix_release(&L.w13); matrix_release(&L.w2);
+        free_device(L.k_cache); free_device(L.v_cache);
+    }
+    free_device(rope_cos_); free_device(rope_sin_);
+    free_device(hidden_); free_device(qkv_); free_device(q_); free_device(gu_); free_device(logits_);
+    free_device(last_hidden_); free_device(xn_); free_device(ctx_); free_device(act_);
+    free_device(d_tokens_); free_device(d_pos_); free_device(d_seq_); free_device(d_out_tokens_);
+}
+
+LlamaRuntime::HostTensor *LlamaRuntime::host_slot(int layer, int slot) {
+    switch (slot) {
+    case SLOT_TOKEN_EMBEDDING: return &h_embedding_;
+    case SLOT_FINAL_NORM: return &h_final_norm_;
+    case SLOT_LM_HEAD: return &h_lm_head_;
+    default: break;
+    }
+    if (layer < 0 || layer >= c_.n_layer) return nullptr;
+    HostLayer &L = h_layers_[layer];
+    switch (slot) {
+    case SLOT_RMS_ATT: return &L.rms_att;
+    case SLOT_WQ: return &L.wq;
+    case SLOT_WK: return &L.wk;
+    case SLOT_WV: return &L.wv;
+    case SLOT_WO: return &L.wo;
+    case SLOT_RMS_FFN: return &L.rms_ffn;
+    case SLOT_W1: return &L.w1;
+    case SLOT_W2: return &L.w2;
+    case SLOT_W3: return &L.w3;
+    case SLOT_Q_NORM: return &L.q_norm;
+    case SLOT_K_NORM: return &L.k_norm;
+    default: return nullptr;
+    }
+}
+
+int LlamaRuntime::set_weight(int layer, int slot, int format, const void *data, size_t bytes) {
+    if (finalized_) return fail(ESP_ERR_INVALID_ARGUMENT, "set_weight after finalize");
+    HostTensor *t = host_slot(layer, slot);
+    if (!t) return fail(ESP_ERR_INVALID_ARGUMENT, "set_weight: no slot %d in layer %d", slot, layer);
+    if (!data || !format_supported(format)) return fail(ESP_ERR_INVALID_ARGUMENT, "set_weight: null data or unknown format %d", format);
+    const size_t d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
+    size_t elems = 0;
+    switch (slot) {
+    case SLOT_TOKEN_EMBEDDING: case SLOT_LM_HEAD: elems = (size_t)c_.vocab * d; break;
+    case SLOT_FINAL_NORM: case SLOT_RMS_ATT: case SLOT_RMS_FFN: elems = d; break;
+    case SLOT_WQ: case SLOT_WO: elems = ad * d; break;
+    case SLOT_WK: case SLOT_WV: elems = kd * d; break;
+    case SLOT_W1: case SLOT_W2: case SLOT_W3: elems = hd * d; break;
+    case SLOT_Q_NORM: case SLOT_K_NORM: elems = (size_t)c_.head_dim; break;
+    }
+    const bool is_vector = slot == SLOT_FINAL_NORM || slot == SLOT_RMS_ATT || slot == SLOT_RMS_FFN ||
+                           slot == SLOT_Q_NORM || slot == SLOT_K_NORM || slot == SLOT_TOKEN_EMBEDDING;
+    if (is_vector && format != FMT_F32 && format != FMT_F16)
+        return fail(ESP_ERR_UNSUPPORTED, "set_weight: slot %d takes f32 or f16 values", slot);
+    if (elems % format_block_elems(format) != 0 || bytes != format_bytes(format, elems))
+        return fail(ESP_ERR_INVALID_ARGUMENT, "set_weight: slot %d expects %zu elements (%zu bytes in format %d), got %zu bytes",
+                    slot, elems, format_bytes(format, elems), format, bytes);
+    t->format = format;
+    t->bytes.assign(static_cast<const uint8_t *>(data), static_cast<const uint8_t *>(data) + bytes);
+    return ESP_OK;
+}
+
+int LlamaRuntime::upload_vector(const HostTensor &t, size_t count, float **out, const char *what) {
+    if (t.format < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "finalize: missing weight %s", what);
+    std::vector<float> v(count);
+    if (t.format == FMT_F32) std::memcpy(v.data(), t.bytes.data(), count * 4);
+    else for (size_t i = 0; i < count; i++) v[i] = half_to_float_host((uint16_t)(t.bytes[2 * i] | (t.bytes[2 * i + 1] << 8)));
+    int rc = device_alloc(out, count);
+    if (rc != ESP_OK) return rc;
+    ESP_HIP_TRY(hipMemcpy(*out, v.data(), count * 4, hipMemcpyHostToDevice));
+    return ESP_OK;
+}
+
+int LlamaRuntime::finalize() {
+    if (finalized_) return ESP_OK;
+    const int d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim, half = c_.head_dim / 2;
+    int rc;
+    // ---- top level ----
+    if (h_embedding_.format < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "finalize: missing token embedding");
+    embedding_f16_ = h_embedding_.format == FMT_F16;
+    {
+        uint8_t *p = nullptr;
+        if ((rc = device_alloc(&p, h_embedding_.bytes.size())) != ESP_OK) return rc;
+        embedding_ = p;
+        ESP_HIP_TRY(hipMemcpy(embedding_, h_embedding_.bytes.data(), h_embedding_.bytes.size(), hipMemcpyHostToDevice));
+    }
+    if ((rc = upload_vector(h_final_norm_, d, &final_norm_, "rms_final")) != ESP_OK) return rc;
+    if (h_lm_head_.format < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "finalize: missing lm_head");
+    if ((rc = matrix_upload(h_lm_head_.format, h_lm_head_.bytes.data(), c_.vocab, d, &lm_head_)) != ESP_OK) return rc;
+    weight_bytes_ = lm_head_.bytes();
+
+    // ---- layers ----
+    layers_.resize(c_.n_layer);
+    const size_t cache_elems = (size_t)c_.max_sequences * kd * c_.max_seq;
+    const size_t cache_bytes = cache_elems * (c_.kv_format == FMT_F16 ? 2 : 4);
+    std::vector<uint8_t> fused;
+    for (int l = 0; l < c_.n_layer; l++) {
+        HostLayer &H = h_layers_[l];
+        Layer &L = layers_[l];
+        const HostTensor *need[] = {&H.wq, &H.wk, &H.wv, &H.wo, &H.w1, &H.w2, &H.w3};
+        for (const HostTensor *t : need)
+            if (t->format < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "finalize: layer %d is missing a projection weight", l);
+        if (H.wq.format != H.wk.format || H.wq.format != H.wv.format)
+            return fail(ESP_ERR_UNSUPPORTED, "finalize: layer %d wq/wk/wv must share one format", l);
+        if (H.w1.format != H.w3.format) return fail(ESP_ERR_UNSUPPORTED, "finalize: layer %d w1/w3 must share one format", l);
+        if ((rc = upload_vector(H.rms_att, d, &L.rms_att, "rms_att")) != ESP_OK) return rc;
+        if ((rc = upload_vector(H.rms_ffn, d, &L.rms_ffn, "rms_ffn")) != ESP_OK) return rc;
+        // q_norm/k_norm are optional and only used when both exist (:6585-6607)
+        if (H.q_norm.format >= 0 && H.k_norm.format >= 0) {
+            if ((rc = upload_vector(H.q_norm, c_.head_dim, &L.q_norm, "q_norm")) != ESP_OK) return rc;
+            if ((rc = upload_vector(H.k_norm, c_.head_dim, &L.k_norm, "k_norm")) != ESP_OK) return rc;
+        }
+        // fused QKV: q and k rows reordered so that the two rows of a RoPE pair (j, j + half) are
+        // adjacent; v rows in natural order.
+        {
+            const size_t rb = format_bytes(H.wq.format, d);
+            fused.resize((size_t)(ad + 2 * kd) * rb);
+            size_t o = 0;
+            auto put_rope_rows = [&](const HostTensor &t, int heads) {
+                for (int h = 0; h < heads; h++)
+                    for (int j = 0; j < half; j++) {
+                        std::memcpy(&fused[o], &t.bytes[(size_t)(h * c_.head_dim + j) * rb], rb); o += rb;
+                        std::memcpy(&fused[o], &t.bytes[(size_t)(h * c_.head_dim + j + half) * rb], rb); o += rb;
+                    }
+            };
+            put_rope_rows(H.wq, c_.n_head);
+            put_rope_rows(H.wk, c_.n_kv_head);
+            std::memcpy(&fused[o], H.wv.bytes.data(), (size_t)kd * rb);
+            if ((rc = matrix_upload(H.wq.format, fused.data(), ad + 2 * kd, d, &L.wqkv)) != ESP_OK) return rc;
+        }
+        // fused gate/up: rows interleaved (g0, u0, g1, u1, ...)
+        {
+            const size_t rb = format_bytes(H.w1.format, d);
+            fused.resize((size_t)2 * hd * rb);
+            for (int i = 0; i < hd; i++) {
+                std::memcpy(&fused[(size_t)(2 * i) * rb], &H.w1.bytes[(size_t)i * rb], rb);
+                std::memcpy(&fused[(size_t)(2 * i + 1) * rb], &H.w3.bytes[(size_t)i * rb], rb);
+            }
+            if ((rc = matrix_upload(H.w1.format, fused.data(), 2 * hd, d, &L.w13)) != ESP_OK) return rc;
+        }
+        if ((rc = matrix_upload(H.wo.format, H.wo.bytes.data(), d, ad, &L.wo)) != ESP_OK) return rc;
+        if ((rc = matrix_upload(H.w2.format, H.w2.bytes.data(), d, hd, &L.w2)) != ESP_OK) return rc;
+        weight_bytes_ += L.wqkv.bytes() + L.wo.bytes() + L.w13.bytes() + L.w2.bytes();
+        uint8_t *kc = nullptr, *vc = nullptr;
+        if ((rc = device_alloc(&kc, cache_bytes)) != ESP_OK) return rc;
+        L.k_cache = kc;
+        if ((rc = device_alloc(&vc, cache_bytes)) != ESP_OK) return rc;
+        L.v_cache = vc;
+        H = HostLayer{};  // drop the host copy
+    }
+    h_embedding_ = HostTensor{}; h_lm_head_ = HostTensor{};
+    fused.clear(); fused.shrink_to_fit();
+
+    // ---- RoPE table, computed on the host with the reference's float expressions (:6759-6762) ----
+    {
+        std::vector<float> cs((size_t)c_.max_seq * half), sn((size_t)c_.max_seq * half);
+        for (int p = 0; p < c_.max_seq; p++)
+            for (int j = 0; j < half; j++) {
+                const float frequency = 1.0f / powf(c_.rope_theta, (float)(2 * j) / (float)c_.head_dim);
+                const float angle = (float)p * frequency;
+                cs[(size_t)p * half + j] = cosf(angle);
+                sn[(size_t)p * half + j] = sinf(angle);
+            }
+        if ((rc = device_alloc(&rope_cos_, cs.size())) != ESP_OK) return rc;
+        if ((rc = device_alloc(&rope_sin_, sn.size())) != ESP_OK) return rc;
+        ESP_HIP_TRY(hipMemcpy(rope_cos_, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
+        ESP_HIP_TRY(hipMemcpy(rope_sin_, sn.data(), sn.size() * 4, hipMemcpyHostToDevice));
+    }
+    // ---- activations ----
+    const size_t R = kMaxStepRows;
+    if ((rc = device_alloc(&hidden_, R * d)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&qkv_, R * (ad + 2 * kd))) != ESP_OK) return rc;
+    if ((rc = device_alloc(&q_, R * ad)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&gu_, R * 2 * hd)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&logits_, R * c_.vocab)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&last_hidden_, (size_t)c_.max_sequences * d)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&xn_, R * (size_t)(d > hd ? d : hd))) != ESP_OK) return rc;
+    if ((rc = device_alloc(&ctx_, R * ad)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&act_, R * hd)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_tokens_, R)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_pos_, R)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_seq_, R)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_out_tokens_, R)) != ESP_OK) return rc;
+    finalized_ = true;
+    return reset();
+}
+
+int LlamaRuntime::reset() {
+    if (!finalized_) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+    Context &ctx = context();
+    const size_t cache_bytes = (size_t)c_.max_sequences * c_.kv_dim() * c_.max_seq * (c_.kv_format == FMT_F16 ? 2 : 4);
+    for (Layer &L : layers_) {
+        ESP_HIP_TRY(hipMemsetAsync(L.k_cache, 0, cache_bytes, ctx.stream));
+        ESP_HIP_TRY(hipMemsetAsync(L.v_cache, 0, cache_bytes, ctx.stream));
+    }
+    ESP_HIP_TRY(hipMemsetAsync(last_hidden_, 0, (size_t)c_.max_sequences * c_.d_model * 4, ctx.stream));
+    ESP_HIP_TRY(hipStreamSynchronize(ctx.stream));
+    std::fill(visible_.begin(), visible_.end(), 0);
+    return ESP_OK;
+}
+
+int LlamaRuntime::visible(int seq) const {
+    return seq >= 0 && seq < c_.max_sequences ? visible_[seq] : -1;
+}
+
+int LlamaRuntime::set_visible(int seq, int count) {
+    if (seq < 0 || seq >= c_.max_sequences || count < 0 || count > c_.max_seq)
+        return fail(ESP_ERR_OUT_OF_RANGE, "set_visible(seq %d, count %d) out of range", seq, count);
+    visible_[seq] = count;
+    return ESP_OK;
+}
+
+int LlamaRuntime::forward_rows(const StepRows &rows) {
+    if (!finalized_) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+    if (rows.count < 1 || rows.count > kMaxStepRows) return fail(ESP_ERR_INVALID_ARGUMENT, "forward_rows: %d rows", rows.count);
+    for (int i = 0; i < rows.count; i++) {
+        if (rows.token[i] < 0 || rows.token[i] >= c_.vocab)
+            return fail(ESP_ERR_OUT_OF_RANGE, "token %d is outside vocab %d", rows.token[i], c_.vocab);   // (:687-689)
+        if (rows.pos[i] < 0 || rows.pos[i] >= c_.max_seq)
+            return fail(ESP_ERR_OUT_OF_RANGE, "position %d exceeds context %d", rows.pos[i], c_.max_seq);  // (:673-677)
+        if (rows.seq[i] < 0 || rows.seq[i] >= c_.max_sequences)
+            return fail(ESP_ERR_OUT_OF_RANGE, "sequence %d of %d", rows.seq[i], c_.max_sequences);
+    }
+    hipStream_t s = context().stream;
+    const int M = rows.count, d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
+    const bool kv16 = c_.kv_format == FMT_F16;
+    ESP_HIP_TRY(launch_set_rows(rows, d_tokens_, d_pos_, d_seq_, s));
+    ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, M, d, hidden_, s));
+    for (Layer &L : layers_) {
+        ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_att, c_.norm_eps, M, d, xn_, nullptr, s));
+        GemvParams g;
+        g.w = L.wqkv; g.x = xn_; g.y = qkv_; g.batch = M; g.epilogue = EPI_STORE_F32;
+        ESP_HIP_TRY(launch_gemv(g, s));
+        QkvPostArgs qa{};
+        qa.qkv = qkv_; qa.q_norm = L.q_norm; qa.k_norm = L.k_norm; qa.norm_eps = c_.norm_eps;
+        qa.n_head = c_.n_head; qa.n_kv_head = c_.n_kv_head; qa.head_dim = c_.head_dim; qa.max_seq = c_.max_seq;
+        qa.rope_cos = rope_cos_; qa.rope_sin = rope_sin_; qa.pos = d_pos_; qa.seq = d_seq_;
+        qa.q_out = q_; qa.k_cache = L.k_cache; qa.v_cache = L.v_cache; qa.cache_seq_stride = (size_t)kd * c_.max_seq;
+        ESP_HIP_TRY(launch_qkv_post(qa, M, kv16, s));
+        AttentionArgs aa{};
+        aa.q = q_; aa.k_cache = L.k_cache; aa.v_cache = L.v_cache; aa.cache_seq_stride = qa.cache_seq_stride;
+        aa.n_head = c_.n_head; aa.n_kv_head = c_.n_kv_head; aa.head_dim = c_.head_dim; aa.max_seq = c_.max_seq;
+        aa.pos = d_pos_; aa.seq = d_seq_; aa.ctx_f16 = ctx_;
+        ESP_HIP_TRY(launch_attention(aa, M, kv16, s));
+        g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
+        ESP_HIP_TRY(launch_gemv(g, s));
+        ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_ffn, c_.norm_eps, M, d, xn_, nullptr, s));
+        g.w = L.w13; g.x = xn_; g.y = gu_; g.residual = nullptr; g.epilogue = EPI_STORE_F32;
+        ESP_HIP_TRY(launch_gemv(g, s));
+        ESP_HIP_TRY(launch_swiglu(gu_, M, hd, act_, s));
+        g.w = L.w2; g.x = act_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
+        ESP_HIP_TRY(launch_gemv(g, s));
+    }
+    (void)ad;
+    return ESP_OK;
+}
+
+int LlamaRuntime::keep_row(int row, int seq) {
+    if (row < 0 || row >= kMaxStepRows || seq < 0 || seq >= c_.max_sequences)
+        return fail(ESP_ERR_OUT_OF_RANGE, "keep_row(%d, %d)", row, seq);
+    ESP_HIP_TRY(launch_copy_rows(hidden_ + (size_t)row * c_.d_model, last_hidden_ + (size_t)seq * c_.d_model, 1, c_.d_model,
+                                 context().stream));
+    return ESP_OK;
+}
+
+int LlamaRuntime::advance(int seq, uint32_t token) {
+    if (seq < 0 || seq >= c_.max_sequences) return fail(ESP_ERR_OUT_OF_RANGE, "sequence %d of %d", seq, c_.max_sequences);
+    if (visible_[seq] >= c_.max_seq)
+        return fail(ESP_ERR_OUT_OF_RANGE, "runtime position %d exceeds context %d", visible_[seq], c_.max_seq);
+    if (token >= (uint32_t)c_.vocab) return fail(ESP_ERR_OUT_OF_RANGE, "token %u is outside vocab %d", token, c_.vocab);
+    StepRows rows{};
+    rows.count = 1; rows.token[0] = (int)token; rows.pos[0] = visible_[seq]; rows.seq[0] = seq;
+    int rc = forward_rows(rows);
+    if (rc != ESP_OK) return rc;
+    if ((rc = keep_row(0, seq)) != ESP_OK) return rc;
+    visible_[seq] += 1;
+    return ESP_OK;
+}
+
+int LlamaRuntime::prefill(int seq, const uint32_t *tokens, int count) {
+    if (count <= 0 || !tokens) return fail(ESP_ERR_INVALID_ARGUMENT, "Prompt tokens must not be empty");
+    if (seq < 0 || seq >= c_.max_sequences) return fail(ESP_ERR_OUT_OF_RANGE, "sequence %d of %d", seq, c_.max_sequences);
+    visible_[seq] = 0;
+    for (int i = 0; i < count; i++) {
+        int rc = advance(seq, tokens[i]);
+        if (rc != ESP_OK) return rc;
+    }
+    return ESP_OK;
+}
+
+int LlamaRuntime::run_head(const float *hidden_rows, int count) {
+    hipStream_t s = context().stream;
+    ESP_HIP_TRY(launch_rmsnorm(hidden_rows, final_norm_, c_.norm_eps, count, c_.d_model, xn_, nullptr, s));
+    GemvParams g;
+    g.w = lm_head_; g.x = xn_; g.y = logits_; g.batch = count; g.epilogue = EPI_STORE_F32;
+    ESP_HIP_TRY(launch_gemv(g, s));
+    ESP_HIP_TRY(launch_argmax(logits_, count, c_.vocab, d_out_tokens_, nullptr, s));
+    return ESP_OK;
+}
+
+int LlamaRuntime::select_greedy(int seq, uint32_t *token) {
+    if (!finalized_) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+    if (seq < 0 || seq >= c_.max_sequences || !token) return fail(ESP_ERR_OUT_OF_RANGE, "select_greedy(seq %d)", seq);
+    int rc = run_head(last_hidden_ + (size_t)seq * c_.d_model, 1);
+    if (rc != ESP_OK) return rc;
+    int t = 0;
+    ESP_HIP_TRY(hipMemcpyAsync(&t, d_out_tokens_, sizeof(int), hipMemcpyDeviceToHost, context().stream));
+    ESP_HIP_TRY(hipStreamSynchronize(context().stream));
+    *token = (uint32_t)t;
+    return ESP_OK;
+}
+
+int LlamaRuntime::head_rows(int count, uint32_t *tokens) {
+    if (!finalized_) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+    if (count < 1 || count > kMaxStepRows || !tokens) return fail(ESP_ERR_INVALID_ARGUMENT, "head_rows(%d)", count);
+    int rc = run_head(hidden_, count);
+    if (rc != ESP_OK) return rc;
+    int t[kMaxStepRows];
+    ESP_HIP_TRY(hipMemcpyAsync(t, d_out_tokens_, sizeof(int) * count, hipMemcpyDeviceToHost, context().stream));
+    ESP_HIP_TRY(hipStreamSynchronize(context().stream));
+    for (int i = 0; i < count; i++) tokens[i] = (uint32_t)t[i];
+    return ESP_OK;
+}
+
+int LlamaRuntime::read_last_hidden(int seq, float *out) {
+    if (!finalized_ || seq < 0 || seq >= c_.max_sequences || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "read_last_hidden");
+    ESP_HIP_TRY(hipMemcpyAsync(out, last_hidden_ + (size_t)seq * c_.d_model, (size_t)c_.d_model * 4, hipMemcpyDeviceToHost,
+                               context().stream));
+    ESP_HIP_TRY(hipStreamSynchronize(context().stream));
+    return ESP_OK;
+}
+
+int LlamaRuntime::read_logits(int seq, float *out) {
+    if (!finalized_ || seq < 0 || seq >= c_.max_sequences || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "read_logits");
+    int rc = run_head(last_hidden_ + (size_t)seq * c_.d_model, 1);
+    if (rc != ESP_OK) return rc;
+    ESP_HIP_TRY(hipMemcpyAsync(out, logits_, (size_t)c_.vocab * 4, hipMemcpyDeviceToHost, context().stream));
+    ESP_HIP_TRY(hipStreamSynchronize(context().stream));
+    return ESP_OK;
+}
+
+}  // namespace esp

@@ -1,0 +1,100 @@
+// Device-resident llama decoder state: the MI355X counterpart of the reference's
+// CPUExactLlamaRuntime (Sources/RealModelInference/RealModelInferenceEngine.swift:548-850).
+#pragma once
+
+#include <string>
+#include <vector>
+
+#include "context.h"
+#include "kernels/decode_ops.h"
+
+namespace esp {
+
+// weight slots; names follow LayerWeightPaths (Sources/ModelSupport/LayerWeightPaths.swift:22-84)
+enum WeightSlot : int {
+    SLOT_TOKEN_EMBEDDING = 0, SLOT_FINAL_NORM = 1, SLOT_LM_HEAD = 2,
+    SLOT_RMS_ATT = 10, SLOT_WQ = 11, SLOT_WK = 12, SLOT_WV = 13, SLOT_WO = 14,
+    SLOT_RMS_FFN = 15, SLOT_W1 = 16, SLOT_W2 = 17, SLOT_W3 = 18, SLOT_Q_NORM = 19, SLOT_K_NORM = 20,
+};
+
+struct LlamaConfig {
+    int n_layer = 0, n_head = 0, n_kv_head = 0, d_model = 0, head_dim = 0, hidden_dim = 0, vocab = 0, max_seq = 0;
+    float norm_eps = 1e-5f, rope_theta = 10000.0f;
+    int eos_token = -1;
+    int kv_format = FMT_F32;  // FMT_F32 or FMT_F16
+    int max_sequences = 1;    // independent KV caches
+    int attention_dim() const { return n_head * head_dim; }
+    int kv_dim() const { return n_kv_head * head_dim; }
+};
+
+class LlamaRuntime {
+  public:
+    static int create(const LlamaConfig &config, LlamaRuntime **out);
+    ~LlamaRuntime();
+
+    const LlamaConfig &config() const { return c_; }
+    bool finalized() const { return finalized_; }
+
+    // Copies the bytes.  Matrices: GGUF block layout, row-major [rows, cols]; norms: f32 or f16 vectors;
+    // embedding: f32 or f16 table.
+    int set_weight(int layer, int slot, int format, const void *data, size_t bytes);
+    // Fuses wq|wk|wv and w1|w3, uploads everything, builds the RoPE table.
+    int finalize();
+
+    int reset();                                  // all sequences (:616-635)
+    int visible(int seq) const;
+    int set_visible(int seq, int count);          // rollback = lower the visible length
+    // Runs the trunk over `rows` (token, position, sequence); positions are written into the KV caches.
+    // Does not change the visible counts.
+    int forward_rows(const StepRows &rows);
+    // forward one token at the sequence's visible position and keep its hidden state (:672-680)
+    int advance(int seq, uint32_t token);
+    int prefill(int seq, const uint32_t *tokens, int count);   // (:637-645)
+    // Final norm + LM head + first-max argmax of kept hidden states (:663-670, :825-849).
+    int select_greedy(int seq, uint32_t *token);
+    // Head over rows of the most recent forward_rows(); tokens[i] for row i.
+    int head_rows(int count, uint32_t *tokens);
+    // Keep row `row` of the most recent forward_rows() as sequence `seq`'s last hidden state.
+    int keep_row(int row, int seq);
+    int read_last_hidden(int seq, float *out);
+    int read_logits(int seq, float *out);         // runs the head on the kept hidden state
+
+    size_t weight_bytes_per_token() const { return weight_bytes_; }
+
+  private:
+    LlamaRuntime() = default;
+    struct HostTensor { int format = -1; std::vector<uint8_t> bytes; };
+    struct HostLayer { HostTensor rms_att, wq, wk, wv, wo, rms_ffn, w1, w2, w3, q_norm, k_norm; };
+    struct Layer {
+        float *rms_att = nullptr, *rms_ffn = nullptr, *q_norm = nullptr, *k_norm = nullptr;
+        DeviceMatrix wqkv, wo, w13, w2;
+        void *k_cache = nullptr, *v_cache = nullptr;
+    };
+    int upload_vector(const HostTensor &t, size_t count, float **out, const char *what);
+    int run_head(const float *hidden_rows, int count);
+    HostTensor *host_slot(int layer, int slot);
+
+    LlamaConfig c_;
+    bool finalized_ = false;
+    HostTensor h_embedding_, h_final_norm_, h_lm_head_;
+    std::vector<HostLayer> h_layers_;
+
+    void *embedding_ = nullptr;
+    bool embedding_f16_ = true;
+    float *final_norm_ = nullptr;
+    DeviceMatrix lm_head_;
+    std::vector<Layer> layers_;
+    float *rope_cos_ = nullptr, *rope_sin_ = nullptr;
+    // activations for up to kMaxStepRows rows
+    float *hidden_ = nullptr, *qkv_ = nullptr, *q_ = nullptr, *gu_ = nullptr, *logits_ = nullptr, *last_hidden_ = nullptr;
+    uint16_t *xn_ = nullptr, *ctx_ = nullptr, *act_ = nullptr;
+    int *d_tokens_ = nullptr, *d_pos_ = nullptr, *d_seq_ = nullptr, *d_out_tokens_ = nullptr;
+    std::vector<int> visible_;
+    size_t weight_bytes_ = 0;
+};
+
+}  // namespace esp
+
+struct ESPLlamaRuntime {
+    esp::LlamaRuntime *rt;
+};

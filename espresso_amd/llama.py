@@ -1,0 +1,147 @@
+"""ctypes face of the GPU-resident llama runtime (ESPLlamaRuntime in include/espresso_hip.h)."""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import _lib
+
+SLOT_TOKEN_EMBEDDING, SLOT_FINAL_NORM, SLOT_LM_HEAD = 0, 1, 2
+SLOT_RMS_ATT, SLOT_WQ, SLOT_WK, SLOT_WV, SLOT_WO, SLOT_RMS_FFN, SLOT_W1, SLOT_W2, SLOT_W3, SLOT_Q_NORM, SLOT_K_NORM = range(10, 21)
+LAYER_SLOTS = {"rms_att": SLOT_RMS_ATT, "wq": SLOT_WQ, "wk": SLOT_WK, "wv": SLOT_WV, "wo": SLOT_WO,
+               "rms_ffn": SLOT_RMS_FFN, "w1": SLOT_W1, "w2": SLOT_W2, "w3": SLOT_W3,
+               "q_norm": SLOT_Q_NORM, "k_norm": SLOT_K_NORM}
+
+
+@dataclass
+class MultiModelConfig:
+    """Sources/ModelSupport/MultiModelConfig.swift:3-55 (llama architecture)."""
+    n_layer: int
+    n_head: int
+    n_kv_head: int
+    d_model: int
+    head_dim: int
+    hidden_dim: int
+    vocab: int
+    max_seq: int
+    norm_eps: float = 1e-5
+    rope_theta: float = 10000.0
+    eos_token: int = -1
+    name: str = "llama"
+
+    @property
+    def attention_dim(self) -> int:
+        return self.n_head * self.head_dim
+
+    @property
+    def kv_dim(self) -> int:
+        return self.n_kv_head * self.head_dim
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class LlamaRuntime:
+    def __init__(self, cfg: MultiModelConfig, kv_format: int = _lib.FORMAT_F32, max_sequences: int = 1):
+        self.cfg = cfg
+        self._L = _lib.load_library()
+        c = _lib.LlamaConfigStruct(cfg.n_layer, cfg.n_head, cfg.n_kv_head, cfg.d_model, cfg.head_dim, cfg.hidden_dim,
+                                   cfg.vocab, cfg.max_seq, cfg.norm_eps, cfg.rope_theta, cfg.eos_token, kv_format,
+                                   max_sequences)
+        self._h = self._L.esp_llama_create(C.byref(c))
+        if not self._h:
+            raise _lib.EspressoError(-1, _lib.last_error())
+
+    def close(self) -> None:
+        if self._h:
+            self._L.esp_llama_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_weight(self, layer: int, slot: int, fmt: int, data: np.ndarray) -> None:
+        a = np.ascontiguousarray(data)
+        raw = a.view(np.uint8).ravel()
+        _lib.check(self._L.esp_llama_set_weight(self._h, layer, slot, fmt, _ptr(raw), raw.size))
+
+    def finalize(self) -> None:
+        _lib.check(self._L.esp_llama_finalize(self._h))
+
+    @property
+    def weight_bytes(self) -> int:
+        return int(self._L.esp_llama_weight_bytes(self._h))
+
+    def reset(self) -> None:
+        _lib.check(self._L.esp_llama_reset(self._h))
+
+    def prefill(self, tokens, sequence: int = 0) -> None:
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        _lib.check(self._L.esp_llama_prefill(self._h, sequence, _ptr(t), t.size))
+
+    def advance(self, token: int, sequence: int = 0) -> None:
+        _lib.check(self._L.esp_llama_advance(self._h, sequence, C.c_uint32(token)))
+
+    def select_greedy(self, sequence: int = 0) -> int:
+        t = C.c_uint32(0)
+        _lib.check(self._L.esp_llama_select_greedy_token(self._h, sequence, C.byref(t)))
+        return int(t.value)
+
+    def visible(self, sequence: int = 0) -> int:
+        return int(self._L.esp_llama_visible_token_count(self._h, sequence))
+
+    def set_visible(self, count: int, sequence: int = 0) -> None:
+        _lib.check(self._L.esp_llama_set_visible_token_count(self._h, sequence, count))
+
+    def last_hidden(self, sequence: int = 0) -> np.ndarray:
+        out = np.empty(self.cfg.d_model, dtype=np.float32)
+        _lib.check(self._L.esp_llama_read_last_hidden(self._h, sequence, _ptr(out)))
+        return out
+
+    def logits(self, sequence: int = 0) -> np.ndarray:
+        out = np.empty(self.cfg.vocab, dtype=np.float32)
+        _lib.check(self._L.esp_llama_read_logits(self._h, sequence, _ptr(out)))
+        return out
+
+    def generate(self, prompt, max_tokens: int):
+        p = np.ascontiguousarray(prompt, dtype=np.uint32)
+        out = np.zeros(max(max_tokens, 1), dtype=np.uint32)
+        lat = np.zeros(max(max_tokens, 1), dtype=np.float64)
+        n = C.c_int(0)
+        st = _lib.GenerationStatsStruct()
+        _lib.check(self._L.esp_llama_generate(self._h, _ptr(p), p.size, max_tokens, _ptr(out), C.byref(n), C.byref(st), _ptr(lat)))
+        stats = {k: getattr(st, k) for k, _ in st._fields_}
+        stats["token_latencies_ms"] = lat[:n.value].tolist()
+        return out[:n.value].tolist(), stats
+
+
+def generate_two_token(target: LlamaRuntime, draft: LlamaRuntime, prompt, max_tokens: int, reference_accounting: bool = True):
+    L = _lib.load_library()
+    p = np.ascontiguousarray(prompt, dtype=np.uint32)
+    out = np.zeros(max(max_tokens, 1), dtype=np.uint32)
+    n = C.c_int(0)
+    st, tt = _lib.GenerationStatsStruct(), _lib.TwoTokenStatsStruct()
+    _lib.check(L.esp_llama_generate_two_token(target._h, draft._h, _ptr(p), p.size, max_tokens, int(reference_accounting),
+                                              _ptr(out), C.byref(n), C.byref(st), C.byref(tt)))
+    stats = {k: getattr(st, k) for k, _ in st._fields_}
+    stats.update({k: getattr(tt, k) for k, _ in tt._fields_})
+    return out[:n.value].tolist(), stats
+
+
+def load_packed_weights(rt: LlamaRuntime, packed: dict, matrix_format: int, embedding_format: int = _lib.FORMAT_F16,
+                        norm_format: int = _lib.FORMAT_F16) -> None:
+    """packed: {"embedding", "final_norm", "lm_head", "layers": [{"rms_att", "wq", ...}]} of raw GGUF-layout bytes."""
+    rt.set_weight(0, SLOT_TOKEN_EMBEDDING, embedding_format, packed["embedding"])
+    rt.set_weight(0, SLOT_FINAL_NORM, norm_format, packed["final_norm"])
+    rt.set_weight(0, SLOT_LM_HEAD, matrix_format, packed["lm_head"])
+    for l, layer in enumerate(packed["layers"]):
+        for name, data in layer.items():
+            is_matrix = name in ("wq", "wk", "wv", "wo", "w1", "w2", "w3")
+            rt.set_weight(l, LAYER_SLOTS[name], matrix_format if is_matrix else norm_format, data)
+    rt.finalize()

@@ -84,6 +84,93 @@ int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y
 int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int rotate,
                   double *mean_us, double *best_us);
 
+/* ---- llama decoder state resident on the GPU -------------------------------------------- *
+ * Replaces CPUExactLlamaRuntime (Sources/RealModelInference/RealModelInferenceEngine.swift:548-850):
+ * create = init(config:weightDirURL:) :562-614, reset :616-635, prefill :637-645, advance :672-680,
+ * select_greedy_token :663-670 + :825-849.  captureCheckpoint/rollback (:647-661) copy every KV
+ * cache in the reference; here a rollback is esp_llama_set_visible_token_count with a smaller count,
+ * because columns beyond the visible length are never read. */
+typedef struct ESPLlamaRuntime ESPLlamaRuntime;
+
+/* MultiModelConfig (Sources/ModelSupport/MultiModelConfig.swift:3-55) plus the two storage choices
+ * this implementation adds. */
+typedef struct ESPLlamaConfig {
+    int32_t n_layer, n_head, n_kv_head, d_model, head_dim, hidden_dim, vocab, max_seq;
+    float norm_eps, rope_theta;
+    int32_t eos_token;      /* -1: none */
+    int32_t kv_format;      /* ESP_FORMAT_F32 (the reference's caches) or ESP_FORMAT_F16 */
+    int32_t max_sequences;  /* independent KV caches (1..16) */
+} ESPLlamaConfig;
+
+/* Weight slots, named after LayerWeightPaths (Sources/ModelSupport/LayerWeightPaths.swift:22-84):
+ * embeddings/token.bin, rms_final.bin, lm_head.bin and layers/<i>/{rms_att,wq,wk,wv,wo,rms_ffn,w1,w2,w3,
+ * q_norm,k_norm}.bin (w1 = gate, w3 = up, w2 = down). */
+#define ESP_SLOT_TOKEN_EMBEDDING 0
+#define ESP_SLOT_FINAL_NORM 1
+#define ESP_SLOT_LM_HEAD 2
+#define ESP_SLOT_RMS_ATT 10
+#define ESP_SLOT_WQ 11
+#define ESP_SLOT_WK 12
+#define ESP_SLOT_WV 13
+#define ESP_SLOT_WO 14
+#define ESP_SLOT_RMS_FFN 15
+#define ESP_SLOT_W1 16
+#define ESP_SLOT_W2 17
+#define ESP_SLOT_W3 18
+#define ESP_SLOT_Q_NORM 19
+#define ESP_SLOT_K_NORM 20
+
+ESPLlamaRuntime *esp_llama_create(const ESPLlamaConfig *config);
+void esp_llama_free(ESPLlamaRuntime *runtime);
+/* Copies `bytes` of one tensor.  Projections and lm_head: GGUF block layout of `format`, row-major
+ * [rows, cols]; norm vectors and the embedding table: f32 or f16.  `layer` is ignored for the three
+ * top-level slots.  q_norm/k_norm are optional and used only when both are given
+ * (RealModelInferenceEngine.swift:6585-6607). */
+int esp_llama_set_weight(ESPLlamaRuntime *runtime, int layer, int slot, int format, const void *data, size_t bytes);
+/* Lays the weights out in HBM; required once, before any of the calls below. */
+int esp_llama_finalize(ESPLlamaRuntime *runtime);
+/* Packed weight bytes one decoded token reads (all projections plus lm_head). */
+size_t esp_llama_weight_bytes(const ESPLlamaRuntime *runtime);
+int esp_llama_reset(ESPLlamaRuntime *runtime);
+int esp_llama_prefill(ESPLlamaRuntime *runtime, int sequence, const uint32_t *tokens, int count);
+int esp_llama_advance(ESPLlamaRuntime *runtime, int sequence, uint32_t token);
+int esp_llama_select_greedy_token(ESPLlamaRuntime *runtime, int sequence, uint32_t *token);
+/* visibleTokenCount; returns -1 for a sequence out of range. */
+int esp_llama_visible_token_count(const ESPLlamaRuntime *runtime, int sequence);
+int esp_llama_set_visible_token_count(ESPLlamaRuntime *runtime, int sequence, int count);
+/* lastHidden [d_model] and the full-vocabulary logits of the current state [vocab], fp32. */
+int esp_llama_read_last_hidden(ESPLlamaRuntime *runtime, int sequence, float *out);
+int esp_llama_read_logits(ESPLlamaRuntime *runtime, int sequence, float *out);
+
+typedef struct ESPGenerationStats {
+    int32_t generated;
+    double prefill_ms, decode_ms, first_token_latency_ms, tokens_per_second;
+} ESPGenerationStats;
+
+/* generateIncrementalExactCPULlama at temperature 0 (RealModelInferenceEngine.swift:6192-6431).
+ * Writes at most max_tokens ids; *out_count receives how many.  token_latencies_ms may be NULL,
+ * else it receives one latency per generated token (GenerationResult.tokenLatenciesMs, :17-55). */
+int esp_llama_generate(ESPLlamaRuntime *runtime, const uint32_t *prompt, int prompt_count, int max_tokens,
+                       uint32_t *out_tokens, int *out_count, ESPGenerationStats *stats, double *token_latencies_ms);
+
+typedef struct ESPTwoTokenStats {
+    /* one pass = one batched verify of [current token, proposed token] by the target model; committed
+     * is 1 or 2 per pass and accepted 0 or 1 (ExactTwoTokenPassMetrics, GenerationHarness.swift:104-131) */
+    int32_t passes, committed_total, accepted_total;
+    /* the reference CPU loop's accounting of the same stream (committedExactTokensPerPass /
+     * acceptedFutureTokensPerPass, RealModelInferenceEngine.swift:6109-6175); accepted is -1 when
+     * reference_accounting was 0 */
+    int32_t reference_passes, reference_committed_total, reference_accepted_total;
+} ESPTwoTokenStats;
+
+/* generateIncrementalExactTwoTokenDraftLlama (RealModelInferenceEngine.swift:6014-6190) with the
+ * target model verifying both tokens of a pass in one batched step.  The emitted stream equals
+ * esp_llama_generate on `target`. */
+int esp_llama_generate_two_token(ESPLlamaRuntime *target, ESPLlamaRuntime *draft, const uint32_t *prompt,
+                                 int prompt_count, int max_tokens, int reference_accounting,
+                                 uint32_t *out_tokens, int *out_count, ESPGenerationStats *stats,
+                                 ESPTwoTokenStats *two_token_stats);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,166 @@
+"""GPU parity of the llama runtime against the CPU oracle on the same seeded weights: hidden state and
+logits within tolerance, greedy tokens identical, two-token stream identical to plain greedy."""
+import numpy as np
+import pytest
+
+import model_util as mu
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+LOGIT_TOL = 2e-2   # max-abs bound on logits for fp16 GEMV inputs with fp32 accumulation
+
+
+@pytest.fixture(scope="module")
+def llama():
+    import espresso_amd.llama as ll
+    import espresso_amd.ops as o
+    o.init()
+    return ll
+
+
+def make_pair(ll, cfg_kw, fmt, seed, std=0.02, kv_fp16=False, norm_jitter=0.0, qk_norm=False):
+    ocfg = orc.LlamaConfig(gemv_inputs_fp16=True, kv_fp16=kv_fp16, **cfg_kw)
+    w = mu.random_weights(ocfg, seed, std=std, norm_jitter=norm_jitter)
+    if qk_norm:
+        rng = np.random.default_rng(seed + 1)
+        for L in w["layers"]:
+            L["q_norm"] = (1 + rng.normal(0, 0.1, ocfg.head_dim)).astype(np.float32)
+            L["k_norm"] = (1 + rng.normal(0, 0.1, ocfg.head_dim)).astype(np.float32)
+    packed, deq = mu.pack_weights(w, fmt)
+    oracle_rt = mu.load_oracle(ocfg, deq)
+    gcfg = ll.MultiModelConfig(**{k: v for k, v in cfg_kw.items()})
+    gpu_rt = ll.LlamaRuntime(gcfg, kv_format=orc.FMT_F16 if kv_fp16 else orc.FMT_F32)
+    ll.load_packed_weights(gpu_rt, packed, fmt)
+    return oracle_rt, gpu_rt
+
+
+TINY = dict(n_layer=2, n_head=4, n_kv_head=2, d_model=256, head_dim=64, hidden_dim=512, vocab=512, max_seq=48)
+
+
+@pytest.mark.parametrize("fmt", [orc.FMT_Q8_0, orc.FMT_Q4_0, orc.FMT_Q4_K, orc.FMT_F16])
+@pytest.mark.parametrize("kv_fp16", [False, True])
+def test_stepwise_hidden_logits_and_tokens(llama, fmt, kv_fp16):
+    o, g = make_pair(llama, TINY, fmt, seed=31 + fmt, std=0.08, kv_fp16=kv_fp16, norm_jitter=0.05)
+    toks = [5, 99, 300, 17, 17, 511, 0, 42]
+    o.prefill(toks[:1]); g.prefill(toks[:1])
+    for t in toks[1:]:
+        ho, hg = o.last_hidden(), g.last_hidden()
+        assert np.abs(ho - hg).max() <= 2e-3 * max(1.0, np.abs(ho).max())
+        lo, lg = o.logits(), g.logits()
+        assert np.abs(lo - lg).max() <= LOGIT_TOL
+        if o.top2_margin() > 1e-3:
+            assert g.select_greedy() == o.select_greedy()
+        assert o.advance(t) == 0
+        g.advance(t)
+    assert g.visible() == o.visible == len(toks)
+
+
+def test_per_head_qk_norm(llama):
+    o, g = make_pair(llama, dict(TINY, head_dim=128, n_head=2, n_kv_head=1), orc.FMT_Q8_0, seed=77, std=0.08, qk_norm=True)
+    o.prefill([1, 2, 3, 4]); g.prefill([1, 2, 3, 4])
+    assert np.abs(o.last_hidden() - g.last_hidden()).max() <= 2e-3 * max(1.0, np.abs(o.last_hidden()).max())
+    assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
+
+
+def test_generate_matches_oracle_and_stops(llama):
+    cfg = dict(TINY, max_seq=40)
+    o, g = make_pair(llama, cfg, orc.FMT_Q8_0, seed=5, std=0.08)
+    prompt = [1, 2, 3, 4, 5, 6]
+    want, margin = o.generate(prompt, 100, with_margin=True)
+    got, stats = g.generate(prompt, 100)
+    assert len(want) == 34 and margin > 1e-4
+    assert got == want
+    assert stats["generated"] == 34 and len(stats["token_latencies_ms"]) == 34 and stats["tokens_per_second"] > 0
+    assert g.generate(prompt, 3)[0] == want[:3]
+    assert g.generate(prompt, 0)[0] == []
+    # EOS is appended and ends generation
+    o2, g2 = make_pair(llama, dict(cfg, eos_token=want[4]), orc.FMT_Q8_0, seed=5, std=0.08)
+    first = want.index(want[4])
+    assert g2.generate(prompt, 100)[0] == want[:first + 1]
+
+
+def test_argument_errors(llama):
+    import espresso_amd._lib as lib
+    o, g = make_pair(llama, dict(TINY, max_seq=8), orc.FMT_Q8_0, seed=6)
+    with pytest.raises(lib.EspressoError, match="must not be empty"):
+        g.generate([], 4)
+    with pytest.raises(lib.EspressoError, match="outside vocab"):
+        g.prefill([TINY["vocab"]])
+    g.prefill(list(range(8)))
+    with pytest.raises(lib.EspressoError, match="exceeds context"):
+        g.advance(1)
+    with pytest.raises(lib.EspressoError):
+        llama.LlamaRuntime(llama.MultiModelConfig(**dict(TINY, n_head=3)))            # nHead % nKVHead
+    rt = llama.LlamaRuntime(llama.MultiModelConfig(**TINY))
+    with pytest.raises(lib.EspressoError, match="missing"):
+        rt.finalize()
+    with pytest.raises(lib.EspressoError, match="expects"):
+        rt.set_weight(0, llama.SLOT_WQ, orc.FMT_Q8_0, np.zeros(10, np.uint8))
+
+
+def test_rollback_by_visible_length(llama):
+    o, g = make_pair(llama, TINY, orc.FMT_Q4_K, seed=8, std=0.08)
+    g.prefill([1, 2, 3]); g.advance(7)
+    want = g.last_hidden()
+    g.prefill([1, 2, 3]); g.advance(30); g.advance(31)
+    g.set_visible(3); g.advance(7)
+    assert np.array_equal(g.last_hidden(), want)
+
+
+def test_two_token_stream_and_counters(llama):
+    full_kw = dict(TINY, n_layer=3, max_seq=40)
+    draft_kw = dict(TINY, n_layer=1, max_seq=40)
+    of, gf = make_pair(llama, full_kw, orc.FMT_Q8_0, seed=21, std=0.08)
+    od, gd = make_pair(llama, draft_kw, orc.FMT_Q8_0, seed=22, std=0.08)
+    prompt = [7, 8, 9, 10, 11]
+    for budget in (1, 2, 3, 10, 35, 100):
+        plain, _ = gf.generate(prompt, budget)
+        want, ostats = orc.generate_two_token(of, od, prompt, budget)
+        got, st = llama.generate_two_token(gf, gd, prompt, budget)
+        assert got == plain == want
+        # the reference loop's accounting is reproduced exactly
+        assert (st["reference_passes"], st["reference_committed_total"], st["reference_accepted_total"]) == \
+               (ostats["passes"], ostats["committed_total"], ostats["accepted_total"])
+        # harness invariants (GenerationHarness.swift:612-686): 1..2 committed per pass, accepted => 2 committed
+        assert st["passes"] <= st["committed_total"] <= 2 * st["passes"]
+        assert st["accepted_total"] == st["committed_total"] - st["passes"]
+    # a draft identical to the target: every proposal is accepted
+    of2, gf2 = make_pair(llama, full_kw, orc.FMT_Q8_0, seed=21, std=0.08)
+    got, st = llama.generate_two_token(gf, gf2, prompt, 21)
+    assert got == gf.generate(prompt, 21)[0]
+    assert st["accepted_total"] == st["passes"] == 10 and st["reference_accepted_total"] == 20
+
+
+def test_local_bigram_golden(llama):
+    """LocalBigramArtifactBuilder model (one-hot embeddings, classifier[next,cur] = 10, zero trunk):
+    golden [35] -> [105, 110, 116, 32]; harness counters committed [2,2], accepted [1,1]
+    (Tests/EspressoTests/GenerationHarnessTests.swift:821-849)."""
+    from test_oracle_runtime import bigram_model
+    ocfg, w = bigram_model(d_model=128, vocab=128)
+    packed, deq = mu.pack_weights(w, orc.FMT_F16)
+    kw = dict(n_layer=1, n_head=2, n_kv_head=2, d_model=128, head_dim=64, hidden_dim=16, vocab=128, max_seq=32)
+    rts = []
+    for _ in range(2):
+        rt = llama.LlamaRuntime(llama.MultiModelConfig(**kw))
+        llama.load_packed_weights(rt, packed, orc.FMT_F16)
+        rts.append(rt)
+    assert rts[0].generate([35], 4)[0] == [105, 110, 116, 32]
+    got, st = llama.generate_two_token(rts[0], rts[1], [35], 5)
+    assert got == [105, 110, 116, 32, 105]
+    # first token comes from the prefill; then two passes each commit 2 and accept 1
+    assert (st["passes"], st["committed_total"], st["accepted_total"]) == (2, 4, 2)
+
+
+def test_config2_model_q8_0_greedy_128_tokens(llama):
+    """BASELINE config 2: 6 layers, d=768, 12 heads x 64, FFN 2048, vocab 32000, context 256, all
+    linears Q8_0, prompt of 16 uniform ids, 128 greedy tokens identical to the oracle."""
+    cfg = dict(n_layer=6, n_head=12, n_kv_head=12, d_model=768, head_dim=64, hidden_dim=2048, vocab=32000, max_seq=256)
+    o, g = make_pair(llama, cfg, orc.FMT_Q8_0, seed=20261125, std=0.02)
+    prompt = np.random.default_rng(16).integers(0, 32000, 16).tolist()
+    want, margin = o.generate(prompt, 128, with_margin=True)
+    got, stats = g.generate(prompt, 128)
+    print(f"config2 q8_0: min top-2 margin {margin:.3e}, gpu {stats['tokens_per_second']:.0f} tok/s")
+    assert len(want) == 128
+    assert got == want
+    assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
