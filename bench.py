@@ -1,0 +1,200 @@
+#!/usr/bin/env python3
+"""Decode throughput of the quantized llama hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3-8b-q4k|stories-6l-q8_0] [--no-cpu-baseline]
+
+One step = one greedy decode token at batch 1 (LM head + argmax, then the trunk for the chosen token).
+The model is random-init from a seed in the packed GGUF format, resident in HBM before the timed region;
+the prompt is prefilled outside the timed region, as the reference excludes prefill from tokens/s
+(RealModelInferenceEngine.swift:6355, 6415-6419).  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E peak
+
+WORKLOADS = {
+    # BASELINE.json configs[3]
+    "llama3-8b-q4k": dict(arch="LLAMA3_8B", fmt="q4_k", kv="f16", prompt=512, decode=256, seed=4,
+                          describe="Llama-3-8B architecture, random-init, Q4_K linears + Q4_K lm_head, fp16 "
+                                   "embedding/norms/KV; 512-token prompt then greedy decode at batch 1"),
+    # BASELINE.json configs[1]
+    "stories-6l-q8_0": dict(arch="STORIES_6L", fmt="q8_0", kv="f32", prompt=16, decode=128, seed=2,
+                            describe="6-layer d=768 llama (12 heads x 64, FFN 2048, vocab 32000, ctx 256), all linears "
+                                     "Q8_0; 16-token prompt then greedy decode at batch 1"),
+}
+
+
+def build_model(name: str):
+    import espresso_amd.llama as ll
+    import espresso_amd.synthetic as syn
+    from espresso_amd import _lib
+    w = WORKLOADS[name]
+    cfg = ll.MultiModelConfig(**getattr(syn, w["arch"]))
+    fmt = _lib.FORMAT_NAMES[w["fmt"]]
+    kv = _lib.FORMAT_F16 if w["kv"] == "f16" else _lib.FORMAT_F32
+    t0 = time.time()
+    rt, packed = syn.build_runtime(cfg, fmt, seed=w["seed"], kv_format=kv, keep_packed=True)
+    return cfg, rt, packed, time.time() - t0
+
+
+def run_gpu(name: str, steps: int, warmup: int):
+    import espresso_amd.llama as ll
+    w = WORKLOADS[name]
+    cfg, rt, packed, build_s = build_model(name)
+    if w["prompt"] + warmup + steps + 1 > cfg.max_seq:
+        raise SystemExit(f"prompt {w['prompt']} + warmup {warmup} + steps {steps} does not fit context {cfg.max_seq}")
+    prompt = np.random.default_rng(1000 + w["seed"]).integers(0, cfg.vocab, w["prompt"]).astype(np.uint32)
+    t0 = time.perf_counter()
+    rt.prefill(prompt)
+    prefill_s = time.perf_counter() - t0
+    warm_tokens = ll.continue_greedy(rt, warmup)
+    # ---- timed region: exactly `steps` decode steps; every step ends with a device-to-host read of the
+    # chosen token, so the region is bracketed by stream synchronisation on both sides
+    rt.last_hidden()
+    t0 = time.perf_counter()
+    tokens = ll.continue_greedy(rt, steps)
+    rt.last_hidden()
+    elapsed = time.perf_counter() - t0
+    # ---- instrumented pass (not part of `value`): HIP events around every GEMV/attention launch
+    extra = min(32, cfg.max_seq - rt.visible() - 1)
+    ll.set_kernel_timing(rt, True)
+    ll.continue_greedy(rt, extra)
+    kt = ll.kernel_times(rt)
+    ll.set_kernel_timing(rt, False)
+    return dict(cfg=cfg, rt=rt, packed=packed, prompt=prompt, tokens=warm_tokens + tokens, elapsed=elapsed,
+                build_s=build_s, prefill_s=prefill_s, kernel_times=kt, weight_bytes=rt.weight_bytes)
+
+
+def cpu_baseline(name: str, gpu: dict) -> dict:
+    """Times the CPU oracle (the C restatement of the reference's CPU-exact path, single thread) on a bounded
+    sample of the same model: same packed bytes, dequantised to fp32 as the reference holds them."""
+    from oracle import oracle as orc
+    import espresso_amd.llama as ll
+    from espresso_amd import _lib
+    w = WORKLOADS[name]
+    cfg, packed = gpu["cfg"], gpu["packed"]
+    fmt = _lib.FORMAT_NAMES[w["fmt"]]
+    shapes = {"wq": (cfg.attention_dim, cfg.d_model), "wk": (cfg.kv_dim, cfg.d_model), "wv": (cfg.kv_dim, cfg.d_model),
+              "wo": (cfg.d_model, cfg.attention_dim), "w1": (cfg.hidden_dim, cfg.d_model),
+              "w3": (cfg.hidden_dim, cfg.d_model), "w2": (cfg.d_model, cfg.hidden_dim)}
+    slot = {"rms_att": orc.W_RMS_ATT, "wq": orc.W_WQ, "wk": orc.W_WK, "wv": orc.W_WV, "wo": orc.W_WO,
+            "rms_ffn": orc.W_RMS_FFN, "w1": orc.W_W1, "w2": orc.W_W2, "w3": orc.W_W3}
+    full = name == "stories-6l-q8_0"
+    n_layer = cfg.n_layer if full else 1
+    ocfg = orc.LlamaConfig(n_layer=n_layer, n_head=cfg.n_head, n_kv_head=cfg.n_kv_head, d_model=cfg.d_model,
+                           head_dim=cfg.head_dim, hidden_dim=cfg.hidden_dim, vocab=cfg.vocab, max_seq=64 if not full else cfg.max_seq,
+                           norm_eps=cfg.norm_eps, rope_theta=cfg.rope_theta, gemv_inputs_fp16=True, kv_fp16=w["kv"] == "f16")
+    rt = orc.LlamaRuntime(ocfg)
+    n = cfg.vocab * cfg.d_model
+    rt.set_weight(0, orc.W_TOKEN_EMBEDDING, orc.dequantize(orc.FMT_F16, packed["embedding"], n))
+    rt.set_weight(0, orc.W_FINAL_NORM, np.ones(cfg.d_model, np.float32))
+    rt.set_weight(0, orc.W_LM_HEAD, orc.dequantize(fmt, packed["lm_head"], n))
+    for l in range(n_layer):
+        for k, s in slot.items():
+            if k in shapes:
+                r, c = shapes[k]
+                rt.set_weight(l, s, orc.dequantize(fmt, packed["layers"][l][k], r * c))
+            else:
+                rt.set_weight(l, s, np.ones(cfg.d_model, np.float32))
+    prompt = gpu["prompt"]
+    if full:
+        t0 = time.perf_counter()
+        rt.prefill(prompt.tolist())
+        n_tok = 32
+        t0 = time.perf_counter()
+        toks = []
+        for _ in range(n_tok):
+            t = rt.select_greedy(); toks.append(t); rt.advance(t)
+        dt = time.perf_counter() - t0
+        same = toks == gpu["tokens"][:n_tok]
+        return {"value": n_tok / dt, "unit": "tok/s", "cores": 1, "kind": "port",
+                "sample": f"whole model, {n_tok} greedy tokens after the same {len(prompt)}-token prompt; "
+                          f"tokens identical to the GPU run: {same}"}
+    # bounded sample of the 8B shape: layer 0 alone plus the LM head
+    rt.prefill(prompt[:8].tolist())
+    n_tok = 6
+    t_layer = t_head = 0.0
+    for i in range(n_tok):
+        t0 = time.perf_counter(); tok = rt.select_greedy(); t_head += time.perf_counter() - t0
+        t0 = time.perf_counter(); rt.advance(tok); t_layer += time.perf_counter() - t0
+    t_layer /= n_tok; t_head /= n_tok
+    est = 1.0 / (cfg.n_layer * t_layer + t_head)
+    return {"value": est, "unit": "tok/s", "cores": 1, "kind": "port",
+            "sample": f"layer 0 of {cfg.n_layer} ({t_layer * 1e3:.0f} ms/token) and the LM head ({t_head * 1e3:.0f} ms/token), "
+                      f"{n_tok} tokens at context <= 16, extrapolated to {cfg.n_layer} layers (attention at the benchmark's "
+                      f"context not included)"}
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="llama3-8b-q4k")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this path is a batch-1 decode on a single MI355X; run with --gpus 1")
+    import espresso_amd.ops as ops
+    ops.init()
+    w = WORKLOADS[args.workload]
+    steps = args.steps if args.steps is not None else w["decode"]
+    gpu = run_gpu(args.workload, steps, args.warmup)
+    tok_s = steps / gpu["elapsed"]
+    kt = gpu["kernel_times"]
+    dominant = max((k for k in kt if kt[k]["bytes_per_launch"]), key=lambda k: kt[k]["total_us"])
+    d = kt[dominant]
+    gemv_us = sum(kt[k]["total_us"] for k in ("qkv", "wo", "gate_up", "down", "head"))
+    gemv_bytes = sum(kt[k]["bytes_per_launch"] * kt[k]["launches"] for k in ("qkv", "wo", "gate_up", "down", "head"))
+    result = {
+        "metric": "decode tok/s bs1 (%s)" % ("8B-arch Q4_K" if args.workload == "llama3-8b-q4k" else "6L d768 Q8_0"),
+        "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": gpu["elapsed"] / steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": args.workload, "description": w["describe"], "prompt_tokens": w["prompt"],
+                   "weight_bytes_per_token": gpu["weight_bytes"],
+                   "token_bytes_over_hbm_peak_tok_s": HBM_PEAK_GBPS * 1e9 / gpu["weight_bytes"]},
+        "roofline": {"bound": "hbm", "kernel": f"dequant-GEMV {dominant}", "achieved": d["gbps"], "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": d["gbps"] / HBM_PEAK_GBPS, "traffic": None,
+                     "bytes_per_launch": d["bytes_per_launch"], "mean_launch_us": d["mean_us"], "launches_timed": d["launches"],
+                     "all_gemv_gbps": gemv_bytes / gemv_us / 1e3 if gemv_us else 0.0,
+                     "all_gemv_frac": gemv_bytes / gemv_us / 1e3 / HBM_PEAK_GBPS if gemv_us else 0.0,
+                     "per_kernel": {k: {"mean_us": round(v["mean_us"], 2), "gbps": round(v["gbps"], 1), "launches": v["launches"]}
+                                    for k, v in kt.items()},
+                     "how": "HIP events around each launch in an instrumented pass run right after the timed region"},
+        "model_build_s": round(gpu["build_s"], 1), "prefill_s": round(gpu["prefill_s"], 3),
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.workload, gpu)
+    gpu["rt"].close()
+    del gpu
+    if not args.no_secondary:
+        other = "stories-6l-q8_0" if args.workload == "llama3-8b-q4k" else None
+        if other:
+            ow = WORKLOADS[other]
+            osteps = ow["decode"]
+            g2 = run_gpu(other, osteps, args.warmup)
+            sec = {"metric": "decode tok/s bs1 (6L d768 Q8_0)", "value": osteps / g2["elapsed"], "unit": "tok/s",
+                   "steps": osteps, "ms_per_step": g2["elapsed"] / osteps * 1e3, "workload": other,
+                   "weight_bytes_per_token": g2["weight_bytes"],
+                   "per_kernel": {k: {"mean_us": round(v["mean_us"], 2), "gbps": round(v["gbps"], 1)} for k, v in g2["kernel_times"].items()}}
+            if not args.no_cpu_baseline:
+                sec["cpu_baseline"] = cpu_baseline(other, g2)
+            result["secondary"] = sec
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -120,3 +120,11 @@ def _declare_llama(L: C.CDLL) -> None:
     L.esp_llama_generate_two_token.restype = i32
     L.esp_llama_generate_two_token.argtypes = [vp, vp, vp, i32, i32, i32, vp, C.POINTER(i32),
                                                C.POINTER(GenerationStatsStruct), C.POINTER(TwoTokenStatsStruct)]
+    L.esp_llama_continue_greedy.restype = i32
+    L.esp_llama_continue_greedy.argtypes = [vp, i32, i32, vp]
+    L.esp_llama_set_kernel_timing.restype = i32
+    L.esp_llama_set_kernel_timing.argtypes = [vp, i32]
+    L.esp_llama_kernel_times.restype = i32
+    L.esp_llama_kernel_times.argtypes = [vp, vp, vp, vp, i32]
+    L.esp_synth_weights.restype = i32
+    L.esp_synth_weights.argtypes = [i32, C.c_uint64, C.c_float, sz, vp]

@@ -115,4 +115,56 @@ int esp_llama_generate_two_token(ESPLlamaRuntime *target, ESPLlamaRuntime *draft
     return ESP_OK;
 }
 
+int esp_llama_continue_greedy(ESPLlamaRuntime *runtime, int sequence, int steps, uint32_t *out_tokens) {
+    if (!runtime) return bad_handle();
+    if (!runtime->rt->finalized()) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+    if (steps < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "steps must be >= 0");
+    for (int i = 0; i < steps; i++) {
+        uint32_t t = 0;
+        int rc = runtime->rt->select_greedy(sequence, &t);
+        if (rc != ESP_OK) return rc;
+        if (out_tokens) out_tokens[i] = t;
+        if ((rc = runtime->rt->advance(sequence, t)) != ESP_OK) return rc;
+    }
+    return ESP_OK;
+}
+
+int esp_llama_set_kernel_timing(ESPLlamaRuntime *runtime, int enabled) {
+    if (!runtime) return bad_handle();
+    runtime->rt->set_kernel_timing(enabled != 0);
+    return ESP_OK;
+}
+
+int esp_llama_kernel_times(ESPLlamaRuntime *runtime, double *total_us, int64_t *launches, uint64_t *bytes_per_launch,
+                           int reset) {
+    if (!runtime) return bad_handle();
+    double t[LlamaRuntime::K_CLASS_COUNT];
+    long n[LlamaRuntime::K_CLASS_COUNT];
+    int rc = runtime->rt->collect_kernel_times(t, n, reset != 0);
+    if (rc != ESP_OK) return rc;
+    for (int k = 0; k < LlamaRuntime::K_CLASS_COUNT; k++) {
+        if (total_us) total_us[k] = t[k];
+        if (launches) launches[k] = n[k];
+        if (bytes_per_launch) bytes_per_launch[k] = runtime->rt->kernel_bytes(k);
+    }
+    return ESP_OK;
+}
+
+int esp_synth_weights(int format, uint64_t seed, float std_dev, size_t elements, void *out_blocks) {
+    if (!out_blocks || elements == 0 || elements % 256 != 0)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "synth_weights: elements must be a positive multiple of 256");
+    if (!(format == FMT_F16 || format == FMT_Q8_0 || format == FMT_Q4_0 || format == FMT_Q4_K))
+        return fail(ESP_ERR_UNSUPPORTED, "synth_weights: format %d", format);
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    const size_t bytes = format_bytes(format, elements);
+    uint8_t *d = nullptr;
+    if ((rc = device_alloc(&d, bytes)) != ESP_OK) return rc;
+    hipError_t e = launch_synth(format, seed, std_dev, elements, d, context().stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(out_blocks, d, bytes, hipMemcpyDeviceToHost, context().stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(context().stream);
+    (void)hipFree(d);
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "synth_weights");
+}
+
 }  // extern "C"

@@ -67,6 +67,67 @@ LlamaRuntime::~LlamaRuntime() {
     free_device(hidden_); free_device(qkv_); free_device(q_); free_device(gu_); free_device(logits_);
     free_device(last_hidden_); free_device(xn_); free_device(ctx_); free_device(act_);
     free_device(d_tokens_); free_device(d_pos_); free_device(d_seq_); free_device(d_out_tokens_);
+    for (TimedLaunch &t : timed_) { (void)hipEventDestroy(t.start); (void)hipEventDestroy(t.stop); }
+    for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
+}
+
+hipEvent_t LlamaRuntime::take_event() {
+    if (!event_pool_.empty()) {
+        hipEvent_t e = event_pool_.back();
+        event_pool_.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+}
+
+int LlamaRuntime::time_begin(int kernel_class) {
+    if (!timing_enabled_) return ESP_OK;
+    TimedLaunch t{kernel_class, take_event(), take_event()};
+    if (!t.start || !t.stop) return fail(ESP_ERR_OUT_OF_MEMORY, "hipEventCreate failed");
+    ESP_HIP_TRY(hipEventRecord(t.start, context().stream));
+    timed_.push_back(t);
+    return ESP_OK;
+}
+
+int LlamaRuntime::time_end() {
+    if (!timing_enabled_) return ESP_OK;
+    ESP_HIP_TRY(hipEventRecord(timed_.back().stop, context().stream));
+    return ESP_OK;
+}
+
+int LlamaRuntime::collect_kernel_times(double total_us[K_CLASS_COUNT], long launches[K_CLASS_COUNT], bool reset) {
+    ESP_HIP_TRY(hipStreamSynchronize(context().stream));
+    for (TimedLaunch &t : timed_) {
+        float ms = 0.0f;
+        ESP_HIP_TRY(hipEventElapsedTime(&ms, t.start, t.stop));
+        time_total_us_[t.kernel_class] += (double)ms * 1e3;
+        time_launches_[t.kernel_class] += 1;
+        event_pool_.push_back(t.start);
+        event_pool_.push_back(t.stop);
+    }
+    timed_.clear();
+    for (int k = 0; k < K_CLASS_COUNT; k++) {
+        if (total_us) total_us[k] = time_total_us_[k];
+        if (launches) launches[k] = time_launches_[k];
+        if (reset) { time_total_us_[k] = 0; time_launches_[k] = 0; }
+    }
+    return ESP_OK;
+}
+
+size_t LlamaRuntime::kernel_bytes(int kernel_class) const {
+    if (!finalized_ || layers_.empty()) return 0;
+    const Layer &L = layers_[0];
+    auto io = [](const DeviceMatrix &m) { return m.bytes() + (size_t)m.cols * 2 + (size_t)m.rows * 4; };
+    switch (kernel_class) {
+    case K_QKV: return io(L.wqkv);
+    case K_WO: return io(L.wo);
+    case K_GATE_UP: return io(L.w13);
+    case K_DOWN: return io(L.w2);
+    case K_HEAD: return io(lm_head_);
+    default: return 0;
+    }
 }
 
 LlamaRuntime::HostTensor *LlamaRuntime::host_slot(int layer, int slot) {
@@ -285,13 +346,16 @@ int LlamaRuntime::forward_rows(const StepRows &rows) {
     hipStream_t s = context().stream;
     const int M = rows.count, d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
     const bool kv16 = c_.kv_format == FMT_F16;
+    int rc = ESP_OK;
     ESP_HIP_TRY(launch_set_rows(rows, d_tokens_, d_pos_, d_seq_, s));
     ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, M, d, hidden_, s));
     for (Layer &L : layers_) {
         ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_att, c_.norm_eps, M, d, xn_, nullptr, s));
         GemvParams g;
         g.w = L.wqkv; g.x = xn_; g.y = qkv_; g.batch = M; g.epilogue = EPI_STORE_F32;
+        if ((rc = time_begin(K_QKV)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
+        if ((rc = time_end()) != ESP_OK) return rc;
         QkvPostArgs qa{};
         qa.qkv = qkv_; qa.q_norm = L.q_norm; qa.k_norm = L.k_norm; qa.norm_eps = c_.norm_eps;
         qa.n_head = c_.n_head; qa.n_kv_head = c_.n_kv_head; qa.head_dim = c_.head_dim; qa.max_seq = c_.max_seq;
@@ -302,15 +366,23 @@ int LlamaRuntime::forward_rows(const StepRows &rows) {
         aa.q = q_; aa.k_cache = L.k_cache; aa.v_cache = L.v_cache; aa.cache_seq_stride = qa.cache_seq_stride;
         aa.n_head = c_.n_head; aa.n_kv_head = c_.n_kv_head; aa.head_dim = c_.head_dim; aa.max_seq = c_.max_seq;
         aa.pos = d_pos_; aa.seq = d_seq_; aa.ctx_f16 = ctx_;
+        if ((rc = time_begin(K_ATTENTION)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_attention(aa, M, kv16, s));
+        if ((rc = time_end()) != ESP_OK) return rc;
         g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
+        if ((rc = time_begin(K_WO)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
+        if ((rc = time_end()) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_ffn, c_.norm_eps, M, d, xn_, nullptr, s));
         g.w = L.w13; g.x = xn_; g.y = gu_; g.residual = nullptr; g.epilogue = EPI_STORE_F32;
+        if ((rc = time_begin(K_GATE_UP)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
+        if ((rc = time_end()) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_swiglu(gu_, M, hd, act_, s));
         g.w = L.w2; g.x = act_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
+        if ((rc = time_begin(K_DOWN)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
+        if ((rc = time_end()) != ESP_OK) return rc;
     }
     (void)ad;
     return ESP_OK;
@@ -354,7 +426,10 @@ int LlamaRuntime::run_head(const float *hidden_rows, int count) {
     ESP_HIP_TRY(launch_rmsnorm(hidden_rows, final_norm_, c_.norm_eps, count, c_.d_model, xn_, nullptr, s));
     GemvParams g;
     g.w = lm_head_; g.x = xn_; g.y = logits_; g.batch = count; g.epilogue = EPI_STORE_F32;
+    int rc;
+    if ((rc = time_begin(K_HEAD)) != ESP_OK) return rc;
     ESP_HIP_TRY(launch_gemv(g, s));
+    if ((rc = time_end()) != ESP_OK) return rc;
     ESP_HIP_TRY(launch_argmax(logits_, count, c_.vocab, d_out_tokens_, nullptr, s));
     return ESP_OK;
 }

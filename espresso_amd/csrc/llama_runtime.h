@@ -61,6 +61,14 @@ class LlamaRuntime {
 
     size_t weight_bytes_per_token() const { return weight_bytes_; }
 
+    // Per-kernel timing with HIP events on the library stream.  While enabled, every launch of the
+    // kernels below is bracketed by an event pair; collect_kernel_times() synchronises and adds the
+    // elapsed times to the totals.
+    enum KernelClass { K_QKV = 0, K_WO, K_GATE_UP, K_DOWN, K_HEAD, K_ATTENTION, K_CLASS_COUNT };
+    void set_kernel_timing(bool enabled) { timing_enabled_ = enabled; }
+    int collect_kernel_times(double total_us[K_CLASS_COUNT], long launches[K_CLASS_COUNT], bool reset);
+    size_t kernel_bytes(int kernel_class) const;   // algorithmic bytes of one batch-1 launch
+
   private:
     LlamaRuntime() = default;
     struct HostTensor { int format = -1; std::vector<uint8_t> bytes; };
@@ -91,6 +99,16 @@ class LlamaRuntime {
     int *d_tokens_ = nullptr, *d_pos_ = nullptr, *d_seq_ = nullptr, *d_out_tokens_ = nullptr;
     std::vector<int> visible_;
     size_t weight_bytes_ = 0;
+
+    struct TimedLaunch { int kernel_class; hipEvent_t start, stop; };
+    bool timing_enabled_ = false;
+    std::vector<TimedLaunch> timed_;        // pending pairs
+    std::vector<hipEvent_t> event_pool_;
+    double time_total_us_[K_CLASS_COUNT] = {};
+    long time_launches_[K_CLASS_COUNT] = {};
+    hipEvent_t take_event();
+    int time_begin(int kernel_class);
+    int time_end();
 };
 
 }  // namespace esp

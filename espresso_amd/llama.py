@@ -145,3 +145,31 @@ def load_packed_weights(rt: LlamaRuntime, packed: dict, matrix_format: int, embe
             is_matrix = name in ("wq", "wk", "wv", "wo", "w1", "w2", "w3")
             rt.set_weight(l, LAYER_SLOTS[name], matrix_format if is_matrix else norm_format, data)
     rt.finalize()
+
+
+KERNEL_CLASSES = ("qkv", "wo", "gate_up", "down", "head", "attention")
+
+
+def continue_greedy(rt: LlamaRuntime, steps: int, sequence: int = 0) -> list[int]:
+    out = np.zeros(max(steps, 1), dtype=np.uint32)
+    _lib.check(rt._L.esp_llama_continue_greedy(rt._h, sequence, steps, _ptr(out)))
+    return out[:steps].tolist()
+
+
+def set_kernel_timing(rt: LlamaRuntime, enabled: bool) -> None:
+    _lib.check(rt._L.esp_llama_set_kernel_timing(rt._h, int(enabled)))
+
+
+def kernel_times(rt: LlamaRuntime, reset: bool = True) -> dict:
+    """{class: {"total_us", "launches", "bytes_per_launch", "mean_us", "gbps"}} from HIP events."""
+    n = len(KERNEL_CLASSES)
+    tot = np.zeros(n, dtype=np.float64)
+    cnt = np.zeros(n, dtype=np.int64)
+    byt = np.zeros(n, dtype=np.uint64)
+    _lib.check(rt._L.esp_llama_kernel_times(rt._h, _ptr(tot), _ptr(cnt), _ptr(byt), int(reset)))
+    out = {}
+    for i, name in enumerate(KERNEL_CLASSES):
+        mean = tot[i] / cnt[i] if cnt[i] else 0.0
+        out[name] = {"total_us": float(tot[i]), "launches": int(cnt[i]), "bytes_per_launch": int(byt[i]),
+                     "mean_us": float(mean), "gbps": float(byt[i] / mean / 1e3) if mean > 0 and byt[i] else 0.0}
+    return out

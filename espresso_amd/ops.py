@@ -84,3 +84,11 @@ class Matrix:
         mean, best = C.c_double(0), C.c_double(0)
         _lib.check(_lib.load_library().esp_gemv_time(self._h, batch, warmup, iters, rotate, C.byref(mean), C.byref(best)))
         return {"mean_us": mean.value, "best_us": best.value}
+
+
+def synth_weights(fmt: int, seed: int, std: float, elements: int) -> np.ndarray:
+    """Seeded N(0, std) weights quantised on the GPU into GGUF-layout blocks (uint8 array)."""
+    L = _lib.load_library()
+    out = np.empty(int(L.esp_format_bytes(fmt, elements)), dtype=np.uint8)
+    _lib.check(L.esp_synth_weights(fmt, C.c_uint64(seed), C.c_float(std), elements, _ptr(out)))
+    return out

@@ -171,6 +171,32 @@ int esp_llama_generate_two_token(ESPLlamaRuntime *target, ESPLlamaRuntime *draft
                                  uint32_t *out_tokens, int *out_count, ESPGenerationStats *stats,
                                  ESPTwoTokenStats *two_token_stats);
 
+/* Continues greedy decoding of `sequence` from its current state for `steps` tokens: select, then
+ * advance, per token (the body of the loop at RealModelInferenceEngine.swift:6365-6413 without the
+ * EOS test).  Fails with ESP_ERR_OUT_OF_RANGE if the context would overflow. */
+int esp_llama_continue_greedy(ESPLlamaRuntime *runtime, int sequence, int steps, uint32_t *out_tokens);
+
+/* Per-kernel timing with HIP events on the library stream.  While enabled every launch of the GEMV
+ * and attention kernels of a step is bracketed by an event pair; esp_llama_kernel_times synchronises
+ * and reports, per kernel class, the summed elapsed microseconds, the launch count and the
+ * algorithmic bytes of one batch-1 launch (packed weights + fp16 input + fp32 output). */
+#define ESP_KERNEL_QKV 0
+#define ESP_KERNEL_WO 1
+#define ESP_KERNEL_GATE_UP 2
+#define ESP_KERNEL_DOWN 3
+#define ESP_KERNEL_HEAD 4
+#define ESP_KERNEL_ATTENTION 5
+#define ESP_KERNEL_CLASS_COUNT 6
+int esp_llama_set_kernel_timing(ESPLlamaRuntime *runtime, int enabled);
+int esp_llama_kernel_times(ESPLlamaRuntime *runtime, double *total_us, int64_t *launches, uint64_t *bytes_per_launch,
+                           int reset);
+
+/* ---- seeded synthetic weights ------------------------------------------------------------- *
+ * Fills `out_blocks` (host memory, esp_format_bytes(format, elements) bytes) with N(0, std_dev) draws
+ * quantised into GGUF-layout blocks; element i of stream `seed` is the same value on every call.
+ * elements must be a multiple of 256.  Formats: F16, Q8_0, Q4_0, Q4_K. */
+int esp_synth_weights(int format, uint64_t seed, float std_dev, size_t elements, void *out_blocks);
+
 #ifdef __cplusplus
 }
 #endif
