@@ -48,10 +48,11 @@ def build_model(name: str):
     return cfg, rt, packed, time.time() - t0
 
 
-def run_gpu(name: str, steps: int, warmup: int):
+def run_gpu(name: str, steps: int, warmup: int, graph: bool = True):
     import espresso_amd.llama as ll
     w = WORKLOADS[name]
     cfg, rt, packed, build_s = build_model(name)
+    ll.set_graph_replay(rt, graph)
     if w["prompt"] + warmup + steps + 1 > cfg.max_seq:
         raise SystemExit(f"prompt {w['prompt']} + warmup {warmup} + steps {steps} does not fit context {cfg.max_seq}")
     prompt = np.random.default_rng(1000 + w["seed"]).integers(0, cfg.vocab, w["prompt"]).astype(np.uint32)
@@ -144,6 +145,9 @@ def main() -> None:
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="llama3-8b-q4k")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch kernels one at a time instead of replaying the captured per-token HIP graph "
+                         "(for rocprofv3 kernel traces)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this path is a batch-1 decode on a single MI355X; run with --gpus 1")
@@ -151,7 +155,7 @@ def main() -> None:
     ops.init()
     w = WORKLOADS[args.workload]
     steps = args.steps if args.steps is not None else w["decode"]
-    gpu = run_gpu(args.workload, steps, args.warmup)
+    gpu = run_gpu(args.workload, steps, args.warmup, graph=not args.no_graph)
     tok_s = steps / gpu["elapsed"]
     kt = gpu["kernel_times"]
     dominant = max((k for k in kt if kt[k]["bytes_per_launch"]), key=lambda k: kt[k]["total_us"])
@@ -185,7 +189,7 @@ def main() -> None:
         if other:
             ow = WORKLOADS[other]
             osteps = ow["decode"]
-            g2 = run_gpu(other, osteps, args.warmup)
+            g2 = run_gpu(other, osteps, args.warmup, graph=not args.no_graph)
             sec = {"metric": "decode tok/s bs1 (6L d768 Q8_0)", "value": osteps / g2["elapsed"], "unit": "tok/s",
                    "steps": osteps, "ms_per_step": g2["elapsed"] / osteps * 1e3, "workload": other,
                    "weight_bytes_per_token": g2["weight_bytes"],

@@ -128,3 +128,5 @@ def _declare_llama(L: C.CDLL) -> None:
     L.esp_llama_kernel_times.argtypes = [vp, vp, vp, vp, i32]
     L.esp_synth_weights.restype = i32
     L.esp_synth_weights.argtypes = [i32, C.c_uint64, C.c_float, sz, vp]
+    L.esp_llama_set_graph_replay.restype = i32
+    L.esp_llama_set_graph_replay.argtypes = [vp, i32]

@@ -118,14 +118,12 @@ int esp_llama_generate_two_token(ESPLlamaRuntime *target, ESPLlamaRuntime *draft
 int esp_llama_continue_greedy(ESPLlamaRuntime *runtime, int sequence, int steps, uint32_t *out_tokens) {
     if (!runtime) return bad_handle();
     if (!runtime->rt->finalized()) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
-    if (steps < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "steps must be >= 0");
-    for (int i = 0; i < steps; i++) {
-        uint32_t t = 0;
-        int rc = runtime->rt->select_greedy(sequence, &t);
-        if (rc != ESP_OK) return rc;
-        if (out_tokens) out_tokens[i] = t;
-        if ((rc = runtime->rt->advance(sequence, t)) != ESP_OK) return rc;
-    }
+    return runtime->rt->continue_greedy(sequence, steps, out_tokens);
+}
+
+int esp_llama_set_graph_replay(ESPLlamaRuntime *runtime, int enabled) {
+    if (!runtime) return bad_handle();
+    runtime->rt->set_use_graph(enabled != 0);
     return ESP_OK;
 }
 

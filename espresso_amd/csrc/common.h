@@ -50,6 +50,20 @@ struct DeviceMatrix {
 enum Epilogue : int {
     EPI_STORE_F32 = 0,     // y[b][r] = acc
     EPI_ADD_RESIDUAL = 1,  // y[b][r] = residual[b][r] + acc
+    EPI_SWIGLU_F16 = 2,    // rows interleaved (gate_i, up_i): out_f16[b][i] = fp16(silu(gate_i) * up_i)
+    EPI_QKV_ROPE = 3,      // fused q|k|v rows: RoPE, q -> q_out, k/v -> KV caches
+};
+
+// Destination of the fused q|k|v GEMV (EPI_QKV_ROPE).  The matrix rows are q and k as RoPE pairs
+// (j, j + head_dim/2) side by side, then v in natural order.
+struct QkvEpilogue {
+    int n_head = 0, n_kv_head = 0, head_dim = 0, max_seq = 0;
+    const float *rope_cos = nullptr, *rope_sin = nullptr;  // [max_seq][head_dim/2]
+    const int *pos = nullptr, *seq = nullptr;              // [batch]
+    float *q_out = nullptr;                                // [batch][attnDim]
+    void *k_cache = nullptr, *v_cache = nullptr;           // this layer: [seq][max_seq][kvDim]
+    size_t cache_seq_stride = 0;
+    int kv_f16 = 0;
 };
 
 struct GemvParams {
@@ -57,6 +71,8 @@ struct GemvParams {
     const uint16_t *x = nullptr;  // fp16 activations [batch][cols]
     float *y = nullptr;           // fp32 out [batch][rows]
     const float *residual = nullptr;
+    uint16_t *out_f16 = nullptr;  // EPI_SWIGLU_F16: [batch][rows/2]
+    QkvEpilogue qkv;              // EPI_QKV_ROPE
     int batch = 1;
     int epilogue = EPI_STORE_F32;
 };

@@ -23,6 +23,19 @@ int generate_greedy(LlamaRuntime &rt, const uint32_t *prompt, int prompt_count, 
 
     auto t_start = Clock::now(), t_emit = t_start;
     int all = prompt_count;
+    if (c.eos_token < 0 && eff > 1) {
+        // No stop token: the first eff-1 tokens need no host decision, so they run as graph replays with
+        // one synchronisation; the last token is selected but not advanced, as in the loop below.
+        out->resize(eff - 1);
+        if ((rc = rt.continue_greedy(0, eff - 1, out->data())) != ESP_OK) return rc;
+        all += eff - 1;
+        if (timing) {
+            const double per_token = ms_since(t_start) / (eff - 1);
+            timing->first_token_latency_ms = per_token;
+            timing->token_latencies_ms.assign(eff - 1, per_token);   // one measurement for the whole run
+        }
+        t_emit = Clock::now();
+    }
     while ((int)out->size() < eff) {
         uint32_t next = 0;
         if ((rc = rt.select_greedy(0, &next)) != ESP_OK) return rc;

@@ -27,7 +27,7 @@ struct QkvPostArgs {
     const int *pos;         // [rows]
     const int *seq;         // [rows]
     float *q_out;           // [rows][attnDim]
-    void *k_cache;          // this layer: [seq][kvDim][max_seq]
+    void *k_cache;          // this layer: [seq][max_seq][kvDim]
     void *v_cache;          // this layer: [seq][max_seq][kvDim]
     size_t cache_seq_stride;  // elements per sequence (kvDim * max_seq)
 };
@@ -51,6 +51,9 @@ hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipSt
 hipError_t launch_swiglu(const float *gu, int rows, int hidden, uint16_t *act_f16, hipStream_t s);
 hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_token, float *out_value, hipStream_t s);
 hipError_t launch_set_rows(const StepRows &rows, int *tokens, int *pos, int *seq, hipStream_t s);
+hipError_t launch_greedy_feed(const int *next_token, int seq, int *visible, int *tokens, int *pos, int *seqs, int *log,
+                              int *log_count, int log_capacity, hipStream_t s);
+hipError_t launch_set_ints(int *dst0, int v0, int *dst1, int v1, hipStream_t s);
 hipError_t launch_copy_rows(const float *src, float *dst, int rows, int d, hipStream_t s);
 
 }  // namespace esp

@@ -65,12 +65,39 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(const float *x, const f
     __shared__ float scratch[16];
     const int m = blockIdx.x;
     const float *xr = x + (size_t)m * d;
-    float s = 0.0f;
-    for (int i = threadIdx.x; i < d; i += kBlock) s += xr[i] * xr[i];
-    const float sum_sq = block_sum(s, scratch);
-    const float inv = 1.0f / sqrtf(sum_sq / (float)d + eps);
-    for (int i = threadIdx.x; i < d; i += kBlock)
-        out_f16[(size_t)m * d + i] = to_half_bits(__fmul_rn(__fmul_rn(xr[i], inv), w[i]));
+    constexpr int kVec = 8;  // float4 per thread held in registers: rows up to 8192 wide in one pass
+    if (d % 4 == 0 && d <= kVec * 4 * kBlock) {
+        // every load is issued before the first use, so the row costs one memory round trip
+        const float4 *x4 = reinterpret_cast<const float4 *>(xr), *w4 = reinterpret_cast<const float4 *>(w);
+        const int n4 = d / 4;
+        float4 v[kVec], g[kVec];
+#pragma unroll
+        for (int k = 0; k < kVec; k++) {
+            const int i = threadIdx.x + k * kBlock;
+            v[k] = i < n4 ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            g[k] = i < n4 ? w4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kVec; k++) s += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+        const float inv = 1.0f / sqrtf(block_sum(s, scratch) / (float)d + eps);
+#pragma unroll
+        for (int k = 0; k < kVec; k++) {
+            const int i = threadIdx.x + k * kBlock;
+            if (i < n4) {
+                uint2 o;
+                o.x = to_half_bits(__fmul_rn(__fmul_rn(v[k].x, inv), g[k].x)) | ((uint32_t)to_half_bits(__fmul_rn(__fmul_rn(v[k].y, inv), g[k].y)) << 16);
+                o.y = to_half_bits(__fmul_rn(__fmul_rn(v[k].z, inv), g[k].z)) | ((uint32_t)to_half_bits(__fmul_rn(__fmul_rn(v[k].w, inv), g[k].w)) << 16);
+                reinterpret_cast<uint2 *>(out_f16 + (size_t)m * d)[i] = o;
+            }
+        }
+    } else {
+        float s = 0.0f;
+        for (int i = threadIdx.x; i < d; i += kBlock) s += xr[i] * xr[i];
+        const float inv = 1.0f / sqrtf(block_sum(s, scratch) / (float)d + eps);
+        for (int i = threadIdx.x; i < d; i += kBlock)
+            out_f16[(size_t)m * d + i] = to_half_bits(__fmul_rn(__fmul_rn(xr[i], inv), w[i]));
+    }
     if (argmax_cells && threadIdx.x == 0) argmax_cells[m] = 0ull;
 }
 
@@ -111,9 +138,9 @@ __global__ void qkv_post_kernel(QkvPostArgs a) {
             q[j] = r0;
             q[j + half] = r1;
         } else {
-            // K cache is channel-major [kvDim][maxSeq]
-            const size_t c0 = seq_base + ((size_t)h * a.head_dim + j) * a.max_seq + pos;
-            const size_t c1 = seq_base + ((size_t)h * a.head_dim + j + half) * a.max_seq + pos;
+            // K cache is token-major [maxSeq][kvDim], like V
+            const size_t c0 = seq_base + (size_t)pos * kd + (size_t)h * a.head_dim + j;
+            const size_t c1 = c0 + half;
             if (KV_F16) {
                 reinterpret_cast<uint16_t *>(a.k_cache)[c0] = to_half_bits(r0);
                 reinterpret_cast<uint16_t *>(a.k_cache)[c1] = to_half_bits(r1);
@@ -134,9 +161,10 @@ __global__ void qkv_post_kernel(QkvPostArgs a) {
     }
 }
 
-// Single-query attention over the visible prefix of one sequence's KV cache (:6774-6823).
-// One workgroup per (head, row).  Scores use the reference's exact per-token sum (dims ascending,
-// separate multiply and add); the softmax sums and the value sums run in parallel order.
+// Single-query attention over the visible prefix of one sequence's KV cache (:6774-6823): the
+// general kernel, one workgroup per (head, row), any head size.  Scores use the reference's exact
+// per-token sum (dims ascending, separate multiply and add); the softmax sums and the value sums
+// run in parallel order.
 template <bool KV_F16>
 __global__ __launch_bounds__(kBlock) void attention_decode_kernel(AttentionArgs a) {
     extern __shared__ float smem[];
@@ -157,10 +185,10 @@ __global__ __launch_bounds__(kBlock) void attention_decode_kernel(AttentionArgs 
     float local_max = -INFINITY;
     for (int t = threadIdx.x; t < visible; t += kBlock) {
         float dot = 0.0f;
-        const size_t kbase = seq_base + (size_t)kvh * hd * a.max_seq + t;
+        const size_t kbase = seq_base + (size_t)t * kd + (size_t)kvh * hd;
         for (int dch = 0; dch < hd; dch++) {
-            const float kv = KV_F16 ? from_half_bits(reinterpret_cast<const uint16_t *>(a.k_cache)[kbase + (size_t)dch * a.max_seq])
-                                    : reinterpret_cast<const float *>(a.k_cache)[kbase + (size_t)dch * a.max_seq];
+            const float kv = KV_F16 ? from_half_bits(reinterpret_cast<const uint16_t *>(a.k_cache)[kbase + dch])
+                                    : reinterpret_cast<const float *>(a.k_cache)[kbase + dch];
             dot = __fadd_rn(dot, __fmul_rn(q_s[dch], kv));
         }
         const float sc = __fmul_rn(dot, scale);
@@ -201,6 +229,180 @@ __global__ __launch_bounds__(kBlock) void attention_decode_kernel(AttentionArgs 
         }
         __syncthreads();
     }
+}
+
+
+// Single-query attention, grouped-query form: one workgroup of 16 wavefronts per (KV head, row)
+// serves the G query heads that share the KV head, so K and V are read once.  Both caches are
+// token-major; a token's head vector is contiguous (HD fp16 = 256 bytes at HD 128).
+//   scores: HD/16 lanes per token, 16 dims (two 128-bit loads) per lane, partial dots reduced over
+//           those lanes; 64/(HD/16) tokens per wavefront pass;
+//   values: HD/8 lanes per token, 8 dims (one 128-bit load) per lane, fp32 accumulators per query
+//           head, reduced over the token slots of the wavefront and then over the 16 wavefronts.
+template <int HD, int G, bool KV_F16>
+__global__ __launch_bounds__(1024) void attention_gqa_kernel(AttentionArgs a) {
+    extern __shared__ float smem[];
+    float *sc = smem;                                  // [G][max_seq] scores, then probabilities
+    float *part = smem + (size_t)G * a.max_seq;        // [16][G][HD] per-wavefront value sums
+    __shared__ float red[16 * G];
+    constexpr int LPT = HD / 16, TPI = 64 / LPT;       // score phase: lanes per token, tokens per pass
+    constexpr int LPV = HD / 8, TPV = 64 / LPV;        // value phase
+    const int kvh = blockIdx.x, m = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int visible = a.pos[m] + 1;
+    const int kd = a.n_kv_head * HD;
+    const size_t seq_base = (size_t)a.seq[m] * a.cache_seq_stride;
+    const float scale = 1.0f / sqrtf((float)HD);
+
+    {   // ---- scores ----
+        const int seg = (lane % LPT) * 16;
+        float q[G][16];
+#pragma unroll
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) q[g][i] = a.q[(size_t)m * a.n_head * HD + (size_t)(kvh * G + g) * HD + seg + i];
+        for (int t0 = wave * TPI; t0 < visible; t0 += 16 * TPI) {
+            const int t = t0 + lane / LPT;
+            const bool valid = t < visible;
+            const size_t off = seq_base + (size_t)(valid ? t : 0) * kd + (size_t)kvh * HD + seg;
+            float k[16];
+            if (KV_F16) {
+                const uint4 *p = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.k_cache) + off);
+                const uint4 v0 = p[0], v1 = p[1];
+                const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) { k[2 * i] = from_half_bits((uint16_t)(w[i] & 0xFFFFu)); k[2 * i + 1] = from_half_bits((uint16_t)(w[i] >> 16)); }
+            } else {
+                const float4 *p = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(a.k_cache) + off);
+#pragma unroll
+                for (int i = 0; i < 4; i++) { const float4 v = p[i]; k[4 * i] = v.x; k[4 * i + 1] = v.y; k[4 * i + 2] = v.z; k[4 * i + 3] = v.w; }
+            }
+            float dot[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                float d = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 16; i++) d += q[g][i] * k[i];
+#pragma unroll
+                for (int o = LPT / 2; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);
+                dot[g] = d;
+            }
+            if (valid && lane % LPT == 0) {
+#pragma unroll
+                for (int g = 0; g < G; g++) sc[(size_t)g * a.max_seq + t] = dot[g] * scale;
+            }
+        }
+    }
+    __syncthreads();
+    // ---- softmax over the visible tokens, per query head ----
+    float inv_denom[G];
+    {
+        float mx[G], sm[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float v = -INFINITY;
+            for (int t = tid; t < visible; t += 1024) v = fmaxf(v, sc[(size_t)g * a.max_seq + t]);
+            v = wave_max_f(v);
+            if (lane == 0) red[wave * G + g] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float v = red[g];
+            for (int w = 1; w < 16; w++) v = fmaxf(v, red[w * G + g]);
+            mx[g] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float s = 0.0f;
+            for (int t = tid; t < visible; t += 1024) {
+                const float e = expf(sc[(size_t)g * a.max_seq + t] - mx[g]);
+                sc[(size_t)g * a.max_seq + t] = e;
+                s += e;
+            }
+            s = wave_sum_f(s);
+            if (lane == 0) red[wave * G + g] = s;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float s = 0.0f;
+            for (int w = 0; w < 16; w++) s += red[w * G + g];
+            sm[g] = s;
+            inv_denom[g] = s > 0.0f ? 1.0f / s : 0.0f;
+        }
+        (void)sm;
+    }
+    // ---- values ----
+    {
+        const int seg = (lane % LPV) * 8;
+        float acc[G][8];
+#pragma unroll
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[g][i] = 0.0f;
+        for (int t0 = wave * TPV; t0 < visible; t0 += 16 * TPV) {
+            const int t = t0 + lane / LPV;
+            const bool valid = t < visible;
+            const size_t off = seq_base + (size_t)(valid ? t : 0) * kd + (size_t)kvh * HD + seg;
+            float v[8];
+            if (KV_F16) {
+                const uint4 r = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.v_cache) + off);
+                const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) { v[2 * i] = from_half_bits((uint16_t)(w[i] & 0xFFFFu)); v[2 * i + 1] = from_half_bits((uint16_t)(w[i] >> 16)); }
+            } else {
+                const float4 *p = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(a.v_cache) + off);
+                const float4 r0 = p[0], r1 = p[1];
+                v[0] = r0.x; v[1] = r0.y; v[2] = r0.z; v[3] = r0.w; v[4] = r1.x; v[5] = r1.y; v[6] = r1.z; v[7] = r1.w;
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float p = valid ? sc[(size_t)g * a.max_seq + t] * inv_denom[g] : 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[g][i] += p * v[i];
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float x = acc[g][i];
+#pragma unroll
+                for (int o = LPV; o < 64; o <<= 1) x += __shfl_xor(x, o, 64);
+                if (lane < LPV) part[((size_t)wave * G + g) * HD + seg + i] = x;
+            }
+    }
+    __syncthreads();
+    for (int i = tid; i < G * HD; i += 1024) {
+        float total = 0.0f;
+        for (int w = 0; w < 16; w++) total += part[(size_t)w * G * HD + i];
+        const int g = i / HD, dch = i % HD;
+        a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)(kvh * G + g) * HD + dch] = to_half_bits(total);
+    }
+}
+
+template <int HD, int G>
+hipError_t launch_attention_gqa(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
+    const size_t lds = ((size_t)G * a.max_seq + (size_t)16 * G * HD) * sizeof(float);
+    dim3 grid(a.n_kv_head, rows);
+    if (kv_f16) {
+        auto kernel = attention_gqa_kernel<HD, G, true>;
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        hipLaunchKernelGGL(kernel, grid, dim3(1024), lds, s, a);
+    } else {
+        auto kernel = attention_gqa_kernel<HD, G, false>;
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        hipLaunchKernelGGL(kernel, grid, dim3(1024), lds, s, a);
+    }
+    return hipGetLastError();
 }
 
 // act[m][i] = fp16( silu_tanh(gate) * up ), gate/up interleaved in `gu` as (g0,u0,g1,u1,...)   (:6825-6827, :6337)
@@ -252,6 +454,29 @@ __global__ void set_rows_kernel(StepRows rows, int *tokens, int *pos, int *seq) 
     }
 }
 
+// Device-side bookkeeping of one greedy step inside a captured graph: the token chosen by the head
+// becomes row 0 of the next trunk pass at the sequence's visible position, is appended to the token
+// log, and the visible length grows by one.
+__global__ void greedy_feed_kernel(const int *next_token, int seq, int *visible, int *tokens, int *pos, int *seqs,
+                                   int *log, int *log_count, int log_capacity) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const int t = *next_token;
+    tokens[0] = t;
+    pos[0] = visible[seq];
+    seqs[0] = seq;
+    const int n = *log_count;
+    if (n < log_capacity) log[n] = t;
+    *log_count = n + 1;
+    visible[seq] += 1;
+}
+
+__global__ void set_ints_kernel(int *dst0, int v0, int *dst1, int v1) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        if (dst0) *dst0 = v0;
+        if (dst1) *dst1 = v1;
+    }
+}
+
 // hidden[dst] = hidden[src] rows of d floats (keeps the last hidden state of a sequence)
 __global__ void copy_rows_kernel(const float *src, float *dst, int d) {
     const int m = blockIdx.y;
@@ -282,6 +507,20 @@ hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStrea
 }
 
 hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
+    // grouped-query kernel for the common head shapes; everything else takes the general kernel
+    const int group = a.n_head / a.n_kv_head;
+    const size_t fast_lds = ((size_t)group * a.max_seq + (size_t)16 * group * a.head_dim) * sizeof(float);
+    if (a.n_head % a.n_kv_head == 0 && fast_lds <= 150 * 1024) {
+        if (a.head_dim == 128) {
+            if (group == 1) return launch_attention_gqa<128, 1>(a, rows, kv_f16, s);
+            if (group == 2) return launch_attention_gqa<128, 2>(a, rows, kv_f16, s);
+            if (group == 4) return launch_attention_gqa<128, 4>(a, rows, kv_f16, s);
+        } else if (a.head_dim == 64) {
+            if (group == 1) return launch_attention_gqa<64, 1>(a, rows, kv_f16, s);
+            if (group == 2) return launch_attention_gqa<64, 2>(a, rows, kv_f16, s);
+            if (group == 4) return launch_attention_gqa<64, 4>(a, rows, kv_f16, s);
+        }
+    }
     if (a.head_dim > kBlock && a.head_dim % kBlock != 0) return hipErrorInvalidValue;
     if (a.head_dim < kBlock && kBlock % a.head_dim != 0) return hipErrorInvalidValue;
     const size_t lds = ((size_t)a.head_dim + a.max_seq + kBlock) * sizeof(float);
@@ -304,6 +543,18 @@ hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_toke
 
 hipError_t launch_set_rows(const StepRows &rows, int *tokens, int *pos, int *seq, hipStream_t s) {
     hipLaunchKernelGGL(set_rows_kernel, dim3(1), dim3(64), 0, s, rows, tokens, pos, seq);
+    return hipGetLastError();
+}
+
+hipError_t launch_greedy_feed(const int *next_token, int seq, int *visible, int *tokens, int *pos, int *seqs, int *log,
+                              int *log_count, int log_capacity, hipStream_t s) {
+    hipLaunchKernelGGL(greedy_feed_kernel, dim3(1), dim3(64), 0, s, next_token, seq, visible, tokens, pos, seqs, log, log_count,
+                       log_capacity);
+    return hipGetLastError();
+}
+
+hipError_t launch_set_ints(int *dst0, int v0, int *dst1, int v1, hipStream_t s) {
+    hipLaunchKernelGGL(set_ints_kernel, dim3(1), dim3(64), 0, s, dst0, v0, dst1, v1);
     return hipGetLastError();
 }
 

@@ -103,6 +103,8 @@ template <>
 struct Traits<FMT_F16> { static constexpr int kItemElems = 8; static constexpr bool kPermuteX = false; static constexpr bool kXSums = false; };
 
 struct KernelArgs {
+    QkvEpilogue qkv;
+    uint16_t *out_f16;
     const uint8_t *qs;
     const uint16_t *scales;
     size_t qs_row_bytes;
@@ -112,6 +114,86 @@ struct KernelArgs {
     const float *residual;
     int epilogue;
 };
+
+// What a wavefront does with the two row sums (rows 2p and 2p+1) of each batch column.
+template <int B>
+__device__ __forceinline__ void pair_epilogue(const KernelArgs &a, int pair, const float va[B], const float vb[B]) {
+    const int r0 = 2 * pair, r1 = 2 * pair + 1;
+    if (a.epilogue == EPI_SWIGLU_F16) {
+        // rows are (gate_i, up_i): act_i = silu_tanh(gate) * up, rounded to fp16 for the next GEMV
+        // (RealModelInferenceEngine.swift:6825-6827, :6337)
+        if (r1 < a.rows) {
+#pragma unroll
+            for (int b = 0; b < B; b++) {
+                const float hg = __fmul_rn(0.5f, va[b]);
+                const float silu = __fmul_rn(hg, __fadd_rn(1.0f, tanhf(hg)));
+                a.out_f16[(size_t)b * (a.rows / 2) + pair] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(silu, vb[b]));
+            }
+        }
+        return;
+    }
+    if (a.epilogue == EPI_QKV_ROPE) {
+        // rows of the fused q|k|v matrix: q and k as RoPE pairs (j, j + half), v in natural order.
+        // Half-split RoPE from the host-built table (:6745-6772), then q -> q_out, k/v -> caches at
+        // (seq, pos), both token-major (:6297-6300).
+        const QkvEpilogue &q = a.qkv;
+        const int half = q.head_dim / 2, ad = q.n_head * q.head_dim, kd = q.n_kv_head * q.head_dim;
+        if (r1 >= a.rows) return;
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+            const int pos = q.pos[b];
+            const size_t seq_base = (size_t)q.seq[b] * q.cache_seq_stride;
+            if (r0 < ad + kd) {
+                const bool is_q = r0 < ad;
+                const int pr = is_q ? pair : pair - ad / 2;
+                const int h = pr / half, j = pr - h * half;
+                const float c = q.rope_cos[(size_t)pos * half + j], sn = q.rope_sin[(size_t)pos * half + j];
+                const float o0 = __fsub_rn(__fmul_rn(va[b], c), __fmul_rn(vb[b], sn));
+                const float o1 = __fadd_rn(__fmul_rn(va[b], sn), __fmul_rn(vb[b], c));
+                if (is_q) {
+                    float *dst = q.q_out + (size_t)b * ad + (size_t)h * q.head_dim + j;
+                    dst[0] = o0;
+                    dst[half] = o1;
+                } else {
+                    const size_t o = seq_base + (size_t)pos * kd + (size_t)h * q.head_dim + j;
+                    if (q.kv_f16) {
+                        uint16_t *kc = reinterpret_cast<uint16_t *>(q.k_cache);
+                        kc[o] = __builtin_bit_cast(uint16_t, (_Float16)o0);
+                        kc[o + half] = __builtin_bit_cast(uint16_t, (_Float16)o1);
+                    } else {
+                        float *kc = reinterpret_cast<float *>(q.k_cache);
+                        kc[o] = o0;
+                        kc[o + half] = o1;
+                    }
+                }
+            } else {
+                const size_t o = seq_base + (size_t)pos * kd + (size_t)(r0 - ad - kd);
+                if (q.kv_f16) {
+                    uint16_t *vc = reinterpret_cast<uint16_t *>(q.v_cache);
+                    vc[o] = __builtin_bit_cast(uint16_t, (_Float16)va[b]);
+                    vc[o + 1] = __builtin_bit_cast(uint16_t, (_Float16)vb[b]);
+                } else {
+                    float *vc = reinterpret_cast<float *>(q.v_cache);
+                    vc[o] = va[b];
+                    vc[o + 1] = vb[b];
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int b = 0; b < B; b++) {
+        if (r0 < a.rows) {
+            const size_t o = (size_t)b * a.rows + r0;
+            a.y[o] = a.epilogue == EPI_ADD_RESIDUAL ? a.residual[o] + va[b] : va[b];
+        }
+        if (r1 < a.rows) {
+            const size_t o = (size_t)b * a.rows + r1;
+            a.y[o] = a.epilogue == EPI_ADD_RESIDUAL ? a.residual[o] + vb[b] : vb[b];
+        }
+    }
+}
+
 
 template <int FMT, int B, int R>
 __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
@@ -249,19 +331,12 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
 #pragma unroll
         for (int b = 0; b < B; b++) acc[r][b] = wave_sum(acc[r][b]);
 
+    static_assert(R == 2, "the epilogues work on row pairs");
     if (lane == 0) {
+        float va[B], vb[B];
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const int row = row0 + r;
-            if (row >= a.rows) break;
-#pragma unroll
-            for (int b = 0; b < B; b++) {
-                const size_t o = (size_t)b * a.rows + row;
-                float v = acc[r][b];
-                if (a.epilogue == EPI_ADD_RESIDUAL) v = a.residual[o] + v;
-                a.y[o] = v;
-            }
-        }
+        for (int b = 0; b < B; b++) { va[b] = acc[0][b]; vb[b] = acc[1][b]; }
+        pair_epilogue<B>(a, row0 / 2, va, vb);
     }
 }
 
@@ -271,8 +346,10 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
 // block's 16-byte header (d, dmin, twelve scale bytes; the four lanes of a block read the same
 // 16 bytes).  A wavefront owns two consecutive rows and walks their items as one flat range, so
 // every lane is busy whenever cols is a multiple of 2048 (4096 -> 2 passes, 14336 -> 7 passes).
-// All loads of the first pass are issued before the activations are staged, and the next pass is
-// loaded while the current one is computed.
+// Weight loads run two passes ahead of the arithmetic and the first ones are issued before the
+// activations are staged.  Because rows hold a multiple of four items, a lane keeps the same chunk
+// index c = lane & 3 for the whole kernel, so everything the 6-bit scale unpacking needs besides
+// the header itself (shift counts, masks, which header word to read) is computed once.
 //
 // Nibbles are turned into fp16 with the exponent trick at offset 64: a nibble placed in mantissa
 // bits 4..7 under exponent 0x5400 reads as 64 + n exactly.  v_dot2_f32_f16 then accumulates
@@ -282,26 +359,80 @@ struct Q4KItem {
     uint4 q0, q1, hdr;
 };
 
-template <int B>
+struct Q4KLane {   // per-lane constants of the scale unpacking
+    bool upper;    // sub-blocks 4..7: six-bit values are split over two header words
+    u32 sh_sc, sh_min, sh_top, mask_low, mask_top;
+};
+
+template <int B, int XSTRIDE>
+__device__ __forceinline__ void q4k_item_dots(const Q4KItem &it, const Q4KLane &L, const uint4 *xs4, const float *xsum, int i,
+                                              int xstride_rt, int cols, float v[B]) {
+    const int xstride = XSTRIDE ? XSTRIDE : xstride_rt;
+    // 6-bit (scale, min) of sub-blocks 2c and 2c+1, two at a time in the low 16 bits
+    const u32 src_sc = L.upper ? it.hdr.w : it.hdr.y, src_min = L.upper ? it.hdr.w : it.hdr.z;
+    const u32 scp = ((src_sc >> L.sh_sc) & L.mask_low) | ((it.hdr.y >> L.sh_top) & L.mask_top);
+    const u32 mp = ((src_min >> L.sh_min) & L.mask_low) | ((it.hdr.z >> L.sh_top) & L.mask_top);
+    const float sc_lo = (float)(scp & 0xFFu), sc_hi = (float)((scp >> 8) & 0xFFu);
+    const float m_lo = (float)(mp & 0xFFu), m_hi = (float)((mp >> 8) & 0xFFu);
+    const float d = half_bits_to_float(it.hdr.x & 0xFFFFu), dmin = half_bits_to_float(it.hdr.x >> 16);
+#pragma unroll
+    for (int b = 0; b < B; b++) {
+        const uint4 *px = xs4 + (size_t)b * 8 * xstride + i;
+        float raw_lo = 0.0f, raw_hi = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const u32 w = dword_of(k < 4 ? it.q0 : it.q1, k & 3);
+            const uint4 vl = px[(k >> 1) * xstride], vh = px[(4 + (k >> 1)) * xstride];
+            const h2 xl02 = as_h2(dword_of(vl, (k & 1) * 2)), xl13 = as_h2(dword_of(vl, (k & 1) * 2 + 1));
+            const h2 xh02 = as_h2(dword_of(vh, (k & 1) * 2)), xh13 = as_h2(dword_of(vh, (k & 1) * 2 + 1));
+            const h2 l02 = as_h2(and_or(w << 4, 0x00F000F0u, 0x54005400u));
+            const h2 l13 = as_h2(and_or(w >> 4, 0x00F000F0u, 0x54005400u));
+            const h2 h02 = as_h2(and_or(w, 0x00F000F0u, 0x54005400u));
+            const h2 h13 = as_h2(and_or(w >> 8, 0x00F000F0u, 0x54005400u));
+            raw_lo = fdot2(l02, xl02, raw_lo);
+            raw_lo = fdot2(l13, xl13, raw_lo);
+            raw_hi = fdot2(h02, xh02, raw_hi);
+            raw_hi = fdot2(h13, xh13, raw_hi);
+        }
+        const float2 xsp = *reinterpret_cast<const float2 *>(xsum + (size_t)b * (cols >> 5) + 2 * i);
+        const float nx_lo = raw_lo - 64.0f * xsp.x, nx_hi = raw_hi - 64.0f * xsp.y;
+        v[b] = d * (sc_lo * nx_lo + sc_hi * nx_hi) - dmin * (m_lo * xsp.x + m_hi * xsp.y);
+    }
+}
+
+// IPR: items (64-weight chunks) per row when known at compile time, 0 = read from the arguments.
+template <int B, int IPR>
 __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a) {
     extern __shared__ uint4 smem_raw[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int cols = a.cols;
-    const int ipr = cols >> 6;       // items per row
-    const int xstride = ipr | 1;     // 16-byte slots between consecutive k of one item
-    uint16_t *xs = reinterpret_cast<uint16_t *>(smem_raw);                       // [B][8][xstride] x 8 fp16, (x0,x2,x1,x3) order
+    const int cols = IPR ? IPR * 64 : a.cols;
+    const int ipr = IPR ? IPR : cols >> 6;   // items per row
+    const int xstride = ipr | 1;             // 16-byte slots between consecutive k of one item
+    constexpr int XSTRIDE = IPR ? (IPR | 1) : 0;
+    const int total = 2 * ipr;               // items of the wavefront's row pair
+    uint4 *xs4 = smem_raw;                                                        // [B][8][xstride] x 8 fp16, (x0,x2,x1,x3) order
     float *xsum = reinterpret_cast<float *>(smem_raw + (size_t)B * 8 * xstride);  // [B][cols/32] sub-block sums
-    const int total = 2 * ipr;       // items of the wavefront's row pair
     const int pair = blockIdx.x * kWaves + wave;
     const int row_a = 2 * pair < a.rows ? 2 * pair : a.rows - 1;          // clamped: loads stay inside the matrix
     const int row_b = 2 * pair + 1 < a.rows ? 2 * pair + 1 : a.rows - 1;
     const uint8_t *base_a = a.qs + (size_t)row_a * a.qs_row_bytes;
     const uint8_t *base_b = a.qs + (size_t)row_b * a.qs_row_bytes;
 
+    Q4KLane L;
+    {
+        const int c = lane & 3, sh = (c & 1) * 16;
+        L.upper = c >= 2;
+        L.sh_sc = sh;
+        L.sh_min = L.upper ? sh + 4 : sh;
+        L.sh_top = sh + 2;
+        L.mask_low = L.upper ? 0x0F0Fu : 0x3F3Fu;
+        L.mask_top = L.upper ? 0x3030u : 0u;
+    }
+
     auto load_item = [&](int t) {
         Q4KItem it;
         const int tt = t < total ? t : 0;
-        const int second = tt >= ipr;
+        const bool second = tt >= ipr;
         const int i = tt - (second ? ipr : 0);
         const uint8_t *bp = (second ? base_b : base_a) + (size_t)(i >> 2) * 144;
         it.hdr = *reinterpret_cast<const uint4 *>(bp);
@@ -310,85 +441,71 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a) {
         it.q1 = q[1];
         return it;
     };
-
-    // ---- activations first (small, L2-resident), then the first pass of weights ----
-    const uint4 *xsrc = reinterpret_cast<const uint4 *>(a.x);
-    const int n16 = B * cols / 8;
-    Q4KItem cur = load_item(lane);
-    for (int i = tid; i < n16; i += kThreads) {
-        const uint4 v = xsrc[i];
-        uint4 p;
-        p.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
-        p.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
-        p.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
-        p.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
-        // LDS layout [b][k][item] with an odd item stride: lanes of a pass (consecutive items) read
-        // consecutive 16-byte slots for each k, and staging writes spread evenly over the banks.
-        {
+    auto stage_x = [&]() {
+        // activations: 128-bit loads, middle elements of each group of four swapped, written to the
+        // LDS layout [b][k][item] with an odd item stride (conflict-free for both the write and the
+        // per-k reads of consecutive items); sub-block sums of 32 alongside
+        const uint4 *xsrc = reinterpret_cast<const uint4 *>(a.x);
+        const int n16 = B * cols / 8;
+        for (int i = tid; i < n16; i += kThreads) {
+            const uint4 v = xsrc[i];
+            uint4 p;
+            p.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
+            p.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
+            p.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
+            p.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
             const int b = i / (cols / 8), g = i - b * (cols / 8);
-            reinterpret_cast<uint4 *>(xs)[(size_t)b * 8 * xstride + (g & 7) * xstride + (g >> 3)] = p;
+            xs4[(size_t)b * 8 * xstride + (g & 7) * xstride + (g >> 3)] = p;
+            float s = ((float)as_h2(v.x).x + (float)as_h2(v.x).y) + ((float)as_h2(v.y).x + (float)as_h2(v.y).y) +
+                      ((float)as_h2(v.z).x + (float)as_h2(v.z).y) + ((float)as_h2(v.w).x + (float)as_h2(v.w).y);
+            s += dpp_term<0xB1, 0xF>(s);
+            s += dpp_term<0x4E, 0xF>(s);
+            if ((lane & 3) == 0) xsum[i >> 2] = s;
         }
-        // sum of the 8 values, then of the 4 lanes that share a 32-element sub-block
-        float s = ((float)as_h2(v.x).x + (float)as_h2(v.x).y) + ((float)as_h2(v.y).x + (float)as_h2(v.y).y) +
-                  ((float)as_h2(v.z).x + (float)as_h2(v.z).y) + ((float)as_h2(v.w).x + (float)as_h2(v.w).y);
-        s += dpp_term<0xB1, 0xF>(s);
-        s += dpp_term<0x4E, 0xF>(s);
-        if ((lane & 3) == 0) xsum[i >> 2] = s;
-    }
-    __syncthreads();
+    };
 
     float acc_a[B], acc_b[B];
 #pragma unroll
     for (int b = 0; b < B; b++) acc_a[b] = acc_b[b] = 0.0f;
 
-    for (int t0 = 0; t0 < total; t0 += 64) {
-        const int t = t0 + lane;
-        Q4KItem nxt = cur;
-        if (t0 + 64 < total) nxt = load_item(t + 64);
-
+    auto consume = [&](const Q4KItem &it, int t) {
         const bool valid = t < total;
         const int tt = valid ? t : 0;
         const bool second = tt >= ipr;
         const int i = tt - (second ? ipr : 0);
-        const int c = i & 3;
-        const int e0 = (i >> 2) * 256 + c * 64;
-
-        // 6-bit (scale, min) of sub-blocks 2c and 2c+1, two at a time
-        const int sh = (c & 1) * 16;
-        const u32 s0 = cur.hdr.y >> sh, s1 = cur.hdr.z >> sh, s2 = cur.hdr.w >> sh;
-        const u32 scp = c < 2 ? (s0 & 0x3F3Fu) : ((s2 & 0x0F0Fu) | ((s0 >> 2) & 0x3030u));
-        const u32 mp = c < 2 ? (s1 & 0x3F3Fu) : (((s2 >> 4) & 0x0F0Fu) | ((s1 >> 2) & 0x3030u));
-        const float sc_lo = (float)(scp & 0xFFu), sc_hi = (float)(scp >> 8);
-        const float m_lo = (float)(mp & 0xFFu), m_hi = (float)(mp >> 8);
-        const float d = half_bits_to_float(cur.hdr.x & 0xFFFFu), dmin = half_bits_to_float(cur.hdr.x >> 16);
-
+        float v[B];
+        q4k_item_dots<B, XSTRIDE>(it, L, xs4, xsum, i, xstride, cols, v);
 #pragma unroll
         for (int b = 0; b < B; b++) {
-            const uint4 *px = reinterpret_cast<const uint4 *>(xs) + (size_t)b * 8 * xstride + i;
-            float raw_lo = 0.0f, raw_hi = 0.0f;
-#pragma unroll
-            for (int k = 0; k < 8; k++) {
-                const u32 w = dword_of(k < 4 ? cur.q0 : cur.q1, k & 3);
-                const uint4 vl = px[(k >> 1) * xstride], vh = px[(4 + (k >> 1)) * xstride];
-                const h2 xl02 = as_h2(dword_of(vl, (k & 1) * 2)), xl13 = as_h2(dword_of(vl, (k & 1) * 2 + 1));
-                const h2 xh02 = as_h2(dword_of(vh, (k & 1) * 2)), xh13 = as_h2(dword_of(vh, (k & 1) * 2 + 1));
-                const h2 l02 = as_h2(and_or(w << 4, 0x00F000F0u, 0x54005400u));
-                const h2 l13 = as_h2(and_or(w >> 4, 0x00F000F0u, 0x54005400u));
-                const h2 h02 = as_h2(and_or(w, 0x00F000F0u, 0x54005400u));
-                const h2 h13 = as_h2(and_or(w >> 8, 0x00F000F0u, 0x54005400u));
-                raw_lo = fdot2(l02, xl02, raw_lo);
-                raw_lo = fdot2(l13, xl13, raw_lo);
-                raw_hi = fdot2(h02, xh02, raw_hi);
-                raw_hi = fdot2(h13, xh13, raw_hi);
-            }
-            const float xs_lo = xsum[b * (cols >> 5) + (e0 >> 5)], xs_hi = xsum[b * (cols >> 5) + (e0 >> 5) + 1];
-            const float nx_lo = raw_lo - 64.0f * xs_lo, nx_hi = raw_hi - 64.0f * xs_hi;
-            float v = d * (sc_lo * nx_lo + sc_hi * nx_hi) - dmin * (m_lo * xs_lo + m_hi * xs_hi);
-            v = valid ? v : 0.0f;
-            acc_a[b] += second ? 0.0f : v;
-            acc_b[b] += second ? v : 0.0f;
+            const float vv = valid ? v[b] : 0.0f;
+            acc_a[b] += second ? 0.0f : vv;
+            acc_b[b] += second ? vv : 0.0f;
         }
-        cur = nxt;
+    };
+
+    if constexpr (IPR != 0) {
+        constexpr int PASSES = (2 * IPR + 63) / 64;
+        constexpr int NBUF = PASSES < 3 ? PASSES : 3;
+        Q4KItem buf[NBUF];
+#pragma unroll
+        for (int p = 0; p < (PASSES > 2 ? 2 : PASSES); p++) buf[p] = load_item(p * 64 + lane);
+        stage_x();
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            if (PASSES > 2 && p + 2 < PASSES) buf[(p + 2) % NBUF] = load_item((p + 2) * 64 + lane);
+            consume(buf[p % NBUF], p * 64 + lane);
+        }
+    } else {
+        Q4KItem cur = load_item(lane);
+        stage_x();
+        __syncthreads();
+        for (int t0 = 0; t0 < total; t0 += 64) {
+            Q4KItem nxt = cur;
+            if (t0 + 64 < total) nxt = load_item(t0 + 64 + lane);
+            consume(cur, t0 + lane);
+            cur = nxt;
+        }
     }
 
 #pragma unroll
@@ -396,27 +513,14 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a) {
         acc_a[b] = wave_sum(acc_a[b]);
         acc_b[b] = wave_sum(acc_b[b]);
     }
-    if (lane == 0) {
-#pragma unroll
-        for (int b = 0; b < B; b++) {
-            const int r0 = 2 * pair, r1 = 2 * pair + 1;
-            if (r0 < a.rows) {
-                const size_t o = (size_t)b * a.rows + r0;
-                a.y[o] = a.epilogue == EPI_ADD_RESIDUAL ? a.residual[o] + acc_a[b] : acc_a[b];
-            }
-            if (r1 < a.rows) {
-                const size_t o = (size_t)b * a.rows + r1;
-                a.y[o] = a.epilogue == EPI_ADD_RESIDUAL ? a.residual[o] + acc_b[b] : acc_b[b];
-            }
-        }
-    }
+    if (lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
 }
 
-template <int B>
-hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
+template <int B, int IPR>
+hipError_t launch_q4k_ipr(const KernelArgs &a, hipStream_t stream) {
     const size_t lds = (size_t)B * 8 * ((a.cols / 64) | 1) * 16 + (size_t)B * (a.cols / 32) * 4;
     if (lds > 160 * 1024) return hipErrorInvalidValue;
-    auto kernel = gemv_q4k_kernel<B>;
+    auto kernel = gemv_q4k_kernel<B, IPR>;
     static size_t configured_lds = 0;
     if (lds > 48 * 1024 && lds > configured_lds) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -428,6 +532,13 @@ hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     const int grid = (pairs + kWaves - 1) / kWaves;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a);
     return hipGetLastError();
+}
+
+template <int B>
+hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
+    if (a.cols == 4096) return launch_q4k_ipr<B, 64>(a, stream);
+    if (a.cols == 14336) return launch_q4k_ipr<B, 224>(a, stream);
+    return launch_q4k_ipr<B, 0>(a, stream);
 }
 
 template <int FMT, int B, int R>
@@ -460,8 +571,16 @@ hipError_t launch_fmt(const KernelArgs &a, int batch, hipStream_t stream) {
 
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     const DeviceMatrix &w = p.w;
-    if (!w.qs || !p.x || !p.y || w.rows <= 0 || w.cols <= 0 || p.batch <= 0) return hipErrorInvalidValue;
+    if (!w.qs || !p.x || w.rows <= 0 || w.cols <= 0 || p.batch <= 0) return hipErrorInvalidValue;
+    if ((p.epilogue == EPI_STORE_F32 || p.epilogue == EPI_ADD_RESIDUAL) && !p.y) return hipErrorInvalidValue;
     if (p.epilogue == EPI_ADD_RESIDUAL && !p.residual) return hipErrorInvalidValue;
+    if (p.epilogue == EPI_SWIGLU_F16 && (!p.out_f16 || w.rows % 2 != 0)) return hipErrorInvalidValue;
+    if (p.epilogue == EPI_QKV_ROPE) {
+        const QkvEpilogue &q = p.qkv;
+        if (!q.rope_cos || !q.rope_sin || !q.pos || !q.seq || !q.q_out || !q.k_cache || !q.v_cache || q.head_dim % 2 != 0 ||
+            w.rows != (q.n_head + 2 * q.n_kv_head) * q.head_dim)
+            return hipErrorInvalidValue;
+    }
     const int block = w.format == FMT_F16 ? 8 : format_block_elems(w.format);
     if (w.cols % block != 0 || w.qs_row_bytes % 16 != 0) return hipErrorInvalidValue;
     if ((w.format == FMT_Q8_0 || w.format == FMT_Q4_0) && !w.scales) return hipErrorInvalidValue;
@@ -472,8 +591,15 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         KernelArgs a;
         a.qs = w.qs; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.rows = w.rows; a.cols = w.cols;
         a.x = p.x + (size_t)b0 * w.cols;
-        a.y = p.y + (size_t)b0 * w.rows;
+        a.y = p.y ? p.y + (size_t)b0 * w.rows : nullptr;
         a.residual = p.residual ? p.residual + (size_t)b0 * w.rows : nullptr;
+        a.out_f16 = p.out_f16 ? p.out_f16 + (size_t)b0 * (w.rows / 2) : nullptr;
+        a.qkv = p.qkv;
+        if (p.epilogue == EPI_QKV_ROPE) {
+            a.qkv.pos += b0;
+            a.qkv.seq += b0;
+            a.qkv.q_out += (size_t)b0 * p.qkv.n_head * p.qkv.head_dim;
+        }
         a.epilogue = p.epilogue;
         hipError_t e;
         switch (w.format) {

@@ -67,6 +67,8 @@ LlamaRuntime::~LlamaRuntime() {
     free_device(hidden_); free_device(qkv_); free_device(q_); free_device(gu_); free_device(logits_);
     free_device(last_hidden_); free_device(xn_); free_device(ctx_); free_device(act_);
     free_device(d_tokens_); free_device(d_pos_); free_device(d_seq_); free_device(d_out_tokens_);
+    free_device(d_visible_); free_device(d_log_); free_device(d_log_count_);
+    for (hipGraphExec_t g : step_graphs_) if (g) (void)hipGraphExecDestroy(g);
     for (TimedLaunch &t : timed_) { (void)hipEventDestroy(t.start); (void)hipEventDestroy(t.stop); }
     for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
 }
@@ -303,6 +305,10 @@ int LlamaRuntime::finalize() {
     if ((rc = device_alloc(&d_pos_, R)) != ESP_OK) return rc;
     if ((rc = device_alloc(&d_seq_, R)) != ESP_OK) return rc;
     if ((rc = device_alloc(&d_out_tokens_, R)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_visible_, (size_t)c_.max_sequences)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_log_, (size_t)c_.max_seq)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_log_count_, 1)) != ESP_OK) return rc;
+    step_graphs_.assign(c_.max_sequences, nullptr);
     finalized_ = true;
     return reset();
 }
@@ -343,43 +349,63 @@ int LlamaRuntime::forward_rows(const StepRows &rows) {
         if (rows.seq[i] < 0 || rows.seq[i] >= c_.max_sequences)
             return fail(ESP_ERR_OUT_OF_RANGE, "sequence %d of %d", rows.seq[i], c_.max_sequences);
     }
+    ESP_HIP_TRY(launch_set_rows(rows, d_tokens_, d_pos_, d_seq_, context().stream));
+    return enqueue_trunk(rows.count);
+}
+
+// The trunk over `M` rows whose (token, position, sequence) already sit in d_tokens_/d_pos_/d_seq_.
+int LlamaRuntime::enqueue_trunk(int M) {
     hipStream_t s = context().stream;
-    const int M = rows.count, d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
+    const int d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
     const bool kv16 = c_.kv_format == FMT_F16;
     int rc = ESP_OK;
-    ESP_HIP_TRY(launch_set_rows(rows, d_tokens_, d_pos_, d_seq_, s));
     ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, M, d, hidden_, s));
     for (Layer &L : layers_) {
         ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_att, c_.norm_eps, M, d, xn_, nullptr, s));
         GemvParams g;
-        g.w = L.wqkv; g.x = xn_; g.y = qkv_; g.batch = M; g.epilogue = EPI_STORE_F32;
-        if ((rc = time_begin(K_QKV)) != ESP_OK) return rc;
-        ESP_HIP_TRY(launch_gemv(g, s));
-        if ((rc = time_end()) != ESP_OK) return rc;
-        QkvPostArgs qa{};
-        qa.qkv = qkv_; qa.q_norm = L.q_norm; qa.k_norm = L.k_norm; qa.norm_eps = c_.norm_eps;
-        qa.n_head = c_.n_head; qa.n_kv_head = c_.n_kv_head; qa.head_dim = c_.head_dim; qa.max_seq = c_.max_seq;
-        qa.rope_cos = rope_cos_; qa.rope_sin = rope_sin_; qa.pos = d_pos_; qa.seq = d_seq_;
-        qa.q_out = q_; qa.k_cache = L.k_cache; qa.v_cache = L.v_cache; qa.cache_seq_stride = (size_t)kd * c_.max_seq;
-        ESP_HIP_TRY(launch_qkv_post(qa, M, kv16, s));
+        g.w = L.wqkv; g.x = xn_; g.batch = M;
+        const size_t cache_seq_stride = (size_t)kd * c_.max_seq;
+        if (L.q_norm) {
+            // per-head q/k norm needs whole heads before RoPE: plain GEMV, then the post kernel
+            g.y = qkv_; g.epilogue = EPI_STORE_F32;
+            if ((rc = time_begin(K_QKV)) != ESP_OK) return rc;
+            ESP_HIP_TRY(launch_gemv(g, s));
+            if ((rc = time_end()) != ESP_OK) return rc;
+            QkvPostArgs qa{};
+            qa.qkv = qkv_; qa.q_norm = L.q_norm; qa.k_norm = L.k_norm; qa.norm_eps = c_.norm_eps;
+            qa.n_head = c_.n_head; qa.n_kv_head = c_.n_kv_head; qa.head_dim = c_.head_dim; qa.max_seq = c_.max_seq;
+            qa.rope_cos = rope_cos_; qa.rope_sin = rope_sin_; qa.pos = d_pos_; qa.seq = d_seq_;
+            qa.q_out = q_; qa.k_cache = L.k_cache; qa.v_cache = L.v_cache; qa.cache_seq_stride = cache_seq_stride;
+            ESP_HIP_TRY(launch_qkv_post(qa, M, kv16, s));
+        } else {
+            g.epilogue = EPI_QKV_ROPE;
+            g.qkv.n_head = c_.n_head; g.qkv.n_kv_head = c_.n_kv_head; g.qkv.head_dim = c_.head_dim; g.qkv.max_seq = c_.max_seq;
+            g.qkv.rope_cos = rope_cos_; g.qkv.rope_sin = rope_sin_; g.qkv.pos = d_pos_; g.qkv.seq = d_seq_;
+            g.qkv.q_out = q_; g.qkv.k_cache = L.k_cache; g.qkv.v_cache = L.v_cache;
+            g.qkv.cache_seq_stride = cache_seq_stride; g.qkv.kv_f16 = kv16 ? 1 : 0;
+            if ((rc = time_begin(K_QKV)) != ESP_OK) return rc;
+            ESP_HIP_TRY(launch_gemv(g, s));
+            if ((rc = time_end()) != ESP_OK) return rc;
+        }
         AttentionArgs aa{};
-        aa.q = q_; aa.k_cache = L.k_cache; aa.v_cache = L.v_cache; aa.cache_seq_stride = qa.cache_seq_stride;
+        aa.q = q_; aa.k_cache = L.k_cache; aa.v_cache = L.v_cache; aa.cache_seq_stride = cache_seq_stride;
         aa.n_head = c_.n_head; aa.n_kv_head = c_.n_kv_head; aa.head_dim = c_.head_dim; aa.max_seq = c_.max_seq;
         aa.pos = d_pos_; aa.seq = d_seq_; aa.ctx_f16 = ctx_;
         if ((rc = time_begin(K_ATTENTION)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_attention(aa, M, kv16, s));
         if ((rc = time_end()) != ESP_OK) return rc;
+        g = GemvParams{};
+        g.batch = M;
         g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
         if ((rc = time_begin(K_WO)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_ffn, c_.norm_eps, M, d, xn_, nullptr, s));
-        g.w = L.w13; g.x = xn_; g.y = gu_; g.residual = nullptr; g.epilogue = EPI_STORE_F32;
+        g.w = L.w13; g.x = xn_; g.y = nullptr; g.residual = nullptr; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
         if ((rc = time_begin(K_GATE_UP)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
-        ESP_HIP_TRY(launch_swiglu(gu_, M, hd, act_, s));
-        g.w = L.w2; g.x = act_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
+        g.w = L.w2; g.x = act_; g.y = hidden_; g.residual = hidden_; g.out_f16 = nullptr; g.epilogue = EPI_ADD_RESIDUAL;
         if ((rc = time_begin(K_DOWN)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
@@ -455,6 +481,70 @@ int LlamaRuntime::head_rows(int count, uint32_t *tokens) {
     ESP_HIP_TRY(hipMemcpyAsync(t, d_out_tokens_, sizeof(int) * count, hipMemcpyDeviceToHost, context().stream));
     ESP_HIP_TRY(hipStreamSynchronize(context().stream));
     for (int i = 0; i < count; i++) tokens[i] = (uint32_t)t[i];
+    return ESP_OK;
+}
+
+// head(last hidden of seq) -> argmax -> feed row 0 -> trunk -> keep row 0, captured once per sequence.
+int LlamaRuntime::capture_step_graph(int seq) {
+    hipStream_t s = context().stream;
+    hipGraph_t graph = nullptr;
+    ESP_HIP_TRY(hipStreamSynchronize(s));
+    ESP_HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+    int rc = run_head(last_hidden_ + (size_t)seq * c_.d_model, 1);
+    if (rc == ESP_OK) {
+        hipError_t e = launch_greedy_feed(d_out_tokens_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_, d_log_count_,
+                                          c_.max_seq, s);
+        if (e != hipSuccess) rc = fail_hip(e, "greedy_feed");
+    }
+    if (rc == ESP_OK) rc = enqueue_trunk(1);
+    if (rc == ESP_OK) rc = keep_row(0, seq);
+    hipError_t e = hipStreamEndCapture(s, &graph);
+    if (rc != ESP_OK) { if (graph) (void)hipGraphDestroy(graph); return rc; }
+    if (e != hipSuccess) return fail_hip(e, "hipStreamEndCapture");
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return fail_hip(e, "hipGraphInstantiate");
+    step_graphs_[seq] = exec;
+    return ESP_OK;
+}
+
+int LlamaRuntime::continue_greedy(int seq, int steps, uint32_t *out_tokens) {
+    if (!finalized_) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+    if (seq < 0 || seq >= c_.max_sequences) return fail(ESP_ERR_OUT_OF_RANGE, "sequence %d of %d", seq, c_.max_sequences);
+    if (steps < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "steps must be >= 0");
+    if (visible_[seq] + steps > c_.max_seq)
+        return fail(ESP_ERR_OUT_OF_RANGE, "runtime position %d + %d steps exceeds context %d", visible_[seq], steps, c_.max_seq);
+    if (steps == 0) return ESP_OK;
+    hipStream_t s = context().stream;
+    int rc;
+    if (!use_graph_ || timing_enabled_) {
+        for (int i = 0; i < steps; i++) {
+            uint32_t t = 0;
+            if ((rc = select_greedy(seq, &t)) != ESP_OK) return rc;
+            if (out_tokens) out_tokens[i] = t;
+            if ((rc = advance(seq, t)) != ESP_OK) return rc;
+        }
+        return ESP_OK;
+    }
+    if (!step_graphs_[seq]) {
+        // one eager step first: it configures every kernel's LDS limit outside the capture
+        uint32_t t = 0;
+        if ((rc = select_greedy(seq, &t)) != ESP_OK) return rc;
+        if (out_tokens) out_tokens[0] = t;
+        if ((rc = advance(seq, t)) != ESP_OK) return rc;
+        if ((rc = capture_step_graph(seq)) != ESP_OK) return rc;
+        if (out_tokens) out_tokens += 1;
+        steps -= 1;
+        if (steps == 0) return ESP_OK;
+    }
+    ESP_HIP_TRY(launch_set_ints(d_visible_ + seq, visible_[seq], d_log_count_, 0, s));
+    for (int i = 0; i < steps; i++) ESP_HIP_TRY(hipGraphLaunch(step_graphs_[seq], s));
+    std::vector<int> log(steps);
+    ESP_HIP_TRY(hipMemcpyAsync(log.data(), d_log_, sizeof(int) * steps, hipMemcpyDeviceToHost, s));
+    ESP_HIP_TRY(hipStreamSynchronize(s));
+    visible_[seq] += steps;
+    if (out_tokens) for (int i = 0; i < steps; i++) out_tokens[i] = (uint32_t)log[i];
     return ESP_OK;
 }
 

@@ -56,6 +56,10 @@ class LlamaRuntime {
     int head_rows(int count, uint32_t *tokens);
     // Keep row `row` of the most recent forward_rows() as sequence `seq`'s last hidden state.
     int keep_row(int row, int seq);
+    // `steps` greedy tokens from the sequence's current state (select, then advance, per token) as
+    // replays of one captured HIP graph per token; the host synchronises once at the end.
+    int continue_greedy(int seq, int steps, uint32_t *out_tokens);
+    void set_use_graph(bool enabled) { use_graph_ = enabled; }
     int read_last_hidden(int seq, float *out);
     int read_logits(int seq, float *out);         // runs the head on the kept hidden state
 
@@ -80,6 +84,8 @@ class LlamaRuntime {
     };
     int upload_vector(const HostTensor &t, size_t count, float **out, const char *what);
     int run_head(const float *hidden_rows, int count);
+    int enqueue_trunk(int rows);
+    int capture_step_graph(int seq);
     HostTensor *host_slot(int layer, int slot);
 
     LlamaConfig c_;
@@ -99,6 +105,10 @@ class LlamaRuntime {
     int *d_tokens_ = nullptr, *d_pos_ = nullptr, *d_seq_ = nullptr, *d_out_tokens_ = nullptr;
     std::vector<int> visible_;
     size_t weight_bytes_ = 0;
+    // captured greedy step per sequence (head -> feed -> trunk -> keep), and its device-side state
+    bool use_graph_ = true;
+    std::vector<hipGraphExec_t> step_graphs_;
+    int *d_visible_ = nullptr, *d_log_ = nullptr, *d_log_count_ = nullptr;
 
     struct TimedLaunch { int kernel_class; hipEvent_t start, stop; };
     bool timing_enabled_ = false;

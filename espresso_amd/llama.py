@@ -156,6 +156,10 @@ def continue_greedy(rt: LlamaRuntime, steps: int, sequence: int = 0) -> list[int
     return out[:steps].tolist()
 
 
+def set_graph_replay(rt: LlamaRuntime, enabled: bool) -> None:
+    _lib.check(rt._L.esp_llama_set_graph_replay(rt._h, int(enabled)))
+
+
 def set_kernel_timing(rt: LlamaRuntime, enabled: bool) -> None:
     _lib.check(rt._L.esp_llama_set_kernel_timing(rt._h, int(enabled)))
 

