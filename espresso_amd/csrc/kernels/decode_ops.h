@@ -41,7 +41,10 @@ struct AttentionArgs {
     const int *pos;
     const int *seq;
     uint16_t *ctx_f16;      // [rows][attnDim]
+    // partial results of the split-prefix kernel: [rows][kvHeads][splits][group][head_dim + 2] floats
+    float *split_scratch;
 };
+constexpr int kAttentionMaxSplits = 32;
 
 hipError_t launch_embed(const void *table, bool table_is_f16, const int *tokens, int rows, int d, float *hidden, hipStream_t s);
 hipError_t launch_rmsnorm(const float *x, const float *w, float eps, int rows, int d, uint16_t *out_f16,
@@ -49,7 +52,14 @@ hipError_t launch_rmsnorm(const float *x, const float *w, float eps, int rows, i
 hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStream_t s);
 hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
 hipError_t launch_swiglu(const float *gu, int rows, int hidden, uint16_t *act_f16, hipStream_t s);
-hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_token, float *out_value, hipStream_t s);
+// Scratch of the two-launch argmax: kMaxStepRows x 128 partial (value, index) pairs.
+struct ArgmaxScratch {
+    float *part_value = nullptr;
+    int *part_index = nullptr;
+};
+constexpr int kArgmaxScratchSlots = kMaxStepRows * 128;
+hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_token, float *out_value, const ArgmaxScratch &scratch,
+                         hipStream_t s);
 hipError_t launch_set_rows(const StepRows &rows, int *tokens, int *pos, int *seq, hipStream_t s);
 hipError_t launch_greedy_feed(const int *next_token, int seq, int *visible, int *tokens, int *pos, int *seqs, int *log,
                               int *log_count, int log_capacity, hipStream_t s);

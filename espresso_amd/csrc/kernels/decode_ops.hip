@@ -45,6 +45,29 @@ __device__ __forceinline__ float block_max(float v, float *scratch) {
     return t;
 }
 
+// DPP row operations (no LDS traffic).  group_sum<N>: sum over aligned groups of N lanes (N = 8 or 16),
+// result in every lane of the group.
+template <int CTRL>
+__device__ __forceinline__ float dpp_get(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
+template <int N>
+__device__ __forceinline__ float group_sum(float v) {
+    v += dpp_get<0xB1>(v);                 // quad_perm [1,0,3,2]
+    v += dpp_get<0x4E>(v);                 // quad_perm [2,3,0,1]
+    v += dpp_get<0x141>(v);                // row_half_mirror
+    if (N == 16) v += dpp_get<0x140>(v);   // row_mirror
+    return v;
+}
+// maximum over the first lane of every group of N lanes, as a wave-uniform value
+template <int N>
+__device__ __forceinline__ float max_over_groups(float v) {
+    float m = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+#pragma unroll
+    for (int l = N; l < 64; l += N) m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l)));
+    return m;
+}
+
 __device__ __forceinline__ uint16_t to_half_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
 __device__ __forceinline__ float from_half_bits(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
 
@@ -232,176 +255,181 @@ __global__ __launch_bounds__(kBlock) void attention_decode_kernel(AttentionArgs 
 }
 
 
-// Single-query attention, grouped-query form: one workgroup of 16 wavefronts per (KV head, row)
-// serves the G query heads that share the KV head, so K and V are read once.  Both caches are
-// token-major; a token's head vector is contiguous (HD fp16 = 256 bytes at HD 128).
-//   scores: HD/16 lanes per token, 16 dims (two 128-bit loads) per lane, partial dots reduced over
-//           those lanes; 64/(HD/16) tokens per wavefront pass;
-//   values: HD/8 lanes per token, 8 dims (one 128-bit load) per lane, fp32 accumulators per query
-//           head, reduced over the token slots of the wavefront and then over the 16 wavefronts.
+// Single-query attention, grouped-query form with a one-pass ("online") softmax.
+// grid (KV heads, rows, splits), 4 wavefronts per workgroup.  The G query heads that share a KV head
+// are served together, so K and V are read once.  Both caches are token-major: a token's head
+// vector is contiguous (HD fp16 = 256 bytes at HD 128).
+//   * a wavefront owns chunks of 4 tokens, round-robin over all wavefronts of the KV head;
+//     16 lanes per token, 8 dims per lane, the same lane mapping for K and V;
+//   * per chunk: K and V rows are loaded first (one 128-bit load each for fp16 caches), the partial
+//     dots are all-reduced over a token's 16 lanes, the running maximum m, the per-slot denominators
+//     l and the value sums acc are updated (acc *= exp(m_old - m_new));
+//   * the token slots and wavefronts of the workgroup are combined through LDS with the usual
+//     (m, l, acc) merge; with more than one split the workgroup writes its partial state and
+//     attention_merge_kernel combines the splits in split order.
 template <int HD, int G, bool KV_F16>
-__global__ __launch_bounds__(1024) void attention_gqa_kernel(AttentionArgs a) {
-    extern __shared__ float smem[];
-    float *sc = smem;                                  // [G][max_seq] scores, then probabilities
-    float *part = smem + (size_t)G * a.max_seq;        // [16][G][HD] per-wavefront value sums
-    __shared__ float red[16 * G];
-    constexpr int LPT = HD / 16, TPI = 64 / LPT;       // score phase: lanes per token, tokens per pass
-    constexpr int LPV = HD / 8, TPV = 64 / LPV;        // value phase
-    const int kvh = blockIdx.x, m = blockIdx.y;
+__global__ __launch_bounds__(256) void attention_flash_kernel(AttentionArgs a) {
+    constexpr int WAVES = 4, LPT = HD / 8, SLOTS = 64 / LPT;   // lanes per token, tokens per chunk
+    constexpr int KW = KV_F16 ? 1 : 2;                         // 128-bit loads per 8 values
+    __shared__ float wm[WAVES][G], wl[WAVES][SLOTS][G];
+    __shared__ float wacc[WAVES][SLOTS][G][HD];
+    const int kvh = blockIdx.x, m = blockIdx.y, split = blockIdx.z, splits = gridDim.z;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int visible = a.pos[m] + 1;
     const int kd = a.n_kv_head * HD;
     const size_t seq_base = (size_t)a.seq[m] * a.cache_seq_stride;
     const float scale = 1.0f / sqrtf((float)HD);
+    const int slot = lane / LPT, seg = (lane % LPT) * 8;
 
-    {   // ---- scores ----
-        const int seg = (lane % LPT) * 16;
-        float q[G][16];
+    float q[G][8];
 #pragma unroll
-        for (int g = 0; g < G; g++)
+    for (int g = 0; g < G; g++) {
+        const float4 *qp = reinterpret_cast<const float4 *>(a.q + (size_t)m * a.n_head * HD + (size_t)(kvh * G + g) * HD + seg);
+        const float4 q0 = qp[0], q1 = qp[1];
+        q[g][0] = q0.x; q[g][1] = q0.y; q[g][2] = q0.z; q[g][3] = q0.w;
+        q[g][4] = q1.x; q[g][5] = q1.y; q[g][6] = q1.z; q[g][7] = q1.w;
+    }
+    float mx[G], l[G], acc[G][8];
 #pragma unroll
-            for (int i = 0; i < 16; i++) q[g][i] = a.q[(size_t)m * a.n_head * HD + (size_t)(kvh * G + g) * HD + seg + i];
-        for (int t0 = wave * TPI; t0 < visible; t0 += 16 * TPI) {
-            const int t = t0 + lane / LPT;
+    for (int g = 0; g < G; g++) {
+        mx[g] = -INFINITY;
+        l[g] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[g][i] = 0.0f;
+    }
+
+    auto unpack8 = [](const uint4 *r, float *out) {
+        if (KV_F16) {
+            const uint32_t w[4] = {r[0].x, r[0].y, r[0].z, r[0].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) { out[2 * i] = from_half_bits((uint16_t)(w[i] & 0xFFFFu)); out[2 * i + 1] = from_half_bits((uint16_t)(w[i] >> 16)); }
+        } else {
+            out[0] = __uint_as_float(r[0].x); out[1] = __uint_as_float(r[0].y); out[2] = __uint_as_float(r[0].z); out[3] = __uint_as_float(r[0].w);
+            out[4] = __uint_as_float(r[KW - 1].x); out[5] = __uint_as_float(r[KW - 1].y); out[6] = __uint_as_float(r[KW - 1].z); out[7] = __uint_as_float(r[KW - 1].w);
+        }
+    };
+
+    constexpr int U = 2;   // chunks whose loads are in flight together
+    const int stride = splits * WAVES * SLOTS;
+    for (int t0 = (split * WAVES + wave) * SLOTS; t0 < visible; t0 += stride * U) {
+        uint4 kr[U][KW], vr[U][KW];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int t = t0 + u * stride + slot;
+            const size_t off = seq_base + (size_t)(t < visible ? t : 0) * kd + (size_t)kvh * HD + seg;
+            const uint4 *kp = KV_F16 ? reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.k_cache) + off)
+                                     : reinterpret_cast<const uint4 *>(reinterpret_cast<const float *>(a.k_cache) + off);
+            const uint4 *vp = KV_F16 ? reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.v_cache) + off)
+                                     : reinterpret_cast<const uint4 *>(reinterpret_cast<const float *>(a.v_cache) + off);
+#pragma unroll
+            for (int i = 0; i < KW; i++) { kr[u][i] = kp[i]; vr[u][i] = vp[i]; }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int t = t0 + u * stride + slot;
             const bool valid = t < visible;
-            const size_t off = seq_base + (size_t)(valid ? t : 0) * kd + (size_t)kvh * HD + seg;
-            float k[16];
-            if (KV_F16) {
-                const uint4 *p = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.k_cache) + off);
-                const uint4 v0 = p[0], v1 = p[1];
-                const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-#pragma unroll
-                for (int i = 0; i < 8; i++) { k[2 * i] = from_half_bits((uint16_t)(w[i] & 0xFFFFu)); k[2 * i + 1] = from_half_bits((uint16_t)(w[i] >> 16)); }
-            } else {
-                const float4 *p = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(a.k_cache) + off);
-#pragma unroll
-                for (int i = 0; i < 4; i++) { const float4 v = p[i]; k[4 * i] = v.x; k[4 * i + 1] = v.y; k[4 * i + 2] = v.z; k[4 * i + 3] = v.w; }
-            }
-            float dot[G];
+            if (t0 + u * stride >= visible) break;   // whole chunk beyond the prefix (uniform)
+            float k[8], v[8];
+            unpack8(kr[u], k);
+            unpack8(vr[u], v);
 #pragma unroll
             for (int g = 0; g < G; g++) {
                 float d = 0.0f;
 #pragma unroll
-                for (int i = 0; i < 16; i++) d += q[g][i] * k[i];
+                for (int i = 0; i < 8; i++) d += q[g][i] * k[i];
+                d = group_sum<LPT>(d);                                  // all lanes of the token
+                const float sc = valid ? d * scale : -INFINITY;
+                const float cm = max_over_groups<LPT>(sc);              // over the chunk's tokens
+                const float m_new = fmaxf(mx[g], cm);      // finite: the chunk holds at least one visible token
+                const float alpha = expf(mx[g] - m_new);   // exp(-inf) = 0 on the first chunk
+                const float p = valid ? expf(sc - m_new) : 0.0f;
+                l[g] = l[g] * alpha + p;
 #pragma unroll
-                for (int o = LPT / 2; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);
-                dot[g] = d;
-            }
-            if (valid && lane % LPT == 0) {
-#pragma unroll
-                for (int g = 0; g < G; g++) sc[(size_t)g * a.max_seq + t] = dot[g] * scale;
+                for (int i = 0; i < 8; i++) acc[g][i] = acc[g][i] * alpha + p * v[i];
+                mx[g] = m_new;
             }
         }
+    }
+    // ---- every (wavefront, token slot) publishes its partial state; m is the same in all lanes ----
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) wacc[wave][slot][g][seg + i] = acc[g][i];
+        if (lane % LPT == 0) wl[wave][slot][g] = l[g];
+        if (lane == 0) wm[wave][g] = mx[g];
     }
     __syncthreads();
-    // ---- softmax over the visible tokens, per query head ----
-    float inv_denom[G];
-    {
-        float mx[G], sm[G];
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            float v = -INFINITY;
-            for (int t = tid; t < visible; t += 1024) v = fmaxf(v, sc[(size_t)g * a.max_seq + t]);
-            v = wave_max_f(v);
-            if (lane == 0) red[wave * G + g] = v;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            float v = red[g];
-            for (int w = 1; w < 16; w++) v = fmaxf(v, red[w * G + g]);
-            mx[g] = v;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            float s = 0.0f;
-            for (int t = tid; t < visible; t += 1024) {
-                const float e = expf(sc[(size_t)g * a.max_seq + t] - mx[g]);
-                sc[(size_t)g * a.max_seq + t] = e;
-                s += e;
-            }
-            s = wave_sum_f(s);
-            if (lane == 0) red[wave * G + g] = s;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            float s = 0.0f;
-            for (int w = 0; w < 16; w++) s += red[w * G + g];
-            sm[g] = s;
-            inv_denom[g] = s > 0.0f ? 1.0f / s : 0.0f;
-        }
-        (void)sm;
-    }
-    // ---- values ----
-    {
-        const int seg = (lane % LPV) * 8;
-        float acc[G][8];
-#pragma unroll
-        for (int g = 0; g < G; g++)
-#pragma unroll
-            for (int i = 0; i < 8; i++) acc[g][i] = 0.0f;
-        for (int t0 = wave * TPV; t0 < visible; t0 += 16 * TPV) {
-            const int t = t0 + lane / LPV;
-            const bool valid = t < visible;
-            const size_t off = seq_base + (size_t)(valid ? t : 0) * kd + (size_t)kvh * HD + seg;
-            float v[8];
-            if (KV_F16) {
-                const uint4 r = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.v_cache) + off);
-                const uint32_t w[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-                for (int i = 0; i < 4; i++) { v[2 * i] = from_half_bits((uint16_t)(w[i] & 0xFFFFu)); v[2 * i + 1] = from_half_bits((uint16_t)(w[i] >> 16)); }
-            } else {
-                const float4 *p = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(a.v_cache) + off);
-                const float4 r0 = p[0], r1 = p[1];
-                v[0] = r0.x; v[1] = r0.y; v[2] = r0.z; v[3] = r0.w; v[4] = r1.x; v[5] = r1.y; v[6] = r1.z; v[7] = r1.w;
-            }
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-                const float p = valid ? sc[(size_t)g * a.max_seq + t] * inv_denom[g] : 0.0f;
-#pragma unroll
-                for (int i = 0; i < 8; i++) acc[g][i] += p * v[i];
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < G; g++)
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                float x = acc[g][i];
-#pragma unroll
-                for (int o = LPV; o < 64; o <<= 1) x += __shfl_xor(x, o, 64);
-                if (lane < LPV) part[((size_t)wave * G + g) * HD + seg + i] = x;
-            }
-    }
-    __syncthreads();
-    for (int i = tid; i < G * HD; i += 1024) {
-        float total = 0.0f;
-        for (int w = 0; w < 16; w++) total += part[(size_t)w * G * HD + i];
+    // ---- merge over wavefronts and slots: thread (g, dim) ----
+    float *scratch = a.split_scratch + (((size_t)m * a.n_kv_head + kvh) * splits) * G * (HD + 2);
+    for (int i = tid; i < G * HD; i += 256) {
         const int g = i / HD, dch = i % HD;
-        a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)(kvh * G + g) * HD + dch] = to_half_bits(total);
+        float M = wm[0][g];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) M = fmaxf(M, wm[w][g]);
+        float L = 0.0f, A = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) {
+            const float f = wm[w][g] == -INFINITY ? 0.0f : expf(wm[w][g] - M);
+            float lw = 0.0f, aw = 0.0f;
+#pragma unroll
+            for (int sl = 0; sl < SLOTS; sl++) { lw += wl[w][sl][g]; aw += wacc[w][sl][g][dch]; }
+            L += lw * f;
+            A += aw * f;
+        }
+        if (splits == 1) {
+            a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)(kvh * G + g) * HD + dch] = to_half_bits(L > 0.0f ? A / L : 0.0f);
+        } else {
+            float *ps = scratch + ((size_t)split * G + g) * (HD + 2);
+            ps[2 + dch] = A;
+            if (dch == 0) { ps[0] = M; ps[1] = L; }
+        }
+    }
+}
+
+// Merges the per-split partial states (m, l, acc) of attention_flash_kernel in split order.
+// grid (KV heads, rows).  A kernel boundary, not a device-scope fence, orders it after the partial
+// writes: fences plus arrival counters in every workgroup cost far more than this launch.
+template <int HD, int G>
+__global__ __launch_bounds__(256) void attention_merge_kernel(AttentionArgs a, int splits) {
+    const int kvh = blockIdx.x, m = blockIdx.y, tid = threadIdx.x;
+    const float *scratch = a.split_scratch + (((size_t)m * a.n_kv_head + kvh) * splits) * G * (HD + 2);
+    for (int i = tid; i < G * HD; i += 256) {
+        const int g = i / HD, dch = i % HD;
+        // all partials are fetched before the first is used (one memory round trip)
+        float pm[kAttentionMaxSplits], pl[kAttentionMaxSplits], pa[kAttentionMaxSplits];
+#pragma unroll
+        for (int sp = 0; sp < kAttentionMaxSplits; sp++) {
+            const float *ps = scratch + ((size_t)(sp < splits ? sp : 0) * G + g) * (HD + 2);
+            pm[sp] = ps[0]; pl[sp] = ps[1]; pa[sp] = ps[2 + dch];
+        }
+        float M = -INFINITY;
+#pragma unroll
+        for (int sp = 0; sp < kAttentionMaxSplits; sp++) if (sp < splits) M = fmaxf(M, pm[sp]);
+        float L = 0.0f, A = 0.0f;
+#pragma unroll
+        for (int sp = 0; sp < kAttentionMaxSplits; sp++) {
+            const float f = (sp < splits && pm[sp] != -INFINITY) ? expf(pm[sp] - M) : 0.0f;
+            L += pl[sp] * f;
+            A += pa[sp] * f;
+        }
+        a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)(kvh * G + g) * HD + dch] = to_half_bits(L > 0.0f ? A / L : 0.0f);
     }
 }
 
 template <int HD, int G>
 hipError_t launch_attention_gqa(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
-    const size_t lds = ((size_t)G * a.max_seq + (size_t)16 * G * HD) * sizeof(float);
-    dim3 grid(a.n_kv_head, rows);
-    if (kv_f16) {
-        auto kernel = attention_gqa_kernel<HD, G, true>;
-        if (lds > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-        }
-        hipLaunchKernelGGL(kernel, grid, dim3(1024), lds, s, a);
-    } else {
-        auto kernel = attention_gqa_kernel<HD, G, false>;
-        if (lds > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return e;
-        }
-        hipLaunchKernelGGL(kernel, grid, dim3(1024), lds, s, a);
-    }
+    // enough workgroups to spread a long prefix over the chip; fixed per runtime so that a captured
+    // graph stays valid as the prefix grows
+    // each wavefront keeps two chunks of loads in flight: with max_seq / (2 chunks * 4 wavefronts * tokens per
+    // chunk) splits, a prefix of any length up to max_seq costs every wavefront one memory round trip
+    const int tokens_per_wg = 2 * 4 * (64 / (HD / 8));
+    int splits = (a.max_seq + tokens_per_wg - 1) / tokens_per_wg;
+    splits = splits < 1 ? 1 : (splits > kAttentionMaxSplits ? kAttentionMaxSplits : splits);
+    if (!a.split_scratch) splits = 1;
+    dim3 grid(a.n_kv_head, rows, splits);
+    if (kv_f16) hipLaunchKernelGGL((attention_flash_kernel<HD, G, true>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((attention_flash_kernel<HD, G, false>), grid, dim3(256), 0, s, a);
+    if (splits > 1) hipLaunchKernelGGL((attention_merge_kernel<HD, G>), dim3(a.n_kv_head, rows), dim3(256), 0, s, a, splits);
     return hipGetLastError();
 }
 
@@ -417,31 +445,63 @@ __global__ void swiglu_kernel(const float *gu, int hidden, uint16_t *act_f16) {
 }
 
 // First-max argmax of logits[m][0..vocab): lowest index wins ties (:8219-8275, neon_convert.c:36-101).
-__global__ __launch_bounds__(kBlock) void argmax_kernel(const float *logits, int vocab, int *out_token, float *out_value) {
-    __shared__ float bv[kBlock];
-    __shared__ int bi[kBlock];
-    const int m = blockIdx.x;
-    const float *row = logits + (size_t)m * vocab;
-    float best = -INFINITY;
-    int best_i = 0x7FFFFFFF;
-    for (int i = threadIdx.x; i < vocab; i += kBlock) {
-        const float v = row[i];
-        if (v > best) { best = v; best_i = i; }   // ascending i per thread: strict > keeps the first
-    }
+// Two launches: argmax_partial_kernel, grid (slices, rows), scans one slice per workgroup and writes
+// (value, index); argmax_final_kernel, grid (rows), reduces the slices in slice order.
+constexpr int kArgmaxBlocks = 128;
+
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+__device__ __forceinline__ void argmax_block_reduce(float &best, int &best_i, float *bv, int *bi) {
     bv[threadIdx.x] = best;
     bi[threadIdx.x] = best_i;
     __syncthreads();
     for (int s = kBlock / 2; s > 0; s >>= 1) {
-        if (threadIdx.x < s) {
-            const float ov = bv[threadIdx.x + s];
-            const int oi = bi[threadIdx.x + s];
-            if (ov > bv[threadIdx.x] || (ov == bv[threadIdx.x] && oi < bi[threadIdx.x])) { bv[threadIdx.x] = ov; bi[threadIdx.x] = oi; }
+        if (threadIdx.x < s && better(bv[threadIdx.x + s], bi[threadIdx.x + s], bv[threadIdx.x], bi[threadIdx.x])) {
+            bv[threadIdx.x] = bv[threadIdx.x + s];
+            bi[threadIdx.x] = bi[threadIdx.x + s];
         }
         __syncthreads();
     }
+    best = bv[0];
+    best_i = bi[0];
+}
+
+__global__ __launch_bounds__(kBlock) void argmax_partial_kernel(const float *logits, int vocab, float *part_value, int *part_index) {
+    __shared__ float bv[kBlock];
+    __shared__ int bi[kBlock];
+    const int m = blockIdx.y, blk = blockIdx.x, nblk = gridDim.x;
+    const float *row = logits + (size_t)m * vocab;
+    const int per = (vocab + nblk - 1) / nblk;
+    const int lo = blk * per, hi = lo + per < vocab ? lo + per : vocab;
+    float best = -INFINITY;
+    int best_i = 0x7FFFFFFF;
+    for (int i = lo + threadIdx.x; i < hi; i += kBlock) {
+        const float v = row[i];
+        if (v > best) { best = v; best_i = i; }   // ascending i per thread: strict > keeps the first
+    }
+    argmax_block_reduce(best, best_i, bv, bi);
     if (threadIdx.x == 0) {
-        out_token[m] = bi[0] == 0x7FFFFFFF ? 0 : bi[0];
-        if (out_value) out_value[m] = bv[0];
+        part_value[(size_t)m * nblk + blk] = best;
+        part_index[(size_t)m * nblk + blk] = best_i;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void argmax_final_kernel(const float *part_value, const int *part_index, int nblk,
+                                                              int *out_token, float *out_value) {
+    __shared__ float bv[kBlock];
+    __shared__ int bi[kBlock];
+    const int m = blockIdx.x;
+    float best = -INFINITY;
+    int best_i = 0x7FFFFFFF;
+    for (int i = threadIdx.x; i < nblk; i += kBlock) {
+        const float v = part_value[(size_t)m * nblk + i];
+        const int idx = part_index[(size_t)m * nblk + i];
+        if (better(v, idx, best, best_i)) { best = v; best_i = idx; }
+    }
+    argmax_block_reduce(best, best_i, bv, bi);
+    if (threadIdx.x == 0) {
+        out_token[m] = best_i == 0x7FFFFFFF ? 0 : best_i;
+        if (out_value) out_value[m] = best;
     }
 }
 
@@ -509,8 +569,7 @@ hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStrea
 hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
     // grouped-query kernel for the common head shapes; everything else takes the general kernel
     const int group = a.n_head / a.n_kv_head;
-    const size_t fast_lds = ((size_t)group * a.max_seq + (size_t)16 * group * a.head_dim) * sizeof(float);
-    if (a.n_head % a.n_kv_head == 0 && fast_lds <= 150 * 1024) {
+    if (a.n_head % a.n_kv_head == 0) {
         if (a.head_dim == 128) {
             if (group == 1) return launch_attention_gqa<128, 1>(a, rows, kv_f16, s);
             if (group == 2) return launch_attention_gqa<128, 2>(a, rows, kv_f16, s);
@@ -536,8 +595,13 @@ hipError_t launch_swiglu(const float *gu, int rows, int hidden, uint16_t *act_f1
     return hipGetLastError();
 }
 
-hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_token, float *out_value, hipStream_t s) {
-    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(kBlock), 0, s, logits, vocab, out_token, out_value);
+hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_token, float *out_value, const ArgmaxScratch &scratch,
+                         hipStream_t s) {
+    if (!scratch.part_value || !scratch.part_index || rows > kMaxStepRows) return hipErrorInvalidValue;
+    const int blocks = vocab < kArgmaxBlocks * kBlock ? (vocab + kBlock - 1) / kBlock : kArgmaxBlocks;
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(blocks, rows), dim3(kBlock), 0, s, logits, vocab, scratch.part_value, scratch.part_index);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(kBlock), 0, s, scratch.part_value, scratch.part_index, blocks, out_token,
+                       out_value);
     return hipGetLastError();
 }
 

@@ -68,6 +68,8 @@ LlamaRuntime::~LlamaRuntime() {
     free_device(last_hidden_); free_device(xn_); free_device(ctx_); free_device(act_);
     free_device(d_tokens_); free_device(d_pos_); free_device(d_seq_); free_device(d_out_tokens_);
     free_device(d_visible_); free_device(d_log_); free_device(d_log_count_);
+    free_device(attn_scratch_);
+    free_device(argmax_scratch_.part_value); free_device(argmax_scratch_.part_index);
     for (hipGraphExec_t g : step_graphs_) if (g) (void)hipGraphExecDestroy(g);
     for (TimedLaunch &t : timed_) { (void)hipEventDestroy(t.start); (void)hipEventDestroy(t.stop); }
     for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
@@ -309,6 +311,12 @@ int LlamaRuntime::finalize() {
     if ((rc = device_alloc(&d_log_, (size_t)c_.max_seq)) != ESP_OK) return rc;
     if ((rc = device_alloc(&d_log_count_, 1)) != ESP_OK) return rc;
     step_graphs_.assign(c_.max_sequences, nullptr);
+    if ((rc = device_alloc(&argmax_scratch_.part_value, (size_t)kArgmaxScratchSlots)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&argmax_scratch_.part_index, (size_t)kArgmaxScratchSlots)) != ESP_OK) return rc;
+    {
+        const size_t per_row = (size_t)c_.n_kv_head * kAttentionMaxSplits * (c_.n_head / c_.n_kv_head) * (c_.head_dim + 2);
+        if ((rc = device_alloc(&attn_scratch_, (size_t)kMaxStepRows * per_row)) != ESP_OK) return rc;
+    }
     finalized_ = true;
     return reset();
 }
@@ -391,6 +399,7 @@ int LlamaRuntime::enqueue_trunk(int M) {
         aa.q = q_; aa.k_cache = L.k_cache; aa.v_cache = L.v_cache; aa.cache_seq_stride = cache_seq_stride;
         aa.n_head = c_.n_head; aa.n_kv_head = c_.n_kv_head; aa.head_dim = c_.head_dim; aa.max_seq = c_.max_seq;
         aa.pos = d_pos_; aa.seq = d_seq_; aa.ctx_f16 = ctx_;
+        aa.split_scratch = attn_scratch_;
         if ((rc = time_begin(K_ATTENTION)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_attention(aa, M, kv16, s));
         if ((rc = time_end()) != ESP_OK) return rc;
@@ -456,7 +465,7 @@ int LlamaRuntime::run_head(const float *hidden_rows, int count) {
     if ((rc = time_begin(K_HEAD)) != ESP_OK) return rc;
     ESP_HIP_TRY(launch_gemv(g, s));
     if ((rc = time_end()) != ESP_OK) return rc;
-    ESP_HIP_TRY(launch_argmax(logits_, count, c_.vocab, d_out_tokens_, nullptr, s));
+    ESP_HIP_TRY(launch_argmax(logits_, count, c_.vocab, d_out_tokens_, nullptr, argmax_scratch_, s));
     return ESP_OK;
 }
 

@@ -109,6 +109,8 @@ class LlamaRuntime {
     bool use_graph_ = true;
     std::vector<hipGraphExec_t> step_graphs_;
     int *d_visible_ = nullptr, *d_log_ = nullptr, *d_log_count_ = nullptr;
+    ArgmaxScratch argmax_scratch_;
+    float *attn_scratch_ = nullptr;
 
     struct TimedLaunch { int kernel_class; hipEvent_t start, stop; };
     bool timing_enabled_ = false;
