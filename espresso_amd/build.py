@@ -20,7 +20,8 @@ HIPCC_FLAGS = [
 
 
 def sources() -> list[str]:
-    return sorted(glob.glob(os.path.join(CSRC, "*.cpp")) + glob.glob(os.path.join(CSRC, "kernels", "*.hip")))
+    return sorted(glob.glob(os.path.join(CSRC, "*.cpp")) + glob.glob(os.path.join(CSRC, "host", "*.cpp")) +
+                  glob.glob(os.path.join(CSRC, "kernels", "*.hip")))
 
 
 def build(verbose: bool = False) -> str:

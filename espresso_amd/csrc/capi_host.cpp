@@ -1,0 +1,234 @@
+// C ABI: weight files, metadata, the GGUF front door, the engine and the exact two-token harness.
+#include <cstring>
+
+#include "host/engine.h"
+#include "host/gguf.h"
+#include "host/harness.h"
+
+using namespace esp;
+
+struct ESPEngine {
+    std::unique_ptr<RealModelInferenceEngine> engine;
+    ESPLlamaRuntime runtime_handle{nullptr};
+};
+
+namespace {
+
+MultiModelConfig from_c(const ESPModelConfig &c) {
+    MultiModelConfig m;
+    m.name = std::string(c.name, strnlen(c.name, sizeof(c.name)));
+    m.nLayer = c.n_layer; m.nHead = c.n_head; m.nKVHead = c.n_kv_head; m.dModel = c.d_model; m.headDim = c.head_dim;
+    m.hiddenDim = c.hidden_dim; m.vocab = c.vocab; m.maxSeq = c.max_seq; m.normEps = c.norm_eps; m.ropeTheta = c.rope_theta;
+    m.hasEosToken = c.eos_token >= 0;
+    m.eosToken = c.eos_token >= 0 ? (TokenID)c.eos_token : 0;
+    m.architecture = c.architecture == 0 ? MultiModelConfig::Architecture::gpt2 : MultiModelConfig::Architecture::llama;
+    return m;
+}
+
+void to_c(const MultiModelConfig &m, ESPModelConfig *c) {
+    std::memset(c, 0, sizeof(*c));
+    std::strncpy(c->name, m.name.c_str(), sizeof(c->name) - 1);
+    c->n_layer = m.nLayer; c->n_head = m.nHead; c->n_kv_head = m.nKVHead; c->d_model = m.dModel; c->head_dim = m.headDim;
+    c->hidden_dim = m.hiddenDim; c->vocab = m.vocab; c->max_seq = m.maxSeq; c->norm_eps = m.normEps; c->rope_theta = m.ropeTheta;
+    c->eos_token = m.hasEosToken ? (int32_t)m.eosToken : -1;
+    c->architecture = m.architecture == MultiModelConfig::Architecture::gpt2 ? 0 : 1;
+}
+
+Environment env_from(const char *const *keys, const char *const *values, int count) {
+    Environment e;
+    for (int i = 0; i < count; i++) if (keys && values && keys[i] && values[i]) e[keys[i]] = values[i];
+    return e;
+}
+
+// adapts the C callback table to the C++ protocol
+class CallbackModel : public ExactTwoTokenGeneratingLanguageModel {
+  public:
+    explicit CallbackModel(const ESPExactTwoTokenModel &m) : m_(m) {}
+    int vocabSize() const override { return 0; }
+    int reset() override { return check(m_.reset(m_.context), "reset"); }
+    int prefillSelectedToken(const std::vector<TokenID> &p, TokenID *sel) override {
+        return check(m_.prefill_selected_token(m_.context, p.data(), (int)p.size(), sel), "prefillSelectedToken");
+    }
+    int performExactTwoTokenPass(TokenID cur, int budget, ExactTwoTokenPassResult *r) override {
+        ESPPassResult c{};
+        int rc = check(m_.perform_exact_two_token_pass(m_.context, cur, budget, &c), "performExactTwoTokenPass");
+        if (rc != ESP_OK) return rc;
+        const int n = c.committed_count < 0 ? 0 : (c.committed_count > 2 ? 3 : c.committed_count);
+        r->committedTokens.clear();
+        for (int i = 0; i < n && i < 2; i++) r->committedTokens.push_back(c.committed_tokens[i]);
+        if (n == 3) r->committedTokens.push_back(0);   // too many: let the harness reject it
+        r->nextCurrentToken = c.next_current_token;
+        r->metrics.proposerLatencyMs = c.proposer_latency_ms;
+        r->metrics.verifierTrunkLatencyMs = c.verifier_trunk_latency_ms;
+        r->metrics.verifierLogitsLatencyMs = c.verifier_logits_latency_ms;
+        r->metrics.stateAdvanceLatencyMs = c.state_advance_latency_ms;
+        r->metrics.acceptedFutureTokenCount = c.accepted_future_token_count;
+        r->metrics.committedExactTokenCount = c.committed_exact_token_count;
+        return ESP_OK;
+    }
+
+  private:
+    static int check(int rc, const char *what) { return rc == 0 ? ESP_OK : fail(ESP_ERR_LAUNCH_FAILED, "model callback %s failed (%d)", what, rc); }
+    ESPExactTwoTokenModel m_;
+};
+
+}  // namespace
+
+extern "C" {
+
+size_t esp_weight_blob_bytes(size_t element_count) { return 128 + element_count * 2; }
+
+int esp_weight_blob_build(const float *weights, size_t element_count, uint8_t *out) {
+    if ((!weights && element_count) || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "weight_blob_build: null pointer");
+    const std::vector<uint8_t> b = WeightBlob::build(weights, element_count);
+    std::memcpy(out, b.data(), b.size());
+    return ESP_OK;
+}
+
+long esp_blob_weight_load(const char *path, float *out, size_t capacity) {
+    if (!path) return -6;
+    std::vector<float> v;
+    const BlobWeightLoaderError e = BlobWeightLoader::load(path, &v);
+    if (e != BlobWeightLoaderError::none) return -(long)e;
+    if (out) std::memcpy(out, v.data(), sizeof(float) * (v.size() < capacity ? v.size() : capacity));
+    return (long)v.size();
+}
+
+int esp_layer_weight_path(int layer, const char *blob_dir, int slot, char *out, size_t capacity) {
+    if (!blob_dir || !out || capacity == 0) return fail(ESP_ERR_INVALID_ARGUMENT, "layer_weight_path: null pointer");
+    const LayerWeightPaths p = LayerWeightPaths::forLayer(layer, MultiModelConfig{}, blob_dir);
+    const std::string *s = nullptr;
+    switch (slot) {
+    case SLOT_RMS_ATT: s = &p.rmsAtt; break;
+    case SLOT_WQ: s = &p.wq; break;
+    case SLOT_WK: s = &p.wk; break;
+    case SLOT_WV: s = &p.wv; break;
+    case SLOT_WO: s = &p.wo; break;
+    case SLOT_RMS_FFN: s = &p.rmsFfn; break;
+    case SLOT_W1: s = &p.w1; break;
+    case SLOT_W2: s = &p.w2; break;
+    case SLOT_W3: s = &p.w3; break;
+    case SLOT_Q_NORM: s = &p.qNorm; break;
+    case SLOT_K_NORM: s = &p.kNorm; break;
+    default: return fail(ESP_ERR_INVALID_ARGUMENT, "layer_weight_path: slot %d is not a layer slot", slot);
+    }
+    if (s->size() + 1 > capacity) return fail(ESP_ERR_OUT_OF_RANGE, "layer_weight_path: buffer too small");
+    std::memcpy(out, s->c_str(), s->size() + 1);
+    return (int)s->size();
+}
+
+int esp_model_config_load_metadata(const char *path, ESPModelConfig *out) {
+    if (!path || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "null pointer");
+    MultiModelConfig m;
+    std::string err;
+    if (!loadConfigFromMetadataFile(path, &m, &err)) return fail(ESP_ERR_IO, "%s", err.c_str());
+    to_c(m, out);
+    return ESP_OK;
+}
+
+int esp_model_config_write_metadata(const ESPModelConfig *config, const char *path) {
+    if (!path || !config) return fail(ESP_ERR_INVALID_ARGUMENT, "null pointer");
+    const std::string j = metadataJSON(from_c(*config));
+    return writeFile(path, j.data(), j.size()) ? ESP_OK : fail(ESP_ERR_IO, "cannot write %s", path);
+}
+
+int esp_gguf_prepare(const char *gguf_path, const char *output_dir, const ESPPrepareOptions *o, ESPModelConfig *out_config,
+                     int *out_tensor_count) {
+    if (!gguf_path || !output_dir) return fail(ESP_ERR_INVALID_ARGUMENT, "null path");
+    PrepareOptions opt;
+    if (o) { opt.emitDequantizedBlobs = o->emit_dequantized_blobs != 0; opt.emitFloat32Sidecars = o->emit_float32_sidecars != 0; opt.qkLayout = o->qk_layout; }
+    PreparedModel pm;
+    int rc = GGUFModelLoader::prepare(gguf_path, output_dir, opt, &pm);
+    if (rc != ESP_OK) return rc;
+    if (out_config) to_c(pm.config, out_config);
+    if (out_tensor_count) *out_tensor_count = pm.tensorCount;
+    return ESP_OK;
+}
+
+ESPEngine *esp_engine_build(const ESPModelConfig *config, const char *weight_dir, const char *tokenizer_dir,
+                            const char *const *env_keys, const char *const *env_values, int env_count) {
+    if (!config || !weight_dir) { fail(ESP_ERR_INVALID_ARGUMENT, "null config or weight directory"); return nullptr; }
+    std::unique_ptr<RealModelInferenceEngine> e;
+    if (RealModelInferenceEngine::build(from_c(*config), weight_dir, tokenizer_dir ? tokenizer_dir : "",
+                                        env_from(env_keys, env_values, env_count), &e) != ESP_OK)
+        return nullptr;
+    ESPEngine *h = new ESPEngine();
+    h->engine = std::move(e);
+    h->runtime_handle.rt = &h->engine->runtime();
+    return h;
+}
+
+void esp_engine_free(ESPEngine *engine) { delete engine; }
+
+ESPLlamaRuntime *esp_engine_runtime(ESPEngine *engine) { return engine ? &engine->runtime_handle : nullptr; }
+
+int esp_engine_generate(ESPEngine *engine, const uint32_t *prompt_tokens, int prompt_count, int max_tokens, float temperature,
+                        const char *const *env_keys, const char *const *env_values, int env_count, uint32_t *out_tokens,
+                        ESPGenerationResult *result) {
+    if (!engine) return fail(ESP_ERR_INVALID_ARGUMENT, "null engine");
+    std::vector<TokenID> prompt;
+    if (prompt_tokens && prompt_count > 0) prompt.assign(prompt_tokens, prompt_tokens + prompt_count);
+    GenerationResult r;
+    int rc = engine->engine->generate(prompt, max_tokens, temperature, env_from(env_keys, env_values, env_count), &r);
+    if (rc != ESP_OK) return rc;
+    if (out_tokens) for (size_t i = 0; i < r.tokens.size(); i++) out_tokens[i] = r.tokens[i];
+    if (result) {
+        std::memset(result, 0, sizeof(*result));
+        result->token_count = (int32_t)r.tokens.size();
+        result->tokens_per_second = r.tokensPerSecond;
+        result->compile_time_ms = r.compileTimeMs;
+        result->first_token_latency_ms = r.firstTokenLatencyMs;
+        result->has_two_token_stats = r.hasTwoTokenStats ? 1 : 0;
+        result->committed_exact_tokens_per_pass = r.committedExactTokensPerPass;
+        result->accepted_future_tokens_per_pass = r.acceptedFutureTokensPerPass;
+        std::strncpy(result->exact_head_backend, r.exactHeadBackend.c_str(), sizeof(result->exact_head_backend) - 1);
+    }
+    return ESP_OK;
+}
+
+void esp_exact_two_token_promotion_plan(uint32_t current_token, uint32_t proposed_future_token, uint32_t exact_next_token,
+                                        uint32_t exact_future_token, int remaining_token_budget, ESPPromotionPlan *out) {
+    if (!out) return;
+    const ExactTwoTokenBranchPromotionPlan p =
+        ExactTwoTokenBranchPromotionPlan::make(current_token, proposed_future_token, exact_next_token, exact_future_token, remaining_token_budget);
+    std::memset(out, 0, sizeof(*out));
+    for (size_t i = 0; i < p.committedTokens.size(); i++) out->committed_tokens[i] = p.committedTokens[i];
+    out->committed_exact_token_count = p.committedExactTokenCount;
+    out->accepted_future_token_count = p.acceptedFutureTokenCount;
+    out->promoted_step_count = p.promotedStepCount;
+    out->next_current_token = p.nextCurrentToken;
+}
+
+int esp_exact_two_token_harness_generate(const ESPExactTwoTokenModel *model, ESPLlamaRuntime *target, ESPLlamaRuntime *draft,
+                                         const uint32_t *prompt_tokens, int prompt_count, int max_new_tokens,
+                                         uint32_t *out_tokens, int *out_token_count, int32_t *out_committed_per_pass,
+                                         int32_t *out_accepted_per_pass, int *out_pass_count) {
+    std::vector<TokenID> prompt;
+    if (prompt_tokens && prompt_count > 0) prompt.assign(prompt_tokens, prompt_tokens + prompt_count);
+    ExactTwoTokenGenerationTrace trace;
+    int rc;
+    if (model) {
+        if (!model->reset || !model->prefill_selected_token || !model->perform_exact_two_token_pass)
+            return fail(ESP_ERR_INVALID_ARGUMENT, "model callback table is incomplete");
+        CallbackModel m(*model);
+        rc = exactTwoTokenHarnessGenerate(m, prompt, max_new_tokens, &trace);
+    } else {
+        if (!target || !draft) return fail(ESP_ERR_INVALID_ARGUMENT, "no model given");
+        if (!target->rt->finalized() || !draft->rt->finalized()) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+        if (!prompt.empty() && (int)prompt.size() + max_new_tokens + 1 > target->rt->config().max_seq)
+            return fail(ESP_ERR_OUT_OF_RANGE, "prompt %zu + %d new tokens exceed context %d", prompt.size(), max_new_tokens, target->rt->config().max_seq);
+        HipExactTwoTokenModel m(*target->rt, *draft->rt);
+        rc = exactTwoTokenHarnessGenerate(m, prompt, max_new_tokens, &trace);
+    }
+    if (rc != ESP_OK) return rc;
+    if (out_tokens) for (size_t i = 0; i < trace.generatedTokens.size(); i++) out_tokens[i] = trace.generatedTokens[i];
+    if (out_token_count) *out_token_count = (int)trace.generatedTokens.size();
+    for (size_t i = 0; i < trace.passMetrics.size(); i++) {
+        if (out_committed_per_pass) out_committed_per_pass[i] = trace.passMetrics[i].committedExactTokenCount;
+        if (out_accepted_per_pass) out_accepted_per_pass[i] = trace.passMetrics[i].acceptedFutureTokenCount;
+    }
+    if (out_pass_count) *out_pass_count = (int)trace.passMetrics.size();
+    return ESP_OK;
+}
+
+}  // extern "C"

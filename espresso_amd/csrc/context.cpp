@@ -55,9 +55,9 @@ int ensure_init() {
 int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, DeviceMatrix *out) {
     *out = DeviceMatrix{};
     if (!gguf_blocks || rows <= 0 || cols <= 0) return fail(ESP_ERR_INVALID_ARGUMENT, "matrix: null data or empty shape");
-    if (!(format == FMT_F16 || format == FMT_Q4_0 || format == FMT_Q8_0 || format == FMT_Q4_K))
+    if (!(format == FMT_F32 || format == FMT_F16 || format == FMT_Q4_0 || format == FMT_Q8_0 || format == FMT_Q4_K))
         return fail(ESP_ERR_UNSUPPORTED, "matrix: format %d has no GEMV kernel", format);
-    const int block = format == FMT_F16 ? 8 : format_block_elems(format);
+    const int block = format == FMT_F16 ? 8 : format == FMT_F32 ? 4 : format_block_elems(format);
     if (cols % block != 0) return fail(ESP_ERR_INVALID_ARGUMENT, "matrix: cols %d is not a multiple of %d", cols, block);
     int rc = ensure_init();
     if (rc != ESP_OK) return rc;
@@ -71,6 +71,7 @@ int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, Devic
     case FMT_Q8_0: m.qs_row_bytes = (size_t)cols; break;
     case FMT_Q4_0: m.qs_row_bytes = (size_t)cols / 2; break;
     case FMT_Q4_K: m.qs_row_bytes = (size_t)cols / 256 * 144; break;
+    case FMT_F32: m.qs_row_bytes = (size_t)cols * 4; break;
     default: m.qs_row_bytes = (size_t)cols * 2; break;
     }
     if (m.qs_row_bytes % 16 != 0) return fail(ESP_ERR_INVALID_ARGUMENT, "matrix: row of %zu bytes is not 16-byte aligned", m.qs_row_bytes);

@@ -1,0 +1,342 @@
+#include "gguf.h"
+
+#include <cstdio>
+#include <cstring>
+
+#include "../context.h"
+
+namespace esp {
+namespace {
+
+enum : uint32_t { T_U8 = 0, T_I8, T_U16, T_I16, T_U32, T_I32, T_F32, T_BOOL, T_STRING, T_ARRAY, T_U64, T_I64, T_F64 };
+enum : uint32_t { GGML_F32 = 0, GGML_F16 = 1, GGML_Q4_0 = 2, GGML_Q8_0 = 8, GGML_Q4_K = 12, GGML_BF16 = 30 };
+
+struct Reader {
+    FILE *f = nullptr;
+    bool ok = true;
+    ~Reader() { if (f) std::fclose(f); }
+    template <typename T>
+    T get() {
+        T v{};
+        if (ok && std::fread(&v, sizeof(T), 1, f) != 1) ok = false;
+        return v;
+    }
+    std::string str() {
+        uint64_t n = get<uint64_t>();
+        if (!ok || n > (1u << 28)) { ok = false; return ""; }
+        std::string s((size_t)n, '\0');
+        if (n && std::fread(&s[0], 1, (size_t)n, f) != n) ok = false;
+        return s;
+    }
+    void skip(uint64_t n) { if (ok && std::fseek(f, (long)n, SEEK_CUR) != 0) ok = false; }
+};
+
+size_t scalar_size(uint32_t t) {
+    switch (t) {
+    case T_U8: case T_I8: case T_BOOL: return 1;
+    case T_U16: case T_I16: return 2;
+    case T_U32: case T_I32: case T_F32: return 4;
+    case T_U64: case T_I64: case T_F64: return 8;
+    default: return 0;
+    }
+}
+
+bool read_value(Reader &r, uint32_t type, GGUFValue *v) {
+    v->type = type;
+    switch (type) {
+    case T_U8: v->u = r.get<uint8_t>(); break;
+    case T_I8: v->u = (uint64_t)(int64_t)r.get<int8_t>(); break;
+    case T_U16: v->u = r.get<uint16_t>(); break;
+    case T_I16: v->u = (uint64_t)(int64_t)r.get<int16_t>(); break;
+    case T_U32: v->u = r.get<uint32_t>(); break;
+    case T_I32: v->u = (uint64_t)(int64_t)r.get<int32_t>(); break;
+    case T_F32: v->f = r.get<float>(); break;
+    case T_BOOL: v->u = r.get<uint8_t>() != 0; break;
+    case T_STRING: v->s = r.str(); break;
+    case T_U64: v->u = r.get<uint64_t>(); break;
+    case T_I64: v->u = (uint64_t)r.get<int64_t>(); break;
+    case T_F64: v->f = r.get<double>(); break;
+    case T_ARRAY: {
+        v->array_type = r.get<uint32_t>();
+        v->array_count = r.get<uint64_t>();
+        if (v->array_type == T_STRING) { for (uint64_t i = 0; i < v->array_count && r.ok; i++) r.skip(r.get<uint64_t>()); }
+        else if (v->array_type == T_ARRAY) r.ok = false;   // nested arrays do not occur in model files
+        else { size_t sz = scalar_size(v->array_type); if (!sz) r.ok = false; else r.skip(sz * v->array_count); }
+        break;
+    }
+    default: r.ok = false;
+    }
+    return r.ok;
+}
+
+}  // namespace
+
+size_t GGUFLoader::tensorBytes(uint32_t type, uint64_t elements) {
+    switch (type) {
+    case GGML_F32: return elements * 4;
+    case GGML_F16: case GGML_BF16: return elements * 2;
+    case GGML_Q4_0: return elements % 32 ? 0 : elements / 32 * 18;
+    case GGML_Q8_0: return elements % 32 ? 0 : elements / 32 * 34;
+    case GGML_Q4_K: return elements % 256 ? 0 : elements / 256 * 144;
+    default: return 0;
+    }
+}
+
+bool GGUFLoader::open(const std::string &path, std::string *error) {
+    auto bad = [&](const std::string &m) { if (error) *error = m; return false; };
+    Reader r;
+    r.f = std::fopen(path.c_str(), "rb");
+    if (!r.f) return bad("cannot open " + path);
+    std::fseek(r.f, 0, SEEK_END);
+    file_size_ = (uint64_t)std::ftell(r.f);
+    std::fseek(r.f, 0, SEEK_SET);
+    if (r.get<uint32_t>() != 0x46554747u) return bad("not a GGUF file (bad magic)");
+    version_ = r.get<uint32_t>();
+    if (version_ != 2 && version_ != 3) return bad("unsupported GGUF version " + std::to_string(version_));
+    const uint64_t n_tensors = r.get<uint64_t>(), n_kv = r.get<uint64_t>();
+    if (!r.ok || n_tensors > (1u << 20) || n_kv > (1u << 20)) return bad("truncated or implausible GGUF header");
+    meta_.clear();
+    tensors_.clear();
+    for (uint64_t i = 0; i < n_kv; i++) {
+        std::string key = r.str();
+        uint32_t type = r.get<uint32_t>();
+        GGUFValue v;
+        if (!r.ok || !read_value(r, type, &v)) return bad("malformed metadata entry " + std::to_string(i) + " (" + key + ")");
+        meta_[key] = v;
+    }
+    for (uint64_t i = 0; i < n_tensors; i++) {
+        GGUFTensorInfo t;
+        t.name = r.str();
+        uint32_t nd = r.get<uint32_t>();
+        if (!r.ok || nd == 0 || nd > 4) return bad("malformed tensor info " + std::to_string(i));
+        for (uint32_t d = 0; d < nd; d++) t.dims.push_back(r.get<uint64_t>());
+        t.type = r.get<uint32_t>();
+        t.offset = r.get<uint64_t>();
+        if (!r.ok) return bad("truncated tensor info " + std::to_string(i));
+        tensors_.push_back(t);
+    }
+    int64_t alignment = 32;
+    getInt("general.alignment", &alignment);
+    if (alignment <= 0) return bad("bad general.alignment");
+    const uint64_t pos = (uint64_t)std::ftell(r.f);
+    data_start_ = (pos + alignment - 1) / alignment * alignment;
+    path_ = path;
+    return true;
+}
+
+const GGUFTensorInfo *GGUFLoader::find(const std::string &name) const {
+    for (const GGUFTensorInfo &t : tensors_) if (t.name == name) return &t;
+    return nullptr;
+}
+bool GGUFLoader::getInt(const std::string &key, int64_t *out) const {
+    auto it = meta_.find(key);
+    if (it == meta_.end()) return false;
+    const uint32_t t = it->second.type;
+    if (t == T_F32 || t == T_F64 || t == T_STRING || t == T_ARRAY) return false;
+    *out = (int64_t)it->second.u;
+    return true;
+}
+bool GGUFLoader::getFloat(const std::string &key, double *out) const {
+    auto it = meta_.find(key);
+    if (it == meta_.end()) return false;
+    if (it->second.type == T_F32 || it->second.type == T_F64) { *out = it->second.f; return true; }
+    int64_t i;
+    if (getInt(key, &i)) { *out = (double)i; return true; }
+    return false;
+}
+bool GGUFLoader::getString(const std::string &key, std::string *out) const {
+    auto it = meta_.find(key);
+    if (it == meta_.end() || it->second.type != T_STRING) return false;
+    *out = it->second.s;
+    return true;
+}
+
+bool GGUFLoader::readTensor(const GGUFTensorInfo &t, std::vector<uint8_t> *out, std::string *error) const {
+    const size_t bytes = tensorBytes(t.type, t.elements());
+    if (!bytes) { if (error) *error = "tensor " + t.name + " has unsupported ggml type " + std::to_string(t.type); return false; }
+    if (data_start_ + t.offset + bytes > file_size_) { if (error) *error = "tensor " + t.name + " runs past the end of the file"; return false; }
+    FILE *f = std::fopen(path_.c_str(), "rb");
+    if (!f) { if (error) *error = "cannot reopen " + path_; return false; }
+    out->resize(bytes);
+    bool ok = std::fseek(f, (long)(data_start_ + t.offset), SEEK_SET) == 0 && std::fread(out->data(), 1, bytes, f) == bytes;
+    std::fclose(f);
+    if (!ok && error) *error = "short read of tensor " + t.name;
+    return ok;
+}
+
+int GGUFModelLoader::configFromMetadata(const GGUFLoader &g, MultiModelConfig *out) {
+    std::string arch;
+    if (!g.getString("general.architecture", &arch)) return fail(ESP_ERR_INVALID_ARGUMENT, "GGUF metadata lacks general.architecture");
+    std::string lower = arch;
+    for (char &ch : lower) ch = (char)std::tolower((unsigned char)ch);
+    MultiModelConfig c;
+    if (lower == "gpt2") c.architecture = MultiModelConfig::Architecture::gpt2;
+    else if (lower == "llama" || lower == "llama2" || lower == "llama3" || lower == "mistral" || lower == "qwen2" || lower == "qwen3")
+        c.architecture = MultiModelConfig::Architecture::llama;
+    else return fail(ESP_ERR_UNSUPPORTED, "unsupported architecture %s", arch.c_str());
+    c.name = arch;
+    auto need = [&](const std::string &key, int *dst) {
+        int64_t v;
+        if (!g.getInt(arch + "." + key, &v)) return fail(ESP_ERR_INVALID_ARGUMENT, "GGUF metadata lacks %s.%s", arch.c_str(), key.c_str());
+        *dst = (int)v;
+        return ESP_OK;
+    };
+    int rc;
+    if ((rc = need("block_count", &c.nLayer)) != ESP_OK) return rc;
+    if ((rc = need("attention.head_count", &c.nHead)) != ESP_OK) return rc;
+    if ((rc = need("embedding_length", &c.dModel)) != ESP_OK) return rc;
+    if ((rc = need("feed_forward_length", &c.hiddenDim)) != ESP_OK) return rc;
+    if ((rc = need("context_length", &c.maxSeq)) != ESP_OK) return rc;
+    int64_t v;
+    c.nKVHead = g.getInt(arch + ".attention.head_count_kv", &v) ? (int)v : c.nHead;
+    c.headDim = g.getInt(arch + ".attention.key_length", &v) ? (int)v : (c.nHead ? c.dModel / c.nHead : 0);
+    double f;
+    c.normEps = g.getFloat(arch + ".attention.layer_norm_rms_epsilon", &f) ? (float)f : 1e-5f;
+    c.ropeTheta = g.getFloat(arch + ".rope.freq_base", &f) ? (float)f : 10000.0f;                    // (:307-308)
+    auto tok = g.metadata().find("tokenizer.ggml.tokens");
+    if (tok != g.metadata().end() && tok->second.type == T_ARRAY) c.vocab = (int)tok->second.array_count;   // (:317-319)
+    else c.vocab = g.getInt(arch + ".vocab_size", &v) ? (int)v : 0;
+    if (g.getInt("tokenizer.ggml.eos_token_id", &v)) { c.hasEosToken = true; c.eosToken = (TokenID)v; }
+    *out = c;
+    return ESP_OK;
+}
+
+namespace {
+
+// fp32 values of a tensor stored as F32 / F16 / BF16 / a supported quantised type (decoded on the GPU)
+int tensor_to_float(const GGUFTensorInfo &t, const std::vector<uint8_t> &raw, std::vector<float> *out) {
+    const size_t n = (size_t)t.elements();
+    out->resize(n);
+    switch (t.type) {
+    case GGML_F32: std::memcpy(out->data(), raw.data(), n * 4); return ESP_OK;
+    case GGML_BF16:
+        for (size_t i = 0; i < n; i++) {
+            uint32_t bits = ((uint32_t)raw[2 * i] | ((uint32_t)raw[2 * i + 1] << 8)) << 16;
+            std::memcpy(&(*out)[i], &bits, 4);
+        }
+        return ESP_OK;
+    case GGML_F16: case GGML_Q4_0: case GGML_Q8_0: case GGML_Q4_K:
+        return esp_dequantize((int)t.type, raw.data(), n, out->data());
+    default: return fail(ESP_ERR_UNSUPPORTED, "tensor %s has unsupported ggml type %u", t.name.c_str(), t.type);
+    }
+}
+
+int write_blob_from_floats(const std::string &path, const std::vector<float> &v) {
+    const std::vector<uint8_t> blob = WeightBlob::build(v.data(), v.size());
+    return writeFile(path, blob.data(), blob.size()) ? ESP_OK : fail(ESP_ERR_IO, "cannot write %s", path.c_str());
+}
+
+// GGUF stores llama q/k projection rows interleaved per head for pairwise RoPE: stored row (h, j, s)
+// holds the half-split row (h, s, j), s in {0,1}, j < head_dim/2.  This restores the half-split order
+// that RoPE.applyDecodeStep assumes (Sources/CPUOps/RoPE.swift:56-110).  Rows are whole numbers of
+// quantisation blocks, so the reorder is a copy of row bytes.
+void undo_qk_interleave(std::vector<uint8_t> &raw, int heads, int head_dim, size_t row_bytes) {
+    std::vector<uint8_t> out(raw.size());
+    const int half = head_dim / 2;
+    for (int h = 0; h < heads; h++)
+        for (int s = 0; s < 2; s++)
+            for (int j = 0; j < half; j++)
+                std::memcpy(&out[(size_t)(h * head_dim + s * half + j) * row_bytes], &raw[(size_t)(h * head_dim + 2 * j + s) * row_bytes], row_bytes);
+    raw.swap(out);
+}
+
+}  // namespace
+
+int GGUFModelLoader::prepare(const std::string &ggufPath, const std::string &outputDir, const PrepareOptions &options,
+                             PreparedModel *out) {
+    GGUFLoader g;
+    std::string err;
+    if (!g.open(ggufPath, &err)) return fail(ESP_ERR_IO, "%s", err.c_str());
+    MultiModelConfig c;
+    int rc = configFromMetadata(g, &c);
+    if (rc != ESP_OK) return rc;
+    if (c.architecture != MultiModelConfig::Architecture::llama) return fail(ESP_ERR_UNSUPPORTED, "only llama-family GGUF files are prepared");
+    const std::string bad = validateRuntimeConfig(c);
+    if (!bad.empty()) return fail(ESP_ERR_INVALID_ARGUMENT, "%s", bad.c_str());
+    std::string arch_lower = c.name;
+    for (char &ch : arch_lower) ch = (char)std::tolower((unsigned char)ch);
+    const bool undo_interleave = options.qkLayout == 1 || (options.qkLayout < 0 && (arch_lower == "llama" || arch_lower == "llama2" ||
+                                                                                    arch_lower == "llama3" || arch_lower == "mistral"));
+    if (!makeDirectories(joinPath(outputDir, "embeddings"))) return fail(ESP_ERR_IO, "cannot create %s", outputDir.c_str());
+
+    int count = 0;
+    // name in the GGUF file -> path under the weight directory, matrix?, q/k head count for the re-order
+    auto convert = [&](const std::string &gguf_name, const std::string &rel, bool matrix, int qk_heads, bool optional) -> int {
+        const GGUFTensorInfo *t = g.find(gguf_name);
+        if (!t) return optional ? ESP_OK : fail(ESP_ERR_INVALID_ARGUMENT, "GGUF file lacks tensor %s", gguf_name.c_str());
+        std::vector<uint8_t> raw;
+        std::string e;
+        if (!g.readTensor(*t, &raw, &e)) return fail(ESP_ERR_UNSUPPORTED, "%s", e.c_str());
+        const std::string path = joinPath(outputDir, rel);
+        if (matrix && t->dims.size() == 2 && qk_heads > 0 && undo_interleave)
+            undo_qk_interleave(raw, qk_heads, c.headDim, raw.size() / (size_t)t->dims[1]);
+        const bool quantised = t->type == GGML_Q4_0 || t->type == GGML_Q8_0 || t->type == GGML_Q4_K;
+        const bool is_embedding = rel == "embeddings/token.bin";
+        if (matrix && quantised && !is_embedding) {
+            if (!writeFile(packedSidecarPath(path, (int)t->type), raw.data(), raw.size())) return fail(ESP_ERR_IO, "cannot write %s", path.c_str());
+            if (!options.emitDequantizedBlobs) { count++; return ESP_OK; }
+        }
+        if (t->type == GGML_F16) {
+            const std::vector<uint8_t> blob = WeightBlob::buildFP16(reinterpret_cast<const uint16_t *>(raw.data()), raw.size() / 2);
+            if (!writeFile(path, blob.data(), blob.size())) return fail(ESP_ERR_IO, "cannot write %s", path.c_str());
+        } else {
+            std::vector<float> values;
+            int r = tensor_to_float(*t, raw, &values);
+            if (r != ESP_OK) return r;
+            if ((r = write_blob_from_floats(path, values)) != ESP_OK) return r;
+            if (options.emitFloat32Sidecars && (t->type == GGML_F32 || t->type == GGML_BF16) &&
+                !writeFile(exactFloat32SidecarPath(path), values.data(), values.size() * 4))
+                return fail(ESP_ERR_IO, "cannot write %s", exactFloat32SidecarPath(path).c_str());
+        }
+        count++;
+        return ESP_OK;
+    };
+
+    if ((rc = convert("token_embd.weight", "embeddings/token.bin", true, 0, false)) != ESP_OK) return rc;
+    if ((rc = convert("output_norm.weight", "rms_final.bin", false, 0, false)) != ESP_OK) return rc;
+    if (g.find("output.weight")) {
+        if ((rc = convert("output.weight", "lm_head.bin", true, 0, false)) != ESP_OK) return rc;
+    } else {
+        // tied head: lm_head is the token embedding (materializeTiedLMHeadIfNeeded, :224-263); quantised
+        // embeddings keep their packed bytes as the head's packed sidecar
+        const GGUFTensorInfo *t = g.find("token_embd.weight");
+        std::vector<uint8_t> raw;
+        if (!readFile(joinPath(outputDir, "embeddings/token.bin"), &raw) || !writeFile(joinPath(outputDir, "lm_head.bin"), raw.data(), raw.size()))
+            return fail(ESP_ERR_IO, "cannot materialise tied lm_head");
+        if (t && (t->type == GGML_Q4_0 || t->type == GGML_Q8_0 || t->type == GGML_Q4_K)) {
+            std::string e;
+            if (!g.readTensor(*t, &raw, &e)) return fail(ESP_ERR_IO, "%s", e.c_str());
+            if (!writeFile(packedSidecarPath(joinPath(outputDir, "lm_head.bin"), (int)t->type), raw.data(), raw.size()))
+                return fail(ESP_ERR_IO, "cannot write tied lm_head sidecar");
+        }
+        const std::string emb_sidecar = exactFloat32SidecarPath(joinPath(outputDir, "embeddings/token.bin"));
+        if (fileExists(emb_sidecar) && readFile(emb_sidecar, &raw))
+            writeFile(exactFloat32SidecarPath(joinPath(outputDir, "lm_head.bin")), raw.data(), raw.size());
+    }
+    for (int l = 0; l < c.nLayer; l++) {
+        const std::string b = "blk." + std::to_string(l) + ".", d = "layers/" + std::to_string(l) + "/";
+        if (!makeDirectories(joinPath(outputDir, "layers/" + std::to_string(l)))) return fail(ESP_ERR_IO, "cannot create layer directory");
+        if ((rc = convert(b + "attn_norm.weight", d + "rms_att.bin", false, 0, false)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_q.weight", d + "wq.bin", true, c.nHead, false)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_k.weight", d + "wk.bin", true, c.nKVHead, false)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_v.weight", d + "wv.bin", true, 0, false)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_output.weight", d + "wo.bin", true, 0, false)) != ESP_OK) return rc;
+        if ((rc = convert(b + "ffn_norm.weight", d + "rms_ffn.bin", false, 0, false)) != ESP_OK) return rc;
+        if ((rc = convert(b + "ffn_gate.weight", d + "w1.bin", true, 0, false)) != ESP_OK) return rc;
+        if ((rc = convert(b + "ffn_down.weight", d + "w2.bin", true, 0, false)) != ESP_OK) return rc;
+        if ((rc = convert(b + "ffn_up.weight", d + "w3.bin", true, 0, false)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_q_norm.weight", d + "q_norm.bin", false, 0, true)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_k_norm.weight", d + "k_norm.bin", false, 0, true)) != ESP_OK) return rc;
+    }
+    if (count == 0) return fail(ESP_ERR_INVALID_ARGUMENT, "no tensors converted");
+    const std::string meta = metadataJSON(c);
+    if (!writeFile(joinPath(outputDir, "metadata.json"), meta.data(), meta.size())) return fail(ESP_ERR_IO, "cannot write metadata.json");
+    const std::string manifest = "{\n  \"source\": \"" + ggufPath + "\",\n  \"tensorCount\": " + std::to_string(count) + "\n}\n";
+    writeFile(joinPath(outputDir, "prepare-manifest.json"), manifest.data(), manifest.size());
+    out->config = c;
+    out->weightDir = outputDir;
+    out->tensorCount = count;
+    return ESP_OK;
+}
+
+}  // namespace esp

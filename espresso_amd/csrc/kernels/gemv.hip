@@ -100,6 +100,8 @@ struct Traits<FMT_Q4_0> { static constexpr int kItemElems = 32; static constexpr
 template <>
 struct Traits<FMT_Q8_0> { static constexpr int kItemElems = 16; static constexpr bool kPermuteX = true; static constexpr bool kXSums = false; };
 template <>
+struct Traits<FMT_F32> { static constexpr int kItemElems = 4; static constexpr bool kPermuteX = false; static constexpr bool kXSums = false; };
+template <>
 struct Traits<FMT_F16> { static constexpr int kItemElems = 8; static constexpr bool kPermuteX = false; static constexpr bool kXSums = false; };
 
 struct KernelArgs {
@@ -305,6 +307,25 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
                         byte_dword(dword_of(q, k), as_h2(dword_of(v, (k & 1) * 2)), as_h2(dword_of(v, (k & 1) * 2 + 1)), dot);
                     }
                     acc[r][b] += d * dot;
+                }
+            }
+        } else if constexpr (FMT == FMT_F32) {
+            // exact fp32 weights (float32 sidecars): four weights per 128-bit load, plain fp32 multiply-adds
+            const int e0 = item * 4;
+            uint2 xv[B];
+#pragma unroll
+            for (int b = 0; b < B; b++) xv[b] = *reinterpret_cast<const uint2 *>(xs + (size_t)b * cols + e0);
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const uint4 q = *reinterpret_cast<const uint4 *>(rowp[r] + (size_t)item * 16);
+#pragma unroll
+                for (int b = 0; b < B; b++) {
+                    const h2 x01 = as_h2(xv[b].x), x23 = as_h2(xv[b].y);
+                    float dot = __uint_as_float(q.x) * (float)x01.x;
+                    dot += __uint_as_float(q.y) * (float)x01.y;
+                    dot += __uint_as_float(q.z) * (float)x23.x;
+                    dot += __uint_as_float(q.w) * (float)x23.y;
+                    acc[r][b] += dot;
                 }
             }
         } else {  // FMT_F16
@@ -581,7 +602,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
             w.rows != (q.n_head + 2 * q.n_kv_head) * q.head_dim)
             return hipErrorInvalidValue;
     }
-    const int block = w.format == FMT_F16 ? 8 : format_block_elems(w.format);
+    const int block = w.format == FMT_F16 ? 8 : w.format == FMT_F32 ? 4 : format_block_elems(w.format);
     if (w.cols % block != 0 || w.qs_row_bytes % 16 != 0) return hipErrorInvalidValue;
     if ((w.format == FMT_Q8_0 || w.format == FMT_Q4_0) && !w.scales) return hipErrorInvalidValue;
 
@@ -607,6 +628,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         case FMT_Q4_0: e = launch_fmt<FMT_Q4_0>(a, nb, stream); break;
         case FMT_Q8_0: e = launch_fmt<FMT_Q8_0>(a, nb, stream); break;
         case FMT_F16: e = launch_fmt<FMT_F16>(a, nb, stream); break;
+        case FMT_F32: e = launch_fmt<FMT_F32>(a, nb, stream); break;
         default: e = hipErrorInvalidValue;
         }
         if (e != hipSuccess) return e;

@@ -1,0 +1,212 @@
+"""ctypes face of the host layer: weight files, metadata, GGUF prepare, the engine and the exact
+two-token harness (declared in include/espresso_hip.h)."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib, llama
+
+
+class ModelConfigStruct(C.Structure):
+    _fields_ = [("name", C.c_char * 64)] + \
+               [(n, C.c_int32) for n in ("n_layer", "n_head", "n_kv_head", "d_model", "head_dim", "hidden_dim", "vocab", "max_seq")] + \
+               [("norm_eps", C.c_float), ("rope_theta", C.c_float), ("eos_token", C.c_int32), ("architecture", C.c_int32)]
+
+
+class PrepareOptionsStruct(C.Structure):
+    _fields_ = [("emit_dequantized_blobs", C.c_int32), ("emit_float32_sidecars", C.c_int32), ("qk_layout", C.c_int32)]
+
+
+class GenerationResultStruct(C.Structure):
+    _fields_ = [("token_count", C.c_int32), ("tokens_per_second", C.c_double), ("compile_time_ms", C.c_double),
+                ("first_token_latency_ms", C.c_double), ("has_two_token_stats", C.c_int32),
+                ("committed_exact_tokens_per_pass", C.c_double), ("accepted_future_tokens_per_pass", C.c_double),
+                ("exact_head_backend", C.c_char * 48)]
+
+
+class PromotionPlanStruct(C.Structure):
+    _fields_ = [("committed_tokens", C.c_uint32 * 2), ("committed_exact_token_count", C.c_int32),
+                ("accepted_future_token_count", C.c_int32), ("promoted_step_count", C.c_int32), ("next_current_token", C.c_uint32)]
+
+
+class PassResultStruct(C.Structure):
+    _fields_ = [("committed_tokens", C.c_uint32 * 2), ("committed_count", C.c_int32), ("next_current_token", C.c_uint32),
+                ("proposer_latency_ms", C.c_double), ("verifier_trunk_latency_ms", C.c_double),
+                ("verifier_logits_latency_ms", C.c_double), ("state_advance_latency_ms", C.c_double),
+                ("accepted_future_token_count", C.c_int32), ("committed_exact_token_count", C.c_int32)]
+
+
+RESET_FN = C.CFUNCTYPE(C.c_int, C.c_void_p)
+PREFILL_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.c_uint32), C.c_int, C.POINTER(C.c_uint32))
+PASS_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_uint32, C.c_int, C.POINTER(PassResultStruct))
+
+
+class ExactTwoTokenModelStruct(C.Structure):
+    _fields_ = [("context", C.c_void_p), ("reset", RESET_FN), ("prefill_selected_token", PREFILL_FN),
+                ("perform_exact_two_token_pass", PASS_FN)]
+
+
+_declared = False
+
+
+def _L():
+    global _declared
+    L = _lib.load_library()
+    if _declared:
+        return L
+    vp, sz, i32, cp = C.c_void_p, C.c_size_t, C.c_int, C.c_char_p
+    L.esp_weight_blob_bytes.restype = sz; L.esp_weight_blob_bytes.argtypes = [sz]
+    L.esp_weight_blob_build.restype = i32; L.esp_weight_blob_build.argtypes = [vp, sz, vp]
+    L.esp_blob_weight_load.restype = C.c_long; L.esp_blob_weight_load.argtypes = [cp, vp, sz]
+    L.esp_layer_weight_path.restype = i32; L.esp_layer_weight_path.argtypes = [i32, cp, i32, cp, sz]
+    L.esp_model_config_load_metadata.restype = i32; L.esp_model_config_load_metadata.argtypes = [cp, C.POINTER(ModelConfigStruct)]
+    L.esp_model_config_write_metadata.restype = i32; L.esp_model_config_write_metadata.argtypes = [C.POINTER(ModelConfigStruct), cp]
+    L.esp_gguf_prepare.restype = i32
+    L.esp_gguf_prepare.argtypes = [cp, cp, C.POINTER(PrepareOptionsStruct), C.POINTER(ModelConfigStruct), C.POINTER(i32)]
+    L.esp_engine_build.restype = vp
+    L.esp_engine_build.argtypes = [C.POINTER(ModelConfigStruct), cp, cp, C.POINTER(cp), C.POINTER(cp), i32]
+    L.esp_engine_free.argtypes = [vp]
+    L.esp_engine_runtime.restype = vp; L.esp_engine_runtime.argtypes = [vp]
+    L.esp_engine_generate.restype = i32
+    L.esp_engine_generate.argtypes = [vp, vp, i32, i32, C.c_float, C.POINTER(cp), C.POINTER(cp), i32, vp, C.POINTER(GenerationResultStruct)]
+    L.esp_exact_two_token_promotion_plan.argtypes = [C.c_uint32] * 4 + [i32, C.POINTER(PromotionPlanStruct)]
+    L.esp_exact_two_token_harness_generate.restype = i32
+    L.esp_exact_two_token_harness_generate.argtypes = [C.POINTER(ExactTwoTokenModelStruct), vp, vp, vp, i32, i32, vp, C.POINTER(i32), vp, vp, C.POINTER(i32)]
+    _declared = True
+    return L
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def config_struct(cfg: llama.MultiModelConfig) -> ModelConfigStruct:
+    return ModelConfigStruct(cfg.name.encode()[:63], cfg.n_layer, cfg.n_head, cfg.n_kv_head, cfg.d_model, cfg.head_dim, cfg.hidden_dim,
+                             cfg.vocab, cfg.max_seq, cfg.norm_eps, cfg.rope_theta, cfg.eos_token, 1)
+
+
+def config_from_struct(s: ModelConfigStruct) -> llama.MultiModelConfig:
+    return llama.MultiModelConfig(n_layer=s.n_layer, n_head=s.n_head, n_kv_head=s.n_kv_head, d_model=s.d_model, head_dim=s.head_dim,
+                                  hidden_dim=s.hidden_dim, vocab=s.vocab, max_seq=s.max_seq, norm_eps=s.norm_eps,
+                                  rope_theta=s.rope_theta, eos_token=s.eos_token, name=s.name.decode())
+
+
+# ---- weight files -----------------------------------------------------------
+def weight_blob_build(weights) -> bytes:
+    w = np.ascontiguousarray(weights, dtype=np.float32).ravel()
+    out = np.zeros(int(_L().esp_weight_blob_bytes(w.size)), dtype=np.uint8)
+    _lib.check(_L().esp_weight_blob_build(_ptr(w), w.size, _ptr(out)))
+    return out.tobytes()
+
+
+def blob_weight_load(path: str):
+    """Returns (count_or_negative_error, values)."""
+    n = _L().esp_blob_weight_load(path.encode(), None, 0)
+    if n < 0:
+        return int(n), None
+    out = np.empty(n, dtype=np.float32)
+    _L().esp_blob_weight_load(path.encode(), _ptr(out), n)
+    return int(n), out
+
+
+def layer_weight_path(layer: int, blob_dir: str, slot: int) -> str:
+    buf = C.create_string_buffer(4096)
+    n = _L().esp_layer_weight_path(layer, blob_dir.encode(), slot, buf, 4096)
+    if n < 0:
+        raise _lib.EspressoError(n, _lib.last_error())
+    return buf.value.decode()
+
+
+def load_metadata(path: str) -> llama.MultiModelConfig:
+    s = ModelConfigStruct()
+    _lib.check(_L().esp_model_config_load_metadata(path.encode(), C.byref(s)))
+    return config_from_struct(s)
+
+
+def write_metadata(cfg: llama.MultiModelConfig, path: str) -> None:
+    s = config_struct(cfg)
+    _lib.check(_L().esp_model_config_write_metadata(C.byref(s), path.encode()))
+
+
+# ---- GGUF ---------------------------------------------------------------------
+def gguf_prepare(gguf_path: str, output_dir: str, emit_dequantized_blobs=False, emit_float32_sidecars=True, qk_layout=-1):
+    """GGUFModelLoader.prepare -> (config, weight_dir, tensor_count)."""
+    opt = PrepareOptionsStruct(int(emit_dequantized_blobs), int(emit_float32_sidecars), qk_layout)
+    s, n = ModelConfigStruct(), C.c_int(0)
+    _lib.check(_L().esp_gguf_prepare(gguf_path.encode(), output_dir.encode(), C.byref(opt), C.byref(s), C.byref(n)))
+    return config_from_struct(s), output_dir, n.value
+
+
+# ---- engine ---------------------------------------------------------------------
+def _env_arrays(env: dict | None):
+    env = env or {}
+    keys = (C.c_char_p * max(len(env), 1))(*[k.encode() for k in env])
+    vals = (C.c_char_p * max(len(env), 1))(*[v.encode() for v in env.values()])
+    return keys, vals, len(env)
+
+
+class RealModelInferenceEngine:
+    """RealModelInferenceEngine.build / generate (token-id form)."""
+
+    def __init__(self, cfg: llama.MultiModelConfig, weight_dir: str, tokenizer_dir: str | None = None, environment: dict | None = None):
+        self.cfg = cfg
+        s = config_struct(cfg)
+        k, v, n = _env_arrays(environment)
+        self._h = _L().esp_engine_build(C.byref(s), weight_dir.encode(), tokenizer_dir.encode() if tokenizer_dir else None, k, v, n)
+        if not self._h:
+            raise _lib.EspressoError(-1, _lib.last_error())
+
+    def close(self):
+        if self._h:
+            _L().esp_engine_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def generate(self, prompt_tokens, max_tokens: int, temperature: float = 0.0, environment: dict | None = None):
+        p = np.ascontiguousarray(prompt_tokens, dtype=np.uint32)
+        out = np.zeros(max(max_tokens, 1), dtype=np.uint32)
+        r = GenerationResultStruct()
+        k, v, n = _env_arrays(environment)
+        _lib.check(_L().esp_engine_generate(self._h, _ptr(p), p.size, max_tokens, C.c_float(temperature), k, v, n, _ptr(out), C.byref(r)))
+        res = {f: getattr(r, f) for f, _ in r._fields_}
+        res["exact_head_backend"] = r.exact_head_backend.decode()
+        return out[:r.token_count].tolist(), res
+
+    def runtime(self) -> llama.LlamaRuntime:
+        """A non-owning view of the engine's runtime."""
+        rt = llama.LlamaRuntime.__new__(llama.LlamaRuntime)
+        rt.cfg, rt._L, rt._h = self.cfg, _L(), _L().esp_engine_runtime(self._h)
+        rt.close = lambda: None
+        return rt
+
+
+# ---- exact two-token harness -----------------------------------------------------
+def promotion_plan(current, proposed, exact_next, exact_future, budget) -> dict:
+    p = PromotionPlanStruct()
+    _L().esp_exact_two_token_promotion_plan(current, proposed, exact_next, exact_future, budget, C.byref(p))
+    return {"committed_tokens": list(p.committed_tokens)[:p.committed_exact_token_count], "next_current_token": p.next_current_token,
+            "committed_exact_token_count": p.committed_exact_token_count, "accepted_future_token_count": p.accepted_future_token_count,
+            "promoted_step_count": p.promoted_step_count}
+
+
+def harness_generate(prompt_tokens, max_new_tokens: int, model: ExactTwoTokenModelStruct | None = None,
+                     target: llama.LlamaRuntime | None = None, draft: llama.LlamaRuntime | None = None):
+    """ExactTwoTokenGenerationHarness.generate -> (tokens, committed per pass, accepted per pass)."""
+    p = np.ascontiguousarray(prompt_tokens, dtype=np.uint32)
+    cap = max(max_new_tokens, 1)
+    out = np.zeros(cap + 1, dtype=np.uint32)
+    com, acc = np.zeros(cap, dtype=np.int32), np.zeros(cap, dtype=np.int32)
+    n, passes = C.c_int(0), C.c_int(0)
+    _lib.check(_L().esp_exact_two_token_harness_generate(C.byref(model) if model is not None else None,
+                                                         target._h if target is not None else None,
+                                                         draft._h if draft is not None else None,
+                                                         _ptr(p), p.size, max_new_tokens, _ptr(out), C.byref(n), _ptr(com), _ptr(acc),
+                                                         C.byref(passes)))
+    return out[:n.value].tolist(), com[:passes.value].tolist(), acc[:passes.value].tolist()

@@ -201,6 +201,109 @@ int esp_llama_kernel_times(ESPLlamaRuntime *runtime, double *total_us, int64_t *
  * elements must be a multiple of 256.  Formats: F16, Q8_0, Q4_0, Q4_K. */
 int esp_synth_weights(int format, uint64_t seed, float std_dev, size_t elements, void *out_blocks);
 
+/* ---- weight files ------------------------------------------------------------------------------- *
+ * BLOBFILE: 128-byte header + little-endian fp16 payload (Sources/ANETypes/WeightBlob.swift:6-38,
+ * Sources/ModelSupport/BlobWeightLoader.swift:25-90).  Pure host code; no GPU needed. */
+size_t esp_weight_blob_bytes(size_t element_count);
+/* WeightBlob.build(from:rows:cols:): fp32 -> fp16 round-to-nearest-even.  `out` holds esp_weight_blob_bytes(count). */
+int esp_weight_blob_build(const float *weights, size_t element_count, uint8_t *out);
+/* BlobWeightLoader.load(from:): returns the element count, or -(1 + BlobWeightLoaderError ordinal):
+ * -1 truncatedHeader, -2 invalidMagic, -3 invalidDataOffset, -4 truncatedPayload, -5 invalidPayloadSize, -6 file unreadable.
+ * `out` may be NULL to query the count. */
+long esp_blob_weight_load(const char *path, float *out, size_t capacity);
+/* LayerWeightPaths.forLayer(_:config:blobDir:) for one ESP_SLOT_* of a llama layer
+ * (Sources/ModelSupport/LayerWeightPaths.swift:56-84).  Returns the length written, or ESP_ERR_*. */
+int esp_layer_weight_path(int layer, const char *blob_dir, int slot, char *out, size_t capacity);
+
+/* MultiModelConfig (Sources/ModelSupport/MultiModelConfig.swift:3-55). */
+typedef struct ESPModelConfig {
+    char name[64];
+    int32_t n_layer, n_head, n_kv_head, d_model, head_dim, hidden_dim, vocab, max_seq;
+    float norm_eps, rope_theta;
+    int32_t eos_token;     /* -1: none */
+    int32_t architecture;  /* 0 gpt2, 1 llama */
+} ESPModelConfig;
+/* metadata.json as GGUFModelLoader writes it (GGUFModelLoader.swift:203-222) and the engine validates it
+ * (RealModelInferenceEngine.swift:7658-7694). */
+int esp_model_config_load_metadata(const char *metadata_json_path, ESPModelConfig *out);
+int esp_model_config_write_metadata(const ESPModelConfig *config, const char *metadata_json_path);
+
+/* ---- GGUF front door ---------------------------------------------------------------------------- *
+ * GGUFModelLoader.prepare(ggufURL:options:) -> PreparedModel (GGUFModelLoader.swift:273-405): parses
+ * the GGUF container, maps its metadata to a MultiModelConfig (:297-326) and writes a weight directory:
+ * fp16 BLOBFILEs for norms and the embedding, exact float32 sidecars for F32/BF16 tensors, and for each
+ * quantised projection a packed sidecar "<stem>.<q8_0|q4_0|q4_k>.bin" holding the GGUF blocks unchanged,
+ * which esp_engine_build uploads as they are.  emit_dequantized_blobs != 0 additionally writes the fp16
+ * BLOBFILE of every quantised projection (the artefact the reference's own engine reads).
+ * qk_layout: -1 by architecture, 0 keep rows as stored, 1 undo the GGUF llama Q/K row interleave. */
+typedef struct ESPPrepareOptions {
+    int32_t emit_dequantized_blobs;
+    int32_t emit_float32_sidecars;
+    int32_t qk_layout;
+} ESPPrepareOptions;
+int esp_gguf_prepare(const char *gguf_path, const char *output_dir, const ESPPrepareOptions *options_or_null,
+                     ESPModelConfig *out_config, int *out_tensor_count);
+
+/* ---- engine -------------------------------------------------------------------------------------- *
+ * RealModelInferenceEngine.build(config:weightDir:tokenizerDir:) (RealModelInferenceEngine.swift:1377):
+ * loads the weight directory into HBM (per tensor: packed sidecar, else float32 sidecar, else fp16
+ * BLOBFILE).  Environment entries are passed as parallel key/value arrays, as the reference's functions
+ * take an `environment:` dictionary.  Recognised: ESPRESSO_BUNDLE_DRAFT_KIND / _HORIZON / _ARTIFACT_REF
+ * (:5324-5390), ESPRESSO_HIP_KV_CACHE=f16. */
+typedef struct ESPEngine ESPEngine;
+ESPEngine *esp_engine_build(const ESPModelConfig *config, const char *weight_dir, const char *tokenizer_dir_or_null,
+                            const char *const *env_keys, const char *const *env_values, int env_count);
+void esp_engine_free(ESPEngine *engine);
+
+/* GenerationResult (:17-55) without text. */
+typedef struct ESPGenerationResult {
+    int32_t token_count;
+    double tokens_per_second, compile_time_ms, first_token_latency_ms;
+    int32_t has_two_token_stats;
+    double committed_exact_tokens_per_pass, accepted_future_tokens_per_pass;
+    char exact_head_backend[48];
+} ESPGenerationResult;
+/* generate(prompt:maxTokens:temperature:) in its token-id form (:1405-1493): greedy decode, or the exact
+ * two-token draft loop when the environment names a draft.  out_tokens holds max_tokens ids. */
+int esp_engine_generate(ESPEngine *engine, const uint32_t *prompt_tokens, int prompt_count, int max_tokens, float temperature,
+                        const char *const *env_keys, const char *const *env_values, int env_count,
+                        uint32_t *out_tokens, ESPGenerationResult *result);
+/* The runtime inside the engine (owned by the engine). */
+ESPLlamaRuntime *esp_engine_runtime(ESPEngine *engine);
+
+/* ---- exact two-token harness ---------------------------------------------------------------------- *
+ * ExactTwoTokenBranchPromotionPlan.make (Sources/Espresso/GenerationHarness.swift:149-180). */
+typedef struct ESPPromotionPlan {
+    uint32_t committed_tokens[2];
+    int32_t committed_exact_token_count, accepted_future_token_count, promoted_step_count;
+    uint32_t next_current_token;
+} ESPPromotionPlan;
+void esp_exact_two_token_promotion_plan(uint32_t current_token, uint32_t proposed_future_token, uint32_t exact_next_token,
+                                        uint32_t exact_future_token, int remaining_token_budget, ESPPromotionPlan *out);
+
+/* ExactTwoTokenPassMetrics / ExactTwoTokenPassResult (:104-147) */
+typedef struct ESPPassResult {
+    uint32_t committed_tokens[2];
+    int32_t committed_count;
+    uint32_t next_current_token;
+    double proposer_latency_ms, verifier_trunk_latency_ms, verifier_logits_latency_ms, state_advance_latency_ms;
+    int32_t accepted_future_token_count, committed_exact_token_count;
+} ESPPassResult;
+/* ExactTwoTokenGeneratingLanguageModel (:239-252) as a table of callbacks; each returns 0 on success. */
+typedef struct ESPExactTwoTokenModel {
+    void *context;
+    int (*reset)(void *context);
+    int (*prefill_selected_token)(void *context, const uint32_t *prompt_tokens, int count, uint32_t *selected);
+    int (*perform_exact_two_token_pass)(void *context, uint32_t current_token, int remaining_token_budget, ESPPassResult *result);
+} ESPExactTwoTokenModel;
+/* ExactTwoTokenGenerationHarness.generate (:612-686): drives `model`, enforcing the pass invariants.
+ * out_tokens holds max_new_tokens + 1 ids; pass arrays hold max_new_tokens entries.  `model` NULL with
+ * target/draft runtimes given runs the GPU model (batched verify of [current, proposed]). */
+int esp_exact_two_token_harness_generate(const ESPExactTwoTokenModel *model, ESPLlamaRuntime *target, ESPLlamaRuntime *draft,
+                                         const uint32_t *prompt_tokens, int prompt_count, int max_new_tokens,
+                                         uint32_t *out_tokens, int *out_token_count, int32_t *out_committed_per_pass,
+                                         int32_t *out_accepted_per_pass, int *out_pass_count);
+
 #ifdef __cplusplus
 }
 #endif

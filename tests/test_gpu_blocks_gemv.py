@@ -8,7 +8,7 @@ from oracle import oracle as orc
 pytestmark = pytest.mark.gpu
 
 FORMATS = {"q8_0": (orc.FMT_Q8_0, 34, 32), "q4_0": (orc.FMT_Q4_0, 18, 32), "q4_k": (orc.FMT_Q4_K, 144, 256),
-           "f16": (orc.FMT_F16, 2, 1)}
+           "f16": (orc.FMT_F16, 2, 1), "f32": (orc.FMT_F32, 4, 1)}
 
 
 def _bits(a):
@@ -79,7 +79,7 @@ def _quantized(fmt, rows, cols, seed):
 @pytest.mark.parametrize("name,rows,cols", [
     ("q8_0", 768, 768), ("q8_0", 2048, 768), ("q8_0", 768, 2048), ("q8_0", 1003, 96),
     ("q4_0", 1024, 4096), ("q4_0", 515, 256), ("q4_k", 1024, 4096), ("q4_k", 257, 1024), ("q4_k", 64, 14336),
-    ("f16", 768, 768), ("f16", 333, 2048),
+    ("f16", 768, 768), ("f16", 333, 2048), ("f32", 301, 512),
 ])
 @pytest.mark.parametrize("batch", [1, 2])
 def test_gemv_matches_oracle(ops, name, rows, cols, batch):
@@ -127,5 +127,5 @@ def test_gemv_argument_errors(ops):
         ops.Matrix(orc.FMT_Q4_K, np.zeros(100, np.uint8), 4, 256)                 # wrong byte count
     with pytest.raises(ValueError):
         ops.Matrix(orc.FMT_Q4_K, np.zeros(144, np.uint8), 1, 100)                 # ragged cols
-    with pytest.raises(lib.EspressoError):
-        ops.Matrix(orc.FMT_F32, np.zeros(4 * 64, np.uint8), 1, 64)                # no fp32 GEMV kernel
+    with pytest.raises(ValueError):
+        ops.Matrix(7, np.zeros(4 * 64, np.uint8), 1, 64)                          # unknown format

@@ -1,0 +1,282 @@
+"""GPU: the engine built from a weight directory (BLOBFILEs, float32 sidecars, packed sidecars), the
+GGUF front door, the draft selection through the environment, and the exact two-token harness."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import model_util as mu
+from gguf_writer import write_gguf
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+KW = dict(n_layer=2, n_head=4, n_kv_head=2, d_model=256, head_dim=64, hidden_dim=512, vocab=512, max_seq=48)
+PROMPT = [3, 141, 59, 26, 5]
+
+
+@pytest.fixture(scope="module")
+def E():
+    import espresso_amd.engine as eng
+    import espresso_amd.ops as ops
+    ops.init()
+    return eng
+
+
+def gpu_cfg(kw, **extra):
+    import espresso_amd.llama as ll
+    return ll.MultiModelConfig(**kw, **extra)
+
+
+def write_weight_dir(root, kw, w, f32_sidecars=False, packed_fmt=None, names=("embedding", "final_norm", "lm_head")):
+    """Writes the reference's directory layout; returns the fp32 values an exact CPU run would see."""
+    import espresso_amd.engine as eng
+    os.makedirs(os.path.join(root, "embeddings"), exist_ok=True)
+    seen = {"layers": []}
+
+    def put(rel, a, matrix):
+        path = os.path.join(root, rel)
+        open(path, "wb").write(orc.blob_build(a))
+        val = a.astype(np.float16).astype(np.float32)
+        if f32_sidecars:
+            a.astype("<f4").tofile(path[:-4] + ".float32.bin")
+            val = a
+        if matrix and packed_fmt is not None:
+            blocks = orc.quantize(packed_fmt, a)
+            tag = {orc.FMT_Q8_0: "q8_0", orc.FMT_Q4_0: "q4_0", orc.FMT_Q4_K: "q4_k"}[packed_fmt]
+            blocks.tofile(path[:-4] + f".{tag}.bin")
+            val = orc.dequantize(packed_fmt, blocks, a.size).reshape(a.shape)
+        return val
+
+    seen["embedding"] = put("embeddings/token.bin", w["embedding"], False)
+    seen["final_norm"] = put("rms_final.bin", w["final_norm"], False)
+    seen["lm_head"] = put("lm_head.bin", w["lm_head"], True)
+    for l, L in enumerate(w["layers"]):
+        os.makedirs(os.path.join(root, "layers", str(l)), exist_ok=True)
+        seen["layers"].append({k: put(f"layers/{l}/{k}.bin", a, k in mu.MATRICES) for k, a in L.items()})
+    eng.write_metadata(gpu_cfg(kw), os.path.join(root, "metadata.json"))
+    return seen
+
+
+def oracle_tokens(kw, seen, prompt, n, **flags):
+    return mu.load_oracle(orc.LlamaConfig(gemv_inputs_fp16=True, **kw, **flags), seen).generate(prompt, n)
+
+
+@pytest.mark.parametrize("mode", ["blobs", "float32_sidecars", "packed_q8_0", "packed_q4_k"])
+def test_engine_from_weight_directory(E, tmp_path, mode):
+    w = mu.random_weights(orc.LlamaConfig(**KW), 41, std=0.08, norm_jitter=0.05)
+    seen = write_weight_dir(str(tmp_path), KW, w, f32_sidecars=mode == "float32_sidecars",
+                            packed_fmt={"packed_q8_0": orc.FMT_Q8_0, "packed_q4_k": orc.FMT_Q4_K}.get(mode))
+    e = E.RealModelInferenceEngine(gpu_cfg(KW), str(tmp_path), tokenizer_dir=None)
+    toks, res = e.generate(PROMPT, 20)
+    assert toks == oracle_tokens(KW, seen, PROMPT, 20)
+    assert res["token_count"] == 20 and res["exact_head_backend"] == "hip_gemv_argmax" and res["has_two_token_stats"] == 0
+    assert res["compile_time_ms"] > 0 and res["tokens_per_second"] > 0
+    # maxTokens is clipped to the context (RealModelInferenceEngine.swift:1425-1426); zero budget returns nothing
+    assert len(e.generate(PROMPT, 1000)[0]) == KW["max_seq"] - len(PROMPT)
+    assert e.generate(PROMPT, 0)[0] == []
+    e.close()
+
+
+def test_engine_errors(E, tmp_path):
+    import espresso_amd._lib as lib
+    w = mu.random_weights(orc.LlamaConfig(**KW), 42, std=0.08)
+    write_weight_dir(str(tmp_path), KW, w)
+    with pytest.raises(lib.EspressoError, match="missing path"):
+        E.RealModelInferenceEngine(gpu_cfg(KW), str(tmp_path / "nope"))
+    with pytest.raises(lib.EspressoError, match="does not match config"):
+        E.RealModelInferenceEngine(gpu_cfg(dict(KW, n_layer=3)), str(tmp_path))                 # metadata.json disagrees
+    e = E.RealModelInferenceEngine(gpu_cfg(KW), str(tmp_path))
+    with pytest.raises(lib.EspressoError, match="must not be empty"):
+        e.generate([], 4)
+    with pytest.raises(lib.EspressoError, match="maxTokens"):
+        e.generate(PROMPT, -1)
+    with pytest.raises(lib.EspressoError, match="temperature"):
+        e.generate(PROMPT, 4, temperature=float("nan"))
+    with pytest.raises(lib.EspressoError, match="does not fit context"):
+        e.generate(list(range(KW["max_seq"])), 4)
+    e.close()
+    os.remove(tmp_path / "layers" / "1" / "w2.bin")
+    with pytest.raises(lib.EspressoError, match="missing weight file"):
+        E.RealModelInferenceEngine(gpu_cfg(KW), str(tmp_path))
+    os.remove(tmp_path / "lm_head.bin")
+    with pytest.raises(lib.EspressoError, match="missing lm head"):
+        E.RealModelInferenceEngine(gpu_cfg(KW), str(tmp_path))
+
+
+def test_exact_two_token_draft_through_environment(E, tmp_path):
+    """ESPRESSO_BUNDLE_DRAFT_* -> descriptor JSON -> draft directory (RealModelInferenceEngine.swift:5324-5390)."""
+    import espresso_amd._lib as lib
+    root = tmp_path / "bundle"
+    wdir = root / "weights"
+    full_kw, draft_kw = dict(KW, n_layer=3), dict(KW, n_layer=1)
+    wf = mu.random_weights(orc.LlamaConfig(**full_kw), 51, std=0.08)
+    wd = mu.random_weights(orc.LlamaConfig(**draft_kw), 52, std=0.08)
+    os.makedirs(wdir)
+    seen_f = write_weight_dir(str(wdir), full_kw, wf)
+    seen_d = write_weight_dir(str(wdir / "draft"), draft_kw, wd)
+    (root / "draft.json").write_text(json.dumps({"model_dir": "draft", "tokenizer_dir": None, "model_id": "d"}))
+    env = {"ESPRESSO_BUNDLE_DRAFT_KIND": "exact_two_token", "ESPRESSO_BUNDLE_DRAFT_HORIZON": "2",
+           "ESPRESSO_BUNDLE_DRAFT_ARTIFACT_REF": "draft.json"}
+    e = E.RealModelInferenceEngine(gpu_cfg(full_kw), str(wdir))
+    plain, _ = e.generate(PROMPT, 24)
+    toks, res = e.generate(PROMPT, 24, environment=env)
+    of = mu.load_oracle(orc.LlamaConfig(gemv_inputs_fp16=True, **full_kw), seen_f)
+    od = mu.load_oracle(orc.LlamaConfig(gemv_inputs_fp16=True, **draft_kw), seen_d)
+    want, st = orc.generate_two_token(of, od, PROMPT, 24)
+    assert toks == plain == want
+    assert res["exact_head_backend"] == "hip_exact_two_token_draft" and res["has_two_token_stats"] == 1
+    assert res["committed_exact_tokens_per_pass"] == pytest.approx(st["committed_total"] / st["passes"])
+    assert res["accepted_future_tokens_per_pass"] == pytest.approx(st["accepted_total"] / st["passes"])
+    for bad_env, message in [(dict(env, ESPRESSO_BUNDLE_DRAFT_HORIZON="3"), "horizon == 2"),
+                             (dict(env, ESPRESSO_BUNDLE_DRAFT_ARTIFACT_REF="../x.json"), "escapes bundle root"),
+                             (dict(env, ESPRESSO_BUNDLE_DRAFT_ARTIFACT_REF="none.json"), "is missing"),
+                             ({"ESPRESSO_BUNDLE_DRAFT_KIND": "exact_two_token"}, "requires ESPRESSO_BUNDLE_DRAFT_ARTIFACT_REF")]:
+        with pytest.raises(lib.EspressoError, match=message):
+            e.generate(PROMPT, 4, environment=bad_env)
+    (root / "draft.json").write_text(json.dumps({"model_dir": "../elsewhere"}))
+    with pytest.raises(lib.EspressoError, match="escapes weights root"):
+        e.generate(PROMPT, 4, environment=env)
+    small = dict(draft_kw, vocab=256)
+    write_weight_dir(str(wdir / "other"), small, mu.random_weights(orc.LlamaConfig(**small), 53, std=0.08))
+    (root / "draft.json").write_text(json.dumps({"model_dir": "other"}))
+    with pytest.raises(lib.EspressoError, match="vocab mismatch"):
+        e.generate(PROMPT, 4, environment=env)
+    e.close()
+
+
+def gguf_model(path, kw, w, arch, matrix_fmt, tied=False, interleave_qk=True):
+    """Writes a llama-family GGUF file the way llama.cpp's converter lays it out; returns the fp32 values
+    (in the half-split row order the decoder uses) that the packed tensors decode to."""
+    hd, half = kw["head_dim"], kw["head_dim"] // 2
+
+    def gguf_rows(a, heads):   # stored row (h, j, s) <- half-split row (h, s, j)
+        if not interleave_qk:
+            return a
+        r = a.reshape(heads, 2, half, a.shape[1])
+        return np.ascontiguousarray(r.transpose(0, 2, 1, 3)).reshape(a.shape)
+
+    meta = {"general.architecture": arch, f"{arch}.block_count": kw["n_layer"], f"{arch}.attention.head_count": kw["n_head"],
+            f"{arch}.attention.head_count_kv": kw["n_kv_head"], f"{arch}.embedding_length": kw["d_model"],
+            f"{arch}.feed_forward_length": kw["hidden_dim"], f"{arch}.context_length": kw["max_seq"],
+            f"{arch}.attention.layer_norm_rms_epsilon": 1e-5, f"{arch}.rope.freq_base": 10000.0,
+            "tokenizer.ggml.tokens": [f"t{i}" for i in range(kw["vocab"])], "tokenizer.ggml.eos_token_id": 2,
+            "general.name": "unit-test"}
+    tensors, seen = [], {"layers": []}
+
+    def quant(a):
+        blocks = orc.quantize(matrix_fmt, a)
+        return blocks, orc.dequantize(matrix_fmt, blocks, a.size).reshape(a.shape)
+
+    emb16 = w["embedding"].astype(np.float16)
+    tensors.append(("token_embd.weight", 1, w["embedding"].shape, emb16.tobytes()))
+    seen["embedding"] = emb16.astype(np.float32)
+    tensors.append(("output_norm.weight", 0, w["final_norm"].shape, w["final_norm"].astype("<f4").tobytes()))
+    seen["final_norm"] = w["final_norm"]
+    if tied:
+        seen["lm_head"] = seen["embedding"]
+    else:
+        b, seen["lm_head"] = quant(w["lm_head"])
+        tensors.append(("output.weight", matrix_fmt, w["lm_head"].shape, b.tobytes()))
+    names = {"wq": "attn_q", "wk": "attn_k", "wv": "attn_v", "wo": "attn_output", "w1": "ffn_gate", "w2": "ffn_down", "w3": "ffn_up"}
+    for l, L in enumerate(w["layers"]):
+        S = {}
+        for k, a in L.items():
+            if k in names:
+                b, S[k] = quant(a)
+                stored = a
+                if k == "wq": stored = gguf_rows(a, kw["n_head"])
+                if k == "wk": stored = gguf_rows(a, kw["n_kv_head"])
+                if stored is not a:
+                    b = orc.quantize(matrix_fmt, stored)      # blocks lie within rows, so this is a row permutation of `b`
+                tensors.append((f"blk.{l}.{names[k]}.weight", matrix_fmt, a.shape, b.tobytes()))
+            else:
+                g = {"rms_att": "attn_norm", "rms_ffn": "ffn_norm"}[k]
+                tensors.append((f"blk.{l}.{g}.weight", 0, a.shape, a.astype("<f4").tobytes()))
+                S[k] = a
+        seen["layers"].append(S)
+    write_gguf(path, meta, tensors)
+    return seen
+
+
+@pytest.mark.parametrize("arch,fmt,tied", [("llama", orc.FMT_Q8_0, False), ("llama", orc.FMT_Q4_K, True), ("qwen2", orc.FMT_Q4_0, False)])
+def test_gguf_prepare_then_engine(E, tmp_path, arch, fmt, tied):
+    w = mu.random_weights(orc.LlamaConfig(**KW), 61, std=0.08, norm_jitter=0.05)
+    path = str(tmp_path / "m.gguf")
+    seen = gguf_model(path, KW, w, arch, fmt, tied=tied, interleave_qk=arch == "llama")
+    cfg, wdir, count = E.gguf_prepare(path, str(tmp_path / "prepared"))
+    assert count == 2 + (0 if tied else 1) + 9 * KW["n_layer"]
+    assert (cfg.n_layer, cfg.n_head, cfg.n_kv_head, cfg.d_model, cfg.head_dim, cfg.hidden_dim, cfg.vocab, cfg.max_seq, cfg.eos_token) == \
+           (2, 4, 2, 256, 64, 512, 512, 48, 2)
+    assert cfg.name == arch and cfg.rope_theta == 10000.0
+    assert json.load(open(os.path.join(wdir, "metadata.json")))["vocab"] == 512
+    tag = {orc.FMT_Q8_0: "q8_0", orc.FMT_Q4_0: "q4_0", orc.FMT_Q4_K: "q4_k"}[fmt]
+    assert os.path.exists(os.path.join(wdir, f"layers/0/wq.{tag}.bin")) and not os.path.exists(os.path.join(wdir, "layers/0/wq.bin"))
+    assert os.path.exists(os.path.join(wdir, "rms_final.float32.bin"))
+    assert os.path.exists(os.path.join(wdir, "lm_head.bin" if tied else f"lm_head.{tag}.bin"))
+    e = E.RealModelInferenceEngine(cfg, wdir)
+    cfg.eos_token = -1
+    toks, _ = e.generate(PROMPT, 16)
+    okw = dict(KW, eos_token=2)
+    assert toks == oracle_tokens(okw, seen, PROMPT, 16)
+    e.close()
+
+
+def test_gguf_prepare_can_emit_reference_blobfiles(E, tmp_path):
+    w = mu.random_weights(orc.LlamaConfig(**KW), 62, std=0.08)
+    path = str(tmp_path / "m.gguf")
+    seen = gguf_model(path, KW, w, "llama", orc.FMT_Q8_0)
+    cfg, wdir, _ = E.gguf_prepare(path, str(tmp_path / "prepared"), emit_dequantized_blobs=True)
+    n, vals = E.blob_weight_load(os.path.join(wdir, "layers/1/wk.bin"))
+    assert n == seen["layers"][1]["wk"].size
+    assert np.array_equal(vals, seen["layers"][1]["wk"].ravel().astype(np.float16).astype(np.float32))   # half-split row order
+
+
+def test_gguf_errors(E, tmp_path):
+    import espresso_amd._lib as lib
+    bad = tmp_path / "bad.gguf"
+    bad.write_bytes(b"GGML" + b"\0" * 64)
+    with pytest.raises(lib.EspressoError, match="bad magic"):
+        E.gguf_prepare(str(bad), str(tmp_path / "o1"))
+    import struct
+    bad.write_bytes(struct.pack("<IIQQ", 0x46554747, 1, 0, 0))
+    with pytest.raises(lib.EspressoError, match="unsupported GGUF version"):
+        E.gguf_prepare(str(bad), str(tmp_path / "o2"))
+    write_gguf(str(bad), {"general.architecture": "bert"}, [])
+    with pytest.raises(lib.EspressoError, match="unsupported architecture"):
+        E.gguf_prepare(str(bad), str(tmp_path / "o3"))
+    w = mu.random_weights(orc.LlamaConfig(**KW), 63, std=0.08)
+    good = str(tmp_path / "g.gguf")
+    gguf_model(good, KW, w, "llama", orc.FMT_Q8_0)
+    data = open(good, "rb").read()
+    bad.write_bytes(data[:len(data) // 2])                                              # tensor data cut short
+    with pytest.raises(lib.EspressoError, match="past the end"):
+        E.gguf_prepare(str(bad), str(tmp_path / "o4"))
+
+
+def test_harness_with_gpu_models(E, tmp_path):
+    import espresso_amd.llama as ll
+    full_kw, draft_kw = dict(KW, n_layer=3), dict(KW, n_layer=1)
+    rts = []
+    for kw, seed in ((full_kw, 71), (draft_kw, 72)):
+        packed, _ = mu.pack_weights(mu.random_weights(orc.LlamaConfig(**kw), seed, std=0.08), orc.FMT_Q8_0)
+        rt = ll.LlamaRuntime(ll.MultiModelConfig(**kw))
+        ll.load_packed_weights(rt, packed, orc.FMT_Q8_0)
+        rts.append(rt)
+    plain, _ = rts[0].generate(PROMPT, 24)
+    toks, com, acc = E.harness_generate(PROMPT, 23, target=rts[0], draft=rts[1])
+    assert toks[:23] == plain[:23] and len(toks) in (23, 24)
+    assert all(c in (1, 2) for c in com) and all(a == c - 1 for a, c in zip(acc, com)) and sum(com) == len(toks)
+    # LocalBigramArtifactBuilder golden: [35] -> [105, 110, 116, 32], committed [2, 2], accepted [1, 1]
+    from test_oracle_runtime import bigram_model
+    _, w = bigram_model(d_model=128, vocab=128)
+    packed, _ = mu.pack_weights(w, orc.FMT_F16)
+    kw = dict(n_layer=1, n_head=2, n_kv_head=2, d_model=128, head_dim=64, hidden_dim=16, vocab=128, max_seq=32)
+    pair = []
+    for _ in range(2):
+        rt = ll.LlamaRuntime(ll.MultiModelConfig(**kw))
+        ll.load_packed_weights(rt, packed, orc.FMT_F16)
+        pair.append(rt)
+    toks, com, acc = E.harness_generate([35], 4, target=pair[0], draft=pair[1])
+    assert toks == [105, 110, 116, 32] and com == [2, 2] and acc == [1, 1]

@@ -1,0 +1,184 @@
+"""Host-side pieces of the boundary that need no GPU: exported symbols, BLOBFILE, paths, metadata,
+the promotion plan and the exact two-token harness driven by scripted models (the reference's own
+test doubles, Tests/EspressoTests/GenerationHarnessTests.swift:63-270, 482-619)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import espresso_amd._lib as lib
+import espresso_amd.engine as eng
+import espresso_amd.llama as ll
+from oracle import oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "espresso_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    names = set(re.findall(r"\b(esp_[a-z0-9_]+)\s*\(", header))
+    assert len(names) > 40
+    L = lib.load_library()
+    missing = [n for n in sorted(names) if not hasattr(L, n)]
+    assert not missing, missing
+
+
+def test_no_device_fails_loudly_without_cpu_fallback():
+    if os.path.exists("/dev/kfd"):
+        pytest.skip("GPU present")
+    import espresso_amd.ops as ops
+    with pytest.raises(lib.EspressoError, match="no CPU fallback"):
+        ops.init()
+    with pytest.raises(lib.EspressoError):
+        ops.dequantize(orc.FMT_Q8_0, np.zeros(34, np.uint8), 32)
+
+
+def test_weight_blob_matches_reference_layout_and_oracle(tmp_path):
+    w = np.random.default_rng(0).normal(0, 0.02, 1000).astype(np.float32)
+    w[:6] = [0.0, -0.0, 65504.0, 1e-8, 6.1e-5, 1.0 + 2 ** -11]
+    blob = eng.weight_blob_build(w)
+    assert blob == orc.blob_build(w)
+    assert blob[0] == 1 and blob[4] == 2 and blob[64:68] == bytes([0xEF, 0xBE, 0xAD, 0xDE]) and blob[68] == 1
+    assert int.from_bytes(blob[72:76], "little") == 2000 and int.from_bytes(blob[80:84], "little") == 128
+    p = tmp_path / "w.bin"
+    p.write_bytes(blob)
+    n, back = eng.blob_weight_load(str(p))
+    assert n == 1000 and np.array_equal(back, w.astype(np.float16).astype(np.float32))
+    # BlobWeightLoaderError cases (Sources/ModelSupport/BlobWeightLoader.swift:3-9, 62-90)
+    cases = {-1: blob[:100], -2: blob[:64] + b"\0" + blob[65:], -3: blob[:80] + bytes([64]) + blob[81:], -4: blob[:-2],
+             -5: blob[:72] + bytes([7]) + blob[73:]}
+    for code, data in cases.items():
+        p.write_bytes(data)
+        assert eng.blob_weight_load(str(p))[0] == code
+    assert eng.blob_weight_load(str(tmp_path / "missing.bin"))[0] == -6
+    p.write_bytes(eng.weight_blob_build(np.zeros(0, np.float32)))
+    assert eng.blob_weight_load(str(p))[0] == 0                                  # empty payload
+
+
+def test_layer_weight_paths():
+    names = {ll.SLOT_RMS_ATT: "rms_att", ll.SLOT_WQ: "wq", ll.SLOT_WK: "wk", ll.SLOT_WV: "wv", ll.SLOT_WO: "wo",
+             ll.SLOT_RMS_FFN: "rms_ffn", ll.SLOT_W1: "w1", ll.SLOT_W2: "w2", ll.SLOT_W3: "w3", ll.SLOT_Q_NORM: "q_norm",
+             ll.SLOT_K_NORM: "k_norm"}
+    for slot, name in names.items():
+        assert eng.layer_weight_path(3, "/tmp/weights", slot) == f"/tmp/weights/layers/3/{name}.bin"
+    with pytest.raises(lib.EspressoError):
+        eng.layer_weight_path(0, "/tmp/weights", ll.SLOT_LM_HEAD)
+
+
+def test_metadata_round_trip_and_reference_keys(tmp_path):
+    cfg = ll.MultiModelConfig(n_layer=6, n_head=12, n_kv_head=4, d_model=768, head_dim=64, hidden_dim=2048, vocab=32000, max_seq=256,
+                              norm_eps=1e-6, rope_theta=500000.0, eos_token=2, name="llama")
+    path = str(tmp_path / "metadata.json")
+    eng.write_metadata(cfg, path)
+    import json
+    raw = json.load(open(path))
+    assert set(raw) == {"name", "nLayer", "nHead", "nKVHead", "dModel", "headDim", "hiddenDim", "vocab", "maxSeq", "normEps",
+                        "ropeTheta", "architecture", "eosToken"}
+    assert raw["architecture"] == "llama" and raw["nKVHead"] == 4 and raw["eosToken"] == 2
+    back = eng.load_metadata(path)
+    assert np.float32(back.norm_eps) == np.float32(cfg.norm_eps)      # normEps is a Float in the reference
+    back.norm_eps = cfg.norm_eps
+    assert back == cfg
+    # a file written by other tooling: extra keys, nested values, no eosToken
+    open(path, "w").write('{"nLayer": 1, "nHead": 2, "nKVHead": 1, "dModel": 8, "headDim": 4, "hiddenDim": 16, "vocab": 32, '
+                          '"maxSeq": 16, "architecture": "llama", "extra": {"a": [1, 2, {"b": null}]}, "name": "tiny\\u002dllama"}')
+    t = eng.load_metadata(path)
+    assert (t.n_layer, t.vocab, t.eos_token, t.name) == (1, 32, -1, "tiny-llama")
+    open(path, "w").write('{"nLayer": 1')
+    with pytest.raises(lib.EspressoError, match="not valid JSON"):
+        eng.load_metadata(path)
+    open(path, "w").write('{"nLayer": 1}')
+    with pytest.raises(lib.EspressoError, match="missing nHead"):
+        eng.load_metadata(path)
+
+
+def test_promotion_plan():
+    """GenerationHarnessTests.swift:589-619"""
+    a = eng.promotion_plan(5, 6, 6, 7, 2)
+    assert a == {"committed_tokens": [5, 6], "next_current_token": 7, "committed_exact_token_count": 2,
+                 "accepted_future_token_count": 1, "promoted_step_count": 2}
+    r = eng.promotion_plan(5, 9, 6, 7, 2)
+    assert r == {"committed_tokens": [5], "next_current_token": 6, "committed_exact_token_count": 1,
+                 "accepted_future_token_count": 0, "promoted_step_count": 1}
+    assert eng.promotion_plan(5, 6, 6, 7, 1)["committed_tokens"] == [5]          # budget 1 never commits two
+
+
+class FakeExactTwoTokenModel:
+    """FakeExactTwoTokenModel: a scripted queue of pass results (GenerationHarnessTests.swift:200-270)."""
+
+    def __init__(self, selected_prefill_token, passes):
+        self.selected, self.queue = selected_prefill_token, list(passes)
+        self.reset_count, self.prefill_calls, self.pass_calls = 0, [], []
+        self._keep = (eng.RESET_FN(self._reset), eng.PREFILL_FN(self._prefill), eng.PASS_FN(self._pass))
+        self.struct = eng.ExactTwoTokenModelStruct(None, *self._keep)
+
+    def _reset(self, ctx):
+        self.reset_count += 1
+        return 0
+
+    def _prefill(self, ctx, toks, n, out):
+        self.prefill_calls.append([toks[i] for i in range(n)])
+        out[0] = self.selected
+        return 0
+
+    def _pass(self, ctx, current, budget, res):
+        self.pass_calls.append((current, budget))
+        if not self.queue:
+            return 1
+        committed, nxt, advance_ms, accepted, count = self.queue.pop(0)
+        r = res.contents
+        for i, t in enumerate(committed[:2]):
+            r.committed_tokens[i] = t
+        r.committed_count = len(committed)
+        r.next_current_token = nxt
+        r.state_advance_latency_ms = advance_ms
+        r.accepted_future_token_count = accepted
+        r.committed_exact_token_count = count
+        return 0
+
+
+def test_harness_tracks_pass_metrics_and_future_acceptance():
+    """GenerationHarnessTests.swift:482-535: trace [5,6,7], accepted [1,0], committed [2,1]."""
+    m = FakeExactTwoTokenModel(5, [([5, 6], 7, 1.15, 1, 2), ([7], 8, 0.0, 0, 1)])
+    toks, com, acc = eng.harness_generate([9], 3, model=m.struct)
+    assert toks == [5, 6, 7] and acc == [1, 0] and com == [2, 1]
+    assert m.reset_count == 1 and m.prefill_calls == [[9]] and m.pass_calls == [(5, 3), (7, 1)]
+    assert sum(com) / len(com) == 1.5 and sum(acc) / len(acc) == 0.5
+
+
+def test_harness_future_rejection():
+    """GenerationHarnessTests.swift:537-587"""
+    m = FakeExactTwoTokenModel(2, [([2], 4, 0.0, 0, 1), ([4], 6, 0.0, 0, 1)])
+    toks, com, acc = eng.harness_generate([1], 2, model=m.struct)
+    assert toks == [2, 4] and acc == [0, 0] and com == [1, 1]
+
+
+@pytest.mark.parametrize("passes,message", [
+    ([([], 1, 0.0, 0, 0)], "must commit at least one token"),
+    ([([9, 6], 7, 1.0, 1, 2)], "must commit current token first"),
+    ([([5, 6], 7, 1.0, 1, 2)], "with remaining budget 1"),                      # budget 1, two committed
+    ([([5, 6, 7], 8, 0.0, 0, 3)], "committed 3 tokens"),
+    ([([5], 6, 0.0, 2, 1)], "must be in 0...1"),
+    ([([5, 6], 7, 0.0, 0, 1)], "must equal committed token count"),
+    ([([5], 6, 1.0, 1, 1)], "requires exactly two committed tokens"),
+    ([([5], 6, 0.5, 0, 1)], "must be zero when no future token is accepted"),
+])
+def test_harness_rejects_invariant_violations(passes, message):
+    """The guards of ExactTwoTokenGenerationHarness.generate (GenerationHarness.swift:640-672)."""
+    budget = 1 if "budget 1" in message else 4
+    m = FakeExactTwoTokenModel(5, passes)
+    with pytest.raises(lib.EspressoError, match=re.escape(message)):
+        eng.harness_generate([9], budget, model=m.struct)
+
+
+def test_harness_argument_errors():
+    m = FakeExactTwoTokenModel(5, [])
+    with pytest.raises(lib.EspressoError, match="promptTokens must not be empty"):
+        eng.harness_generate([], 3, model=m.struct)
+    with pytest.raises(lib.EspressoError, match="maxNewTokens must be > 0"):
+        eng.harness_generate([1], 0, model=m.struct)
+    with pytest.raises(lib.EspressoError, match="callback"):
+        eng.harness_generate([1], 2, model=m.struct)                             # the scripted queue is empty
