@@ -1,0 +1,509 @@
+// C ABI: kernel handles and surfaces in the call shape of the reference's ANEInterop module
+// (Sources/ANEInterop/include/ane_interop.h).  See the header for the contract of every function.
+#include <atomic>
+#include <cstring>
+#include <map>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "context.h"
+#include "host/model_support.h"
+#include "kernels/decode_ops.h"
+#include "kernels/surface_ops.h"
+
+using namespace esp;
+
+// A surface: HBM buffer + host shadow; `host_valid` / `device_valid` say which copy is current.
+struct ESPSurface {
+    std::atomic<int> refs{1};
+    size_t bytes = 0;
+    std::vector<uint8_t> host;
+    uint8_t *device = nullptr;
+    bool host_valid = true, device_valid = false;
+    int write_locks = 0, read_locks = 0;
+};
+
+namespace {
+
+std::atomic<int> g_compile_count{0}, g_live_handles{0};
+std::atomic<int> g_last_compile_error{ESP_INTEROP_COMPILE_ERROR_NONE};
+std::atomic<bool> g_force_eval_failure{false};
+
+bool surface_to_host(ESPSurface *s) {
+    if (s->host_valid) return true;
+    if (!s->device) return false;
+    if (hipMemcpy(s->host.data(), s->device, s->bytes, hipMemcpyDeviceToHost) != hipSuccess) return false;
+    s->host_valid = true;
+    return true;
+}
+
+bool surface_to_device(ESPSurface *s) {
+    if (ensure_init() != ESP_OK) return false;
+    if (!s->device) {
+        void *p = nullptr;
+        if (hipMalloc(&p, s->bytes ? s->bytes : 16) != hipSuccess) return false;
+        s->device = static_cast<uint8_t *>(p);
+        s->device_valid = false;
+    }
+    if (s->device_valid) return true;
+    if (!s->host_valid) return false;
+    if (hipMemcpy(s->device, s->host.data(), s->bytes, hipMemcpyHostToDevice) != hipSuccess) return false;
+    s->device_valid = true;
+    return true;
+}
+
+// fp16 view of the shadow for reading / writing [channels, spatial] regions
+uint16_t *shadow_for_write(ESPSurface *s) {
+    if (!s || !surface_to_host(s)) return nullptr;
+    s->device_valid = false;
+    return reinterpret_cast<uint16_t *>(s->host.data());
+}
+const uint16_t *shadow_for_read(ESPSurface *s) {
+    if (!s || !surface_to_host(s)) return nullptr;
+    return reinterpret_cast<const uint16_t *>(s->host.data());
+}
+bool region_ok(const ESPSurface *s, int ch_off, int channels, int spatial) {
+    if (!s || ch_off < 0 || channels < 0 || spatial <= 0) return false;
+    return ((size_t)ch_off + (size_t)channels) * (size_t)spatial * 2 <= s->bytes;
+}
+bool slice_ok(const ESPSurface *s, int ch_off, int channels, int spatial, int index) {
+    return region_ok(s, ch_off, channels, spatial) && index >= 0 && index < spatial;
+}
+
+enum KernelKind { KIND_GEMV, KIND_CLASSIFIER, KIND_FFN };
+
+std::string trim(const std::string &s) {
+    size_t a = s.find_first_not_of(" \t\r"), b = s.find_last_not_of(" \t\r");
+    return a == std::string::npos ? "" : s.substr(a, b - a + 1);
+}
+
+// "key: value" pairs; several pairs may share a line
+std::map<std::string, std::string> parse_program(const std::string &text) {
+    std::map<std::string, std::string> kv;
+    std::stringstream lines(text);
+    std::string line;
+    while (std::getline(lines, line)) {
+        std::stringstream words(line);
+        std::string tok, key;
+        while (words >> tok) {
+            if (!tok.empty() && tok.back() == ':') key = tok.substr(0, tok.size() - 1);
+            else if (!key.empty()) { kv[key] = trim(tok); key.clear(); }
+        }
+    }
+    return kv;
+}
+
+int format_by_name(const std::string &n) {
+    if (n == "f32") return FMT_F32;
+    if (n == "f16") return FMT_F16;
+    if (n == "q4_0") return FMT_Q4_0;
+    if (n == "q8_0") return FMT_Q8_0;
+    if (n == "q4_k") return FMT_Q4_K;
+    return -1;
+}
+
+std::string weight_stem(const char *path) {
+    std::string p = path ? path : "";
+    size_t slash = p.find_last_of('/');
+    if (slash != std::string::npos) p = p.substr(slash + 1);
+    if (p.size() > 4 && p.compare(p.size() - 4, 4, ".bin") == 0) p = p.substr(0, p.size() - 4);
+    return p;
+}
+
+struct WeightBytes { const uint8_t *data; size_t len; };
+
+// fp16 payload of a BLOBFILE, or the bytes themselves when they carry no BLOBFILE header
+WeightBytes payload_of(WeightBytes w) {
+    BlobWeightLoader::Header h;
+    if (w.len >= 128 && BlobWeightLoader::parseHeader(w.data, w.len, &h) == BlobWeightLoaderError::none && 128 + (size_t)h.dataSize == w.len)
+        return {w.data + 128, (size_t)h.dataSize};
+    return w;
+}
+
+}  // namespace
+
+struct ESPHandle {
+    int kind = KIND_GEMV;
+    int lanes = 1, spatial = 1, rows = 0, cols = 0, dim = 0, hidden = 0, vocab = 0;
+    float norm_eps = 1e-5f;
+    DeviceMatrix w, w13, w2, classifier;
+    float *norm = nullptr;
+    std::vector<ESPSurface *> inputs, outputs;
+    // scratch
+    uint16_t *x16 = nullptr, *act16 = nullptr;
+    float *x32 = nullptr, *y32 = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    uint64_t last_ns = 0;
+};
+
+namespace {
+
+void destroy_handle(ESPHandle *h) {
+    if (!h) return;
+    matrix_release(&h->w); matrix_release(&h->w13); matrix_release(&h->w2); matrix_release(&h->classifier);
+    if (h->norm) (void)hipFree(h->norm);
+    if (h->x16) (void)hipFree(h->x16);
+    if (h->act16) (void)hipFree(h->act16);
+    if (h->x32) (void)hipFree(h->x32);
+    if (h->y32) (void)hipFree(h->y32);
+    if (h->ev0) (void)hipEventDestroy(h->ev0);
+    if (h->ev1) (void)hipEventDestroy(h->ev1);
+    for (ESPSurface *s : h->inputs) esp_surface_release(s);
+    for (ESPSurface *s : h->outputs) esp_surface_release(s);
+    delete h;
+}
+
+ESPHandle *compile_fail(ESPHandle *h, int code, const char *fmt, const char *arg = "") {
+    g_last_compile_error = code;
+    fail(ESP_ERR_INVALID_ARGUMENT, fmt, arg);
+    destroy_handle(h);
+    return nullptr;
+}
+
+int upload_norm(WeightBytes raw, int count, float **out) {
+    WeightBytes p = payload_of(raw);
+    if (p.len != (size_t)count * 2) return fail(ESP_ERR_INVALID_ARGUMENT, "norm weight holds %zu bytes, expected %d fp16 values", p.len, count);
+    std::vector<float> v(count);
+    for (int i = 0; i < count; i++) v[i] = half_to_float((uint16_t)(p.data[2 * i] | (p.data[2 * i + 1] << 8)));
+    int rc = device_alloc(out, (size_t)count);
+    if (rc != ESP_OK) return rc;
+    ESP_HIP_TRY(hipMemcpy(*out, v.data(), (size_t)count * 4, hipMemcpyHostToDevice));
+    return ESP_OK;
+}
+
+int upload_matrix(WeightBytes raw, int format, int rows, int cols, DeviceMatrix *out) {
+    WeightBytes p = format == FMT_F16 ? payload_of(raw) : raw;
+    const size_t want = format_bytes(format, (size_t)rows * cols);
+    if (p.len != want) return fail(ESP_ERR_INVALID_ARGUMENT, "weight matrix holds %zu bytes, format needs %zu for %dx%d", p.len, want, rows, cols);
+    return matrix_upload(format, p.data, rows, cols, out);
+}
+
+}  // namespace
+
+extern "C" {
+
+void esp_interop_init(void) { (void)ensure_init(); }
+
+ESPSurfaceRef esp_interop_create_surface(size_t bytes) {
+    ESPSurface *s = new ESPSurface();
+    s->bytes = bytes;
+    s->host.assign(bytes, 0);
+    return s;
+}
+
+ESPSurfaceRef esp_surface_retain(ESPSurfaceRef s) {
+    if (s) s->refs.fetch_add(1);
+    return s;
+}
+
+void esp_surface_release(ESPSurfaceRef s) {
+    if (!s) return;
+    if (s->refs.fetch_sub(1) == 1) {
+        if (s->device) (void)hipFree(s->device);
+        delete s;
+    }
+}
+
+size_t esp_surface_bytes(ESPSurfaceRef s) { return s ? s->bytes : 0; }
+
+ESPHandle *esp_interop_compile(const uint8_t *program, size_t program_len, const char **weight_paths,
+                               const uint8_t **weight_datas, const size_t *weight_lens, int weight_count,
+                               int n_inputs, const size_t *input_sizes, int n_outputs, const size_t *output_sizes) {
+    g_last_compile_error = ESP_INTEROP_COMPILE_ERROR_NONE;
+    if (!program || program_len == 0 || weight_count < 0 || n_inputs < 0 || n_outputs < 0 ||
+        (weight_count > 0 && (!weight_paths || !weight_datas || !weight_lens)) || (n_inputs > 0 && !input_sizes) ||
+        (n_outputs > 0 && !output_sizes))
+        return compile_fail(nullptr, ESP_INTEROP_COMPILE_ERROR_INVALID_ARGUMENTS, "compile: invalid arguments%s");
+    std::map<std::string, WeightBytes> weights;
+    for (int i = 0; i < weight_count; i++) {
+        if (!weight_paths[i]) return compile_fail(nullptr, ESP_INTEROP_COMPILE_ERROR_INVALID_ARGUMENTS, "compile: null weight path%s");
+        // a weight path never leaves the model directory (ane_interop.m rejects ".." components)
+        const std::string raw_path = weight_paths[i];
+        if (raw_path == ".." || raw_path.rfind("../", 0) == 0 || raw_path.find("/../") != std::string::npos ||
+            (raw_path.size() >= 3 && raw_path.compare(raw_path.size() - 3, 3, "/..") == 0))
+            return compile_fail(nullptr, ESP_INTEROP_COMPILE_ERROR_INVALID_ARGUMENTS, "compile: weight path %s leaves the model directory", weight_paths[i]);
+        const std::string stem = weight_stem(weight_paths[i]);
+        if (weights.count(stem)) return compile_fail(nullptr, ESP_INTEROP_COMPILE_ERROR_DUPLICATE_WEIGHT_PATH, "compile: duplicate weight path %s", weight_paths[i]);
+        weights[stem] = {weight_datas[i], weight_datas[i] ? weight_lens[i] : 0};
+    }
+    if (ensure_init() != ESP_OK) { g_last_compile_error = ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE; return nullptr; }
+
+    const auto kv = parse_program(std::string(reinterpret_cast<const char *>(program), program_len));
+    auto get_int = [&](const char *k, int dflt) { auto it = kv.find(k); return it == kv.end() ? dflt : std::atoi(it->second.c_str()); };
+    auto get_str = [&](const char *k) { auto it = kv.find(k); return it == kv.end() ? std::string() : it->second; };
+    ESPHandle *h = new ESPHandle();
+    const std::string kind = get_str("kernel");
+    const int format = format_by_name(get_str("format"));
+    h->spatial = get_int("spatial", 1);
+    h->lanes = get_int("lanes", 1);
+    if (!get_str("norm_eps").empty()) h->norm_eps = (float)std::atof(get_str("norm_eps").c_str());
+    if (get_str("program") != "espresso.hip/1") return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: program header must be espresso.hip/1%s");
+    if (h->spatial < 1 || h->lanes < 1 || h->lanes > kMaxStepRows || h->lanes > h->spatial)
+        return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: spatial/lanes out of range%s");
+    auto need = [&](const char *name) -> WeightBytes * { auto it = weights.find(name); return it == weights.end() || !it->second.data ? nullptr : &it->second; };
+    std::vector<size_t> want_in, want_out;
+    int rc = ESP_OK;
+    if (kind == "gemv") {
+        h->kind = KIND_GEMV;
+        h->rows = get_int("rows", 0); h->cols = get_int("cols", 0);
+        WeightBytes *w = need("w");
+        if (format < 0 || h->rows <= 0 || h->cols <= 0 || !w) return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: gemv needs format, rows, cols and weight w%s");
+        rc = upload_matrix(*w, format, h->rows, h->cols, &h->w);
+        want_in = {(size_t)h->cols * h->spatial * 2};
+        want_out = {(size_t)h->rows * h->spatial * 2};
+    } else if (kind == "rmsnorm_classifier") {
+        h->kind = KIND_CLASSIFIER;
+        h->dim = get_int("dim", 0); h->vocab = get_int("vocab", 0);
+        WeightBytes *g = need("rms_final"), *c = need("classifier");
+        if (format < 0 || h->dim <= 0 || h->vocab <= 0 || !g || !c) return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: rmsnorm_classifier needs format, dim, vocab, rms_final and classifier%s");
+        rc = upload_norm(*g, h->dim, &h->norm);
+        if (rc == ESP_OK) rc = upload_matrix(*c, format, h->vocab, h->dim, &h->classifier);
+        want_in = {(size_t)h->dim * h->spatial * 2};
+        want_out = {(size_t)h->vocab * h->spatial * 2, (size_t)h->spatial * 2};
+        h->rows = h->vocab; h->cols = h->dim;
+    } else if (kind == "decode_ffn") {
+        h->kind = KIND_FFN;
+        h->dim = get_int("dim", 0); h->hidden = get_int("hidden", 0);
+        WeightBytes *g = need("rms_ffn"), *w1 = need("w1"), *w3 = need("w3"), *w2 = need("w2");
+        if (format < 0 || h->dim <= 0 || h->hidden <= 0 || !g || !w1 || !w3 || !w2) return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: decode_ffn needs format, dim, hidden, rms_ffn, w1, w3 and w2%s");
+        rc = upload_norm(*g, h->dim, &h->norm);
+        const size_t rb = format_bytes(format, (size_t)h->dim);
+        if (rc == ESP_OK && (w1->len != rb * h->hidden || w3->len != rb * h->hidden) && format != FMT_F16)
+            rc = fail(ESP_ERR_INVALID_ARGUMENT, "w1/w3 byte counts do not match %dx%d", h->hidden, h->dim);
+        if (rc == ESP_OK) {
+            // gate and up rows interleaved (g0, u0, g1, u1, ...) so that one GEMV feeds the SwiGLU epilogue
+            WeightBytes p1 = format == FMT_F16 ? payload_of(*w1) : *w1, p3 = format == FMT_F16 ? payload_of(*w3) : *w3;
+            if (p1.len != rb * h->hidden || p3.len != rb * h->hidden) rc = fail(ESP_ERR_INVALID_ARGUMENT, "w1/w3 byte counts do not match %dx%d", h->hidden, h->dim);
+            else {
+                std::vector<uint8_t> fused(2 * rb * h->hidden);
+                for (int i = 0; i < h->hidden; i++) {
+                    std::memcpy(&fused[(size_t)(2 * i) * rb], p1.data + (size_t)i * rb, rb);
+                    std::memcpy(&fused[(size_t)(2 * i + 1) * rb], p3.data + (size_t)i * rb, rb);
+                }
+                rc = matrix_upload(format, fused.data(), 2 * h->hidden, h->dim, &h->w13);
+            }
+        }
+        if (rc == ESP_OK) rc = upload_matrix(*w2, format, h->dim, h->hidden, &h->w2);
+        want_in = {(size_t)h->dim * h->spatial * 2};
+        want_out = {(size_t)h->dim * h->spatial * 2};
+        h->rows = h->dim; h->cols = h->dim;
+    } else {
+        return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: unknown kernel kind %s", kind.c_str());
+    }
+    if (rc != ESP_OK) { g_last_compile_error = ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE; destroy_handle(h); return nullptr; }
+    if ((size_t)n_inputs != want_in.size() || (size_t)n_outputs != want_out.size())
+        return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_INVALID_ARGUMENTS, "compile: surface counts do not match the kernel%s");
+    for (size_t i = 0; i < want_in.size(); i++)
+        if (input_sizes[i] != want_in[i]) return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_INVALID_ARGUMENTS, "compile: input surface size does not match channels x spatial x 2%s");
+    for (size_t i = 0; i < want_out.size(); i++)
+        if (output_sizes[i] != want_out[i]) return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_INVALID_ARGUMENTS, "compile: output surface size does not match channels x spatial x 2%s");
+    for (size_t b : want_in) h->inputs.push_back(esp_interop_create_surface(b));
+    for (size_t b : want_out) h->outputs.push_back(esp_interop_create_surface(b));
+    const size_t widest = (size_t)std::max(std::max(h->rows, h->cols), std::max(h->hidden, h->vocab));
+    bool ok = device_alloc(&h->x16, (size_t)h->lanes * widest) == ESP_OK && device_alloc(&h->act16, (size_t)h->lanes * widest) == ESP_OK &&
+              device_alloc(&h->x32, (size_t)h->lanes * widest) == ESP_OK && device_alloc(&h->y32, (size_t)h->lanes * widest) == ESP_OK &&
+              hipEventCreate(&h->ev0) == hipSuccess && hipEventCreate(&h->ev1) == hipSuccess;
+    for (ESPSurface *s : h->inputs) ok = ok && surface_to_device(s);
+    for (ESPSurface *s : h->outputs) ok = ok && surface_to_device(s);
+    if (!ok) return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_SURFACE_ALLOCATION_FAILED, "compile: surface allocation failed%s");
+    g_live_handles.fetch_add(1);
+    g_compile_count.fetch_add(1);  // successful compiles only
+    clear_error();
+    return h;
+}
+
+bool esp_interop_eval(ESPHandle *h) {
+    if (!h) return false;
+    if (g_force_eval_failure.load()) { fail(ESP_ERR_FORCED_FAILURE, "eval failure forced by esp_interop_set_force_eval_failure"); return false; }
+    hipStream_t s = context().stream;
+    for (ESPSurface *in : h->inputs) if (!surface_to_device(in)) { fail(ESP_ERR_LAUNCH_FAILED, "eval: input surface upload failed"); return false; }
+    for (ESPSurface *out : h->outputs) if (!surface_to_device(out)) { fail(ESP_ERR_LAUNCH_FAILED, "eval: output surface upload failed"); return false; }
+    const uint16_t *in0 = reinterpret_cast<const uint16_t *>(h->inputs[0]->device);
+    uint16_t *out0 = reinterpret_cast<uint16_t *>(h->outputs[0]->device);
+    hipError_t e = hipEventRecord(h->ev0, s);
+    GemvParams g;
+    g.batch = h->lanes;
+    if (e == hipSuccess && h->kind == KIND_GEMV) {
+        e = launch_gather_columns(in0, h->cols, h->spatial, h->lanes, h->x16, nullptr, s);
+        g.w = h->w; g.x = h->x16; g.y = h->y32; g.epilogue = EPI_STORE_F32;
+        if (e == hipSuccess) e = launch_gemv(g, s);
+        if (e == hipSuccess) e = launch_scatter_columns(h->y32, h->rows, h->spatial, h->lanes, out0, s);
+    } else if (e == hipSuccess && h->kind == KIND_CLASSIFIER) {
+        e = launch_gather_columns(in0, h->dim, h->spatial, h->lanes, nullptr, h->x32, s);
+        if (e == hipSuccess) e = launch_rmsnorm(h->x32, h->norm, h->norm_eps, h->lanes, h->dim, h->x16, nullptr, s);
+        g.w = h->classifier; g.x = h->x16; g.y = h->y32; g.epilogue = EPI_STORE_F32;
+        if (e == hipSuccess) e = launch_gemv(g, s);
+        if (e == hipSuccess) e = launch_scatter_columns(h->y32, h->vocab, h->spatial, h->lanes, out0, s);
+        if (e == hipSuccess) e = launch_row_max(h->y32, h->vocab, h->spatial, h->lanes, reinterpret_cast<uint16_t *>(h->outputs[1]->device), s);
+    } else if (e == hipSuccess) {
+        e = launch_gather_columns(in0, h->dim, h->spatial, h->lanes, nullptr, h->x32, s);
+        if (e == hipSuccess) e = launch_rmsnorm(h->x32, h->norm, h->norm_eps, h->lanes, h->dim, h->x16, nullptr, s);
+        g.w = h->w13; g.x = h->x16; g.out_f16 = h->act16; g.epilogue = EPI_SWIGLU_F16;
+        if (e == hipSuccess) e = launch_gemv(g, s);
+        g.w = h->w2; g.x = h->act16; g.out_f16 = nullptr; g.y = h->y32; g.residual = h->x32; g.epilogue = EPI_ADD_RESIDUAL;
+        if (e == hipSuccess) e = launch_gemv(g, s);
+        if (e == hipSuccess) e = launch_scatter_columns(h->y32, h->dim, h->spatial, h->lanes, out0, s);
+    }
+    if (e == hipSuccess) e = hipEventRecord(h->ev1, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) { fail_hip(e, "eval"); return false; }
+    float ms = 0.0f;
+    if (hipEventElapsedTime(&ms, h->ev0, h->ev1) == hipSuccess) h->last_ns = (uint64_t)((double)ms * 1e6);
+    for (ESPSurface *out : h->outputs) { out->device_valid = true; out->host_valid = false; }
+    return true;
+}
+
+ESPSurfaceRef esp_interop_get_input(ESPHandle *h, int i) { return h && i >= 0 && i < (int)h->inputs.size() ? h->inputs[i] : nullptr; }
+ESPSurfaceRef esp_interop_get_output(ESPHandle *h, int i) { return h && i >= 0 && i < (int)h->outputs.size() ? h->outputs[i] : nullptr; }
+ESPSurfaceRef esp_interop_copy_input(ESPHandle *h, int i) { return esp_surface_retain(esp_interop_get_input(h, i)); }
+ESPSurfaceRef esp_interop_copy_output(ESPHandle *h, int i) { return esp_surface_retain(esp_interop_get_output(h, i)); }
+
+void esp_interop_free(ESPHandle *h) {
+    if (!h) return;
+    g_live_handles.fetch_sub(1);
+    destroy_handle(h);
+}
+
+int esp_interop_compile_count(void) { return g_compile_count.load(); }
+void esp_interop_set_compile_count(int v) { g_compile_count = v; }
+int esp_interop_last_compile_error(void) { return g_last_compile_error.load(); }
+void esp_interop_set_force_eval_failure(bool v) { g_force_eval_failure = v; }
+int esp_interop_live_handle_count(void) { return g_live_handles.load(); }
+uint64_t esp_interop_last_hw_execution_time_ns(ESPHandle *h) { return h ? h->last_ns : 0; }
+bool esp_interop_has_perf_stats(ESPHandle *h) { return h != nullptr; }
+
+bool esp_interop_rebind_input(ESPHandle *h, int index, ESPSurfaceRef s) {
+    if (!h || !s || index < 0 || index >= (int)h->inputs.size() || s->bytes != h->inputs[index]->bytes) return false;
+    esp_surface_retain(s);
+    esp_surface_release(h->inputs[index]);
+    h->inputs[index] = s;
+    return true;
+}
+
+void esp_interop_cvt_f32_to_f16(void *dst, const float *src, int count) {
+    uint16_t *d = static_cast<uint16_t *>(dst);
+    for (int i = 0; i < count; i++) d[i] = float_to_half_rne(src[i]);
+}
+void esp_interop_cvt_f16_to_f32(float *dst, const void *src, int count) {
+    const uint16_t *s = static_cast<const uint16_t *>(src);
+    for (int i = 0; i < count; i++) dst[i] = half_to_float(s[i]);
+}
+void esp_interop_argmax_f16_strided(const void *src, int count, int stride, int *out_index, float *out_value) {
+    const uint16_t *s = static_cast<const uint16_t *>(src);
+    int best = 0;
+    float bv = count > 0 ? half_to_float(s[0]) : 0.0f;
+    for (int i = 1; i < count; i++) {
+        const float v = half_to_float(s[(size_t)i * stride]);
+        if (v > bv) { bv = v; best = i; }
+    }
+    if (out_index) *out_index = best;
+    if (out_value) *out_value = bv;
+}
+void esp_interop_argmax_f16(const void *src, int count, int *out_index, float *out_value) {
+    esp_interop_argmax_f16_strided(src, count, 1, out_index, out_value);
+}
+
+bool esp_interop_io_copy(ESPSurfaceRef dst, int dst_ch_off, ESPSurfaceRef src, int src_ch_off, int channels, int spatial) {
+    if (!region_ok(dst, dst_ch_off, channels, spatial) || !region_ok(src, src_ch_off, channels, spatial)) return false;
+    const uint16_t *s = shadow_for_read(src);
+    uint16_t *d = shadow_for_write(dst);
+    if (!s || !d) return false;
+    std::memmove(d + (size_t)dst_ch_off * spatial, s + (size_t)src_ch_off * spatial, (size_t)channels * spatial * 2);
+    return true;
+}
+
+bool esp_interop_io_copy_fp16_spatial_slice(ESPSurfaceRef dst, int dst_ch_off, int dst_index, int dst_spatial, ESPSurfaceRef src,
+                                            int src_ch_off, int src_index, int src_spatial, int channels) {
+    if (!slice_ok(dst, dst_ch_off, channels, dst_spatial, dst_index) || !slice_ok(src, src_ch_off, channels, src_spatial, src_index)) return false;
+    const uint16_t *s = shadow_for_read(src);
+    uint16_t *d = shadow_for_write(dst);
+    if (!s || !d) return false;
+    for (int c = 0; c < channels; c++) d[(size_t)(dst_ch_off + c) * dst_spatial + dst_index] = s[(size_t)(src_ch_off + c) * src_spatial + src_index];
+    return true;
+}
+
+bool esp_interop_io_write_fp16_spatial_slice(ESPSurfaceRef surface, int ch_off, int index, int spatial, const float *data, int channels) {
+    if (!data || !slice_ok(surface, ch_off, channels, spatial, index)) return false;
+    uint16_t *d = shadow_for_write(surface);
+    if (!d) return false;
+    for (int c = 0; c < channels; c++) d[(size_t)(ch_off + c) * spatial + index] = float_to_half_rne(data[c]);
+    return true;
+}
+
+bool esp_interop_io_read_fp16_spatial_slice(ESPSurfaceRef surface, int ch_off, int index, int spatial, float *data, int channels) {
+    if (!data || !slice_ok(surface, ch_off, channels, spatial, index)) return false;
+    const uint16_t *s = shadow_for_read(surface);
+    if (!s) return false;
+    for (int c = 0; c < channels; c++) data[c] = half_to_float(s[(size_t)(ch_off + c) * spatial + index]);
+    return true;
+}
+
+bool esp_interop_io_argmax_fp16_spatial_slice(ESPSurfaceRef surface, int ch_off, int index, int spatial, int channels, int *out_index,
+                                              float *out_value) {
+    if (channels <= 0 || !slice_ok(surface, ch_off, channels, spatial, index)) return false;
+    const uint16_t *s = shadow_for_read(surface);
+    if (!s) return false;
+    esp_interop_argmax_f16_strided(s + (size_t)ch_off * spatial + index, channels, spatial, out_index, out_value);
+    return true;
+}
+
+bool esp_interop_io_write_fp16_at(ESPSurfaceRef surface, int ch_off, const float *data, int channels, int spatial) {
+    if (!data || !region_ok(surface, ch_off, channels, spatial)) return false;
+    uint16_t *d = shadow_for_write(surface);
+    if (!d) return false;
+    esp_interop_cvt_f32_to_f16(d + (size_t)ch_off * spatial, data, channels * spatial);
+    return true;
+}
+bool esp_interop_io_write_fp16(ESPSurfaceRef surface, const float *data, int channels, int spatial) {
+    return esp_interop_io_write_fp16_at(surface, 0, data, channels, spatial);
+}
+bool esp_interop_io_read_fp16(ESPSurfaceRef surface, int ch_off, float *data, int channels, int spatial) {
+    if (!data || !region_ok(surface, ch_off, channels, spatial)) return false;
+    const uint16_t *s = shadow_for_read(surface);
+    if (!s) return false;
+    esp_interop_cvt_f16_to_f32(data, s + (size_t)ch_off * spatial, channels * spatial);
+    return true;
+}
+bool esp_interop_io_read_fp16_batched(ESPSurfaceRef surface, int spatial, float *const *destinations, const int *channel_offsets,
+                                      const int *channels, int region_count) {
+    if (!destinations || !channel_offsets || !channels || region_count < 0) return false;
+    for (int r = 0; r < region_count; r++) if (!region_ok(surface, channel_offsets[r], channels[r], spatial) || !destinations[r]) return false;
+    for (int r = 0; r < region_count; r++) if (!esp_interop_io_read_fp16(surface, channel_offsets[r], destinations[r], channels[r], spatial)) return false;
+    return true;
+}
+
+bool esp_interop_io_write_embedding_batch_fp16(ESPSurfaceRef surface, int ch_off, int spatial, const float *table, int vocab_size, int dim,
+                                               const uint16_t *token_ids, int stream_count) {
+    if (!table || !token_ids || stream_count < 0 || stream_count > spatial || !region_ok(surface, ch_off, dim, spatial)) return false;
+    for (int s = 0; s < stream_count; s++) if (token_ids[s] >= vocab_size) return false;
+    uint16_t *d = shadow_for_write(surface);
+    if (!d) return false;
+    for (int s = 0; s < stream_count; s++)
+        for (int c = 0; c < dim; c++) d[(size_t)(ch_off + c) * spatial + s] = float_to_half_rne(table[(size_t)token_ids[s] * dim + c]);
+    return true;
+}
+
+bool esp_interop_io_argmax_batch_fp16_spatial(ESPSurfaceRef surface, int ch_off, int spatial, int channels, int stream_count, int *out_indices,
+                                              float *out_values) {
+    if (!out_indices || !out_values || stream_count < 0 || stream_count > spatial || channels <= 0 || !region_ok(surface, ch_off, channels, spatial)) return false;
+    const uint16_t *s = shadow_for_read(surface);
+    if (!s) return false;
+    for (int i = 0; i < stream_count; i++) esp_interop_argmax_f16_strided(s + (size_t)ch_off * spatial + i, channels, spatial, &out_indices[i], &out_values[i]);
+    return true;
+}
+
+bool esp_interop_io_lock_write(ESPSurfaceRef s) { if (!s || !surface_to_host(s)) return false; s->write_locks++; return true; }
+bool esp_interop_io_unlock_write(ESPSurfaceRef s) { if (!s || s->write_locks <= 0) return false; s->write_locks--; s->device_valid = false; return true; }
+bool esp_interop_io_lock_read(ESPSurfaceRef s) { if (!s || !surface_to_host(s)) return false; s->read_locks++; return true; }
+bool esp_interop_io_unlock_read(ESPSurfaceRef s) { if (!s || s->read_locks <= 0) return false; s->read_locks--; return true; }
+bool esp_interop_io_write_fp16_unlocked(ESPSurfaceRef s, const float *data, int channels, int spatial) {
+    if (!s || s->write_locks <= 0) return false;
+    return esp_interop_io_write_fp16_at(s, 0, data, channels, spatial);
+}
+bool esp_interop_io_read_fp16_unlocked(ESPSurfaceRef s, int ch_off, float *data, int channels, int spatial) {
+    if (!s || s->read_locks <= 0) return false;
+    return esp_interop_io_read_fp16(s, ch_off, data, channels, spatial);
+}
+
+}  // extern "C"

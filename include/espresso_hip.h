@@ -304,6 +304,101 @@ int esp_exact_two_token_harness_generate(const ESPExactTwoTokenModel *model, ESP
                                          uint32_t *out_tokens, int *out_token_count, int32_t *out_committed_per_pass,
                                          int32_t *out_accepted_per_pass, int *out_pass_count);
 
+/* ================================================================================================== *
+ * Kernel handles and surfaces: the call shape of the reference's ANEInterop module
+ * (Sources/ANEInterop/include/ane_interop.h), one esp_interop_* function per ane_interop_* function
+ * the decode path uses, same argument order and return conventions (NULL / false on failure, the
+ * cause in esp_interop_last_compile_error()).  Swift's ANEKernel (Sources/ANERuntime/ANEKernel.swift:
+ * 65-745) and SurfaceIO (Sources/ANETypes/SurfaceIO.swift) bind to these one for one.
+ *
+ * A surface is a flat fp16 buffer read as channel-first [channels, spatial], element (c, s) at
+ * c * spatial + s (ane_interop.h:171-174).  It lives in HBM with a host shadow; the io functions work
+ * on the shadow and eval moves what changed, so "lock, copy, unlock" keeps its meaning.
+ * ================================================================================================== */
+typedef struct ESPHandle ESPHandle;          /* ANEHandle, ane_interop.h:13 */
+typedef struct ESPSurface *ESPSurfaceRef;    /* stands in for IOSurfaceRef; reference counted */
+
+void esp_interop_init(void);                                     /* :15 */
+ESPSurfaceRef esp_interop_create_surface(size_t bytes);          /* :16, returns +1 retained */
+ESPSurfaceRef esp_surface_retain(ESPSurfaceRef surface);         /* CFRetain / CFRelease of the reference's surfaces */
+void esp_surface_release(ESPSurfaceRef surface);
+size_t esp_surface_bytes(ESPSurfaceRef surface);                 /* IOSurfaceGetAllocSize */
+
+#define ESP_INTEROP_COMPILE_ERROR_NONE 0                          /* :18-22, same values */
+#define ESP_INTEROP_COMPILE_ERROR_INVALID_ARGUMENTS 1
+#define ESP_INTEROP_COMPILE_ERROR_DUPLICATE_WEIGHT_PATH 2
+#define ESP_INTEROP_COMPILE_ERROR_SURFACE_ALLOCATION_FAILED 3
+#define ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE 4
+
+/* ane_interop_compile (:24-28).  `program` is a text description of one HIP kernel set instead of MIL
+ * text: "key: value" lines, e.g.
+ *     program: espresso.hip/1
+ *     kernel: gemv            (gemv | rmsnorm_classifier | decode_ffn)
+ *     format: q8_0            (f32 | f16 | q4_0 | q8_0 | q4_k; weight matrices)
+ *     rows: 768  cols: 768    (gemv)   dim / hidden (decode_ffn)   dim / vocab (rmsnorm_classifier)
+ *     spatial: 32             (surface width S; a decode token lives in column 0, DecodeKernelSet.swift:10)
+ *     lanes: 1                (how many leading columns are computed, 1..16)
+ *     norm_eps: 1e-5
+ * Weights are matched by the file name at the end of their path ("@model_path/weights/w.bin" -> "w"):
+ * gemv: w; rmsnorm_classifier: rms_final, classifier; decode_ffn: rms_ffn, w1, w3, w2.  Matrices are GGUF
+ * blocks of `format`, or a BLOBFILE when format is f16; norm vectors are BLOBFILEs.  The bytes are copied
+ * during the call.  Surfaces: gemv in [cols,S] -> out [rows,S]; rmsnorm_classifier in [dim,S] -> logits
+ * [vocab,S], max [1,S] (GenerationRMSNormClassifierGenerator.swift:27-63); decode_ffn in [dim,S] -> [dim,S]
+ * computing x + W2(silu(W1 n) * W3 n), n = rmsnorm(x) (DecodeFFNGenerator.swift:40-91). */
+ESPHandle *esp_interop_compile(const uint8_t *program, size_t program_len,
+                               const char **weight_paths, const uint8_t **weight_datas,
+                               const size_t *weight_lens, int weight_count,
+                               int n_inputs, const size_t *input_sizes,
+                               int n_outputs, const size_t *output_sizes);
+bool esp_interop_eval(ESPHandle *handle);                                   /* :30, synchronous */
+ESPSurfaceRef esp_interop_get_input(ESPHandle *handle, int index);          /* :31, not retained */
+ESPSurfaceRef esp_interop_get_output(ESPHandle *handle, int index);         /* :32, not retained */
+ESPSurfaceRef esp_interop_copy_input(ESPHandle *handle, int index);         /* :33, +1 retained */
+ESPSurfaceRef esp_interop_copy_output(ESPHandle *handle, int index);        /* :34, +1 retained */
+void esp_interop_free(ESPHandle *handle);                                   /* :35 */
+int esp_interop_compile_count(void);                                        /* :37 */
+void esp_interop_set_compile_count(int value);                              /* :38 */
+int esp_interop_last_compile_error(void);                                   /* :39 */
+void esp_interop_set_force_eval_failure(bool value);                        /* :40, host-side fault injection */
+int esp_interop_live_handle_count(void);                                    /* :41 */
+uint64_t esp_interop_last_hw_execution_time_ns(ESPHandle *handle);          /* :42, HIP-event time of the last eval */
+bool esp_interop_has_perf_stats(ESPHandle *handle);                         /* :43 */
+bool esp_interop_rebind_input(ESPHandle *handle, int index, ESPSurfaceRef new_surface);   /* :50 */
+
+void esp_interop_cvt_f32_to_f16(void *dst, const float *src, int count);    /* :143, round to nearest even */
+void esp_interop_cvt_f16_to_f32(float *dst, const void *src, int count);    /* :144 */
+/* First-max argmax over fp16 values: lowest index wins ties (:146-156, neon_convert.c:36-101). */
+void esp_interop_argmax_f16(const void *src, int count, int *out_index, float *out_value);
+void esp_interop_argmax_f16_strided(const void *src, int count, int stride, int *out_index, float *out_value);
+
+/* Surface I/O (:168-348): fp32 on the caller's side, fp16 on the surface; all return false on a
+ * range error instead of touching memory. */
+bool esp_interop_io_copy(ESPSurfaceRef dst, int dst_ch_off, ESPSurfaceRef src, int src_ch_off, int channels, int spatial);   /* :168 */
+bool esp_interop_io_copy_fp16_spatial_slice(ESPSurfaceRef dst, int dst_ch_off, int dst_spatial_index, int dst_spatial,
+                                            ESPSurfaceRef src, int src_ch_off, int src_spatial_index, int src_spatial,
+                                            int channels);                                                                 /* :175 */
+bool esp_interop_io_write_fp16_spatial_slice(ESPSurfaceRef surface, int ch_off, int spatial_index, int spatial,
+                                             const float *data, int channels);                                             /* :202 */
+bool esp_interop_io_read_fp16_spatial_slice(ESPSurfaceRef surface, int ch_off, int spatial_index, int spatial,
+                                            float *data, int channels);                                                    /* :208 */
+bool esp_interop_io_argmax_fp16_spatial_slice(ESPSurfaceRef surface, int ch_off, int spatial_index, int spatial,
+                                              int channels, int *out_index, float *out_value);                             /* :214 */
+bool esp_interop_io_write_fp16(ESPSurfaceRef surface, const float *data, int channels, int spatial);                       /* :235 */
+bool esp_interop_io_read_fp16(ESPSurfaceRef surface, int ch_off, float *data, int channels, int spatial);                  /* :237 */
+bool esp_interop_io_read_fp16_batched(ESPSurfaceRef surface, int spatial, float *const *destinations,
+                                      const int *channel_offsets, const int *channels, int region_count);                  /* :239 */
+bool esp_interop_io_write_fp16_at(ESPSurfaceRef surface, int ch_off, const float *data, int channels, int spatial);        /* :244 */
+bool esp_interop_io_write_embedding_batch_fp16(ESPSurfaceRef surface, int ch_off, int spatial, const float *embedding_table,
+                                               int vocab_size, int dim, const uint16_t *token_ids, int stream_count);      /* :270 */
+bool esp_interop_io_argmax_batch_fp16_spatial(ESPSurfaceRef surface, int ch_off, int spatial, int channels, int stream_count,
+                                              int *out_indices, float *out_values);                                        /* :282 */
+bool esp_interop_io_lock_write(ESPSurfaceRef surface);                                                                     /* :335 */
+bool esp_interop_io_unlock_write(ESPSurfaceRef surface);
+bool esp_interop_io_lock_read(ESPSurfaceRef surface);
+bool esp_interop_io_unlock_read(ESPSurfaceRef surface);
+bool esp_interop_io_write_fp16_unlocked(ESPSurfaceRef surface, const float *data, int channels, int spatial);              /* :342 */
+bool esp_interop_io_read_fp16_unlocked(ESPSurfaceRef surface, int ch_off, float *data, int channels, int spatial);         /* :347 */
+
 #ifdef __cplusplus
 }
 #endif
