@@ -69,6 +69,10 @@ struct QkvEpilogue {
 struct GemvParams {
     DeviceMatrix w;
     const uint16_t *x = nullptr;  // fp16 activations [batch][cols]
+    // fused RMSNorm: when norm_x is set the activations are fp16((norm_x * inv_rms) * norm_w), computed
+    // while staging, and `x` is ignored.  norm_x: fp32 [batch][cols]; norm_w: fp32 [cols].
+    const float *norm_x = nullptr, *norm_w = nullptr;
+    float norm_eps = 0.0f;
     float *y = nullptr;           // fp32 out [batch][rows]
     const float *residual = nullptr;
     uint16_t *out_f16 = nullptr;  // EPI_SWIGLU_F16: [batch][rows/2]

@@ -387,33 +387,31 @@ __global__ __launch_bounds__(256) void attention_flash_kernel(AttentionArgs a) {
 }
 
 // Merges the per-split partial states (m, l, acc) of attention_flash_kernel in split order.
-// grid (KV heads, rows).  A kernel boundary, not a device-scope fence, orders it after the partial
+// grid (query heads, rows).  A kernel boundary, not a device-scope fence, orders it after the partial
 // writes: fences plus arrival counters in every workgroup cost far more than this launch.
 template <int HD, int G>
-__global__ __launch_bounds__(256) void attention_merge_kernel(AttentionArgs a, int splits) {
-    const int kvh = blockIdx.x, m = blockIdx.y, tid = threadIdx.x;
+__global__ __launch_bounds__(HD) void attention_merge_kernel(AttentionArgs a, int splits) {
+    // one workgroup per query head, one thread per channel
+    const int head = blockIdx.x, m = blockIdx.y, kvh = head / G, g = head % G, dch = threadIdx.x;
     const float *scratch = a.split_scratch + (((size_t)m * a.n_kv_head + kvh) * splits) * G * (HD + 2);
-    for (int i = tid; i < G * HD; i += 256) {
-        const int g = i / HD, dch = i % HD;
-        // all partials are fetched before the first is used (one memory round trip)
-        float pm[kAttentionMaxSplits], pl[kAttentionMaxSplits], pa[kAttentionMaxSplits];
+    // all partials are fetched before the first is used (one memory round trip)
+    float pm[kAttentionMaxSplits], pl[kAttentionMaxSplits], pa[kAttentionMaxSplits];
 #pragma unroll
-        for (int sp = 0; sp < kAttentionMaxSplits; sp++) {
-            const float *ps = scratch + ((size_t)(sp < splits ? sp : 0) * G + g) * (HD + 2);
-            pm[sp] = ps[0]; pl[sp] = ps[1]; pa[sp] = ps[2 + dch];
-        }
-        float M = -INFINITY;
-#pragma unroll
-        for (int sp = 0; sp < kAttentionMaxSplits; sp++) if (sp < splits) M = fmaxf(M, pm[sp]);
-        float L = 0.0f, A = 0.0f;
-#pragma unroll
-        for (int sp = 0; sp < kAttentionMaxSplits; sp++) {
-            const float f = (sp < splits && pm[sp] != -INFINITY) ? expf(pm[sp] - M) : 0.0f;
-            L += pl[sp] * f;
-            A += pa[sp] * f;
-        }
-        a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)(kvh * G + g) * HD + dch] = to_half_bits(L > 0.0f ? A / L : 0.0f);
+    for (int sp = 0; sp < kAttentionMaxSplits; sp++) {
+        const float *ps = scratch + ((size_t)(sp < splits ? sp : 0) * G + g) * (HD + 2);
+        pm[sp] = ps[0]; pl[sp] = ps[1]; pa[sp] = ps[2 + dch];
     }
+    float M = -INFINITY;
+#pragma unroll
+    for (int sp = 0; sp < kAttentionMaxSplits; sp++) if (sp < splits) M = fmaxf(M, pm[sp]);
+    float L = 0.0f, A = 0.0f;
+#pragma unroll
+    for (int sp = 0; sp < kAttentionMaxSplits; sp++) {
+        const float f = (sp < splits && pm[sp] != -INFINITY) ? expf(pm[sp] - M) : 0.0f;
+        L += pl[sp] * f;
+        A += pa[sp] * f;
+    }
+    a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)head * HD + dch] = to_half_bits(L > 0.0f ? A / L : 0.0f);
 }
 
 template <int HD, int G>
@@ -429,7 +427,7 @@ hipError_t launch_attention_gqa(const AttentionArgs &a, int rows, bool kv_f16, h
     dim3 grid(a.n_kv_head, rows, splits);
     if (kv_f16) hipLaunchKernelGGL((attention_flash_kernel<HD, G, true>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((attention_flash_kernel<HD, G, false>), grid, dim3(256), 0, s, a);
-    if (splits > 1) hipLaunchKernelGGL((attention_merge_kernel<HD, G>), dim3(a.n_kv_head, rows), dim3(256), 0, s, a, splits);
+    if (splits > 1) hipLaunchKernelGGL((attention_merge_kernel<HD, G>), dim3(a.n_head, rows), dim3(HD), 0, s, a, splits);
     return hipGetLastError();
 }
 

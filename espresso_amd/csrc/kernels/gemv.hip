@@ -21,6 +21,8 @@
 //
 // HBM traffic per launch = packed weight bytes + batch*cols*2 (x) + batch*rows*4 (y): the kernel is
 // bound by HBM bandwidth; x is re-read from L2 once per workgroup.
+#include <cstdlib>
+
 #include "../common.h"
 
 namespace esp {
@@ -115,7 +117,59 @@ struct KernelArgs {
     float *y;
     const float *residual;
     int epilogue;
+    // when norm_x is set the activations are rmsnorm(norm_x) * norm_w computed while staging (x is unused)
+    const float *norm_x, *norm_w;
+    float norm_eps;
 };
+
+// ---- activations -----------------------------------------------------------------------------
+// Sum over the workgroup's four wavefronts; `red` holds kWaves floats that nobody else touches until
+// the next barrier.  The same value, summed in the same order, reaches every thread.
+__device__ __forceinline__ float workgroup_sum(float v, float *red) {
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+__device__ __forceinline__ float sum_squares(const float4 &a, const float4 &b) {
+    return a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+}
+__device__ __forceinline__ u32 pack_half2(float lo, float hi) {
+    return (u32)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((u32)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+}
+// Eight normalised activations as fp16:  fp16((x * inv) * w), the order of operations of rmsNorm
+// (RealModelInferenceEngine.swift:6724-6743).
+__device__ __forceinline__ uint4 normalized_group(const float4 &v0, const float4 &v1, const float4 &g0, const float4 &g1, float inv) {
+    uint4 h;
+    h.x = pack_half2(__fmul_rn(__fmul_rn(v0.x, inv), g0.x), __fmul_rn(__fmul_rn(v0.y, inv), g0.y));
+    h.y = pack_half2(__fmul_rn(__fmul_rn(v0.z, inv), g0.z), __fmul_rn(__fmul_rn(v0.w, inv), g0.w));
+    h.z = pack_half2(__fmul_rn(__fmul_rn(v1.x, inv), g1.x), __fmul_rn(__fmul_rn(v1.y, inv), g1.y));
+    h.w = pack_half2(__fmul_rn(__fmul_rn(v1.z, inv), g1.z), __fmul_rn(__fmul_rn(v1.w, inv), g1.w));
+    return h;
+}
+// 1 / sqrt(mean(x^2) + eps) of row b of norm_x (any cols that is a multiple of 8); `red` as above.
+__device__ __forceinline__ float row_inverse_rms(const KernelArgs &a, int b, int cols, float *red) {
+    const float4 *x4 = reinterpret_cast<const float4 *>(a.norm_x + (size_t)b * cols);
+    float s = 0.0f;
+    for (int g = threadIdx.x; g < cols / 8; g += kThreads) s += sum_squares(x4[2 * g], x4[2 * g + 1]);
+    return 1.0f / sqrtf(workgroup_sum(s, red) / (float)cols + a.norm_eps);
+}
+// Group g (eight consecutive elements) of row b of the activations, as fp16.
+__device__ __forceinline__ uint4 activation_group(const KernelArgs &a, int b, int g, int cols, float inv) {
+    if (!a.norm_x) return reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + g];
+    const float4 *x4 = reinterpret_cast<const float4 *>(a.norm_x + (size_t)b * cols);
+    const float4 *w4 = reinterpret_cast<const float4 *>(a.norm_w);
+    return normalized_group(x4[2 * g], x4[2 * g + 1], w4[2 * g], w4[2 * g + 1], inv);
+}
+// (x0,x1,x2,x3, x4,...) -> (x0,x2,x1,x3, x4,x6,x5,x7): the order the masked nibble / byte pairs meet
+__device__ __forceinline__ uint4 swap_middle(const uint4 &v) {
+    uint4 p;
+    p.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
+    p.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
+    p.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
+    p.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
+    return p;
+}
 
 // What a wavefront does with the two row sums (rows 2p and 2p+1) of each batch column.
 template <int B>
@@ -206,22 +260,19 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cols = a.cols;
 
-    // ---- stage activations: 128-bit loads, middle elements of each group of four swapped ----
+    // ---- stage activations: 128-bit loads (or the fused RMSNorm), middle elements of each group of
+    // four swapped for the integer formats ----
     {
-        const uint4 *src = reinterpret_cast<const uint4 *>(a.x);
+        __shared__ float norm_red[B * kWaves];
         uint4 *dst = reinterpret_cast<uint4 *>(xs);
-        const int n16 = B * cols / 8;
-        for (int i = tid; i < n16; i += kThreads) {
-            uint4 v = src[i];
-            if (T::kPermuteX) {
-                uint4 p;
-                p.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
-                p.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
-                p.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
-                p.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
-                v = p;
+        const int per_row = cols / 8;
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+            const float inv = a.norm_x ? row_inverse_rms(a, b, cols, norm_red + b * kWaves) : 0.0f;
+            for (int g = tid; g < per_row; g += kThreads) {
+                const uint4 v = activation_group(a, b, g, cols, inv);
+                dst[(size_t)b * per_row + g] = T::kPermuteX ? swap_middle(v) : v;
             }
-            dst[i] = v;
         }
     }
     __syncthreads();
@@ -365,17 +416,19 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
 // Q4_K.  A lane's item is one 64-weight chunk of a super-block: 32 bytes of nibbles (two 128-bit
 // loads) whose low nibbles are sub-block 2c and whose high nibbles are sub-block 2c+1, plus the
 // block's 16-byte header (d, dmin, twelve scale bytes; the four lanes of a block read the same
-// 16 bytes).  A wavefront owns two consecutive rows and walks their items as one flat range, so
-// every lane is busy whenever cols is a multiple of 2048 (4096 -> 2 passes, 14336 -> 7 passes).
-// Weight loads run two passes ahead of the arithmetic and the first ones are issued before the
-// activations are staged.  Because rows hold a multiple of four items, a lane keeps the same chunk
-// index c = lane & 3 for the whole kernel, so everything the 6-bit scale unpacking needs besides
-// the header itself (shift counts, masks, which header word to read) is computed once.
+// 16 bytes).  The items of a row pair form one flat range of 2 * cols / 64 items.  Because rows hold
+// a multiple of four items, a lane keeps the same chunk index c = lane & 3 for the whole kernel, so
+// everything the 6-bit scale unpacking needs besides the header itself (shift counts, masks, which
+// header word to read) is computed once.
 //
-// Nibbles are turned into fp16 with the exponent trick at offset 64: a nibble placed in mantissa
-// bits 4..7 under exponent 0x5400 reads as 64 + n exactly.  v_dot2_f32_f16 then accumulates
-// sum (64 + n) x in fp32 with exact products, and the offset is removed once per sub-block with
-// the precomputed sum of its 32 activations:  sum n x = raw - 64 * sum x.
+// Nibbles are turned into fp16 with the exponent trick, without moving them: a low nibble (bits
+// 0..3) under exponent 0x5400 reads as 64 + n/16, a high nibble (bits 4..7) under 0x4400 reads as
+// 4 + n/16, both exactly.  v_dot2_f32_f16 accumulates sum (offset + n/16) x in fp32 with exact
+// products, and the offset is removed once per sub-block with the precomputed sum of its 32
+// activations:  sum n x = 16 * (raw - offset * sum x).  The same sums serve the dmin * m term.
+//
+// Two kernels: gemv_q4k_kernel for the column counts known at compile time (persistent workgroups,
+// described there) and gemv_q4k_generic_kernel for any other multiple of 256.
 struct Q4KItem {
     uint4 q0, q1, hdr;
 };
@@ -383,7 +436,22 @@ struct Q4KItem {
 struct Q4KLane {   // per-lane constants of the scale unpacking
     bool upper;    // sub-blocks 4..7: six-bit values are split over two header words
     u32 sh_sc, sh_min, sh_top, mask_low, mask_top;
+    u32 magic_lo, magic_hi;   // kept in vector registers for v_and_or_b32
 };
+
+__device__ __forceinline__ Q4KLane q4k_lane_constants(int lane) {
+    Q4KLane L;
+    const int c = lane & 3, sh = (c & 1) * 16;
+    L.upper = c >= 2;
+    L.sh_sc = sh;
+    L.sh_min = L.upper ? sh + 4 : sh;
+    L.sh_top = sh + 2;
+    L.mask_low = L.upper ? 0x0F0Fu : 0x3F3Fu;
+    L.mask_top = L.upper ? 0x3030u : 0u;
+    L.magic_lo = 0x54005400u;
+    L.magic_hi = 0x44004400u;
+    return L;
+}
 
 template <int B, int XSTRIDE>
 __device__ __forceinline__ void q4k_item_dots(const Q4KItem &it, const Q4KLane &L, const uint4 *xs4, const float *xsum, int i,
@@ -395,60 +463,222 @@ __device__ __forceinline__ void q4k_item_dots(const Q4KItem &it, const Q4KLane &
     const u32 mp = ((src_min >> L.sh_min) & L.mask_low) | ((it.hdr.z >> L.sh_top) & L.mask_top);
     const float sc_lo = (float)(scp & 0xFFu), sc_hi = (float)((scp >> 8) & 0xFFu);
     const float m_lo = (float)(mp & 0xFFu), m_hi = (float)((mp >> 8) & 0xFFu);
-    const float d = half_bits_to_float(it.hdr.x & 0xFFFFu), dmin = half_bits_to_float(it.hdr.x >> 16);
+    const float d16 = 16.0f * half_bits_to_float(it.hdr.x & 0xFFFFu), dmin = half_bits_to_float(it.hdr.x >> 16);
 #pragma unroll
     for (int b = 0; b < B; b++) {
         const uint4 *px = xs4 + (size_t)b * 8 * xstride + i;
         float raw_lo = 0.0f, raw_hi = 0.0f;
 #pragma unroll
         for (int k = 0; k < 8; k++) {
-            const u32 w = dword_of(k < 4 ? it.q0 : it.q1, k & 3);
+            const u32 w = dword_of(k < 4 ? it.q0 : it.q1, k & 3), w8 = w >> 8;
             const uint4 vl = px[(k >> 1) * xstride], vh = px[(4 + (k >> 1)) * xstride];
             const h2 xl02 = as_h2(dword_of(vl, (k & 1) * 2)), xl13 = as_h2(dword_of(vl, (k & 1) * 2 + 1));
             const h2 xh02 = as_h2(dword_of(vh, (k & 1) * 2)), xh13 = as_h2(dword_of(vh, (k & 1) * 2 + 1));
-            const h2 l02 = as_h2(and_or(w << 4, 0x00F000F0u, 0x54005400u));
-            const h2 l13 = as_h2(and_or(w >> 4, 0x00F000F0u, 0x54005400u));
-            const h2 h02 = as_h2(and_or(w, 0x00F000F0u, 0x54005400u));
-            const h2 h13 = as_h2(and_or(w >> 8, 0x00F000F0u, 0x54005400u));
+            const h2 l02 = as_h2(and_or(w, 0x000F000Fu, L.magic_lo));
+            const h2 h02 = as_h2(and_or(w, 0x00F000F0u, L.magic_hi));
+            const h2 l13 = as_h2(and_or(w8, 0x000F000Fu, L.magic_lo));
+            const h2 h13 = as_h2(and_or(w8, 0x00F000F0u, L.magic_hi));
             raw_lo = fdot2(l02, xl02, raw_lo);
             raw_lo = fdot2(l13, xl13, raw_lo);
             raw_hi = fdot2(h02, xh02, raw_hi);
             raw_hi = fdot2(h13, xh13, raw_hi);
         }
         const float2 xsp = *reinterpret_cast<const float2 *>(xsum + (size_t)b * (cols >> 5) + 2 * i);
-        const float nx_lo = raw_lo - 64.0f * xsp.x, nx_hi = raw_hi - 64.0f * xsp.y;
-        v[b] = d * (sc_lo * nx_lo + sc_hi * nx_hi) - dmin * (m_lo * xsp.x + m_hi * xsp.y);
+        const float nx_lo = raw_lo - 64.0f * xsp.x, nx_hi = raw_hi - 4.0f * xsp.y;
+        v[b] = d16 * (sc_lo * nx_lo + sc_hi * nx_hi) - dmin * (m_lo * xsp.x + m_hi * xsp.y);
     }
 }
 
-// IPR: items (64-weight chunks) per row when known at compile time, 0 = read from the arguments.
-template <int B, int IPR>
-__global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a) {
+// Activations into LDS for the Q4_K kernels: middle elements of each group of four swapped, written as
+// [b][k][item] with an odd item stride (conflict-free for the write and for the per-k reads of
+// consecutive items); sums of each 32 alongside.
+__device__ __forceinline__ void q4k_store_group(const uint4 &v, int b, int g, int cols, int xstride, uint4 *xs4, float *xsum) {
+    xs4[(size_t)b * 8 * xstride + (g & 7) * xstride + (g >> 3)] = swap_middle(v);
+    float s = ((float)as_h2(v.x).x + (float)as_h2(v.x).y) + ((float)as_h2(v.y).x + (float)as_h2(v.y).y) +
+              ((float)as_h2(v.z).x + (float)as_h2(v.z).y) + ((float)as_h2(v.w).x + (float)as_h2(v.w).y);
+    s += dpp_term<0xB1, 0xF>(s);   // the four lanes of a quad hold the four groups of one 32
+    s += dpp_term<0x4E, 0xF>(s);
+    if ((threadIdx.x & 3) == 0) xsum[(size_t)b * (cols >> 5) + (g >> 2)] = s;
+}
+
+// cols known only at run time (a multiple of 256, so every quad of lanes is inside the row)
+template <int B>
+__device__ __forceinline__ void q4k_stage_x(const KernelArgs &a, int cols, int xstride, uint4 *xs4, float *xsum, float *red) {
+#pragma unroll
+    for (int b = 0; b < B; b++) {
+        const float inv = a.norm_x ? row_inverse_rms(a, b, cols, red + b * kWaves) : 0.0f;
+        for (int g = threadIdx.x; g < cols / 8; g += kThreads) q4k_store_group(activation_group(a, b, g, cols, inv), b, g, cols, xstride, xs4, xsum);
+    }
+}
+
+// cols = 64 * IPR: every load of the row is issued before the first use, so staging costs one memory
+// round trip (two with the fused RMSNorm: values, then nothing else - the weights ride along).
+template <int B, int IPR, bool NORM>
+__device__ __forceinline__ void q4k_stage_x_static(const KernelArgs &a, uint4 *xs4, float *xsum, float *red) {
+    static_assert(IPR % 32 == 0, "whole groups per thread");
+    constexpr int K = IPR / 32, cols = IPR * 64, XSTRIDE = IPR | 1;
+    const int tid = threadIdx.x;
+    if constexpr (NORM) {
+        float4 v0[B][K], v1[B][K], g0[K], g1[K];
+        const float4 *w4 = reinterpret_cast<const float4 *>(a.norm_w);
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int g = tid + k * kThreads;
+            g0[k] = w4[2 * g];
+            g1[k] = w4[2 * g + 1];
+#pragma unroll
+            for (int b = 0; b < B; b++) {
+                const float4 *x4 = reinterpret_cast<const float4 *>(a.norm_x + (size_t)b * cols);
+                v0[b][k] = x4[2 * g];
+                v1[b][k] = x4[2 * g + 1];
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+            float s = 0.0f;
+#pragma unroll
+            for (int k = 0; k < K; k++) s += sum_squares(v0[b][k], v1[b][k]);
+            const float inv = 1.0f / sqrtf(workgroup_sum(s, red + b * kWaves) / (float)cols + a.norm_eps);
+#pragma unroll
+            for (int k = 0; k < K; k++)
+                q4k_store_group(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
+        }
+    } else {
+        uint4 v[B][K];
+#pragma unroll
+        for (int b = 0; b < B; b++)
+#pragma unroll
+            for (int k = 0; k < K; k++) v[b][k] = reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + tid + k * kThreads];
+#pragma unroll
+        for (int b = 0; b < B; b++)
+#pragma unroll
+            for (int k = 0; k < K; k++) q4k_store_group(v[b][k], b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
+    }
+}
+
+// Persistent kernel for cols = 64 * IPR.  TEAM wavefronts share one row pair at a time (TEAM = 1: a
+// wavefront streams whole pairs on its own; TEAM = 4: the workgroup splits a long row pair and adds
+// the four partial sums through LDS).  Teams take pairs team, team + n_teams, ...: the chip reads
+// one contiguous band of rows at a time, the activations are staged once per workgroup however many
+// pairs it handles, and the loads of a team's next pair are issued before the arithmetic of the
+// current one, so weight traffic never waits for the arithmetic.  Every workgroup runs `iters`
+// rounds, so the barriers of the TEAM > 1 reduction line up even when the last round is ragged.
+template <int B, int IPR, int TEAM, bool NORM>
+__global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int iters) {
+    constexpr int cols = IPR * 64, XSTRIDE = IPR | 1, TOTAL = 2 * IPR, TEAM_LANES = TEAM * 64;
+    constexpr int PASSES = (TOTAL + TEAM_LANES - 1) / TEAM_LANES, TEAMS = kWaves / TEAM;
+    static_assert(PASSES <= 2 && kWaves % TEAM == 0, "pick TEAM so that a lane holds at most two items per pair");
+    extern __shared__ uint4 smem_raw[];
+    uint4 *xs4 = smem_raw;                                                       // [B][8][XSTRIDE] x 8 fp16
+    float *xsum = reinterpret_cast<float *>(smem_raw + (size_t)B * 8 * XSTRIDE);  // [B][cols/32]
+    float *red = xsum + (size_t)B * (cols / 32);                                  // [2][kWaves][2 * B]
+    float *norm_red = red + 2 * kWaves * 2 * B;                                   // [B][kWaves]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tl = (wave % TEAM) * 64 + lane;
+    const int n_teams = gridDim.x * TEAMS, npairs = (a.rows + 1) / 2;
+    const Q4KLane L = q4k_lane_constants(lane);
+
+    auto load_pair = [&](int pair, Q4KItem (&buf)[PASSES]) {
+        const int row_a = 2 * pair < a.rows ? 2 * pair : a.rows - 1;   // clamped: loads stay inside the matrix
+        const int row_b = 2 * pair + 1 < a.rows ? 2 * pair + 1 : a.rows - 1;
+        const uint8_t *base_a = a.qs + (size_t)row_a * a.qs_row_bytes, *base_b = a.qs + (size_t)row_b * a.qs_row_bytes;
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            const int t = tl + p * TEAM_LANES, tt = t < TOTAL ? t : 0;
+            const bool second = tt >= IPR;
+            const int i = tt - (second ? IPR : 0);
+            const uint8_t *bp = (second ? base_b : base_a) + (size_t)(i >> 2) * 144;
+            buf[p].hdr = *reinterpret_cast<const uint4 *>(bp);
+            const uint4 *q = reinterpret_cast<const uint4 *>(bp + 16 + (i & 3) * 32);
+            buf[p].q0 = q[0];
+            buf[p].q1 = q[1];
+        }
+    };
+
+    auto process = [&](const Q4KItem (&buf)[PASSES], int pair, int parity) {
+        float acc_a[B], acc_b[B];
+#pragma unroll
+        for (int b = 0; b < B; b++) acc_a[b] = acc_b[b] = 0.0f;
+        if (pair < npairs) {
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) {
+                const int t = tl + p * TEAM_LANES;
+                const bool valid = t < TOTAL;
+                const int tt = valid ? t : 0;
+                const bool second = tt >= IPR;
+                float v[B];
+                q4k_item_dots<B, XSTRIDE>(buf[p], L, xs4, xsum, tt - (second ? IPR : 0), XSTRIDE, cols, v);
+#pragma unroll
+                for (int b = 0; b < B; b++) {
+                    const float vv = valid ? v[b] : 0.0f;
+                    acc_a[b] += second ? 0.0f : vv;
+                    acc_b[b] += second ? vv : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < B; b++) {
+                acc_a[b] = wave_sum(acc_a[b]);
+                acc_b[b] = wave_sum(acc_b[b]);
+            }
+        }
+        if constexpr (TEAM == 1) {
+            if (pair < npairs && lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
+        } else {
+            float *slot = red + (size_t)parity * kWaves * 2 * B;
+            if (lane == 0) {
+#pragma unroll
+                for (int b = 0; b < B; b++) { slot[wave * 2 * B + 2 * b] = acc_a[b]; slot[wave * 2 * B + 2 * b + 1] = acc_b[b]; }
+            }
+            __syncthreads();
+            if (pair < npairs && tl == 0) {
+                const int w0 = wave;   // first wavefront of the team
+#pragma unroll
+                for (int b = 0; b < B; b++) {
+                    float sa = slot[w0 * 2 * B + 2 * b], sb = slot[w0 * 2 * B + 2 * b + 1];
+#pragma unroll
+                    for (int w = 1; w < TEAM; w++) { sa += slot[(w0 + w) * 2 * B + 2 * b]; sb += slot[(w0 + w) * 2 * B + 2 * b + 1]; }
+                    acc_a[b] = sa;
+                    acc_b[b] = sb;
+                }
+                pair_epilogue<B>(a, pair, acc_a, acc_b);
+            }
+        }
+    };
+
+    Q4KItem buf0[PASSES], buf1[PASSES];
+    int pair = blockIdx.x * TEAMS + wave / TEAM;
+    if (pair < npairs) load_pair(pair, buf0);
+    q4k_stage_x_static<B, IPR, NORM>(a, xs4, xsum, norm_red);
+    __syncthreads();
+    for (int j = 0; j < iters; j += 2) {
+        int next = pair + n_teams;
+        if (next < npairs) load_pair(next, buf1);
+        process(buf0, pair, 0);
+        pair = next;
+        if (j + 1 < iters) {
+            next = pair + n_teams;
+            if (next < npairs) load_pair(next, buf0);
+            process(buf1, pair, 1);
+            pair = next;
+        }
+    }
+}
+
+// Any cols that is a multiple of 256: one workgroup per eight rows, a wavefront per row pair, loads
+// one pass ahead of the arithmetic.
+template <int B>
+__global__ __launch_bounds__(kThreads) void gemv_q4k_generic_kernel(KernelArgs a) {
     extern __shared__ uint4 smem_raw[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int cols = IPR ? IPR * 64 : a.cols;
-    const int ipr = IPR ? IPR : cols >> 6;   // items per row
-    const int xstride = ipr | 1;             // 16-byte slots between consecutive k of one item
-    constexpr int XSTRIDE = IPR ? (IPR | 1) : 0;
-    const int total = 2 * ipr;               // items of the wavefront's row pair
-    uint4 *xs4 = smem_raw;                                                        // [B][8][xstride] x 8 fp16, (x0,x2,x1,x3) order
-    float *xsum = reinterpret_cast<float *>(smem_raw + (size_t)B * 8 * xstride);  // [B][cols/32] sub-block sums
+    const int cols = a.cols, ipr = cols >> 6, xstride = ipr | 1, total = 2 * ipr;
+    uint4 *xs4 = smem_raw;
+    float *xsum = reinterpret_cast<float *>(smem_raw + (size_t)B * 8 * xstride);
+    float *norm_red = xsum + (size_t)B * (cols / 32);   // [B][kWaves]
     const int pair = blockIdx.x * kWaves + wave;
-    const int row_a = 2 * pair < a.rows ? 2 * pair : a.rows - 1;          // clamped: loads stay inside the matrix
+    const int row_a = 2 * pair < a.rows ? 2 * pair : a.rows - 1;
     const int row_b = 2 * pair + 1 < a.rows ? 2 * pair + 1 : a.rows - 1;
-    const uint8_t *base_a = a.qs + (size_t)row_a * a.qs_row_bytes;
-    const uint8_t *base_b = a.qs + (size_t)row_b * a.qs_row_bytes;
-
-    Q4KLane L;
-    {
-        const int c = lane & 3, sh = (c & 1) * 16;
-        L.upper = c >= 2;
-        L.sh_sc = sh;
-        L.sh_min = L.upper ? sh + 4 : sh;
-        L.sh_top = sh + 2;
-        L.mask_low = L.upper ? 0x0F0Fu : 0x3F3Fu;
-        L.mask_top = L.upper ? 0x3030u : 0u;
-    }
+    const uint8_t *base_a = a.qs + (size_t)row_a * a.qs_row_bytes, *base_b = a.qs + (size_t)row_b * a.qs_row_bytes;
+    const Q4KLane L = q4k_lane_constants(lane);
 
     auto load_item = [&](int t) {
         Q4KItem it;
@@ -462,73 +692,30 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a) {
         it.q1 = q[1];
         return it;
     };
-    auto stage_x = [&]() {
-        // activations: 128-bit loads, middle elements of each group of four swapped, written to the
-        // LDS layout [b][k][item] with an odd item stride (conflict-free for both the write and the
-        // per-k reads of consecutive items); sub-block sums of 32 alongside
-        const uint4 *xsrc = reinterpret_cast<const uint4 *>(a.x);
-        const int n16 = B * cols / 8;
-        for (int i = tid; i < n16; i += kThreads) {
-            const uint4 v = xsrc[i];
-            uint4 p;
-            p.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
-            p.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
-            p.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
-            p.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
-            const int b = i / (cols / 8), g = i - b * (cols / 8);
-            xs4[(size_t)b * 8 * xstride + (g & 7) * xstride + (g >> 3)] = p;
-            float s = ((float)as_h2(v.x).x + (float)as_h2(v.x).y) + ((float)as_h2(v.y).x + (float)as_h2(v.y).y) +
-                      ((float)as_h2(v.z).x + (float)as_h2(v.z).y) + ((float)as_h2(v.w).x + (float)as_h2(v.w).y);
-            s += dpp_term<0xB1, 0xF>(s);
-            s += dpp_term<0x4E, 0xF>(s);
-            if ((lane & 3) == 0) xsum[i >> 2] = s;
-        }
-    };
 
     float acc_a[B], acc_b[B];
 #pragma unroll
     for (int b = 0; b < B; b++) acc_a[b] = acc_b[b] = 0.0f;
-
-    auto consume = [&](const Q4KItem &it, int t) {
+    Q4KItem cur = load_item(lane);
+    q4k_stage_x<B>(a, cols, xstride, xs4, xsum, norm_red);
+    __syncthreads();
+    for (int t0 = 0; t0 < total; t0 += 64) {
+        Q4KItem nxt = cur;
+        if (t0 + 64 < total) nxt = load_item(t0 + 64 + lane);
+        const int t = t0 + lane;
         const bool valid = t < total;
         const int tt = valid ? t : 0;
         const bool second = tt >= ipr;
-        const int i = tt - (second ? ipr : 0);
         float v[B];
-        q4k_item_dots<B, XSTRIDE>(it, L, xs4, xsum, i, xstride, cols, v);
+        q4k_item_dots<B, 0>(cur, L, xs4, xsum, tt - (second ? ipr : 0), xstride, cols, v);
 #pragma unroll
         for (int b = 0; b < B; b++) {
             const float vv = valid ? v[b] : 0.0f;
             acc_a[b] += second ? 0.0f : vv;
             acc_b[b] += second ? vv : 0.0f;
         }
-    };
-
-    if constexpr (IPR != 0) {
-        constexpr int PASSES = (2 * IPR + 63) / 64;
-        constexpr int NBUF = PASSES < 3 ? PASSES : 3;
-        Q4KItem buf[NBUF];
-#pragma unroll
-        for (int p = 0; p < (PASSES > 2 ? 2 : PASSES); p++) buf[p] = load_item(p * 64 + lane);
-        stage_x();
-        __syncthreads();
-#pragma unroll
-        for (int p = 0; p < PASSES; p++) {
-            if (PASSES > 2 && p + 2 < PASSES) buf[(p + 2) % NBUF] = load_item((p + 2) * 64 + lane);
-            consume(buf[p % NBUF], p * 64 + lane);
-        }
-    } else {
-        Q4KItem cur = load_item(lane);
-        stage_x();
-        __syncthreads();
-        for (int t0 = 0; t0 < total; t0 += 64) {
-            Q4KItem nxt = cur;
-            if (t0 + 64 < total) nxt = load_item(t0 + 64 + lane);
-            consume(cur, t0 + lane);
-            cur = nxt;
-        }
+        cur = nxt;
     }
-
 #pragma unroll
     for (int b = 0; b < B; b++) {
         acc_a[b] = wave_sum(acc_a[b]);
@@ -537,29 +724,73 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a) {
     if (lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
 }
 
-template <int B, int IPR>
-hipError_t launch_q4k_ipr(const KernelArgs &a, hipStream_t stream) {
-    const size_t lds = (size_t)B * 8 * ((a.cols / 64) | 1) * 16 + (size_t)B * (a.cols / 32) * 4;
+inline hipError_t ensure_lds(const void *kernel, size_t lds, size_t *configured) {
     if (lds > 160 * 1024) return hipErrorInvalidValue;
-    auto kernel = gemv_q4k_kernel<B, IPR>;
-    static size_t configured_lds = 0;
-    if (lds > 48 * 1024 && lds > configured_lds) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (lds > 48 * 1024 && lds > *configured) {
+        hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        configured_lds = lds;
+        *configured = lds;
     }
-    const int pairs = (a.rows + 1) / 2;
-    const int grid = (pairs + kWaves - 1) / kWaves;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a);
+    return hipSuccess;
+}
+
+// Workgroups resident per compute unit that the persistent grid is sized for.
+int q4k_wgs_per_cu() {
+    static int v = [] {
+        const char *e = getenv("ESPRESSO_HIP_Q4K_WGS_PER_CU");
+        const int n = e ? atoi(e) : 0;
+        return n >= 1 && n <= 16 ? n : 16;
+    }();
+    return v;
+}
+int compute_units() {
+    static int v = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        return n;
+    }();
+    return v;
+}
+
+template <int B, int IPR, int TEAM, bool NORM>
+hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
+    constexpr int TEAMS = kWaves / TEAM;
+    const size_t lds = (size_t)B * 8 * (IPR | 1) * 16 + (size_t)B * (IPR * 2) * 4 + (size_t)(2 * kWaves * 2 * B + B * kWaves) * 4;
+    auto kernel = gemv_q4k_kernel<B, IPR, TEAM, NORM>;
+    static size_t configured_lds = 0;
+    hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
+    if (e != hipSuccess) return e;
+    // the persistent grid never exceeds what the chip holds at once
+    static int resident_per_cu = 0;
+    if (resident_per_cu == 0) {
+        int n = 0;
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, kThreads, lds);
+        if (e != hipSuccess) return e;
+        const int limit = q4k_wgs_per_cu();
+        resident_per_cu = n < 1 ? 1 : (n > limit ? limit : n);
+    }
+    const int npairs = (a.rows + 1) / 2;
+    const int want = (npairs + TEAMS - 1) / TEAMS;            // one round
+    const int cap = compute_units() * resident_per_cu;
+    int grid = want < cap ? want : cap;
+    const int iters = (npairs + grid * TEAMS - 1) / (grid * TEAMS);
+    grid = (npairs + iters * TEAMS - 1) / (iters * TEAMS);    // same rounds, no idle workgroups
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, iters);
     return hipGetLastError();
 }
 
 template <int B>
 hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
-    if (a.cols == 4096) return launch_q4k_ipr<B, 64>(a, stream);
-    if (a.cols == 14336) return launch_q4k_ipr<B, 224>(a, stream);
-    return launch_q4k_ipr<B, 0>(a, stream);
+    if (a.cols == 4096) return a.norm_x ? launch_q4k_persistent<B, 64, 1, true>(a, stream) : launch_q4k_persistent<B, 64, 1, false>(a, stream);
+    if (a.cols == 14336 && !a.norm_x) return launch_q4k_persistent<B, 224, 4, false>(a, stream);
+    const size_t lds = (size_t)B * 8 * ((a.cols / 64) | 1) * 16 + (size_t)B * (a.cols / 32) * 4 + (size_t)B * kWaves * 4;
+    auto kernel = gemv_q4k_generic_kernel<B>;
+    static size_t configured_lds = 0;
+    hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
+    if (e != hipSuccess) return e;
+    const int pairs = (a.rows + 1) / 2;
+    hipLaunchKernelGGL(kernel, dim3((pairs + kWaves - 1) / kWaves), dim3(kThreads), lds, stream, a);
+    return hipGetLastError();
 }
 
 template <int FMT, int B, int R>
@@ -592,7 +823,7 @@ hipError_t launch_fmt(const KernelArgs &a, int batch, hipStream_t stream) {
 
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     const DeviceMatrix &w = p.w;
-    if (!w.qs || !p.x || w.rows <= 0 || w.cols <= 0 || p.batch <= 0) return hipErrorInvalidValue;
+    if (!w.qs || (!p.x && !p.norm_x) || (p.norm_x && !p.norm_w) || w.rows <= 0 || w.cols <= 0 || p.batch <= 0) return hipErrorInvalidValue;
     if ((p.epilogue == EPI_STORE_F32 || p.epilogue == EPI_ADD_RESIDUAL) && !p.y) return hipErrorInvalidValue;
     if (p.epilogue == EPI_ADD_RESIDUAL && !p.residual) return hipErrorInvalidValue;
     if (p.epilogue == EPI_SWIGLU_F16 && (!p.out_f16 || w.rows % 2 != 0)) return hipErrorInvalidValue;
@@ -603,7 +834,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
             return hipErrorInvalidValue;
     }
     const int block = w.format == FMT_F16 ? 8 : w.format == FMT_F32 ? 4 : format_block_elems(w.format);
-    if (w.cols % block != 0 || w.qs_row_bytes % 16 != 0) return hipErrorInvalidValue;
+    if (w.cols % block != 0 || w.qs_row_bytes % 16 != 0 || (p.norm_x && w.cols % 8 != 0)) return hipErrorInvalidValue;
     if ((w.format == FMT_Q8_0 || w.format == FMT_Q4_0) && !w.scales) return hipErrorInvalidValue;
 
     // batches beyond 2 run as successive pairs (each pair re-reads the weights)
@@ -622,6 +853,9 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
             a.qkv.q_out += (size_t)b0 * p.qkv.n_head * p.qkv.head_dim;
         }
         a.epilogue = p.epilogue;
+        a.norm_x = p.norm_x ? p.norm_x + (size_t)b0 * w.cols : nullptr;
+        a.norm_w = p.norm_w;
+        a.norm_eps = p.norm_eps;
         hipError_t e;
         switch (w.format) {
         case FMT_Q4_K: e = nb == 1 ? launch_q4k<1>(a, stream) : launch_q4k<2>(a, stream); break;

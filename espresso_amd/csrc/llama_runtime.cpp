@@ -369,9 +369,9 @@ int LlamaRuntime::enqueue_trunk(int M) {
     int rc = ESP_OK;
     ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, M, d, hidden_, s));
     for (Layer &L : layers_) {
-        ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_att, c_.norm_eps, M, d, xn_, nullptr, s));
+        // both RMSNorms of the layer run inside the staging of the GEMV that consumes them
         GemvParams g;
-        g.w = L.wqkv; g.x = xn_; g.batch = M;
+        g.w = L.wqkv; g.norm_x = hidden_; g.norm_w = L.rms_att; g.norm_eps = c_.norm_eps; g.batch = M;
         const size_t cache_seq_stride = (size_t)kd * c_.max_seq;
         if (L.q_norm) {
             // per-head q/k norm needs whole heads before RoPE: plain GEMV, then the post kernel
@@ -409,12 +409,13 @@ int LlamaRuntime::enqueue_trunk(int M) {
         if ((rc = time_begin(K_WO)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
-        ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_ffn, c_.norm_eps, M, d, xn_, nullptr, s));
-        g.w = L.w13; g.x = xn_; g.y = nullptr; g.residual = nullptr; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
+        g.w = L.w13; g.x = nullptr; g.norm_x = hidden_; g.norm_w = L.rms_ffn; g.norm_eps = c_.norm_eps;
+        g.y = nullptr; g.residual = nullptr; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
         if ((rc = time_begin(K_GATE_UP)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
-        g.w = L.w2; g.x = act_; g.y = hidden_; g.residual = hidden_; g.out_f16 = nullptr; g.epilogue = EPI_ADD_RESIDUAL;
+        g.w = L.w2; g.x = act_; g.norm_x = nullptr; g.norm_w = nullptr;
+        g.y = hidden_; g.residual = hidden_; g.out_f16 = nullptr; g.epilogue = EPI_ADD_RESIDUAL;
         if ((rc = time_begin(K_DOWN)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
@@ -458,9 +459,9 @@ int LlamaRuntime::prefill(int seq, const uint32_t *tokens, int count) {
 
 int LlamaRuntime::run_head(const float *hidden_rows, int count) {
     hipStream_t s = context().stream;
-    ESP_HIP_TRY(launch_rmsnorm(hidden_rows, final_norm_, c_.norm_eps, count, c_.d_model, xn_, nullptr, s));
-    GemvParams g;
-    g.w = lm_head_; g.x = xn_; g.y = logits_; g.batch = count; g.epilogue = EPI_STORE_F32;
+    GemvParams g;   // final RMSNorm fused into the head GEMV's staging
+    g.w = lm_head_; g.norm_x = hidden_rows; g.norm_w = final_norm_; g.norm_eps = c_.norm_eps;
+    g.y = logits_; g.batch = count; g.epilogue = EPI_STORE_F32;
     int rc;
     if ((rc = time_begin(K_HEAD)) != ESP_OK) return rc;
     ESP_HIP_TRY(launch_gemv(g, s));
