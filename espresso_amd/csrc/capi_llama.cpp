@@ -127,6 +127,12 @@ int esp_llama_set_graph_replay(ESPLlamaRuntime *runtime, int enabled) {
     return ESP_OK;
 }
 
+int esp_llama_set_matrix_prefill(ESPLlamaRuntime *runtime, int enabled) {
+    if (!runtime || !runtime->rt) return fail(ESP_ERR_INVALID_ARGUMENT, "set_matrix_prefill: null runtime");
+    runtime->rt->set_matrix_prefill(enabled != 0);
+    return ESP_OK;
+}
+
 int esp_llama_set_kernel_timing(ESPLlamaRuntime *runtime, int enabled) {
     if (!runtime) return bad_handle();
     runtime->rt->set_kernel_timing(enabled != 0);

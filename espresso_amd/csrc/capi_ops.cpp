@@ -82,6 +82,24 @@ int esp_matrix_dequantize(const ESPMatrix *matrix, float *out) {
     return e == hipSuccess ? ESP_OK : fail_hip(e, "matrix_dequantize");
 }
 
+namespace {
+// More than two rows of activations go to the matrix-core kernel (fp32 matrices stay on the GEMV path).
+bool use_gemm(const DeviceMatrix &m, int batch) { return batch > 2 && m.format != FMT_F32 && m.cols % 64 == 0; }
+constexpr size_t kGemmWorkspaceFloats = (size_t)8 << 20;   // 32 MiB of split-K partial sums
+
+hipError_t run_matvec(const DeviceMatrix &m, const uint16_t *d_x, int batch, float *d_y, const float *d_res, float *workspace, hipStream_t s) {
+    if (use_gemm(m, batch)) {
+        GemmParams g;
+        g.w = m; g.x = d_x; g.y = d_y; g.residual = d_res; g.rows = batch; g.workspace = workspace; g.workspace_floats = workspace ? kGemmWorkspaceFloats : 0;
+        return launch_gemm(g, s);
+    }
+    GemvParams p;
+    p.w = m; p.x = d_x; p.y = d_y; p.residual = d_res; p.batch = batch;
+    p.epilogue = d_res ? EPI_ADD_RESIDUAL : EPI_STORE_F32;
+    return launch_gemv(p, s);
+}
+}  // namespace
+
 int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y, const float *residual) {
     if (!matrix || !x_f16 || !y) return fail(ESP_ERR_INVALID_ARGUMENT, "gemv: null pointer");
     if (batch <= 0) return fail(ESP_ERR_INVALID_ARGUMENT, "gemv: batch %d", batch);
@@ -91,22 +109,22 @@ int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y
     const DeviceMatrix &m = matrix->m;
     const size_t nx = (size_t)batch * m.cols, ny = (size_t)batch * m.rows;
     uint16_t *d_x = nullptr;
-    float *d_y = nullptr, *d_res = nullptr;
+    float *d_y = nullptr, *d_res = nullptr, *d_ws = nullptr;
     if ((rc = device_alloc(&d_x, nx)) != ESP_OK) return rc;
     if ((rc = device_alloc(&d_y, ny)) != ESP_OK) { (void)hipFree(d_x); return rc; }
     if (residual && (rc = device_alloc(&d_res, ny)) != ESP_OK) { (void)hipFree(d_x); (void)hipFree(d_y); return rc; }
+    if (use_gemm(m, batch) && (rc = device_alloc(&d_ws, kGemmWorkspaceFloats)) != ESP_OK) {
+        (void)hipFree(d_x); (void)hipFree(d_y); if (d_res) (void)hipFree(d_res);
+        return rc;
+    }
     hipError_t e = hipMemcpyAsync(d_x, x_f16, nx * 2, hipMemcpyHostToDevice, c.stream);
     if (e == hipSuccess && residual) e = hipMemcpyAsync(d_res, residual, ny * 4, hipMemcpyHostToDevice, c.stream);
-    if (e == hipSuccess) {
-        GemvParams p;
-        p.w = m; p.x = d_x; p.y = d_y; p.residual = d_res; p.batch = batch;
-        p.epilogue = residual ? EPI_ADD_RESIDUAL : EPI_STORE_F32;
-        e = launch_gemv(p, c.stream);
-    }
+    if (e == hipSuccess) e = run_matvec(m, d_x, batch, d_y, d_res, d_ws, c.stream);
     if (e == hipSuccess) e = hipMemcpyAsync(y, d_y, ny * 4, hipMemcpyDeviceToHost, c.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
     (void)hipFree(d_x); (void)hipFree(d_y);
     if (d_res) (void)hipFree(d_res);
+    if (d_ws) (void)hipFree(d_ws);
     return e == hipSuccess ? ESP_OK : fail_hip(e, "gemv");
 }
 
@@ -123,7 +141,7 @@ int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int
 
     std::vector<DeviceMatrix> copies(rotate, m);
     uint16_t *d_x = nullptr;
-    float *d_y = nullptr;
+    float *d_y = nullptr, *d_ws = nullptr;
     std::vector<hipEvent_t> marks;
     hipError_t e = hipSuccess;
     rc = ESP_OK;
@@ -138,6 +156,7 @@ int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int
     }
     if (rc == ESP_OK) rc = device_alloc(&d_x, nx);
     if (rc == ESP_OK) rc = device_alloc(&d_y, ny);
+    if (rc == ESP_OK && use_gemm(m, batch)) rc = device_alloc(&d_ws, kGemmWorkspaceFloats);
     if (rc == ESP_OK) {
         // activations ~ small deterministic values; the kernel's timing does not depend on them
         std::vector<uint16_t> hx(nx);
@@ -147,24 +166,21 @@ int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int
         if (e != hipSuccess) rc = fail_hip(e, "gemv_time upload");
     }
     if (rc == ESP_OK) {
-        GemvParams p;
-        p.x = d_x; p.y = d_y; p.batch = batch; p.epilogue = EPI_STORE_F32;
-        for (int i = 0; i < warmup && e == hipSuccess; i++) { p.w = copies[i % rotate]; e = launch_gemv(p, c.stream); }
+        auto launch = [&](const DeviceMatrix &w) { return run_matvec(w, d_x, batch, d_y, nullptr, d_ws, c.stream); };
+        for (int i = 0; i < warmup && e == hipSuccess; i++) e = launch(copies[i % rotate]);
         // mean: `iters` launches queued back to back between two events
         marks.resize(iters + 3, nullptr);
         for (auto &ev : marks) if (e == hipSuccess) e = hipEventCreate(&ev);
         hipEvent_t t0 = marks[iters + 1], t1 = marks[iters + 2];
         if (e == hipSuccess) e = hipEventRecord(t0, c.stream);
         for (int i = 0; i < iters && e == hipSuccess; i++) {
-            p.w = copies[(warmup + i) % rotate];
-            e = launch_gemv(p, c.stream);
+            e = launch(copies[(warmup + i) % rotate]);
         }
         if (e == hipSuccess) e = hipEventRecord(t1, c.stream);
         // best: every launch bracketed by its own events
         if (e == hipSuccess) e = hipEventRecord(marks[0], c.stream);
         for (int i = 0; i < iters && e == hipSuccess; i++) {
-            p.w = copies[(warmup + i) % rotate];
-            e = launch_gemv(p, c.stream);
+            e = launch(copies[(warmup + i) % rotate]);
             if (e == hipSuccess) e = hipEventRecord(marks[i + 1], c.stream);
         }
         if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
@@ -186,6 +202,7 @@ int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int
     for (int i = 1; i < rotate; i++) { if (copies[i].qs) (void)hipFree(copies[i].qs); if (copies[i].scales) (void)hipFree(copies[i].scales); }
     if (d_x) (void)hipFree(d_x);
     if (d_y) (void)hipFree(d_y);
+    if (d_ws) (void)hipFree(d_ws);
     return rc;
 }
 

@@ -81,8 +81,21 @@ struct GemvParams {
     int epilogue = EPI_STORE_F32;
 };
 
+// y[rows][w.rows] = x[rows][w.cols] * dequant(w)^T (+ residual) for more than two rows, on the matrix cores.
+struct GemmParams {
+    DeviceMatrix w;
+    const uint16_t *x = nullptr;      // fp16 activations [rows][cols]
+    float *y = nullptr;               // fp32 out [rows][w.rows]
+    const float *residual = nullptr;  // optional [rows][w.rows], may alias y
+    int rows = 0;
+    float *workspace = nullptr;       // split-K partial sums for short row counts (optional)
+    size_t workspace_floats = 0;
+};
+
 // kernels/gemv.hip
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
+// kernels/gemm.hip
+hipError_t launch_gemm(const GemmParams &p, hipStream_t stream);
 // kernels/dequant.hip — GGUF-layout blocks -> fp32, bit-exact to the block definitions
 hipError_t launch_dequant(int format, const uint8_t *blocks, size_t elems, float *out, hipStream_t stream);
 // GGUF-layout blocks -> DeviceMatrix planes (device to device)

@@ -1,0 +1,576 @@
+// Dequant-fused MFMA GEMM for more than two activation rows (prompt prefill, batched verify, batch-8
+// microbenchmarks):   y[m][n] = sum_k x[m][k] * dequant(W)[n][k],   fp16 operands, fp32 accumulation.
+//
+// Replaces the per-token vDSP_mmul calls the reference issues while it walks a prompt
+// (RealModelInferenceEngine.swift:6674-6697 inside the prefill loop :6365-6375) by one pass over the
+// packed weights per block of rows.
+//
+// Shape of the kernel (gfx950, wave64)
+//   * a workgroup of four wavefronts owns 128 weight rows (n) x MT activation rows (m) and walks K in
+//     tiles of 64;
+//   * per K tile every thread fetches the packed bytes of (one weight row, one half of the tile) with
+//     128-bit loads, turns them into 32 fp16 weights in registers (nibble / byte exponent tricks, one
+//     packed fp16 multiply-add with the block's scale and minimum) and writes them to LDS; the fp16
+//     activations of the tile are copied to LDS next to them;
+//   * every weight reaches the matrix core as its dequantised value rounded to fp16 exactly once (Q4_K:
+//     n * d*sc - dmin*m in fp32 first; Q4_0 / Q8_0: one exact packed fp16 product);
+//   * the Q4_0 / Q8_0 exponent tricks yield elements in (0,2,1,3) order inside every group of four; the
+//     activations are stored with the same swap, which costs nothing because a dot product does not care
+//     about the order of k as long as both operands agree;
+//   * v_mfma_f32_32x32x16_f16: activations are the A operand (rows m), weights the B operand (columns
+//     n), so a lane's 16 accumulators belong to one weight row and 16 activation rows;
+//   * the global loads of several tiles ahead are in flight while the matrix cores work on tile t;
+//   * when the (n, m) grid is too small to fill the chip, K is split over grid.y and a small kernel
+//     adds the partial sums in split order (deterministic, no atomics).
+#include "../common.h"
+
+namespace esp {
+namespace {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32;
+
+constexpr int kThreads = 256;
+constexpr int KT = 64;        // k per tile
+constexpr int LDK = KT + 8;   // fp16 per LDS row: 144 bytes, so eight rows cover all banks
+constexpr int NT = 128;       // weight rows per workgroup: two threads per row
+
+struct GemmArgs {
+    const uint8_t *qs;
+    const uint16_t *scales;
+    size_t qs_row_bytes;
+    int N, K, M;
+    const uint16_t *x;      // [M][K] fp16
+    float *y;               // [M][N]
+    const float *residual;  // [M][N] or null
+    float *partial;         // [splits][M][N] when gridDim.y > 1
+    int tiles_per_split;
+};
+
+__device__ __forceinline__ h2 as_h2(u32 v) { return __builtin_bit_cast(h2, v); }
+__device__ __forceinline__ u32 as_u32(h2 v) { return __builtin_bit_cast(u32, v); }
+__device__ __forceinline__ float half_bits_to_float(u32 bits16) { return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16); }
+__device__ __forceinline__ h2 splat(float v) { const _Float16 h = (_Float16)v; return h2{h, h}; }
+__device__ __forceinline__ u32 dword_of(const uint4 &v, int k) { return k == 0 ? v.x : k == 1 ? v.y : k == 2 ? v.z : v.w; }
+__device__ __forceinline__ uint4 swap_middle(const uint4 &v) {
+    uint4 p;
+    p.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
+    p.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
+    p.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
+    p.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
+    return p;
+}
+
+// The packed bytes one thread holds for (weight row, half h of a K tile), per format.
+template <int FMT>
+struct Raw;
+template <>
+struct Raw<FMT_Q4_K> { uint4 q, hdr; };          // 16 bytes of nibbles + the super-block header
+template <>
+struct Raw<FMT_Q4_0> { uint4 q; u32 d; };        // one block
+template <>
+struct Raw<FMT_Q8_0> { uint4 q0, q1; u32 d; };   // one block
+template <>
+struct Raw<FMT_F16> { uint4 v[4]; };
+
+template <int FMT>
+__device__ __forceinline__ Raw<FMT> fetch_raw(const GemmArgs &a, int row, int tile, int h) {
+    Raw<FMT> r;
+    const uint8_t *base = a.qs + (size_t)row * a.qs_row_bytes;
+    if constexpr (FMT == FMT_Q4_K) {
+        const uint8_t *blk = base + (size_t)(tile >> 2) * 144;
+        r.hdr = *reinterpret_cast<const uint4 *>(blk);
+        r.q = *reinterpret_cast<const uint4 *>(blk + 16 + (tile & 3) * 32 + h * 16);
+    } else if constexpr (FMT == FMT_Q4_0) {
+        const int block = tile * 2 + h;
+        r.q = *reinterpret_cast<const uint4 *>(base + (size_t)block * 16);
+        r.d = a.scales[(size_t)row * (a.K / 32) + block];
+    } else if constexpr (FMT == FMT_Q8_0) {
+        const int block = tile * 2 + h;
+        const uint4 *q = reinterpret_cast<const uint4 *>(base + (size_t)block * 32);
+        r.q0 = q[0];
+        r.q1 = q[1];
+        r.d = a.scales[(size_t)row * (a.K / 32) + block];
+    } else {
+        const uint4 *q = reinterpret_cast<const uint4 *>(base + ((size_t)tile * KT + h * 32) * 2);
+#pragma unroll
+        for (int i = 0; i < 4; i++) r.v[i] = q[i];
+    }
+    return r;
+}
+
+// Byte `idx` (0..11) of the twelve scale bytes that follow d and dmin in a Q4_K header.
+__device__ __forceinline__ u32 scale_byte(const uint4 &hdr, int idx) {
+    const u32 word = idx < 4 ? hdr.y : idx < 8 ? hdr.z : hdr.w;
+    return (word >> ((idx & 3) * 8)) & 0xFFu;
+}
+// ggml's get_scale_min_k4
+__device__ __forceinline__ void q4k_scale_min(const uint4 &hdr, int j, float &sc, float &m) {
+    if (j < 4) {
+        sc = (float)(scale_byte(hdr, j) & 63u);
+        m = (float)(scale_byte(hdr, j + 4) & 63u);
+    } else {
+        sc = (float)((scale_byte(hdr, j + 4) & 0xFu) | ((scale_byte(hdr, j - 4) >> 6) << 4));
+        m = (float)((scale_byte(hdr, j + 4) >> 4) | ((scale_byte(hdr, j) >> 6) << 4));
+    }
+}
+
+// Four weights of dword `w` per call: nibbles at bits 0..3 (offset 1024) or 4..7 (offset 64) become exact
+// fp16 integers, then w = n * s - dm in packed fp16 (one rounding per weight).
+__device__ __forceinline__ uint2 nibbles_to_half(u32 w, bool high, h2 s, h2 dm) {
+    const u32 mask = high ? 0x00F000F0u : 0x000F000Fu, magic = high ? 0x54005400u : 0x64006400u;
+    const h2 off = high ? h2{(_Float16)64.0f, (_Float16)64.0f} : h2{(_Float16)1024.0f, (_Float16)1024.0f};
+    const h2 n02 = as_h2((w & mask) | magic) - off, n13 = as_h2(((w >> 8) & mask) | magic) - off;
+    return make_uint2(as_u32(__builtin_elementwise_fma(n02, s, -dm)), as_u32(__builtin_elementwise_fma(n13, s, -dm)));
+}
+
+// Q4_K: four nibbles spread over the bytes of `b` -> fp16(n * s - dm) with the product and the subtraction in
+// fp32, so each weight is the dequantised value rounded to fp16 once (n * s and dm can both be several
+// times larger than their difference; rounding them separately in fp16 would cost two more bits).
+__device__ __forceinline__ uint2 q4k_bytes_to_half(u32 b, float s, float dm) {
+    const float w0 = __builtin_fmaf((float)(b & 0xFFu), s, -dm), w1 = __builtin_fmaf((float)((b >> 8) & 0xFFu), s, -dm);
+    const float w2 = __builtin_fmaf((float)((b >> 16) & 0xFFu), s, -dm), w3 = __builtin_fmaf((float)(b >> 24), s, -dm);
+    return make_uint2(as_u32(h2{(_Float16)w0, (_Float16)w1}), as_u32(h2{(_Float16)w2, (_Float16)w3}));
+}
+
+// Writes the thread's 32 fp16 weights into its LDS row (`wrow` points at k = 0 of the tile).
+// Element order inside each group of four is (0,2,1,3) for Q4_0 and Q8_0, natural for Q4_K and F16.
+template <int FMT>
+__device__ __forceinline__ void dequant_to_lds(const Raw<FMT> &r, int tile, int h, _Float16 *wrow) {
+    if constexpr (FMT == FMT_Q4_K) {
+        // low nibbles: sub-block 2c, elements 16h..16h+15 (k = 16h..); high nibbles: sub-block 2c+1 (k = 32+16h..)
+        const int c = tile & 3;
+        const float d = half_bits_to_float(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float(r.hdr.x >> 16);
+        float sc_lo, m_lo, sc_hi, m_hi;
+        q4k_scale_min(r.hdr, 2 * c, sc_lo, m_lo);
+        q4k_scale_min(r.hdr, 2 * c + 1, sc_hi, m_hi);
+        const float s_lo = d * sc_lo, dm_lo = dmin * m_lo, s_hi = d * sc_hi, dm_hi = dmin * m_hi;
+        uint2 lo[4], hi[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            lo[k] = q4k_bytes_to_half(dword_of(r.q, k) & 0x0F0F0F0Fu, s_lo, dm_lo);
+            hi[k] = q4k_bytes_to_half((dword_of(r.q, k) >> 4) & 0x0F0F0F0Fu, s_hi, dm_hi);
+        }
+        uint4 *plo = reinterpret_cast<uint4 *>(wrow + 16 * h), *phi = reinterpret_cast<uint4 *>(wrow + 32 + 16 * h);
+        plo[0] = make_uint4(lo[0].x, lo[0].y, lo[1].x, lo[1].y);
+        plo[1] = make_uint4(lo[2].x, lo[2].y, lo[3].x, lo[3].y);
+        phi[0] = make_uint4(hi[0].x, hi[0].y, hi[1].x, hi[1].y);
+        phi[1] = make_uint4(hi[2].x, hi[2].y, hi[3].x, hi[3].y);
+    } else if constexpr (FMT == FMT_Q4_0) {
+        // byte j: low nibble = element j, high nibble = element j + 16; w = (n - 8) * d
+        const h2 s = splat(half_bits_to_float(r.d)), dm = splat(8.0f * half_bits_to_float(r.d));
+        uint2 lo[4], hi[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            lo[k] = nibbles_to_half(dword_of(r.q, k), false, s, dm);
+            hi[k] = nibbles_to_half(dword_of(r.q, k), true, s, dm);
+        }
+        uint4 *p = reinterpret_cast<uint4 *>(wrow + 32 * h);
+        p[0] = make_uint4(lo[0].x, lo[0].y, lo[1].x, lo[1].y);
+        p[1] = make_uint4(lo[2].x, lo[2].y, lo[3].x, lo[3].y);
+        p[2] = make_uint4(hi[0].x, hi[0].y, hi[1].x, hi[1].y);
+        p[3] = make_uint4(hi[2].x, hi[2].y, hi[3].x, hi[3].y);
+    } else if constexpr (FMT == FMT_Q8_0) {
+        const h2 s = splat(half_bits_to_float(r.d)), off = h2{(_Float16)1152.0f, (_Float16)1152.0f};   // 1024 + 128
+        uint4 *p = reinterpret_cast<uint4 *>(wrow + 32 * h);
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const uint4 &q = half ? r.q1 : r.q0;
+            u32 out[8];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const u32 t = dword_of(q, k) ^ 0x80808080u;   // signed -> biased
+                const h2 f02 = as_h2(__builtin_amdgcn_perm(0x64646464u, t, 0x04020400u)) - off;
+                const h2 f13 = as_h2(__builtin_amdgcn_perm(0x64646464u, t, 0x04030401u)) - off;
+                out[2 * k] = as_u32(f02 * s);
+                out[2 * k + 1] = as_u32(f13 * s);
+            }
+            p[2 * half] = make_uint4(out[0], out[1], out[2], out[3]);
+            p[2 * half + 1] = make_uint4(out[4], out[5], out[6], out[7]);
+        }
+    } else {
+        uint4 *p = reinterpret_cast<uint4 *>(wrow + 32 * h);
+#pragma unroll
+        for (int i = 0; i < 4; i++) p[i] = r.v[i];
+    }
+}
+
+// WM x WN wavefronts, each TM x TN MFMA tiles of 32 x 32: the workgroup covers 32*WM*TM rows of x and
+// 32*WN*TN = 128 weight rows.  DEPTH tiles of packed weights and activations are in flight in registers
+// (a slot is refilled as soon as its tile has gone to LDS), and LDS holds two tiles so that one barrier
+// per tile is enough: tile t+1 is written while other wavefronts still read tile t.
+template <int FMT, int WM, int WN, int TM, int TN, int DEPTH>
+__global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs a) {
+    static_assert(WM * WN == 4 && 32 * WN * TN == NT, "four wavefronts over 128 weight rows");
+    constexpr int MT = 32 * WM * TM;
+    constexpr bool kSwap = FMT == FMT_Q4_0 || FMT == FMT_Q8_0;   // formats whose unpacking yields (0,2,1,3) order
+    constexpr int XV = MT * KT / 8 / kThreads;   // 128-bit pieces of x per thread per tile
+    static_assert(XV >= 1, "tile too small for the copy loop");
+    __shared__ _Float16 xt[2][MT * LDK];
+    __shared__ _Float16 wt[2][NT * LDK];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int n0 = blockIdx.x * NT, m0 = blockIdx.z * MT;
+    const int tiles = a.K / KT;
+    const int t_begin = blockIdx.y * a.tiles_per_split;
+    const int t_end = t_begin + a.tiles_per_split < tiles ? t_begin + a.tiles_per_split : tiles;
+
+    // dequantisation role: weight row and half of the tile
+    const int wr = tid >> 1, wh = tid & 1;
+    const int w_row = n0 + wr < a.N ? n0 + wr : a.N - 1;   // clamped, the result is never stored
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    auto fetch_x = [&](int tile, uint4 (&xv)[XV]) {
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const int piece = tid + i * kThreads, row = piece >> 3, part = piece & 7;   // eight pieces per row
+            const int m = m0 + row;
+            xv[i] = m < a.M ? reinterpret_cast<const uint4 *>(a.x + (size_t)m * a.K + (size_t)tile * KT)[part] : make_uint4(0, 0, 0, 0);
+        }
+    };
+
+    Raw<FMT> raw[DEPTH];
+    uint4 xv[DEPTH][XV];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+        if (t_begin + d < t_end) {
+            raw[d] = fetch_raw<FMT>(a, w_row, t_begin + d, wh);
+            fetch_x(t_begin + d, xv[d]);
+        }
+    }
+    for (int t0 = t_begin; t0 < t_end; t0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            const int t = t0 + d, buf = d & 1;   // DEPTH is even, so the parity of d is the parity of the tile count
+            if (t < t_end) {
+                dequant_to_lds<FMT>(raw[d], t, wh, wt[buf] + wr * LDK);
+#pragma unroll
+                for (int i = 0; i < XV; i++) {
+                    const int piece = tid + i * kThreads, row = piece >> 3, part = piece & 7;
+                    *reinterpret_cast<uint4 *>(xt[buf] + row * LDK + part * 8) = kSwap ? swap_middle(xv[d][i]) : xv[d][i];
+                }
+                if (t + DEPTH < t_end) {   // refill the slot: DEPTH tiles of global loads stay in flight
+                    raw[d] = fetch_raw<FMT>(a, w_row, t + DEPTH, wh);
+                    fetch_x(t + DEPTH, xv[d]);
+                }
+            }
+            __syncthreads();
+            if (t < t_end) {
+#pragma unroll
+                for (int ks = 0; ks < KT / 16; ks++) {
+                    const int kk = ks * 16 + 8 * (lane >> 5);
+                    half8 af[TM], bf[TN];
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+                        af[i] = *reinterpret_cast<const half8 *>(xt[buf] + ((wm * TM + i) * 32 + (lane & 31)) * LDK + kk);
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        bf[j] = *reinterpret_cast<const half8 *>(wt[buf] + ((wn * TN + j) * 32 + (lane & 31)) * LDK + kk);
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // accumulator r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32 x 32 tile
+    const bool split = gridDim.y > 1;
+    float *out = split ? a.partial + (size_t)blockIdx.y * a.M * a.N : a.y;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + (wn * TN + j) * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < a.M && n < a.N) {
+                    const size_t o = (size_t)m * a.N + n;
+                    out[o] = (!split && a.residual) ? a.residual[o] + acc[i][j][r] : acc[i][j][r];
+                }
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Short M (at most 64 activation rows): the weights never touch LDS.  In v_mfma_f32_32x32x16_f16 a lane
+// of the B operand holds eight consecutive k of ONE column, so a lane can load 16 packed bytes of its
+// own weight row, dequantise them in registers and feed them to the matrix core directly; lanes 0..31
+// and 32..63 of a wavefront take the two halves of each 64-k tile of the same 32 weight rows.  A
+// wavefront owns 32 weight rows, a workgroup 128.  Only the activations go through LDS, 256 k at a
+// time and double-buffered, so there is one barrier per 256 k.  Packed weights for DEPTH chunks of
+// 256 k are in flight per lane.
+constexpr int CK = 256;        // k per activation stage
+constexpr int LDX = CK + 8;    // fp16 per LDS row of activations
+
+template <int FMT>
+struct RawChunk;
+template <>
+struct RawChunk<FMT_Q4_K> { uint4 hdr, q[4]; };
+template <>
+struct RawChunk<FMT_Q4_0> { uint4 q[4]; u32 d[4]; };
+template <>
+struct RawChunk<FMT_Q8_0> { uint4 q[8]; u32 d[4]; };
+
+template <int FMT>
+__device__ __forceinline__ RawChunk<FMT> fetch_chunk(const GemmArgs &a, int row, int chunk, int h) {
+    RawChunk<FMT> r;
+    const uint8_t *base = a.qs + (size_t)row * a.qs_row_bytes;
+    if constexpr (FMT == FMT_Q4_K) {
+        const uint8_t *blk = base + (size_t)chunk * 144;
+        r.hdr = *reinterpret_cast<const uint4 *>(blk);
+#pragma unroll
+        for (int c = 0; c < 4; c++) r.q[c] = *reinterpret_cast<const uint4 *>(blk + 16 + c * 32 + h * 16);
+    } else if constexpr (FMT == FMT_Q4_0) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int block = chunk * 8 + t * 2 + h;
+            r.q[t] = *reinterpret_cast<const uint4 *>(base + (size_t)block * 16);
+            r.d[t] = a.scales[(size_t)row * (a.K / 32) + block];
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int block = chunk * 8 + t * 2 + h;
+            const uint4 *q = reinterpret_cast<const uint4 *>(base + (size_t)block * 32);
+            r.q[2 * t] = q[0];
+            r.q[2 * t + 1] = q[1];
+            r.d[t] = a.scales[(size_t)row * (a.K / 32) + block];
+        }
+    }
+    return r;
+}
+
+__device__ __forceinline__ half8 as_half8(const uint4 &v) { return __builtin_bit_cast(half8, v); }
+
+// The four B fragments (eight fp16 each) a lane contributes to 64-k tile `t` of its chunk, and the k offset
+// inside the tile at which the matching activations start.  Element order inside groups of four matches
+// the activations' LDS copy (natural for Q4_K, (0,2,1,3) for Q4_0 and Q8_0).
+template <int FMT>
+__device__ __forceinline__ void tile_fragments(const RawChunk<FMT> &r, int t, int h, half8 frag[4], int koff[4]) {
+    if constexpr (FMT == FMT_Q4_K) {
+        const float d = half_bits_to_float(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float(r.hdr.x >> 16);
+        float sc_lo, m_lo, sc_hi, m_hi;
+        q4k_scale_min(r.hdr, 2 * t, sc_lo, m_lo);
+        q4k_scale_min(r.hdr, 2 * t + 1, sc_hi, m_hi);
+        const float s_lo = d * sc_lo, dm_lo = dmin * m_lo, s_hi = d * sc_hi, dm_hi = dmin * m_hi;
+        uint2 lo[4], hi[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            lo[k] = q4k_bytes_to_half(dword_of(r.q[t], k) & 0x0F0F0F0Fu, s_lo, dm_lo);
+            hi[k] = q4k_bytes_to_half((dword_of(r.q[t], k) >> 4) & 0x0F0F0F0Fu, s_hi, dm_hi);
+        }
+        frag[0] = as_half8(make_uint4(lo[0].x, lo[0].y, lo[1].x, lo[1].y));
+        frag[1] = as_half8(make_uint4(lo[2].x, lo[2].y, lo[3].x, lo[3].y));
+        frag[2] = as_half8(make_uint4(hi[0].x, hi[0].y, hi[1].x, hi[1].y));
+        frag[3] = as_half8(make_uint4(hi[2].x, hi[2].y, hi[3].x, hi[3].y));
+        koff[0] = 16 * h; koff[1] = 16 * h + 8; koff[2] = 32 + 16 * h; koff[3] = 40 + 16 * h;
+    } else if constexpr (FMT == FMT_Q4_0) {
+        const h2 s = splat(half_bits_to_float(r.d[t])), dm = splat(8.0f * half_bits_to_float(r.d[t]));
+        uint2 lo[4], hi[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            lo[k] = nibbles_to_half(dword_of(r.q[t], k), false, s, dm);
+            hi[k] = nibbles_to_half(dword_of(r.q[t], k), true, s, dm);
+        }
+        frag[0] = as_half8(make_uint4(lo[0].x, lo[0].y, lo[1].x, lo[1].y));
+        frag[1] = as_half8(make_uint4(lo[2].x, lo[2].y, lo[3].x, lo[3].y));
+        frag[2] = as_half8(make_uint4(hi[0].x, hi[0].y, hi[1].x, hi[1].y));
+        frag[3] = as_half8(make_uint4(hi[2].x, hi[2].y, hi[3].x, hi[3].y));
+#pragma unroll
+        for (int f = 0; f < 4; f++) koff[f] = 32 * h + 8 * f;
+    } else {
+        const h2 s = splat(half_bits_to_float(r.d[t])), off = h2{(_Float16)1152.0f, (_Float16)1152.0f};
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const uint4 &q = r.q[2 * t + half];
+            u32 out[8];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const u32 b = dword_of(q, k) ^ 0x80808080u;
+                const h2 f02 = as_h2(__builtin_amdgcn_perm(0x64646464u, b, 0x04020400u)) - off;
+                const h2 f13 = as_h2(__builtin_amdgcn_perm(0x64646464u, b, 0x04030401u)) - off;
+                out[2 * k] = as_u32(f02 * s);
+                out[2 * k + 1] = as_u32(f13 * s);
+            }
+            frag[2 * half] = as_half8(make_uint4(out[0], out[1], out[2], out[3]));
+            frag[2 * half + 1] = as_half8(make_uint4(out[4], out[5], out[6], out[7]));
+        }
+#pragma unroll
+        for (int f = 0; f < 4; f++) koff[f] = 32 * h + 8 * f;
+    }
+}
+
+template <int FMT, int TM, int DEPTH>
+__global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(GemmArgs a) {
+    constexpr int MT = 32 * TM;
+    constexpr int XV = MT * CK / 8 / kThreads;   // 128-bit pieces of x per thread per chunk (4 per 32 rows)
+    __shared__ _Float16 xt[2][MT * LDX];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+    const int n = blockIdx.x * NT + wave * 32 + (lane & 31);
+    const int w_row = n < a.N ? n : a.N - 1;     // clamped, the result is never stored
+    const int chunks = a.K / CK;
+    const int c_begin = blockIdx.y * a.tiles_per_split;   // split granularity is a chunk here
+    const int c_end = c_begin + a.tiles_per_split < chunks ? c_begin + a.tiles_per_split : chunks;
+
+    floatx16 acc[TM];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0.0f;
+
+    auto fetch_x = [&](int chunk, uint4 (&xv)[XV]) {
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const int piece = tid + i * kThreads, row = piece >> 5, part = piece & 31;   // 32 pieces per row
+            xv[i] = row < a.M ? reinterpret_cast<const uint4 *>(a.x + (size_t)row * a.K + (size_t)chunk * CK)[part] : make_uint4(0, 0, 0, 0);
+        }
+    };
+
+    RawChunk<FMT> raw[DEPTH];
+    uint4 xv[XV];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++)
+        if (c_begin + d < c_end) raw[d] = fetch_chunk<FMT>(a, w_row, c_begin + d, h);
+    if (c_begin < c_end) fetch_x(c_begin, xv);
+
+    for (int c0 = c_begin; c0 < c_end; c0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            const int c = c0 + d, buf = d & 1;   // DEPTH is even
+            if (c < c_end) {
+#pragma unroll
+                for (int i = 0; i < XV; i++) {
+                    const int piece = tid + i * kThreads, row = piece >> 5, part = piece & 31;
+                    *reinterpret_cast<uint4 *>(xt[buf] + row * LDX + part * 8) = FMT == FMT_Q4_K ? xv[i] : swap_middle(xv[i]);
+                }
+                if (c + 1 < c_end) fetch_x(c + 1, xv);
+            }
+            __syncthreads();
+            if (c < c_end) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    half8 frag[4];
+                    int koff[4];
+                    tile_fragments<FMT>(raw[d], t, h, frag, koff);
+#pragma unroll
+                    for (int f = 0; f < 4; f++)
+#pragma unroll
+                        for (int i = 0; i < TM; i++) {
+                            const half8 af = *reinterpret_cast<const half8 *>(xt[buf] + (i * 32 + (lane & 31)) * LDX + t * KT + koff[f]);
+                            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, frag[f], acc[i], 0, 0, 0);
+                        }
+                }
+                if (c + DEPTH < c_end) raw[d] = fetch_chunk<FMT>(a, w_row, c + DEPTH, h);
+            }
+        }
+    }
+
+    const bool split = gridDim.y > 1;
+    float *out = split ? a.partial + (size_t)blockIdx.y * a.M * a.N : a.y;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (m < a.M && n < a.N) {
+                const size_t o = (size_t)m * a.N + n;
+                out[o] = (!split && a.residual) ? a.residual[o] + acc[i][r] : acc[i][r];
+            }
+        }
+}
+
+// y = (residual +) sum over splits of partial, in split order
+__global__ void gemm_reduce_kernel(const float *partial, int splits, size_t count, const float *residual, float *y) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float s = partial[i];
+    for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + i];
+    y[i] = residual ? residual[i] + s : s;
+}
+
+template <int FMT, int WM, int WN, int TM, int TN, int DEPTH>
+hipError_t launch_tile(const GemmArgs &a, int splits, hipStream_t stream) {
+    constexpr int MT = 32 * WM * TM;
+    dim3 grid((a.N + NT - 1) / NT, splits, (a.M + MT - 1) / MT);
+    hipLaunchKernelGGL((gemm_kernel<FMT, WM, WN, TM, TN, DEPTH>), grid, dim3(kThreads), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_reduce(const GemmArgs &a, int splits, hipStream_t stream) {
+    const size_t count = (size_t)a.M * a.N;
+    hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, a.partial, splits, count, a.residual, a.y);
+    return hipGetLastError();
+}
+
+// splits so that about `target` workgroups exist, each with at least `min_units` units of K
+int choose_splits(int blocks, int units, int min_units, int target, const GemmArgs &a, size_t workspace_floats) {
+    if (!a.partial || blocks >= target) return 1;
+    int splits = (target + blocks - 1) / blocks;
+    if (splits > units / min_units) splits = units / min_units;
+    if (splits < 1) splits = 1;
+    while (splits > 1 && (size_t)splits * a.M * a.N > workspace_floats) splits--;
+    return splits;
+}
+
+template <int FMT>
+hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, hipStream_t stream) {
+    const int n_blocks = (a.N + NT - 1) / NT;
+    a.partial = workspace;
+    hipError_t e;
+    int splits;
+    if constexpr (FMT != FMT_F16) {
+        if (a.M <= 64 && a.K % CK == 0) {
+            const int chunks = a.K / CK;
+            splits = choose_splits(n_blocks, chunks, 2, 1024, a, workspace_floats);
+            a.tiles_per_split = (chunks + splits - 1) / splits;
+            splits = (chunks + a.tiles_per_split - 1) / a.tiles_per_split;
+            dim3 grid(n_blocks, splits, 1);
+            if (a.M <= 32) hipLaunchKernelGGL((gemm_skinny_kernel<FMT, 1, 2>), grid, dim3(kThreads), 0, stream, a);
+            else hipLaunchKernelGGL((gemm_skinny_kernel<FMT, 2, 2>), grid, dim3(kThreads), 0, stream, a);
+            e = hipGetLastError();
+            return e != hipSuccess || splits == 1 ? e : launch_reduce(a, splits, stream);
+        }
+    }
+    const int tiles = a.K / KT;
+    const int mt = a.M <= 32 ? 32 : a.M <= 64 ? 64 : 128;
+    splits = choose_splits(n_blocks * ((a.M + mt - 1) / mt), tiles, 8, 1024, a, workspace_floats);
+    a.tiles_per_split = (tiles + splits - 1) / splits;
+    splits = (tiles + a.tiles_per_split - 1) / a.tiles_per_split;
+    if (mt == 32) e = launch_tile<FMT, 1, 4, 1, 1, 4>(a, splits, stream);
+    else if (mt == 64) e = launch_tile<FMT, 1, 4, 2, 1, 4>(a, splits, stream);
+    else e = launch_tile<FMT, 2, 2, 2, 2, 2>(a, splits, stream);
+    return e != hipSuccess || splits == 1 ? e : launch_reduce(a, splits, stream);
+}
+
+}  // namespace
+
+hipError_t launch_gemm(const GemmParams &p, hipStream_t stream) {
+    const DeviceMatrix &w = p.w;
+    if (!w.qs || !p.x || !p.y || p.rows <= 0 || w.rows <= 0 || w.cols <= 0 || w.cols % KT != 0 || w.qs_row_bytes % 16 != 0) return hipErrorInvalidValue;
+    if ((w.format == FMT_Q8_0 || w.format == FMT_Q4_0) && !w.scales) return hipErrorInvalidValue;
+    if (w.format == FMT_Q4_K && w.cols % 256 != 0) return hipErrorInvalidValue;
+    GemmArgs a{};
+    a.qs = w.qs; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.N = w.rows; a.K = w.cols; a.M = p.rows;
+    a.x = p.x; a.y = p.y; a.residual = p.residual;
+    switch (w.format) {
+    case FMT_Q4_K: return launch_format<FMT_Q4_K>(a, p.workspace, p.workspace_floats, stream);
+    case FMT_Q4_0: return launch_format<FMT_Q4_0>(a, p.workspace, p.workspace_floats, stream);
+    case FMT_Q8_0: return launch_format<FMT_Q8_0>(a, p.workspace, p.workspace_floats, stream);
+    case FMT_F16: return launch_format<FMT_F16>(a, p.workspace, p.workspace_floats, stream);
+    default: return hipErrorInvalidValue;   // fp32 matrices stay on the GEMV path
+    }
+}
+
+}  // namespace esp

@@ -69,6 +69,7 @@ LlamaRuntime::~LlamaRuntime() {
     free_device(d_tokens_); free_device(d_pos_); free_device(d_seq_); free_device(d_out_tokens_);
     free_device(d_visible_); free_device(d_log_); free_device(d_log_count_);
     free_device(attn_scratch_);
+    free_device(gemm_workspace_);
     free_device(argmax_scratch_.part_value); free_device(argmax_scratch_.part_index);
     for (hipGraphExec_t g : step_graphs_) if (g) (void)hipGraphExecDestroy(g);
     for (TimedLaunch &t : timed_) { (void)hipEventDestroy(t.start); (void)hipEventDestroy(t.stop); }
@@ -293,12 +294,12 @@ int LlamaRuntime::finalize() {
         ESP_HIP_TRY(hipMemcpy(rope_sin_, sn.data(), sn.size() * 4, hipMemcpyHostToDevice));
     }
     // ---- activations ----
-    const size_t R = kMaxStepRows;
+    const size_t R = kPrefillBlockRows > kMaxStepRows ? kPrefillBlockRows : kMaxStepRows, RS = kMaxStepRows;
     if ((rc = device_alloc(&hidden_, R * d)) != ESP_OK) return rc;
     if ((rc = device_alloc(&qkv_, R * (ad + 2 * kd))) != ESP_OK) return rc;
     if ((rc = device_alloc(&q_, R * ad)) != ESP_OK) return rc;
     if ((rc = device_alloc(&gu_, R * 2 * hd)) != ESP_OK) return rc;
-    if ((rc = device_alloc(&logits_, R * c_.vocab)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&logits_, RS * c_.vocab)) != ESP_OK) return rc;
     if ((rc = device_alloc(&last_hidden_, (size_t)c_.max_sequences * d)) != ESP_OK) return rc;
     if ((rc = device_alloc(&xn_, R * (size_t)(d > hd ? d : hd))) != ESP_OK) return rc;
     if ((rc = device_alloc(&ctx_, R * ad)) != ESP_OK) return rc;
@@ -315,8 +316,9 @@ int LlamaRuntime::finalize() {
     if ((rc = device_alloc(&argmax_scratch_.part_index, (size_t)kArgmaxScratchSlots)) != ESP_OK) return rc;
     {
         const size_t per_row = (size_t)c_.n_kv_head * kAttentionMaxSplits * (c_.n_head / c_.n_kv_head) * (c_.head_dim + 2);
-        if ((rc = device_alloc(&attn_scratch_, (size_t)kMaxStepRows * per_row)) != ESP_OK) return rc;
+        if ((rc = device_alloc(&attn_scratch_, R * per_row)) != ESP_OK) return rc;
     }
+    if ((rc = device_alloc(&gemm_workspace_, kGemmWorkspaceFloats)) != ESP_OK) return rc;
     finalized_ = true;
     return reset();
 }
@@ -425,7 +427,7 @@ int LlamaRuntime::enqueue_trunk(int M) {
 }
 
 int LlamaRuntime::keep_row(int row, int seq) {
-    if (row < 0 || row >= kMaxStepRows || seq < 0 || seq >= c_.max_sequences)
+    if (row < 0 || row >= kPrefillBlockRows || seq < 0 || seq >= c_.max_sequences)
         return fail(ESP_ERR_OUT_OF_RANGE, "keep_row(%d, %d)", row, seq);
     ESP_HIP_TRY(launch_copy_rows(hidden_ + (size_t)row * c_.d_model, last_hidden_ + (size_t)seq * c_.d_model, 1, c_.d_model,
                                  context().stream));
@@ -450,10 +452,78 @@ int LlamaRuntime::prefill(int seq, const uint32_t *tokens, int count) {
     if (count <= 0 || !tokens) return fail(ESP_ERR_INVALID_ARGUMENT, "Prompt tokens must not be empty");
     if (seq < 0 || seq >= c_.max_sequences) return fail(ESP_ERR_OUT_OF_RANGE, "sequence %d of %d", seq, c_.max_sequences);
     visible_[seq] = 0;
+    if (matrix_prefill_ && count >= kMatrixPrefillMinTokens && matrix_prefill_supported()) {
+        // long prompts: blocks of rows through the MFMA kernels (one pass over the weights per block)
+        if (count > c_.max_seq) return fail(ESP_ERR_OUT_OF_RANGE, "runtime position %d exceeds context %d", c_.max_seq, c_.max_seq);
+        for (int i = 0; i < count; i++)
+            if (tokens[i] >= (uint32_t)c_.vocab) return fail(ESP_ERR_OUT_OF_RANGE, "token %u is outside vocab %d", tokens[i], c_.vocab);
+        int rc = ESP_OK;
+        for (int base = 0; base < count && rc == ESP_OK; base += kPrefillBlockRows) {
+            const int rows = count - base < kPrefillBlockRows ? count - base : kPrefillBlockRows;
+            rc = prefill_block(seq, tokens + base, rows, base);
+            if (rc == ESP_OK && base + rows == count) rc = keep_row(rows - 1, seq);
+        }
+        if (rc != ESP_OK) return rc;
+        ESP_HIP_TRY(hipStreamSynchronize(context().stream));
+        visible_[seq] = count;
+        return ESP_OK;
+    }
     for (int i = 0; i < count; i++) {
         int rc = advance(seq, tokens[i]);
         if (rc != ESP_OK) return rc;
     }
+    return ESP_OK;
+}
+
+bool LlamaRuntime::matrix_prefill_supported() const {
+    auto ok = [](const DeviceMatrix &m) { return m.format != FMT_F32 && m.cols % 64 == 0; };
+    for (const Layer &L : layers_)
+        if (!ok(L.wqkv) || !ok(L.wo) || !ok(L.w13) || !ok(L.w2)) return false;
+    return true;
+}
+
+// `rows` prompt tokens at positions base.. of one sequence: the layer loop of forwardToken (:6221-6347) over
+// a block of rows, every projection as one dequant-fused MFMA GEMM.  Rows of the block see each other's
+// keys and values causally because the whole block's K/V is written before its attention runs.
+int LlamaRuntime::prefill_block(int seq, const uint32_t *tokens, int rows, int base) {
+    hipStream_t s = context().stream;
+    const int d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
+    const bool kv16 = c_.kv_format == FMT_F16;
+    std::vector<int> h_tok(rows), h_pos(rows), h_seq(rows, seq);
+    for (int i = 0; i < rows; i++) { h_tok[i] = (int)tokens[i]; h_pos[i] = base + i; }
+    ESP_HIP_TRY(hipMemcpyAsync(d_tokens_, h_tok.data(), sizeof(int) * rows, hipMemcpyHostToDevice, s));
+    ESP_HIP_TRY(hipMemcpyAsync(d_pos_, h_pos.data(), sizeof(int) * rows, hipMemcpyHostToDevice, s));
+    ESP_HIP_TRY(hipMemcpyAsync(d_seq_, h_seq.data(), sizeof(int) * rows, hipMemcpyHostToDevice, s));
+    ESP_HIP_TRY(hipStreamSynchronize(s));   // the host vectors go out of scope
+    ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, rows, d, hidden_, s));
+    const size_t cache_seq_stride = (size_t)kd * c_.max_seq;
+    GemmParams g;
+    g.rows = rows; g.workspace = gemm_workspace_; g.workspace_floats = kGemmWorkspaceFloats;
+    for (Layer &L : layers_) {
+        ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_att, c_.norm_eps, rows, d, xn_, nullptr, s));
+        g.w = L.wqkv; g.x = xn_; g.y = qkv_; g.residual = nullptr;
+        ESP_HIP_TRY(launch_gemm(g, s));
+        QkvPostArgs qa{};
+        qa.qkv = qkv_; qa.q_norm = L.q_norm; qa.k_norm = L.k_norm; qa.norm_eps = c_.norm_eps;
+        qa.n_head = c_.n_head; qa.n_kv_head = c_.n_kv_head; qa.head_dim = c_.head_dim; qa.max_seq = c_.max_seq;
+        qa.rope_cos = rope_cos_; qa.rope_sin = rope_sin_; qa.pos = d_pos_; qa.seq = d_seq_;
+        qa.q_out = q_; qa.k_cache = L.k_cache; qa.v_cache = L.v_cache; qa.cache_seq_stride = cache_seq_stride;
+        ESP_HIP_TRY(launch_qkv_post(qa, rows, kv16, s));
+        AttentionArgs aa{};
+        aa.q = q_; aa.k_cache = L.k_cache; aa.v_cache = L.v_cache; aa.cache_seq_stride = cache_seq_stride;
+        aa.n_head = c_.n_head; aa.n_kv_head = c_.n_kv_head; aa.head_dim = c_.head_dim; aa.max_seq = c_.max_seq;
+        aa.pos = d_pos_; aa.seq = d_seq_; aa.ctx_f16 = ctx_; aa.split_scratch = attn_scratch_;
+        ESP_HIP_TRY(launch_attention(aa, rows, kv16, s));
+        g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_;
+        ESP_HIP_TRY(launch_gemm(g, s));
+        ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_ffn, c_.norm_eps, rows, d, xn_, nullptr, s));
+        g.w = L.w13; g.x = xn_; g.y = gu_; g.residual = nullptr;
+        ESP_HIP_TRY(launch_gemm(g, s));
+        ESP_HIP_TRY(launch_swiglu(gu_, rows, hd, act_, s));
+        g.w = L.w2; g.x = act_; g.y = hidden_; g.residual = hidden_;
+        ESP_HIP_TRY(launch_gemm(g, s));
+    }
+    (void)ad;
     return ESP_OK;
 }
 

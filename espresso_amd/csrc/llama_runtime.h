@@ -27,6 +27,10 @@ struct LlamaConfig {
     int kv_dim() const { return n_kv_head * head_dim; }
 };
 
+constexpr int kPrefillBlockRows = 256;        // rows per MFMA prefill block
+constexpr int kMatrixPrefillMinTokens = 32;   // shorter prompts take the exact per-token path
+constexpr size_t kGemmWorkspaceFloats = (size_t)8 << 20;
+
 class LlamaRuntime {
   public:
     static int create(const LlamaConfig &config, LlamaRuntime **out);
@@ -60,6 +64,8 @@ class LlamaRuntime {
     // replays of one captured HIP graph per token; the host synchronises once at the end.
     int continue_greedy(int seq, int steps, uint32_t *out_tokens);
     void set_use_graph(bool enabled) { use_graph_ = enabled; }
+    // Prompts of kMatrixPrefillMinTokens or more run in blocks through the MFMA kernels (default on).
+    void set_matrix_prefill(bool enabled) { matrix_prefill_ = enabled; }
     int read_last_hidden(int seq, float *out);
     int read_logits(int seq, float *out);         // runs the head on the kept hidden state
 
@@ -85,6 +91,8 @@ class LlamaRuntime {
     int upload_vector(const HostTensor &t, size_t count, float **out, const char *what);
     int run_head(const float *hidden_rows, int count);
     int enqueue_trunk(int rows);
+    int prefill_block(int seq, const uint32_t *tokens, int rows, int base);
+    bool matrix_prefill_supported() const;
     int capture_step_graph(int seq);
     HostTensor *host_slot(int layer, int slot);
 
@@ -111,6 +119,8 @@ class LlamaRuntime {
     int *d_visible_ = nullptr, *d_log_ = nullptr, *d_log_count_ = nullptr;
     ArgmaxScratch argmax_scratch_;
     float *attn_scratch_ = nullptr;
+    bool matrix_prefill_ = true;
+    float *gemm_workspace_ = nullptr;
 
     struct TimedLaunch { int kernel_class; hipEvent_t start, stop; };
     bool timing_enabled_ = false;

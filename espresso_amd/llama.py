@@ -160,6 +160,10 @@ def set_graph_replay(rt: LlamaRuntime, enabled: bool) -> None:
     _lib.check(rt._L.esp_llama_set_graph_replay(rt._h, int(enabled)))
 
 
+def set_matrix_prefill(rt: LlamaRuntime, enabled: bool) -> None:
+    _lib.check(rt._L.esp_llama_set_matrix_prefill(rt._h, int(enabled)))
+
+
 def set_kernel_timing(rt: LlamaRuntime, enabled: bool) -> None:
     _lib.check(rt._L.esp_llama_set_kernel_timing(rt._h, int(enabled)))
 

@@ -75,7 +75,9 @@ int esp_matrix_dequantize(const ESPMatrix *matrix, float *out);
 /* ---- dequant-fused GEMV ----------------------------------------------------------------- *
  * y[b][r] = (residual ? residual[b][r] : 0) + sum_c dequant(W)[r][c] * x[b][c]
  * Replaces multiplyRowMajorMatrix (Sources/RealModelInference/RealModelInferenceEngine.swift:6674-6718).
- * x: fp16 bit patterns [batch][cols]; y, residual: fp32 [batch][rows]; host pointers. */
+ * x: fp16 bit patterns [batch][cols]; y, residual: fp32 [batch][rows]; host pointers.
+ * batch 1 and 2 run the wave-per-row-pair GEMV; batch > 2 (prompt blocks, batched verify; any count) runs
+ * the dequant-fused MFMA kernel, which rounds each dequantised weight to fp16 once (the GEMV does not). */
 int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y, const float *residual);
 /* Times the GEMV kernel alone on buffers already resident in HBM: `warmup` untimed launches, then
  * `iters` launches bracketed by HIP events on the library stream.  Reports the mean and the best
@@ -179,6 +181,11 @@ int esp_llama_continue_greedy(ESPLlamaRuntime *runtime, int sequence, int steps,
  * synchronises once at the end; 0 switches it to one kernel launch at a time with a host read of
  * every token (same results).  Default: enabled. */
 int esp_llama_set_graph_replay(ESPLlamaRuntime *runtime, int enabled);
+/* Prompts of 32 tokens or more are prefilled in blocks of up to 256 rows with every projection as one
+ * dequant-fused MFMA GEMM (fp16 weights after dequantisation, fp32 accumulation), instead of the
+ * reference's token-by-token walk (RealModelInferenceEngine.swift:6365-6375).  enabled = 0 restores the
+ * per-token path, whose arithmetic keeps the dequantised weights in fp32.  Default: enabled. */
+int esp_llama_set_matrix_prefill(ESPLlamaRuntime *runtime, int enabled);
 
 /* Per-kernel timing with HIP events on the library stream.  While enabled every launch of the GEMV
  * and attention kernels of a step is bracketed by an event pair; esp_llama_kernel_times synchronises

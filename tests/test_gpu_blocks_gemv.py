@@ -129,3 +129,32 @@ def test_gemv_argument_errors(ops):
         ops.Matrix(orc.FMT_Q4_K, np.zeros(144, np.uint8), 1, 100)                 # ragged cols
     with pytest.raises(ValueError):
         ops.Matrix(7, np.zeros(4 * 64, np.uint8), 1, 64)                          # unknown format
+
+
+@pytest.mark.parametrize("name,rows,cols", [
+    ("q4_k", 1024, 4096), ("q4_k", 200, 1024), ("q4_k", 256, 14336), ("q8_0", 768, 768), ("q8_0", 1003, 2048),
+    ("q4_0", 515, 256), ("q4_0", 1024, 4096), ("f16", 333, 2048),
+])
+@pytest.mark.parametrize("batch", [3, 8, 32, 33, 64, 100, 130])
+def test_mfma_gemm_matches_oracle(ops, name, rows, cols, batch):
+    """More than two activation rows run the dequant-fused MFMA kernel: fp16 weights (one rounding of the
+    dequantised value), fp32 accumulation; compared per row with the oracle's fp32 matvec."""
+    fmt = FORMATS[name][0]
+    blocks, deq = _quantized(fmt, rows, cols, seed=rows + 3 * cols)
+    rng = np.random.default_rng(batch * 1000 + rows)
+    x = rng.normal(0, 1, (batch, cols)).astype(np.float16)
+    mat = ops.Matrix(fmt, blocks, rows, cols)
+    y = mat.gemv(x)
+    check = [0, 1, batch // 2, batch - 2, batch - 1]
+    want = np.stack([orc.matvec(deq, x[b].astype(np.float32)) for b in check])
+    # each weight carries one fp16 rounding (2^-11 relative): random-sign errors over cols terms
+    tol = 2.0 ** -11 * np.abs(deq).max() * 4.0 * np.sqrt(cols) + 1e-5
+    assert np.abs(y[check] - want).max() <= tol, (np.abs(y[check] - want).max(), tol)
+    # every format feeds the matrix cores fp16(dequantised weight), rounded once: against those weights in
+    # float64 only fp32 summation noise remains (pins the tile indexing and the single rounding)
+    ref = x.astype(np.float64) @ deq.astype(np.float16).astype(np.float64).T
+    assert np.abs(y - ref).max() <= 2e-5 * np.abs(deq).max() * np.sqrt(cols) * 4 + 1e-6, np.abs(y - ref).max()
+    res = rng.normal(0, 1, (batch, rows)).astype(np.float32)
+    y2 = mat.gemv(x, residual=res)
+    assert np.abs(y2 - (res + y)).max() <= 1e-5 * (1 + np.abs(y).max())
+    mat.close()
