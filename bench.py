@@ -137,6 +137,12 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
                       f"context not included)"}
 
 
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# workload (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors a 256 MiB copy kernel gave);
+# the runs and the per-kernel table are in profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt.
+MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66578534}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -171,7 +177,7 @@ def main() -> None:
                    "weight_bytes_per_token": gpu["weight_bytes"],
                    "token_bytes_over_hbm_peak_tok_s": HBM_PEAK_GBPS * 1e9 / gpu["weight_bytes"]},
         "roofline": {"bound": "hbm", "kernel": f"dequant-GEMV {dominant}", "achieved": d["gbps"], "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": d["gbps"] / HBM_PEAK_GBPS, "traffic": None,
+                     "unit": "GB/s", "frac": d["gbps"] / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get((args.workload, dominant)),
                      "bytes_per_launch": d["bytes_per_launch"], "mean_launch_us": d["mean_us"], "launches_timed": d["launches"],
                      "all_gemv_gbps": gemv_bytes / gemv_us / 1e3 if gemv_us else 0.0,
                      "all_gemv_frac": gemv_bytes / gemv_us / 1e3 / HBM_PEAK_GBPS if gemv_us else 0.0,

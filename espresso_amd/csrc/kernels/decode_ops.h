@@ -45,6 +45,8 @@ struct AttentionArgs {
     float *split_scratch;
 };
 constexpr int kAttentionMaxSplits = 32;
+// Slices of the prefix the grouped-query attention kernel works on in parallel (fixed per runtime).
+int attention_split_count(int max_seq, int head_dim);
 
 hipError_t launch_embed(const void *table, bool table_is_f16, const int *tokens, int rows, int d, float *hidden, hipStream_t s);
 hipError_t launch_rmsnorm(const float *x, const float *w, float eps, int rows, int d, uint16_t *out_f16,

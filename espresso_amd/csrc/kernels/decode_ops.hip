@@ -336,16 +336,16 @@ __global__ __launch_bounds__(256) void attention_flash_kernel(AttentionArgs a) {
             for (int g = 0; g < G; g++) {
                 float d = 0.0f;
 #pragma unroll
-                for (int i = 0; i < 8; i++) d += q[g][i] * k[i];
+                for (int i = 0; i < 8; i++) d = __builtin_fmaf(q[g][i], k[i], d);
                 d = group_sum<LPT>(d);                                  // all lanes of the token
-                const float sc = valid ? d * scale : -INFINITY;
+                const float sc = valid ? __fmul_rn(d, scale) : -INFINITY;
                 const float cm = max_over_groups<LPT>(sc);              // over the chunk's tokens
                 const float m_new = fmaxf(mx[g], cm);      // finite: the chunk holds at least one visible token
                 const float alpha = expf(mx[g] - m_new);   // exp(-inf) = 0 on the first chunk
                 const float p = valid ? expf(sc - m_new) : 0.0f;
-                l[g] = l[g] * alpha + p;
+                l[g] = __builtin_fmaf(l[g], alpha, p);
 #pragma unroll
-                for (int i = 0; i < 8; i++) acc[g][i] = acc[g][i] * alpha + p * v[i];
+                for (int i = 0; i < 8; i++) acc[g][i] = __builtin_fmaf(p, v[i], __fmul_rn(acc[g][i], alpha));
                 mx[g] = m_new;
             }
         }
@@ -373,8 +373,8 @@ __global__ __launch_bounds__(256) void attention_flash_kernel(AttentionArgs a) {
             float lw = 0.0f, aw = 0.0f;
 #pragma unroll
             for (int sl = 0; sl < SLOTS; sl++) { lw += wl[w][sl][g]; aw += wacc[w][sl][g][dch]; }
-            L += lw * f;
-            A += aw * f;
+            L = __builtin_fmaf(lw, f, L);
+            A = __builtin_fmaf(aw, f, A);
         }
         if (splits == 1) {
             a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)(kvh * G + g) * HD + dch] = to_half_bits(L > 0.0f ? A / L : 0.0f);
@@ -408,8 +408,8 @@ __global__ __launch_bounds__(HD) void attention_merge_kernel(AttentionArgs a, in
 #pragma unroll
     for (int sp = 0; sp < kAttentionMaxSplits; sp++) {
         const float f = (sp < splits && pm[sp] != -INFINITY) ? expf(pm[sp] - M) : 0.0f;
-        L += pl[sp] * f;
-        A += pa[sp] * f;
+        L = __builtin_fmaf(pl[sp], f, L);
+        A = __builtin_fmaf(pa[sp], f, A);
     }
     a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)head * HD + dch] = to_half_bits(L > 0.0f ? A / L : 0.0f);
 }
@@ -420,9 +420,7 @@ hipError_t launch_attention_gqa(const AttentionArgs &a, int rows, bool kv_f16, h
     // graph stays valid as the prefix grows
     // each wavefront keeps two chunks of loads in flight: with max_seq / (2 chunks * 4 wavefronts * tokens per
     // chunk) splits, a prefix of any length up to max_seq costs every wavefront one memory round trip
-    const int tokens_per_wg = 2 * 4 * (64 / (HD / 8));
-    int splits = (a.max_seq + tokens_per_wg - 1) / tokens_per_wg;
-    splits = splits < 1 ? 1 : (splits > kAttentionMaxSplits ? kAttentionMaxSplits : splits);
+    int splits = attention_split_count(a.max_seq, HD);
     if (!a.split_scratch) splits = 1;
     dim3 grid(a.n_kv_head, rows, splits);
     if (kv_f16) hipLaunchKernelGGL((attention_flash_kernel<HD, G, true>), grid, dim3(256), 0, s, a);
@@ -562,6 +560,12 @@ hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStrea
     if (kv_f16) hipLaunchKernelGGL(qkv_post_kernel<true>, grid, dim3(threads), 0, s, a);
     else hipLaunchKernelGGL(qkv_post_kernel<false>, grid, dim3(threads), 0, s, a);
     return hipGetLastError();
+}
+
+int attention_split_count(int max_seq, int head_dim) {
+    const int tokens_per_wg = 2 * 4 * (64 / (head_dim / 8));
+    int splits = (max_seq + tokens_per_wg - 1) / tokens_per_wg;
+    return splits < 1 ? 1 : (splits > kAttentionMaxSplits ? kAttentionMaxSplits : splits);
 }
 
 hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {

@@ -1,6 +1,7 @@
 #include "llama_runtime.h"
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 
 namespace esp {
@@ -70,6 +71,8 @@ LlamaRuntime::~LlamaRuntime() {
     free_device(d_visible_); free_device(d_log_); free_device(d_log_count_);
     free_device(attn_scratch_);
     free_device(gemm_workspace_);
+    free_device(trunk_layers_);
+    free_device(trunk_sync_);
     free_device(argmax_scratch_.part_value); free_device(argmax_scratch_.part_index);
     for (hipGraphExec_t g : step_graphs_) if (g) (void)hipGraphExecDestroy(g);
     for (TimedLaunch &t : timed_) { (void)hipEventDestroy(t.start); (void)hipEventDestroy(t.stop); }
@@ -319,6 +322,21 @@ int LlamaRuntime::finalize() {
         if ((rc = device_alloc(&attn_scratch_, R * per_row)) != ESP_OK) return rc;
     }
     if ((rc = device_alloc(&gemm_workspace_, kGemmWorkspaceFloats)) != ESP_OK) return rc;
+    {
+        bool all_q4k = true;
+        for (const Layer &L : layers_)
+            all_q4k = all_q4k && L.wqkv.format == FMT_Q4_K && L.wo.format == FMT_Q4_K && L.w13.format == FMT_Q4_K && L.w2.format == FMT_Q4_K && !L.q_norm;
+        const char *env = getenv("ESPRESSO_HIP_FUSED_TRUNK");
+        fused_trunk_ = env && env[0] == '1';   // measured slower than the separate kernels: opt-in
+        if (all_q4k && trunk_kernel_supports(d, hd, c_.head_dim, c_.n_head, c_.n_kv_head)) {
+            std::vector<TrunkLayer> table;
+            for (const Layer &L : layers_) table.push_back(TrunkLayer{L.wqkv.qs, L.wo.qs, L.w13.qs, L.w2.qs, L.rms_att, L.rms_ffn, L.k_cache, L.v_cache});
+            if ((rc = device_alloc(&trunk_layers_, table.size())) != ESP_OK) return rc;
+            ESP_HIP_TRY(hipMemcpy(trunk_layers_, table.data(), table.size() * sizeof(TrunkLayer), hipMemcpyHostToDevice));
+            if ((rc = device_alloc(&trunk_sync_, (size_t)kTrunkSyncWords)) != ESP_OK) return rc;
+            ESP_HIP_TRY(hipMemset(trunk_sync_, 0, kTrunkSyncWords * sizeof(unsigned)));
+        }
+    }
     finalized_ = true;
     return reset();
 }
@@ -370,6 +388,16 @@ int LlamaRuntime::enqueue_trunk(int M) {
     const bool kv16 = c_.kv_format == FMT_F16;
     int rc = ESP_OK;
     ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, M, d, hidden_, s));
+    if (M == 1 && fused_trunk_active() && !timing_enabled_) {
+        TrunkArgs t{};
+        t.layers = trunk_layers_; t.n_layer = c_.n_layer; t.hidden = hidden_; t.q = q_; t.ctx = ctx_; t.act = act_;
+        t.attn_scratch = attn_scratch_; t.rope_cos = rope_cos_; t.rope_sin = rope_sin_; t.pos = d_pos_; t.seq = d_seq_;
+        t.n_head = c_.n_head; t.n_kv_head = c_.n_kv_head; t.max_seq = c_.max_seq; t.kv_f16 = kv16 ? 1 : 0;
+        t.cache_seq_stride = (size_t)kd * c_.max_seq; t.norm_eps = c_.norm_eps; t.sync = trunk_sync_;
+        t.splits = attention_split_count(c_.max_seq, c_.head_dim);
+        ESP_HIP_TRY(launch_trunk_kernel(t, d, hd, s));
+        return ESP_OK;
+    }
     for (Layer &L : layers_) {
         // both RMSNorms of the layer run inside the staging of the GEMV that consumes them
         GemvParams g;
@@ -423,6 +451,32 @@ int LlamaRuntime::enqueue_trunk(int M) {
         if ((rc = time_end()) != ESP_OK) return rc;
     }
     (void)ad;
+    return ESP_OK;
+}
+
+void LlamaRuntime::set_fused_trunk(bool enabled) {
+    if (enabled == fused_trunk_) return;
+    fused_trunk_ = enabled;
+    for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }   // captured with the other path
+}
+
+// A barrier of the fused trunk kernel that timed out means its results are garbage: fail loudly and fall
+// back to the separate kernels for the rest of the runtime's life.
+int LlamaRuntime::check_fused_trunk() {
+    if (!fused_trunk_active()) return ESP_OK;
+    unsigned n = 0;
+    int rc = fused_trunk_timeouts(&n);
+    if (rc != ESP_OK) return rc;
+    if (n == 0) return ESP_OK;
+    fused_trunk_ = false;
+    for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+    return fail(ESP_ERR_LAUNCH_FAILED, "fused trunk kernel: %u barrier time-outs; its output is invalid (fused path disabled)", n);
+}
+
+int LlamaRuntime::fused_trunk_timeouts(unsigned *out) {
+    *out = 0;
+    if (!trunk_sync_) return ESP_OK;
+    ESP_HIP_TRY(trunk_kernel_timeouts(trunk_sync_, context().stream, out));
     return ESP_OK;
 }
 
@@ -548,6 +602,7 @@ int LlamaRuntime::select_greedy(int seq, uint32_t *token) {
     int t = 0;
     ESP_HIP_TRY(hipMemcpyAsync(&t, d_out_tokens_, sizeof(int), hipMemcpyDeviceToHost, context().stream));
     ESP_HIP_TRY(hipStreamSynchronize(context().stream));
+    if ((rc = check_fused_trunk()) != ESP_OK) return rc;
     *token = (uint32_t)t;
     return ESP_OK;
 }
@@ -623,6 +678,7 @@ int LlamaRuntime::continue_greedy(int seq, int steps, uint32_t *out_tokens) {
     std::vector<int> log(steps);
     ESP_HIP_TRY(hipMemcpyAsync(log.data(), d_log_, sizeof(int) * steps, hipMemcpyDeviceToHost, s));
     ESP_HIP_TRY(hipStreamSynchronize(s));
+    if ((rc = check_fused_trunk()) != ESP_OK) return rc;
     visible_[seq] += steps;
     if (out_tokens) for (int i = 0; i < steps; i++) out_tokens[i] = (uint32_t)log[i];
     return ESP_OK;

@@ -7,6 +7,7 @@
 
 #include "context.h"
 #include "kernels/decode_ops.h"
+#include "kernels/layer_kernel.h"
 
 namespace esp {
 
@@ -66,6 +67,12 @@ class LlamaRuntime {
     void set_use_graph(bool enabled) { use_graph_ = enabled; }
     // Prompts of kMatrixPrefillMinTokens or more run in blocks through the MFMA kernels (default on).
     void set_matrix_prefill(bool enabled) { matrix_prefill_ = enabled; }
+    // Batch-1 steps of an all-Q4_K model whose shape the fused trunk kernel covers run the whole layer
+    // stack as one persistent launch (default on where supported).
+    void set_fused_trunk(bool enabled);
+    bool fused_trunk_active() const { return fused_trunk_ && trunk_layers_ != nullptr; }
+    int fused_trunk_timeouts(unsigned *out);
+    int check_fused_trunk();
     int read_last_hidden(int seq, float *out);
     int read_logits(int seq, float *out);         // runs the head on the kept hidden state
 
@@ -120,6 +127,9 @@ class LlamaRuntime {
     ArgmaxScratch argmax_scratch_;
     float *attn_scratch_ = nullptr;
     bool matrix_prefill_ = true;
+    bool fused_trunk_ = true;
+    TrunkLayer *trunk_layers_ = nullptr;   // device table, set when the fused trunk kernel covers this model
+    unsigned *trunk_sync_ = nullptr;
     float *gemm_workspace_ = nullptr;
 
     struct TimedLaunch { int kernel_class; hipEvent_t start, stop; };
