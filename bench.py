@@ -143,6 +143,65 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
 MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66578534}
 
 
+# BASELINE.json configs[2]: weight-GEMV microbenchmark at the Llama-3-8B layer shapes
+MICRO_SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
+
+
+def run_microbench() -> dict:
+    """Isolated dequant-GEMV (batch 1, 2: wave-per-row-pair kernel; batch 8: MFMA kernel) for Q4_K and Q4_0, weights
+    rotated through enough copies that no launch finds them in the last-level cache."""
+    import espresso_amd.ops as ops
+    from espresso_amd import _lib
+    rows_out = []
+    for name in ("q4_k", "q4_0"):
+        fmt = _lib.FORMAT_NAMES[name]
+        for rows, cols in MICRO_SHAPES:
+            blocks = ops.synth_weights(fmt, 7 + rows + cols, 0.02, rows * cols)
+            m = ops.Matrix(fmt, blocks, rows, cols)
+            rotate = max(2, min(64, int(600e6 // m.bytes) + 1))
+            for batch in (1, 2, 8):
+                t = m.time_gemv(batch, 10, 100, rotate)
+                nbytes = m.bytes + batch * cols * 2 + batch * rows * 4
+                rows_out.append({"format": name, "rows": rows, "cols": cols, "batch": batch, "mean_us": round(t["mean_us"], 2),
+                                 "gbps": round(nbytes / t["mean_us"] / 1e3, 1), "frac_hbm_peak": round(nbytes / t["mean_us"] / 1e3 / HBM_PEAK_GBPS, 3),
+                                 "bytes": nbytes})
+            m.close()
+    return {"metric": "dequant-GEMV HBM GB/s (Llama-3-8B layer shapes)", "unit": "GB/s", "n_gpus": 1, "data": "synthetic",
+            "how": "mean of 100 back-to-back launches between two HIP events after 10 warm-up launches; weights rotate "
+                   "through copies totalling > 600 MB so every launch reads HBM",
+            "results": rows_out}
+
+
+def run_two_token(steps: int) -> dict:
+    """BASELINE.json configs[4] at batch 1: 6-layer fp16 target, 1-layer draft of the same width and vocabulary, both
+    random-init; 16-token prompt; the exact two-token loop until the context is full."""
+    import espresso_amd.llama as ll
+    import espresso_amd.synthetic as syn
+    from espresso_amd import _lib
+    tcfg = ll.MultiModelConfig(**syn.STORIES_6L)
+    dcfg = ll.MultiModelConfig(**dict(syn.STORIES_6L, n_layer=1))
+    target, _ = syn.build_runtime(tcfg, _lib.FORMAT_F16, seed=1)
+    draft, _ = syn.build_runtime(dcfg, _lib.FORMAT_F16, seed=9)
+    prompt = np.random.default_rng(1001).integers(0, tcfg.vocab, 16).astype(np.uint32)
+    n = min(steps, tcfg.max_seq - len(prompt))
+    ll.generate_two_token(target, draft, prompt, 8)          # warm-up
+    t0 = time.perf_counter()
+    tokens, stats = ll.generate_two_token(target, draft, prompt, n)
+    dt = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    plain, _ = target.generate(prompt, n)
+    dt_plain = time.perf_counter() - t0
+    return {"metric": "exact two-token decode tok/s bs1 (6L d768 fp16 target, 1L draft)", "value": len(tokens) / dt, "unit": "tok/s",
+            "n_gpus": 1, "steps": len(tokens), "data": "synthetic", "higher_is_better": True,
+            "passes": stats["passes"],
+            "accepted_future_tokens_per_pass": stats["accepted_total"] / max(stats["passes"], 1),
+            "committed_exact_tokens_per_pass": stats["committed_total"] / max(stats["passes"], 1),
+            "stream_identical_to_plain_greedy": tokens == plain[:len(tokens)],
+            "plain_greedy_tok_s_same_loop_style": len(plain) / dt_plain,
+            "note": "a random-init draft almost never agrees with a random-init target, so acceptance is ~0 and the figure "
+                    "is the cost of verification; batch 16 is not built"}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -154,11 +213,19 @@ def main() -> None:
     ap.add_argument("--no-graph", action="store_true",
                     help="launch kernels one at a time instead of replaying the captured per-token HIP graph "
                          "(for rocprofv3 kernel traces)")
+    ap.add_argument("--microbench", action="store_true", help="weight-GEMV microbenchmark (Q4_K / Q4_0, batch 1, 2, 8) instead of decode")
+    ap.add_argument("--two-token", action="store_true", help="exact two-token draft/verify decode on the 6-layer model instead of plain decode")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this path is a batch-1 decode on a single MI355X; run with --gpus 1")
     import espresso_amd.ops as ops
     ops.init()
+    if args.microbench:
+        print(json.dumps(run_microbench()))
+        return
+    if args.two_token:
+        print(json.dumps(run_two_token(args.steps or 240)))
+        return
     w = WORKLOADS[args.workload]
     steps = args.steps if args.steps is not None else w["decode"]
     gpu = run_gpu(args.workload, steps, args.warmup, graph=not args.no_graph)
@@ -185,6 +252,9 @@ def main() -> None:
                                     for k, v in kt.items()},
                      "how": "HIP events around each launch in an instrumented pass run right after the timed region"},
         "model_build_s": round(gpu["build_s"], 1), "prefill_s": round(gpu["prefill_s"], 3),
+        "prefill": {"tokens": w["prompt"], "tok_s": w["prompt"] / gpu["prefill_s"],
+                    "path": "blocks of up to 256 rows through the dequant-fused MFMA GEMM" if w["prompt"] >= 32
+                            else "token by token (prompts under 32 tokens)"},
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, gpu)
