@@ -250,7 +250,10 @@ def main() -> None:
                      "all_gemv_frac": gemv_bytes / gemv_us / 1e3 / HBM_PEAK_GBPS if gemv_us else 0.0,
                      "per_kernel": {k: {"mean_us": round(v["mean_us"], 2), "gbps": round(v["gbps"], 1), "launches": v["launches"]}
                                     for k, v in kt.items()},
-                     "how": "HIP events around each launch in an instrumented pass run right after the timed region"},
+                     "how": "HIP events around each launch in an instrumented pass run right after the timed region",
+                     "plain_read_kernel_gbps": round(ops.hbm_read_probe(1 << 30, 10), 1),
+                     "plain_read_kernel_note": "a kernel that only streams 1 GiB with 128-bit loads, same process: the ceiling "
+                                               "the memory system gives the simplest reader, to read `frac` against"},
         "model_build_s": round(gpu["build_s"], 1), "prefill_s": round(gpu["prefill_s"], 3),
         "prefill": {"tokens": w["prompt"], "tok_s": w["prompt"] / gpu["prefill_s"],
                     "path": "blocks of up to 256 rows through the dequant-fused MFMA GEMM" if w["prompt"] >= 32

@@ -206,4 +206,31 @@ int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int
     return rc;
 }
 
+int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s) {
+    if (bytes < (1u << 20) || bytes % 16 != 0 || iters <= 0 || !gb_per_s) return fail(ESP_ERR_INVALID_ARGUMENT, "hbm_read_probe: bad argument");
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    uint8_t *buf = nullptr;
+    unsigned *sink = nullptr;
+    if ((rc = device_alloc(&buf, bytes)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&sink, (size_t)4)) != ESP_OK) { (void)hipFree(buf); return rc; }
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    hipError_t e = hipMemsetAsync(buf, 1, bytes, c.stream);
+    if (e == hipSuccess) e = hipEventCreate(&t0);
+    if (e == hipSuccess) e = hipEventCreate(&t1);
+    for (int i = 0; i < 3 && e == hipSuccess; i++) e = launch_stream_read(buf, bytes, sink, c.stream);
+    if (e == hipSuccess) e = hipEventRecord(t0, c.stream);
+    for (int i = 0; i < iters && e == hipSuccess; i++) e = launch_stream_read(buf, bytes, sink, c.stream);
+    if (e == hipSuccess) e = hipEventRecord(t1, c.stream);
+    if (e == hipSuccess) e = hipEventSynchronize(t1);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+    if (e == hipSuccess && ms > 0.0f) *gb_per_s = (double)bytes * iters / (ms * 1e-3) / 1e9;
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
+    (void)hipFree(buf); (void)hipFree(sink);
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "hbm_read_probe");
+}
+
 }  // extern "C"

@@ -104,6 +104,9 @@ hipError_t launch_repack(int format, const uint8_t *blocks, int rows, int cols, 
 // DeviceMatrix -> fp32 [rows][cols] (used to check the planes carry the same bits)
 hipError_t launch_dequant_matrix(const DeviceMatrix &m, float *out, hipStream_t stream);
 
+// kernels/probe.hip — plain streaming read of `bytes` (a multiple of 16)
+hipError_t launch_stream_read(const void *src, size_t bytes, unsigned *sink, hipStream_t stream);
+
 // kernels/synth.hip — seeded N(0, std) weights quantised into GGUF-layout blocks on the GPU
 hipError_t launch_synth(int format, uint64_t seed, float std_dev, size_t elems, uint8_t *out, hipStream_t stream);
 

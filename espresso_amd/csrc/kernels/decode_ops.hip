@@ -421,6 +421,8 @@ hipError_t launch_attention_gqa(const AttentionArgs &a, int rows, bool kv_f16, h
     // each wavefront keeps two chunks of loads in flight: with max_seq / (2 chunks * 4 wavefronts * tokens per
     // chunk) splits, a prefix of any length up to max_seq costs every wavefront one memory round trip
     int splits = attention_split_count(a.max_seq, HD);
+    // blocks of prompt rows already fill the chip: fewer slices per row, down to one (no merge launch)
+    while (splits > 1 && (long)rows * a.n_kv_head * (splits / 2) >= 2048) splits /= 2;
     if (!a.split_scratch) splits = 1;
     dim3 grid(a.n_kv_head, rows, splits);
     if (kv_f16) hipLaunchKernelGGL((attention_flash_kernel<HD, G, true>), grid, dim3(256), 0, s, a);

@@ -86,6 +86,16 @@ class Matrix:
         return {"mean_us": mean.value, "best_us": best.value}
 
 
+def hbm_read_probe(nbytes: int = 1 << 30, iters: int = 10) -> float:
+    """GB/s a plain streaming-read kernel reaches over `nbytes` of HBM."""
+    L = _lib.load_library()
+    L.esp_hbm_read_probe.restype = C.c_int
+    L.esp_hbm_read_probe.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
+    out = C.c_double(0)
+    _lib.check(L.esp_hbm_read_probe(nbytes, iters, C.byref(out)))
+    return out.value
+
+
 def synth_weights(fmt: int, seed: int, std: float, elements: int) -> np.ndarray:
     """Seeded N(0, std) weights quantised on the GPU into GGUF-layout blocks (uint8 array)."""
     L = _lib.load_library()

@@ -86,6 +86,11 @@ int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y
 int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int rotate,
                   double *mean_us, double *best_us);
 
+/* Measurement aid with no counterpart in the reference: a kernel that only streams `bytes` (>= 1 MiB, a
+ * multiple of 16) from HBM with 128-bit loads, `iters` times; reports GB/s.  bench.py prints it next to the
+ * GEMV bandwidth so that fractions of the published peak can be read against what a plain reader gets. */
+int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s);
+
 /* ---- llama decoder state resident on the GPU -------------------------------------------- *
  * Replaces CPUExactLlamaRuntime (Sources/RealModelInference/RealModelInferenceEngine.swift:548-850):
  * create = init(config:weightDirURL:) :562-614, reset :616-635, prefill :637-645, advance :672-680,
