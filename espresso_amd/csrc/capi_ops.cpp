@@ -2,7 +2,11 @@
 #include <cstring>
 #include <vector>
 
+#include <cmath>
+#include <cstring>
+
 #include "context.h"
+#include "kernels/decode_ops.h"
 
 using namespace esp;
 
@@ -204,6 +208,79 @@ int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int
     if (d_y) (void)hipFree(d_y);
     if (d_ws) (void)hipFree(d_ws);
     return rc;
+}
+
+// ---- INT4 classifier ------------------------------------------------------------------------------------
+struct ESPInt4Classifier {
+    int rows = 0, cols = 0;
+    std::vector<uint8_t> h_packed;
+    std::vector<float> h_scales, h_biases;
+    uint8_t *packed = nullptr;
+    float *scales = nullptr, *biases = nullptr, *input = nullptr, *logits = nullptr;
+    int *token = nullptr;
+    esp::ArgmaxScratch scratch;
+};
+
+ESPInt4Classifier *esp_int4_classifier_create(const float *weights, int rows, int cols) {
+    if (!weights || rows <= 0 || cols <= 0) { fail(ESP_ERR_INVALID_ARGUMENT, "int4_classifier_create: bad argument"); return nullptr; }
+    if (ensure_init() != ESP_OK) return nullptr;
+    ESPInt4Classifier *h = new ESPInt4Classifier();
+    h->rows = rows; h->cols = cols;
+    const int bpr = (cols + 1) / 2;
+    h->h_packed.assign((size_t)rows * bpr, 0);
+    h->h_scales.resize(rows);
+    h->h_biases.resize(rows);
+    // TensorBufferINT4(quantizing:rows:cols:), TensorBufferINT4.swift:53-135
+    auto q4 = [](float v, float row_min, float scale) { int q = (int)roundf((v - row_min) / scale); return q < 0 ? 0 : (q > 15 ? 15 : q); };
+    for (int r = 0; r < rows; r++) {
+        const float *row = weights + (size_t)r * cols;
+        float row_min = row[0], row_max = row[0];
+        for (int c = 1; c < cols; c++) { if (row[c] < row_min) row_min = row[c]; if (row[c] > row_max) row_max = row[c]; }
+        const float range = row_max - row_min, scale = range < 1e-10f ? 1.0f : range / 15.0f;
+        h->h_scales[r] = scale;
+        h->h_biases[r] = row_min;
+        uint8_t *out = h->h_packed.data() + (size_t)r * bpr;
+        int c = 0, b = 0;
+        for (; c + 1 < cols; c += 2) out[b++] = (uint8_t)((q4(row[c], row_min, scale) << 4) | q4(row[c + 1], row_min, scale));
+        if (c < cols) out[b] = (uint8_t)(q4(row[c], row_min, scale) << 4);
+    }
+    bool ok = device_alloc(&h->packed, h->h_packed.size()) == ESP_OK && device_alloc(&h->scales, (size_t)rows) == ESP_OK &&
+              device_alloc(&h->biases, (size_t)rows) == ESP_OK && device_alloc(&h->input, (size_t)cols) == ESP_OK &&
+              device_alloc(&h->logits, (size_t)rows) == ESP_OK && device_alloc(&h->token, (size_t)1) == ESP_OK &&
+              device_alloc(&h->scratch.part_value, (size_t)kArgmaxScratchSlots) == ESP_OK &&
+              device_alloc(&h->scratch.part_index, (size_t)kArgmaxScratchSlots) == ESP_OK;
+    ok = ok && hipMemcpy(h->packed, h->h_packed.data(), h->h_packed.size(), hipMemcpyHostToDevice) == hipSuccess &&
+         hipMemcpy(h->scales, h->h_scales.data(), (size_t)rows * 4, hipMemcpyHostToDevice) == hipSuccess &&
+         hipMemcpy(h->biases, h->h_biases.data(), (size_t)rows * 4, hipMemcpyHostToDevice) == hipSuccess;
+    if (!ok) { esp_int4_classifier_free(h); fail(ESP_ERR_OUT_OF_MEMORY, "int4_classifier_create: device setup failed"); return nullptr; }
+    return h;
+}
+
+void esp_int4_classifier_free(ESPInt4Classifier *h) {
+    if (!h) return;
+    void *ptrs[] = {h->packed, h->scales, h->biases, h->input, h->logits, h->token, h->scratch.part_value, h->scratch.part_index};
+    for (void *p : ptrs) if (p) (void)hipFree(p);
+    delete h;
+}
+
+int esp_int4_classifier_export(const ESPInt4Classifier *h, uint8_t *packed, float *scales, float *biases) {
+    if (!h) return fail(ESP_ERR_INVALID_ARGUMENT, "int4_classifier_export: null handle");
+    if (packed) std::memcpy(packed, h->h_packed.data(), h->h_packed.size());
+    if (scales) std::memcpy(scales, h->h_scales.data(), h->h_scales.size() * 4);
+    if (biases) std::memcpy(biases, h->h_biases.data(), h->h_biases.size() * 4);
+    return ESP_OK;
+}
+
+int esp_int4_classifier_matvec_argmax(ESPInt4Classifier *h, const float *input, float *logits_or_null, int *index) {
+    if (!h || !input) return fail(ESP_ERR_INVALID_ARGUMENT, "int4_classifier: null pointer");
+    Context &c = context();
+    hipError_t e = hipMemcpyAsync(h->input, input, (size_t)h->cols * 4, hipMemcpyHostToDevice, c.stream);
+    if (e == hipSuccess) e = launch_int4_matvec(h->packed, h->scales, h->biases, h->input, h->rows, h->cols, h->logits, c.stream);
+    if (e == hipSuccess && index) e = launch_argmax(h->logits, 1, h->rows, h->token, nullptr, h->scratch, c.stream);
+    if (e == hipSuccess && logits_or_null) e = hipMemcpyAsync(logits_or_null, h->logits, (size_t)h->rows * 4, hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess && index) e = hipMemcpyAsync(index, h->token, sizeof(int), hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "int4_classifier");
 }
 
 int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s) {

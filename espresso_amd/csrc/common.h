@@ -104,6 +104,10 @@ hipError_t launch_repack(int format, const uint8_t *blocks, int rows, int cols, 
 // DeviceMatrix -> fp32 [rows][cols] (used to check the planes carry the same bits)
 hipError_t launch_dequant_matrix(const DeviceMatrix &m, float *out, hipStream_t stream);
 
+// kernels/int4_classifier.hip — logits of the per-row 4-bit output head (fp32 input, fp32 logits)
+hipError_t launch_int4_matvec(const uint8_t *packed, const float *scales, const float *biases, const float *input, int vocab, int dim,
+                              float *logits, hipStream_t stream);
+
 // kernels/probe.hip — plain streaming read of `bytes` (a multiple of 16)
 hipError_t launch_stream_read(const void *src, size_t bytes, unsigned *sink, hipStream_t stream);
 

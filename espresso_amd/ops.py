@@ -86,6 +86,47 @@ class Matrix:
         return {"mean_us": mean.value, "best_us": best.value}
 
 
+class Int4Classifier:
+    """INT4Classifier over TensorBufferINT4: per-row 4-bit quantisation on the host, logits and argmax on the GPU."""
+
+    def __init__(self, weights: np.ndarray):
+        w = np.ascontiguousarray(weights, dtype=np.float32)
+        self.rows, self.cols = w.shape
+        L = _lib.load_library()
+        L.esp_int4_classifier_create.restype = C.c_void_p
+        L.esp_int4_classifier_create.argtypes = [C.c_void_p, C.c_int, C.c_int]
+        L.esp_int4_classifier_free.argtypes = [C.c_void_p]
+        L.esp_int4_classifier_export.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.esp_int4_classifier_matvec_argmax.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int)]
+        self._h = L.esp_int4_classifier_create(_ptr(w), self.rows, self.cols)
+        if not self._h:
+            raise _lib.EspressoError(-1, _lib.last_error())
+
+    def export(self):
+        packed = np.empty((self.rows, (self.cols + 1) // 2), np.uint8)
+        scales, biases = np.empty(self.rows, np.float32), np.empty(self.rows, np.float32)
+        _lib.check(_lib.load_library().esp_int4_classifier_export(self._h, _ptr(packed), _ptr(scales), _ptr(biases)))
+        return packed, scales, biases
+
+    def matvec_argmax(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        logits = np.empty(self.rows, np.float32)
+        idx = C.c_int(-1)
+        _lib.check(_lib.load_library().esp_int4_classifier_matvec_argmax(self._h, _ptr(x), _ptr(logits), C.byref(idx)))
+        return logits, idx.value
+
+    def close(self):
+        if self._h:
+            _lib.load_library().esp_int4_classifier_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def hbm_read_probe(nbytes: int = 1 << 30, iters: int = 10) -> float:
     """GB/s a plain streaming-read kernel reaches over `nbytes` of HBM."""
     L = _lib.load_library()

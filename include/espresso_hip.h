@@ -86,6 +86,19 @@ int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y
 int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int rotate,
                   double *mean_us, double *best_us);
 
+/* ---- INT4 output head ---------------------------------------------------------------------------- *
+ * INT4Classifier (Sources/Espresso/INT4Classifier.swift:40-160) over TensorBufferINT4
+ * (Sources/ANETypes/TensorBufferINT4.swift:53-135).  create quantises fp32 [rows][cols] per row exactly as
+ * TensorBufferINT4(quantizing:rows:cols:) does (scale = (max-min)/15, bias = min, high nibble first) and
+ * uploads the result; export returns those bytes ((cols+1)/2 per row), scales and biases for inspection.
+ * matvec_argmax = int4Matvec (all logits, optional) and int4MatvecArgmax (lowest index wins ties) on the GPU:
+ * logit = scale * sum(nibble * x) + bias * sum(x), fp32 input. */
+typedef struct ESPInt4Classifier ESPInt4Classifier;
+ESPInt4Classifier *esp_int4_classifier_create(const float *weights_f32, int rows, int cols);
+void esp_int4_classifier_free(ESPInt4Classifier *classifier);
+int esp_int4_classifier_export(const ESPInt4Classifier *classifier, uint8_t *packed, float *scales, float *biases);
+int esp_int4_classifier_matvec_argmax(ESPInt4Classifier *classifier, const float *input, float *logits_or_null, int *index_or_null);
+
 /* Measurement aid with no counterpart in the reference: a kernel that only streams `bytes` (>= 1 MiB, a
  * multiple of 16) from HBM with 128-bit loads, `iters` times; reports GB/s.  bench.py prints it next to the
  * GEMV bandwidth so that fractions of the published peak can be read against what a plain reader gets. */

@@ -851,3 +851,70 @@ int orc_llama_generate_two_token(orc_llama_runtime *full, orc_llama_runtime *dra
     if (stats) { stats->passes = passes; stats->committed_total = committed_total; stats->accepted_total = accepted_total; }
     return generated;
 }
+
+/* ---- INT4 classifier (TensorBufferINT4.swift:53-135, INT4Classifier.swift:40-160) -------------------- */
+static int int4_q(float v, float row_min, float scale) {
+    int q = (int)roundf((v - row_min) / scale);
+    return q < 0 ? 0 : (q > 15 ? 15 : q);
+}
+
+void orc_int4_quantize(const float *src, int rows, int cols, uint8_t *packed, float *scales, float *biases) {
+    const int bpr = (cols + 1) / 2;
+    memset(packed, 0, (size_t)rows * bpr);
+    for (int r = 0; r < rows; r++) {
+        const float *row = src + (size_t)r * cols;
+        float row_min = row[0], row_max = row[0];
+        for (int c = 1; c < cols; c++) {
+            if (row[c] < row_min) row_min = row[c];
+            if (row[c] > row_max) row_max = row[c];
+        }
+        const float range = row_max - row_min;
+        const float scale = range < 1e-10f ? 1.0f : range / 15.0f;
+        scales[r] = scale;
+        biases[r] = row_min;
+        uint8_t *out = packed + (size_t)r * bpr;
+        int c = 0, b = 0;
+        while (c + 1 < cols) {
+            out[b++] = (uint8_t)((int4_q(row[c], row_min, scale) << 4) | int4_q(row[c + 1], row_min, scale));
+            c += 2;
+        }
+        if (c < cols) out[b] = (uint8_t)(int4_q(row[c], row_min, scale) << 4);
+    }
+}
+
+float orc_int4_input_sum(const float *input, int dim) {
+    float s = 0.0f;
+    for (int i = 0; i < dim; i++) s += input[i];
+    return s;
+}
+
+static float int4_row_dot(const uint8_t *row, float scale, float bias, const float *input, float input_sum, int dim) {
+    float dot = 0.0f;
+    const int pairs = dim / 2;
+    for (int i = 0; i < pairs; i++) {
+        const float hi = (float)((row[i] >> 4) & 0xF), lo = (float)(row[i] & 0xF);
+        dot += hi * input[2 * i] + lo * input[2 * i + 1];
+    }
+    if (dim & 1) dot += (float)((row[pairs] >> 4) & 0xF) * input[dim - 1];
+    return scale * dot + bias * input_sum;
+}
+
+void orc_int4_matvec(const uint8_t *packed, const float *scales, const float *biases, const float *input,
+                     int vocab, int dim, float *out) {
+    const int bpr = (dim + 1) / 2;
+    const float sum = orc_int4_input_sum(input, dim);
+    for (int r = 0; r < vocab; r++) out[r] = int4_row_dot(packed + (size_t)r * bpr, scales[r], biases[r], input, sum, dim);
+}
+
+int orc_int4_argmax(const uint8_t *packed, const float *scales, const float *biases, const float *input,
+                    int vocab, int dim) {
+    const int bpr = (dim + 1) / 2;
+    const float sum = orc_int4_input_sum(input, dim);
+    int best = 0;
+    float best_value = -3.4028234663852886e38f;
+    for (int r = 0; r < vocab; r++) {
+        const float logit = int4_row_dot(packed + (size_t)r * bpr, scales[r], biases[r], input, sum, dim);
+        if (logit > best_value) { best_value = logit; best = r; }
+    }
+    return best;
+}

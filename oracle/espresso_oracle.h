@@ -146,6 +146,20 @@ int orc_llama_generate_two_token(orc_llama_runtime *full, orc_llama_runtime *dra
                                  const uint32_t *prompt, int prompt_count, int max_tokens,
                                  uint32_t *out_tokens, orc_two_token_stats *stats);
 
+/* ---- INT4 classifier --------------------------------------------------------------------
+ * TensorBufferINT4(quantizing:rows:cols:) (Sources/ANETypes/TensorBufferINT4.swift:53-135): per-row
+ * min-max 4-bit, scale = (max - min) / 15 (1.0 when max - min < 1e-10), bias = min,
+ * q = clamp(roundf((v - min) / scale), 0, 15), two nibbles per byte with the HIGH nibble first,
+ * (cols + 1) / 2 bytes per row, trailing low nibble zero. */
+void orc_int4_quantize(const float *src, int rows, int cols, uint8_t *packed, float *scales, float *biases);
+/* INT4Classifier.rowDotProduct / int4Matvec / int4MatvecArgmax (Sources/Espresso/INT4Classifier.swift:40-160):
+ * logit = scale * sum(nibble * x) + bias * sum(x); argmax with strict '>' (lowest index wins ties). */
+float orc_int4_input_sum(const float *input, int dim);
+void orc_int4_matvec(const uint8_t *packed, const float *scales, const float *biases, const float *input,
+                     int vocab, int dim, float *out);
+int orc_int4_argmax(const uint8_t *packed, const float *scales, const float *biases, const float *input,
+                    int vocab, int dim);
+
 #ifdef __cplusplus
 }
 #endif

@@ -192,6 +192,35 @@ def partitioned_argmax(classifier, x, block_size=4000):
     return int(idx), int(pruned.value)
 
 
+# ---- INT4 classifier -----------------------------------------------------
+def int4_quantize(weights):
+    """TensorBufferINT4(quantizing:): (packed [rows][(cols+1)//2] uint8, scales [rows], biases [rows])."""
+    w = _f32(weights)
+    rows, cols = w.shape
+    packed = np.zeros((rows, (cols + 1) // 2), dtype=np.uint8)
+    scales, biases = np.empty(rows, np.float32), np.empty(rows, np.float32)
+    L = lib()
+    L.orc_int4_quantize.restype = None
+    L.orc_int4_quantize(_ptr(w), rows, cols, _ptr(packed), _ptr(scales), _ptr(biases))
+    return packed, scales, biases
+
+
+def int4_matvec(packed, scales, biases, x, dim):
+    packed, x = np.ascontiguousarray(packed, np.uint8), _f32(x)
+    out = np.empty(packed.shape[0], np.float32)
+    L = lib()
+    L.orc_int4_matvec.restype = None
+    L.orc_int4_matvec(_ptr(packed), _ptr(_f32(scales)), _ptr(_f32(biases)), _ptr(x), packed.shape[0], dim, _ptr(out))
+    return out
+
+
+def int4_argmax(packed, scales, biases, x, dim) -> int:
+    packed, x = np.ascontiguousarray(packed, np.uint8), _f32(x)
+    L = lib()
+    L.orc_int4_argmax.restype = C.c_int
+    return int(L.orc_int4_argmax(_ptr(packed), _ptr(_f32(scales)), _ptr(_f32(biases)), _ptr(x), packed.shape[0], dim))
+
+
 # ---- BLOBFILE -----------------------------------------------------------
 def blob_build(weights) -> bytes:
     w = _f32(weights).ravel()

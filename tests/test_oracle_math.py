@@ -188,3 +188,46 @@ def test_blobfile_layout_and_errors():
     assert orc.blob_parse(blob[:-2])[0] == -4                        # truncatedPayload
     bad = bytearray(blob); bad[72] = 7
     assert orc.blob_parse(bytes(bad))[0] == -5                       # invalidPayloadSize
+
+
+# ---- INT4 classifier (Tests/EspressoTests/INT4ClassifierTests.swift) ---------------------------------------
+def test_int4_argmax_matches_naive_row_73():            # :8-71
+    w = np.zeros((100, 32), np.float32)
+    for r in range(100):
+        w[r] = np.float32(r) * np.float32(0.01) + np.arange(32, dtype=np.float32) * np.float32(0.001)
+    w[73] = 10.0
+    x = np.ones(32, np.float32)
+    assert int(np.argmax(w @ x)) == 73
+    packed, scales, biases = orc.int4_quantize(w)
+    assert orc.int4_argmax(packed, scales, biases, x, 32) == 73
+    assert scales[73] == 1.0 and biases[73] == 10.0 and not packed[73].any()     # constant row: scale 1, all nibbles 0
+
+
+def test_int4_matvec_approximation_and_packing():       # :74-131
+    w = (np.arange(20 * 16, dtype=np.float32) * np.float32(0.01)).reshape(20, 16)
+    x = np.ones(16, np.float32)
+    packed, scales, biases = orc.int4_quantize(w)
+    got = orc.int4_matvec(packed, scales, biases, x, 16)
+    ref = w @ x
+    assert np.all(np.abs(got - ref) <= np.abs(ref) * 0.15 + 1.0)
+    # closed form of the packing: row r = r*0.16 + 0.01*c, so scale = 0.01 and nibble c = c: bytes (2i << 4) | (2i + 1)
+    assert np.allclose(scales, 0.01, rtol=1e-5) and np.allclose(biases, w[:, 0])
+    assert packed[0].tolist() == [((2 * i) << 4) | (2 * i + 1) for i in range(8)]
+    # dequantised weights are within half a step
+    nib = np.stack([packed >> 4, packed & 0xF], axis=2).reshape(20, 16).astype(np.float32)
+    assert np.abs(nib * scales[:, None] + biases[:, None] - w).max() <= 0.005 + 1e-5
+
+
+def test_int4_input_sum_and_odd_dimension():            # :134-173
+    assert orc.lib().orc_int4_input_sum is not None
+    w = np.full((5, 7), 0.5, np.float32)
+    w[3] = 10.0
+    packed, scales, biases = orc.int4_quantize(w)
+    assert packed.shape == (5, 4) and np.all((packed[:, 3] & 0xF) == 0)          # trailing low nibble is zero
+    assert orc.int4_argmax(packed, scales, biases, np.ones(7, np.float32), 7) == 3
+    x = np.arange(1, 8, dtype=np.float32)
+    mixed = np.random.default_rng(3).normal(0, 1, (9, 7)).astype(np.float32)
+    p2, s2, b2 = orc.int4_quantize(mixed)
+    nib = np.stack([p2 >> 4, p2 & 0xF], axis=2).reshape(9, 8)[:, :7].astype(np.float64)
+    want = (nib * s2[:, None].astype(np.float64) + b2[:, None].astype(np.float64)) @ x.astype(np.float64)
+    assert np.allclose(orc.int4_matvec(p2, s2, b2, x, 7), want, rtol=1e-5, atol=1e-5)
