@@ -239,7 +239,7 @@ ESPHandle *esp_interop_compile(const uint8_t *program, size_t program_len, const
     h->lanes = get_int("lanes", 1);
     if (!get_str("norm_eps").empty()) h->norm_eps = (float)std::atof(get_str("norm_eps").c_str());
     if (get_str("program") != "espresso.hip/1") return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: program header must be espresso.hip/1%s");
-    if (h->spatial < 1 || h->lanes < 1 || h->lanes > kMaxStepRows || h->lanes > h->spatial)
+    if (h->spatial < 1 || h->lanes < 1 || h->lanes > 16 || h->lanes > h->spatial)
         return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: spatial/lanes out of range%s");
     auto need = [&](const char *name) -> WeightBytes * { auto it = weights.find(name); return it == weights.end() || !it->second.data ? nullptr : &it->second; };
     std::vector<size_t> want_in, want_out;

@@ -115,6 +115,32 @@ int esp_llama_generate_two_token(ESPLlamaRuntime *target, ESPLlamaRuntime *draft
     return ESP_OK;
 }
 
+int esp_llama_generate_batch(ESPLlamaRuntime *target, ESPLlamaRuntime *draft_or_null, const uint32_t *const *prompts,
+                             const int *prompt_counts, int n_seq, int max_tokens, uint32_t *out_tokens, int *out_counts,
+                             ESPTwoTokenStats *two_token_stats, double *decode_ms) {
+    if (!target) return bad_handle();
+    if (!target->rt->finalized() || (draft_or_null && !draft_or_null->rt->finalized())) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+    if (!prompts || !prompt_counts || n_seq < 1 || max_tokens < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "generate_batch: bad argument");
+    std::vector<std::vector<uint32_t>> toks;
+    TwoTokenStats st;
+    int rc = draft_or_null ? generate_two_token_batch(*target->rt, *draft_or_null->rt, prompts, prompt_counts, n_seq, max_tokens, &toks, &st, decode_ms)
+                           : generate_greedy_batch(*target->rt, prompts, prompt_counts, n_seq, max_tokens, &toks, decode_ms);
+    if (rc != ESP_OK) return rc;
+    for (int s = 0; s < n_seq; s++) {
+        if (out_counts) out_counts[s] = (int)toks[s].size();
+        if (out_tokens) for (size_t i = 0; i < toks[s].size(); i++) out_tokens[(size_t)s * max_tokens + i] = toks[s][i];
+    }
+    if (two_token_stats) {
+        two_token_stats->passes = st.passes;
+        two_token_stats->committed_total = st.committed_total;
+        two_token_stats->accepted_total = st.accepted_total;
+        two_token_stats->reference_passes = 0;
+        two_token_stats->reference_committed_total = 0;
+        two_token_stats->reference_accepted_total = -1;
+    }
+    return ESP_OK;
+}
+
 int esp_llama_continue_greedy(ESPLlamaRuntime *runtime, int sequence, int steps, uint32_t *out_tokens) {
     if (!runtime) return bad_handle();
     if (!runtime->rt->finalized()) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");

@@ -158,4 +158,138 @@ int generate_two_token(LlamaRuntime &full, LlamaRuntime &draft, const uint32_t *
     return finish();
 }
 
+// ---- lock-step batches of independent sequences ---------------------------------------------------
+// Sequence s of `n_seq` uses KV cache s of both runtimes.  Greedy, no EOS handling (the batched configs
+// decode a fixed budget); every sequence produces exactly `eff` tokens.
+static int batch_budget(const LlamaRuntime &a, const LlamaRuntime *b, const int *prompt_counts, int n_seq, int max_tokens, int *eff) {
+    if (n_seq < 1 || n_seq > a.config().max_sequences || (b && n_seq > b->config().max_sequences) || 2 * n_seq > kMaxStepRows)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "batch of %d sequences does not fit the runtime", n_seq);
+    int max_seq = a.config().max_seq;
+    if (b && b->config().max_seq < max_seq) max_seq = b->config().max_seq;
+    int budget = max_tokens;
+    for (int s = 0; s < n_seq; s++) {
+        if (prompt_counts[s] <= 0) return fail(ESP_ERR_INVALID_ARGUMENT, "Prompt tokens must not be empty");
+        if (prompt_counts[s] >= max_seq) return fail(ESP_ERR_OUT_OF_RANGE, "prompt of %d tokens does not fit the context", prompt_counts[s]);
+        if (max_seq - prompt_counts[s] < budget) budget = max_seq - prompt_counts[s];
+    }
+    *eff = budget < 0 ? 0 : budget;
+    return ESP_OK;
+}
+
+int generate_greedy_batch(LlamaRuntime &rt, const uint32_t *const *prompts, const int *prompt_counts, int n_seq, int max_tokens,
+                          std::vector<std::vector<uint32_t>> *out, double *decode_ms) {
+    out->assign(n_seq, {});
+    int eff = 0, rc = batch_budget(rt, nullptr, prompt_counts, n_seq, max_tokens, &eff);
+    if (rc != ESP_OK) return rc;
+    for (int s = 0; s < n_seq; s++)
+        if ((rc = rt.prefill(s, prompts[s], prompt_counts[s])) != ESP_OK) return rc;
+    auto t0 = Clock::now();
+    if (eff > 0) {
+        std::vector<uint32_t> current(n_seq);
+        for (int s = 0; s < n_seq; s++) {
+            if ((rc = rt.select_greedy(s, &current[s])) != ESP_OK) return rc;
+            (*out)[s].push_back(current[s]);
+        }
+        for (int step = 1; step < eff; step++) {
+            StepRows rows{};
+            rows.count = n_seq;
+            for (int s = 0; s < n_seq; s++) { rows.token[s] = (int)current[s]; rows.pos[s] = rt.visible(s); rows.seq[s] = s; }
+            uint32_t next[kMaxStepRows];
+            if ((rc = rt.forward_rows(rows)) != ESP_OK) return rc;
+            if ((rc = rt.head_rows(n_seq, next)) != ESP_OK) return rc;
+            for (int s = 0; s < n_seq; s++) {
+                rt.set_visible(s, rows.pos[s] + 1);
+                current[s] = next[s];
+                (*out)[s].push_back(next[s]);
+            }
+        }
+    }
+    if (decode_ms) *decode_ms = ms_since(t0);
+    return ESP_OK;
+}
+
+// The exact two-token loop over `n_seq` sequences in lock step: one draft pass over the sequences' current
+// tokens, one target pass over (current, proposed) of every sequence (2 * n_seq rows sharing one read of the
+// weights), a second draft pass over the sequences whose proposal was right.  Per sequence the rule is the
+// single-sequence loop's: row 0 is always exact; row 1 stands iff the proposal equals the exact successor.
+int generate_two_token_batch(LlamaRuntime &full, LlamaRuntime &draft, const uint32_t *const *prompts, const int *prompt_counts,
+                             int n_seq, int max_tokens, std::vector<std::vector<uint32_t>> *out, TwoTokenStats *stats, double *decode_ms) {
+    out->assign(n_seq, {});
+    TwoTokenStats st;
+    if (draft.config().vocab != full.config().vocab)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "draft vocab %d does not match target vocab %d", draft.config().vocab, full.config().vocab);
+    int eff = 0, rc = batch_budget(full, &draft, prompt_counts, n_seq, max_tokens, &eff);
+    if (rc != ESP_OK) return rc;
+    for (int s = 0; s < n_seq; s++) {
+        if ((rc = full.prefill(s, prompts[s], prompt_counts[s])) != ESP_OK) return rc;
+        if ((rc = draft.prefill(s, prompts[s], prompt_counts[s])) != ESP_OK) return rc;
+    }
+    auto t0 = Clock::now();
+    std::vector<uint32_t> current(n_seq);
+    if (eff > 0) {
+        for (int s = 0; s < n_seq; s++) {
+            if ((rc = full.select_greedy(s, &current[s])) != ESP_OK) return rc;
+            (*out)[s].push_back(current[s]);
+        }
+    }
+    auto active = [&](int s) { return (int)(*out)[s].size() < eff; };
+    for (;;) {
+        std::vector<int> live;
+        for (int s = 0; s < n_seq; s++) if (active(s)) live.push_back(s);
+        if (live.empty()) break;
+        st.passes++;
+        // draft: consume every live sequence's current token, propose its successor
+        StepRows dr{};
+        dr.count = (int)live.size();
+        for (int i = 0; i < dr.count; i++) { const int s = live[i]; dr.token[i] = (int)current[s]; dr.pos[i] = draft.visible(s); dr.seq[i] = s; }
+        uint32_t proposed[kMaxStepRows];
+        if ((rc = draft.forward_rows(dr)) != ESP_OK) return rc;
+        if ((rc = draft.head_rows(dr.count, proposed)) != ESP_OK) return rc;
+        for (int i = 0; i < dr.count; i++) draft.set_visible(live[i], dr.pos[i] + 1);
+        // target: (current, proposed) of every live sequence; the second row only where two tokens still fit
+        StepRows vr{};
+        std::vector<int> row0(live.size()), row1(live.size(), -1);
+        for (size_t i = 0; i < live.size(); i++) {
+            const int s = live[i], pos = full.visible(s);
+            row0[i] = vr.count;
+            vr.token[vr.count] = (int)current[s]; vr.pos[vr.count] = pos; vr.seq[vr.count] = s; vr.count++;
+            if (eff - (int)(*out)[s].size() >= 2) {
+                row1[i] = vr.count;
+                vr.token[vr.count] = (int)proposed[i]; vr.pos[vr.count] = pos + 1; vr.seq[vr.count] = s; vr.count++;
+            }
+        }
+        uint32_t exact[kMaxStepRows];
+        if ((rc = full.forward_rows(vr)) != ESP_OK) return rc;
+        if ((rc = full.head_rows(vr.count, exact)) != ESP_OK) return rc;
+        StepRows ar{};   // accepted sequences: the draft consumes the proposal as well
+        for (size_t i = 0; i < live.size(); i++) {
+            const int s = live[i], pos = vr.pos[row0[i]];
+            const uint32_t e0 = exact[row0[i]];
+            (*out)[s].push_back(e0);
+            st.committed_total++;
+            const bool accepted = row1[i] >= 0 && proposed[i] == e0;
+            if (!accepted) {
+                full.set_visible(s, pos + 1);
+                if ((rc = full.keep_row(row0[i], s)) != ESP_OK) return rc;
+                current[s] = e0;
+                continue;
+            }
+            st.accepted_total++;
+            st.committed_total++;
+            full.set_visible(s, pos + 2);
+            if ((rc = full.keep_row(row1[i], s)) != ESP_OK) return rc;
+            (*out)[s].push_back(exact[row1[i]]);
+            current[s] = exact[row1[i]];
+            ar.token[ar.count] = (int)proposed[i]; ar.pos[ar.count] = draft.visible(s); ar.seq[ar.count] = s; ar.count++;
+        }
+        if (ar.count > 0) {
+            if ((rc = draft.forward_rows(ar)) != ESP_OK) return rc;
+            for (int i = 0; i < ar.count; i++) draft.set_visible(ar.seq[i], ar.pos[i] + 1);
+        }
+    }
+    if (stats) *stats = st;
+    if (decode_ms) *decode_ms = ms_since(t0);
+    return ESP_OK;
+}
+
 }  // namespace esp

@@ -33,4 +33,14 @@ int generate_two_token(LlamaRuntime &full, LlamaRuntime &draft, const uint32_t *
                        int max_tokens, bool reference_accounting, std::vector<uint32_t> *out,
                        TwoTokenStats *stats, GenerationTiming *timing);
 
+// `n_seq` independent sequences in lock step (sequence s uses KV cache s), greedy, fixed budget: every
+// sequence yields min(max_tokens, context left for the longest prompt) tokens.  Steps of more than two rows
+// run on the matrix cores.  The closest reference notion is lane/stream packing (ane_interop.h:270-289).
+int generate_greedy_batch(LlamaRuntime &rt, const uint32_t *const *prompts, const int *prompt_counts, int n_seq, int max_tokens,
+                          std::vector<std::vector<uint32_t>> *out, double *decode_ms);
+// The exact two-token loop over `n_seq` sequences: each target pass verifies (current, proposed) of every
+// sequence at once.  Every sequence's stream equals its stream from generate_greedy_batch.
+int generate_two_token_batch(LlamaRuntime &full, LlamaRuntime &draft, const uint32_t *const *prompts, const int *prompt_counts,
+                             int n_seq, int max_tokens, std::vector<std::vector<uint32_t>> *out, TwoTokenStats *stats, double *decode_ms);
+
 }  // namespace esp

@@ -6,7 +6,7 @@
 
 namespace esp {
 
-constexpr int kMaxStepRows = 16;
+constexpr int kMaxStepRows = 32;   // rows of one step: 16 sequences x (current, proposed) in a batched verify pass
 
 // The rows (tokens) of one step, passed by value so that no host-to-device copy is needed.
 struct StepRows {

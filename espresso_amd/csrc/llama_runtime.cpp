@@ -388,6 +388,8 @@ int LlamaRuntime::enqueue_trunk(int M) {
     const bool kv16 = c_.kv_format == FMT_F16;
     int rc = ESP_OK;
     ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, M, d, hidden_, s));
+    // more than two rows (batched sequences, batched verify): one pass over the weights on the matrix cores
+    if (M > 2 && matrix_prefill_ && matrix_prefill_supported()) return enqueue_layers_matrix(M);
     if (M == 1 && fused_trunk_active() && !timing_enabled_) {
         TrunkArgs t{};
         t.layers = trunk_layers_; t.n_layer = c_.n_layer; t.hidden = hidden_; t.q = q_; t.ctx = ctx_; t.act = act_;
@@ -550,6 +552,16 @@ int LlamaRuntime::prefill_block(int seq, const uint32_t *tokens, int rows, int b
     ESP_HIP_TRY(hipMemcpyAsync(d_seq_, h_seq.data(), sizeof(int) * rows, hipMemcpyHostToDevice, s));
     ESP_HIP_TRY(hipStreamSynchronize(s));   // the host vectors go out of scope
     ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, rows, d, hidden_, s));
+    (void)ad; (void)kd; (void)hd; (void)kv16;
+    return enqueue_layers_matrix(rows);
+}
+
+// The layer loop over `rows` rows whose embeddings sit in hidden_ and whose (position, sequence) sit in
+// d_pos_/d_seq_, every projection as one dequant-fused MFMA GEMM.
+int LlamaRuntime::enqueue_layers_matrix(int rows) {
+    hipStream_t s = context().stream;
+    const int d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
+    const bool kv16 = c_.kv_format == FMT_F16;
     const size_t cache_seq_stride = (size_t)kd * c_.max_seq;
     GemmParams g;
     g.rows = rows; g.workspace = gemm_workspace_; g.workspace_floats = kGemmWorkspaceFloats;
@@ -583,6 +595,15 @@ int LlamaRuntime::prefill_block(int seq, const uint32_t *tokens, int rows, int b
 
 int LlamaRuntime::run_head(const float *hidden_rows, int count) {
     hipStream_t s = context().stream;
+    if (count > 2 && matrix_prefill_ && lm_head_.format != FMT_F32 && lm_head_.cols % 64 == 0) {
+        // batched rows: final RMSNorm, then the head as one MFMA GEMM
+        ESP_HIP_TRY(launch_rmsnorm(hidden_rows, final_norm_, c_.norm_eps, count, c_.d_model, xn_, nullptr, s));
+        GemmParams m;
+        m.w = lm_head_; m.x = xn_; m.y = logits_; m.rows = count; m.workspace = gemm_workspace_; m.workspace_floats = kGemmWorkspaceFloats;
+        ESP_HIP_TRY(launch_gemm(m, s));
+        ESP_HIP_TRY(launch_argmax(logits_, count, c_.vocab, d_out_tokens_, nullptr, argmax_scratch_, s));
+        return ESP_OK;
+    }
     GemvParams g;   // final RMSNorm fused into the head GEMV's staging
     g.w = lm_head_; g.norm_x = hidden_rows; g.norm_w = final_norm_; g.norm_eps = c_.norm_eps;
     g.y = logits_; g.batch = count; g.epilogue = EPI_STORE_F32;

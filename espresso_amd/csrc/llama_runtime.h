@@ -99,6 +99,7 @@ class LlamaRuntime {
     int run_head(const float *hidden_rows, int count);
     int enqueue_trunk(int rows);
     int prefill_block(int seq, const uint32_t *tokens, int rows, int base);
+    int enqueue_layers_matrix(int rows);
     bool matrix_prefill_supported() const;
     int capture_step_graph(int seq);
     HostTensor *host_slot(int layer, int slot);

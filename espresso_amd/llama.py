@@ -134,6 +134,27 @@ def generate_two_token(target: LlamaRuntime, draft: LlamaRuntime, prompt, max_to
     return out[:n.value].tolist(), stats
 
 
+def generate_batch(target: LlamaRuntime, prompts, max_tokens: int, draft: LlamaRuntime | None = None):
+    """Lock-step greedy decode of len(prompts) sequences; with `draft`, the exact two-token loop over all of them.
+    Returns (list of token lists, stats)."""
+    L = _lib.load_library()
+    L.esp_llama_generate_batch.restype = C.c_int
+    n = len(prompts)
+    arrays = [np.ascontiguousarray(p, dtype=np.uint32) for p in prompts]
+    ptrs = (C.c_void_p * n)(*[a.ctypes.data for a in arrays])
+    counts = (C.c_int * n)(*[a.size for a in arrays])
+    out = np.zeros((n, max(max_tokens, 1)), dtype=np.uint32)
+    out_counts = (C.c_int * n)()
+    tt = _lib.TwoTokenStatsStruct()
+    ms = C.c_double(0)
+    L.esp_llama_generate_batch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                           C.c_void_p, C.POINTER(C.c_double)]
+    _lib.check(L.esp_llama_generate_batch(target._h, draft._h if draft is not None else None, ptrs, counts, n, max_tokens, _ptr(out),
+                                          out_counts, C.byref(tt), C.byref(ms)))
+    stats = {"decode_ms": ms.value, "passes": tt.passes, "committed_total": tt.committed_total, "accepted_total": tt.accepted_total}
+    return [out[s, :out_counts[s]].tolist() for s in range(n)], stats
+
+
 def load_packed_weights(rt: LlamaRuntime, packed: dict, matrix_format: int, embedding_format: int = _lib.FORMAT_F16,
                         norm_format: int = _lib.FORMAT_F16) -> None:
     """packed: {"embedding", "final_norm", "lm_head", "layers": [{"rms_att", "wq", ...}]} of raw GGUF-layout bytes."""

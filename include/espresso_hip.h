@@ -191,6 +191,16 @@ int esp_llama_generate_two_token(ESPLlamaRuntime *target, ESPLlamaRuntime *draft
                                  uint32_t *out_tokens, int *out_count, ESPGenerationStats *stats,
                                  ESPTwoTokenStats *two_token_stats);
 
+/* `n_seq` independent sequences (sequence s uses KV cache s; create the runtimes with max_sequences >= n_seq,
+ * at most 16) decoded greedily in lock step for a fixed budget; steps of more than two rows run on the matrix
+ * cores.  With a draft runtime the exact two-token loop (RealModelInferenceEngine.swift:6014-6190) runs over
+ * all sequences at once: one target pass verifies (current, proposed) of every sequence.  Each sequence's stream
+ * is the same with and without the draft.  out_tokens: [n_seq][max_tokens]; the reference's nearest notion of a
+ * batch is lane/stream packing (ane_interop.h:270-289).  two_token_stats sums over sequences. */
+int esp_llama_generate_batch(ESPLlamaRuntime *target, ESPLlamaRuntime *draft_or_null, const uint32_t *const *prompts,
+                             const int *prompt_counts, int n_seq, int max_tokens, uint32_t *out_tokens, int *out_counts,
+                             ESPTwoTokenStats *two_token_stats, double *decode_ms);
+
 /* Continues greedy decoding of `sequence` from its current state for `steps` tokens: select, then
  * advance, per token (the body of the loop at RealModelInferenceEngine.swift:6365-6413 without the
  * EOS test).  Fails with ESP_ERR_OUT_OF_RANGE if the context would overflow. */

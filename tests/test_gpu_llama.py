@@ -242,3 +242,43 @@ def test_matrix_prefill_matches_oracle_and_per_token_path(llama, fmt, count, kv_
         t = o.select_greedy()
         o.advance(t); g.advance(t)
         assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
+
+
+def _batch_pair(llama, kw, fmt, seed, n_seq, std=0.08):
+    ocfg = orc.LlamaConfig(gemv_inputs_fp16=True, **kw)
+    w = mu.random_weights(ocfg, seed, std=std, norm_jitter=0.05)
+    packed, deq = mu.pack_weights(w, fmt)
+    rt = llama.LlamaRuntime(llama.MultiModelConfig(**kw), max_sequences=n_seq)
+    llama.load_packed_weights(rt, packed, fmt)
+    return ocfg, deq, rt
+
+
+@pytest.mark.parametrize("fmt", [orc.FMT_Q8_0, orc.FMT_Q4_K])
+def test_batch16_two_token_equals_batch16_greedy(llama, fmt):
+    """BASELINE config 5 at batch 16: sixteen sequences in lock step; the verify pass carries 32 rows through the
+    MFMA path.  Every sequence's two-token stream equals its plain greedy stream from the same batched path, and
+    the plain batched stream agrees with the oracle wherever the oracle's top-2 margin is comfortable."""
+    n_seq = 16
+    full_kw, draft_kw = dict(TINY, n_layer=3, max_seq=64), dict(TINY, n_layer=1, max_seq=64)
+    ocfg, deq, target = _batch_pair(llama, full_kw, fmt, 51, n_seq)
+    _, _, draft = _batch_pair(llama, draft_kw, fmt, 52, n_seq)
+    rng = np.random.default_rng(7)
+    prompts = [rng.integers(0, 512, int(n)).tolist() for n in rng.integers(3, 12, n_seq)]
+    plain, _ = llama.generate_batch(target, prompts, 40)
+    target.reset(); draft.reset()
+    two, st = llama.generate_batch(target, prompts, 40, draft=draft)
+    assert two == plain
+    assert all(len(t) == 40 for t in plain)
+    assert st["passes"] >= 20 and st["committed_total"] == 16 * 39
+    # a draft identical to the target accepts everything: 39 tokens after the first need 20 passes
+    _, _, twin = _batch_pair(llama, full_kw, fmt, 51, n_seq)
+    target.reset()
+    two2, st2 = llama.generate_batch(target, prompts, 40, draft=twin)
+    assert two2 == plain
+    assert st2["passes"] == 20 and st2["accepted_total"] == 16 * 19
+    # against the oracle's single-sequence greedy walk
+    for s in (0, 5, 15):
+        o = mu.load_oracle(ocfg, deq)
+        want, margin = o.generate(prompts[s], 40, with_margin=True)
+        if margin > 5e-3:
+            assert plain[s] == want, (s, margin)
