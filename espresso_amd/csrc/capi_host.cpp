@@ -1,6 +1,7 @@
 // C ABI: weight files, metadata, the GGUF front door, the engine and the exact two-token harness.
 #include <cstring>
 
+#include "generation.h"
 #include "host/engine.h"
 #include "host/gguf.h"
 #include "host/harness.h"
@@ -229,6 +230,19 @@ int esp_exact_two_token_harness_generate(const ESPExactTwoTokenModel *model, ESP
     }
     if (out_pass_count) *out_pass_count = (int)trace.passMetrics.size();
     return ESP_OK;
+}
+
+int esp_sample_token(const float *logits, int count, float temperature, double unit) {
+    if (!logits || count <= 0) return fail(ESP_ERR_INVALID_ARGUMENT, "sample_token: bad argument");
+    return sample_token(logits, count, temperature, unit);
+}
+
+double esp_splitmix64_unit(uint64_t *state) {
+    if (!state) return 0.0;
+    SplitMix64 g{*state};
+    const double u = g.unit();
+    *state = g.state;
+    return u;
 }
 
 }  // extern "C"

@@ -1,5 +1,7 @@
 #include "generation.h"
 
+#include <cmath>
+
 #include <chrono>
 
 namespace esp {
@@ -156,6 +158,62 @@ int generate_two_token(LlamaRuntime &full, LlamaRuntime &draft, const uint32_t *
         if (eos >= 0 && exact[1] == (uint32_t)eos) break;
     }
     return finish();
+}
+
+int sample_token(const float *logits, int count, float temperature, double unit) {
+    if (count <= 0) return 0;
+    auto first_max = [&]() { int b = 0; for (int i = 1; i < count; i++) if (logits[b] < logits[i]) b = i; return b; };
+    if (temperature <= 0.0f) return first_max();
+    float max_logit = logits[0];
+    for (int i = 1; i < count; i++) if (logits[i] > max_logit) max_logit = logits[i];
+    std::vector<double> scaled(count);
+    double total = 0.0;
+    for (int i = 0; i < count; i++) {
+        scaled[i] = std::exp((double)((logits[i] - max_logit) / temperature));
+        total += scaled[i];
+    }
+    if (!std::isfinite(total) || total <= 0.0) return first_max();
+    double threshold = unit * total;
+    for (int i = 0; i < count; i++) {
+        threshold -= scaled[i];
+        if (threshold <= 0.0) return i;
+    }
+    return count - 1;
+}
+
+int generate_sampled(LlamaRuntime &rt, const uint32_t *prompt, int prompt_count, int max_tokens, float temperature,
+                     uint64_t seed, std::vector<uint32_t> *out, GenerationTiming *timing) {
+    out->clear();
+    const LlamaConfig &c = rt.config();
+    if (prompt_count <= 0 || !prompt) return fail(ESP_ERR_INVALID_ARGUMENT, "Prompt tokens must not be empty");
+    if (max_tokens < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "maxTokens must be >= 0");
+    if (prompt_count >= c.max_seq) return fail(ESP_ERR_OUT_OF_RANGE, "prompt of %d tokens does not fit the context", prompt_count);
+    const int eff = max_tokens < c.max_seq - prompt_count ? max_tokens : c.max_seq - prompt_count;
+    auto t_prefill = Clock::now();
+    int rc = rt.prefill(0, prompt, prompt_count);
+    if (rc != ESP_OK) return rc;
+    if (timing) timing->prefill_ms = ms_since(t_prefill);
+    auto t_start = Clock::now(), t_emit = t_start;
+    SplitMix64 rng{seed};
+    std::vector<float> logits(c.vocab);
+    int all = prompt_count;
+    while ((int)out->size() < eff && all < c.max_seq) {
+        if ((rc = rt.read_logits(0, logits.data())) != ESP_OK) return rc;
+        const uint32_t tok = (uint32_t)sample_token(logits.data(), c.vocab, temperature, rng.unit());
+        auto now = Clock::now();
+        if (timing) {
+            if (out->empty()) timing->first_token_latency_ms = std::chrono::duration<double, std::milli>(now - t_start).count();
+            timing->token_latencies_ms.push_back(std::chrono::duration<double, std::milli>(now - t_emit).count());
+        }
+        t_emit = now;
+        out->push_back(tok);
+        all++;
+        if (c.eos_token >= 0 && tok == (uint32_t)c.eos_token) break;        // appended, then stop (:6385-6388)
+        if ((int)out->size() >= eff || all >= c.max_seq) break;
+        if ((rc = rt.advance(0, tok)) != ESP_OK) return rc;
+    }
+    if (timing) timing->decode_ms = ms_since(t_start);
+    return ESP_OK;
 }
 
 // ---- lock-step batches of independent sequences ---------------------------------------------------

@@ -2,6 +2,7 @@
 // draft/verify loop.
 #pragma once
 
+#include <cstdint>
 #include <vector>
 
 #include "llama_runtime.h"
@@ -17,6 +18,26 @@ struct GenerationTiming {
 // effectiveMaxTokens = min(maxTokens, maxSeq - promptLen) (:1425-1426).
 int generate_greedy(LlamaRuntime &rt, const uint32_t *prompt, int prompt_count, int max_tokens,
                     std::vector<uint32_t> *out, GenerationTiming *timing);
+
+// sampleToken (RealModelInferenceEngine.swift:8036-8068).  `unit` in [0, 1) plays Double.random(in: 0..<total) / total.
+int sample_token(const float *logits, int count, float temperature, double unit);
+// SplitMix64 (the generator the reference's tests seed, Tests/CPUOpsTests/CPUOpsTests.swift:6-21) and the unit
+// double Swift's BinaryFloatingPoint.random(in:using:) derives from one 64-bit draw: 53 high bits * 2^-53.
+struct SplitMix64 {
+    uint64_t state;
+    uint64_t next() {
+        state += 0x9E3779B97F4A7C15ull;
+        uint64_t z = state;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+    double unit() { return (double)(next() >> 11) * (1.0 / 9007199254740992.0); }
+};
+// generate(prompt:maxTokens:temperature:) with temperature > 0 (:1405-1493 with :8070-8081): per token the full
+// logits come back from the GPU and the reference's sampling runs on the host.
+int generate_sampled(LlamaRuntime &rt, const uint32_t *prompt, int prompt_count, int max_tokens, float temperature,
+                     uint64_t seed, std::vector<uint32_t> *out, GenerationTiming *timing);
 
 struct TwoTokenStats {
     // one pass = one batched verify of [current token, proposed future token] by the full model

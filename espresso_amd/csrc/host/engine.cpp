@@ -158,7 +158,6 @@ int RealModelInferenceEngine::generate(const std::vector<TokenID> &promptTokens,
     // argument contract of generate() (:1411-1437)
     if (maxTokens < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "maxTokens must be >= 0");
     if (!std::isfinite(temperature) || temperature < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "temperature must be finite and >= 0");
-    if (temperature != 0) return fail(ESP_ERR_UNSUPPORTED, "this path decodes greedily (temperature 0)");
     if (promptTokens.empty()) return fail(ESP_ERR_INVALID_ARGUMENT, "Prompt tokens must not be empty");
     if ((int)promptTokens.size() >= config_.maxSeq)
         return fail(ESP_ERR_OUT_OF_RANGE, "Prompt of %zu tokens does not fit context %d", promptTokens.size(), config_.maxSeq);
@@ -170,7 +169,15 @@ int RealModelInferenceEngine::generate(const std::vector<TokenID> &promptTokens,
     int rc = resolveExactTwoTokenDraft(config_, weight_dir_, environment, &draftDir, &draftConfig);
     if (rc != ESP_OK) return rc;
     GenerationTiming timing;
-    if (!draftDir.empty()) {
+    if (temperature > 0) {
+        // sampling needs the full logits of every step: plain loop, never the two-token path (:8070-8081)
+        uint64_t seed = 0x5EED5EED5EEDull;
+        auto it = environment.find("ESPRESSO_HIP_SAMPLING_SEED");
+        if (it != environment.end()) seed = std::strtoull(it->second.c_str(), nullptr, 0);
+        if ((rc = generate_sampled(*runtime_, promptTokens.data(), (int)promptTokens.size(), maxTokens, temperature, seed, &out->tokens, &timing)) != ESP_OK)
+            return rc;
+        out->exactHeadBackend = "hip_gemv_logits_host_sampling";
+    } else if (!draftDir.empty()) {
         if (!draft_runtime_ || draft_dir_loaded_ != draftDir) {
             if ((rc = loadRuntime(draftConfig, draftDir, environment, &draft_runtime_)) != ESP_OK) return rc;
             draft_dir_loaded_ = draftDir;

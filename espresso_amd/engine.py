@@ -187,6 +187,25 @@ class RealModelInferenceEngine:
         return rt
 
 
+def sample_token(logits, temperature: float, unit: float) -> int:
+    x = np.ascontiguousarray(logits, dtype=np.float32)
+    L = _L()
+    L.esp_sample_token.restype = C.c_int
+    L.esp_sample_token.argtypes = [C.c_void_p, C.c_int, C.c_float, C.c_double]
+    r = L.esp_sample_token(_ptr(x), x.size, temperature, unit)
+    if r < 0:
+        raise _lib.EspressoError(r, _lib.last_error())
+    return r
+
+
+def splitmix64_units(seed: int, count: int) -> list[float]:
+    L = _L()
+    L.esp_splitmix64_unit.restype = C.c_double
+    L.esp_splitmix64_unit.argtypes = [C.POINTER(C.c_uint64)]
+    state = C.c_uint64(seed)
+    return [L.esp_splitmix64_unit(C.byref(state)) for _ in range(count)]
+
+
 # ---- exact two-token harness -----------------------------------------------------
 def promotion_plan(current, proposed, exact_next, exact_future, budget) -> dict:
     p = PromotionPlanStruct()

@@ -316,6 +316,16 @@ int esp_engine_generate(ESPEngine *engine, const uint32_t *prompt_tokens, int pr
 /* The runtime inside the engine (owned by the engine). */
 ESPLlamaRuntime *esp_engine_runtime(ESPEngine *engine);
 
+/* sampleToken (RealModelInferenceEngine.swift:8036-8068) on the host: temperature <= 0 -> first maximum; else
+ * weights exp(double((logit - max) / T)), threshold = unit * total, first index whose running remainder is <= 0.
+ * `unit` in [0, 1) stands for Double.random(in: 0..<total) / total; esp_splitmix64_unit draws it from a SplitMix64
+ * state (53 high bits * 2^-53) and advances the state.  esp_engine_generate with temperature > 0 reads the full
+ * logits back every token and samples this way, seeded by ESPRESSO_HIP_SAMPLING_SEED (default 0x5EED5EED5EED);
+ * the reference draws from the system generator, so only the distribution, not the stream, is comparable.
+ * Returns the index (>= 0) or ESP_ERR_INVALID_ARGUMENT. */
+int esp_sample_token(const float *logits, int count, float temperature, double unit);
+double esp_splitmix64_unit(uint64_t *state);
+
 /* ---- exact two-token harness ---------------------------------------------------------------------- *
  * ExactTwoTokenBranchPromotionPlan.make (Sources/Espresso/GenerationHarness.swift:149-180). */
 typedef struct ESPPromotionPlan {

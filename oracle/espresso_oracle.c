@@ -918,3 +918,35 @@ int orc_int4_argmax(const uint8_t *packed, const float *scales, const float *bia
     }
     return best;
 }
+
+/* ---- temperature sampling (RealModelInferenceEngine.swift:8036-8068) ----------------------------------- */
+static int first_max(const float *v, int n) {
+    int best = 0;
+    for (int i = 1; i < n; i++) if (v[best] < v[i]) best = i;
+    return best;
+}
+
+int orc_sample_token(const float *logits, int count, float temperature, double unit) {
+    if (count <= 0) return 0;
+    if (temperature <= 0.0f) return first_max(logits, count);
+    float max_logit = logits[0];
+    for (int i = 1; i < count; i++) if (logits[i] > max_logit) max_logit = logits[i];
+    double *scaled = (double *)malloc(sizeof(double) * (size_t)count);
+    double total = 0.0;
+    for (int i = 0; i < count; i++) {
+        scaled[i] = exp((double)((logits[i] - max_logit) / temperature));
+        total += scaled[i];
+    }
+    int out = count - 1;
+    if (!isfinite(total) || total <= 0.0) {
+        out = first_max(logits, count);
+    } else {
+        double threshold = unit * total;
+        for (int i = 0; i < count; i++) {
+            threshold -= scaled[i];
+            if (threshold <= 0.0) { out = i; break; }
+        }
+    }
+    free(scaled);
+    return out;
+}

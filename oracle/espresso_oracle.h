@@ -146,6 +146,14 @@ int orc_llama_generate_two_token(orc_llama_runtime *full, orc_llama_runtime *dra
                                  const uint32_t *prompt, int prompt_count, int max_tokens,
                                  uint32_t *out_tokens, orc_two_token_stats *stats);
 
+/* ---- temperature sampling -----------------------------------------------------------------
+ * sampleToken (RealModelInferenceEngine.swift:8036-8068): temperature <= 0 -> first maximum; otherwise
+ * weights exp(double((logit - max) / T)) (the division in float, the exponential in double), total in index
+ * order, threshold = unit * total, first index at which the running remainder drops to <= 0; a total that is
+ * not finite or not positive falls back to the first maximum.  `unit` in [0, 1) stands for Swift's
+ * Double.random(in: 0..<total) / total. */
+int orc_sample_token(const float *logits, int count, float temperature, double unit);
+
 /* ---- INT4 classifier --------------------------------------------------------------------
  * TensorBufferINT4(quantizing:rows:cols:) (Sources/ANETypes/TensorBufferINT4.swift:53-135): per-row
  * min-max 4-bit, scale = (max - min) / 15 (1.0 when max - min < 1e-10), bias = min,

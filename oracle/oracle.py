@@ -192,6 +192,14 @@ def partitioned_argmax(classifier, x, block_size=4000):
     return int(idx), int(pruned.value)
 
 
+def sample_token(logits, temperature: float, unit: float) -> int:
+    x = _f32(logits)
+    L = lib()
+    L.orc_sample_token.restype = C.c_int
+    L.orc_sample_token.argtypes = [C.c_void_p, C.c_int, C.c_float, C.c_double]
+    return int(L.orc_sample_token(_ptr(x), x.size, temperature, unit))
+
+
 # ---- INT4 classifier -----------------------------------------------------
 def int4_quantize(weights):
     """TensorBufferINT4(quantizing:): (packed [rows][(cols+1)//2] uint8, scales [rows], biases [rows])."""

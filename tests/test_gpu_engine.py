@@ -280,3 +280,33 @@ def test_harness_with_gpu_models(E, tmp_path):
         pair.append(rt)
     toks, com, acc = E.harness_generate([35], 4, target=pair[0], draft=pair[1])
     assert toks == [105, 110, 116, 32] and com == [2, 2] and acc == [1, 1]
+
+
+def test_engine_temperature_sampling_replays_on_the_oracle(E, tmp_path):
+    """generate(temperature > 0): every step reads the GPU's logits back and applies sampleToken
+    (RealModelInferenceEngine.swift:8036-8081) with SplitMix64 draws.  Replayed here: the oracle runtime is advanced with
+    the engine's tokens and must choose the same token from its own logits whenever the draw is not within the logit
+    tolerance of a bucket edge; the stream is reproducible per seed and differs between seeds."""
+    w = mu.random_weights(orc.LlamaConfig(**KW), 43, std=0.08, norm_jitter=0.05)
+    seen = write_weight_dir(str(tmp_path), KW, w)
+    e = E.RealModelInferenceEngine(gpu_cfg(KW), str(tmp_path))
+    env = {"ESPRESSO_HIP_SAMPLING_SEED": "12345"}
+    toks, res = e.generate(PROMPT, 24, temperature=0.8, environment=env)
+    assert len(toks) == 24 and res["exact_head_backend"] == "hip_gemv_logits_host_sampling"
+    assert e.generate(PROMPT, 24, temperature=0.8, environment=env)[0] == toks
+    assert e.generate(PROMPT, 24, temperature=0.8, environment={"ESPRESSO_HIP_SAMPLING_SEED": "999"})[0] != toks
+    units = E.splitmix64_units(12345, 24)
+    o = mu.load_oracle(orc.LlamaConfig(gemv_inputs_fp16=True, **KW), seen)
+    o.prefill(PROMPT)
+    agree = 0
+    for t, u in zip(toks, units):
+        lo = o.logits()
+        mine = orc.sample_token(lo, 0.8, u)
+        # the same draw a hair to either side: if all three agree the choice is insensitive to the logit tolerance
+        stable = mine == orc.sample_token(lo, 0.8, min(u + 5e-4, 0.999999)) == orc.sample_token(lo, 0.8, max(u - 5e-4, 0.0))
+        if stable:
+            assert mine == t
+            agree += 1
+        o.advance(t)
+    assert agree >= 12
+    e.close()

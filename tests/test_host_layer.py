@@ -182,3 +182,33 @@ def test_harness_argument_errors():
         eng.harness_generate([1], 0, model=m.struct)
     with pytest.raises(lib.EspressoError, match="callback"):
         eng.harness_generate([1], 2, model=m.struct)                             # the scripted queue is empty
+
+
+def test_sample_token_follows_reference_rule():
+    """sampleToken (RealModelInferenceEngine.swift:8036-8068): host code of the library and the oracle against the rule
+    restated with numpy cumulative sums."""
+    rng = np.random.default_rng(12)
+    logits = rng.normal(0, 2, 1000).astype(np.float32)
+    assert eng.sample_token(logits, 0.0, 0.3) == orc.sample_token(logits, 0.0, 0.3) == int(np.argmax(logits))
+    tie = np.array([1, 5, 5, 2], np.float32)
+    assert eng.sample_token(tie, 0.0, 0.9) == 1                                  # first maximum
+    for temperature in (0.5, 1.0, 2.0):
+        w = np.exp(((logits - logits.max()) / np.float32(temperature)).astype(np.float64))
+        cum = np.cumsum(w)
+        for unit in (0.0, 1e-12, 0.1, 0.5, 0.9, 0.999999):
+            want = int(np.searchsorted(cum, unit * cum[-1], side="left"))
+            got = eng.sample_token(logits, temperature, unit)
+            assert got == orc.sample_token(logits, temperature, unit)
+            assert abs(got - want) <= 1                                           # running subtraction vs prefix sums: last-ulp ties
+    # degenerate totals fall back to the first maximum
+    assert eng.sample_token(np.array([0, np.inf, 1], np.float32), 1.0, 0.5) == 1
+    # SplitMix64 unit doubles: in [0, 1), reproducible, first value of seed 0 known in closed form
+    u = eng.splitmix64_units(0, 4)
+    assert u == eng.splitmix64_units(0, 4) and all(0.0 <= v < 1.0 for v in u)
+    assert u[0] == (0xE220A8397B1DCDAF >> 11) * 2.0 ** -53                      # SplitMix64(0).next() = 0xE220A8397B1DCDAF
+    # empirical distribution over many draws matches softmax(logits / T)
+    small = np.array([0.0, 1.0, 2.0, -1.0], np.float32)
+    units = eng.splitmix64_units(7, 20000)
+    counts = np.bincount([eng.sample_token(small, 1.0, v) for v in units], minlength=4) / 20000
+    p = np.exp(small - small.max()); p /= p.sum()
+    assert np.abs(counts - p).max() < 0.015
