@@ -3,24 +3,25 @@
 // Replaces the seven vDSP_mmul GEMVs per layer of the reference's CPU-exact path
 // (RealModelInferenceEngine.swift:6674-6697) with kernels that read the *packed* weights once.
 //
-// Shape of the kernel
-//   * one workgroup = 4 wavefronts of 64 lanes; a wavefront owns R consecutive rows at a time;
-//   * a lane's unit of work ("item") is one aligned 128-bit load of packed weights
-//     (Q4_K/Q4_0: 32 weights, Q8_0: 16, F16: 8); consecutive lanes read consecutive 16-byte
-//     pieces of the row, so a wavefront load covers 1 KiB of contiguous HBM;
-//   * the fp16 activations are staged once per workgroup in LDS.  For the integer formats they are
-//     stored with the two middle elements of every group of four swapped, (x0,x2,x1,x3): masking a
-//     weight dword with 0x000F000F / 0x00FF00FF yields elements 0 and 2 of a group, so the matching
-//     activation pair is then one aligned LDS dword;
-//   * nibbles / bytes become exact fp16 integers with the 0x6400 exponent trick (1024 + n, then an
-//     exact packed subtract), and v_dot2_f32_f16 forms exact products accumulated in fp32;
-//   * block scales multiply the per-block partial sums, never the individual weights;
-//   * Q4_K minimums use per-16-element sums of x precomputed in LDS:  sum (d*sc*n - dmin*m) x
-//     = d*sc*sum(n x) - dmin*m*sum(x);
-//   * a wavefront butterfly reduction leaves the row sums in every lane; lane 0 applies the epilogue.
+// Shape of the kernels
+//   * one workgroup = 4 wavefronts of 64 lanes; a wavefront (or, for long Q4_K rows, a team of four) owns a pair
+//     of consecutive rows at a time - a RoPE pair or a (gate, up) pair, so the epilogues stay in registers;
+//   * a lane's unit of work ("item") is built from aligned 128-bit loads of packed weights; consecutive lanes read
+//     consecutive pieces of the row, so a wavefront load covers 1 KiB+ of contiguous HBM;
+//   * the activations are staged once per workgroup in LDS as fp16 - copied, or computed on the spot as
+//     fp16((x * inv_rms) * w) from the fp32 residual stream (fused RMSNorm).  For the integer formats they are stored
+//     with the two middle elements of every group of four swapped, (x0,x2,x1,x3): masking a weight dword with
+//     0x000F000F / 0x00FF00FF yields elements 0 and 2 of a group, so the matching activation pair is one LDS dword;
+//   * nibbles / bytes become exact fp16 values with exponent tricks (Q4_0, Q8_0: 0x6400 | n = 1024 + n, then an
+//     exact packed subtract; Q4_K: in place under 0x5400 / 0x4400 with the offset removed per sub-block through
+//     precomputed sums of x), and v_dot2_f32_f16 forms exact products accumulated in fp32;
+//   * block scales multiply the per-block partial sums, never the individual weights; Q4_K minimums use the same
+//     per-32 sums of x:  sum (d*sc*n - dmin*m) x = d*sc*sum(n x) - dmin*m*sum(x);
+//   * DPP row operations reduce a row over the wavefront; one lane applies the epilogue
+//     (store / + residual / SiLU(gate)*up -> fp16 / RoPE + KV-cache write).
 //
-// HBM traffic per launch = packed weight bytes + batch*cols*2 (x) + batch*rows*4 (y): the kernel is
-// bound by HBM bandwidth; x is re-read from L2 once per workgroup.
+// HBM traffic per launch = packed weight bytes + batch*cols*2 (x) + batch*rows*4 (y): measured 1.006x the
+// algorithmic bytes; x is re-read from L2 once per workgroup.
 #include <cstdlib>
 
 #include "../common.h"
