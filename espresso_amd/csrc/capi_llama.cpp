@@ -195,6 +195,11 @@ int esp_llama_kernel_times(ESPLlamaRuntime *runtime, double *total_us, int64_t *
     return ESP_OK;
 }
 
+int esp_llama_time_kernel(ESPLlamaRuntime *runtime, int kernel_class, int iters, double *mean_us) {
+    if (!runtime) return bad_handle();
+    return runtime->rt->time_kernel_class(kernel_class, iters, mean_us);
+}
+
 int esp_synth_weights(int format, uint64_t seed, float std_dev, size_t elements, void *out_blocks) {
     if (!out_blocks || elements == 0 || elements % 256 != 0)
         return fail(ESP_ERR_INVALID_ARGUMENT, "synth_weights: elements must be a positive multiple of 256");

@@ -124,6 +124,56 @@ int LlamaRuntime::collect_kernel_times(double total_us[K_CLASS_COUNT], long laun
     return ESP_OK;
 }
 
+// Launches the GEMV of one class for every layer in turn (the head: the same matrix), `iters` rounds, between
+// two events: back-to-back dependent launches at the real shapes over the real weights, which no cache can hold
+// across a round.  The epilogues write into the step's buffers, so sequence state is garbage afterwards.
+int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us) {
+    if (!finalized_ || iters < 1 || !mean_us) return fail(ESP_ERR_INVALID_ARGUMENT, "time_kernel_class: bad argument");
+    if (kernel_class < K_QKV || kernel_class > K_HEAD) return fail(ESP_ERR_INVALID_ARGUMENT, "time_kernel_class: class %d", kernel_class);
+    hipStream_t s = context().stream;
+    const int kd = c_.kv_dim();
+    const bool kv16 = c_.kv_format == FMT_F16;
+    auto launch = [&](const Layer *L) -> hipError_t {
+        GemvParams g;
+        g.batch = 1;
+        switch (kernel_class) {
+        case K_QKV:
+            if (L->q_norm) { g.w = L->wqkv; g.norm_x = hidden_; g.norm_w = L->rms_att; g.norm_eps = c_.norm_eps; g.y = qkv_; g.epilogue = EPI_STORE_F32; break; }
+            g.w = L->wqkv; g.norm_x = hidden_; g.norm_w = L->rms_att; g.norm_eps = c_.norm_eps; g.epilogue = EPI_QKV_ROPE;
+            g.qkv.n_head = c_.n_head; g.qkv.n_kv_head = c_.n_kv_head; g.qkv.head_dim = c_.head_dim; g.qkv.max_seq = c_.max_seq;
+            g.qkv.rope_cos = rope_cos_; g.qkv.rope_sin = rope_sin_; g.qkv.pos = d_pos_; g.qkv.seq = d_seq_;
+            g.qkv.q_out = q_; g.qkv.k_cache = L->k_cache; g.qkv.v_cache = L->v_cache;
+            g.qkv.cache_seq_stride = (size_t)kd * c_.max_seq; g.qkv.kv_f16 = kv16 ? 1 : 0;
+            break;
+        case K_WO: g.w = L->wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL; break;
+        case K_GATE_UP:
+            g.w = L->w13; g.norm_x = hidden_; g.norm_w = L->rms_ffn; g.norm_eps = c_.norm_eps; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
+            break;
+        case K_DOWN: g.w = L->w2; g.x = act_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL; break;
+        default: g.w = lm_head_; g.norm_x = hidden_; g.norm_w = final_norm_; g.norm_eps = c_.norm_eps; g.y = logits_; g.epilogue = EPI_STORE_F32; break;
+        }
+        return launch_gemv(g, s);
+    };
+    StepRows rows{};
+    rows.count = 1;
+    ESP_HIP_TRY(launch_set_rows(rows, d_tokens_, d_pos_, d_seq_, s));
+    hipEvent_t t0 = take_event(), t1 = take_event();
+    if (!t0 || !t1) return fail(ESP_ERR_OUT_OF_MEMORY, "time_kernel_class: events");
+    const int per_round = kernel_class == K_HEAD ? 1 : (int)layers_.size();
+    for (int i = 0; i < per_round; i++) ESP_HIP_TRY(launch(kernel_class == K_HEAD ? nullptr : &layers_[(size_t)i]));   // warm-up round
+    ESP_HIP_TRY(hipEventRecord(t0, s));
+    for (int r = 0; r < iters; r++)
+        for (int i = 0; i < per_round; i++) ESP_HIP_TRY(launch(kernel_class == K_HEAD ? nullptr : &layers_[(size_t)i]));
+    ESP_HIP_TRY(hipEventRecord(t1, s));
+    ESP_HIP_TRY(hipEventSynchronize(t1));
+    float ms = 0.0f;
+    ESP_HIP_TRY(hipEventElapsedTime(&ms, t0, t1));
+    event_pool_.push_back(t0);
+    event_pool_.push_back(t1);
+    *mean_us = (double)ms * 1e3 / ((double)iters * per_round);
+    return ESP_OK;
+}
+
 size_t LlamaRuntime::kernel_bytes(int kernel_class) const {
     if (!finalized_ || layers_.empty()) return 0;
     const Layer &L = layers_[0];
@@ -388,6 +438,10 @@ int LlamaRuntime::enqueue_trunk(int M) {
     const bool kv16 = c_.kv_format == FMT_F16;
     int rc = ESP_OK;
     ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, M, d, hidden_, s));
+    if (timing_enabled_) {   // an empty event pair: the overhead the pairs around real kernels carry
+        if ((rc = time_begin(K_EVENT_PAIR)) != ESP_OK) return rc;
+        if ((rc = time_end()) != ESP_OK) return rc;
+    }
     // more than two rows (batched sequences, batched verify): one pass over the weights on the matrix cores
     if (M > 2 && matrix_prefill_ && matrix_prefill_supported()) return enqueue_layers_matrix(M);
     if (M == 1 && fused_trunk_active() && !timing_enabled_) {

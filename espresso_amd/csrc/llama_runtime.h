@@ -81,10 +81,11 @@ class LlamaRuntime {
     // Per-kernel timing with HIP events on the library stream.  While enabled, every launch of the
     // kernels below is bracketed by an event pair; collect_kernel_times() synchronises and adds the
     // elapsed times to the totals.
-    enum KernelClass { K_QKV = 0, K_WO, K_GATE_UP, K_DOWN, K_HEAD, K_ATTENTION, K_CLASS_COUNT };
+    enum KernelClass { K_QKV = 0, K_WO, K_GATE_UP, K_DOWN, K_HEAD, K_ATTENTION, K_EVENT_PAIR, K_CLASS_COUNT };
     void set_kernel_timing(bool enabled) { timing_enabled_ = enabled; }
     int collect_kernel_times(double total_us[K_CLASS_COUNT], long launches[K_CLASS_COUNT], bool reset);
     size_t kernel_bytes(int kernel_class) const;   // algorithmic bytes of one batch-1 launch
+    int time_kernel_class(int kernel_class, int iters, double *mean_us);
 
   private:
     LlamaRuntime() = default;

@@ -168,7 +168,7 @@ def load_packed_weights(rt: LlamaRuntime, packed: dict, matrix_format: int, embe
     rt.finalize()
 
 
-KERNEL_CLASSES = ("qkv", "wo", "gate_up", "down", "head", "attention")
+KERNEL_CLASSES = ("qkv", "wo", "gate_up", "down", "head", "attention", "event_pair")
 
 
 def continue_greedy(rt: LlamaRuntime, steps: int, sequence: int = 0) -> list[int]:
@@ -199,6 +199,15 @@ def set_matrix_prefill(rt: LlamaRuntime, enabled: bool) -> None:
 
 def set_kernel_timing(rt: LlamaRuntime, enabled: bool) -> None:
     _lib.check(rt._L.esp_llama_set_kernel_timing(rt._h, int(enabled)))
+
+
+def time_kernel(rt: LlamaRuntime, name: str, iters: int = 8) -> float:
+    """Mean microseconds of back-to-back launches of one GEMV class over all layers (invalidates sequence state)."""
+    rt._L.esp_llama_time_kernel.restype = C.c_int
+    rt._L.esp_llama_time_kernel.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_double)]
+    out = C.c_double(0)
+    _lib.check(rt._L.esp_llama_time_kernel(rt._h, KERNEL_CLASSES.index(name), iters, C.byref(out)))
+    return out.value
 
 
 def kernel_times(rt: LlamaRuntime, reset: bool = True) -> dict:

@@ -228,17 +228,26 @@ int esp_llama_fused_trunk_status(ESPLlamaRuntime *runtime, int *active, unsigned
 /* Per-kernel timing with HIP events on the library stream.  While enabled every launch of the GEMV
  * and attention kernels of a step is bracketed by an event pair; esp_llama_kernel_times synchronises
  * and reports, per kernel class, the summed elapsed microseconds, the launch count and the
- * algorithmic bytes of one batch-1 launch (packed weights + fp16 input + fp32 output). */
+ * algorithmic bytes of one batch-1 launch (packed weights + fp16 input + fp32 output).  Class
+ * ESP_KERNEL_EVENT_PAIR brackets nothing, once per step: its mean is what an event pair itself adds to
+ * every other class's mean. */
 #define ESP_KERNEL_QKV 0
 #define ESP_KERNEL_WO 1
 #define ESP_KERNEL_GATE_UP 2
 #define ESP_KERNEL_DOWN 3
 #define ESP_KERNEL_HEAD 4
 #define ESP_KERNEL_ATTENTION 5
-#define ESP_KERNEL_CLASS_COUNT 6
+#define ESP_KERNEL_EVENT_PAIR 6
+#define ESP_KERNEL_CLASS_COUNT 7
 int esp_llama_set_kernel_timing(ESPLlamaRuntime *runtime, int enabled);
 int esp_llama_kernel_times(ESPLlamaRuntime *runtime, double *total_us, int64_t *launches, uint64_t *bytes_per_launch,
                            int reset);
+/* The GEMV of one class (ESP_KERNEL_QKV .. ESP_KERNEL_HEAD) launched for every layer in turn, `iters` rounds,
+ * between two HIP events: the mean duration of back-to-back dependent launches at the model's real shapes over
+ * its real weights (a round moves more bytes than any cache holds).  No per-launch event overhead, so the mean
+ * is directly comparable with a rocprofv3 kernel trace.  The epilogues write into live buffers: reset the
+ * runtime before decoding again. */
+int esp_llama_time_kernel(ESPLlamaRuntime *runtime, int kernel_class, int iters, double *mean_us);
 
 /* ---- seeded synthetic weights ------------------------------------------------------------- *
  * Fills `out_blocks` (host memory, esp_format_bytes(format, elements) bytes) with N(0, std_dev) draws
