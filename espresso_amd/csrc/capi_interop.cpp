@@ -331,17 +331,16 @@ bool esp_interop_eval(ESPHandle *h) {
         if (e == hipSuccess) e = launch_scatter_columns(h->y32, h->rows, h->spatial, h->lanes, out0, s);
     } else if (e == hipSuccess && h->kind == KIND_CLASSIFIER) {
         e = launch_gather_columns(in0, h->dim, h->spatial, h->lanes, nullptr, h->x32, s);
-        if (e == hipSuccess) e = launch_rmsnorm(h->x32, h->norm, h->norm_eps, h->lanes, h->dim, h->x16, nullptr, s);
-        g.w = h->classifier; g.x = h->x16; g.y = h->y32; g.epilogue = EPI_STORE_F32;
+        // RMSNorm runs inside the GEMV's staging
+        g.w = h->classifier; g.norm_x = h->x32; g.norm_w = h->norm; g.norm_eps = h->norm_eps; g.y = h->y32; g.epilogue = EPI_STORE_F32;
         if (e == hipSuccess) e = launch_gemv(g, s);
         if (e == hipSuccess) e = launch_scatter_columns(h->y32, h->vocab, h->spatial, h->lanes, out0, s);
         if (e == hipSuccess) e = launch_row_max(h->y32, h->vocab, h->spatial, h->lanes, reinterpret_cast<uint16_t *>(h->outputs[1]->device), s);
     } else if (e == hipSuccess) {
         e = launch_gather_columns(in0, h->dim, h->spatial, h->lanes, nullptr, h->x32, s);
-        if (e == hipSuccess) e = launch_rmsnorm(h->x32, h->norm, h->norm_eps, h->lanes, h->dim, h->x16, nullptr, s);
-        g.w = h->w13; g.x = h->x16; g.out_f16 = h->act16; g.epilogue = EPI_SWIGLU_F16;
+        g.w = h->w13; g.norm_x = h->x32; g.norm_w = h->norm; g.norm_eps = h->norm_eps; g.out_f16 = h->act16; g.epilogue = EPI_SWIGLU_F16;
         if (e == hipSuccess) e = launch_gemv(g, s);
-        g.w = h->w2; g.x = h->act16; g.out_f16 = nullptr; g.y = h->y32; g.residual = h->x32; g.epilogue = EPI_ADD_RESIDUAL;
+        g.w = h->w2; g.x = h->act16; g.norm_x = nullptr; g.norm_w = nullptr; g.out_f16 = nullptr; g.y = h->y32; g.residual = h->x32; g.epilogue = EPI_ADD_RESIDUAL;
         if (e == hipSuccess) e = launch_gemv(g, s);
         if (e == hipSuccess) e = launch_scatter_columns(h->y32, h->dim, h->spatial, h->lanes, out0, s);
     }

@@ -357,22 +357,24 @@ __device__ __forceinline__ void q4k_stage_x(const KernelArgs &a, int cols, int x
 // round trip (two with the fused RMSNorm: values, then nothing else - the weights ride along).
 template <int B, int IPR, bool NORM>
 __device__ __forceinline__ void q4k_stage_x_static(const KernelArgs &a, uint4 *xs4, float *xsum, float *red) {
-    static_assert(IPR % 32 == 0, "whole groups per thread");
-    constexpr int K = IPR / 32, cols = IPR * 64, XSTRIDE = IPR | 1;
+    static_assert(IPR % 4 == 0, "whole super-blocks per row");
+    constexpr int GROUPS = IPR * 8, K = (GROUPS + kThreads - 1) / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1;
     const int tid = threadIdx.x;
     if constexpr (NORM) {
         float4 v0[B][K], v1[B][K], g0[K], g1[K];
         const float4 *w4 = reinterpret_cast<const float4 *>(a.norm_w);
+        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
         for (int k = 0; k < K; k++) {
             const int g = tid + k * kThreads;
-            g0[k] = w4[2 * g];
-            g1[k] = w4[2 * g + 1];
+            const bool in = g < GROUPS;   // whole quads of lanes: GROUPS is a multiple of 32
+            g0[k] = in ? w4[2 * g] : zero;
+            g1[k] = in ? w4[2 * g + 1] : zero;
 #pragma unroll
             for (int b = 0; b < B; b++) {
                 const float4 *x4 = reinterpret_cast<const float4 *>(a.norm_x + (size_t)b * cols);
-                v0[b][k] = x4[2 * g];
-                v1[b][k] = x4[2 * g + 1];
+                v0[b][k] = in ? x4[2 * g] : zero;
+                v1[b][k] = in ? x4[2 * g + 1] : zero;
             }
         }
 #pragma unroll
@@ -383,18 +385,22 @@ __device__ __forceinline__ void q4k_stage_x_static(const KernelArgs &a, uint4 *x
             const float inv = 1.0f / sqrtf(workgroup_sum(s, red + b * kWaves) / (float)cols + a.norm_eps);
 #pragma unroll
             for (int k = 0; k < K; k++)
-                q4k_store_group(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
+                if (tid + k * kThreads < GROUPS)
+                    q4k_store_group(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
         }
     } else {
         uint4 v[B][K];
 #pragma unroll
         for (int b = 0; b < B; b++)
 #pragma unroll
-            for (int k = 0; k < K; k++) v[b][k] = reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + tid + k * kThreads];
+            for (int k = 0; k < K; k++)
+                v[b][k] = tid + k * kThreads < GROUPS ? reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + tid + k * kThreads]
+                                                       : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int b = 0; b < B; b++)
 #pragma unroll
-            for (int k = 0; k < K; k++) q4k_store_group(v[b][k], b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
+            for (int k = 0; k < K; k++)
+                if (tid + k * kThreads < GROUPS) q4k_store_group(v[b][k], b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
     }
 }
 
@@ -621,10 +627,19 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// Column counts with a compile-time instantiation of the persistent kernel (items per row, wavefronts per
+// row pair): the model widths and FFN sizes of the llama family (2048, 4096, 8192; 11008, 14336).
 template <int B>
 hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
-    if (a.cols == 4096) return a.norm_x ? launch_q4k_persistent<B, 64, 1, true>(a, stream) : launch_q4k_persistent<B, 64, 1, false>(a, stream);
-    if (a.cols == 14336 && !a.norm_x) return launch_q4k_persistent<B, 224, 4, false>(a, stream);
+    const bool norm = a.norm_x != nullptr;
+    switch (a.cols) {
+    case 2048: return norm ? launch_q4k_persistent<B, 32, 1, true>(a, stream) : launch_q4k_persistent<B, 32, 1, false>(a, stream);
+    case 4096: return norm ? launch_q4k_persistent<B, 64, 1, true>(a, stream) : launch_q4k_persistent<B, 64, 1, false>(a, stream);
+    case 8192: return norm ? launch_q4k_persistent<B, 128, 2, true>(a, stream) : launch_q4k_persistent<B, 128, 2, false>(a, stream);
+    case 11008: if (!norm) return launch_q4k_persistent<B, 172, 4, false>(a, stream); break;
+    case 14336: if (!norm) return launch_q4k_persistent<B, 224, 4, false>(a, stream); break;
+    default: break;
+    }
     const size_t lds = (size_t)B * 8 * ((a.cols / 64) | 1) * 16 + (size_t)B * (a.cols / 32) * 4 + (size_t)B * kWaves * 4;
     auto kernel = gemv_q4k_generic_kernel<B>;
     static size_t configured_lds = 0;

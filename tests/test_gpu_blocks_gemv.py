@@ -79,6 +79,7 @@ def _quantized(fmt, rows, cols, seed):
 @pytest.mark.parametrize("name,rows,cols", [
     ("q8_0", 768, 768), ("q8_0", 2048, 768), ("q8_0", 768, 2048), ("q8_0", 1003, 96),
     ("q4_0", 1024, 4096), ("q4_0", 515, 256), ("q4_k", 1024, 4096), ("q4_k", 257, 1024), ("q4_k", 64, 14336),
+    ("q4_k", 515, 2048), ("q4_k", 300, 8192), ("q4_k", 131, 11008), ("q4_k", 6000, 4096),
     ("f16", 768, 768), ("f16", 333, 2048), ("f32", 301, 512),
 ])
 @pytest.mark.parametrize("batch", [1, 2])

@@ -89,7 +89,7 @@ def test_rmsnorm_classifier_kernel_matches_oracle(io):
     k.free()
 
 
-@pytest.mark.parametrize("name,dim,hidden", [("q8_0", 768, 2048), ("q4_k", 512, 1024)])
+@pytest.mark.parametrize("name,dim,hidden", [("q8_0", 768, 2048), ("q4_k", 512, 1024), ("q4_k", 2048, 8192), ("q4_k", 4096, 11008)])
 def test_decode_ffn_kernel_matches_oracle(io, name, dim, hidden):
     spatial, lanes = 32, 2
     rng = np.random.default_rng(dim)
@@ -110,7 +110,8 @@ def test_decode_ffn_kernel_matches_oracle(io, name, dim, hidden):
         g, u = orc.matvec(w1, n), orc.matvec(w3, n)
         act = _f16(np.array([orc.silu_tanh(float(v)) for v in g], dtype=np.float32) * u)
         want = xl + orc.matvec(w2, act)
-        _fp16_close(got[:, lane], want, extra=1e-3)
+        # the fp16 rounding of the hidden activations adds noise that grows with the number of terms of the down projection
+        _fp16_close(got[:, lane], want, extra=1e-3 * max(1.0, hidden / 2048))
     k.free()
 
 
