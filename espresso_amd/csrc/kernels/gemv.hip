@@ -356,53 +356,69 @@ __device__ __forceinline__ void q4k_stage_x(const KernelArgs &a, int cols, int x
 // cols = 64 * IPR: every load of the row is issued before the first use, so staging costs one memory
 // round trip (two with the fused RMSNorm: values, then nothing else - the weights ride along).
 template <int B, int IPR, bool NORM>
-__device__ __forceinline__ void q4k_stage_x_static(const KernelArgs &a, uint4 *xs4, float *xsum, float *red) {
+struct Q4KStage {
     static_assert(IPR % 4 == 0, "whole super-blocks per row");
-    constexpr int GROUPS = IPR * 8, K = (GROUPS + kThreads - 1) / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1;
-    const int tid = threadIdx.x;
-    if constexpr (NORM) {
-        float4 v0[B][K], v1[B][K], g0[K], g1[K];
-        const float4 *w4 = reinterpret_cast<const float4 *>(a.norm_w);
-        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    static constexpr int GROUPS = IPR * 8, K = (GROUPS + kThreads - 1) / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1;
+    // every thread holds K groups: no guards, so all loads issue at once (guarded loads become
+    // branches, and each branch waits for its own round trip to the L2)
+    static constexpr bool FULL = GROUPS % kThreads == 0;
+    float4 v0[NORM ? B : 1][K], v1[NORM ? B : 1][K], g0[K], g1[K];   // NORM: fp32 values and norm weights
+    uint4 v[NORM ? 1 : B][K];                                        // otherwise: fp16 values
+
+    // Issues the loads.  Called before the first weight loads: memory returns in order, so the
+    // activations (L2 hits) must not queue behind weight lines that come from HBM.
+    __device__ __forceinline__ void issue(const KernelArgs &a) {
+        const int tid = threadIdx.x;
+        if constexpr (NORM) {
+            const float4 *w4 = reinterpret_cast<const float4 *>(a.norm_w);
+            const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int k = 0; k < K; k++) {
-            const int g = tid + k * kThreads;
-            const bool in = g < GROUPS;   // whole quads of lanes: GROUPS is a multiple of 32
-            g0[k] = in ? w4[2 * g] : zero;
-            g1[k] = in ? w4[2 * g + 1] : zero;
+            for (int k = 0; k < K; k++) {
+                const int g = tid + k * kThreads;
+                const bool in = FULL || g < GROUPS;   // whole quads of lanes: GROUPS is a multiple of 32
+                g0[k] = in ? w4[2 * g] : zero;
+                g1[k] = in ? w4[2 * g + 1] : zero;
+#pragma unroll
+                for (int b = 0; b < B; b++) {
+                    const float4 *x4 = reinterpret_cast<const float4 *>(a.norm_x + (size_t)b * cols);
+                    v0[b][k] = in ? x4[2 * g] : zero;
+                    v1[b][k] = in ? x4[2 * g + 1] : zero;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < B; b++)
+#pragma unroll
+                for (int k = 0; k < K; k++)
+                    v[b][k] = FULL || tid + k * kThreads < GROUPS ? reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + tid + k * kThreads]
+                                                                   : make_uint4(0, 0, 0, 0);
+        }
+    }
+
+    // Normalises (NORM) and writes the fp16 groups and their sums to LDS; the caller's barrier follows.
+    __device__ __forceinline__ void finish(const KernelArgs &a, uint4 *xs4, float *xsum, float *red) {
+        const int tid = threadIdx.x;
+        if constexpr (NORM) {
 #pragma unroll
             for (int b = 0; b < B; b++) {
-                const float4 *x4 = reinterpret_cast<const float4 *>(a.norm_x + (size_t)b * cols);
-                v0[b][k] = in ? x4[2 * g] : zero;
-                v1[b][k] = in ? x4[2 * g + 1] : zero;
+                float s = 0.0f;
+#pragma unroll
+                for (int k = 0; k < K; k++) s += sum_squares(v0[b][k], v1[b][k]);
+                const float inv = 1.0f / sqrtf(workgroup_sum(s, red + b * kWaves) / (float)cols + a.norm_eps);
+#pragma unroll
+                for (int k = 0; k < K; k++)
+                    if (FULL || tid + k * kThreads < GROUPS)
+                        q4k_store_group(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
             }
+        } else {
+#pragma unroll
+            for (int b = 0; b < B; b++)
+#pragma unroll
+                for (int k = 0; k < K; k++)
+                    if (FULL || tid + k * kThreads < GROUPS) q4k_store_group(v[b][k], b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
         }
-#pragma unroll
-        for (int b = 0; b < B; b++) {
-            float s = 0.0f;
-#pragma unroll
-            for (int k = 0; k < K; k++) s += sum_squares(v0[b][k], v1[b][k]);
-            const float inv = 1.0f / sqrtf(workgroup_sum(s, red + b * kWaves) / (float)cols + a.norm_eps);
-#pragma unroll
-            for (int k = 0; k < K; k++)
-                if (tid + k * kThreads < GROUPS)
-                    q4k_store_group(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
-        }
-    } else {
-        uint4 v[B][K];
-#pragma unroll
-        for (int b = 0; b < B; b++)
-#pragma unroll
-            for (int k = 0; k < K; k++)
-                v[b][k] = tid + k * kThreads < GROUPS ? reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + tid + k * kThreads]
-                                                       : make_uint4(0, 0, 0, 0);
-#pragma unroll
-        for (int b = 0; b < B; b++)
-#pragma unroll
-            for (int k = 0; k < K; k++)
-                if (tid + k * kThreads < GROUPS) q4k_store_group(v[b][k], b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
     }
-}
+};
 
 // Persistent kernel for cols = 64 * IPR.  TEAM wavefronts share one row pair at a time (TEAM = 1: a
 // wavefront streams whole pairs on its own; TEAM = 4: the workgroup splits a long row pair and adds
@@ -494,9 +510,11 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int it
     };
 
     Q4KItem buf0[PASSES], buf1[PASSES];
+    Q4KStage<B, IPR, NORM> stage;
     int pair = blockIdx.x * TEAMS + wave / TEAM;
+    stage.issue(a);
     if (pair < npairs) load_pair(pair, buf0);
-    q4k_stage_x_static<B, IPR, NORM>(a, xs4, xsum, norm_red);
+    stage.finish(a, xs4, xsum, norm_red);
     __syncthreads();
     for (int j = 0; j < iters; j += 2) {
         int next = pair + n_teams;
