@@ -359,8 +359,8 @@ template <int B, int IPR, bool NORM>
 struct Q4KStage {
     static_assert(IPR % 4 == 0, "whole super-blocks per row");
     static constexpr int GROUPS = IPR * 8, K = (GROUPS + kThreads - 1) / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1;
-    // every thread holds K groups: no guards, so all loads issue at once (guarded loads become
-    // branches, and each branch waits for its own round trip to the L2)
+    // Threads past the last group load group 0 and drop it: a guarded load becomes a branch, and
+    // each branch waits for its own round trip to the L2, while clamped loads all issue at once.
     static constexpr bool FULL = GROUPS % kThreads == 0;
     float4 v0[NORM ? B : 1][K], v1[NORM ? B : 1][K], g0[K], g1[K];   // NORM: fp32 values and norm weights
     uint4 v[NORM ? 1 : B][K];                                        // otherwise: fp16 values
@@ -374,15 +374,16 @@ struct Q4KStage {
             const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
             for (int k = 0; k < K; k++) {
-                const int g = tid + k * kThreads;
-                const bool in = FULL || g < GROUPS;   // whole quads of lanes: GROUPS is a multiple of 32
-                g0[k] = in ? w4[2 * g] : zero;
-                g1[k] = in ? w4[2 * g + 1] : zero;
+                const bool in = FULL || tid + k * kThreads < GROUPS;   // whole quads of lanes: GROUPS is a multiple of 32
+                const int g = in ? tid + k * kThreads : 0;
+                g0[k] = w4[2 * g];
+                g1[k] = w4[2 * g + 1];
 #pragma unroll
                 for (int b = 0; b < B; b++) {
                     const float4 *x4 = reinterpret_cast<const float4 *>(a.norm_x + (size_t)b * cols);
-                    v0[b][k] = in ? x4[2 * g] : zero;
-                    v1[b][k] = in ? x4[2 * g + 1] : zero;
+                    v0[b][k] = x4[2 * g];
+                    v1[b][k] = x4[2 * g + 1];
+                    if (!in) v0[b][k] = v1[b][k] = zero;   // no part in the sum of squares
                 }
             }
         } else {
@@ -390,8 +391,7 @@ struct Q4KStage {
             for (int b = 0; b < B; b++)
 #pragma unroll
                 for (int k = 0; k < K; k++)
-                    v[b][k] = FULL || tid + k * kThreads < GROUPS ? reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + tid + k * kThreads]
-                                                                   : make_uint4(0, 0, 0, 0);
+                    v[b][k] = reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + (FULL || tid + k * kThreads < GROUPS ? tid + k * kThreads : 0)];
         }
     }
 
