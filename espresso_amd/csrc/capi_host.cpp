@@ -1,10 +1,12 @@
 // C ABI: weight files, metadata, the GGUF front door, the engine and the exact two-token harness.
+#include <algorithm>
 #include <cstring>
 
 #include "generation.h"
 #include "host/engine.h"
 #include "host/gguf.h"
 #include "host/harness.h"
+#include "host/tokenizer.h"
 
 using namespace esp;
 
@@ -146,6 +148,20 @@ int esp_gguf_prepare(const char *gguf_path, const char *output_dir, const ESPPre
     return ESP_OK;
 }
 
+namespace {
+void fill_result(const GenerationResult &r, ESPGenerationResult *result) {
+    std::memset(result, 0, sizeof(*result));
+    result->token_count = (int32_t)r.tokens.size();
+    result->tokens_per_second = r.tokensPerSecond;
+    result->compile_time_ms = r.compileTimeMs;
+    result->first_token_latency_ms = r.firstTokenLatencyMs;
+    result->has_two_token_stats = r.hasTwoTokenStats ? 1 : 0;
+    result->committed_exact_tokens_per_pass = r.committedExactTokensPerPass;
+    result->accepted_future_tokens_per_pass = r.acceptedFutureTokensPerPass;
+    std::strncpy(result->exact_head_backend, r.exactHeadBackend.c_str(), sizeof(result->exact_head_backend) - 1);
+}
+}  // namespace
+
 ESPEngine *esp_engine_build(const ESPModelConfig *config, const char *weight_dir, const char *tokenizer_dir,
                             const char *const *env_keys, const char *const *env_values, int env_count) {
     if (!config || !weight_dir) { fail(ESP_ERR_INVALID_ARGUMENT, "null config or weight directory"); return nullptr; }
@@ -173,18 +189,110 @@ int esp_engine_generate(ESPEngine *engine, const uint32_t *prompt_tokens, int pr
     int rc = engine->engine->generate(prompt, max_tokens, temperature, env_from(env_keys, env_values, env_count), &r);
     if (rc != ESP_OK) return rc;
     if (out_tokens) for (size_t i = 0; i < r.tokens.size(); i++) out_tokens[i] = r.tokens[i];
-    if (result) {
-        std::memset(result, 0, sizeof(*result));
-        result->token_count = (int32_t)r.tokens.size();
-        result->tokens_per_second = r.tokensPerSecond;
-        result->compile_time_ms = r.compileTimeMs;
-        result->first_token_latency_ms = r.firstTokenLatencyMs;
-        result->has_two_token_stats = r.hasTwoTokenStats ? 1 : 0;
-        result->committed_exact_tokens_per_pass = r.committedExactTokensPerPass;
-        result->accepted_future_tokens_per_pass = r.acceptedFutureTokensPerPass;
-        std::strncpy(result->exact_head_backend, r.exactHeadBackend.c_str(), sizeof(result->exact_head_backend) - 1);
-    }
+    if (result) fill_result(r, result);
     return ESP_OK;
+}
+
+int esp_engine_generate_text(ESPEngine *engine, const char *prompt_utf8, size_t prompt_bytes, int max_tokens, float temperature,
+                             const char *const *env_keys, const char *const *env_values, int env_count, uint32_t *out_tokens,
+                             char *out_text, size_t text_capacity, size_t *out_text_bytes, ESPGenerationResult *result) {
+    if (!engine || (!prompt_utf8 && prompt_bytes)) return fail(ESP_ERR_INVALID_ARGUMENT, "null engine or prompt");
+    GenerationResult r;
+    int rc = engine->engine->generateText(std::string(prompt_utf8 ? prompt_utf8 : "", prompt_bytes), max_tokens, temperature,
+                                          env_from(env_keys, env_values, env_count), &r);
+    if (rc != ESP_OK) return rc;
+    if (out_tokens) for (size_t i = 0; i < r.tokens.size(); i++) out_tokens[i] = r.tokens[i];
+    if (out_text_bytes) *out_text_bytes = r.text.size();
+    if (out_text && text_capacity) std::memcpy(out_text, r.text.data(), std::min(text_capacity, r.text.size()));
+    if (result) fill_result(r, result);
+    return ESP_OK;
+}
+
+// ---- tokenizers ----------------------------------------------------------------------------------------
+struct ESPTokenizer { std::unique_ptr<Tokenizer> impl; };
+
+namespace {
+thread_local ESPTokenizerError g_tokenizer_error = {};
+
+ESPTokenizer *finish_tokenizer(const TokenizerStatus &st, std::unique_ptr<Tokenizer> t) {
+    g_tokenizer_error = ESPTokenizerError{};
+    g_tokenizer_error.code = (int32_t)st.error;
+    g_tokenizer_error.detail = st.detail;
+    g_tokenizer_error.detail2 = st.detail2;
+    std::strncpy(g_tokenizer_error.text, st.text.c_str(), sizeof(g_tokenizer_error.text) - 1);
+    if (!st.ok()) { fail(ESP_ERR_INVALID_ARGUMENT, "tokenizer load failed: error %d %s", (int)st.error, st.text.c_str()); return nullptr; }
+    ESPTokenizer *h = new ESPTokenizer();
+    h->impl = std::move(t);
+    return h;
+}
+}  // namespace
+
+ESPTokenizer *esp_tokenizer_load_sentencepiece(const char *model_path) {
+    if (!model_path) { fail(ESP_ERR_INVALID_ARGUMENT, "null path"); return nullptr; }
+    std::unique_ptr<SentencePieceTokenizer> t;
+    const TokenizerStatus st = SentencePieceTokenizer::load(model_path, &t);
+    return finish_tokenizer(st, std::move(t));
+}
+
+ESPTokenizer *esp_tokenizer_load_gpt2(const char *vocab_json_path, const char *merges_txt_path) {
+    if (!vocab_json_path || !merges_txt_path) { fail(ESP_ERR_INVALID_ARGUMENT, "null path"); return nullptr; }
+    std::unique_ptr<GPT2BPETokenizer> t;
+    const TokenizerStatus st = GPT2BPETokenizer::load(vocab_json_path, merges_txt_path, &t);
+    return finish_tokenizer(st, std::move(t));
+}
+
+ESPTokenizer *esp_tokenizer_load_tokenizer_json(const char *tokenizer_json_path) {
+    if (!tokenizer_json_path) { fail(ESP_ERR_INVALID_ARGUMENT, "null path"); return nullptr; }
+    std::unique_ptr<GPT2BPETokenizer> t;
+    const TokenizerStatus st = GPT2BPETokenizer::loadTokenizerJSON(tokenizer_json_path, &t);
+    return finish_tokenizer(st, std::move(t));
+}
+
+ESPTokenizer *esp_tokenizer_load_dir(const ESPModelConfig *config, const char *tokenizer_dir) {
+    if (!config || !tokenizer_dir) { fail(ESP_ERR_INVALID_ARGUMENT, "null config or directory"); return nullptr; }
+    std::unique_ptr<Tokenizer> t;
+    const TokenizerStatus st = loadTokenizer(from_c(*config), tokenizer_dir, &t);
+    return finish_tokenizer(st, std::move(t));
+}
+
+void esp_tokenizer_last_error(ESPTokenizerError *out) { if (out) *out = g_tokenizer_error; }
+void esp_tokenizer_free(ESPTokenizer *tokenizer) { delete tokenizer; }
+int esp_tokenizer_vocab_size(const ESPTokenizer *tokenizer) { return tokenizer ? tokenizer->impl->vocabSize() : 0; }
+const char *esp_tokenizer_kind(const ESPTokenizer *tokenizer) { return tokenizer ? tokenizer->impl->kind() : ""; }
+
+long esp_tokenizer_encode(const ESPTokenizer *tokenizer, const char *text_utf8, size_t text_bytes, int32_t *out_tokens, size_t capacity) {
+    if (!tokenizer || (!text_utf8 && text_bytes)) return fail(ESP_ERR_INVALID_ARGUMENT, "null tokenizer or text");
+    const std::vector<int> tokens = tokenizer->impl->encode(std::string(text_utf8 ? text_utf8 : "", text_bytes));
+    if (out_tokens) for (size_t i = 0; i < tokens.size() && i < capacity; i++) out_tokens[i] = tokens[i];
+    return (long)tokens.size();
+}
+
+long esp_pretokenize(const char *pattern_utf8, const char *text_utf8, size_t text_bytes, int64_t *out_ranges, size_t capacity_pairs) {
+    if (!text_utf8 && text_bytes) return fail(ESP_ERR_INVALID_ARGUMENT, "null text");
+    Regex re;
+    std::string err;
+    if (!re.compile(pattern_utf8 ? pattern_utf8 : GPT2BPETokenizer::defaultPreTokenizerPattern(), &err))
+        return fail(ESP_ERR_INVALID_ARGUMENT, "invalid pre-tokenizer pattern: %s", err.c_str());
+    const std::vector<uint32_t> cps = utf8_to_code_points(std::string(text_utf8 ? text_utf8 : "", text_bytes));
+    std::vector<size_t> byte_offset(cps.size() + 1, 0);   // of the re-encoded text, equal to the input's when that is valid UTF-8
+    for (size_t i = 0; i < cps.size(); i++) {
+        std::string one;
+        append_utf8(cps[i], &one);
+        byte_offset[i + 1] = byte_offset[i] + one.size();
+    }
+    const auto ms = re.matches(cps);
+    for (size_t i = 0; i < ms.size() && i < capacity_pairs && out_ranges; i++) {
+        out_ranges[2 * i] = (int64_t)byte_offset[ms[i].first];
+        out_ranges[2 * i + 1] = (int64_t)byte_offset[ms[i].second];
+    }
+    return (long)ms.size();
+}
+
+long esp_tokenizer_decode(const ESPTokenizer *tokenizer, const int32_t *tokens, size_t count, char *out_utf8, size_t capacity) {
+    if (!tokenizer || (!tokens && count)) return fail(ESP_ERR_INVALID_ARGUMENT, "null tokenizer or tokens");
+    const std::string text = tokenizer->impl->decode(std::vector<int>(tokens, tokens + count));
+    if (out_utf8 && capacity) std::memcpy(out_utf8, text.data(), std::min(capacity, text.size()));
+    return (long)text.size();
 }
 
 void esp_exact_two_token_promotion_plan(uint32_t current_token, uint32_t proposed_future_token, uint32_t exact_next_token,

@@ -1,5 +1,6 @@
 #include "engine.h"
 
+#include <algorithm>
 #include <chrono>
 #include <cmath>
 
@@ -100,12 +101,19 @@ int RealModelInferenceEngine::loadRuntime(const MultiModelConfig &config, const 
     return ESP_OK;
 }
 
-int RealModelInferenceEngine::build(const MultiModelConfig &config, const std::string &weightDir, const std::string &,
+int RealModelInferenceEngine::build(const MultiModelConfig &config, const std::string &weightDir, const std::string &tokenizerDir,
                                     const Environment &environment, std::unique_ptr<RealModelInferenceEngine> *out) {
     auto t0 = std::chrono::steady_clock::now();
     std::unique_ptr<RealModelInferenceEngine> e(new RealModelInferenceEngine());
     e->config_ = config;
     e->weight_dir_ = weightDir;
+    if (!tokenizerDir.empty()) {
+        if (!directoryExists(tokenizerDir)) return fail(ESP_ERR_IO, "missing path: %s", tokenizerDir.c_str());
+        const TokenizerStatus st = loadTokenizer(config, tokenizerDir, &e->tokenizer_);
+        if (st.error == TokenizerError::MissingPath) return fail(ESP_ERR_IO, "missing path: %s", st.text.c_str());
+        if (!st.ok()) return fail(ESP_ERR_INVALID_ARGUMENT, "Failed to load tokenizer from %s: error %d (%ld, %ld) %s", tokenizerDir.c_str(),
+                                  (int)st.error, st.detail, st.detail2, st.text.c_str());
+    }
     int rc = loadRuntime(config, weightDir, environment, &e->runtime_);
     if (rc != ESP_OK) return rc;
     e->build_ms_ = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
@@ -200,6 +208,34 @@ int RealModelInferenceEngine::generate(const std::vector<TokenID> &promptTokens,
     out->tokenLatenciesMs = timing.token_latencies_ms;
     out->firstTokenLatencyMs = timing.first_token_latency_ms;
     out->tokensPerSecond = out->tokens.empty() ? 0.0 : (double)out->tokens.size() / std::max(timing.decode_ms / 1e3, 1e-9);
+    return ESP_OK;
+}
+
+int RealModelInferenceEngine::generateText(const std::string &prompt, int maxTokens, float temperature, const Environment &environment,
+                                           GenerationResult *out) {
+    *out = GenerationResult{};
+    if (!tokenizer_) return fail(ESP_ERR_INVALID_ARGUMENT, "the engine was built without a tokenizer directory");
+    if (maxTokens < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "maxTokens must be >= 0");
+    if (!std::isfinite(temperature) || temperature < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "temperature must be finite and >= 0");
+    // encodePrompt (:5404-5418)
+    const std::vector<int> raw = tokenizer_->encode(prompt);
+    if (raw.empty()) return fail(ESP_ERR_INVALID_ARGUMENT, "Prompt produced no tokens");
+    std::vector<TokenID> promptTokens;
+    for (int t : raw) {
+        if (t < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "Token %d does not fit TokenID", t);
+        promptTokens.push_back((TokenID)t);
+    }
+    if ((int)promptTokens.size() >= config_.maxSeq)
+        return fail(ESP_ERR_OUT_OF_RANGE, "Prompt token count %zu exceeds model context %d", promptTokens.size(), config_.maxSeq - 1);
+    std::vector<int> all(raw);
+    if (std::min(maxTokens, config_.maxSeq - (int)promptTokens.size()) > 0) {
+        int rc = generate(promptTokens, maxTokens, temperature, environment, out);
+        if (rc != ESP_OK) return rc;
+        for (TokenID t : out->tokens) all.push_back((int)t);
+    } else {
+        out->promptTokens = promptTokens;   // nothing to generate: the prompt decoded back (:1427-1437)
+    }
+    out->text = tokenizer_->decode(all);
     return ESP_OK;
 }
 

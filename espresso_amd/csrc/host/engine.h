@@ -11,13 +11,15 @@
 
 #include "../llama_runtime.h"
 #include "model_support.h"
+#include "tokenizer.h"
 
 namespace esp {
 
 using Environment = std::map<std::string, std::string>;
 
-// GenerationResult (:17-55) without the text fields (tokenizers are outside this path)
+// GenerationResult (:17-55); `text` is filled by the prompt-text entry point only
 struct GenerationResult {
+    std::string text;
     std::vector<TokenID> tokens, promptTokens;
     std::vector<double> tokenLatenciesMs;
     double tokensPerSecond = 0, compileTimeMs = 0, firstTokenLatencyMs = 0;
@@ -29,12 +31,17 @@ struct GenerationResult {
 class RealModelInferenceEngine {
   public:
     // Loads the weight directory (packed sidecar, else float32 sidecar, else fp16 BLOBFILE, per tensor) into HBM.
-    // tokenizerDir is accepted for signature parity and not read.
+    // A non-empty tokenizerDir is searched in the reference's order (loadTokenizer, :7558-7613) and must hold a
+    // tokenizer; an empty one leaves the engine with the token-id entry points only.
     static int build(const MultiModelConfig &config, const std::string &weightDir, const std::string &tokenizerDir,
                      const Environment &environment, std::unique_ptr<RealModelInferenceEngine> *out);
     // Greedy generation from token ids.  temperature must be 0 on this path.
     int generate(const std::vector<TokenID> &promptTokens, int maxTokens, float temperature, const Environment &environment,
                  GenerationResult *out);
+    // generate(prompt:maxTokens:temperature:) (:1405-1437): encodePrompt (:5404-5418), the token-id path above,
+    // text = decode(prompt tokens + generated tokens).  Needs a tokenizer.
+    int generateText(const std::string &prompt, int maxTokens, float temperature, const Environment &environment, GenerationResult *out);
+    const Tokenizer *tokenizer() const { return tokenizer_.get(); }
     static int generateTokensForTesting(const MultiModelConfig &config, const std::string &weightDir,
                                         const std::vector<TokenID> &promptTokens, int maxTokens, std::vector<TokenID> *out);
     const MultiModelConfig &config() const { return config_; }
@@ -53,6 +60,7 @@ class RealModelInferenceEngine {
     std::string weight_dir_;
     std::unique_ptr<LlamaRuntime> runtime_;
     std::unique_ptr<LlamaRuntime> draft_runtime_;
+    std::unique_ptr<Tokenizer> tokenizer_;
     std::string draft_dir_loaded_;
     double build_ms_ = 0;
 };

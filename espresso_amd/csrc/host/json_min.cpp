@@ -35,9 +35,16 @@ bool parse_string(Cursor &c, std::string *out) {
                 if (c.i + 4 > c.s.size()) return c.fail("bad \\u escape");
                 unsigned cp = (unsigned)std::strtoul(c.s.substr(c.i, 4).c_str(), nullptr, 16);
                 c.i += 4;
+                // a high surrogate followed by an escaped low surrogate is one code point
+                if (cp >= 0xD800 && cp < 0xDC00 && c.i + 6 <= c.s.size() && c.s[c.i] == '\\' && c.s[c.i + 1] == 'u') {
+                    const unsigned lo = (unsigned)std::strtoul(c.s.substr(c.i + 2, 4).c_str(), nullptr, 16);
+                    if (lo >= 0xDC00 && lo < 0xE000) { cp = 0x10000 + ((cp - 0xD800) << 10) + (lo - 0xDC00); c.i += 6; }
+                }
+                if (cp >= 0xD800 && cp < 0xE000) cp = 0xFFFD;   // lone surrogate
                 if (cp < 0x80) out->push_back((char)cp);
                 else if (cp < 0x800) { out->push_back((char)(0xC0 | (cp >> 6))); out->push_back((char)(0x80 | (cp & 0x3F))); }
-                else { out->push_back((char)(0xE0 | (cp >> 12))); out->push_back((char)(0x80 | ((cp >> 6) & 0x3F))); out->push_back((char)(0x80 | (cp & 0x3F))); }
+                else if (cp < 0x10000) { out->push_back((char)(0xE0 | (cp >> 12))); out->push_back((char)(0x80 | ((cp >> 6) & 0x3F))); out->push_back((char)(0x80 | (cp & 0x3F))); }
+                else { out->push_back((char)(0xF0 | (cp >> 18))); out->push_back((char)(0x80 | ((cp >> 12) & 0x3F))); out->push_back((char)(0x80 | ((cp >> 6) & 0x3F))); out->push_back((char)(0x80 | (cp & 0x3F))); }
                 break;
             }
             default: out->push_back(e);
@@ -86,7 +93,64 @@ bool parse_scalar(Cursor &c, JsonValue *v) {
 
 bool skip_value(Cursor &c) { JsonValue v; return parse_scalar(c, &v); }
 
+bool parse_node(Cursor &c, JsonNode *n, int depth) {
+    if (depth > 64) return c.fail("nesting too deep");
+    c.ws();
+    if (c.i >= c.s.size()) return c.fail("unexpected end");
+    const char ch = c.s[c.i];
+    if (ch == '{') {
+        c.i++;
+        n->kind = JsonNode::Object;
+        if (c.eat('}')) return true;
+        for (;;) {
+            std::string key;
+            if (!parse_string(c, &key)) return false;
+            if (!c.eat(':')) return c.fail("expected :");
+            n->members.emplace_back(std::move(key), JsonNode{});
+            if (!parse_node(c, &n->members.back().second, depth + 1)) return false;
+            if (c.eat('}')) return true;
+            if (!c.eat(',')) return c.fail("expected , or }");
+        }
+    }
+    if (ch == '[') {
+        c.i++;
+        n->kind = JsonNode::Array;
+        if (c.eat(']')) return true;
+        for (;;) {
+            n->items.emplace_back();
+            if (!parse_node(c, &n->items.back(), depth + 1)) return false;
+            if (c.eat(']')) return true;
+            if (!c.eat(',')) return c.fail("expected , or ]");
+        }
+    }
+    JsonValue v;
+    if (!parse_scalar(c, &v)) return false;
+    switch (v.kind) {
+    case JsonValue::Bool: n->kind = JsonNode::Bool; n->boolean = v.boolean; break;
+    case JsonValue::Number: n->kind = JsonNode::Number; n->number = v.number; break;
+    case JsonValue::String: n->kind = JsonNode::String; n->text = std::move(v.text); break;
+    default: n->kind = JsonNode::Null; break;
+    }
+    return true;
+}
+
 }  // namespace
+
+const JsonNode *JsonNode::find(const std::string &key) const {
+    const JsonNode *hit = nullptr;
+    for (const auto &m : members)
+        if (m.first == key) hit = &m.second;
+    return hit;
+}
+
+bool json_parse(const std::string &text, JsonNode *out, std::string *error) {
+    Cursor c{text};
+    *out = JsonNode{};
+    bool ok = parse_node(c, out, 0);
+    if (ok) { c.ws(); if (c.i != text.size()) ok = c.fail("trailing characters"); }
+    if (!ok && error) *error = c.err;
+    return ok;
+}
 
 bool json_parse_object(const std::string &text, JsonObject *out, std::string *error) {
     Cursor c{text};

@@ -71,6 +71,9 @@ def _L():
     L.esp_engine_runtime.restype = vp; L.esp_engine_runtime.argtypes = [vp]
     L.esp_engine_generate.restype = i32
     L.esp_engine_generate.argtypes = [vp, vp, i32, i32, C.c_float, C.POINTER(cp), C.POINTER(cp), i32, vp, C.POINTER(GenerationResultStruct)]
+    L.esp_engine_generate_text.restype = i32
+    L.esp_engine_generate_text.argtypes = [vp, cp, sz, i32, C.c_float, C.POINTER(cp), C.POINTER(cp), i32, vp, vp, sz, C.POINTER(sz),
+                                           C.POINTER(GenerationResultStruct)]
     L.esp_exact_two_token_promotion_plan.argtypes = [C.c_uint32] * 4 + [i32, C.POINTER(PromotionPlanStruct)]
     L.esp_exact_two_token_harness_generate.restype = i32
     L.esp_exact_two_token_harness_generate.argtypes = [C.POINTER(ExactTwoTokenModelStruct), vp, vp, vp, i32, i32, vp, C.POINTER(i32), vp, vp, C.POINTER(i32)]
@@ -178,6 +181,20 @@ class RealModelInferenceEngine:
         res = {f: getattr(r, f) for f, _ in r._fields_}
         res["exact_head_backend"] = r.exact_head_backend.decode()
         return out[:r.token_count].tolist(), res
+
+    def generate_text(self, prompt: str, max_tokens: int, temperature: float = 0.0, environment: dict | None = None):
+        """generate(prompt:maxTokens:temperature:) -> (text of prompt + generated tokens, generated tokens, result fields)."""
+        raw = prompt.encode("utf-8")
+        out = np.zeros(max(max_tokens, 1), dtype=np.uint32)
+        r = GenerationResultStruct()
+        k, v, n = _env_arrays(environment)
+        cap = 1 << 20
+        buf, nbytes = C.create_string_buffer(cap), C.c_size_t(0)
+        _lib.check(_L().esp_engine_generate_text(self._h, raw, len(raw), max_tokens, C.c_float(temperature), k, v, n, _ptr(out), buf, cap,
+                                                 C.byref(nbytes), C.byref(r)))
+        res = {f: getattr(r, f) for f, _ in r._fields_}
+        res["exact_head_backend"] = r.exact_head_backend.decode()
+        return buf.raw[:min(nbytes.value, cap)].decode("utf-8", errors="replace"), out[:r.token_count].tolist(), res
 
     def runtime(self) -> llama.LlamaRuntime:
         """A non-owning view of the engine's runtime."""

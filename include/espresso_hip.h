@@ -325,6 +325,66 @@ int esp_engine_generate(ESPEngine *engine, const uint32_t *prompt_tokens, int pr
 /* The runtime inside the engine (owned by the engine). */
 ESPLlamaRuntime *esp_engine_runtime(ESPEngine *engine);
 
+/* generate(prompt:maxTokens:temperature:) on text (:1405-1437): the prompt is encoded by the tokenizer found in the
+ * tokenizer directory given to esp_engine_build (encodePrompt, :5404-5418), generation runs as in
+ * esp_engine_generate, and the text of prompt + generated tokens is written to out_text (UTF-8, not terminated;
+ * *out_text_bytes = its full length, of which at most text_capacity bytes are written).  Fails with
+ * ESP_ERR_INVALID_ARGUMENT when the engine has no tokenizer or the prompt encodes to nothing. */
+int esp_engine_generate_text(ESPEngine *engine, const char *prompt_utf8, size_t prompt_bytes, int max_tokens, float temperature,
+                             const char *const *env_keys, const char *const *env_values, int env_count,
+                             uint32_t *out_tokens, char *out_text, size_t text_capacity, size_t *out_text_bytes,
+                             ESPGenerationResult *result);
+
+/* ---- tokenizers ----------------------------------------------------------------------------------- *
+ * The Tokenizer protocol (Sources/ModelSupport/Tokenizer.swift:1-5: encode, decode, vocabSize) and its two
+ * implementations, on the host.
+ *   esp_tokenizer_load_sentencepiece    SentencePieceTokenizer(modelURL:)  SentencePieceTokenizer.swift:19-66
+ *   esp_tokenizer_load_gpt2             GPT2BPETokenizer(vocabURL:mergesURL:)  GPT2BPETokenizer.swift:30-45
+ *   esp_tokenizer_load_tokenizer_json   GPT2BPETokenizer(tokenizerJSONURL:)    GPT2BPETokenizer.swift:47-77
+ *   esp_tokenizer_load_dir              loadTokenizer(config:tokenizerDirURL:) RealModelInferenceEngine.swift:7558-7613
+ * A loader returns NULL on failure; esp_tokenizer_last_error then holds the case of
+ * SentencePieceTokenizerError / GPT2BPETokenizerError (this thread's last load). */
+typedef struct ESPTokenizer ESPTokenizer;
+enum {
+    ESP_TOK_OK = 0,
+    ESP_TOK_UNREADABLE_FILE = 1,
+    ESP_TOK_SP_TRUNCATED_MODEL = 10,
+    ESP_TOK_SP_INVALID_MAX_TOKEN_LENGTH = 11,      /* detail = the value */
+    ESP_TOK_SP_TRUNCATED_ENTRY = 12,               /* detail = entry index */
+    ESP_TOK_SP_INVALID_UTF8_ENTRY = 13,            /* detail = entry index */
+    ESP_TOK_SP_EMPTY_VOCABULARY = 14,
+    ESP_TOK_BPE_MALFORMED_VOCABULARY = 20,
+    ESP_TOK_BPE_EMPTY_VOCABULARY = 21,
+    ESP_TOK_BPE_NON_CONTIGUOUS_TOKEN_IDS = 22,     /* detail = expectedCount, detail2 = actualMaxTokenID */
+    ESP_TOK_BPE_MALFORMED_TOKENIZER_JSON = 23,
+    ESP_TOK_BPE_UNSUPPORTED_TOKENIZER_MODEL = 24,  /* text = model type */
+    ESP_TOK_BPE_INVALID_PRE_TOKENIZER_PATTERN = 25,/* text = pattern */
+    ESP_TOK_MISSING_PATH = 30                      /* text = what was looked for */
+};
+typedef struct ESPTokenizerError {
+    int32_t code;
+    int64_t detail, detail2;
+    char text[256];
+} ESPTokenizerError;
+ESPTokenizer *esp_tokenizer_load_sentencepiece(const char *model_path);
+ESPTokenizer *esp_tokenizer_load_gpt2(const char *vocab_json_path, const char *merges_txt_path);
+ESPTokenizer *esp_tokenizer_load_tokenizer_json(const char *tokenizer_json_path);
+ESPTokenizer *esp_tokenizer_load_dir(const ESPModelConfig *config, const char *tokenizer_dir);
+void esp_tokenizer_last_error(ESPTokenizerError *out);
+void esp_tokenizer_free(ESPTokenizer *tokenizer);
+int esp_tokenizer_vocab_size(const ESPTokenizer *tokenizer);
+/* "sentencePiece" or "gpt2" (the cases of LoadedTokenizer) */
+const char *esp_tokenizer_kind(const ESPTokenizer *tokenizer);
+/* Returns the number of tokens of the text and writes the first `capacity` of them. */
+long esp_tokenizer_encode(const ESPTokenizer *tokenizer, const char *text_utf8, size_t text_bytes, int32_t *out_tokens, size_t capacity);
+/* The split GPT2BPETokenizer.encode applies before BPE (preTokenizer.matches(in:range:), GPT2BPETokenizer.swift:80-82):
+ * non-overlapping matches of `pattern_utf8` (NULL = the GPT-2 default pattern, :13-14) from left to right, as byte
+ * offsets [begin, end) into the text, two entries per match, the first `capacity_pairs` matches written.  Returns the
+ * number of matches, or ESP_ERR_INVALID_ARGUMENT for a pattern outside the supported ICU subset. */
+long esp_pretokenize(const char *pattern_utf8, const char *text_utf8, size_t text_bytes, int64_t *out_ranges, size_t capacity_pairs);
+/* Returns the UTF-8 length of the decoded text and writes its first `capacity` bytes (not terminated). */
+long esp_tokenizer_decode(const ESPTokenizer *tokenizer, const int32_t *tokens, size_t count, char *out_utf8, size_t capacity);
+
 /* sampleToken (RealModelInferenceEngine.swift:8036-8068) on the host: temperature <= 0 -> first maximum; else
  * weights exp(double((logit - max) / T)), threshold = unit * total, first index whose running remainder is <= 0.
  * `unit` in [0, 1) stands for Double.random(in: 0..<total) / total; esp_splitmix64_unit draws it from a SplitMix64

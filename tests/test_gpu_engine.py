@@ -310,3 +310,61 @@ def test_engine_temperature_sampling_replays_on_the_oracle(E, tmp_path):
         o.advance(t)
     assert agree >= 12
     e.close()
+
+
+def test_engine_generates_from_prompt_text(E, tmp_path):
+    """generate(prompt:maxTokens:temperature:) (:1405-1437): the tokenizer found in tokenizerDir encodes the prompt,
+    the token-id path runs, and the text is the decoded prompt + generated tokens."""
+    import struct
+
+    import espresso_amd._lib as lib
+    import espresso_amd.tokenizer as T
+    w = mu.random_weights(orc.LlamaConfig(**KW), 47, std=0.08, norm_jitter=0.05)
+    weights = tmp_path / "weights"
+    seen = write_weight_dir(str(weights), KW, w)
+    # a byte-fallback SentencePiece vocabulary of the model's size: "▁", 26 letters, word pieces, then <0xNN> bytes
+    pieces = [("▁", 0.0)] + [(chr(97 + i), 0.0) for i in range(26)] + [("▁a", 1.0), ("▁ab", 2.0), ("bc", 1.5), ("▁the", 3.0), ("th", 1.0), ("▁th", 2.0)]
+    pieces += [(f"<0x{b:02X}>", 0.0) for b in range(256)]
+    pieces += [(f"zz{i}", 0.0) for i in range(KW["vocab"] - len(pieces))]
+    tok_dir = tmp_path / "tok"
+    tok_dir.mkdir()
+    data = struct.pack("<i", 16)
+    for piece, score in pieces:
+        raw = piece.encode()
+        data += struct.pack("<fi", score, len(raw)) + raw
+    (tok_dir / "tokenizer.model").write_bytes(data)
+    tok = T.Tokenizer.from_dir(gpu_cfg(KW), str(tok_dir))
+    prompt = "the abc é"
+    prompt_ids = tok.encode(prompt)
+    assert tok.decode(prompt_ids) == prompt
+
+    e = E.RealModelInferenceEngine(gpu_cfg(KW), str(weights), tokenizer_dir=str(tok_dir))
+    text, toks, res = e.generate_text(prompt, 12)
+    assert toks == oracle_tokens(KW, seen, prompt_ids, 12)                     # same ids as the token-id entry point
+    assert toks == e.generate(prompt_ids, 12)[0]
+    assert text == tok.decode(prompt_ids + toks)
+    assert res["token_count"] == 12
+    # nothing to generate: the prompt decoded back (:1427-1437)
+    text0, toks0, _ = e.generate_text(prompt, 0)
+    assert (text0, toks0) == (prompt, [])
+    e.close()
+    # a prompt that encodes to nothing is refused (encodePrompt, :5404-5408): byte-level BPE of the empty string
+    bpe_dir = tmp_path / "bpe"
+    bpe_dir.mkdir()
+    (bpe_dir / "vocab.json").write_text(json.dumps({chr(33 + i): i for i in range(8)}))
+    (bpe_dir / "merges.txt").write_text("#version: 0.2\n")
+    e = E.RealModelInferenceEngine(gpu_cfg(KW), str(weights), tokenizer_dir=str(bpe_dir))
+    with pytest.raises(lib.EspressoError, match="no tokens"):
+        e.generate_text("", 4)
+    assert e.generate_text("!#", 3)[0].startswith("!#")
+    e.close()
+    # an engine without a tokenizer directory has the token-id entry points only
+    e = E.RealModelInferenceEngine(gpu_cfg(KW), str(weights))
+    with pytest.raises(lib.EspressoError, match="without a tokenizer"):
+        e.generate_text(prompt, 4)
+    e.close()
+    # a tokenizer directory that holds none of the candidates fails the build, as loadTokenizer throws (:7609-7611)
+    empty = tmp_path / "empty"
+    empty.mkdir()
+    with pytest.raises(lib.EspressoError, match="missing path"):
+        E.RealModelInferenceEngine(gpu_cfg(KW), str(weights), tokenizer_dir=str(empty))
