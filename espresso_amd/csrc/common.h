@@ -73,6 +73,10 @@ struct GemvParams {
     // while staging, and `x` is ignored.  norm_x: fp32 [batch][cols]; norm_w: fp32 [cols].
     const float *norm_x = nullptr, *norm_w = nullptr;
     float norm_eps = 0.0f;
+    // attention context merged while staging: when merge_partials is set (see gemv_merges_attention_partials)
+    // the activations are the per-head partial states of launch_attention_partials, merged and rounded to
+    // fp16; `x` and `norm_x` are ignored.  [batch][cols / 128][4][132] floats.
+    const float *merge_partials = nullptr;
     float *y = nullptr;           // fp32 out [batch][rows]
     const float *residual = nullptr;
     uint16_t *out_f16 = nullptr;  // EPI_SWIGLU_F16: [batch][rows/2]
@@ -94,6 +98,8 @@ struct GemmParams {
 
 // kernels/gemv.hip
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
+// True when launch_gemv can take its input as attention partial states (Q4_K, 2048 or 4096 columns, batch <= 2).
+bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch);
 // kernels/gemm.hip
 hipError_t launch_gemm(const GemmParams &p, hipStream_t stream);
 // kernels/dequant.hip — GGUF-layout blocks -> fp32, bit-exact to the block definitions

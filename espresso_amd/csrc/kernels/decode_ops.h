@@ -43,6 +43,8 @@ struct AttentionArgs {
     uint16_t *ctx_f16;      // [rows][attnDim]
     // partial results of the split-prefix kernel: [rows][kvHeads][splits][group][head_dim + 2] floats
     float *split_scratch;
+    // partial results of attention_partial_kernel: [rows][heads][attention_head_splits][head_dim + 4] floats
+    float *head_partials;
 };
 constexpr int kAttentionMaxSplits = 32;
 // Slices of the prefix the grouped-query attention kernel works on in parallel (fixed per runtime).
@@ -53,6 +55,11 @@ hipError_t launch_rmsnorm(const float *x, const float *w, float eps, int rows, i
                           unsigned long long *argmax_cells, hipStream_t s);
 hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStream_t s);
 hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
+// Attention that stops at per-split partial states (head_dim 128, up to kMaxStepRows rows); the GEMV that reads
+// the context merges them (GemvParams::merge_partials).  attention_head_splits: slices per query head.
+constexpr int kAttentionHeadSplits = 4;   // the GEMV's merge is written for this many
+int attention_head_splits(int max_seq);
+hipError_t launch_attention_partials(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
 hipError_t launch_swiglu(const float *gu, int rows, int hidden, uint16_t *act_f16, hipStream_t s);
 // Scratch of the two-launch argmax: kMaxStepRows x 128 partial (value, index) pairs.
 struct ArgmaxScratch {

@@ -324,6 +324,9 @@ __global__ __launch_bounds__(256) void attention_flash_kernel(AttentionArgs a) {
 #pragma unroll
             for (int i = 0; i < KW; i++) { kr[u][i] = kp[i]; vr[u][i] = vp[i]; }
         }
+        // every load above is issued before the first use below: one memory round trip for all U chunks
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int t = t0 + u * stride + slot;
@@ -412,6 +415,119 @@ __global__ __launch_bounds__(HD) void attention_merge_kernel(AttentionArgs a, in
         A = __builtin_fmaf(pa[sp], f, A);
     }
     a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)head * HD + dch] = to_half_bits(L > 0.0f ? A / L : 0.0f);
+}
+
+// Single-query attention whose merge is left to the consumer: grid (query heads, rows, kHeadSplits), four
+// wavefronts per workgroup, one query head each.  Chunks, lane mapping and the (m, l, acc) arithmetic are
+// those of attention_flash_kernel; a wavefront keeps U chunks of loads in flight, so kHeadSplits * 4 * U
+// chunks of the prefix cost one memory round trip and longer prefixes loop.  Every workgroup writes its
+// state to `head_partials` as [row][head][split][HD values, m, l, 2 pad] (16-byte aligned rows); the GEMV
+// that consumes the context merges the splits while it stages its input, so no merge launch follows.
+// Workgroups x, x + kvHeads, ... serve the query heads of KV head x: with eight KV heads the group shares
+// one L2, which then reads K and V from memory once.
+template <int HD, bool KV_F16, int U>
+__global__ __launch_bounds__(256) void attention_partial_kernel(AttentionArgs a) {
+    constexpr int WAVES = 4, LPT = HD / 8, SLOTS = 64 / LPT, KW = KV_F16 ? 1 : 2, STRIDE = HD + 4;
+    __shared__ float wm[WAVES], wl[WAVES][SLOTS];
+    __shared__ float wacc[WAVES][SLOTS][HD];
+    const int group = a.n_head / a.n_kv_head;
+    const int kvh = blockIdx.x % a.n_kv_head, head = kvh * group + blockIdx.x / a.n_kv_head, m = blockIdx.y;
+    const int split = blockIdx.z, splits = gridDim.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int visible = a.pos[m] + 1;
+    const int kd = a.n_kv_head * HD;
+    const size_t seq_base = (size_t)a.seq[m] * a.cache_seq_stride;
+    const float scale = 1.0f / sqrtf((float)HD);
+    const int slot = lane / LPT, seg = (lane % LPT) * 8;
+
+    float q[8];
+    {
+        const float4 *qp = reinterpret_cast<const float4 *>(a.q + (size_t)m * a.n_head * HD + (size_t)head * HD + seg);
+        const float4 q0 = qp[0], q1 = qp[1];
+        q[0] = q0.x; q[1] = q0.y; q[2] = q0.z; q[3] = q0.w;
+        q[4] = q1.x; q[5] = q1.y; q[6] = q1.z; q[7] = q1.w;
+    }
+    float mx = -INFINITY, l = 0.0f, acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.0f;
+
+    auto unpack8 = [](const uint4 *r, float *out) {
+        if (KV_F16) {
+            const uint32_t w[4] = {r[0].x, r[0].y, r[0].z, r[0].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) { out[2 * i] = from_half_bits((uint16_t)(w[i] & 0xFFFFu)); out[2 * i + 1] = from_half_bits((uint16_t)(w[i] >> 16)); }
+        } else {
+            out[0] = __uint_as_float(r[0].x); out[1] = __uint_as_float(r[0].y); out[2] = __uint_as_float(r[0].z); out[3] = __uint_as_float(r[0].w);
+            out[4] = __uint_as_float(r[KW - 1].x); out[5] = __uint_as_float(r[KW - 1].y); out[6] = __uint_as_float(r[KW - 1].z); out[7] = __uint_as_float(r[KW - 1].w);
+        }
+    };
+
+    const int stride = splits * WAVES * SLOTS;
+    for (int t0 = (split * WAVES + wave) * SLOTS; t0 < visible; t0 += stride * U) {
+        uint4 kr[U][KW], vr[U][KW];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int t = t0 + u * stride + slot;
+            const size_t off = seq_base + (size_t)(t < visible ? t : 0) * kd + (size_t)kvh * HD + seg;
+            const uint4 *kp = KV_F16 ? reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.k_cache) + off)
+                                     : reinterpret_cast<const uint4 *>(reinterpret_cast<const float *>(a.k_cache) + off);
+            const uint4 *vp = KV_F16 ? reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(a.v_cache) + off)
+                                     : reinterpret_cast<const uint4 *>(reinterpret_cast<const float *>(a.v_cache) + off);
+#pragma unroll
+            for (int i = 0; i < KW; i++) { kr[u][i] = kp[i]; vr[u][i] = vp[i]; }
+        }
+        // every load above is issued before the first use below: one memory round trip for all U chunks
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int t = t0 + u * stride + slot;
+            const bool valid = t < visible;
+            // a chunk wholly beyond the prefix changes nothing (alpha = 1, p = 0): no branch, so the loop unrolls and
+            // all U chunks stay in registers
+            float k[8], v[8];
+            unpack8(kr[u], k);
+            unpack8(vr[u], v);
+            float d = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) d = __builtin_fmaf(q[i], k[i], d);
+            d = group_sum<LPT>(d);                                  // all lanes of the token
+            const float sc = valid ? __fmul_rn(d, scale) : -INFINITY;
+            const float cm = max_over_groups<LPT>(sc);              // over the chunk's tokens
+            const float m_new = fmaxf(mx, cm);         // finite: the chunk holds at least one visible token
+            const float alpha = expf(mx - m_new);      // exp(-inf) = 0 on the first chunk
+            const float p = valid ? expf(sc - m_new) : 0.0f;
+            l = __builtin_fmaf(l, alpha, p);
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[i] = __builtin_fmaf(p, v[i], __fmul_rn(acc[i], alpha));
+            mx = m_new;
+        }
+    }
+    // ---- every (wavefront, token slot) publishes its partial state; m is the same in all lanes ----
+#pragma unroll
+    for (int i = 0; i < 8; i++) wacc[wave][slot][seg + i] = acc[i];
+    if (lane % LPT == 0) wl[wave][slot] = l;
+    if (lane == 0) wm[wave] = mx;
+    __syncthreads();
+    // ---- merge over wavefronts and slots in wavefront order: thread = channel ----
+    float *ps = a.head_partials + (((size_t)m * a.n_head + head) * splits + split) * STRIDE;
+    for (int dch = tid; dch < HD; dch += 256) {
+        float M = wm[0];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) M = fmaxf(M, wm[w]);
+        float L = 0.0f, A = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) {
+            const float f = wm[w] == -INFINITY ? 0.0f : expf(wm[w] - M);
+            float lw = 0.0f, aw = 0.0f;
+#pragma unroll
+            for (int sl = 0; sl < SLOTS; sl++) { lw += wl[w][sl]; aw += wacc[w][sl][dch]; }
+            L = __builtin_fmaf(lw, f, L);
+            A = __builtin_fmaf(aw, f, A);
+        }
+        ps[dch] = A;
+        if (dch == 0) { ps[HD] = M; ps[HD + 1] = L; }
+    }
 }
 
 template <int HD, int G>
@@ -591,6 +707,16 @@ hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipSt
     dim3 grid(a.n_head, rows);
     if (kv_f16) hipLaunchKernelGGL(attention_decode_kernel<true>, grid, dim3(kBlock), lds, s, a);
     else hipLaunchKernelGGL(attention_decode_kernel<false>, grid, dim3(kBlock), lds, s, a);
+    return hipGetLastError();
+}
+
+int attention_head_splits(int) { return kAttentionHeadSplits; }
+
+hipError_t launch_attention_partials(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
+    if (!a.head_partials || a.head_dim != 128 || a.n_head % a.n_kv_head != 0 || rows < 1 || rows > kMaxStepRows) return hipErrorInvalidValue;
+    dim3 grid(a.n_head, rows, attention_head_splits(a.max_seq));
+    if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<128, true, 12>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((attention_partial_kernel<128, false, 6>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 

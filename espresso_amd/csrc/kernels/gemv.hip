@@ -24,6 +24,8 @@
 // algorithmic bytes; x is re-read from L2 once per workgroup.
 #include <cstdlib>
 
+#include <type_traits>
+
 #include "../common.h"
 #include "gemv_device.h"
 
@@ -86,6 +88,9 @@ struct KernelArgs {
     // when norm_x is set the activations are rmsnorm(norm_x) * norm_w computed while staging (x is unused)
     const float *norm_x, *norm_w;
     float norm_eps;
+    // when merge_partials is set the activations are the attention context merged from per-split partial states
+    // while staging (x and norm_x unused): [batch][cols / 128 heads][kMergeSplits][128 values, m, l, 2 pad]
+    const float *merge_partials;
 };
 
 // 1 / sqrt(mean(x^2) + eps) of row b of norm_x (any cols that is a multiple of 8); `red` as above.
@@ -420,6 +425,69 @@ struct Q4KStage {
     }
 };
 
+// Staging for a GEMV whose input is the attention context (head size 128): merges the kMergeSplits partial
+// states (m, l, acc) that attention_partial_kernel left per query head, in split order and with the arithmetic
+// of attention_merge_kernel (max of m, f = exp(m - M), L = fma(l, f, L), A = fma(acc, f, A), A / L), rounds the
+// context to fp16 and stages it like any other activation vector.  Row 0's loads are issued with issue();
+// further rows take one more round trip each inside finish().
+constexpr int kMergeSplits = 4, kMergeHeadDim = 128, kMergeStride = kMergeHeadDim + 4;
+template <int B, int IPR>
+struct Q4KMergeStage {
+    static constexpr int GROUPS = IPR * 8, K = GROUPS / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1, HEADS = cols / kMergeHeadDim;
+    static_assert(GROUPS % kThreads == 0 && cols % kMergeHeadDim == 0, "whole groups per thread, whole heads per row");
+    float4 a0[K][kMergeSplits], a1[K][kMergeSplits];
+    float2 ml[K][kMergeSplits];
+
+    __device__ __forceinline__ void load_row(const KernelArgs &a, int b) {
+        const int tid = threadIdx.x;
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int g = tid + k * kThreads, head = g / (kMergeHeadDim / 8), d0 = (g % (kMergeHeadDim / 8)) * 8;
+            const float *base = a.merge_partials + ((size_t)b * HEADS + head) * kMergeSplits * kMergeStride;
+#pragma unroll
+            for (int sp = 0; sp < kMergeSplits; sp++) {
+                const float *ps = base + sp * kMergeStride;
+                a0[k][sp] = *reinterpret_cast<const float4 *>(ps + d0);
+                a1[k][sp] = *reinterpret_cast<const float4 *>(ps + d0 + 4);
+                ml[k][sp] = *reinterpret_cast<const float2 *>(ps + kMergeHeadDim);
+            }
+        }
+    }
+    __device__ __forceinline__ void store_row(int b, uint4 *xs4, float *xsum) {
+        const int tid = threadIdx.x;
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            float M = ml[k][0].x;
+#pragma unroll
+            for (int sp = 1; sp < kMergeSplits; sp++) M = fmaxf(M, ml[k][sp].x);
+            float L = 0.0f, A[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int sp = 0; sp < kMergeSplits; sp++) {
+                const float f = ml[k][sp].x != -INFINITY ? expf(ml[k][sp].x - M) : 0.0f;
+                L = __builtin_fmaf(ml[k][sp].y, f, L);
+                const float v[8] = {a0[k][sp].x, a0[k][sp].y, a0[k][sp].z, a0[k][sp].w, a1[k][sp].x, a1[k][sp].y, a1[k][sp].z, a1[k][sp].w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) A[i] = __builtin_fmaf(v[i], f, A[i]);
+            }
+            float c[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) c[i] = L > 0.0f ? A[i] / L : 0.0f;
+            uint4 h;
+            h.x = pack_half2(c[0], c[1]); h.y = pack_half2(c[2], c[3]); h.z = pack_half2(c[4], c[5]); h.w = pack_half2(c[6], c[7]);
+            q4k_store_group(h, b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
+        }
+    }
+    __device__ __forceinline__ void issue(const KernelArgs &a) { load_row(a, 0); }
+    __device__ __forceinline__ void finish(const KernelArgs &a, uint4 *xs4, float *xsum, float *) {
+        store_row(0, xs4, xsum);
+#pragma unroll
+        for (int b = 1; b < B; b++) {
+            load_row(a, b);
+            store_row(b, xs4, xsum);
+        }
+    }
+};
+
 // Persistent kernel for cols = 64 * IPR.  TEAM wavefronts share one row pair at a time (TEAM = 1: a
 // wavefront streams whole pairs on its own; TEAM = 4: the workgroup splits a long row pair and adds
 // the four partial sums through LDS).  Teams take pairs team, team + n_teams, ...: the chip reads
@@ -427,7 +495,8 @@ struct Q4KStage {
 // pairs it handles, and the loads of a team's next pair are issued before the arithmetic of the
 // current one, so weight traffic never waits for the arithmetic.  Every workgroup runs `iters`
 // rounds, so the barriers of the TEAM > 1 reduction line up even when the last round is ragged.
-template <int B, int IPR, int TEAM, bool NORM>
+// MODE: 0 = fp16 activations as given, 1 = RMSNorm fused into the staging, 2 = attention partial states merged in the staging.
+template <int B, int IPR, int TEAM, int MODE>
 __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int iters) {
     constexpr int cols = IPR * 64, XSTRIDE = IPR | 1, TOTAL = 2 * IPR, TEAM_LANES = TEAM * 64;
     constexpr int PASSES = (TOTAL + TEAM_LANES - 1) / TEAM_LANES, TEAMS = kWaves / TEAM;
@@ -510,7 +579,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int it
     };
 
     Q4KItem buf0[PASSES], buf1[PASSES];
-    Q4KStage<B, IPR, NORM> stage;
+    typename std::conditional<MODE == 2, Q4KMergeStage<B, MODE == 2 ? IPR : 32>, Q4KStage<B, IPR, MODE == 1>>::type stage;
     int pair = blockIdx.x * TEAMS + wave / TEAM;
     stage.issue(a);
     if (pair < npairs) load_pair(pair, buf0);
@@ -618,11 +687,11 @@ int compute_units() {
     return v;
 }
 
-template <int B, int IPR, int TEAM, bool NORM>
+template <int B, int IPR, int TEAM, int MODE>
 hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     constexpr int TEAMS = kWaves / TEAM;
     const size_t lds = (size_t)B * 8 * (IPR | 1) * 16 + (size_t)B * (IPR * 2) * 4 + (size_t)(2 * kWaves * 2 * B + B * kWaves) * 4;
-    auto kernel = gemv_q4k_kernel<B, IPR, TEAM, NORM>;
+    auto kernel = gemv_q4k_kernel<B, IPR, TEAM, MODE>;
     static size_t configured_lds = 0;
     hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
     if (e != hipSuccess) return e;
@@ -650,12 +719,17 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
 template <int B>
 hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     const bool norm = a.norm_x != nullptr;
+    if (a.merge_partials) {   // launch_gemv has checked the width
+        if (a.cols == 2048) return launch_q4k_persistent<B, 32, 1, 2>(a, stream);
+        if (a.cols == 4096) return launch_q4k_persistent<B, 64, 1, 2>(a, stream);
+        return hipErrorInvalidValue;
+    }
     switch (a.cols) {
-    case 2048: return norm ? launch_q4k_persistent<B, 32, 1, true>(a, stream) : launch_q4k_persistent<B, 32, 1, false>(a, stream);
-    case 4096: return norm ? launch_q4k_persistent<B, 64, 1, true>(a, stream) : launch_q4k_persistent<B, 64, 1, false>(a, stream);
-    case 8192: return norm ? launch_q4k_persistent<B, 128, 2, true>(a, stream) : launch_q4k_persistent<B, 128, 2, false>(a, stream);
-    case 11008: if (!norm) return launch_q4k_persistent<B, 172, 4, false>(a, stream); break;
-    case 14336: if (!norm) return launch_q4k_persistent<B, 224, 4, false>(a, stream); break;
+    case 2048: return norm ? launch_q4k_persistent<B, 32, 1, 1>(a, stream) : launch_q4k_persistent<B, 32, 1, 0>(a, stream);
+    case 4096: return norm ? launch_q4k_persistent<B, 64, 1, 1>(a, stream) : launch_q4k_persistent<B, 64, 1, 0>(a, stream);
+    case 8192: return norm ? launch_q4k_persistent<B, 128, 2, 1>(a, stream) : launch_q4k_persistent<B, 128, 2, 0>(a, stream);
+    case 11008: if (!norm) return launch_q4k_persistent<B, 172, 4, 0>(a, stream); break;
+    case 14336: if (!norm) return launch_q4k_persistent<B, 224, 4, 0>(a, stream); break;
     default: break;
     }
     const size_t lds = (size_t)B * 8 * ((a.cols / 64) | 1) * 16 + (size_t)B * (a.cols / 32) * 4 + (size_t)B * kWaves * 4;
@@ -696,9 +770,14 @@ hipError_t launch_fmt(const KernelArgs &a, int batch, hipStream_t stream) {
 
 }  // namespace
 
+bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch) {
+    return w.format == FMT_Q4_K && (w.cols == 2048 || w.cols == 4096) && batch >= 1 && batch <= 2;
+}
+
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     const DeviceMatrix &w = p.w;
-    if (!w.qs || (!p.x && !p.norm_x) || (p.norm_x && !p.norm_w) || w.rows <= 0 || w.cols <= 0 || p.batch <= 0) return hipErrorInvalidValue;
+    if (!w.qs || (!p.x && !p.norm_x && !p.merge_partials) || (p.norm_x && !p.norm_w) || w.rows <= 0 || w.cols <= 0 || p.batch <= 0) return hipErrorInvalidValue;
+    if (p.merge_partials && !gemv_merges_attention_partials(w, p.batch)) return hipErrorInvalidValue;
     if ((p.epilogue == EPI_STORE_F32 || p.epilogue == EPI_ADD_RESIDUAL) && !p.y) return hipErrorInvalidValue;
     if (p.epilogue == EPI_ADD_RESIDUAL && !p.residual) return hipErrorInvalidValue;
     if (p.epilogue == EPI_SWIGLU_F16 && (!p.out_f16 || w.rows % 2 != 0)) return hipErrorInvalidValue;
@@ -717,7 +796,8 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         const int nb = p.batch - b0 >= 2 ? 2 : 1;
         KernelArgs a;
         a.qs = w.qs; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.rows = w.rows; a.cols = w.cols;
-        a.x = p.x + (size_t)b0 * w.cols;
+        a.x = p.x ? p.x + (size_t)b0 * w.cols : nullptr;
+        a.merge_partials = p.merge_partials;   // batch <= 2 here: one launch
         a.y = p.y ? p.y + (size_t)b0 * w.rows : nullptr;
         a.residual = p.residual ? p.residual + (size_t)b0 * w.rows : nullptr;
         a.out_f16 = p.out_f16 ? p.out_f16 + (size_t)b0 * (w.rows / 2) : nullptr;

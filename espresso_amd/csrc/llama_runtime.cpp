@@ -127,6 +127,14 @@ int LlamaRuntime::collect_kernel_times(double total_us[K_CLASS_COUNT], long laun
 // Launches the GEMV of one class for every layer in turn (the head: the same matrix), `iters` rounds, between
 // two events: back-to-back dependent launches at the real shapes over the real weights, which no cache can hold
 // across a round.  The epilogues write into the step's buffers, so sequence state is garbage afterwards.
+// The decode step (one or two rows) runs attention as a single launch that leaves per-head partial states, and
+// the wo GEMV merges them while staging, when the head size and the matrix allow it.  The fused trunk keeps the
+// split-and-merge arithmetic it is compared with.
+bool LlamaRuntime::wo_merges_attention(const Layer &L, int rows) const {
+    return merged_attention_ && !fused_trunk_active() && c_.head_dim == 128 && c_.n_head % c_.n_kv_head == 0 && rows <= 2 &&
+           L.wo.cols == c_.attention_dim() && gemv_merges_attention_partials(L.wo, rows);
+}
+
 int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us) {
     if (!finalized_ || iters < 1 || !mean_us) return fail(ESP_ERR_INVALID_ARGUMENT, "time_kernel_class: bad argument");
     if (kernel_class < K_QKV || kernel_class > K_HEAD) return fail(ESP_ERR_INVALID_ARGUMENT, "time_kernel_class: class %d", kernel_class);
@@ -145,7 +153,10 @@ int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us
             g.qkv.q_out = q_; g.qkv.k_cache = L->k_cache; g.qkv.v_cache = L->v_cache;
             g.qkv.cache_seq_stride = (size_t)kd * c_.max_seq; g.qkv.kv_f16 = kv16 ? 1 : 0;
             break;
-        case K_WO: g.w = L->wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL; break;
+        case K_WO:
+            g.w = L->wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
+            if (wo_merges_attention(*L, 1)) { g.x = nullptr; g.merge_partials = attn_scratch_; }
+            break;
         case K_GATE_UP:
             g.w = L->w13; g.norm_x = hidden_; g.norm_w = L->rms_ffn; g.norm_eps = c_.norm_eps; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
             break;
@@ -486,16 +497,21 @@ int LlamaRuntime::enqueue_trunk(int M) {
         aa.n_head = c_.n_head; aa.n_kv_head = c_.n_kv_head; aa.head_dim = c_.head_dim; aa.max_seq = c_.max_seq;
         aa.pos = d_pos_; aa.seq = d_seq_; aa.ctx_f16 = ctx_;
         aa.split_scratch = attn_scratch_;
+        aa.head_partials = attn_scratch_;
+        // one attention launch instead of two where the wo GEMV can merge the partial states in its staging
+        const bool merge_in_wo = wo_merges_attention(L, M);
         if ((rc = time_begin(K_ATTENTION)) != ESP_OK) return rc;
-        ESP_HIP_TRY(launch_attention(aa, M, kv16, s));
+        if (merge_in_wo) ESP_HIP_TRY(launch_attention_partials(aa, M, kv16, s));
+        else ESP_HIP_TRY(launch_attention(aa, M, kv16, s));
         if ((rc = time_end()) != ESP_OK) return rc;
         g = GemvParams{};
         g.batch = M;
         g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
+        if (merge_in_wo) { g.x = nullptr; g.merge_partials = attn_scratch_; }
         if ((rc = time_begin(K_WO)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
-        g.w = L.w13; g.x = nullptr; g.norm_x = hidden_; g.norm_w = L.rms_ffn; g.norm_eps = c_.norm_eps;
+        g.w = L.w13; g.x = nullptr; g.merge_partials = nullptr; g.norm_x = hidden_; g.norm_w = L.rms_ffn; g.norm_eps = c_.norm_eps;
         g.y = nullptr; g.residual = nullptr; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
         if ((rc = time_begin(K_GATE_UP)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
@@ -513,6 +529,12 @@ int LlamaRuntime::enqueue_trunk(int M) {
 void LlamaRuntime::set_fused_trunk(bool enabled) {
     if (enabled == fused_trunk_) return;
     fused_trunk_ = enabled;
+    for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }   // captured with the other path
+}
+
+void LlamaRuntime::set_merged_attention(bool enabled) {
+    if (enabled == merged_attention_) return;
+    merged_attention_ = enabled;
     for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }   // captured with the other path
 }
 

@@ -71,6 +71,10 @@ class LlamaRuntime {
     // stack as one persistent launch (default on where supported).
     void set_fused_trunk(bool enabled);
     bool fused_trunk_active() const { return fused_trunk_ && trunk_layers_ != nullptr; }
+    // Decode steps of one or two rows: attention as one launch that leaves partial states, merged by the wo GEMV
+    // (on by default where the shapes allow); off = the split kernel plus the merge kernel.
+    void set_merged_attention(bool enabled);
+    bool merged_attention_in_use() const { return !layers_.empty() && wo_merges_attention(layers_[0], 1); }
     int fused_trunk_timeouts(unsigned *out);
     int check_fused_trunk();
     int read_last_hidden(int seq, float *out);
@@ -102,6 +106,7 @@ class LlamaRuntime {
     int prefill_block(int seq, const uint32_t *tokens, int rows, int base);
     int enqueue_layers_matrix(int rows);
     bool matrix_prefill_supported() const;
+    bool wo_merges_attention(const Layer &L, int rows) const;
     int capture_step_graph(int seq);
     HostTensor *host_slot(int layer, int slot);
 
@@ -130,6 +135,7 @@ class LlamaRuntime {
     float *attn_scratch_ = nullptr;
     bool matrix_prefill_ = true;
     bool fused_trunk_ = true;
+    bool merged_attention_ = true;
     TrunkLayer *trunk_layers_ = nullptr;   // device table, set when the fused trunk kernel covers this model
     unsigned *trunk_sync_ = nullptr;
     float *gemm_workspace_ = nullptr;

@@ -185,6 +185,14 @@ def set_fused_trunk(rt: LlamaRuntime, enabled: bool) -> None:
     _lib.check(rt._L.esp_llama_set_fused_trunk(rt._h, int(enabled)))
 
 
+def set_merged_attention(rt: LlamaRuntime, enabled: bool) -> bool:
+    """Returns whether the one-launch attention merged by the wo GEMV is in use after the call."""
+    r = rt._L.esp_llama_set_merged_attention(rt._h, int(enabled))
+    if r < 0:
+        _lib.check(r)
+    return bool(r)
+
+
 def fused_trunk_status(rt: LlamaRuntime) -> tuple[bool, int]:
     """(fused trunk kernel in use, barrier time-outs so far)."""
     import ctypes as C

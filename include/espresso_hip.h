@@ -225,6 +225,12 @@ int esp_llama_set_matrix_prefill(ESPLlamaRuntime *runtime, int enabled);
 int esp_llama_set_fused_trunk(ESPLlamaRuntime *runtime, int enabled);
 int esp_llama_fused_trunk_status(ESPLlamaRuntime *runtime, int *active, unsigned *barrier_timeouts);
 
+/* Decode steps of one or two rows run attention (decodeContextFromCaches, :6774-6823) as one launch that leaves
+ * per-head partial softmax states, and the wo GEMV merges them while it stages its input, where the shapes allow
+ * (head size 128, Q4_K wo of 2048 or 4096 columns).  enabled = 0 restores the split kernel plus the merge kernel
+ * everywhere.  Returns 1 when the merged form is in use after the call, 0 when not, negative on error. */
+int esp_llama_set_merged_attention(ESPLlamaRuntime *runtime, int enabled);
+
 /* Per-kernel timing with HIP events on the library stream.  While enabled every launch of the GEMV
  * and attention kernels of a step is bracketed by an event pair; esp_llama_kernel_times synchronises
  * and reports, per kernel class, the summed elapsed microseconds, the launch count and the

@@ -282,3 +282,40 @@ def test_batch16_two_token_equals_batch16_greedy(llama, fmt):
         want, margin = o.generate(prompts[s], 40, with_margin=True)
         if margin > 5e-3:
             assert plain[s] == want, (s, margin)
+
+
+MERGED = dict(n_layer=2, n_head=16, n_kv_head=4, d_model=2048, head_dim=128, hidden_dim=512, vocab=512, max_seq=320)
+
+
+@pytest.mark.parametrize("kv_fp16", [False, True])
+def test_attention_merged_in_the_wo_gemv(llama, kv_fp16):
+    """Head size 128 with a Q4_K wo of 2048 columns: decode steps run attention as one launch and the wo GEMV
+    merges the partial states.  Against the oracle, and against the split + merge kernels of the same runtime."""
+    o, g = make_pair(llama, MERGED, orc.FMT_Q4_K, seed=77, std=0.04, kv_fp16=kv_fp16, norm_jitter=0.05)
+    assert llama.set_merged_attention(g, True)
+    rng = np.random.default_rng(5)
+    prompt = rng.integers(0, MERGED["vocab"], 20).tolist()
+    o.prefill(prompt)
+    g.prefill(prompt)
+    for step in range(6):
+        assert np.abs(o.last_hidden() - g.last_hidden()).max() <= 2e-3 * max(1.0, np.abs(o.last_hidden()).max())
+        assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
+        tok = o.select_greedy()
+        if o.top2_margin() > 1e-3:
+            assert g.select_greedy() == tok
+        o.advance(tok); g.advance(tok)
+    # long prefix (several rounds of chunks per wavefront), graph replay, and the two-row verify step
+    long_prompt = rng.integers(0, MERGED["vocab"], 290).tolist()
+    merged_tokens = g.generate(long_prompt, 24)[0]
+    merged_logits = g.logits().copy()
+    assert not llama.set_merged_attention(g, False)
+    split_tokens = g.generate(long_prompt, 24)[0]
+    assert merged_tokens == split_tokens
+    assert np.abs(merged_logits - g.logits()).max() <= 1e-2     # different split counts: different fp32 orders, fp16 context
+    llama.set_merged_attention(g, True)
+    _, draft = make_pair(llama, dict(MERGED, n_layer=1), orc.FMT_Q4_K, seed=78, std=0.04, kv_fp16=kv_fp16)
+    got, st = llama.generate_two_token(g, draft, long_prompt[:40], 30)
+    assert got == g.generate(long_prompt[:40], 30)[0]
+    # models whose shapes do not qualify keep the two-kernel form
+    _, tiny = make_pair(llama, TINY, orc.FMT_Q4_K, seed=3)
+    assert not llama.set_merged_attention(tiny, True)
