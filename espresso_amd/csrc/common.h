@@ -98,6 +98,11 @@ struct GemmParams {
 
 // kernels/gemv.hip
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
+// Slices of the prefix per query head that launch_attention_partials writes and the merging GEMV reads.
+#ifndef ESP_ATTENTION_HEAD_SPLITS
+#define ESP_ATTENTION_HEAD_SPLITS 4
+#endif
+constexpr int kAttentionHeadSplits = ESP_ATTENTION_HEAD_SPLITS;
 // True when launch_gemv can take its input as attention partial states (Q4_K, 2048 or 4096 columns, batch <= 2).
 bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch);
 // kernels/gemm.hip

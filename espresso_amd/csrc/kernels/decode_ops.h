@@ -57,7 +57,6 @@ hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStrea
 hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
 // Attention that stops at per-split partial states (head_dim 128, up to kMaxStepRows rows); the GEMV that reads
 // the context merges them (GemvParams::merge_partials).  attention_head_splits: slices per query head.
-constexpr int kAttentionHeadSplits = 4;   // the GEMV's merge is written for this many
 int attention_head_splits(int max_seq);
 hipError_t launch_attention_partials(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
 hipError_t launch_swiglu(const float *gu, int rows, int hidden, uint16_t *act_f16, hipStream_t s);

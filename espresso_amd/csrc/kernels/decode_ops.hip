@@ -417,17 +417,18 @@ __global__ __launch_bounds__(HD) void attention_merge_kernel(AttentionArgs a, in
     a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)head * HD + dch] = to_half_bits(L > 0.0f ? A / L : 0.0f);
 }
 
-// Single-query attention whose merge is left to the consumer: grid (query heads, rows, kHeadSplits), four
-// wavefronts per workgroup, one query head each.  Chunks, lane mapping and the (m, l, acc) arithmetic are
-// those of attention_flash_kernel; a wavefront keeps U chunks of loads in flight, so kHeadSplits * 4 * U
-// chunks of the prefix cost one memory round trip and longer prefixes loop.  Every workgroup writes its
+// Single-query attention whose merge is left to the consumer: grid (query heads, rows, kAttentionHeadSplits),
+// WAVES wavefronts per workgroup, one query head each.  Chunks, lane mapping and the (m, l, acc) arithmetic are
+// those of attention_flash_kernel; a wavefront keeps U chunks of loads in flight, so kAttentionHeadSplits *
+// WAVES * U chunks of the prefix cost one memory round trip and longer prefixes loop.  The arithmetic per
+// chunk is what a wavefront spends its time on, hence many wavefronts with few chunks each.  Every workgroup writes its
 // state to `head_partials` as [row][head][split][HD values, m, l, 2 pad] (16-byte aligned rows); the GEMV
 // that consumes the context merges the splits while it stages its input, so no merge launch follows.
 // Workgroups x, x + kvHeads, ... serve the query heads of KV head x: with eight KV heads the group shares
 // one L2, which then reads K and V from memory once.
-template <int HD, bool KV_F16, int U>
-__global__ __launch_bounds__(256) void attention_partial_kernel(AttentionArgs a) {
-    constexpr int WAVES = 4, LPT = HD / 8, SLOTS = 64 / LPT, KW = KV_F16 ? 1 : 2, STRIDE = HD + 4;
+template <int HD, bool KV_F16, int WAVES, int U>
+__global__ __launch_bounds__(WAVES * 64) void attention_partial_kernel(AttentionArgs a) {
+    constexpr int LPT = HD / 8, SLOTS = 64 / LPT, KW = KV_F16 ? 1 : 2, STRIDE = HD + 4;
     __shared__ float wm[WAVES], wl[WAVES][SLOTS];
     __shared__ float wacc[WAVES][SLOTS][HD];
     const int group = a.n_head / a.n_kv_head;
@@ -511,7 +512,7 @@ __global__ __launch_bounds__(256) void attention_partial_kernel(AttentionArgs a)
     __syncthreads();
     // ---- merge over wavefronts and slots in wavefront order: thread = channel ----
     float *ps = a.head_partials + (((size_t)m * a.n_head + head) * splits + split) * STRIDE;
-    for (int dch = tid; dch < HD; dch += 256) {
+    for (int dch = tid; dch < HD; dch += WAVES * 64) {
         float M = wm[0];
 #pragma unroll
         for (int w = 1; w < WAVES; w++) M = fmaxf(M, wm[w]);
@@ -715,8 +716,9 @@ int attention_head_splits(int) { return kAttentionHeadSplits; }
 hipError_t launch_attention_partials(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
     if (!a.head_partials || a.head_dim != 128 || a.n_head % a.n_kv_head != 0 || rows < 1 || rows > kMaxStepRows) return hipErrorInvalidValue;
     dim3 grid(a.n_head, rows, attention_head_splits(a.max_seq));
-    if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<128, true, 12>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((attention_partial_kernel<128, false, 6>), grid, dim3(256), 0, s, a);
+    constexpr int WAVES = 8;   // measured: 4 wavefronts x 12 chunks 6.2 us, 8 x 6 5.0 us, 16 x 3 4.7 us but a slower step
+    if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<128, true, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a);
+    else hipLaunchKernelGGL((attention_partial_kernel<128, false, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a);
     return hipGetLastError();
 }
 

@@ -430,7 +430,7 @@ struct Q4KStage {
 // of attention_merge_kernel (max of m, f = exp(m - M), L = fma(l, f, L), A = fma(acc, f, A), A / L), rounds the
 // context to fp16 and stages it like any other activation vector.  Row 0's loads are issued with issue();
 // further rows take one more round trip each inside finish().
-constexpr int kMergeSplits = 4, kMergeHeadDim = 128, kMergeStride = kMergeHeadDim + 4;
+constexpr int kMergeSplits = kAttentionHeadSplits, kMergeHeadDim = 128, kMergeStride = kMergeHeadDim + 4;
 template <int B, int IPR>
 struct Q4KMergeStage {
     static constexpr int GROUPS = IPR * 8, K = GROUPS / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1, HEADS = cols / kMergeHeadDim;
