@@ -495,6 +495,8 @@ struct Q4KMergeStage {
 // pairs it handles, and the loads of a team's next pair are issued before the arithmetic of the
 // current one, so weight traffic never waits for the arithmetic.  Every workgroup runs `iters`
 // rounds, so the barriers of the TEAM > 1 reduction line up even when the last round is ragged.
+constexpr int kDeferredRounds = 16;   // rounds whose team reductions wait for one barrier at the end of the kernel
+
 // MODE: 0 = fp16 activations as given, 1 = RMSNorm fused into the staging, 2 = attention partial states merged in the staging.
 template <int B, int IPR, int TEAM, int MODE>
 __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int iters) {
@@ -504,8 +506,8 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int it
     extern __shared__ uint4 smem_raw[];
     uint4 *xs4 = smem_raw;                                                       // [B][8][XSTRIDE] x 8 fp16
     float *xsum = reinterpret_cast<float *>(smem_raw + (size_t)B * 8 * XSTRIDE);  // [B][cols/32]
-    float *red = xsum + (size_t)B * (cols / 32);                                  // [2][kWaves][2 * B]
-    float *norm_red = red + 2 * kWaves * 2 * B;                                   // [B][kWaves]
+    float *red = xsum + (size_t)B * (cols / 32);                                  // [kDeferredRounds][kWaves][2 * B]
+    float *norm_red = red + kDeferredRounds * kWaves * 2 * B;                     // [B][kWaves]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tl = (wave % TEAM) * 64 + lane;
     const int n_teams = gridDim.x * TEAMS, npairs = (a.rows + 1) / 2;
@@ -528,7 +530,24 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int it
         }
     };
 
-    auto process = [&](const Q4KItem (&buf)[PASSES], int pair, int parity) {
+    // TEAM > 1: the partial sums of a round go to LDS.  With few rounds every round has its own slot and the
+    // wavefronts run all rounds without meeting; one barrier after the last round, then the first lanes of each
+    // team add the partial sums (wavefront order) and run the epilogues, one round per lane.  With more
+    // rounds than slots the team meets after every round (two slots, alternating).
+    const bool deferred = TEAM > 1 && iters <= kDeferredRounds;
+    auto team_sum = [&](const float *slot, float (&sa)[B], float (&sb)[B]) {
+        const int w0 = (wave / TEAM) * TEAM;   // first wavefront of the team
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+            float ta = slot[w0 * 2 * B + 2 * b], tb = slot[w0 * 2 * B + 2 * b + 1];
+#pragma unroll
+            for (int w = 1; w < TEAM; w++) { ta += slot[(w0 + w) * 2 * B + 2 * b]; tb += slot[(w0 + w) * 2 * B + 2 * b + 1]; }
+            sa[b] = ta;
+            sb[b] = tb;
+        }
+    };
+
+    auto process = [&](const Q4KItem (&buf)[PASSES], int pair, int round) {
         float acc_a[B], acc_b[B];
 #pragma unroll
         for (int b = 0; b < B; b++) acc_a[b] = acc_b[b] = 0.0f;
@@ -557,22 +576,15 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int it
         if constexpr (TEAM == 1) {
             if (pair < npairs && lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
         } else {
-            float *slot = red + (size_t)parity * kWaves * 2 * B;
+            float *slot = red + (size_t)(deferred ? round : (round & 1)) * kWaves * 2 * B;
             if (lane == 0) {
 #pragma unroll
                 for (int b = 0; b < B; b++) { slot[wave * 2 * B + 2 * b] = acc_a[b]; slot[wave * 2 * B + 2 * b + 1] = acc_b[b]; }
             }
+            if (deferred) return;
             __syncthreads();
             if (pair < npairs && tl == 0) {
-                const int w0 = wave;   // first wavefront of the team
-#pragma unroll
-                for (int b = 0; b < B; b++) {
-                    float sa = slot[w0 * 2 * B + 2 * b], sb = slot[w0 * 2 * B + 2 * b + 1];
-#pragma unroll
-                    for (int w = 1; w < TEAM; w++) { sa += slot[(w0 + w) * 2 * B + 2 * b]; sb += slot[(w0 + w) * 2 * B + 2 * b + 1]; }
-                    acc_a[b] = sa;
-                    acc_b[b] = sb;
-                }
+                team_sum(slot, acc_a, acc_b);
                 pair_epilogue<B>(a, pair, acc_a, acc_b);
             }
         }
@@ -580,7 +592,8 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int it
 
     Q4KItem buf0[PASSES], buf1[PASSES];
     typename std::conditional<MODE == 2, Q4KMergeStage<B, MODE == 2 ? IPR : 32>, Q4KStage<B, IPR, MODE == 1>>::type stage;
-    int pair = blockIdx.x * TEAMS + wave / TEAM;
+    const int first_pair = blockIdx.x * TEAMS + wave / TEAM;
+    int pair = first_pair;
     stage.issue(a);
     if (pair < npairs) load_pair(pair, buf0);
     stage.finish(a, xs4, xsum, norm_red);
@@ -588,13 +601,25 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int it
     for (int j = 0; j < iters; j += 2) {
         int next = pair + n_teams;
         if (next < npairs) load_pair(next, buf1);
-        process(buf0, pair, 0);
+        process(buf0, pair, j);
         pair = next;
         if (j + 1 < iters) {
             next = pair + n_teams;
             if (next < npairs) load_pair(next, buf0);
-            process(buf1, pair, 1);
+            process(buf1, pair, j + 1);
             pair = next;
+        }
+    }
+    if constexpr (TEAM > 1) {
+        if (deferred) {
+            __syncthreads();
+            const int round = tl;   // lane `round` of the team finishes that round's pair
+            const int p = first_pair + round * n_teams;
+            if (round < iters && p < npairs) {
+                float sa[B], sb[B];
+                team_sum(red + (size_t)round * kWaves * 2 * B, sa, sb);
+                pair_epilogue<B>(a, p, sa, sb);
+            }
         }
     }
 }
@@ -690,7 +715,7 @@ int compute_units() {
 template <int B, int IPR, int TEAM, int MODE>
 hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     constexpr int TEAMS = kWaves / TEAM;
-    const size_t lds = (size_t)B * 8 * (IPR | 1) * 16 + (size_t)B * (IPR * 2) * 4 + (size_t)(2 * kWaves * 2 * B + B * kWaves) * 4;
+    const size_t lds = (size_t)B * 8 * (IPR | 1) * 16 + (size_t)B * (IPR * 2) * 4 + (size_t)(kDeferredRounds * kWaves * 2 * B + B * kWaves) * 4;
     auto kernel = gemv_q4k_kernel<B, IPR, TEAM, MODE>;
     static size_t configured_lds = 0;
     hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
