@@ -75,8 +75,9 @@ struct GemvParams {
     float norm_eps = 0.0f;
     // attention context merged while staging: when merge_partials is set (see gemv_merges_attention_partials)
     // the activations are the per-head partial states of launch_attention_partials, merged and rounded to
-    // fp16; `x` and `norm_x` are ignored.  [batch][cols / 128][4][132] floats.
+    // fp16; `x` and `norm_x` are ignored.  [batch][cols / head_dim][kAttentionHeadSplits][head_dim + 4] floats.
     const float *merge_partials = nullptr;
+    int merge_head_dim = 0;
     float *y = nullptr;           // fp32 out [batch][rows]
     const float *residual = nullptr;
     uint16_t *out_f16 = nullptr;  // EPI_SWIGLU_F16: [batch][rows/2]
@@ -103,8 +104,8 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
 #define ESP_ATTENTION_HEAD_SPLITS 4
 #endif
 constexpr int kAttentionHeadSplits = ESP_ATTENTION_HEAD_SPLITS;
-// True when launch_gemv can take its input as attention partial states (Q4_K, 2048 or 4096 columns, batch <= 2).
-bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch);
+// True when launch_gemv can take its input as attention partial states (batch <= 2, head size 64 or 128).
+bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch, int head_dim);
 // kernels/gemm.hip
 hipError_t launch_gemm(const GemmParams &p, hipStream_t stream);
 // kernels/dequant.hip — GGUF-layout blocks -> fp32, bit-exact to the block definitions

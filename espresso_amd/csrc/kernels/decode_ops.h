@@ -55,7 +55,7 @@ hipError_t launch_rmsnorm(const float *x, const float *w, float eps, int rows, i
                           unsigned long long *argmax_cells, hipStream_t s);
 hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStream_t s);
 hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
-// Attention that stops at per-split partial states (head_dim 128, up to kMaxStepRows rows); the GEMV that reads
+// Attention that stops at per-split partial states (head_dim 64 or 128, up to kMaxStepRows rows); the GEMV that reads
 // the context merges them (GemvParams::merge_partials).  attention_head_splits: slices per query head.
 int attention_head_splits(int max_seq);
 hipError_t launch_attention_partials(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);

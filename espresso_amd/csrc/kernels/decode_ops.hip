@@ -714,11 +714,17 @@ hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipSt
 int attention_head_splits(int) { return kAttentionHeadSplits; }
 
 hipError_t launch_attention_partials(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
-    if (!a.head_partials || a.head_dim != 128 || a.n_head % a.n_kv_head != 0 || rows < 1 || rows > kMaxStepRows) return hipErrorInvalidValue;
+    if (!a.head_partials || (a.head_dim != 128 && a.head_dim != 64) || a.n_head % a.n_kv_head != 0 || rows < 1 || rows > kMaxStepRows)
+        return hipErrorInvalidValue;
     dim3 grid(a.n_head, rows, attention_head_splits(a.max_seq));
-    constexpr int WAVES = 8;   // measured: 4 wavefronts x 12 chunks 6.2 us, 8 x 6 5.0 us, 16 x 3 4.7 us but a slower step
-    if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<128, true, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a);
-    else hipLaunchKernelGGL((attention_partial_kernel<128, false, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a);
+    constexpr int WAVES = 8;   // measured at head size 128: 4 wavefronts x 12 chunks 6.2 us, 8 x 6 5.0 us, 16 x 3 4.7 us but a slower step
+    if (a.head_dim == 128) {
+        if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<128, true, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a);
+        else hipLaunchKernelGGL((attention_partial_kernel<128, false, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a);
+    } else {
+        if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<64, true, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a);
+        else hipLaunchKernelGGL((attention_partial_kernel<64, false, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a);
+    }
     return hipGetLastError();
 }
 

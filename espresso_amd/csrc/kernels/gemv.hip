@@ -89,9 +89,49 @@ struct KernelArgs {
     const float *norm_x, *norm_w;
     float norm_eps;
     // when merge_partials is set the activations are the attention context merged from per-split partial states
-    // while staging (x and norm_x unused): [batch][cols / 128 heads][kMergeSplits][128 values, m, l, 2 pad]
+    // while staging (x and norm_x unused): [batch][cols / head_dim heads][kMergeSplits][head_dim values, m, l, 2 pad]
     const float *merge_partials;
+    int merge_head_dim;
 };
+
+// ---- attention context merged from per-split partial states -------------------------------------------
+// The arithmetic of attention_merge_kernel: M = max m, f = exp(m - M) (0 for an empty split), L = fma(l, f, L),
+// A = fma(acc, f, A) in split order, context = A / L, rounded to fp16.  Eight channels of one query head.
+constexpr int kMergeSplits = kAttentionHeadSplits;
+__device__ __forceinline__ uint4 merge_group(const float2 (&ml)[kMergeSplits], const float4 (&a0)[kMergeSplits], const float4 (&a1)[kMergeSplits]) {
+    float M = ml[0].x;
+#pragma unroll
+    for (int sp = 1; sp < kMergeSplits; sp++) M = fmaxf(M, ml[sp].x);
+    float L = 0.0f, A[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sp = 0; sp < kMergeSplits; sp++) {
+        const float f = ml[sp].x != -INFINITY ? expf(ml[sp].x - M) : 0.0f;
+        L = __builtin_fmaf(ml[sp].y, f, L);
+        const float v[8] = {a0[sp].x, a0[sp].y, a0[sp].z, a0[sp].w, a1[sp].x, a1[sp].y, a1[sp].z, a1[sp].w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) A[i] = __builtin_fmaf(v[i], f, A[i]);
+    }
+    float c[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) c[i] = L > 0.0f ? A[i] / L : 0.0f;
+    uint4 h;
+    h.x = pack_half2(c[0], c[1]); h.y = pack_half2(c[2], c[3]); h.z = pack_half2(c[4], c[5]); h.w = pack_half2(c[6], c[7]);
+    return h;
+}
+// Loads of group g (eight channels) of row b; head size known at run time.
+__device__ __forceinline__ void merge_group_load(const KernelArgs &a, int b, int g, int cols, float2 (&ml)[kMergeSplits],
+                                                 float4 (&a0)[kMergeSplits], float4 (&a1)[kMergeSplits]) {
+    const int hd = a.merge_head_dim, stride = hd + 4, per_head = hd / 8;
+    const int head = g / per_head, d0 = (g - head * per_head) * 8;
+    const float *base = a.merge_partials + ((size_t)b * (cols / hd) + head) * kMergeSplits * stride;
+#pragma unroll
+    for (int sp = 0; sp < kMergeSplits; sp++) {
+        const float *ps = base + sp * stride;
+        a0[sp] = *reinterpret_cast<const float4 *>(ps + d0);
+        a1[sp] = *reinterpret_cast<const float4 *>(ps + d0 + 4);
+        ml[sp] = *reinterpret_cast<const float2 *>(ps + hd);
+    }
+}
 
 // 1 / sqrt(mean(x^2) + eps) of row b of norm_x (any cols that is a multiple of 8); `red` as above.
 __device__ __forceinline__ float row_inverse_rms(const KernelArgs &a, int b, int cols, float *red) {
@@ -102,6 +142,12 @@ __device__ __forceinline__ float row_inverse_rms(const KernelArgs &a, int b, int
 }
 // Group g (eight consecutive elements) of row b of the activations, as fp16.
 __device__ __forceinline__ uint4 activation_group(const KernelArgs &a, int b, int g, int cols, float inv) {
+    if (a.merge_partials) {
+        float2 ml[kMergeSplits];
+        float4 a0[kMergeSplits], a1[kMergeSplits];
+        merge_group_load(a, b, g, cols, ml, a0, a1);
+        return merge_group(ml, a0, a1);
+    }
     if (!a.norm_x) return reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + g];
     const float4 *x4 = reinterpret_cast<const float4 *>(a.norm_x + (size_t)b * cols);
     const float4 *w4 = reinterpret_cast<const float4 *>(a.norm_w);
@@ -425,57 +471,23 @@ struct Q4KStage {
     }
 };
 
-// Staging for a GEMV whose input is the attention context (head size 128): merges the kMergeSplits partial
-// states (m, l, acc) that attention_partial_kernel left per query head, in split order and with the arithmetic
-// of attention_merge_kernel (max of m, f = exp(m - M), L = fma(l, f, L), A = fma(acc, f, A), A / L), rounds the
-// context to fp16 and stages it like any other activation vector.  Row 0's loads are issued with issue();
-// further rows take one more round trip each inside finish().
-constexpr int kMergeSplits = kAttentionHeadSplits, kMergeHeadDim = 128, kMergeStride = kMergeHeadDim + 4;
+// Staging of the persistent kernel when its input is the attention context left as partial states (merge_group
+// above).  Row 0's loads are issued with issue(), before the first weight loads; further rows take one more
+// round trip each inside finish().
 template <int B, int IPR>
 struct Q4KMergeStage {
-    static constexpr int GROUPS = IPR * 8, K = GROUPS / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1, HEADS = cols / kMergeHeadDim;
-    static_assert(GROUPS % kThreads == 0 && cols % kMergeHeadDim == 0, "whole groups per thread, whole heads per row");
+    static constexpr int GROUPS = IPR * 8, K = GROUPS / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1;
+    static_assert(GROUPS % kThreads == 0, "whole groups per thread");
     float4 a0[K][kMergeSplits], a1[K][kMergeSplits];
     float2 ml[K][kMergeSplits];
 
     __device__ __forceinline__ void load_row(const KernelArgs &a, int b) {
-        const int tid = threadIdx.x;
 #pragma unroll
-        for (int k = 0; k < K; k++) {
-            const int g = tid + k * kThreads, head = g / (kMergeHeadDim / 8), d0 = (g % (kMergeHeadDim / 8)) * 8;
-            const float *base = a.merge_partials + ((size_t)b * HEADS + head) * kMergeSplits * kMergeStride;
-#pragma unroll
-            for (int sp = 0; sp < kMergeSplits; sp++) {
-                const float *ps = base + sp * kMergeStride;
-                a0[k][sp] = *reinterpret_cast<const float4 *>(ps + d0);
-                a1[k][sp] = *reinterpret_cast<const float4 *>(ps + d0 + 4);
-                ml[k][sp] = *reinterpret_cast<const float2 *>(ps + kMergeHeadDim);
-            }
-        }
+        for (int k = 0; k < K; k++) merge_group_load(a, b, threadIdx.x + k * kThreads, cols, ml[k], a0[k], a1[k]);
     }
     __device__ __forceinline__ void store_row(int b, uint4 *xs4, float *xsum) {
-        const int tid = threadIdx.x;
 #pragma unroll
-        for (int k = 0; k < K; k++) {
-            float M = ml[k][0].x;
-#pragma unroll
-            for (int sp = 1; sp < kMergeSplits; sp++) M = fmaxf(M, ml[k][sp].x);
-            float L = 0.0f, A[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int sp = 0; sp < kMergeSplits; sp++) {
-                const float f = ml[k][sp].x != -INFINITY ? expf(ml[k][sp].x - M) : 0.0f;
-                L = __builtin_fmaf(ml[k][sp].y, f, L);
-                const float v[8] = {a0[k][sp].x, a0[k][sp].y, a0[k][sp].z, a0[k][sp].w, a1[k][sp].x, a1[k][sp].y, a1[k][sp].z, a1[k][sp].w};
-#pragma unroll
-                for (int i = 0; i < 8; i++) A[i] = __builtin_fmaf(v[i], f, A[i]);
-            }
-            float c[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++) c[i] = L > 0.0f ? A[i] / L : 0.0f;
-            uint4 h;
-            h.x = pack_half2(c[0], c[1]); h.y = pack_half2(c[2], c[3]); h.z = pack_half2(c[4], c[5]); h.w = pack_half2(c[6], c[7]);
-            q4k_store_group(h, b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
-        }
+        for (int k = 0; k < K; k++) q4k_store_group(merge_group(ml[k], a0[k], a1[k]), b, threadIdx.x + k * kThreads, cols, XSTRIDE, xs4, xsum);
     }
     __device__ __forceinline__ void issue(const KernelArgs &a) { load_row(a, 0); }
     __device__ __forceinline__ void finish(const KernelArgs &a, uint4 *xs4, float *xsum, float *) {
@@ -744,12 +756,9 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
 template <int B>
 hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     const bool norm = a.norm_x != nullptr;
-    if (a.merge_partials) {   // launch_gemv has checked the width
-        if (a.cols == 2048) return launch_q4k_persistent<B, 32, 1, 2>(a, stream);
-        if (a.cols == 4096) return launch_q4k_persistent<B, 64, 1, 2>(a, stream);
-        return hipErrorInvalidValue;
-    }
-    switch (a.cols) {
+    if (a.merge_partials && a.cols == 2048) return launch_q4k_persistent<B, 32, 1, 2>(a, stream);
+    if (a.merge_partials && a.cols == 4096) return launch_q4k_persistent<B, 64, 1, 2>(a, stream);
+    if (!a.merge_partials) switch (a.cols) {
     case 2048: return norm ? launch_q4k_persistent<B, 32, 1, 1>(a, stream) : launch_q4k_persistent<B, 32, 1, 0>(a, stream);
     case 4096: return norm ? launch_q4k_persistent<B, 64, 1, 1>(a, stream) : launch_q4k_persistent<B, 64, 1, 0>(a, stream);
     case 8192: return norm ? launch_q4k_persistent<B, 128, 2, 1>(a, stream) : launch_q4k_persistent<B, 128, 2, 0>(a, stream);
@@ -795,14 +804,17 @@ hipError_t launch_fmt(const KernelArgs &a, int batch, hipStream_t stream) {
 
 }  // namespace
 
-bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch) {
-    return w.format == FMT_Q4_K && (w.cols == 2048 || w.cols == 4096) && batch >= 1 && batch <= 2;
+bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch, int head_dim) {
+    if (batch < 1 || batch > 2 || (head_dim != 64 && head_dim != 128) || w.cols % head_dim != 0) return false;
+    // the persistent Q4_K instantiations for the wider inputs have no merging form
+    if (w.format == FMT_Q4_K && (w.cols == 8192 || w.cols == 11008 || w.cols == 14336)) return false;
+    return true;
 }
 
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     const DeviceMatrix &w = p.w;
     if (!w.qs || (!p.x && !p.norm_x && !p.merge_partials) || (p.norm_x && !p.norm_w) || w.rows <= 0 || w.cols <= 0 || p.batch <= 0) return hipErrorInvalidValue;
-    if (p.merge_partials && !gemv_merges_attention_partials(w, p.batch)) return hipErrorInvalidValue;
+    if (p.merge_partials && !gemv_merges_attention_partials(w, p.batch, p.merge_head_dim)) return hipErrorInvalidValue;
     if ((p.epilogue == EPI_STORE_F32 || p.epilogue == EPI_ADD_RESIDUAL) && !p.y) return hipErrorInvalidValue;
     if (p.epilogue == EPI_ADD_RESIDUAL && !p.residual) return hipErrorInvalidValue;
     if (p.epilogue == EPI_SWIGLU_F16 && (!p.out_f16 || w.rows % 2 != 0)) return hipErrorInvalidValue;
@@ -823,6 +835,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         a.qs = w.qs; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.rows = w.rows; a.cols = w.cols;
         a.x = p.x ? p.x + (size_t)b0 * w.cols : nullptr;
         a.merge_partials = p.merge_partials;   // batch <= 2 here: one launch
+        a.merge_head_dim = p.merge_head_dim;
         a.y = p.y ? p.y + (size_t)b0 * w.rows : nullptr;
         a.residual = p.residual ? p.residual + (size_t)b0 * w.rows : nullptr;
         a.out_f16 = p.out_f16 ? p.out_f16 + (size_t)b0 * (w.rows / 2) : nullptr;

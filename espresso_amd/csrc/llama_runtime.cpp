@@ -131,8 +131,8 @@ int LlamaRuntime::collect_kernel_times(double total_us[K_CLASS_COUNT], long laun
 // the wo GEMV merges them while staging, when the head size and the matrix allow it.  The fused trunk keeps the
 // split-and-merge arithmetic it is compared with.
 bool LlamaRuntime::wo_merges_attention(const Layer &L, int rows) const {
-    return merged_attention_ && !fused_trunk_active() && c_.head_dim == 128 && c_.n_head % c_.n_kv_head == 0 && rows <= 2 &&
-           L.wo.cols == c_.attention_dim() && gemv_merges_attention_partials(L.wo, rows);
+    return merged_attention_ && !fused_trunk_active() && c_.n_head % c_.n_kv_head == 0 && rows <= 2 &&
+           L.wo.cols == c_.attention_dim() && gemv_merges_attention_partials(L.wo, rows, c_.head_dim);
 }
 
 int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us) {
@@ -155,7 +155,7 @@ int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us
             break;
         case K_WO:
             g.w = L->wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
-            if (wo_merges_attention(*L, 1)) { g.x = nullptr; g.merge_partials = attn_scratch_; }
+            if (wo_merges_attention(*L, 1)) { g.x = nullptr; g.merge_partials = attn_scratch_; g.merge_head_dim = c_.head_dim; }
             break;
         case K_GATE_UP:
             g.w = L->w13; g.norm_x = hidden_; g.norm_w = L->rms_ffn; g.norm_eps = c_.norm_eps; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
@@ -507,7 +507,7 @@ int LlamaRuntime::enqueue_trunk(int M) {
         g = GemvParams{};
         g.batch = M;
         g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
-        if (merge_in_wo) { g.x = nullptr; g.merge_partials = attn_scratch_; }
+        if (merge_in_wo) { g.x = nullptr; g.merge_partials = attn_scratch_; g.merge_head_dim = c_.head_dim; }
         if ((rc = time_begin(K_WO)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;

@@ -316,6 +316,25 @@ def test_attention_merged_in_the_wo_gemv(llama, kv_fp16):
     _, draft = make_pair(llama, dict(MERGED, n_layer=1), orc.FMT_Q4_K, seed=78, std=0.04, kv_fp16=kv_fp16)
     got, st = llama.generate_two_token(g, draft, long_prompt[:40], 30)
     assert got == g.generate(long_prompt[:40], 30)[0]
-    # models whose shapes do not qualify keep the two-kernel form
-    _, tiny = make_pair(llama, TINY, orc.FMT_Q4_K, seed=3)
-    assert not llama.set_merged_attention(tiny, True)
+    # a head size outside {64, 128} keeps the two-kernel form
+    _, odd = make_pair(llama, dict(TINY, n_head=8, n_kv_head=8, head_dim=32), orc.FMT_Q4_K, seed=3)
+    assert not llama.set_merged_attention(odd, True)
+
+
+@pytest.mark.parametrize("fmt", [orc.FMT_Q8_0, orc.FMT_Q4_0, orc.FMT_Q4_K, orc.FMT_F16])
+def test_attention_merged_in_the_wo_gemv_head_size_64(llama, fmt):
+    """Head size 64 and every weight format: the general GEMV kernels merge the partial states too."""
+    kw = dict(n_layer=2, n_head=12, n_kv_head=12, d_model=768, head_dim=64, hidden_dim=512, vocab=512, max_seq=200)
+    o, g = make_pair(llama, kw, fmt, seed=90 + fmt, std=0.05, norm_jitter=0.05)
+    assert llama.set_merged_attention(g, True)
+    prompt = np.random.default_rng(6).integers(0, 512, 150).tolist()
+    o.prefill(prompt[:24]); g.prefill(prompt[:24])
+    for step in range(5):
+        assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
+        tok = o.select_greedy()
+        if o.top2_margin() > 1e-3:
+            assert g.select_greedy() == tok
+        o.advance(tok); g.advance(tok)
+    merged = g.generate(prompt, 30)[0]
+    llama.set_merged_attention(g, False)
+    assert g.generate(prompt, 30)[0] == merged
