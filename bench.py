@@ -139,9 +139,9 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
 
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# workload (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors a 256 MiB copy kernel gave);
+# workload (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors kernels of known size in the same runs gave);
 # the runs and the per-kernel table are in profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt.
-MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66578534}
+MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66569318}
 
 
 # BASELINE.json configs[2]: weight-GEMV microbenchmark at the Llama-3-8B layer shapes
