@@ -744,9 +744,11 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     const int npairs = (a.rows + 1) / 2;
     const int want = (npairs + TEAMS - 1) / TEAMS;            // one round
     const int cap = compute_units() * resident_per_cu;
-    int grid = want < cap ? want : cap;
+    const int grid = want < cap ? want : cap;
+    // The last round is ragged and goes to the workgroups with the lowest indices.  Those are dispatched first and
+    // get their first weights first (the memory system serves the opening burst roughly in order), and they stay
+    // ahead by one to three microseconds to the end: one pair less for the later workgroups evens the finish.
     const int iters = (npairs + grid * TEAMS - 1) / (grid * TEAMS);
-    grid = (npairs + iters * TEAMS - 1) / (iters * TEAMS);    // same rounds, no idle workgroups
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, iters);
     return hipGetLastError();
 }
