@@ -744,7 +744,11 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     const int npairs = (a.rows + 1) / 2;
     const int want = (npairs + TEAMS - 1) / TEAMS;            // one round
     const int cap = compute_units() * resident_per_cu;
-    const int grid = want < cap ? want : cap;
+    int grid = want < cap ? want : cap;
+    // Just one round with every slot of the chip taken (the 8B q|k|v matrix) is slower than a round and a half at
+    // one workgroup fewer per compute unit: 5.9 against 5.4 us; grids that are not whole multiples of the compute
+    // units lose more than that (6.3-6.9 us).
+    if (resident_per_cu >= 3 && want > cap - compute_units() && want <= cap) grid = cap - compute_units();
     // The last round is ragged and goes to the workgroups with the lowest indices.  Those are dispatched first and
     // get their first weights first (the memory system serves the opening burst roughly in order), and they stay
     // ahead by one to three microseconds to the end: one pair less for the later workgroups evens the finish.
