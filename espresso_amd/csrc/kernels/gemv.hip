@@ -8,8 +8,9 @@
 //     of consecutive rows at a time - a RoPE pair or a (gate, up) pair, so the epilogues stay in registers;
 //   * a lane's unit of work ("item") is built from aligned 128-bit loads of packed weights; consecutive lanes read
 //     consecutive pieces of the row, so a wavefront load covers 1 KiB+ of contiguous HBM;
-//   * the activations are staged once per workgroup in LDS as fp16 - copied, or computed on the spot as
-//     fp16((x * inv_rms) * w) from the fp32 residual stream (fused RMSNorm).  For the integer formats they are stored
+//   * the activations are staged once per workgroup in LDS as fp16 - copied, computed on the spot as
+//     fp16((x * inv_rms) * w) from the fp32 residual stream (fused RMSNorm), or merged from the partial softmax
+//     states the attention kernel left per query head (the wo GEMV).  For the integer formats they are stored
 //     with the two middle elements of every group of four swapped, (x0,x2,x1,x3): masking a weight dword with
 //     0x000F000F / 0x00FF00FF yields elements 0 and 2 of a group, so the matching activation pair is one LDS dword;
 //   * nibbles / bytes become exact fp16 values with exponent tricks (Q4_0, Q8_0: 0x6400 | n = 1024 + n, then an
@@ -22,6 +23,10 @@
 //
 // HBM traffic per launch = packed weight bytes + batch*cols*2 (x) + batch*rows*4 (y): measured 1.006x the
 // algorithmic bytes; x is re-read from L2 once per workgroup.
+//
+// The Q4_K kernels for the llama family's widths are persistent: the grid is what the chip holds at once, teams
+// take row pairs round by round with the next pair's loads in flight, and the ragged last round goes to the
+// workgroups that were dispatched first (they get their first weights first and stay ahead).
 #include <cstdlib>
 
 #include <type_traits>
