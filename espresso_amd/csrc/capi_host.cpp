@@ -5,6 +5,7 @@
 #include "generation.h"
 #include "host/engine.h"
 #include "host/gguf.h"
+#include "host/bundle.h"
 #include "host/harness.h"
 #include "host/tokenizer.h"
 
@@ -293,6 +294,109 @@ long esp_tokenizer_decode(const ESPTokenizer *tokenizer, const int32_t *tokens, 
     const std::string text = tokenizer->impl->decode(std::vector<int>(tokens, tokens + count));
     if (out_utf8 && capacity) std::memcpy(out_utf8, text.data(), std::min(capacity, text.size()));
     return (long)text.size();
+}
+
+// ---- bundles ---------------------------------------------------------------------------------------------
+struct ESPBundle { ESPRuntimeBundle bundle; };
+
+namespace {
+thread_local ESPBundleError g_bundle_error = {};
+
+int bundle_status(const BundleStatus &st) {
+    g_bundle_error = ESPBundleError{};
+    g_bundle_error.code = (int32_t)st.error;
+    g_bundle_error.detail = st.detail;
+    g_bundle_error.detail2 = st.detail2;
+    std::strncpy(g_bundle_error.text, st.text.c_str(), sizeof(g_bundle_error.text) - 1);
+    if (st.ok()) return ESP_OK;
+    return fail(ESP_ERR_INVALID_ARGUMENT, "bundle error %d (%ld, %ld) %s", (int)st.error, st.detail, st.detail2, st.text.c_str());
+}
+
+void fill_selection(const ESPRuntimeSelection &s, ESPRuntimeSelectionInfo *out) {
+    std::memset(out, 0, sizeof(*out));
+    std::strncpy(out->backend, s.backend.c_str(), sizeof(out->backend) - 1);
+    std::strncpy(out->profile, s.profile.c_str(), sizeof(out->profile) - 1);
+    std::strncpy(out->reason, s.reason.c_str(), sizeof(out->reason) - 1);
+    out->context_target_tokens = s.contextTargetTokens;
+    out->has_output_head = s.hasOutputHead ? 1 : 0;
+    out->has_draft = s.hasDraft ? 1 : 0;
+}
+}  // namespace
+
+void esp_bundle_last_error(ESPBundleError *out) { if (out) *out = g_bundle_error; }
+
+int esp_manifest_parse_toml(const char *text, size_t text_bytes, char *out_toml, size_t capacity, size_t *out_bytes) {
+    if (!text && text_bytes) return fail(ESP_ERR_INVALID_ARGUMENT, "null manifest text");
+    ESPManifest m;
+    int rc = bundle_status(ESPManifest::parseTOML(std::string(text ? text : "", text_bytes), &m));
+    if (rc != ESP_OK) return rc;
+    const std::string rendered = m.renderTOML();
+    if (out_bytes) *out_bytes = rendered.size();
+    if (out_toml && capacity) std::memcpy(out_toml, rendered.data(), std::min(capacity, rendered.size()));
+    return ESP_OK;
+}
+
+int esp_bundle_write_signature_catalog(const char *bundle_dir) {
+    if (!bundle_dir) return fail(ESP_ERR_INVALID_ARGUMENT, "null bundle directory");
+    ESPBundleArchive a;
+    a.bundleDir = bundle_dir;
+    return bundle_status(a.writeSignatureCatalog());
+}
+
+ESPBundle *esp_bundle_open(const char *bundle_dir, int verify_signatures) {
+    if (!bundle_dir) { fail(ESP_ERR_INVALID_ARGUMENT, "null bundle directory"); return nullptr; }
+    std::unique_ptr<ESPBundle> b(new ESPBundle());
+    if (bundle_status(ESPRuntimeBundle::open(bundle_dir, verify_signatures != 0, &b->bundle)) != ESP_OK) return nullptr;
+    return b.release();
+}
+
+void esp_bundle_free(ESPBundle *bundle) { delete bundle; }
+
+int esp_bundle_model_config(const ESPBundle *bundle, ESPModelConfig *out) {
+    if (!bundle || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "null bundle or config");
+    to_c(bundle->bundle.config, out);
+    return ESP_OK;
+}
+
+int esp_bundle_resolve(const ESPBundle *bundle, long requested_context_tokens, int supports_ane_private, ESPRuntimeSelectionInfo *out) {
+    if (!bundle || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "null bundle or selection");
+    ESPRuntimeSelection s;
+    int rc = bundle_status(selectBackend(supports_ane_private != 0, bundle->bundle.archive.manifest, requested_context_tokens, &s));
+    if (rc != ESP_OK) return rc;
+    fill_selection(s, out);
+    return ESP_OK;
+}
+
+long esp_bundle_environment_overrides(const ESPBundle *bundle, long requested_context_tokens, int supports_ane_private, char *out,
+                                      size_t capacity) {
+    if (!bundle) return fail(ESP_ERR_INVALID_ARGUMENT, "null bundle");
+    ESPRuntimeSelection s;
+    int rc = bundle_status(selectBackend(supports_ane_private != 0, bundle->bundle.archive.manifest, requested_context_tokens, &s));
+    if (rc != ESP_OK) return rc;
+    std::string text;
+    for (const auto &kv : environmentOverrides(s)) text += kv.first + "=" + kv.second + "\n";
+    if (out && capacity) std::memcpy(out, text.data(), std::min(capacity, text.size()));
+    return (long)text.size();
+}
+
+int esp_bundle_generate(const ESPBundle *bundle, const char *prompt_utf8, size_t prompt_bytes, int max_tokens, float temperature,
+                        const char *const *env_keys, const char *const *env_values, int env_count, uint32_t *out_tokens,
+                        char *out_text, size_t text_capacity, size_t *out_text_bytes, ESPGenerationResult *result,
+                        ESPRuntimeSelectionInfo *selection) {
+    if (!bundle || (!prompt_utf8 && prompt_bytes)) return fail(ESP_ERR_INVALID_ARGUMENT, "null bundle or prompt");
+    GenerationResult r;
+    ESPRuntimeSelection sel;
+    BundleStatus st;
+    int rc = bundle->bundle.generate(std::string(prompt_utf8 ? prompt_utf8 : "", prompt_bytes), max_tokens, temperature,
+                                     env_from(env_keys, env_values, env_count), &r, &sel, &st);
+    if (!st.ok()) return bundle_status(st);
+    if (rc != ESP_OK) return rc;
+    if (selection) fill_selection(sel, selection);
+    if (out_tokens) for (size_t i = 0; i < r.tokens.size(); i++) out_tokens[i] = r.tokens[i];
+    if (out_text_bytes) *out_text_bytes = r.text.size();
+    if (out_text && text_capacity) std::memcpy(out_text, r.text.data(), std::min(text_capacity, r.text.size()));
+    if (result) fill_result(r, result);
+    return ESP_OK;
 }
 
 void esp_exact_two_token_promotion_plan(uint32_t current_token, uint32_t proposed_future_token, uint32_t exact_next_token,

@@ -391,6 +391,60 @@ long esp_pretokenize(const char *pattern_utf8, const char *text_utf8, size_t tex
 /* Returns the UTF-8 length of the decoded text and writes its first `capacity` bytes (not terminated). */
 long esp_tokenizer_decode(const ESPTokenizer *tokenizer, const int32_t *tokens, size_t count, char *out_utf8, size_t capacity);
 
+/* ---- .esp bundles ---------------------------------------------------------------------------------- *
+ * The bridge from a bundle to the engine: ESPBundleArchive.open (Sources/ESPBundle/ESPBundle.swift:563-590: the
+ * manifest, the ten top-level directories, the SHA-256 catalog signatures/content-hashes.json, referenced artefacts),
+ * ESPManifest.parseTOML / validate / renderTOML (:219-394), ESPRuntimeResolver.selectBackend
+ * (Sources/ESPRuntime/ESPRuntimeContracts.swift:77-138) and ESPRuntimeRunner.generate with environmentOverrides
+ * (Sources/ESPRuntime/ESPBundledRuntime.swift:49-180): a [draft] section selects the exact two-token path, an
+ * [output_head] section is passed on in the environment (the engine here always runs the dense head).
+ * Both of the reference's backends ("ane-private", "cpu-safe") run the same GPU engine here.
+ * Loaders return NULL / negative on failure; esp_bundle_last_error then holds the case of
+ * ESPBundleValidationError or ESPRuntimeSelectionError (this thread's last call). */
+typedef struct ESPBundle ESPBundle;
+enum {
+    ESP_BUNDLE_OK = 0, ESP_BUNDLE_EMPTY_FIELD = 1, ESP_BUNDLE_INVALID_MAX_CONTEXT = 2, ESP_BUNDLE_INVALID_CONTEXT_TARGET = 3,
+    ESP_BUNDLE_INVALID_ADAPTER_SLOTS = 4, ESP_BUNDLE_MISSING_BACKENDS = 5, ESP_BUNDLE_MISSING_PROFILES = 6,
+    ESP_BUNDLE_INVALID_WEIGHT_BITS = 7, ESP_BUNDLE_INVALID_ACTIVATION_BITS = 8, ESP_BUNDLE_MISSING_TOP_LEVEL_ENTRY = 9,
+    ESP_BUNDLE_MISSING_MANIFEST = 10, ESP_BUNDLE_MALFORMED_LINE = 11, ESP_BUNDLE_MALFORMED_SECTION = 12,
+    ESP_BUNDLE_UNSUPPORTED_VALUE = 13, ESP_BUNDLE_INVALID_OUTPUT_HEAD = 14, ESP_BUNDLE_INVALID_DRAFT = 15,
+    ESP_BUNDLE_INVALID_REFERENCED_PATH = 16, ESP_BUNDLE_MISSING_REFERENCED_FILE = 17, ESP_BUNDLE_SIGNATURE_MISMATCH = 18,
+    ESP_BUNDLE_UNREADABLE_FILE = 19, ESP_BUNDLE_NO_COMPATIBLE_BACKEND = 30, ESP_BUNDLE_NO_COMPATIBLE_PROFILE = 31,
+    ESP_BUNDLE_REQUESTED_CONTEXT_EXCEEDS_TARGET = 32   /* detail = requested, detail2 = supported */
+};
+typedef struct ESPBundleError {
+    int32_t code;
+    int64_t detail, detail2;
+    char text[256];
+} ESPBundleError;
+typedef struct ESPRuntimeSelectionInfo {   /* ESPRuntimeSelection (ESPRuntimeContracts.swift:43-69) */
+    char backend[16];                      /* "ane-private" | "cpu-safe" */
+    char profile[16];                      /* "prefill_256" | "prefill_2048" | "decode_1" | "decode_2" */
+    int64_t context_target_tokens;
+    int32_t has_output_head, has_draft;
+    char reason[64];
+} ESPRuntimeSelectionInfo;
+void esp_bundle_last_error(ESPBundleError *out);
+/* ESPManifest.parseTOML(text) then renderTOML(): 0 and the canonical text (its length in *out_bytes, the first
+ * `capacity` bytes written), or ESP_ERR_INVALID_ARGUMENT with esp_bundle_last_error set. */
+int esp_manifest_parse_toml(const char *text, size_t text_bytes, char *out_toml, size_t capacity, size_t *out_bytes);
+/* ESPBundleArchive.writeSignatureCatalog for a bundle directory. */
+int esp_bundle_write_signature_catalog(const char *bundle_dir);
+/* ESPRuntimeBundle.open(at:) (ESPBundledRuntime.swift:17-23): archive + config from weights/metadata.json. */
+ESPBundle *esp_bundle_open(const char *bundle_dir, int verify_signatures);
+void esp_bundle_free(ESPBundle *bundle);
+int esp_bundle_model_config(const ESPBundle *bundle, ESPModelConfig *out);
+/* selectBackend; requested_context_tokens < 0 = none.  supports_ane_private mirrors ESPDeviceCapabilities. */
+int esp_bundle_resolve(const ESPBundle *bundle, long requested_context_tokens, int supports_ane_private, ESPRuntimeSelectionInfo *out);
+/* environmentOverrides(for:) of that selection as "KEY=VALUE\n" lines; returns the text length. */
+long esp_bundle_environment_overrides(const ESPBundle *bundle, long requested_context_tokens, int supports_ane_private, char *out,
+                                      size_t capacity);
+/* ESPRuntimeRunner.generate(bundle:prompt:maxTokens:temperature:); outputs as esp_engine_generate_text. */
+int esp_bundle_generate(const ESPBundle *bundle, const char *prompt_utf8, size_t prompt_bytes, int max_tokens, float temperature,
+                        const char *const *env_keys, const char *const *env_values, int env_count, uint32_t *out_tokens,
+                        char *out_text, size_t text_capacity, size_t *out_text_bytes, ESPGenerationResult *result,
+                        ESPRuntimeSelectionInfo *selection);
+
 /* sampleToken (RealModelInferenceEngine.swift:8036-8068) on the host: temperature <= 0 -> first maximum; else
  * weights exp(double((logit - max) / T)), threshold = unit * total, first index whose running remainder is <= 0.
  * `unit` in [0, 1) stands for Double.random(in: 0..<total) / total; esp_splitmix64_unit draws it from a SplitMix64

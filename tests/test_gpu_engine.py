@@ -368,3 +368,78 @@ def test_engine_generates_from_prompt_text(E, tmp_path):
     empty.mkdir()
     with pytest.raises(lib.EspressoError, match="missing path"):
         E.RealModelInferenceEngine(gpu_cfg(KW), str(weights), tokenizer_dir=str(empty))
+
+
+def test_bundle_selects_the_exact_two_token_path(E, tmp_path):
+    """ESPRuntimeRunner.generate (ESPBundledRuntime.swift:49-80): the bundle's [draft] section reaches the engine as
+    ESPRESSO_BUNDLE_DRAFT_* and the text comes from the bundle's tokenizer."""
+    import struct
+
+    import espresso_amd.bundle as B
+    import espresso_amd.tokenizer as T
+    root = tmp_path / "model.esp"
+    for entry in B.REQUIRED_TOP_LEVEL_ENTRIES:
+        os.makedirs(root / entry)
+    full_kw, draft_kw = dict(KW, n_layer=3), dict(KW, n_layer=1)
+    seen_f = write_weight_dir(str(root / "weights"), full_kw, mu.random_weights(orc.LlamaConfig(**full_kw), 61, std=0.08))
+    seen_d = write_weight_dir(str(root / "weights" / "draft"), draft_kw, mu.random_weights(orc.LlamaConfig(**draft_kw), 62, std=0.08))
+    (root / "weights" / "draft.json").write_text(json.dumps({"model_dir": "draft", "tokenizer_dir": None, "model_id": "d"}))
+    pieces = [("▁", 0.0)] + [(chr(97 + i), 0.0) for i in range(26)] + [("▁the", 2.0), ("▁t", 1.0), ("▁th", 1.5)] + [(f"<0x{b:02X}>", 0.0) for b in range(256)]
+    pieces += [(f"zz{i}", 0.0) for i in range(KW["vocab"] - len(pieces))]
+    data = struct.pack("<i", 16)
+    for piece, score in pieces:
+        raw = piece.encode()
+        data += struct.pack("<fi", score, len(raw)) + raw
+    (root / "tokenizer" / "tokenizer.model").write_bytes(data)
+
+    def manifest(draft_class="exact", target=40):
+        return f"""format_version = "1.1.0"
+model_id = "tiny.llama"
+model_family = "llama"
+architecture_version = "decoder-v1"
+tokenizer_contract = "sentencepiece-v1"
+supported_backends = ["ane-private", "cpu-safe"]
+supported_profiles = ["prefill_256", "decode_1"]
+max_context = {KW['max_seq']}
+context_target_tokens = {target}
+adapter_slots = 0
+accuracy_baseline_ref = "benchmarks/accuracy.json"
+performance_baseline_ref = "benchmarks/perf.json"
+signature_ref = "signatures/content-hashes.json"
+[compression_policy]
+name = "fp16"
+weight_bits = 16
+[draft]
+kind = "exact_two_token"
+behavior_class = "{draft_class}"
+horizon = 2
+verifier = "exact"
+rollback = "exact_replay"
+artifact_ref = "weights/draft.json"
+acceptance_metric = "accepted_future_tokens"
+"""
+    (root / "manifest.toml").write_text(manifest())
+    B.write_signature_catalog(str(root))
+    b = B.RuntimeBundle(str(root))
+    prompt = "the cat"
+    ids = T.Tokenizer.from_dir(gpu_cfg(full_kw), str(root / "tokenizer")).encode(prompt)
+    text, toks, res, sel = b.generate(prompt, 20)
+    of = mu.load_oracle(orc.LlamaConfig(gemv_inputs_fp16=True, **full_kw), seen_f)
+    od = mu.load_oracle(orc.LlamaConfig(gemv_inputs_fp16=True, **draft_kw), seen_d)
+    want, st = orc.generate_two_token(of, od, ids, 20)
+    assert toks == want
+    assert res["exact_head_backend"] == "hip_exact_two_token_draft" and res["has_two_token_stats"] == 1
+    assert res["accepted_future_tokens_per_pass"] == pytest.approx(st["accepted_total"] / st["passes"])
+    assert sel["backend"] == "ane-private" and sel["has_draft"]
+    assert text.startswith(prompt)
+    # host without the private backend: the other backend, the same engine, the same tokens
+    assert b.generate(prompt, 20, environment={"ESPRESSO_DISABLE_ANE_PRIVATE": "1"})[3]["backend"] == "cpu-safe"
+    # prompt + maxTokens beyond the bundle's context target is refused before the model is built (ESPRuntimeResolverTests.swift:267-326)
+    with pytest.raises(B.BundleError) as e:
+        b.generate(prompt, 40)
+    assert (e.value.case, e.value.detail, e.value.detail2) == ("requestedContextExceedsTarget", len(ids) + 40, 40)
+    b.close()
+    # an approximate draft is not passed on: plain greedy
+    (root / "manifest.toml").write_text(manifest(draft_class="approximate"))
+    text2, toks2, res2, _ = B.RuntimeBundle(str(root), verify_signatures=False).generate(prompt, 20)
+    assert res2["exact_head_backend"] == "hip_gemv_argmax" and toks2 == toks and text2 == text
