@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libespresso_hip.so")
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wall", "-Wno-unused-function",
 ]
 

@@ -427,17 +427,28 @@ __global__ __launch_bounds__(HD) void attention_merge_kernel(AttentionArgs a, in
 // Workgroups x, x + kvHeads, ... serve the query heads of KV head x: with eight KV heads the group shares
 // one L2, which then reads K and V from memory once.
 template <int HD, bool KV_F16, int WAVES, int U>
-__global__ __launch_bounds__(WAVES * 64) void attention_partial_kernel(AttentionArgs a) {
+__global__ __launch_bounds__(WAVES * 64) void attention_partial_kernel(const float *q_rows, const void *k_cache, const void *v_cache, const int *pos,
+                                                                       const int *seq, float *head_partials, unsigned cache_seq_stride, unsigned heads) {
+    // Fourteen 32-bit words of scalar arguments (heads = query heads | key/value heads << 16): all of them are
+    // preloaded into registers with the wavefront's launch, so the first loads do not wait for an argument fetch
+    // from memory, which the fields of a structure passed by value would need.
+    AttentionArgs a = {};
+    a.q = q_rows; a.k_cache = k_cache; a.v_cache = v_cache; a.pos = pos; a.seq = seq; a.head_partials = head_partials;
+    a.cache_seq_stride = cache_seq_stride; a.n_head = (int)(heads & 0xFFFFu); a.n_kv_head = (int)(heads >> 16);
     constexpr int LPT = HD / 8, SLOTS = 64 / LPT, KW = KV_F16 ? 1 : 2, STRIDE = HD + 4;
     __shared__ float wm[WAVES], wl[WAVES][SLOTS];
     __shared__ float wacc[WAVES][SLOTS][HD];
     const int group = a.n_head / a.n_kv_head;
     const int kvh = blockIdx.x % a.n_kv_head, head = kvh * group + blockIdx.x / a.n_kv_head, m = blockIdx.y;
-    const int split = blockIdx.z, splits = gridDim.z;
+    const int split = blockIdx.z;
+    constexpr int splits = kAttentionHeadSplits;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int visible = a.pos[m] + 1;
+    // both row descriptors are fetched in one round trip, before anything branches on the first
+    const int row_pos = a.pos[m], row_seq = a.seq[m];
+    asm volatile("" ::"s"(row_pos), "s"(row_seq));
+    const int visible = row_pos + 1;
     const int kd = a.n_kv_head * HD;
-    const size_t seq_base = (size_t)a.seq[m] * a.cache_seq_stride;
+    const size_t seq_base = (size_t)row_seq * a.cache_seq_stride;
     const float scale = 1.0f / sqrtf((float)HD);
     const int slot = lane / LPT, seg = (lane % LPT) * 8;
 
@@ -716,14 +727,16 @@ int attention_head_splits(int) { return kAttentionHeadSplits; }
 hipError_t launch_attention_partials(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
     if (!a.head_partials || (a.head_dim != 128 && a.head_dim != 64) || a.n_head % a.n_kv_head != 0 || rows < 1 || rows > kMaxStepRows)
         return hipErrorInvalidValue;
+    if (a.cache_seq_stride > 0xFFFFFFFFull || a.n_head > 0xFFFF || a.n_kv_head > 0xFFFF) return hipErrorInvalidValue;
+    const unsigned heads = (unsigned)a.n_head | ((unsigned)a.n_kv_head << 16);
     dim3 grid(a.n_head, rows, attention_head_splits(a.max_seq));
     constexpr int WAVES = 8;   // measured at head size 128: 4 wavefronts x 12 chunks 6.2 us, 8 x 6 5.0 us, 16 x 3 4.7 us but a slower step
     if (a.head_dim == 128) {
-        if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<128, true, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a);
-        else hipLaunchKernelGGL((attention_partial_kernel<128, false, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a);
+        if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<128, true, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
+        else hipLaunchKernelGGL((attention_partial_kernel<128, false, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
     } else {
-        if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<64, true, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a);
-        else hipLaunchKernelGGL((attention_partial_kernel<64, false, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a);
+        if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<64, true, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
+        else hipLaunchKernelGGL((attention_partial_kernel<64, false, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
     }
     return hipGetLastError();
 }

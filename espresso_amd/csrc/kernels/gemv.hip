@@ -238,14 +238,66 @@ __device__ __forceinline__ void pair_epilogue(const KernelArgs &a, int pair, con
     }
 }
 
+// The scalar arguments that the first loads of a GEMV kernel need.  Leading scalar arguments are preloaded
+// into registers with the wavefront's launch; the fields of a structure passed by value are fetched from
+// memory first, which costs the start of every kernel a memory round trip.
+// mode: 0 = fp16 activations, 1 = RMSNorm fused into the staging, 2 = attention partial states (head size in bits 8..).
+__device__ __forceinline__ KernelArgs with_leading_args(const KernelArgs &rest, const uint8_t *qs, const uint16_t *scales, const void *activations,
+                                                        const float *norm_w, int rows, int cols, int row_bytes, int mode, float norm_eps) {
+    KernelArgs a = rest;
+    a.qs = qs;
+    a.scales = scales;
+    a.rows = rows;
+    a.cols = cols;
+    a.qs_row_bytes = (size_t)row_bytes;
+    a.norm_w = norm_w;
+    a.norm_eps = norm_eps;
+    a.x = (mode & 0xFF) == 0 ? static_cast<const uint16_t *>(activations) : nullptr;
+    a.norm_x = (mode & 0xFF) == 1 ? static_cast<const float *>(activations) : nullptr;
+    a.merge_partials = (mode & 0xFF) == 2 ? static_cast<const float *>(activations) : nullptr;
+    a.merge_head_dim = mode >> 8;
+    return a;
+}
+inline const void *leading_activations(const KernelArgs &a) {
+    return a.merge_partials ? static_cast<const void *>(a.merge_partials) : a.norm_x ? static_cast<const void *>(a.norm_x) : static_cast<const void *>(a.x);
+}
+inline int leading_mode(const KernelArgs &a) { return a.merge_partials ? (2 | (a.merge_head_dim << 8)) : a.norm_x ? 1 : 0; }
+
 template <int FMT, int B, int R>
-__global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
+__global__ __launch_bounds__(kThreads) void gemv_kernel(const uint8_t *qs, const uint16_t *scales, const void *activations, const float *norm_w, int rows,
+                                                        int cols_arg, int row_bytes, int mode, float norm_eps, KernelArgs rest) {
+    const KernelArgs a = with_leading_args(rest, qs, scales, activations, norm_w, rows, cols_arg, row_bytes, mode, norm_eps);
     using T = Traits<FMT>;
     extern __shared__ uint4 smem_raw[];
     uint16_t *xs = reinterpret_cast<uint16_t *>(smem_raw);                 // [B][cols] fp16
     float *xsum = reinterpret_cast<float *>(xs + (size_t)B * a.cols);      // [B][cols/16] (Q4_K)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cols = a.cols;
+
+    // ---- the wavefront's rows and the first 128 bits of weights per lane: in flight while the activations are staged ----
+    const int row0 = (blockIdx.x * kWaves + wave) * R;
+    const int items = cols / T::kItemElems;
+    const uint8_t *rowp[R];
+    const uint16_t *scalep[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = row0 + r < a.rows ? row0 + r : a.rows - 1;  // clamp: never read past the matrix
+        rowp[r] = a.qs + (size_t)row * a.qs_row_bytes;
+        scalep[r] = (FMT == FMT_Q4_0 || FMT == FMT_Q8_0) ? a.scales + (size_t)row * (cols / 32) : nullptr;
+    }
+    struct Item { uint4 q[R]; uint16_t d[R]; };
+    auto load_item = [&](int item) {
+        Item it;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            it.q[r] = *reinterpret_cast<const uint4 *>(rowp[r] + (size_t)item * 16);
+            if constexpr (FMT == FMT_Q4_0) it.d[r] = scalep[r][item];
+            else if constexpr (FMT == FMT_Q8_0) it.d[r] = scalep[r][item >> 1];
+            else it.d[r] = 0;
+        }
+        return it;
+    };
+    Item cur = load_item(lane < items ? lane : items - 1);
 
     // ---- stage activations: 128-bit loads (or the fused RMSNorm), middle elements of each group of
     // four swapped for the integer formats ----
@@ -275,9 +327,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
         __syncthreads();
     }
 
-    const int row0 = (blockIdx.x * kWaves + wave) * R;
     if (row0 >= a.rows) return;
-    const int items = cols / T::kItemElems;
 
     float acc[R][B];
 #pragma unroll
@@ -285,14 +335,9 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
 #pragma unroll
         for (int b = 0; b < B; b++) acc[r][b] = 0.0f;
 
-    const uint8_t *rowp[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        int row = row0 + r < a.rows ? row0 + r : a.rows - 1;  // clamp: never read past the matrix
-        rowp[r] = a.qs + (size_t)row * a.qs_row_bytes;
-    }
-
     for (int item = lane; item < items; item += 64) {
+        Item nxt = cur;
+        if (item + 64 < items) nxt = load_item(item + 64);   // one step ahead of the arithmetic
         if constexpr (FMT == FMT_Q4_0) {
             const int e_lo = item * 32;
             uint4 xl[B][2], xh[B][2];
@@ -304,9 +349,8 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
             }
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const uint4 q = *reinterpret_cast<const uint4 *>(rowp[r] + (size_t)item * 16);
-                const int row = row0 + r < a.rows ? row0 + r : a.rows - 1;
-                const float d = half_bits_to_float(a.scales[(size_t)row * (cols / 32) + item]);
+                const uint4 q = cur.q[r];
+                const float d = half_bits_to_float(cur.d[r]);
 #pragma unroll
                 for (int b = 0; b < B; b++) {
                     float dlo = 0.0f, dhi = 0.0f;
@@ -333,9 +377,8 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
             }
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const uint4 q = *reinterpret_cast<const uint4 *>(rowp[r] + (size_t)item * 16);
-                const int row = row0 + r < a.rows ? row0 + r : a.rows - 1;
-                const float d = half_bits_to_float(a.scales[(size_t)row * (cols / 32) + (item >> 1)]);
+                const uint4 q = cur.q[r];
+                const float d = half_bits_to_float(cur.d[r]);
 #pragma unroll
                 for (int b = 0; b < B; b++) {
                     float dot = 0.0f;
@@ -355,7 +398,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
             for (int b = 0; b < B; b++) xv[b] = *reinterpret_cast<const uint2 *>(xs + (size_t)b * cols + e0);
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const uint4 q = *reinterpret_cast<const uint4 *>(rowp[r] + (size_t)item * 16);
+                const uint4 q = cur.q[r];
 #pragma unroll
                 for (int b = 0; b < B; b++) {
                     const h2 x01 = as_h2(xv[b].x), x23 = as_h2(xv[b].y);
@@ -373,7 +416,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
             for (int b = 0; b < B; b++) xv[b] = *reinterpret_cast<const uint4 *>(xs + (size_t)b * cols + e0);
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const uint4 q = *reinterpret_cast<const uint4 *>(rowp[r] + (size_t)item * 16);
+                const uint4 q = cur.q[r];
 #pragma unroll
                 for (int b = 0; b < B; b++) {
                     float dot = 0.0f;
@@ -383,6 +426,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(KernelArgs a) {
                 }
             }
         }
+        cur = nxt;
     }
 
 #pragma unroll
@@ -516,7 +560,17 @@ constexpr int kDeferredRounds = 16;   // rounds whose team reductions wait for o
 
 // MODE: 0 = fp16 activations as given, 1 = RMSNorm fused into the staging, 2 = attention partial states merged in the staging.
 template <int B, int IPR, int TEAM, int MODE>
-__global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int iters) {
+__global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, const void *activations, const float *norm_w, int rows, int row_bytes,
+                                                            int iters, int workgroups, float norm_eps, KernelArgs rest) {
+    // The arguments that the first loads need come as leading scalars: those can be preloaded into registers
+    // with the wavefront's launch, where fields of a structure passed by value are fetched from memory first.
+    KernelArgs a = rest;
+    a.qs = qs;
+    a.rows = rows;
+    a.qs_row_bytes = (size_t)row_bytes;
+    if constexpr (MODE == 1) { a.norm_x = static_cast<const float *>(activations); a.norm_w = norm_w; a.norm_eps = norm_eps; }
+    else if constexpr (MODE == 2) a.merge_partials = static_cast<const float *>(activations);
+    else a.x = static_cast<const uint16_t *>(activations);
     constexpr int cols = IPR * 64, XSTRIDE = IPR | 1, TOTAL = 2 * IPR, TEAM_LANES = TEAM * 64;
     constexpr int PASSES = (TOTAL + TEAM_LANES - 1) / TEAM_LANES, TEAMS = kWaves / TEAM;
     static_assert(PASSES <= 2 && kWaves % TEAM == 0, "pick TEAM so that a lane holds at most two items per pair");
@@ -527,7 +581,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int it
     float *norm_red = red + kDeferredRounds * kWaves * 2 * B;                     // [B][kWaves]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tl = (wave % TEAM) * 64 + lane;
-    const int n_teams = gridDim.x * TEAMS, npairs = (a.rows + 1) / 2;
+    const int n_teams = workgroups * TEAMS, npairs = (a.rows + 1) / 2;
     const Q4KLane L = q4k_lane_constants(lane);
 
     auto load_pair = [&](int pair, Q4KItem (&buf)[PASSES]) {
@@ -644,7 +698,9 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(KernelArgs a, int it
 // Any cols that is a multiple of 256: one workgroup per eight rows, a wavefront per row pair, loads
 // one pass ahead of the arithmetic.
 template <int B>
-__global__ __launch_bounds__(kThreads) void gemv_q4k_generic_kernel(KernelArgs a) {
+__global__ __launch_bounds__(kThreads) void gemv_q4k_generic_kernel(const uint8_t *qs, const void *activations, const float *norm_w, int rows, int cols_arg,
+                                                                    int row_bytes, int mode, float norm_eps, KernelArgs rest) {
+    const KernelArgs a = with_leading_args(rest, qs, nullptr, activations, norm_w, rows, cols_arg, row_bytes, mode, norm_eps);
     extern __shared__ uint4 smem_raw[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cols = a.cols, ipr = cols >> 6, xstride = ipr | 1, total = 2 * ipr;
@@ -758,7 +814,8 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     // get their first weights first (the memory system serves the opening burst roughly in order), and they stay
     // ahead by one to three microseconds to the end: one pair less for the later workgroups evens the finish.
     const int iters = (npairs + grid * TEAMS - 1) / (grid * TEAMS);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a, iters);
+    const void *activations = MODE == 1 ? static_cast<const void *>(a.norm_x) : MODE == 2 ? static_cast<const void *>(a.merge_partials) : static_cast<const void *>(a.x);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a.qs, activations, a.norm_w, a.rows, (int)a.qs_row_bytes, iters, grid, a.norm_eps, a);
     return hipGetLastError();
 }
 
@@ -783,7 +840,8 @@ hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
     if (e != hipSuccess) return e;
     const int pairs = (a.rows + 1) / 2;
-    hipLaunchKernelGGL(kernel, dim3((pairs + kWaves - 1) / kWaves), dim3(kThreads), lds, stream, a);
+    hipLaunchKernelGGL(kernel, dim3((pairs + kWaves - 1) / kWaves), dim3(kThreads), lds, stream, a.qs, leading_activations(a), a.norm_w, a.rows, a.cols,
+                       (int)a.qs_row_bytes, leading_mode(a), a.norm_eps, a);
     return hipGetLastError();
 }
 
@@ -802,7 +860,8 @@ hipError_t launch_one(const KernelArgs &a, hipStream_t stream) {
     }
     const int rows_per_wg = kWaves * R;
     const int grid = (a.rows + rows_per_wg - 1) / rows_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a.qs, a.scales, leading_activations(a), a.norm_w, a.rows, a.cols, (int)a.qs_row_bytes,
+                       leading_mode(a), a.norm_eps, a);
     return hipGetLastError();
 }
 
