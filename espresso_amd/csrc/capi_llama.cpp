@@ -206,6 +206,11 @@ int esp_llama_time_kernel(ESPLlamaRuntime *runtime, int kernel_class, int iters,
     return runtime->rt->time_kernel_class(kernel_class, iters, mean_us);
 }
 
+int esp_llama_time_kernel_dispatch(ESPLlamaRuntime *runtime, int kernel_class, int iters, double *back_to_back_us, double *kernel_us) {
+    if (!runtime) return bad_handle();
+    return runtime->rt->time_kernel_class(kernel_class, iters, back_to_back_us, kernel_us);
+}
+
 int esp_synth_weights(int format, uint64_t seed, float std_dev, size_t elements, void *out_blocks) {
     if (!out_blocks || elements == 0 || elements % 256 != 0)
         return fail(ESP_ERR_INVALID_ARGUMENT, "synth_weights: elements must be a positive multiple of 256");

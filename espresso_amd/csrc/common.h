@@ -84,6 +84,8 @@ struct GemvParams {
     QkvEpilogue qkv;              // EPI_QKV_ROPE
     int batch = 1;
     int epilogue = EPI_STORE_F32;
+    // optional (batch <= 2): events that take the kernel's own start and end times
+    hipEvent_t start_event = nullptr, stop_event = nullptr;
 };
 
 // y[rows][w.rows] = x[rows][w.cols] * dequant(w)^T (+ residual) for more than two rows, on the matrix cores.

@@ -32,6 +32,8 @@
 #include <type_traits>
 
 #include "../common.h"
+
+#include <hip/hip_ext.h>
 #include "gemv_device.h"
 
 namespace esp {
@@ -757,6 +759,15 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_generic_kernel(const uint8_
     if (lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
 }
 
+// Launch through the extension entry point when the caller gave the launch a pair of events of its own: they
+// take the kernel's own start and end times (what a kernel trace reports), without the gaps between launches.
+static thread_local hipEvent_t tl_start_event = nullptr, tl_stop_event = nullptr;
+template <typename K, typename... Args>
+inline void launch_kernel(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args... args) {
+    if (tl_start_event && tl_stop_event) hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, stream, tl_start_event, tl_stop_event, 0, args...);
+    else hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
+}
+
 inline hipError_t ensure_lds(const void *kernel, size_t lds, size_t *configured) {
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     if (lds > 48 * 1024 && lds > *configured) {
@@ -815,7 +826,7 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     // ahead by one to three microseconds to the end: one pair less for the later workgroups evens the finish.
     const int iters = (npairs + grid * TEAMS - 1) / (grid * TEAMS);
     const void *activations = MODE == 1 ? static_cast<const void *>(a.norm_x) : MODE == 2 ? static_cast<const void *>(a.merge_partials) : static_cast<const void *>(a.x);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a.qs, activations, a.norm_w, a.rows, (int)a.qs_row_bytes, iters, grid, a.norm_eps, a);
+    launch_kernel(kernel, dim3(grid), dim3(kThreads), lds, stream, a.qs, activations, a.norm_w, a.rows, (int)a.qs_row_bytes, iters, grid, a.norm_eps, a);
     return hipGetLastError();
 }
 
@@ -840,7 +851,7 @@ hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
     if (e != hipSuccess) return e;
     const int pairs = (a.rows + 1) / 2;
-    hipLaunchKernelGGL(kernel, dim3((pairs + kWaves - 1) / kWaves), dim3(kThreads), lds, stream, a.qs, leading_activations(a), a.norm_w, a.rows, a.cols,
+    launch_kernel(kernel, dim3((pairs + kWaves - 1) / kWaves), dim3(kThreads), lds, stream, a.qs, leading_activations(a), a.norm_w, a.rows, a.cols,
                        (int)a.qs_row_bytes, leading_mode(a), a.norm_eps, a);
     return hipGetLastError();
 }
@@ -860,7 +871,7 @@ hipError_t launch_one(const KernelArgs &a, hipStream_t stream) {
     }
     const int rows_per_wg = kWaves * R;
     const int grid = (a.rows + rows_per_wg - 1) / rows_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a.qs, a.scales, leading_activations(a), a.norm_w, a.rows, a.cols, (int)a.qs_row_bytes,
+    launch_kernel(kernel, dim3(grid), dim3(kThreads), lds, stream, a.qs, a.scales, leading_activations(a), a.norm_w, a.rows, a.cols, (int)a.qs_row_bytes,
                        leading_mode(a), a.norm_eps, a);
     return hipGetLastError();
 }
@@ -898,6 +909,11 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     if (w.cols % block != 0 || w.qs_row_bytes % 16 != 0 || (p.norm_x && w.cols % 8 != 0)) return hipErrorInvalidValue;
     if ((w.format == FMT_Q8_0 || w.format == FMT_Q4_0) && !w.scales) return hipErrorInvalidValue;
 
+    // events of its own only for a single launch
+    struct EventScope {
+        EventScope(hipEvent_t a, hipEvent_t b) { tl_start_event = a; tl_stop_event = b; }
+        ~EventScope() { tl_start_event = tl_stop_event = nullptr; }
+    } scope(p.batch <= 2 ? p.start_event : nullptr, p.batch <= 2 ? p.stop_event : nullptr);
     // batches beyond 2 run as successive pairs (each pair re-reads the weights)
     for (int b0 = 0; b0 < p.batch; b0 += 2) {
         const int nb = p.batch - b0 >= 2 ? 2 : 1;

@@ -135,15 +135,17 @@ bool LlamaRuntime::wo_merges_attention(const Layer &L, int rows) const {
            L.wo.cols == c_.attention_dim() && gemv_merges_attention_partials(L.wo, rows, c_.head_dim);
 }
 
-int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us) {
+int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us, double *kernel_only_us) {
     if (!finalized_ || iters < 1 || !mean_us) return fail(ESP_ERR_INVALID_ARGUMENT, "time_kernel_class: bad argument");
     if (kernel_class < K_QKV || kernel_class > K_HEAD) return fail(ESP_ERR_INVALID_ARGUMENT, "time_kernel_class: class %d", kernel_class);
     hipStream_t s = context().stream;
     const int kd = c_.kv_dim();
     const bool kv16 = c_.kv_format == FMT_F16;
-    auto launch = [&](const Layer *L) -> hipError_t {
+    auto launch = [&](const Layer *L, hipEvent_t start = nullptr, hipEvent_t stop = nullptr) -> hipError_t {
         GemvParams g;
         g.batch = 1;
+        g.start_event = start;
+        g.stop_event = stop;
         switch (kernel_class) {
         case K_QKV:
             if (L->q_norm) { g.w = L->wqkv; g.norm_x = hidden_; g.norm_w = L->rms_att; g.norm_eps = c_.norm_eps; g.y = qkv_; g.epilogue = EPI_STORE_F32; break; }
@@ -182,6 +184,22 @@ int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us
     event_pool_.push_back(t0);
     event_pool_.push_back(t1);
     *mean_us = (double)ms * 1e3 / ((double)iters * per_round);
+    if (kernel_only_us) {
+        // the same launches again, each with events of its own that take the kernel's start and end
+        std::vector<hipEvent_t> ev((size_t)iters * per_round * 2, nullptr);
+        for (hipEvent_t &e : ev) if (!(e = take_event())) return fail(ESP_ERR_OUT_OF_MEMORY, "time_kernel_class: events");
+        for (int r = 0, k = 0; r < iters; r++)
+            for (int i = 0; i < per_round; i++, k += 2)
+                ESP_HIP_TRY(launch(kernel_class == K_HEAD ? nullptr : &layers_[(size_t)i], ev[(size_t)k], ev[(size_t)k + 1]));
+        ESP_HIP_TRY(hipStreamSynchronize(s));
+        double total = 0.0;
+        for (size_t k = 0; k < ev.size(); k += 2) {
+            ESP_HIP_TRY(hipEventElapsedTime(&ms, ev[k], ev[k + 1]));
+            total += ms;
+        }
+        for (hipEvent_t e : ev) event_pool_.push_back(e);
+        *kernel_only_us = total * 1e3 / ((double)iters * per_round);
+    }
     return ESP_OK;
 }
 

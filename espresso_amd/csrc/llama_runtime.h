@@ -89,7 +89,9 @@ class LlamaRuntime {
     void set_kernel_timing(bool enabled) { timing_enabled_ = enabled; }
     int collect_kernel_times(double total_us[K_CLASS_COUNT], long launches[K_CLASS_COUNT], bool reset);
     size_t kernel_bytes(int kernel_class) const;   // algorithmic bytes of one batch-1 launch
-    int time_kernel_class(int kernel_class, int iters, double *mean_us);
+    // mean_us: launches back to back between two events; kernel_only_us (optional): the same launches with events
+    // of their own per launch (the kernels' own durations, as a kernel trace reports them)
+    int time_kernel_class(int kernel_class, int iters, double *mean_us, double *kernel_only_us = nullptr);
 
   private:
     LlamaRuntime() = default;

@@ -218,6 +218,16 @@ def time_kernel(rt: LlamaRuntime, name: str, iters: int = 8) -> float:
     return out.value
 
 
+def time_kernel_dispatch(rt: LlamaRuntime, name: str, iters: int = 8) -> tuple[float, float]:
+    """(back-to-back mean, mean kernel duration from events attached to each launch) in microseconds for one GEMV class
+    over all layers (invalidates sequence state)."""
+    rt._L.esp_llama_time_kernel_dispatch.restype = C.c_int
+    rt._L.esp_llama_time_kernel_dispatch.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
+    b2b, own = C.c_double(0), C.c_double(0)
+    _lib.check(rt._L.esp_llama_time_kernel_dispatch(rt._h, KERNEL_CLASSES.index(name), iters, C.byref(b2b), C.byref(own)))
+    return b2b.value, own.value
+
+
 def kernel_times(rt: LlamaRuntime, reset: bool = True) -> dict:
     """{class: {"total_us", "launches", "bytes_per_launch", "mean_us", "gbps"}} from HIP events."""
     n = len(KERNEL_CLASSES)

@@ -254,6 +254,10 @@ int esp_llama_kernel_times(ESPLlamaRuntime *runtime, double *total_us, int64_t *
  * is directly comparable with a rocprofv3 kernel trace.  The epilogues write into live buffers: reset the
  * runtime before decoding again. */
 int esp_llama_time_kernel(ESPLlamaRuntime *runtime, int kernel_class, int iters, double *mean_us);
+/* The same launches twice: back to back between two events (back_to_back_us, as above) and then with a pair of
+ * events attached to every launch, which take the kernel's own start and end (kernel_us: the mean kernel duration,
+ * the figure a rocprofv3 kernel trace reports for the kernel).  Measurement only; no counterpart in the reference. */
+int esp_llama_time_kernel_dispatch(ESPLlamaRuntime *runtime, int kernel_class, int iters, double *back_to_back_us, double *kernel_us);
 
 /* ---- seeded synthetic weights ------------------------------------------------------------- *
  * Fills `out_blocks` (host memory, esp_format_bytes(format, elements) bytes) with N(0, std_dev) draws
