@@ -1,5 +1,6 @@
 // C ABI: weight files, metadata, the GGUF front door, the engine and the exact two-token harness.
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 
 #include "generation.h"
@@ -150,6 +151,82 @@ int esp_gguf_prepare(const char *gguf_path, const char *output_dir, const ESPPre
 }
 
 namespace {
+std::map<std::string, std::string> env_map(const char *const *keys, const char *const *values, int n) {
+    std::map<std::string, std::string> m;
+    for (int i = 0; i < n; i++) if (keys && values && keys[i] && values[i]) m[keys[i]] = values[i];
+    return m;
+}
+PrepareOptions from_c(const ESPPrepareCacheOptions &c, const ESPPrepareOptions *convert) {
+    PrepareOptions o;
+    if (convert) { o.emitDequantizedBlobs = convert->emit_dequantized_blobs != 0; o.emitFloat32Sidecars = convert->emit_float32_sidecars != 0; o.qkLayout = convert->qk_layout; }
+    o.artifactCacheEnabled = c.cache_enabled != 0;
+    o.cacheRoot = std::string(c.cache_root, strnlen(c.cache_root, sizeof(c.cache_root)));
+    o.exactFloat32SidecarMode = c.sidecar_mode == ESP_SIDECAR_NONE ? ExactFloat32SidecarMode::none
+                              : c.sidecar_mode == ESP_SIDECAR_ESSENTIAL ? ExactFloat32SidecarMode::essential
+                              : c.sidecar_mode == ESP_SIDECAR_SELECTED ? ExactFloat32SidecarMode::selected
+                              : c.sidecar_mode == ESP_SIDECAR_FULL ? ExactFloat32SidecarMode::full : ExactFloat32SidecarMode::automatic;
+    const std::string names(c.selected_sidecars, strnlen(c.selected_sidecars, sizeof(c.selected_sidecars)));
+    for (size_t at = 0; at <= names.size();) {
+        const size_t comma = names.find(',', at);
+        const std::string n = names.substr(at, comma == std::string::npos ? std::string::npos : comma - at);
+        if (!n.empty()) o.selectedSidecars.insert(n);
+        if (comma == std::string::npos) break;
+        at = comma + 1;
+    }
+    return o;
+}
+int copy_out(const std::string &v, char *out, size_t bytes, const char *what) {
+    if (!out || bytes < v.size() + 1) return fail(ESP_ERR_INVALID_ARGUMENT, "%s: buffer of %zu bytes is too small", what, bytes);
+    std::memcpy(out, v.c_str(), v.size() + 1);
+    return ESP_OK;
+}
+}  // namespace
+
+int esp_gguf_prepare_options_from_environment(const char *const *env_keys, const char *const *env_values, int env_count,
+                                              ESPPrepareCacheOptions *out) {
+    if (!out || env_count < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "prepare options: bad argument");
+    const PrepareOptions o = PrepareOptions::environment(env_map(env_keys, env_values, env_count));
+    std::memset(out, 0, sizeof(*out));
+    out->cache_enabled = o.artifactCacheEnabled ? 1 : 0;
+    out->sidecar_mode = (int32_t)o.exactFloat32SidecarMode;
+    std::string names;
+    for (const std::string &n : o.selectedSidecars) names += (names.empty() ? "" : ",") + n;
+    if (o.cacheRoot.size() >= sizeof(out->cache_root) || names.size() >= sizeof(out->selected_sidecars))
+        return fail(ESP_ERR_INVALID_ARGUMENT, "prepare options: cache root or sidecar list too long");
+    std::memcpy(out->cache_root, o.cacheRoot.c_str(), o.cacheRoot.size());
+    std::memcpy(out->selected_sidecars, names.c_str(), names.size());
+    return ESP_OK;
+}
+
+int esp_gguf_artifact_cache_key(const char *gguf_path, const ESPPrepareCacheOptions *options, const char *const *env_keys,
+                                const char *const *env_values, int env_count, char *out_key, size_t out_key_bytes) {
+    if (!gguf_path || !options) return fail(ESP_ERR_INVALID_ARGUMENT, "cache key: null argument");
+    std::string key;
+    const int rc = GGUFModelLoader::artifactCacheKey(gguf_path, from_c(*options, nullptr), env_map(env_keys, env_values, env_count), &key);
+    return rc != ESP_OK ? rc : copy_out(key, out_key, out_key_bytes, "cache key");
+}
+
+int esp_gguf_prepare_cached(const char *gguf_path, const ESPPrepareCacheOptions *options, const ESPPrepareOptions *convert,
+                            const char *const *env_keys, const char *const *env_values, int env_count, ESPModelConfig *out_config,
+                            int *out_tensor_count, char *out_weight_dir, size_t out_weight_dir_bytes) {
+    if (!gguf_path || !options) return fail(ESP_ERR_INVALID_ARGUMENT, "prepare: null argument");
+    PreparedModel pm;
+    int rc = GGUFModelLoader::prepare(gguf_path, from_c(*options, convert), env_map(env_keys, env_values, env_count), &pm);
+    if (rc != ESP_OK) return rc;
+    if (out_config) to_c(pm.config, out_config);
+    if (out_tensor_count) *out_tensor_count = pm.tensorCount;
+    return out_weight_dir ? copy_out(pm.weightDir, out_weight_dir, out_weight_dir_bytes, "weight directory") : ESP_OK;
+}
+
+int esp_gguf_cleanup(const char *weight_dir) {
+    if (!weight_dir) return fail(ESP_ERR_INVALID_ARGUMENT, "cleanup: null path");
+    GGUFModelLoader::cleanup(weight_dir);
+    return ESP_OK;
+}
+
+int esp_gguf_default_cache_root(char *out, size_t out_bytes) { return copy_out(GGUFModelLoader::defaultPreparedArtifactCacheRoot(), out, out_bytes, "cache root"); }
+
+namespace {
 void fill_result(const GenerationResult &r, ESPGenerationResult *result) {
     std::memset(result, 0, sizeof(*result));
     result->token_count = (int32_t)r.tokens.size();
@@ -207,6 +284,45 @@ int esp_engine_generate_text(ESPEngine *engine, const char *prompt_utf8, size_t 
     if (out_text && text_capacity) std::memcpy(out_text, r.text.data(), std::min(text_capacity, r.text.size()));
     if (result) fill_result(r, result);
     return ESP_OK;
+}
+
+int esp_run_gguf(const char *gguf_path, const char *tokenizer_dir, const char *prompt_utf8, size_t prompt_bytes, int max_tokens,
+                 const char *const *env_keys, const char *const *env_values, int env_count, uint32_t *out_tokens, char *out_text,
+                 size_t text_capacity, size_t *out_text_bytes, ESPGenerationResult *result, ESPRunGGUFInfo *info) {
+    if (!gguf_path || !tokenizer_dir || (!prompt_utf8 && prompt_bytes)) return fail(ESP_ERR_INVALID_ARGUMENT, "run_gguf: null argument");
+    const Environment env = env_from(env_keys, env_values, env_count);
+    auto now_ms = [] { return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count(); };
+    const double t0 = now_ms();
+    PreparedModel pm;
+    int rc = GGUFModelLoader::prepare(gguf_path, PrepareOptions::environment(env), env, &pm);
+    if (rc != ESP_OK) return rc;
+    const double t1 = now_ms();
+    auto env_it = env.find("ESPRESSO_GGUF_KEEP_WEIGHT_DIR");
+    const bool keep = env_it != env.end() && env_it->second == "1";
+    auto finish = [&](int code) {
+        if (!keep) GGUFModelLoader::cleanup(pm.weightDir);
+        if (info) info->kept_weight_dir = directoryExists(pm.weightDir) ? 1 : 0;
+        return code;
+    };
+    if (info) {
+        std::memset(info, 0, sizeof(*info));
+        to_c(pm.config, &info->config);
+        info->tensor_count = pm.tensorCount;
+        info->prepare_ms = t1 - t0;
+        std::strncpy(info->weight_dir, pm.weightDir.c_str(), sizeof(info->weight_dir) - 1);
+    }
+    std::unique_ptr<RealModelInferenceEngine> engine;
+    if ((rc = RealModelInferenceEngine::build(pm.config, pm.weightDir, tokenizer_dir, env, &engine)) != ESP_OK) return finish(rc);
+    if (info) info->build_ms = now_ms() - t1;
+    GenerationResult r;
+    rc = engine->generateText(std::string(prompt_utf8 ? prompt_utf8 : "", prompt_bytes), max_tokens, 0.0f, env, &r);
+    engine.reset();
+    if (rc != ESP_OK) return finish(rc);
+    if (out_tokens) for (size_t i = 0; i < r.tokens.size(); i++) out_tokens[i] = r.tokens[i];
+    if (out_text_bytes) *out_text_bytes = r.text.size();
+    if (out_text && text_capacity) std::memcpy(out_text, r.text.data(), std::min(text_capacity, r.text.size()));
+    if (result) fill_result(r, result);
+    return finish(ESP_OK);
 }
 
 // ---- tokenizers ----------------------------------------------------------------------------------------

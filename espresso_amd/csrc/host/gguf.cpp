@@ -1,9 +1,19 @@
 #include "gguf.h"
 
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <cctype>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <filesystem>
+#include <random>
 
 #include "../context.h"
+#include "bundle.h"
+#include "json_min.h"
 
 namespace esp {
 namespace {
@@ -284,7 +294,10 @@ int GGUFModelLoader::prepare(const std::string &ggufPath, const std::string &out
             int r = tensor_to_float(*t, raw, &values);
             if (r != ESP_OK) return r;
             if ((r = write_blob_from_floats(path, values)) != ESP_OK) return r;
-            if (options.emitFloat32Sidecars && (t->type == GGML_F32 || t->type == GGML_BF16) &&
+            const bool wanted = options.exactFloat32SidecarMode == ExactFloat32SidecarMode::selected
+                                    ? options.selectedSidecars.count(gguf_name) != 0
+                                    : options.exactFloat32SidecarMode != ExactFloat32SidecarMode::none;
+            if (options.emitFloat32Sidecars && wanted && (t->type == GGML_F32 || t->type == GGML_BF16) &&
                 !writeFile(exactFloat32SidecarPath(path), values.data(), values.size() * 4))
                 return fail(ESP_ERR_IO, "cannot write %s", exactFloat32SidecarPath(path).c_str());
         }
@@ -331,11 +344,220 @@ int GGUFModelLoader::prepare(const std::string &ggufPath, const std::string &out
     if (count == 0) return fail(ESP_ERR_INVALID_ARGUMENT, "no tensors converted");
     const std::string meta = metadataJSON(c);
     if (!writeFile(joinPath(outputDir, "metadata.json"), meta.data(), meta.size())) return fail(ESP_ERR_IO, "cannot write metadata.json");
-    const std::string manifest = "{\n  \"source\": \"" + ggufPath + "\",\n  \"tensorCount\": " + std::to_string(count) + "\n}\n";
-    writeFile(joinPath(outputDir, "prepare-manifest.json"), manifest.data(), manifest.size());
     out->config = c;
     out->weightDir = outputDir;
     out->tensorCount = count;
+    return ESP_OK;
+}
+
+// ---- prepared-artifact cache ------------------------------------------------------------------------
+namespace {
+
+constexpr int kPreparedArtifactCacheVersion = 1;
+const char *const kManifestFileName = "prepare-manifest.json";
+const char *const kCacheMarkerFileName = ".espresso-gguf-cache-artifact";
+// converterCacheEnvironmentKeys (:29-36)
+const char *const kConverterEnvironmentKeys[] = {
+    "ESPRESSO_FORCE_LLAMA_MATRIX_TRANSPOSE", "ESPRESSO_SKIP_LLAMA_MATRIX_TRANSPOSE", "ESPRESSO_FORCE_QK_INVERSE_INTERLEAVE",
+    "ESPRESSO_DIM_MAJOR_TO_HEAD_MAJOR_V_WEIGHT", "ESPRESSO_INVERSE_INTERLEAVE_V_WEIGHT", "ESPRESSO_FORWARD_INTERLEAVE_V_WEIGHT",
+};
+
+std::string trimmed(const std::string &v) {
+    size_t a = 0, b = v.size();
+    while (a < b && std::isspace((unsigned char)v[a])) a++;
+    while (b > a && std::isspace((unsigned char)v[b - 1])) b--;
+    return v.substr(a, b - a);
+}
+std::string lowered(std::string v) {
+    for (char &c : v) c = (char)std::tolower((unsigned char)c);
+    return v;
+}
+bool isEnabled(const std::string *raw) {   // :607-615
+    if (!raw) return false;
+    const std::string v = lowered(trimmed(*raw));
+    return v == "1" || v == "true" || v == "yes" || v == "on";
+}
+const std::string *lookup(const std::map<std::string, std::string> &env, const char *key) {
+    auto it = env.find(key);
+    return it == env.end() ? nullptr : &it->second;
+}
+const char *sidecarModeName(ExactFloat32SidecarMode m) {   // sidecarModeCacheDescription (:579-593)
+    switch (m) {
+    case ExactFloat32SidecarMode::none: return "none";
+    case ExactFloat32SidecarMode::essential: return "essential";
+    case ExactFloat32SidecarMode::selected: return "selected";
+    case ExactFloat32SidecarMode::full: return "full";
+    default: return "automatic";
+    }
+}
+std::string jsonString(const std::string &v) {
+    std::string out = "\"";
+    for (char c : v) {
+        if (c == '"' || c == '\\') { out += '\\'; out += c; }
+        else if ((unsigned char)c < 0x20) { char b[8]; std::snprintf(b, sizeof(b), "\\u%04x", c); out += b; }
+        else out += c;
+    }
+    return out + "\"";
+}
+std::string standardizedPath(const std::string &path) {
+    std::error_code ec;
+    const std::filesystem::path abs = std::filesystem::absolute(path, ec);
+    return normalizePath(ec ? path : abs.string());
+}
+bool fileIdentity(const std::string &path, uint64_t *size, double *mtime) {
+    struct stat st;
+    if (::stat(path.c_str(), &st) != 0) return false;
+    *size = (uint64_t)st.st_size;
+    *mtime = (double)st.st_mtim.tv_sec + 1e-9 * (double)st.st_mtim.tv_nsec;
+    return true;
+}
+// converterEnvironmentFingerprint (:595-605): the non-empty values of the converter's switches, by key
+std::map<std::string, std::string> converterFingerprint(const std::map<std::string, std::string> &env) {
+    std::map<std::string, std::string> out;
+    for (const char *k : kConverterEnvironmentKeys) {
+        const std::string *v = lookup(env, k);
+        if (v && !v->empty()) out[k] = *v;
+    }
+    return out;
+}
+// The cache payload with its keys in sorted order (cachePayload, :433-443), shared by the key and the manifest.
+std::string cachePayloadJSON(const std::string &path, uint64_t size, double mtime, const PrepareOptions &o,
+                             const std::map<std::string, std::string> &env, int tensorCount) {
+    std::string j = "{\"converterEnvironment\":{";
+    bool first = true;
+    for (const auto &kv : converterFingerprint(env)) {
+        if (!first) j += ",";
+        j += jsonString(kv.first) + ":" + jsonString(kv.second);
+        first = false;
+    }
+    char num[64];
+    std::snprintf(num, sizeof(num), "%.9f", mtime);
+    j += "},\"fileSize\":" + std::to_string(size) + ",\"ggufPath\":" + jsonString(path) + ",\"modificationTime\":" + num + ",\"selectedSidecars\":[";
+    first = true;
+    if (o.exactFloat32SidecarMode == ExactFloat32SidecarMode::selected)
+        for (const std::string &n : o.selectedSidecars) {   // std::set: sorted
+            if (!first) j += ",";
+            j += jsonString(n);
+            first = false;
+        }
+    j += std::string("],\"sidecarMode\":\"") + sidecarModeName(o.exactFloat32SidecarMode) + "\"";
+    if (tensorCount >= 0) j += ",\"tensorCount\":" + std::to_string(tensorCount);
+    j += ",\"version\":" + std::to_string(kPreparedArtifactCacheVersion) + "}";
+    return j;
+}
+std::string randomSuffix() {
+    std::random_device rd;
+    char b[40];
+    std::snprintf(b, sizeof(b), "%08x%08x%08x", (unsigned)rd(), (unsigned)rd(), (unsigned)rd());
+    return b;
+}
+
+}  // namespace
+
+PrepareOptions PrepareOptions::environment(const std::map<std::string, std::string> &env) {
+    PrepareOptions o;
+    if (isEnabled(lookup(env, "ESPRESSO_GGUF_FORCE_FRESH_PREPARE"))) o.artifactCacheEnabled = false;
+    else if (const std::string *raw = lookup(env, "ESPRESSO_GGUF_PREPARE_CACHE")) o.artifactCacheEnabled = isEnabled(raw);
+    if (const std::string *root = lookup(env, "ESPRESSO_GGUF_PREPARE_CACHE_ROOT")) {
+        std::string r = trimmed(*root);
+        if (!r.empty() && r[0] == '~') {   // expandingTildeInPath
+            const char *home = std::getenv("HOME");
+            if (home && (r.size() == 1 || r[1] == '/')) r = std::string(home) + r.substr(1);
+        }
+        o.cacheRoot = r;
+    }
+    if (const std::string *names = lookup(env, "ESPRESSO_GGUF_SELECTED_SIDECARS")) {
+        size_t at = 0;
+        while (at <= names->size()) {
+            const size_t comma = names->find(',', at);
+            const std::string n = trimmed(names->substr(at, comma == std::string::npos ? std::string::npos : comma - at));
+            if (!n.empty()) o.selectedSidecars.insert(n);
+            if (comma == std::string::npos) break;
+            at = comma + 1;
+        }
+    }
+    const std::string *policy = lookup(env, "ESPRESSO_GGUF_SIDECAR_POLICY");
+    const std::string p = policy ? lowered(trimmed(*policy)) : "";
+    if (p == "none" || p == "off") o.exactFloat32SidecarMode = ExactFloat32SidecarMode::none;
+    else if (p == "essential") o.exactFloat32SidecarMode = ExactFloat32SidecarMode::essential;
+    else if (p == "selected") o.exactFloat32SidecarMode = ExactFloat32SidecarMode::selected;
+    else if (p == "full") o.exactFloat32SidecarMode = ExactFloat32SidecarMode::full;
+    else o.exactFloat32SidecarMode = ExactFloat32SidecarMode::automatic;   // unset, "automatic", "auto" and anything else
+    if (o.exactFloat32SidecarMode != ExactFloat32SidecarMode::selected) o.selectedSidecars.clear();
+    return o;
+}
+
+std::string GGUFModelLoader::defaultPreparedArtifactCacheRoot() {
+    const char *xdg = std::getenv("XDG_CACHE_HOME"), *home = std::getenv("HOME");
+    std::string base = xdg && xdg[0] ? xdg : (home && home[0] ? joinPath(home, ".cache") : std::filesystem::temp_directory_path().string());
+    return joinPath(joinPath(base, "Espresso"), "gguf-prepared");
+}
+
+int GGUFModelLoader::artifactCacheKey(const std::string &ggufPath, const PrepareOptions &options,
+                                      const std::map<std::string, std::string> &environment, std::string *out) {
+    const std::string path = standardizedPath(ggufPath);
+    uint64_t size = 0;
+    double mtime = 0;
+    if (!fileIdentity(path, &size, &mtime)) return fail(ESP_ERR_IO, "cannot stat %s", path.c_str());
+    const std::string payload = cachePayloadJSON(path, size, mtime, options, environment, -1);
+    *out = sha256_hex(payload.data(), payload.size());
+    return ESP_OK;
+}
+
+bool GGUFModelLoader::isManagedCachedArtifactDirectory(const std::string &dir) { return fileExists(joinPath(dir, kCacheMarkerFileName)); }
+
+void GGUFModelLoader::cleanup(const std::string &weightDir) {
+    if (isManagedCachedArtifactDirectory(weightDir)) return;
+    std::error_code ec;
+    std::filesystem::remove_all(weightDir, ec);
+}
+
+int GGUFModelLoader::prepare(const std::string &ggufPath, const PrepareOptions &options, const std::map<std::string, std::string> &environment,
+                             PreparedModel *out) {
+    const std::string path = standardizedPath(ggufPath);
+    std::error_code ec;
+    std::string outputDir;
+    if (options.artifactCacheEnabled) {
+        std::string key;
+        int rc = artifactCacheKey(path, options, environment, &key);
+        if (rc != ESP_OK) return rc;
+        outputDir = joinPath(options.cacheRoot.empty() ? defaultPreparedArtifactCacheRoot() : options.cacheRoot, key);
+        if (directoryExists(outputDir)) {   // loadCachedPreparedModelIfAvailable (:495-533)
+            std::vector<uint8_t> raw;
+            std::string err;
+            JsonNode manifest;
+            MultiModelConfig config;
+            if (readFile(joinPath(outputDir, kManifestFileName), &raw) && json_parse(std::string(raw.begin(), raw.end()), &manifest, &err) &&
+                manifest.kind == JsonNode::Object && manifest.find("tensorCount") && manifest.find("tensorCount")->kind == JsonNode::Number &&
+                loadConfigFromMetadataFile(joinPath(outputDir, "metadata.json"), &config, &err)) {
+                out->config = config;
+                out->weightDir = outputDir;
+                out->tensorCount = (int)manifest.find("tensorCount")->number;
+                return ESP_OK;
+            }
+            std::filesystem::remove_all(outputDir, ec);   // an incomplete or unreadable entry is rebuilt
+        }
+    } else {
+        outputDir = joinPath(std::filesystem::temp_directory_path().string(), "espresso_gguf_" + randomSuffix());
+    }
+    PreparedModel pm;
+    const int rc = prepare(path, outputDir, options, &pm);
+    if (rc != ESP_OK) {
+        std::filesystem::remove_all(outputDir, ec);   // shouldCleanupOnFailure (:399-403)
+        return rc;
+    }
+    if (options.artifactCacheEnabled) {   // writePreparedArtifactManifest (:535-566)
+        uint64_t size = 0;
+        double mtime = 0;
+        fileIdentity(path, &size, &mtime);
+        const std::string manifest = cachePayloadJSON(path, size, mtime, options, environment, pm.tensorCount) + "\n";
+        if (!writeFile(joinPath(outputDir, kManifestFileName), manifest.data(), manifest.size()) ||
+            !writeFile(joinPath(outputDir, kCacheMarkerFileName), "", 0)) {
+            std::filesystem::remove_all(outputDir, ec);
+            return fail(ESP_ERR_IO, "cannot write the cache manifest in %s", outputDir.c_str());
+        }
+    }
+    *out = pm;
     return ESP_OK;
 }
 

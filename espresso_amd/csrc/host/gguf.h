@@ -6,6 +6,7 @@
 
 #include <cstdint>
 #include <map>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -53,13 +54,26 @@ class GGUFLoader {
     std::vector<GGUFTensorInfo> tensors_;
 };
 
-// GGUFModelLoader.PrepareOptions (Sources/EspressoGGUF/GGUFModelLoader.swift:38-138), reduced to what
-// this build acts on.
+// GGUFModelLoader.PrepareOptions (Sources/EspressoGGUF/GGUFModelLoader.swift:38-138).
+enum class ExactFloat32SidecarMode { automatic, none, essential, selected, full };
+
 struct PrepareOptions {
     bool emitDequantizedBlobs = false;   // also write fp16 BLOBFILEs for quantised projections (what the reference's
                                          // own engine reads); the packed sidecars are always written
-    bool emitFloat32Sidecars = true;     // exact fp32 sidecars for tensors stored as F32/BF16
+    bool emitFloat32Sidecars = true;     // exact fp32 sidecars for tensors stored as F32/BF16 (subject to the mode below)
     int qkLayout = -1;                   // -1: by architecture; 0: rows as stored; 1: undo the GGUF llama Q/K row interleave
+    // Prepared-artifact cache (:38-63): used by the prepare() that chooses the directory itself.
+    bool artifactCacheEnabled = true;
+    std::string cacheRoot;               // empty: defaultPreparedArtifactCacheRoot()
+    // Which tensors get an exact float32 sidecar.  Quantised tensors stay packed in this build, so the mode only
+    // matters for tensors stored as F32/BF16: none writes no sidecar, selected only those named (GGUF names), every
+    // other mode all of them.
+    ExactFloat32SidecarMode exactFloat32SidecarMode = ExactFloat32SidecarMode::automatic;
+    std::set<std::string> selectedSidecars;
+
+    // PrepareOptions.environment(_:) (:65-127): ESPRESSO_GGUF_FORCE_FRESH_PREPARE, ESPRESSO_GGUF_PREPARE_CACHE,
+    // ESPRESSO_GGUF_PREPARE_CACHE_ROOT, ESPRESSO_GGUF_SIDECAR_POLICY, ESPRESSO_GGUF_SELECTED_SIDECARS.
+    static PrepareOptions environment(const std::map<std::string, std::string> &environment);
 };
 
 struct PreparedModel {     // GGUFModelLoader.PreparedModel (:140-160)
@@ -69,10 +83,24 @@ struct PreparedModel {     // GGUFModelLoader.PreparedModel (:140-160)
 };
 
 struct GGUFModelLoader {
-    // GGUF -> directory of BLOBFILEs / sidecars + metadata.json (GGUFModelLoader.prepare, :273-405).
+    // GGUF -> directory of BLOBFILEs / sidecars + metadata.json into a directory the caller names (the conversion
+    // of GGUFModelLoader.prepare, :303-405).
     static int prepare(const std::string &ggufPath, const std::string &outputDir, const PrepareOptions &options, PreparedModel *out);
+    // GGUFModelLoader.prepare(ggufURL:options:) (:273-405): returns the cached directory when one matches the file
+    // and the options (:495-533); otherwise converts into <cache root>/<key> (cache on: manifest + marker written,
+    // :535-566) or into a fresh temporary directory (cache off).
+    static int prepare(const std::string &ggufPath, const PrepareOptions &options, const std::map<std::string, std::string> &environment,
+                       PreparedModel *out);
     // Metadata -> MultiModelConfig (:297-326)
     static int configFromMetadata(const GGUFLoader &gguf, MultiModelConfig *out);
+    // SHA-256 over a sorted-key JSON of cache version, standardised path, file size, modification time, sidecar mode,
+    // selected sidecars and the converter environment (:424-447).  The digest is this build's own rendering of that
+    // payload: equal inputs give equal keys, any difference in them a different key.
+    static int artifactCacheKey(const std::string &ggufPath, const PrepareOptions &options,
+                                const std::map<std::string, std::string> &environment, std::string *out);
+    static std::string defaultPreparedArtifactCacheRoot();                     // :414-422 ($XDG_CACHE_HOME or ~/.cache here)
+    static bool isManagedCachedArtifactDirectory(const std::string &dir);      // :449-453
+    static void cleanup(const std::string &weightDir);                         // :408-412: keeps managed cache directories
 };
 
 }  // namespace esp

@@ -142,6 +142,101 @@ def gguf_prepare(gguf_path: str, output_dir: str, emit_dequantized_blobs=False, 
     return config_from_struct(s), output_dir, n.value
 
 
+class PrepareCacheOptionsStruct(C.Structure):
+    _fields_ = [("cache_enabled", C.c_int32), ("sidecar_mode", C.c_int32), ("cache_root", C.c_char * 1024),
+                ("selected_sidecars", C.c_char * 2048)]
+
+
+SIDECAR_MODES = ("automatic", "none", "essential", "selected", "full")
+
+
+class PrepareOptions:
+    """GGUFModelLoader.PrepareOptions: artifact cache mode, cache root, exact-float32 sidecar mode."""
+
+    def __init__(self, artifact_cache_enabled=True, cache_root=None, sidecar_mode="automatic", selected_sidecars=()):
+        self.artifact_cache_enabled = artifact_cache_enabled
+        self.cache_root = cache_root
+        self.sidecar_mode = sidecar_mode
+        self.selected_sidecars = set(selected_sidecars)
+
+    @classmethod
+    def environment(cls, environment: dict):
+        """PrepareOptions.environment(_:)."""
+        L = _L()
+        L.esp_gguf_prepare_options_from_environment.restype = C.c_int
+        k, v, n = _env_arrays(environment)
+        s = PrepareCacheOptionsStruct()
+        _lib.check(L.esp_gguf_prepare_options_from_environment(k, v, n, C.byref(s)))
+        names = [x for x in s.selected_sidecars.decode().split(",") if x]
+        return cls(bool(s.cache_enabled), s.cache_root.decode() or None, SIDECAR_MODES[s.sidecar_mode], names)
+
+    def struct(self) -> PrepareCacheOptionsStruct:
+        return PrepareCacheOptionsStruct(int(self.artifact_cache_enabled), SIDECAR_MODES.index(self.sidecar_mode),
+                                         (self.cache_root or "").encode(), ",".join(sorted(self.selected_sidecars)).encode())
+
+
+def gguf_artifact_cache_key(gguf_path: str, options: PrepareOptions, environment: dict | None = None) -> str:
+    """GGUFModelLoader.artifactCacheKey."""
+    L = _L()
+    L.esp_gguf_artifact_cache_key.restype = C.c_int
+    k, v, n = _env_arrays(environment)
+    s, out = options.struct(), C.create_string_buffer(80)
+    _lib.check(L.esp_gguf_artifact_cache_key(gguf_path.encode(), C.byref(s), k, v, n, out, C.c_size_t(80)))
+    return out.value.decode()
+
+
+def gguf_prepare_cached(gguf_path: str, options: PrepareOptions, environment: dict | None = None, emit_dequantized_blobs=False,
+                        emit_float32_sidecars=True, qk_layout=-1):
+    """GGUFModelLoader.prepare(ggufURL:options:) -> (config, weight_dir, tensor_count); the directory is chosen by the cache."""
+    L = _L()
+    L.esp_gguf_prepare_cached.restype = C.c_int
+    k, v, n = _env_arrays(environment)
+    s, conv = options.struct(), PrepareOptionsStruct(int(emit_dequantized_blobs), int(emit_float32_sidecars), qk_layout)
+    cfg, count, out = ModelConfigStruct(), C.c_int(0), C.create_string_buffer(4096)
+    _lib.check(L.esp_gguf_prepare_cached(gguf_path.encode(), C.byref(s), C.byref(conv), k, v, n, C.byref(cfg), C.byref(count), out,
+                                         C.c_size_t(4096)))
+    return config_from_struct(cfg), out.value.decode(), count.value
+
+
+def gguf_cleanup(weight_dir: str) -> None:
+    """GGUFModelLoader.cleanup(weightDir:): managed cache directories are kept."""
+    L = _L()
+    L.esp_gguf_cleanup.restype = C.c_int
+    _lib.check(L.esp_gguf_cleanup(weight_dir.encode()))
+
+
+def gguf_default_cache_root() -> str:
+    L = _L()
+    L.esp_gguf_default_cache_root.restype = C.c_int
+    out = C.create_string_buffer(4096)
+    _lib.check(L.esp_gguf_default_cache_root(out, C.c_size_t(4096)))
+    return out.value.decode()
+
+
+class RunGGUFInfoStruct(C.Structure):
+    _fields_ = [("config", ModelConfigStruct), ("tensor_count", C.c_int32), ("kept_weight_dir", C.c_int32), ("prepare_ms", C.c_double),
+                ("build_ms", C.c_double), ("weight_dir", C.c_char * 1024)]
+
+
+def run_gguf(gguf_path: str, tokenizer_dir: str, prompt: str, max_tokens: int = 32, environment: dict | None = None) -> dict:
+    """RunGGUF.main: prepare -> build -> generate(prompt) -> cleanup.  Returns text, tokens, the generation figures and
+    what was prepared (config, tensor count, times, the weight directory and whether it was kept)."""
+    L = _L()
+    L.esp_run_gguf.restype = C.c_int
+    k, v, n = _env_arrays(environment)
+    p = prompt.encode()
+    toks = (C.c_uint32 * max(max_tokens, 1))()
+    text = C.create_string_buffer(1 << 20)
+    nbytes, res, info = C.c_size_t(0), GenerationResultStruct(), RunGGUFInfoStruct()
+    _lib.check(L.esp_run_gguf(gguf_path.encode(), tokenizer_dir.encode(), p, C.c_size_t(len(p)), max_tokens, k, v, n, toks, text,
+                              C.c_size_t(len(text)), C.byref(nbytes), C.byref(res), C.byref(info)))
+    return {"text": text.raw[:min(nbytes.value, len(text))].decode("utf-8", "replace"), "tokens": list(toks[:res.token_count]),
+            "tokens_per_second": res.tokens_per_second, "compile_time_ms": res.compile_time_ms,
+            "first_token_latency_ms": res.first_token_latency_ms, "config": config_from_struct(info.config),
+            "tensor_count": info.tensor_count, "prepare_ms": info.prepare_ms, "build_ms": info.build_ms,
+            "weight_dir": info.weight_dir.decode(), "kept_weight_dir": bool(info.kept_weight_dir)}
+
+
 # ---- engine ---------------------------------------------------------------------
 def _env_arrays(env: dict | None):
     env = env or {}

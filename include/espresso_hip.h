@@ -308,6 +308,32 @@ typedef struct ESPPrepareOptions {
 int esp_gguf_prepare(const char *gguf_path, const char *output_dir, const ESPPrepareOptions *options_or_null,
                      ESPModelConfig *out_config, int *out_tensor_count);
 
+/* The prepared-artifact cache of GGUFModelLoader.prepare(ggufURL:options:) (GGUFModelLoader.swift:38-127, :273-296,
+ * :408-453, :472-566).  Options come from environment pairs as PrepareOptions.environment(_:) reads them
+ * (ESPRESSO_GGUF_FORCE_FRESH_PREPARE, ESPRESSO_GGUF_PREPARE_CACHE, ESPRESSO_GGUF_PREPARE_CACHE_ROOT,
+ * ESPRESSO_GGUF_SIDECAR_POLICY, ESPRESSO_GGUF_SELECTED_SIDECARS); the converter switches among the pairs enter the
+ * cache key (:595-605). */
+enum { ESP_SIDECAR_AUTOMATIC = 0, ESP_SIDECAR_NONE = 1, ESP_SIDECAR_ESSENTIAL = 2, ESP_SIDECAR_SELECTED = 3, ESP_SIDECAR_FULL = 4 };
+typedef struct ESPPrepareCacheOptions {
+    int32_t cache_enabled;            /* PrepareOptions.artifactCacheMode */
+    int32_t sidecar_mode;             /* ESP_SIDECAR_* */
+    char cache_root[1024];            /* "" = the default root */
+    char selected_sidecars[2048];     /* sorted tensor names, comma separated (sidecar_mode == ESP_SIDECAR_SELECTED) */
+} ESPPrepareCacheOptions;
+int esp_gguf_prepare_options_from_environment(const char *const *env_keys, const char *const *env_values, int env_count,
+                                              ESPPrepareCacheOptions *out);
+/* 64 hexadecimal digits + NUL into out_key (artifactCacheKey, :424-447). */
+int esp_gguf_artifact_cache_key(const char *gguf_path, const ESPPrepareCacheOptions *options, const char *const *env_keys,
+                                const char *const *env_values, int env_count, char *out_key, size_t out_key_bytes);
+/* prepare(ggufURL:options:): the cached directory when one matches, else a conversion into <cache root>/<key> (cache
+ * on) or a fresh temporary directory (cache off).  out_weight_dir receives the directory. */
+int esp_gguf_prepare_cached(const char *gguf_path, const ESPPrepareCacheOptions *options, const ESPPrepareOptions *convert_or_null,
+                            const char *const *env_keys, const char *const *env_values, int env_count, ESPModelConfig *out_config,
+                            int *out_tensor_count, char *out_weight_dir, size_t out_weight_dir_bytes);
+/* GGUFModelLoader.cleanup(weightDir:) (:408-412): removes the directory unless it is a managed cache entry. */
+int esp_gguf_cleanup(const char *weight_dir);
+int esp_gguf_default_cache_root(char *out, size_t out_bytes);
+
 /* ---- engine -------------------------------------------------------------------------------------- *
  * RealModelInferenceEngine.build(config:weightDir:tokenizerDir:) (RealModelInferenceEngine.swift:1377):
  * loads the weight directory into HBM (per tensor: packed sidecar, else float32 sidecar, else fp16
@@ -344,6 +370,24 @@ int esp_engine_generate_text(ESPEngine *engine, const char *prompt_utf8, size_t 
                              const char *const *env_keys, const char *const *env_values, int env_count,
                              uint32_t *out_tokens, char *out_text, size_t text_capacity, size_t *out_text_bytes,
                              ESPGenerationResult *result);
+
+/* RunGGUF.main(ggufPath:tokenizerDir:prompt:maxTokens:) (Sources/EspressoGGUF/RunGGUF.swift:68-113, the body of the
+ * runner's `<gguf> <tokenizer-dir> <prompt> [max]` form, Sources/EspressoGGUFRunner/main.swift:43-57): prepare with
+ * PrepareOptions.environment, build the engine with the tokenizer directory, generate greedily from the prompt text,
+ * then GGUFModelLoader.cleanup unless ESPRESSO_GGUF_KEEP_WEIGHT_DIR=1 (a managed cache entry is kept either way).
+ * The environment pairs stand for the process environment the reference reads.  Text output as in
+ * esp_engine_generate_text; out_tokens holds max_tokens ids.  The verify-qwen form needs the Qwen3 model file and its
+ * golden tokens (RunGGUF.swift:115-214) and is not part of this library. */
+typedef struct ESPRunGGUFInfo {
+    ESPModelConfig config;
+    int32_t tensor_count;
+    int32_t kept_weight_dir;      /* 1: the directory still exists after the call */
+    double prepare_ms, build_ms;
+    char weight_dir[1024];
+} ESPRunGGUFInfo;
+int esp_run_gguf(const char *gguf_path, const char *tokenizer_dir, const char *prompt_utf8, size_t prompt_bytes, int max_tokens,
+                 const char *const *env_keys, const char *const *env_values, int env_count, uint32_t *out_tokens, char *out_text,
+                 size_t text_capacity, size_t *out_text_bytes, ESPGenerationResult *result, ESPRunGGUFInfo *info);
 
 /* ---- tokenizers ----------------------------------------------------------------------------------- *
  * The Tokenizer protocol (Sources/ModelSupport/Tokenizer.swift:1-5: encode, decode, vocabSize) and its two

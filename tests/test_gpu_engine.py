@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import model_util as mu
-from gguf_writer import write_gguf
+from gguf_writer import gguf_model, write_gguf
 from oracle import oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -144,60 +144,6 @@ def test_exact_two_token_draft_through_environment(E, tmp_path):
     with pytest.raises(lib.EspressoError, match="vocab mismatch"):
         e.generate(PROMPT, 4, environment=env)
     e.close()
-
-
-def gguf_model(path, kw, w, arch, matrix_fmt, tied=False, interleave_qk=True):
-    """Writes a llama-family GGUF file the way llama.cpp's converter lays it out; returns the fp32 values
-    (in the half-split row order the decoder uses) that the packed tensors decode to."""
-    hd, half = kw["head_dim"], kw["head_dim"] // 2
-
-    def gguf_rows(a, heads):   # stored row (h, j, s) <- half-split row (h, s, j)
-        if not interleave_qk:
-            return a
-        r = a.reshape(heads, 2, half, a.shape[1])
-        return np.ascontiguousarray(r.transpose(0, 2, 1, 3)).reshape(a.shape)
-
-    meta = {"general.architecture": arch, f"{arch}.block_count": kw["n_layer"], f"{arch}.attention.head_count": kw["n_head"],
-            f"{arch}.attention.head_count_kv": kw["n_kv_head"], f"{arch}.embedding_length": kw["d_model"],
-            f"{arch}.feed_forward_length": kw["hidden_dim"], f"{arch}.context_length": kw["max_seq"],
-            f"{arch}.attention.layer_norm_rms_epsilon": 1e-5, f"{arch}.rope.freq_base": 10000.0,
-            "tokenizer.ggml.tokens": [f"t{i}" for i in range(kw["vocab"])], "tokenizer.ggml.eos_token_id": 2,
-            "general.name": "unit-test"}
-    tensors, seen = [], {"layers": []}
-
-    def quant(a):
-        blocks = orc.quantize(matrix_fmt, a)
-        return blocks, orc.dequantize(matrix_fmt, blocks, a.size).reshape(a.shape)
-
-    emb16 = w["embedding"].astype(np.float16)
-    tensors.append(("token_embd.weight", 1, w["embedding"].shape, emb16.tobytes()))
-    seen["embedding"] = emb16.astype(np.float32)
-    tensors.append(("output_norm.weight", 0, w["final_norm"].shape, w["final_norm"].astype("<f4").tobytes()))
-    seen["final_norm"] = w["final_norm"]
-    if tied:
-        seen["lm_head"] = seen["embedding"]
-    else:
-        b, seen["lm_head"] = quant(w["lm_head"])
-        tensors.append(("output.weight", matrix_fmt, w["lm_head"].shape, b.tobytes()))
-    names = {"wq": "attn_q", "wk": "attn_k", "wv": "attn_v", "wo": "attn_output", "w1": "ffn_gate", "w2": "ffn_down", "w3": "ffn_up"}
-    for l, L in enumerate(w["layers"]):
-        S = {}
-        for k, a in L.items():
-            if k in names:
-                b, S[k] = quant(a)
-                stored = a
-                if k == "wq": stored = gguf_rows(a, kw["n_head"])
-                if k == "wk": stored = gguf_rows(a, kw["n_kv_head"])
-                if stored is not a:
-                    b = orc.quantize(matrix_fmt, stored)      # blocks lie within rows, so this is a row permutation of `b`
-                tensors.append((f"blk.{l}.{names[k]}.weight", matrix_fmt, a.shape, b.tobytes()))
-            else:
-                g = {"rms_att": "attn_norm", "rms_ffn": "ffn_norm"}[k]
-                tensors.append((f"blk.{l}.{g}.weight", 0, a.shape, a.astype("<f4").tobytes()))
-                S[k] = a
-        seen["layers"].append(S)
-    write_gguf(path, meta, tensors)
-    return seen
 
 
 @pytest.mark.parametrize("arch,fmt,tied", [("llama", orc.FMT_Q8_0, False), ("llama", orc.FMT_Q4_K, True), ("qwen2", orc.FMT_Q4_0, False)])
@@ -443,3 +389,57 @@ acceptance_metric = "accepted_future_tokens"
     (root / "manifest.toml").write_text(manifest(draft_class="approximate"))
     text2, toks2, res2, _ = B.RuntimeBundle(str(root), verify_signatures=False).generate(prompt, 20)
     assert res2["exact_head_backend"] == "hip_gemv_argmax" and toks2 == toks and text2 == text
+
+
+def test_run_gguf_front_door(E, tmp_path):
+    """RunGGUF.main (RunGGUF.swift:68-113): prepare through the artifact cache, build with the tokenizer directory,
+    generate from the prompt text, clean up what is not a managed cache entry."""
+    import struct
+    import subprocess
+    import sys
+
+    import espresso_amd.tokenizer as T
+    w = mu.random_weights(orc.LlamaConfig(**KW), 71, std=0.08, norm_jitter=0.05)
+    path = str(tmp_path / "m.gguf")
+    seen = gguf_model(path, KW, w, "llama", orc.FMT_Q8_0)
+    pieces = [("▁", 0.0)] + [(chr(97 + i), 0.0) for i in range(26)] + [("▁the", 3.0), ("th", 1.0), ("▁th", 2.0)] + [(f"<0x{b:02X}>", 0.0) for b in range(256)]
+    pieces += [(f"zz{i}", 0.0) for i in range(KW["vocab"] - len(pieces))]
+    tok_dir = tmp_path / "tok"
+    tok_dir.mkdir()
+    data = struct.pack("<i", 16)
+    for piece, score in pieces:
+        raw = piece.encode()
+        data += struct.pack("<fi", score, len(raw)) + raw
+    (tok_dir / "tokenizer.model").write_bytes(data)
+    tok = T.Tokenizer.from_dir(gpu_cfg(KW), str(tok_dir))
+    prompt = "the cat"
+    ids = tok.encode(prompt)
+    want = oracle_tokens(dict(KW, eos_token=2), seen, ids, 10)
+
+    cache = tmp_path / "cache"
+    env = {"ESPRESSO_GGUF_PREPARE_CACHE_ROOT": str(cache)}
+    r = E.run_gguf(path, str(tok_dir), prompt, 10, env)
+    assert r["tokens"] == want and r["text"] == tok.decode(ids + want)
+    assert r["tensor_count"] == 3 + 9 * KW["n_layer"] and r["config"].d_model == KW["d_model"]
+    assert r["kept_weight_dir"] and os.path.dirname(r["weight_dir"]) == str(cache)      # a managed cache entry survives cleanup
+    again = E.run_gguf(path, str(tok_dir), prompt, 10, env)
+    assert again["weight_dir"] == r["weight_dir"] and again["tokens"] == want
+    # cache off: a temporary directory, removed unless ESPRESSO_GGUF_KEEP_WEIGHT_DIR=1
+    off = E.run_gguf(path, str(tok_dir), prompt, 4, {"ESPRESSO_GGUF_PREPARE_CACHE": "0"})
+    assert off["tokens"] == want[:4] and not off["kept_weight_dir"] and not os.path.exists(off["weight_dir"])
+    kept = E.run_gguf(path, str(tok_dir), prompt, 4, {"ESPRESSO_GGUF_FORCE_FRESH_PREPARE": "1", "ESPRESSO_GGUF_KEEP_WEIGHT_DIR": "1"})
+    assert kept["kept_weight_dir"] and os.path.exists(os.path.join(kept["weight_dir"], "metadata.json"))
+    E.gguf_cleanup(kept["weight_dir"])
+    # a missing tokenizer fails the build and still cleans up
+    import espresso_amd._lib as lib
+    with pytest.raises(lib.EspressoError):
+        E.run_gguf(path, str(tmp_path / "no-tokenizer"), prompt, 4, {"ESPRESSO_GGUF_PREPARE_CACHE": "0"})
+    # the runner's command line: text on stdout, the report on stderr, exit status 1 with usage when arguments are missing
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    run = subprocess.run([sys.executable, "-m", "espresso_amd.run_gguf", path, str(tok_dir), prompt, "10"], cwd=root, capture_output=True, text=True,
+                         env=dict(os.environ, **env), timeout=300)
+    assert run.returncode == 0, run.stderr
+    assert run.stdout.rstrip("\n") == r["text"]
+    assert "Tokens generated: 10" in run.stderr and "Prepared: llama, 2 layers" in run.stderr
+    short = subprocess.run([sys.executable, "-m", "espresso_amd.run_gguf", path], cwd=root, capture_output=True, text=True, timeout=120)
+    assert short.returncode == 1 and "Usage" in short.stderr

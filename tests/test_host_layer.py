@@ -212,3 +212,109 @@ def test_sample_token_follows_reference_rule():
     counts = np.bincount([eng.sample_token(small, 1.0, v) for v in units], minlength=4) / 20000
     p = np.exp(small - small.max()); p /= p.sum()
     assert np.abs(counts - p).max() < 0.015
+
+
+# ---- prepared-artifact cache of the GGUF front door (Tests/EspressoGGUFTests/GGUFModelLoaderTests.swift:110-176) ----
+def test_prepare_options_parse_cache_and_sidecar_controls_from_the_environment():
+    o = eng.PrepareOptions.environment({
+        "ESPRESSO_GGUF_PREPARE_CACHE": "0",
+        "ESPRESSO_GGUF_PREPARE_CACHE_ROOT": "/tmp/espresso-cache",
+        "ESPRESSO_GGUF_SIDECAR_POLICY": "selected",
+        "ESPRESSO_GGUF_SELECTED_SIDECARS": "blk.27.attn_q.weight, blk.27.attn_k.weight",
+    })
+    assert o.artifact_cache_enabled is False
+    assert o.cache_root == "/tmp/espresso-cache"
+    assert o.sidecar_mode == "selected" and o.selected_sidecars == {"blk.27.attn_q.weight", "blk.27.attn_k.weight"}
+    # defaults, the force-fresh switch, spellings of the policy, an unknown policy
+    d = eng.PrepareOptions.environment({})
+    assert d.artifact_cache_enabled and d.cache_root is None and d.sidecar_mode == "automatic" and not d.selected_sidecars
+    assert not eng.PrepareOptions.environment({"ESPRESSO_GGUF_FORCE_FRESH_PREPARE": "yes", "ESPRESSO_GGUF_PREPARE_CACHE": "1"}).artifact_cache_enabled
+    assert eng.PrepareOptions.environment({"ESPRESSO_GGUF_PREPARE_CACHE": " On "}).artifact_cache_enabled
+    for raw, mode in (("OFF", "none"), (" none ", "none"), ("auto", "automatic"), ("Essential", "essential"), ("full", "full"), ("bogus", "automatic")):
+        assert eng.PrepareOptions.environment({"ESPRESSO_GGUF_SIDECAR_POLICY": raw}).sidecar_mode == mode
+    assert eng.PrepareOptions.environment({"ESPRESSO_GGUF_PREPARE_CACHE_ROOT": "   "}).cache_root is None
+    assert eng.PrepareOptions.environment({"ESPRESSO_GGUF_PREPARE_CACHE_ROOT": "~/c"}).cache_root == os.path.expanduser("~/c")
+
+
+def test_artifact_cache_key_tracks_prepare_options(tmp_path):
+    path = tmp_path / "k.gguf"
+    path.write_bytes(b"QGUF")
+    essential = eng.gguf_artifact_cache_key(str(path), eng.PrepareOptions(sidecar_mode="essential"))
+    assert essential == eng.gguf_artifact_cache_key(str(path), eng.PrepareOptions(sidecar_mode="essential"))
+    selected = eng.gguf_artifact_cache_key(str(path), eng.PrepareOptions(sidecar_mode="selected", selected_sidecars=["blk.27.attn_q.weight"]))
+    assert essential != selected and re.fullmatch(r"[0-9a-f]{64}", essential)
+    # the selection, the converter's switches, the file's size and its path all enter the key; other variables do not
+    assert selected != eng.gguf_artifact_cache_key(str(path), eng.PrepareOptions(sidecar_mode="selected", selected_sidecars=["blk.27.attn_k.weight"]))
+    assert essential != eng.gguf_artifact_cache_key(str(path), eng.PrepareOptions(sidecar_mode="essential"), {"ESPRESSO_FORCE_QK_INVERSE_INTERLEAVE": "1"})
+    assert essential == eng.gguf_artifact_cache_key(str(path), eng.PrepareOptions(sidecar_mode="essential"), {"HOME": "/elsewhere", "ESPRESSO_FORCE_QK_INVERSE_INTERLEAVE": ""})
+    assert essential == eng.gguf_artifact_cache_key(str(tmp_path / "sub" / ".." / "k.gguf"), eng.PrepareOptions(sidecar_mode="essential"))
+    path.write_bytes(b"QGUF+")
+    assert essential != eng.gguf_artifact_cache_key(str(path), eng.PrepareOptions(sidecar_mode="essential"))
+    with pytest.raises(lib.EspressoError):
+        eng.gguf_artifact_cache_key(str(tmp_path / "absent.gguf"), eng.PrepareOptions())
+
+
+def test_cleanup_removes_a_directory_and_keeps_managed_cache_entries(tmp_path):
+    plain = tmp_path / "espresso_gguf_test"
+    plain.mkdir()
+    (plain / "test.bin").write_bytes(b"\x01")
+    eng.gguf_cleanup(str(plain))
+    assert not plain.exists()
+    cached = tmp_path / "espresso_gguf_cached"
+    cached.mkdir()
+    (cached / ".espresso-gguf-cache-artifact").write_bytes(b"")
+    eng.gguf_cleanup(str(cached))
+    assert cached.exists()
+    assert eng.gguf_default_cache_root().endswith(os.path.join("Espresso", "gguf-prepared"))
+
+
+def test_prepare_through_the_artifact_cache(tmp_path):
+    import json
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import model_util as mu
+    from gguf_writer import gguf_model
+    kw = dict(n_layer=1, n_head=2, n_kv_head=1, d_model=64, head_dim=32, hidden_dim=256, vocab=256, max_seq=16)
+    w = mu.random_weights(orc.LlamaConfig(**kw), 5, std=0.08)
+    path = str(tmp_path / "m.gguf")
+    gguf_model(path, kw, w, "llama", orc.FMT_Q8_0)
+    root = tmp_path / "cache"
+    opts = eng.PrepareOptions(cache_root=str(root))
+    cfg, wdir, count = eng.gguf_prepare_cached(path, opts)
+    key = eng.gguf_artifact_cache_key(path, opts)
+    assert wdir == str(root / key) and count == 3 + 9 and cfg.d_model == 64
+    manifest = json.load(open(os.path.join(wdir, "prepare-manifest.json")))
+    assert manifest["tensorCount"] == count and manifest["ggufPath"] == path and manifest["sidecarMode"] == "automatic"
+    assert manifest["fileSize"] == os.path.getsize(path) and manifest["version"] == 1
+    assert os.path.exists(os.path.join(wdir, ".espresso-gguf-cache-artifact"))
+    # a second prepare returns the cached directory untouched (a file planted in it survives), and cleanup keeps it
+    open(os.path.join(wdir, "planted"), "w").close()
+    cfg2, wdir2, count2 = eng.gguf_prepare_cached(path, opts)
+    assert (wdir2, count2, cfg2.vocab) == (wdir, count, cfg.vocab) and os.path.exists(os.path.join(wdir, "planted"))
+    eng.gguf_cleanup(wdir)
+    assert os.path.isdir(wdir)
+    # an entry without its metadata is rebuilt
+    os.remove(os.path.join(wdir, "metadata.json"))
+    _, wdir3, _ = eng.gguf_prepare_cached(path, opts)
+    assert wdir3 == wdir and os.path.exists(os.path.join(wdir, "metadata.json")) and not os.path.exists(os.path.join(wdir, "planted"))
+    # other options, another entry; sidecar policy "none" writes no float32 sidecar, "selected" only the named tensor
+    none = eng.PrepareOptions(cache_root=str(root), sidecar_mode="none")
+    _, wdir_none, _ = eng.gguf_prepare_cached(path, none)
+    assert wdir_none != wdir and not os.path.exists(os.path.join(wdir_none, "rms_final.float32.bin"))
+    assert os.path.exists(os.path.join(wdir, "rms_final.float32.bin"))
+    sel = eng.PrepareOptions(cache_root=str(root), sidecar_mode="selected", selected_sidecars=["blk.0.attn_norm.weight"])
+    _, wdir_sel, _ = eng.gguf_prepare_cached(path, sel)
+    assert os.path.exists(os.path.join(wdir_sel, "layers/0/rms_att.float32.bin")) and not os.path.exists(os.path.join(wdir_sel, "rms_final.float32.bin"))
+    # cache off: a fresh temporary directory each time, no marker, removed by cleanup
+    off = eng.PrepareOptions(artifact_cache_enabled=False)
+    _, t1, _ = eng.gguf_prepare_cached(path, off)
+    _, t2, _ = eng.gguf_prepare_cached(path, off)
+    assert t1 != t2 and os.path.basename(t1).startswith("espresso_gguf_") and not os.path.exists(os.path.join(t1, ".espresso-gguf-cache-artifact"))
+    eng.gguf_cleanup(t1); eng.gguf_cleanup(t2)
+    assert not os.path.exists(t1) and not os.path.exists(t2)
+    # a file that is no GGUF container leaves no directory behind
+    bad = tmp_path / "bad.gguf"
+    bad.write_bytes(b"QGUF")
+    with pytest.raises(lib.EspressoError):
+        eng.gguf_prepare_cached(str(bad), opts)
+    assert not os.path.exists(str(root / eng.gguf_artifact_cache_key(str(bad), opts)))
