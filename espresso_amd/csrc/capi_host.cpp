@@ -137,6 +137,26 @@ int esp_model_config_write_metadata(const ESPModelConfig *config, const char *pa
     return writeFile(path, j.data(), j.size()) ? ESP_OK : fail(ESP_ERR_IO, "cannot write %s", path);
 }
 
+int esp_model_registry_count(void) { return (int)ModelRegistry::all().size(); }
+int esp_model_registry_at(int index, ESPModelConfig *out) {
+    if (!out || index < 0 || index >= (int)ModelRegistry::all().size()) return fail(ESP_ERR_INVALID_ARGUMENT, "model registry: index %d", index);
+    to_c(ModelRegistry::all()[(size_t)index], out);
+    return ESP_OK;
+}
+int esp_model_registry_config(const char *name, ESPModelConfig *out) {
+    if (!name || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "model registry: null argument");
+    const MultiModelConfig *c = ModelRegistry::config(name);
+    if (!c) return fail(ESP_ERR_INVALID_ARGUMENT, "model registry: no configuration named %s", name);
+    to_c(*c, out);
+    return ESP_OK;
+}
+int esp_classifier_strategy_select(const ESPModelConfig *config, int has_exact_float32_lm_head, char *out_label, size_t label_bytes) {
+    if (!config) return fail(ESP_ERR_INVALID_ARGUMENT, "classifier strategy: null config");
+    const ClassifierStrategy s = selectClassifierStrategy(from_c(*config), has_exact_float32_lm_head != 0);
+    if (out_label && label_bytes) { std::strncpy(out_label, exactHeadBackendLabel(s), label_bytes - 1); out_label[label_bytes - 1] = 0; }
+    return (int)s;
+}
+
 int esp_gguf_prepare(const char *gguf_path, const char *output_dir, const ESPPrepareOptions *o, ESPModelConfig *out_config,
                      int *out_tensor_count) {
     if (!gguf_path || !output_dir) return fail(ESP_ERR_INVALID_ARGUMENT, "null path");

@@ -1,5 +1,9 @@
 #include "model_support.h"
 
+#include <cctype>
+
+#include <algorithm>
+
 #include <sys/stat.h>
 
 #include <cstdio>
@@ -249,6 +253,64 @@ std::string validateMetadataIfPresent(const MultiModelConfig &config, const std:
     if (m.vocab != config.vocab) return mismatch("vocab", config.vocab, m.vocab);
     if (m.maxSeq != config.maxSeq) return mismatch("maxSeq", config.maxSeq, m.maxSeq);
     return "";
+}
+
+// ---- ModelRegistry ----------------------------------------------------------------------------------
+namespace {
+MultiModelConfig entry(const char *name, int nLayer, int nHead, int nKVHead, int dModel, int headDim, int hiddenDim, int vocab, int maxSeq,
+                       MultiModelConfig::Architecture arch, float ropeTheta = 10000.0f, long eos = -1) {
+    MultiModelConfig c;
+    c.name = name; c.nLayer = nLayer; c.nHead = nHead; c.nKVHead = nKVHead; c.dModel = dModel; c.headDim = headDim;
+    c.hiddenDim = hiddenDim; c.vocab = vocab; c.maxSeq = maxSeq; c.normEps = 1e-5f; c.ropeTheta = ropeTheta; c.architecture = arch;
+    if (eos >= 0) { c.hasEosToken = true; c.eosToken = (TokenID)eos; }
+    return c;
+}
+}  // namespace
+
+const std::vector<MultiModelConfig> &ModelRegistry::all() {
+    using A = MultiModelConfig::Architecture;
+    static const std::vector<MultiModelConfig> table = [] {
+        std::vector<MultiModelConfig> t = {
+            entry("gpt2_124m", 12, 12, 12, 768, 64, 3072, 50257, 1024, A::gpt2),
+            entry("stories110m", 12, 12, 12, 768, 64, 2048, 32000, 256, A::llama),
+            entry("smolLM_135m", 30, 9, 3, 576, 64, 1536, 49152, 2048, A::llama),
+            entry("tinyLlama_1_1b", 22, 32, 4, 2048, 64, 5632, 32000, 2048, A::llama),
+            entry("llama3_2_1b", 16, 32, 8, 2048, 64, 8192, 128256, 2048, A::llama, 500000.0f, 128001),
+            entry("llama3_2_1b_ctx512", 16, 32, 8, 2048, 64, 8192, 128256, 512, A::llama, 500000.0f, 128001),
+            entry("llama3_2_3b", 28, 24, 8, 3072, 128, 8192, 128256, 2048, A::llama, 500000.0f, 128001),
+        };
+        std::sort(t.begin(), t.end(), [](const MultiModelConfig &a, const MultiModelConfig &b) { return a.name < b.name; });
+        return t;
+    }();
+    return table;
+}
+
+const MultiModelConfig *ModelRegistry::config(const std::string &name) {
+    for (const MultiModelConfig &c : all()) if (c.name == name) return &c;
+    return nullptr;
+}
+
+// ---- ClassifierStrategy -----------------------------------------------------------------------------
+ClassifierStrategy selectClassifierStrategy(const MultiModelConfig &config, bool hasExactFloat32LMHead) {
+    constexpr long kANESRAMElementLimit = 16000000;   // 32 MB of fp16
+    size_t a = 0, b = config.name.size();
+    while (a < b && std::isspace((unsigned char)config.name[a])) a++;
+    while (b > a && std::isspace((unsigned char)config.name[b - 1])) b--;
+    std::string name = config.name.substr(a, b - a);
+    for (char &ch : name) ch = (char)std::tolower((unsigned char)ch);
+    const bool llama = config.architecture == MultiModelConfig::Architecture::llama;
+    if (llama && name.find("stories110m") != std::string::npos) return ClassifierStrategy::ane;   // the reference's allowlist entry
+    if ((long)config.vocab * (long)config.dModel <= kANESRAMElementLimit) return ClassifierStrategy::ane;
+    if (llama && !hasExactFloat32LMHead) return ClassifierStrategy::cpuFP16Tiled;
+    return ClassifierStrategy::cpuPartitionedFP32;
+}
+
+const char *exactHeadBackendLabel(ClassifierStrategy s) {
+    switch (s) {
+    case ClassifierStrategy::ane: return "ane_classifier";
+    case ClassifierStrategy::cpuPartitionedFP32: return "cpu_partitioned_fp32";
+    default: return "cpu_fp16_tiled";
+    }
 }
 
 }  // namespace esp

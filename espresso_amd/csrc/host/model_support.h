@@ -26,6 +26,19 @@ struct MultiModelConfig {
     int kvDim() const { return nKVHead * headDim; }
 };
 
+// ModelRegistry (Sources/ModelSupport/ModelRegistry.swift:1-122): the named configurations the reference ships.
+struct ModelRegistry {
+    static const std::vector<MultiModelConfig> &all();                 // sorted by name
+    static const MultiModelConfig *config(const std::string &name);   // nullptr when unknown
+};
+
+// ClassifierStrategy (Sources/RealModelInference/ClassifierStrategy.swift:11-69): which output head the reference
+// picks for a model.  Every strategy returns the first maximum of the same logits (Sources/Espresso/
+// PartitionedArgmax.swift:9), which is what the GPU head computes; the selection is kept for callers that report it.
+enum class ClassifierStrategy { ane = 0, cpuPartitionedFP32 = 1, cpuFP16Tiled = 2 };
+ClassifierStrategy selectClassifierStrategy(const MultiModelConfig &config, bool hasExactFloat32LMHead);
+const char *exactHeadBackendLabel(ClassifierStrategy s);
+
 // validateRuntimeConfig, RealModelInferenceEngine.swift:7615-7634.  Empty string = valid.
 std::string validateRuntimeConfig(const MultiModelConfig &c);
 

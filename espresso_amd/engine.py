@@ -87,13 +87,46 @@ def _ptr(a):
 
 def config_struct(cfg: llama.MultiModelConfig) -> ModelConfigStruct:
     return ModelConfigStruct(cfg.name.encode()[:63], cfg.n_layer, cfg.n_head, cfg.n_kv_head, cfg.d_model, cfg.head_dim, cfg.hidden_dim,
-                             cfg.vocab, cfg.max_seq, cfg.norm_eps, cfg.rope_theta, cfg.eos_token, 1)
+                             cfg.vocab, cfg.max_seq, cfg.norm_eps, cfg.rope_theta, cfg.eos_token, 0 if cfg.architecture == "gpt2" else 1)
 
 
 def config_from_struct(s: ModelConfigStruct) -> llama.MultiModelConfig:
     return llama.MultiModelConfig(n_layer=s.n_layer, n_head=s.n_head, n_kv_head=s.n_kv_head, d_model=s.d_model, head_dim=s.head_dim,
                                   hidden_dim=s.hidden_dim, vocab=s.vocab, max_seq=s.max_seq, norm_eps=s.norm_eps,
-                                  rope_theta=s.rope_theta, eos_token=s.eos_token, name=s.name.decode())
+                                  rope_theta=s.rope_theta, eos_token=s.eos_token, name=s.name.decode(),
+                                  architecture="gpt2" if s.architecture == 0 else "llama")
+
+
+# ---- registry and head strategy ----------------------------------------------
+def model_registry() -> dict:
+    """ModelRegistry.all: {name: config}."""
+    L = _L()
+    out = {}
+    for i in range(L.esp_model_registry_count()):
+        s = ModelConfigStruct()
+        _lib.check(L.esp_model_registry_at(i, C.byref(s)))
+        out[s.name.decode()] = config_from_struct(s)
+    return out
+
+
+def model_registry_config(name: str):
+    """ModelRegistry.config(named:): None when unknown."""
+    s = ModelConfigStruct()
+    return config_from_struct(s) if _L().esp_model_registry_config(name.encode(), C.byref(s)) == 0 else None
+
+
+CLASSIFIER_STRATEGIES = ("ane", "cpuPartitionedFP32", "cpuFP16Tiled")
+
+
+def classifier_strategy(cfg: llama.MultiModelConfig, has_exact_float32_lm_head: bool = False) -> tuple[str, str]:
+    """ClassifierStrategy.select -> (case name, exactHeadBackendLabel)."""
+    L = _L()
+    L.esp_classifier_strategy_select.restype = C.c_int
+    s, label = config_struct(cfg), C.create_string_buffer(48)
+    k = L.esp_classifier_strategy_select(C.byref(s), int(has_exact_float32_lm_head), label, C.c_size_t(48))
+    if k < 0:
+        raise _lib.EspressoError(k, _lib.last_error())
+    return CLASSIFIER_STRATEGIES[k], label.value.decode()
 
 
 # ---- weight files -----------------------------------------------------------

@@ -30,6 +30,7 @@ class MultiModelConfig:
     rope_theta: float = 10000.0
     eos_token: int = -1
     name: str = "llama"
+    architecture: str = "llama"   # or "gpt2" (registry entries only: the runtime runs the llama family)
 
     @property
     def attention_dim(self) -> int:

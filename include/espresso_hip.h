@@ -292,6 +292,16 @@ typedef struct ESPModelConfig {
 int esp_model_config_load_metadata(const char *metadata_json_path, ESPModelConfig *out);
 int esp_model_config_write_metadata(const ESPModelConfig *config, const char *metadata_json_path);
 
+/* ModelRegistry (Sources/ModelSupport/ModelRegistry.swift): esp_model_registry_count() named configurations in name
+ * order; esp_model_registry_config(name, &out) = ModelRegistry.config(named:), ESP_ERR_INVALID_ARGUMENT when unknown. */
+int esp_model_registry_count(void);
+int esp_model_registry_at(int index, ESPModelConfig *out);
+int esp_model_registry_config(const char *name, ESPModelConfig *out);
+/* ClassifierStrategy.select(for:hasExactFloat32LMHead:) (Sources/RealModelInference/ClassifierStrategy.swift:46-69):
+ * returns 0 ane, 1 cpuPartitionedFP32, 2 cpuFP16Tiled and writes exactHeadBackendLabel (:31-40) when out_label is given.
+ * All three return the first maximum of the same logits; the GPU head does too. */
+int esp_classifier_strategy_select(const ESPModelConfig *config, int has_exact_float32_lm_head, char *out_label, size_t label_bytes);
+
 /* ---- GGUF front door ---------------------------------------------------------------------------- *
  * GGUFModelLoader.prepare(ggufURL:options:) -> PreparedModel (GGUFModelLoader.swift:273-405): parses
  * the GGUF container, maps its metadata to a MultiModelConfig (:297-326) and writes a weight directory:

@@ -318,3 +318,42 @@ def test_prepare_through_the_artifact_cache(tmp_path):
     with pytest.raises(lib.EspressoError):
         eng.gguf_prepare_cached(str(bad), opts)
     assert not os.path.exists(str(root / eng.gguf_artifact_cache_key(str(bad), opts)))
+
+
+# ---- ModelRegistry (Tests/ModelSupportTests/ModelConfigTests.swift:5-52) and ClassifierStrategy.select
+# (Tests/RealModelInferenceTests/ClassifierStrategyTests.swift:6-148) ----
+def test_model_registry_matches_the_reference_table():
+    reg = eng.model_registry()
+    assert len(reg) == 7 and list(reg) == sorted(reg)
+    gpt2, stories = eng.model_registry_config("gpt2_124m"), eng.model_registry_config("stories110m")
+    assert (gpt2.vocab, gpt2.hidden_dim, gpt2.architecture) == (50257, 3072, "gpt2")
+    assert (stories.vocab, stories.hidden_dim, stories.architecture) == (32000, 2048, "llama")
+    assert reg["smolLM_135m"].n_kv_head == 3 and reg["tinyLlama_1_1b"].n_head == 32 and reg["llama3_2_1b_ctx512"].max_seq == 512
+    c = reg["llama3_2_1b"]
+    assert (c.n_layer, c.n_head, c.n_kv_head, c.d_model, c.head_dim, c.hidden_dim, c.vocab, c.max_seq) == (16, 32, 8, 2048, 64, 8192, 128256, 2048)
+    assert c.d_model == c.n_head * c.head_dim and c.rope_theta == 500000.0 and c.eos_token == 128001
+    c = reg["llama3_2_3b"]
+    assert (c.n_layer, c.n_head, c.n_kv_head, c.d_model, c.head_dim, c.hidden_dim, c.vocab, c.max_seq) == (28, 24, 8, 3072, 128, 8192, 128256, 2048)
+    assert c.d_model == c.n_head * c.head_dim
+    assert reg["stories110m"].eos_token == -1 and reg["stories110m"].rope_theta == 10000.0
+    assert eng.model_registry_config("no-such-model") is None
+
+
+def _cfg(name, d_model, vocab, architecture="llama"):
+    return ll.MultiModelConfig(n_layer=1, n_head=1, n_kv_head=1, d_model=d_model, head_dim=64, hidden_dim=128, vocab=vocab, max_seq=32,
+                               name=name, architecture=architecture)
+
+
+def test_classifier_strategy_selection():
+    S = eng.classifier_strategy
+    assert S(_cfg("tiny-test", 64, 256)) == ("ane", "ane_classifier")
+    assert S(_cfg("tinyllama-test", 2048, 32000)) == ("cpuFP16Tiled", "cpu_fp16_tiled")          # 65.5 M elements > 16 M
+    assert S(eng.model_registry_config("stories110m"))[0] == "ane"                                 # the allowlist entry
+    assert S(_cfg("llama2.c-stories110M", 768, 32000))[0] == "ane"                                 # bundle-style name
+    assert S(_cfg("  Stories110M ", 768, 32000))[0] == "ane"
+    assert S(_cfg("stories110m", 768, 50257, "gpt2"))[0] == "cpuPartitionedFP32"                   # the allowlist is for llama only
+    assert S(_cfg("tinyllama-test", 2048, 32000), True) == ("cpuPartitionedFP32", "cpu_partitioned_fp32")
+    assert S(_cfg("qwen3-0.6b-test", 1024, 151936))[0] == "cpuFP16Tiled"
+    assert S(_cfg("gpt2-large-vocab", 768, 50257, "gpt2"))[0] == "cpuPartitionedFP32"
+    assert S(_cfg("boundary-test", 64, 250000))[0] == "ane"                                        # exactly 16 M elements
+    assert S(_cfg("boundary-plus-one", 64, 250001))[0] == "cpuFP16Tiled"
