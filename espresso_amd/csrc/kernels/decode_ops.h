@@ -71,6 +71,11 @@ hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_toke
 hipError_t launch_set_rows(const StepRows &rows, int *tokens, int *pos, int *seq, hipStream_t s);
 hipError_t launch_greedy_feed(const int *next_token, int seq, int *visible, int *tokens, int *pos, int *seqs, int *log,
                               int *log_count, int log_capacity, hipStream_t s);
+// A greedy step's end in two launches instead of four: the argmax slices of the row of logits, then one workgroup
+// that reduces them, feeds the token as launch_greedy_feed does and writes its embedding row to hidden[0..d).
+hipError_t launch_greedy_step_tail(const float *logits, int vocab, int *out_token, const ArgmaxScratch &scratch, int seq, int *visible,
+                                   int *tokens, int *pos, int *seqs, int *log, int *log_count, int log_capacity, const void *table,
+                                   bool table_is_f16, int d, float *hidden, hipStream_t s);
 hipError_t launch_set_ints(int *dst0, int v0, int *dst1, int v1, hipStream_t s);
 hipError_t launch_copy_rows(const float *src, float *dst, int rows, int d, hipStream_t s);
 

@@ -656,6 +656,48 @@ __global__ void greedy_feed_kernel(const int *next_token, int seq, int *visible,
     visible[seq] += 1;
 }
 
+// The end of a greedy step in one launch: reduce the argmax slices of row 0 (argmax_final_kernel), feed the token
+// (greedy_feed_kernel) and fetch its embedding row as the next trunk pass's input (embed_kernel).
+struct GreedyTailArgs {
+    const float *part_value;
+    const int *part_index;
+    int nblk;
+    int *out_token;
+    int seq;
+    int *visible, *tokens, *pos, *seqs, *log, *log_count;
+    int log_capacity;
+    const void *table;
+    int table_is_f16, d;
+    float *hidden;
+};
+__global__ __launch_bounds__(kBlock) void greedy_tail_kernel(GreedyTailArgs a) {
+    __shared__ float bv[kBlock];
+    __shared__ int bi[kBlock];
+    float best = -INFINITY;
+    int best_i = 0x7FFFFFFF;
+    for (int i = threadIdx.x; i < a.nblk; i += kBlock) {
+        const float v = a.part_value[i];
+        const int idx = a.part_index[i];
+        if (better(v, idx, best, best_i)) { best = v; best_i = idx; }
+    }
+    argmax_block_reduce(best, best_i, bv, bi);
+    const int t = best_i == 0x7FFFFFFF ? 0 : best_i;
+    if (threadIdx.x == 0) {
+        a.out_token[0] = t;
+        a.tokens[0] = t;
+        a.pos[0] = a.visible[a.seq];
+        a.seqs[0] = a.seq;
+        const int n = *a.log_count;
+        if (n < a.log_capacity) a.log[n] = t;
+        *a.log_count = n + 1;
+        a.visible[a.seq] += 1;
+    }
+    const size_t row = (size_t)t * a.d;
+    for (int i = threadIdx.x; i < a.d; i += kBlock)
+        a.hidden[i] = a.table_is_f16 ? from_half_bits(reinterpret_cast<const uint16_t *>(a.table)[row + i])
+                                     : reinterpret_cast<const float *>(a.table)[row + i];
+}
+
 __global__ void set_ints_kernel(int *dst0, int v0, int *dst1, int v1) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         if (dst0) *dst0 = v0;
@@ -753,6 +795,18 @@ hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_toke
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(blocks, rows), dim3(kBlock), 0, s, logits, vocab, scratch.part_value, scratch.part_index);
     hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(kBlock), 0, s, scratch.part_value, scratch.part_index, blocks, out_token,
                        out_value);
+    return hipGetLastError();
+}
+
+hipError_t launch_greedy_step_tail(const float *logits, int vocab, int *out_token, const ArgmaxScratch &scratch, int seq, int *visible,
+                                   int *tokens, int *pos, int *seqs, int *log, int *log_count, int log_capacity, const void *table,
+                                   bool table_is_f16, int d, float *hidden, hipStream_t s) {
+    if (!scratch.part_value || !scratch.part_index) return hipErrorInvalidValue;
+    const int blocks = vocab < kArgmaxBlocks * kBlock ? (vocab + kBlock - 1) / kBlock : kArgmaxBlocks;
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(blocks, 1), dim3(kBlock), 0, s, logits, vocab, scratch.part_value, scratch.part_index);
+    GreedyTailArgs a{scratch.part_value, scratch.part_index, blocks, out_token, seq, visible, tokens, pos, seqs, log, log_count, log_capacity,
+                     table, table_is_f16 ? 1 : 0, d, hidden};
+    hipLaunchKernelGGL(greedy_tail_kernel, dim3(1), dim3(kBlock), 0, s, a);
     return hipGetLastError();
 }
 

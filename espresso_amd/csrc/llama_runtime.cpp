@@ -461,12 +461,12 @@ int LlamaRuntime::forward_rows(const StepRows &rows) {
 }
 
 // The trunk over `M` rows whose (token, position, sequence) already sit in d_tokens_/d_pos_/d_seq_.
-int LlamaRuntime::enqueue_trunk(int M) {
+int LlamaRuntime::enqueue_trunk(int M, bool embedded, float *final_out) {
     hipStream_t s = context().stream;
     const int d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
     const bool kv16 = c_.kv_format == FMT_F16;
     int rc = ESP_OK;
-    ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, M, d, hidden_, s));
+    if (!embedded) ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, M, d, hidden_, s));
     if (timing_enabled_) {   // an empty event pair: the overhead the pairs around real kernels carry
         if ((rc = time_begin(K_EVENT_PAIR)) != ESP_OK) return rc;
         if ((rc = time_end()) != ESP_OK) return rc;
@@ -535,7 +535,8 @@ int LlamaRuntime::enqueue_trunk(int M) {
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
         g.w = L.w2; g.x = act_; g.norm_x = nullptr; g.norm_w = nullptr;
-        g.y = hidden_; g.residual = hidden_; g.out_f16 = nullptr; g.epilogue = EPI_ADD_RESIDUAL;
+        g.y = final_out && &L == &layers_.back() ? final_out : hidden_;   // the last layer's output may go straight to its keeper
+        g.residual = hidden_; g.out_f16 = nullptr; g.epilogue = EPI_ADD_RESIDUAL;
         if ((rc = time_begin(K_DOWN)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
@@ -740,14 +741,30 @@ int LlamaRuntime::capture_step_graph(int seq) {
     hipGraph_t graph = nullptr;
     ESP_HIP_TRY(hipStreamSynchronize(s));
     ESP_HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
-    int rc = run_head(last_hidden_ + (size_t)seq * c_.d_model, 1);
-    if (rc == ESP_OK) {
-        hipError_t e = launch_greedy_feed(d_out_tokens_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_, d_log_count_,
-                                          c_.max_seq, s);
-        if (e != hipSuccess) rc = fail_hip(e, "greedy_feed");
+    int rc = ESP_OK;
+    float *kept = last_hidden_ + (size_t)seq * c_.d_model;
+    if (fused_trunk_active()) {
+        rc = run_head(kept, 1);
+        if (rc == ESP_OK) {
+            hipError_t e = launch_greedy_feed(d_out_tokens_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_, d_log_count_,
+                                              c_.max_seq, s);
+            if (e != hipSuccess) rc = fail_hip(e, "greedy_feed");
+        }
+        if (rc == ESP_OK) rc = enqueue_trunk(1);
+        if (rc == ESP_OK) rc = keep_row(0, seq);
+    } else {
+        // head GEMV, argmax slices, then one launch that picks the token, feeds it and fetches its embedding; the
+        // last layer writes the new hidden state where the next step's head reads it: 3 + 5 per layer launches
+        GemvParams g;
+        g.w = lm_head_; g.norm_x = kept; g.norm_w = final_norm_; g.norm_eps = c_.norm_eps;
+        g.y = logits_; g.batch = 1; g.epilogue = EPI_STORE_F32;
+        hipError_t e = launch_gemv(g, s);
+        if (e == hipSuccess)
+            e = launch_greedy_step_tail(logits_, c_.vocab, d_out_tokens_, argmax_scratch_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_,
+                                        d_log_count_, c_.max_seq, embedding_, embedding_f16_, c_.d_model, hidden_, s);
+        if (e != hipSuccess) rc = fail_hip(e, "greedy step head");
+        if (rc == ESP_OK) rc = enqueue_trunk(1, true, kept);
     }
-    if (rc == ESP_OK) rc = enqueue_trunk(1);
-    if (rc == ESP_OK) rc = keep_row(0, seq);
     hipError_t e = hipStreamEndCapture(s, &graph);
     if (rc != ESP_OK) { if (graph) (void)hipGraphDestroy(graph); return rc; }
     if (e != hipSuccess) return fail_hip(e, "hipStreamEndCapture");

@@ -104,7 +104,8 @@ class LlamaRuntime {
     };
     int upload_vector(const HostTensor &t, size_t count, float **out, const char *what);
     int run_head(const float *hidden_rows, int count);
-    int enqueue_trunk(int rows);
+    // embedded: hidden_ already holds the rows' embeddings; final_out: where the last layer writes (default hidden_)
+    int enqueue_trunk(int rows, bool embedded = false, float *final_out = nullptr);
     int prefill_block(int seq, const uint32_t *tokens, int rows, int base);
     int enqueue_layers_matrix(int rows);
     bool matrix_prefill_supported() const;
