@@ -130,6 +130,10 @@ __device__ __forceinline__ uint2 nibbles_to_half(u32 w, bool high, h2 s, h2 dm) 
 // fp32, so each weight is the dequantised value rounded to fp16 once (n * s and dm can both be several
 // times larger than their difference; rounding them separately in fp16 would cost two more bits).
 __device__ __forceinline__ uint2 q4k_bytes_to_half(u32 b, float s, float dm) {
+    // The empty statement hides where `b` came from: otherwise the compiler folds the caller's nibble mask into four
+    // bit-field extracts followed by byte conversions, two operations per weight where v_cvt_f32_ubyte0..3 on the masked
+    // word need one.
+    asm volatile("" : "+v"(b));
     const float w0 = __builtin_fmaf((float)(b & 0xFFu), s, -dm), w1 = __builtin_fmaf((float)((b >> 8) & 0xFFu), s, -dm);
     const float w2 = __builtin_fmaf((float)((b >> 16) & 0xFFu), s, -dm), w3 = __builtin_fmaf((float)(b >> 24), s, -dm);
     return make_uint2(as_u32(h2{(_Float16)w0, (_Float16)w1}), as_u32(h2{(_Float16)w2, (_Float16)w3}));
