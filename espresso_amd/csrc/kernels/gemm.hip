@@ -495,6 +495,173 @@ __global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(GemmArgs a) {
         }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Up to sixteen activation rows against Q4_K weights without dequantising them.  Below about sixteen rows the
+// register-B kernel above is bound by the exact dequantisation (three vector operations per weight however few rows
+// there are).  Here the B operand is the nibble itself under an fp16 exponent, as in the GEMV kernels: one
+// v_and_or_b32 turns two low nibbles into (64 + n/16, 64 + n/16) and two high nibbles into (4 + n/16, 4 + n/16),
+// exactly; two MFMAs contract a 32-weight sub-block into sum (offset + n/16) x with exact products, and scale and
+// minimum of the sub-block are folded into the few accumulator registers that hold real rows afterwards:
+//     sum_k (d sc n_k - dmin m) x_k = (16 d sc) raw - (16 d sc offset + dmin m) sum_k x_k,
+// with the sums of the activations over each sub-block computed once per workgroup while they are staged.
+// Lane mapping, loads, LDS staging of the activations (in (0,2,1,3) order inside fours, which is how the masked
+// nibble pairs come out) are those of gemm_skinny_kernel; the rows 0..7 are accumulator registers 0..3 of a lane.
+__device__ __forceinline__ float quad_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+    return v;
+}
+
+// The workgroup owns 32 weight rows and its WAVES wavefronts split K between them, so a launch has one workgroup per 32 rows
+// whatever K is, needs no split-K workspace and no reduce launch; the wavefronts' partial results meet in LDS and are added
+// in wavefront order.  The activations are staged a span of SPAN chunks (of 256 k) at a time into one of two LDS buffers: the
+// next span's are loaded into registers before the current span is computed and written after it, one barrier per span.
+// Inside a span wavefront w takes chunks w, w + WAVES, ...; the packed weights of its chunks of the next two spans are always
+// in flight (they do not wait for the staging).  Short spans measure faster than long ones (one chunk per wavefront and span:
+// 15.7 us for 14336 x 4096 against 18.2 us with two and 17.9 us with all of K staged at once), and eight wavefronts
+// faster than four when the rows fill no more than one workgroup per compute unit.
+constexpr int kRowsMaxRows = 8;
+template <int WAVES, int SPAN> constexpr size_t rows_lds_bytes() {
+    return 2 * ((size_t)kRowsMaxRows * (SPAN * CK + 8) * 2 + (size_t)SPAN * 8 * kRowsMaxRows * 4) + (size_t)WAVES * 4 * 64 * 4;
+}
+
+template <int WAVES, int SPAN>
+__global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gemm_rows_q4k_kernel(GemmArgs a) {
+    constexpr int MR = kRowsMaxRows, THREADS = WAVES * 64, LDW = SPAN * CK + 8;
+    constexpr int CPW = SPAN / WAVES;                     // chunks per wavefront and span
+    constexpr int PIECES = MR * SPAN * 32 / THREADS;      // 128-bit pieces of x per thread and span
+    extern __shared__ uint4 rows_smem[];
+    _Float16 *xt_base = reinterpret_cast<_Float16 *>(rows_smem);               // [2][MR][LDW]
+    float *xsum_base = reinterpret_cast<float *>(xt_base + 2 * MR * LDW);      // [2][SPAN * 8 sub-blocks][MR]
+    float *red = xsum_base + 2 * SPAN * 8 * MR;                                // [WAVES][4][64]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+    const int n = blockIdx.x * 32 + (lane & 31);
+    const int w_row = n < a.N ? n : a.N - 1;     // clamped, the result is never stored
+    const int chunks = a.K / CK, spans = (chunks + SPAN - 1) / SPAN;
+    // constants of the nibble trick, hidden from the optimiser so that (w & mask) | magic stays one v_and_or_b32
+    u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x54005400u, magic_hi = 0x44004400u;
+    asm volatile("" : "+s"(mask_lo), "+s"(mask_hi));
+    asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
+
+    float total[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto chunk_of = [&](int sp, int j) { return sp * SPAN + j * WAVES + wave; };
+    RawChunk<FMT_Q4_K> ring[2 * CPW];
+#pragma unroll
+    for (int q = 0; q < 2 * CPW; q++)
+        if (chunk_of(q / CPW, q % CPW) < chunks) ring[q] = fetch_chunk<FMT_Q4_K>(a, w_row, chunk_of(q / CPW, q % CPW), h);
+
+    uint4 xv[PIECES];
+    auto load_x = [&](int sp) {
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const int piece = tid + i * THREADS, row = piece / (SPAN * 32), part = piece % (SPAN * 32);
+            const int k0 = sp * SPAN * CK + part * 8;
+            xv[i] = row < a.M && k0 < a.K ? *reinterpret_cast<const uint4 *>(a.x + (size_t)row * a.K + k0) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    // (0,2,1,3) order inside fours, sums of every 32 alongside
+    auto store_x = [&](int buf) {
+        _Float16 *xt = xt_base + buf * MR * LDW;
+        float *xsum = xsum_base + buf * SPAN * 8 * MR;
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const int piece = tid + i * THREADS, row = piece / (SPAN * 32), part = piece % (SPAN * 32);
+            *reinterpret_cast<uint4 *>(xt + row * LDW + part * 8) = swap_middle(xv[i]);
+            const h2 p0 = as_h2(xv[i].x), p1 = as_h2(xv[i].y), p2 = as_h2(xv[i].z), p3 = as_h2(xv[i].w);
+            float sum = (((float)p0.x + (float)p0.y) + ((float)p1.x + (float)p1.y)) + (((float)p2.x + (float)p2.y) + ((float)p3.x + (float)p3.y));
+            sum = quad_sum(sum);                 // the four pieces of a 32-weight sub-block sit in one quad of lanes
+            if ((part & 3) == 0) xsum[(part >> 2) * MR + row] = sum;
+        }
+    };
+    auto compute_span = [&](int sp, auto parity) {
+        constexpr int P = decltype(parity)::value;
+        const _Float16 *xt = xt_base + P * MR * LDW;
+        const float *xsum = xsum_base + P * SPAN * 8 * MR;
+#pragma unroll
+        for (int j = 0; j < CPW; j++) {
+            const int c = chunk_of(sp, j);
+            if (c < chunks) {
+                const RawChunk<FMT_Q4_K> r = ring[P * CPW + j];
+                if (chunk_of(sp + 2, j) < chunks) ring[P * CPW + j] = fetch_chunk<FMT_Q4_K>(a, w_row, chunk_of(sp + 2, j), h);
+                const float dd = half_bits_to_float(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float(r.hdr.x >> 16);
+                const int local = j * WAVES + wave;   // chunk index inside the span
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    float sc_lo, m_lo, sc_hi, m_hi;
+                    q4k_scale_min(r.hdr, 2 * t, sc_lo, m_lo);
+                    q4k_scale_min(r.hdr, 2 * t + 1, sc_hi, m_hi);
+                    const float a_lo = 16.0f * dd * sc_lo, b_lo = 64.0f * a_lo + dmin * m_lo;
+                    const float a_hi = 16.0f * dd * sc_hi, b_hi = 4.0f * a_hi + dmin * m_hi;
+                    half8 frag[4];
+                    {
+                        const u32 w0 = r.q[t].x, w1 = r.q[t].y, w2 = r.q[t].z, w3 = r.q[t].w;
+                        frag[0] = as_half8(make_uint4((w0 & mask_lo) | magic_lo, ((w0 >> 8) & mask_lo) | magic_lo, (w1 & mask_lo) | magic_lo, ((w1 >> 8) & mask_lo) | magic_lo));
+                        frag[1] = as_half8(make_uint4((w2 & mask_lo) | magic_lo, ((w2 >> 8) & mask_lo) | magic_lo, (w3 & mask_lo) | magic_lo, ((w3 >> 8) & mask_lo) | magic_lo));
+                        frag[2] = as_half8(make_uint4((w0 & mask_hi) | magic_hi, ((w0 >> 8) & mask_hi) | magic_hi, (w1 & mask_hi) | magic_hi, ((w1 >> 8) & mask_hi) | magic_hi));
+                        frag[3] = as_half8(make_uint4((w2 & mask_hi) | magic_hi, ((w2 >> 8) & mask_hi) | magic_hi, (w3 & mask_hi) | magic_hi, ((w3 >> 8) & mask_hi) | magic_hi));
+                    }
+                    // rows of x beyond MR alias real ones: they only reach accumulator registers that are never read
+                    const _Float16 *xrow = xt + ((lane & 31) & (MR - 1)) * LDW + local * CK + t * KT;
+                    floatx16 lo, hi;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) lo[i] = hi[i] = 0.0f;
+                    lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 16 * h), frag[0], lo, 0, 0, 0);
+                    hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 32 + 16 * h), frag[2], hi, 0, 0, 0);
+                    lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 16 * h + 8), frag[1], lo, 0, 0, 0);
+                    hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 40 + 16 * h), frag[3], hi, 0, 0, 0);
+                    const float4 xs_lo = *reinterpret_cast<const float4 *>(xsum + (local * 8 + 2 * t) * MR + 4 * h);
+                    const float4 xs_hi = *reinterpret_cast<const float4 *>(xsum + (local * 8 + 2 * t + 1) * MR + 4 * h);
+                    const float sl[4] = {xs_lo.x, xs_lo.y, xs_lo.z, xs_lo.w}, sh[4] = {xs_hi.x, xs_hi.y, xs_hi.z, xs_hi.w};
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {   // accumulator registers 0..3 of a lane: rows 4 (lane / 32) + i
+                        float acc = total[i];
+                        acc = __builtin_fmaf(lo[i], a_lo, acc);
+                        acc = __builtin_fmaf(-b_lo, sl[i], acc);
+                        acc = __builtin_fmaf(hi[i], a_hi, acc);
+                        acc = __builtin_fmaf(-b_hi, sh[i], acc);
+                        total[i] = acc;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);   // one sub-block pair at a time keeps the accumulators few
+                }
+            }
+        }
+    };
+    auto span_step = [&](int sp, auto parity) {
+        constexpr int P = decltype(parity)::value;
+        const bool more = sp + 1 < spans;
+        if (more) load_x(sp + 1);
+        compute_span(sp, parity);
+        if (more) store_x(1 - P);
+        __syncthreads();
+    };
+
+    load_x(0);
+    store_x(0);
+    __syncthreads();
+    for (int sp = 0; sp < spans; sp += 2) {
+        span_step(sp, std::integral_constant<int, 0>{});
+        if (sp + 1 < spans) span_step(sp + 1, std::integral_constant<int, 1>{});
+    }
+
+    // ---- the wavefronts' shares of K meet in LDS; wavefront 0 adds them in order and writes the rows ----
+#pragma unroll
+    for (int i = 0; i < 4; i++) red[(wave * 4 + i) * 64 + lane] = total[i];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float v = red[i * 64 + lane];
+#pragma unroll
+            for (int w = 1; w < WAVES; w++) v += red[(w * 4 + i) * 64 + lane];
+            const int m = 4 * h + i;
+            if (m < a.M && n < a.N) {
+                const size_t o = (size_t)m * a.N + n;
+                a.y[o] = a.residual ? a.residual[o] + v : v;
+            }
+        }
+    }
+}
+
 // y = (residual +) sum over splits of partial, in split order
 __global__ void gemm_reduce_kernel(const float *partial, int splits, size_t count, const float *residual, float *y) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -534,6 +701,19 @@ hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, 
     a.partial = workspace;
     hipError_t e;
     int splits;
+    if constexpr (FMT == FMT_Q4_K) {
+        if (a.M <= kRowsMaxRows && a.K % CK == 0) {   // one workgroup per 32 weight rows, K split over its wavefronts
+            const int groups = (a.N + 31) / 32;
+            auto go = [&](auto kernel, int waves, size_t lds) {
+                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                if (err != hipSuccess) return err;
+                hipLaunchKernelGGL(kernel, dim3(groups), dim3(waves * 64), lds, stream, a);
+                return hipGetLastError();
+            };
+            if (groups <= 256) return go(gemm_rows_q4k_kernel<8, 8>, 8, rows_lds_bytes<8, 8>());
+            return go(gemm_rows_q4k_kernel<4, 4>, 4, rows_lds_bytes<4, 4>());
+        }
+    }
     if constexpr (FMT != FMT_F16) {
         if (a.M <= 64 && a.K % CK == 0) {
             const int chunks = a.K / CK;
