@@ -141,11 +141,11 @@ __device__ __forceinline__ uint2 q4k_bytes_to_half(u32 b, float s, float dm) {
 
 // Writes the thread's 32 fp16 weights into its LDS row (`wrow` points at k = 0 of the tile).
 // Element order inside each group of four is (0,2,1,3) for Q4_0 and Q8_0, natural for Q4_K and F16.
+// `c` = tile % 4, the pair of Q4_K sub-blocks the tile covers (a constant where the caller's loop is unrolled by four).
 template <int FMT>
-__device__ __forceinline__ void dequant_to_lds(const Raw<FMT> &r, int tile, int h, _Float16 *wrow) {
+__device__ __forceinline__ void dequant_to_lds(const Raw<FMT> &r, int c, int h, _Float16 *wrow) {
     if constexpr (FMT == FMT_Q4_K) {
         // low nibbles: sub-block 2c, elements 16h..16h+15 (k = 16h..); high nibbles: sub-block 2c+1 (k = 32+16h..)
-        const int c = tile & 3;
         const float d = half_bits_to_float(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float(r.hdr.x >> 16);
         float sc_lo, m_lo, sc_hi, m_hi;
         q4k_scale_min(r.hdr, 2 * c, sc_lo, m_lo);
@@ -206,17 +206,18 @@ __device__ __forceinline__ void dequant_to_lds(const Raw<FMT> &r, int tile, int 
 // (a slot is refilled as soon as its tile has gone to LDS), and LDS holds two tiles so that one barrier
 // per tile is enough: tile t+1 is written while other wavefronts still read tile t.
 template <int FMT, int WM, int WN, int TM, int TN, int DEPTH>
-__global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs a) {
-    static_assert(WM * WN == 4 && 32 * WN * TN == NT, "four wavefronts over 128 weight rows");
+__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs a) {
+    constexpr int THREADS = 64 * WM * WN, NTILE = 32 * WN * TN;   // two threads per weight row dequantise
+    static_assert(2 * NTILE == THREADS, "one (weight row, half tile) per thread");
     constexpr int MT = 32 * WM * TM;
     constexpr bool kSwap = FMT == FMT_Q4_0 || FMT == FMT_Q8_0;   // formats whose unpacking yields (0,2,1,3) order
-    constexpr int XV = MT * KT / 8 / kThreads;   // 128-bit pieces of x per thread per tile
+    constexpr int XV = MT * KT / 8 / THREADS;   // 128-bit pieces of x per thread per tile
     static_assert(XV >= 1, "tile too small for the copy loop");
     __shared__ _Float16 xt[2][MT * LDK];
-    __shared__ _Float16 wt[2][NT * LDK];
+    __shared__ _Float16 wt[2][NTILE * LDK];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
-    const int n0 = blockIdx.x * NT, m0 = blockIdx.z * MT;
+    const int n0 = blockIdx.x * NTILE, m0 = blockIdx.z * MT;
     const int tiles = a.K / KT;
     const int t_begin = blockIdx.y * a.tiles_per_split;
     const int t_end = t_begin + a.tiles_per_split < tiles ? t_begin + a.tiles_per_split : tiles;
@@ -236,38 +237,43 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs a) {
     auto fetch_x = [&](int tile, uint4 (&xv)[XV]) {
 #pragma unroll
         for (int i = 0; i < XV; i++) {
-            const int piece = tid + i * kThreads, row = piece >> 3, part = piece & 7;   // eight pieces per row
-            const int m = m0 + row;
-            xv[i] = m < a.M ? reinterpret_cast<const uint4 *>(a.x + (size_t)m * a.K + (size_t)tile * KT)[part] : make_uint4(0, 0, 0, 0);
+            const int piece = tid + i * THREADS, row = piece >> 3, part = piece & 7;   // eight pieces per row
+            const int m = m0 + row < a.M ? m0 + row : a.M - 1;   // rows beyond M repeat the last one; their results are never stored
+            xv[i] = reinterpret_cast<const uint4 *>(a.x + (size_t)m * a.K + (size_t)tile * KT)[part];
         }
     };
 
+    // Slot j % DEPTH holds the packed bytes and activations of tile t_begin + j.  Staging a tile (dequantise into LDS,
+    // copy the activations, refill the slot DEPTH tiles ahead) sits in the same barrier interval as the matrix-core work
+    // on the tile before it, so the vector ALU and the LDS writes run in the shadow of the MFMAs of the same wavefront.
+    // Tile indices beyond the last are clamped: the extra stage of the last interval is in bounds and never read.
     Raw<FMT> raw[DEPTH];
     uint4 xv[DEPTH][XV];
+    const int t_last = t_end - 1;
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) {
-        if (t_begin + d < t_end) {
-            raw[d] = fetch_raw<FMT>(a, w_row, t_begin + d, wh);
-            fetch_x(t_begin + d, xv[d]);
-        }
+        const int tile = t_begin + d < t_last ? t_begin + d : t_last;
+        raw[d] = fetch_raw<FMT>(a, w_row, tile, wh);
+        fetch_x(tile, xv[d]);
     }
-    for (int t0 = t_begin; t0 < t_end; t0 += DEPTH) {
+    static_assert(4 % DEPTH == 0, "the main loop is unrolled by four");
+    auto stage = [&](int S, int c, int tile, int buf) {   // S and c are constants after unrolling
+        dequant_to_lds<FMT>(raw[S], c, wh, wt[buf] + wr * LDK);
 #pragma unroll
-        for (int d = 0; d < DEPTH; d++) {
-            const int t = t0 + d, buf = d & 1;   // DEPTH is even, so the parity of d is the parity of the tile count
-            if (t < t_end) {
-                dequant_to_lds<FMT>(raw[d], t, wh, wt[buf] + wr * LDK);
+        for (int i = 0; i < XV; i++) {
+            const int piece = tid + i * THREADS, row = piece >> 3, part = piece & 7;
+            *reinterpret_cast<uint4 *>(xt[buf] + row * LDK + part * 8) = kSwap ? swap_middle(xv[S][i]) : xv[S][i];
+        }
+        const int ahead = tile + DEPTH < t_last ? tile + DEPTH : t_last;
+        raw[S] = fetch_raw<FMT>(a, w_row, ahead, wh);
+        fetch_x(ahead, xv[S]);
+    };
+    stage(0, 0, t_begin, 0);   // t_begin is a multiple of four
+    __syncthreads();
+    for (int t0 = t_begin; t0 < t_end; t0 += 4) {
 #pragma unroll
-                for (int i = 0; i < XV; i++) {
-                    const int piece = tid + i * kThreads, row = piece >> 3, part = piece & 7;
-                    *reinterpret_cast<uint4 *>(xt[buf] + row * LDK + part * 8) = kSwap ? swap_middle(xv[d][i]) : xv[d][i];
-                }
-                if (t + DEPTH < t_end) {   // refill the slot: DEPTH tiles of global loads stay in flight
-                    raw[d] = fetch_raw<FMT>(a, w_row, t + DEPTH, wh);
-                    fetch_x(t + DEPTH, xv[d]);
-                }
-            }
-            __syncthreads();
+        for (int u = 0; u < 4; u++) {
+            const int t = t0 + u, buf = u & 1;
             if (t < t_end) {
 #pragma unroll
                 for (int ks = 0; ks < KT / 16; ks++) {
@@ -284,6 +290,8 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs a) {
 #pragma unroll
                         for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
                 }
+                stage((u + 1) % DEPTH, (u + 1) & 3, t + 1, buf ^ 1);
+                __syncthreads();
             }
         }
     }
@@ -674,8 +682,9 @@ __global__ void gemm_reduce_kernel(const float *partial, int splits, size_t coun
 template <int FMT, int WM, int WN, int TM, int TN, int DEPTH>
 hipError_t launch_tile(const GemmArgs &a, int splits, hipStream_t stream) {
     constexpr int MT = 32 * WM * TM;
-    dim3 grid((a.N + NT - 1) / NT, splits, (a.M + MT - 1) / MT);
-    hipLaunchKernelGGL((gemm_kernel<FMT, WM, WN, TM, TN, DEPTH>), grid, dim3(kThreads), 0, stream, a);
+    constexpr int NTILE = 32 * WN * TN;
+    dim3 grid((a.N + NTILE - 1) / NTILE, splits, (a.M + MT - 1) / MT);
+    hipLaunchKernelGGL((gemm_kernel<FMT, WM, WN, TM, TN, DEPTH>), grid, dim3(64 * WM * WN), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -729,8 +738,10 @@ hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, 
     }
     const int tiles = a.K / KT;
     const int mt = a.M <= 32 ? 32 : a.M <= 64 ? 64 : 128;
+    // (eight wavefronts on a 128 x 256 tile measure 2-5 % faster at 4096 and more weight rows and 10 % slower at 1024;
+    //  a 256 x 256 tile is 25 % slower: not instantiated)
     splits = choose_splits(n_blocks * ((a.M + mt - 1) / mt), tiles, 8, 1024, a, workspace_floats);
-    a.tiles_per_split = (tiles + splits - 1) / splits;
+    a.tiles_per_split = ((tiles + splits - 1) / splits + 3) & ~3;   // every split starts on a multiple of four tiles
     splits = (tiles + a.tiles_per_split - 1) / a.tiles_per_split;
     if (mt == 32) e = launch_tile<FMT, 1, 4, 1, 1, 4>(a, splits, stream);
     else if (mt == 64) e = launch_tile<FMT, 1, 4, 2, 1, 4>(a, splits, stream);
