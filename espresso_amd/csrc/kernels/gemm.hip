@@ -504,7 +504,7 @@ __global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(GemmArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Up to sixteen activation rows against Q4_K weights without dequantising them.  Below about sixteen rows the
+// Up to eight activation rows against Q4_K weights without dequantising them.  With so few rows the
 // register-B kernel above is bound by the exact dequantisation (three vector operations per weight however few rows
 // there are).  Here the B operand is the nibble itself under an fp16 exponent, as in the GEMV kernels: one
 // v_and_or_b32 turns two low nibbles into (64 + n/16, 64 + n/16) and two high nibbles into (4 + n/16, 4 + n/16),
