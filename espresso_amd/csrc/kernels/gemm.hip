@@ -528,19 +528,44 @@ __device__ __forceinline__ float quad_sum(float v) {
 // in flight (they do not wait for the staging).  Short spans measure faster than long ones (one chunk per wavefront and span:
 // 15.7 us for 14336 x 4096 against 18.2 us with two and 17.9 us with all of K staged at once), and eight wavefronts
 // faster than four when the rows fill no more than one workgroup per compute unit.
+// Q4_0 takes the same route: a lane holds eight bytes of each block (low nibbles = elements 8h.., high = 16 + 8h..), the two
+// MFMAs of a block share one accumulator, and w = d (n - 8) = 16 d pattern - (1032 | 72) d folds as
+//     total += d (16 raw - (1032 sum of x over the block's first sixteen + 72 sum over its last sixteen)).
 constexpr int kRowsMaxRows = 8;
 template <int WAVES, int SPAN> constexpr size_t rows_lds_bytes() {
     return 2 * ((size_t)kRowsMaxRows * (SPAN * CK + 8) * 2 + (size_t)SPAN * 8 * kRowsMaxRows * 4) + (size_t)WAVES * 4 * 64 * 4;
 }
 
-template <int WAVES, int SPAN>
-__global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gemm_rows_q4k_kernel(GemmArgs a) {
+template <int FMT>
+struct RowsChunk;
+template <>
+struct RowsChunk<FMT_Q4_K> { RawChunk<FMT_Q4_K> r; };
+template <>
+struct RowsChunk<FMT_Q4_0> { uint2 q[8]; uint4 d; };   // eight bytes of each of the chunk's eight blocks, their eight fp16 scales
+
+template <int FMT>
+__device__ __forceinline__ RowsChunk<FMT> fetch_rows_chunk(const GemmArgs &a, int row, int chunk, int h) {
+    RowsChunk<FMT> c;
+    if constexpr (FMT == FMT_Q4_K) {
+        c.r = fetch_chunk<FMT_Q4_K>(a, row, chunk, h);
+    } else {
+        const uint8_t *base = a.qs + (size_t)row * a.qs_row_bytes + (size_t)chunk * 128 + 8 * h;
+#pragma unroll
+        for (int b = 0; b < 8; b++) c.q[b] = *reinterpret_cast<const uint2 *>(base + 16 * b);
+        c.d = *reinterpret_cast<const uint4 *>(a.scales + (size_t)row * (a.K / 32) + (size_t)chunk * 8);
+    }
+    return c;
+}
+
+template <int FMT, int WAVES, int SPAN>
+__global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gemm_rows_kernel(GemmArgs a) {
+    static_assert(FMT == FMT_Q4_K || FMT == FMT_Q4_0, "formats whose weights are nibbles");
     constexpr int MR = kRowsMaxRows, THREADS = WAVES * 64, LDW = SPAN * CK + 8;
     constexpr int CPW = SPAN / WAVES;                     // chunks per wavefront and span
     constexpr int PIECES = MR * SPAN * 32 / THREADS;      // 128-bit pieces of x per thread and span
     extern __shared__ uint4 rows_smem[];
     _Float16 *xt_base = reinterpret_cast<_Float16 *>(rows_smem);               // [2][MR][LDW]
-    float *xsum_base = reinterpret_cast<float *>(xt_base + 2 * MR * LDW);      // [2][SPAN * 8 sub-blocks][MR]
+    float *xsum_base = reinterpret_cast<float *>(xt_base + 2 * MR * LDW);      // [2][SPAN * 8 groups of 32][MR]
     float *red = xsum_base + 2 * SPAN * 8 * MR;                                // [WAVES][4][64]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
     const int n = blockIdx.x * 32 + (lane & 31);
@@ -550,13 +575,15 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gemm_rows_q4k_
     u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x54005400u, magic_hi = 0x44004400u;
     asm volatile("" : "+s"(mask_lo), "+s"(mask_hi));
     asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
+    auto pattern_lo = [&](u32 w0, u32 w1) { return as_half8(make_uint4((w0 & mask_lo) | magic_lo, ((w0 >> 8) & mask_lo) | magic_lo, (w1 & mask_lo) | magic_lo, ((w1 >> 8) & mask_lo) | magic_lo)); };
+    auto pattern_hi = [&](u32 w0, u32 w1) { return as_half8(make_uint4((w0 & mask_hi) | magic_hi, ((w0 >> 8) & mask_hi) | magic_hi, (w1 & mask_hi) | magic_hi, ((w1 >> 8) & mask_hi) | magic_hi)); };
 
     float total[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     auto chunk_of = [&](int sp, int j) { return sp * SPAN + j * WAVES + wave; };
-    RawChunk<FMT_Q4_K> ring[2 * CPW];
+    RowsChunk<FMT> ring[2 * CPW];
 #pragma unroll
     for (int q = 0; q < 2 * CPW; q++)
-        if (chunk_of(q / CPW, q % CPW) < chunks) ring[q] = fetch_chunk<FMT_Q4_K>(a, w_row, chunk_of(q / CPW, q % CPW), h);
+        if (chunk_of(q / CPW, q % CPW) < chunks) ring[q] = fetch_rows_chunk<FMT>(a, w_row, chunk_of(q / CPW, q % CPW), h);
 
     uint4 xv[PIECES];
     auto load_x = [&](int sp) {
@@ -567,7 +594,8 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gemm_rows_q4k_
             xv[i] = row < a.M && k0 < a.K ? *reinterpret_cast<const uint4 *>(a.x + (size_t)row * a.K + k0) : make_uint4(0, 0, 0, 0);
         }
     };
-    // (0,2,1,3) order inside fours, sums of every 32 alongside
+    // (0,2,1,3) order inside fours; alongside, per group of 32: Q4_K the sum of the activations, Q4_0 1032 times the sum of
+    // the first sixteen plus 72 times the sum of the last sixteen
     auto store_x = [&](int buf) {
         _Float16 *xt = xt_base + buf * MR * LDW;
         float *xsum = xsum_base + buf * SPAN * 8 * MR;
@@ -577,7 +605,8 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gemm_rows_q4k_
             *reinterpret_cast<uint4 *>(xt + row * LDW + part * 8) = swap_middle(xv[i]);
             const h2 p0 = as_h2(xv[i].x), p1 = as_h2(xv[i].y), p2 = as_h2(xv[i].z), p3 = as_h2(xv[i].w);
             float sum = (((float)p0.x + (float)p0.y) + ((float)p1.x + (float)p1.y)) + (((float)p2.x + (float)p2.y) + ((float)p3.x + (float)p3.y));
-            sum = quad_sum(sum);                 // the four pieces of a 32-weight sub-block sit in one quad of lanes
+            if constexpr (FMT == FMT_Q4_0) sum *= (part & 2) ? 72.0f : 1032.0f;
+            sum = quad_sum(sum);                 // the four pieces of a group of 32 sit in one quad of lanes
             if ((part & 3) == 0) xsum[(part >> 2) * MR + row] = sum;
         }
     };
@@ -589,47 +618,64 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gemm_rows_q4k_
         for (int j = 0; j < CPW; j++) {
             const int c = chunk_of(sp, j);
             if (c < chunks) {
-                const RawChunk<FMT_Q4_K> r = ring[P * CPW + j];
-                if (chunk_of(sp + 2, j) < chunks) ring[P * CPW + j] = fetch_chunk<FMT_Q4_K>(a, w_row, chunk_of(sp + 2, j), h);
-                const float dd = half_bits_to_float(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float(r.hdr.x >> 16);
+                const RowsChunk<FMT> rc = ring[P * CPW + j];
+                if (chunk_of(sp + 2, j) < chunks) ring[P * CPW + j] = fetch_rows_chunk<FMT>(a, w_row, chunk_of(sp + 2, j), h);
                 const int local = j * WAVES + wave;   // chunk index inside the span
+                // rows of x beyond MR alias real ones: they only reach accumulator registers that are never read
+                const _Float16 *xchunk = xt + ((lane & 31) & (MR - 1)) * LDW + local * CK;
+                if constexpr (FMT == FMT_Q4_K) {
+                    const RawChunk<FMT_Q4_K> &r = rc.r;
+                    const float dd = half_bits_to_float(r.hdr.x & 0xFFFFu), dmin = half_bits_to_float(r.hdr.x >> 16);
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    float sc_lo, m_lo, sc_hi, m_hi;
-                    q4k_scale_min(r.hdr, 2 * t, sc_lo, m_lo);
-                    q4k_scale_min(r.hdr, 2 * t + 1, sc_hi, m_hi);
-                    const float a_lo = 16.0f * dd * sc_lo, b_lo = 64.0f * a_lo + dmin * m_lo;
-                    const float a_hi = 16.0f * dd * sc_hi, b_hi = 4.0f * a_hi + dmin * m_hi;
-                    half8 frag[4];
-                    {
+                    for (int t = 0; t < 4; t++) {
+                        float sc_lo, m_lo, sc_hi, m_hi;
+                        q4k_scale_min(r.hdr, 2 * t, sc_lo, m_lo);
+                        q4k_scale_min(r.hdr, 2 * t + 1, sc_hi, m_hi);
+                        const float a_lo = 16.0f * dd * sc_lo, b_lo = 64.0f * a_lo + dmin * m_lo;
+                        const float a_hi = 16.0f * dd * sc_hi, b_hi = 4.0f * a_hi + dmin * m_hi;
                         const u32 w0 = r.q[t].x, w1 = r.q[t].y, w2 = r.q[t].z, w3 = r.q[t].w;
-                        frag[0] = as_half8(make_uint4((w0 & mask_lo) | magic_lo, ((w0 >> 8) & mask_lo) | magic_lo, (w1 & mask_lo) | magic_lo, ((w1 >> 8) & mask_lo) | magic_lo));
-                        frag[1] = as_half8(make_uint4((w2 & mask_lo) | magic_lo, ((w2 >> 8) & mask_lo) | magic_lo, (w3 & mask_lo) | magic_lo, ((w3 >> 8) & mask_lo) | magic_lo));
-                        frag[2] = as_half8(make_uint4((w0 & mask_hi) | magic_hi, ((w0 >> 8) & mask_hi) | magic_hi, (w1 & mask_hi) | magic_hi, ((w1 >> 8) & mask_hi) | magic_hi));
-                        frag[3] = as_half8(make_uint4((w2 & mask_hi) | magic_hi, ((w2 >> 8) & mask_hi) | magic_hi, (w3 & mask_hi) | magic_hi, ((w3 >> 8) & mask_hi) | magic_hi));
-                    }
-                    // rows of x beyond MR alias real ones: they only reach accumulator registers that are never read
-                    const _Float16 *xrow = xt + ((lane & 31) & (MR - 1)) * LDW + local * CK + t * KT;
-                    floatx16 lo, hi;
+                        const half8 f0 = pattern_lo(w0, w1), f1 = pattern_lo(w2, w3), f2 = pattern_hi(w0, w1), f3 = pattern_hi(w2, w3);
+                        const _Float16 *xrow = xchunk + t * KT;
+                        floatx16 lo, hi;
 #pragma unroll
-                    for (int i = 0; i < 16; i++) lo[i] = hi[i] = 0.0f;
-                    lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 16 * h), frag[0], lo, 0, 0, 0);
-                    hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 32 + 16 * h), frag[2], hi, 0, 0, 0);
-                    lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 16 * h + 8), frag[1], lo, 0, 0, 0);
-                    hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 40 + 16 * h), frag[3], hi, 0, 0, 0);
-                    const float4 xs_lo = *reinterpret_cast<const float4 *>(xsum + (local * 8 + 2 * t) * MR + 4 * h);
-                    const float4 xs_hi = *reinterpret_cast<const float4 *>(xsum + (local * 8 + 2 * t + 1) * MR + 4 * h);
-                    const float sl[4] = {xs_lo.x, xs_lo.y, xs_lo.z, xs_lo.w}, sh[4] = {xs_hi.x, xs_hi.y, xs_hi.z, xs_hi.w};
+                        for (int i = 0; i < 16; i++) lo[i] = hi[i] = 0.0f;
+                        lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 16 * h), f0, lo, 0, 0, 0);
+                        hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 32 + 16 * h), f2, hi, 0, 0, 0);
+                        lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 16 * h + 8), f1, lo, 0, 0, 0);
+                        hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 40 + 16 * h), f3, hi, 0, 0, 0);
+                        const float4 xs_lo = *reinterpret_cast<const float4 *>(xsum + (local * 8 + 2 * t) * MR + 4 * h);
+                        const float4 xs_hi = *reinterpret_cast<const float4 *>(xsum + (local * 8 + 2 * t + 1) * MR + 4 * h);
+                        const float sl[4] = {xs_lo.x, xs_lo.y, xs_lo.z, xs_lo.w}, sh[4] = {xs_hi.x, xs_hi.y, xs_hi.z, xs_hi.w};
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {   // accumulator registers 0..3 of a lane: rows 4 (lane / 32) + i
-                        float acc = total[i];
-                        acc = __builtin_fmaf(lo[i], a_lo, acc);
-                        acc = __builtin_fmaf(-b_lo, sl[i], acc);
-                        acc = __builtin_fmaf(hi[i], a_hi, acc);
-                        acc = __builtin_fmaf(-b_hi, sh[i], acc);
-                        total[i] = acc;
+                        for (int i = 0; i < 4; i++) {   // accumulator registers 0..3 of a lane: rows 4 (lane / 32) + i
+                            float acc = total[i];
+                            acc = __builtin_fmaf(lo[i], a_lo, acc);
+                            acc = __builtin_fmaf(-b_lo, sl[i], acc);
+                            acc = __builtin_fmaf(hi[i], a_hi, acc);
+                            acc = __builtin_fmaf(-b_hi, sh[i], acc);
+                            total[i] = acc;
+                        }
+                        __builtin_amdgcn_sched_barrier(0);   // one sub-block pair at a time keeps the accumulators few
                     }
-                    __builtin_amdgcn_sched_barrier(0);   // one sub-block pair at a time keeps the accumulators few
+                } else {
+                    const u32 dw[4] = {rc.d.x, rc.d.y, rc.d.z, rc.d.w};
+#pragma unroll
+                    for (int b = 0; b < 8; b++) {
+                        const float d = half_bits_to_float((dw[b >> 1] >> (16 * (b & 1))) & 0xFFFFu);
+                        const half8 f_lo = pattern_lo(rc.q[b].x, rc.q[b].y), f_hi = pattern_hi(rc.q[b].x, rc.q[b].y);
+                        const _Float16 *xrow = xchunk + b * 32;
+                        floatx16 raw;
+#pragma unroll
+                        for (int i = 0; i < 16; i++) raw[i] = 0.0f;
+                        raw = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 8 * h), f_lo, raw, 0, 0, 0);
+                        raw = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(xrow + 16 + 8 * h), f_hi, raw, 0, 0, 0);
+                        const float4 xs = *reinterpret_cast<const float4 *>(xsum + (local * 8 + b) * MR + 4 * h);
+                        const float sx[4] = {xs.x, xs.y, xs.z, xs.w};
+                        const float d16 = 16.0f * d;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) total[i] = __builtin_fmaf(-d, sx[i], __builtin_fmaf(raw[i], d16, total[i]));
+                        if (b & 1) __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
             }
         }
@@ -710,8 +756,10 @@ hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, 
     a.partial = workspace;
     hipError_t e;
     int splits;
-    if constexpr (FMT == FMT_Q4_K) {
-        if (a.M <= kRowsMaxRows && a.K % CK == 0) {   // one workgroup per 32 weight rows, K split over its wavefronts
+    if constexpr (FMT == FMT_Q4_K || FMT == FMT_Q4_0) {
+        // one workgroup per 32 weight rows, K split over its wavefronts (Q4_0 at 14336 columns measures 27 us here against 24 us
+        // on the register-B kernel with split-K, so long rows of Q4_0 stay there)
+        if (a.M <= kRowsMaxRows && a.K % CK == 0 && (FMT == FMT_Q4_K || a.K <= 8192)) {
             const int groups = (a.N + 31) / 32;
             auto go = [&](auto kernel, int waves, size_t lds) {
                 hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -719,8 +767,8 @@ hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, 
                 hipLaunchKernelGGL(kernel, dim3(groups), dim3(waves * 64), lds, stream, a);
                 return hipGetLastError();
             };
-            if (groups <= 256) return go(gemm_rows_q4k_kernel<8, 8>, 8, rows_lds_bytes<8, 8>());
-            return go(gemm_rows_q4k_kernel<4, 4>, 4, rows_lds_bytes<4, 4>());
+            if (groups <= 256) return go(gemm_rows_kernel<FMT, 8, 8>, 8, rows_lds_bytes<8, 8>());
+            return go(gemm_rows_kernel<FMT, 4, 4>, 4, rows_lds_bytes<4, 4>());
         }
     }
     if constexpr (FMT != FMT_F16) {

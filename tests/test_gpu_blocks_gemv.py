@@ -153,8 +153,8 @@ def test_mfma_gemm_matches_oracle(ops, name, rows, cols, batch):
     assert np.abs(y[check] - want).max() <= tol, (np.abs(y[check] - want).max(), tol)
     # every format feeds the matrix cores fp16(dequantised weight), rounded once: against those weights in
     # float64 only fp32 summation noise remains (pins the tile indexing and the single rounding)
-    # (up to eight rows against Q4_K run on the nibbles themselves with exact products: no weight rounding at all)
-    exact = name == "q4_k" and batch <= 8 and cols % 256 == 0
+    # (up to eight rows against Q4_K and Q4_0 run on the nibbles themselves with exact products: no weight rounding at all)
+    exact = batch <= 8 and cols % 256 == 0 and (name == "q4_k" or (name == "q4_0" and cols <= 8192))
     ref = x.astype(np.float64) @ (deq if exact else deq.astype(np.float16)).astype(np.float64).T
     assert np.abs(y - ref).max() <= 2e-5 * np.abs(deq).max() * np.sqrt(cols) * 4 + 1e-6, np.abs(y - ref).max()
     res = rng.normal(0, 1, (batch, rows)).astype(np.float32)
