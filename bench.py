@@ -288,7 +288,7 @@ def main() -> None:
                                                "the memory system gives the simplest reader, to read `frac` against"},
         "model_build_s": round(gpu["build_s"], 1), "prefill_s": round(gpu["prefill_s"], 3),
         "prefill": {"tokens": w["prompt"], "tok_s": w["prompt"] / gpu["prefill_s"],
-                    "path": "blocks of up to 256 rows through the dequant-fused MFMA GEMM" if w["prompt"] >= 32
+                    "path": "blocks of up to 512 rows through the dequant-fused MFMA GEMM" if w["prompt"] >= 32
                             else "token by token (prompts under 32 tokens)"},
     }
     if not args.no_cpu_baseline:

@@ -28,7 +28,7 @@ struct LlamaConfig {
     int kv_dim() const { return n_kv_head * head_dim; }
 };
 
-constexpr int kPrefillBlockRows = 256;        // rows per MFMA prefill block
+constexpr int kPrefillBlockRows = 512;        // rows per MFMA prefill block
 constexpr int kMatrixPrefillMinTokens = 32;   // shorter prompts take the exact per-token path
 constexpr size_t kGemmWorkspaceFloats = (size_t)8 << 20;
 

@@ -209,7 +209,7 @@ int esp_llama_continue_greedy(ESPLlamaRuntime *runtime, int sequence, int steps,
  * synchronises once at the end; 0 switches it to one kernel launch at a time with a host read of
  * every token (same results).  Default: enabled. */
 int esp_llama_set_graph_replay(ESPLlamaRuntime *runtime, int enabled);
-/* Prompts of 32 tokens or more are prefilled in blocks of up to 256 rows with every projection as one
+/* Prompts of 32 tokens or more are prefilled in blocks of up to 512 rows with every projection as one
  * dequant-fused MFMA GEMM (fp16 weights after dequantisation, fp32 accumulation), instead of the
  * reference's token-by-token walk (RealModelInferenceEngine.swift:6365-6375).  enabled = 0 restores the
  * per-token path, whose arithmetic keeps the dequantised weights in fp32.  Default: enabled. */
