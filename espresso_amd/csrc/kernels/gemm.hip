@@ -23,6 +23,7 @@
 //   * when the (n, m) grid is too small to fill the chip, K is split over grid.y and a small kernel
 //     adds the partial sums in split order (deterministic, no atomics).
 #include "../common.h"
+#include <atomic>
 
 namespace esp {
 namespace {
@@ -761,14 +762,23 @@ hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, 
         // on the register-B kernel with split-K, so long rows of Q4_0 stay there)
         if (a.M <= kRowsMaxRows && a.K % CK == 0 && (FMT == FMT_Q4_K || a.K <= 8192)) {
             const int groups = (a.N + 31) / 32;
-            auto go = [&](auto kernel, int waves, size_t lds) {
-                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            // the kernels' LDS (above 64 KB) is dynamic: the limit is raised once per kernel and device
+            auto go = [&](auto kernel, int waves, size_t lds, std::atomic<uint64_t> &raised) {
+                int device = 0;
+                hipError_t err = hipGetDevice(&device);
                 if (err != hipSuccess) return err;
+                const uint64_t bit = 1ull << (device & 63);
+                if (!(raised.load(std::memory_order_acquire) & bit)) {
+                    err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                    if (err != hipSuccess) return err;
+                    raised.fetch_or(bit, std::memory_order_release);
+                }
                 hipLaunchKernelGGL(kernel, dim3(groups), dim3(waves * 64), lds, stream, a);
                 return hipGetLastError();
             };
-            if (groups <= 256) return go(gemm_rows_kernel<FMT, 8, 8>, 8, rows_lds_bytes<8, 8>());
-            return go(gemm_rows_kernel<FMT, 4, 4>, 4, rows_lds_bytes<4, 4>());
+            static std::atomic<uint64_t> raised8{0}, raised4{0};   // one pair per format: this function is a template
+            if (groups <= 256) return go(gemm_rows_kernel<FMT, 8, 8>, 8, rows_lds_bytes<8, 8>(), raised8);
+            return go(gemm_rows_kernel<FMT, 4, 4>, 4, rows_lds_bytes<4, 4>(), raised4);
         }
     }
     if constexpr (FMT != FMT_F16) {
