@@ -55,6 +55,10 @@ hipError_t launch_rmsnorm(const float *x, const float *w, float eps, int rows, i
                           unsigned long long *argmax_cells, hipStream_t s);
 hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStream_t s);
 hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
+// Causal attention of `rows` rows that are ONE sequence at consecutive positions (a prompt block), on the matrix cores.
+// Head dim 64 or 128, 1, 2 or 4 query heads per KV head (attention_prompt_supported); Q, K, V, P as fp16, fp32 sums.
+bool attention_prompt_supported(int n_head, int n_kv_head, int head_dim);
+hipError_t launch_attention_prompt(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
 // Attention that stops at per-split partial states (head_dim 64 or 128, up to kMaxStepRows rows); the GEMV that reads
 // the context merges them (GemvParams::merge_partials).  attention_head_splits: slices per query head.
 int attention_head_splits(int max_seq);

@@ -417,6 +417,165 @@ __global__ __launch_bounds__(HD) void attention_merge_kernel(AttentionArgs a, in
     a.ctx_f16[(size_t)m * a.n_head * HD + (size_t)head * HD + dch] = to_half_bits(L > 0.0f ? A / L : 0.0f);
 }
 
+// Causal attention of a block of prompt rows on the matrix cores (v_mfma_f32_32x32x16_f16), for rows that are one
+// sequence at consecutive positions (pos[m0 + i] = pos[m0] + i), which is what a prompt block is.  Replaces the per-row
+// loop of the reference's attention (:6774-6823) over a block: the single-query kernels above read a row's whole prefix
+// once per row, this one reads a key tile once per 32 rows.
+// grid (KV heads, tiles of 32 rows); wavefront g of a workgroup serves query head kvh * G + g, so the G heads that share
+// a KV head share the value tiles.  Per tile of 32 keys:
+//   * S^T = K Q^T: keys are the A rows (a lane loads eight consecutive dims of its key straight from the cache, the next
+//     tile's while this one is computed), queries the B columns (fragments kept in registers); a lane's 16 accumulators are
+//     16 keys of ONE query, so the row maximum and sum of the online softmax are in-lane plus one exchange with lane ^ 32;
+//   * O^T += V^T P: the probabilities a lane holds are already a B fragment (column = its query, k slots = its keys), and
+//     the A operand is the value tile transposed in LDS (written once per workgroup, double-buffered: one barrier per tile),
+//     read so that k slot (lane / 32, i) is key 16 j + 8 (i / 4) + 4 (lane / 32) + i % 4, the key of accumulator 8 j + i.
+// Q, K, V and the probabilities enter the matrix cores as fp16, sums are fp32.
+typedef _Float16 attn_half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 attn_half4 __attribute__((ext_vector_type(4)));
+typedef float attn_floatx16 __attribute__((ext_vector_type(16)));
+
+template <int HD, int G, bool KV_F16>
+__global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs a, int rows) {
+    constexpr int THREADS = G * 64, QT = 32, KS = HD / 16, MTILES = HD / 32, LDV = 32 + 8;   // LDV: fp16 per row of V^T
+    constexpr int VP = 32 * (HD / 8) / THREADS;                                            // 8-dim pieces of V per thread
+    static_assert(VP >= 1 && 32 * (HD / 8) % THREADS == 0, "value tile divides over the workgroup");
+    __shared__ _Float16 vt[2][HD * LDV];
+    const int kvh = blockIdx.x, m0 = blockIdx.y * QT;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+    const int head = kvh * G + wave;
+    const int pos0 = a.pos[m0];
+    const int last_row = rows - 1 - m0 < QT - 1 ? rows - 1 - m0 : QT - 1;
+    const int t_max = pos0 + last_row;             // last key any row of the tile sees
+    const int kd = a.n_kv_head * HD;
+    const size_t seq_base = (size_t)a.seq[m0] * a.cache_seq_stride;
+    const float scale = 1.0f / sqrtf((float)HD);
+
+    auto to_half8 = [](const float4 &x0, const float4 &x1) {
+        return attn_half8{(_Float16)x0.x, (_Float16)x0.y, (_Float16)x0.z, (_Float16)x0.w, (_Float16)x1.x, (_Float16)x1.y, (_Float16)x1.z, (_Float16)x1.w};
+    };
+    // query fragments: column = query `col` (rows beyond the block repeat its last row, never stored), dims 16 ks + 8 half ..
+    attn_half8 qf[KS];
+    {
+        const float *qp = a.q + (size_t)(m0 + (col <= last_row ? col : last_row)) * a.n_head * HD + (size_t)head * HD + 8 * half;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) qf[ks] = to_half8(*reinterpret_cast<const float4 *>(qp + 16 * ks), *reinterpret_cast<const float4 *>(qp + 16 * ks + 4));
+    }
+    // keys beyond t_max are clamped to it: in bounds, and masked below
+    auto load_k = [&](int t0, attn_half8 (&kf)[KS]) {
+        const int t = t0 + col < t_max ? t0 + col : t_max;
+        const size_t off = seq_base + (size_t)t * kd + (size_t)kvh * HD + 8 * half;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            if (KV_F16) kf[ks] = *reinterpret_cast<const attn_half8 *>(reinterpret_cast<const uint16_t *>(a.k_cache) + off + 16 * ks);
+            else {
+                const float *kp = reinterpret_cast<const float *>(a.k_cache) + off + 16 * ks;
+                kf[ks] = to_half8(*reinterpret_cast<const float4 *>(kp), *reinterpret_cast<const float4 *>(kp + 4));
+            }
+        }
+    };
+    // value tile: piece = (key, group of eight dims); consecutive lanes take consecutive keys so that the transposed
+    // two-byte LDS writes of a wavefront spread over the banks
+    attn_half8 vreg[VP];
+    auto load_v = [&](int t0) {
+#pragma unroll
+        for (int i = 0; i < VP; i++) {
+            const int piece = tid + i * THREADS, key = piece & 31, dg = piece >> 5;
+            const int t = t0 + key < t_max ? t0 + key : t_max;
+            const size_t off = seq_base + (size_t)t * kd + (size_t)kvh * HD + 8 * dg;
+            if (KV_F16) vreg[i] = *reinterpret_cast<const attn_half8 *>(reinterpret_cast<const uint16_t *>(a.v_cache) + off);
+            else {
+                const float *vp = reinterpret_cast<const float *>(a.v_cache) + off;
+                vreg[i] = to_half8(*reinterpret_cast<const float4 *>(vp), *reinterpret_cast<const float4 *>(vp + 4));
+            }
+        }
+    };
+    auto store_v = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < VP; i++) {
+            const int piece = tid + i * THREADS, key = piece & 31, dg = piece >> 5;
+#pragma unroll
+            for (int e = 0; e < 8; e++) vt[buf][(8 * dg + e) * LDV + key] = vreg[i][e];
+        }
+    };
+
+    attn_floatx16 o[MTILES];
+#pragma unroll
+    for (int mt = 0; mt < MTILES; mt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[mt][r] = 0.0f;
+    float mx = -INFINITY, l = 0.0f;
+    const int qpos = pos0 + col;
+
+    attn_half8 kf[KS];
+    load_k(0, kf);
+    load_v(0);
+    store_v(0);
+    __syncthreads();
+    for (int t0 = 0, buf = 0; t0 <= t_max; t0 += 32, buf ^= 1) {
+        const bool more = t0 + 32 <= t_max;
+        attn_half8 kn[KS];
+        if (more) { load_k(t0 + 32, kn); load_v(t0 + 32); }
+        attn_floatx16 sc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) sc[r] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], sc, 0, 0, 0);
+        // accumulator r: key t0 + 8 (r / 4) + 4 half + r % 4 against query `col`
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int key = t0 + 8 * (r >> 2) + 4 * half + (r & 3);
+            sc[r] = key <= qpos ? __fmul_rn(sc[r], scale) : -INFINITY;
+            tile_max = fmaxf(tile_max, sc[r]);
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+        const float m_new = fmaxf(mx, tile_max);    // finite from the first tile on: key 0 is visible to every query
+        const float alpha = __expf(mx - m_new);      // exp(-inf) = 0 on the first tile
+        float psum = 0.0f;
+        _Float16 ph[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float pr = __expf(sc[r] - m_new);  // masked keys: exp(-inf) = 0
+            psum += pr;
+            ph[r] = (_Float16)pr;
+        }
+        l = __builtin_fmaf(l, alpha, psum);
+        mx = m_new;
+        const attn_half8 pf[2] = {attn_half8{ph[0], ph[1], ph[2], ph[3], ph[4], ph[5], ph[6], ph[7]},
+                                  attn_half8{ph[8], ph[9], ph[10], ph[11], ph[12], ph[13], ph[14], ph[15]}};
+#pragma unroll
+        for (int mt = 0; mt < MTILES; mt++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[mt][r] *= alpha;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const _Float16 *vrow = vt[buf] + (32 * mt + col) * LDV + 16 * j + 4 * half;
+                const attn_half4 lo = *reinterpret_cast<const attn_half4 *>(vrow), hi = *reinterpret_cast<const attn_half4 *>(vrow + 8);
+                const attn_half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[j], o[mt], 0, 0, 0);
+            }
+        }
+        if (more) {
+            store_v(buf ^ 1);
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) kf[ks] = kn[ks];
+        }
+        __syncthreads();
+    }
+    l += __shfl_xor(l, 32);
+    if (col <= last_row) {
+        const float inv = 1.0f / l;
+        uint16_t *out = a.ctx_f16 + (size_t)(m0 + col) * a.n_head * HD + (size_t)head * HD;
+#pragma unroll
+        for (int mt = 0; mt < MTILES; mt++)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                const attn_half4 v = {(_Float16)(o[mt][4 * q4] * inv), (_Float16)(o[mt][4 * q4 + 1] * inv), (_Float16)(o[mt][4 * q4 + 2] * inv), (_Float16)(o[mt][4 * q4 + 3] * inv)};
+                *reinterpret_cast<attn_half4 *>(out + 32 * mt + 8 * q4 + 4 * half) = v;
+            }
+    }
+}
+
 // Single-query attention whose merge is left to the consumer: grid (query heads, rows, kAttentionHeadSplits),
 // WAVES wavefronts per workgroup, one query head each.  Chunks, lane mapping and the (m, l, acc) arithmetic are
 // those of attention_flash_kernel; a wavefront keeps U chunks of loads in flight, so kAttentionHeadSplits *
@@ -762,6 +921,33 @@ hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipSt
     if (kv_f16) hipLaunchKernelGGL(attention_decode_kernel<true>, grid, dim3(kBlock), lds, s, a);
     else hipLaunchKernelGGL(attention_decode_kernel<false>, grid, dim3(kBlock), lds, s, a);
     return hipGetLastError();
+}
+
+bool attention_prompt_supported(int n_head, int n_kv_head, int head_dim) {
+    if (n_kv_head <= 0 || n_head % n_kv_head != 0) return false;
+    const int group = n_head / n_kv_head;
+    return (head_dim == 128 || head_dim == 64) && (group == 1 || group == 2 || group == 4);
+}
+
+template <int HD, int G>
+hipError_t launch_attention_prompt_shape(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
+    dim3 grid(a.n_kv_head, (rows + 31) / 32);
+    if (kv_f16) hipLaunchKernelGGL((attention_prompt_kernel<HD, G, true>), grid, dim3(G * 64), 0, s, a, rows);
+    else hipLaunchKernelGGL((attention_prompt_kernel<HD, G, false>), grid, dim3(G * 64), 0, s, a, rows);
+    return hipGetLastError();
+}
+
+hipError_t launch_attention_prompt(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
+    if (rows <= 0 || !attention_prompt_supported(a.n_head, a.n_kv_head, a.head_dim)) return hipErrorInvalidValue;
+    const int group = a.n_head / a.n_kv_head;
+    if (a.head_dim == 128) {
+        if (group == 1) return launch_attention_prompt_shape<128, 1>(a, rows, kv_f16, s);
+        if (group == 2) return launch_attention_prompt_shape<128, 2>(a, rows, kv_f16, s);
+        return launch_attention_prompt_shape<128, 4>(a, rows, kv_f16, s);
+    }
+    if (group == 1) return launch_attention_prompt_shape<64, 1>(a, rows, kv_f16, s);
+    if (group == 2) return launch_attention_prompt_shape<64, 2>(a, rows, kv_f16, s);
+    return launch_attention_prompt_shape<64, 4>(a, rows, kv_f16, s);
 }
 
 int attention_head_splits(int) { return kAttentionHeadSplits; }

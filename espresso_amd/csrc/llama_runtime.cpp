@@ -405,6 +405,8 @@ int LlamaRuntime::finalize() {
         bool all_q4k = true;
         for (const Layer &L : layers_)
             all_q4k = all_q4k && L.wqkv.format == FMT_Q4_K && L.wo.format == FMT_Q4_K && L.w13.format == FMT_Q4_K && L.w2.format == FMT_Q4_K && !L.q_norm;
+        const char *pa = getenv("ESPRESSO_HIP_PROMPT_ATTENTION");   // "0": prompt blocks keep the single-query attention kernel
+        prompt_attention_ = attention_prompt_supported(c_.n_head, c_.n_kv_head, c_.head_dim) && !(pa && pa[0] == '0');
         const char *env = getenv("ESPRESSO_HIP_FUSED_TRUNK");
         fused_trunk_ = env && env[0] == '1';   // measured slower than the separate kernels: opt-in
         if (all_q4k && trunk_kernel_supports(d, hd, c_.head_dim, c_.n_head, c_.n_kv_head)) {
@@ -648,12 +650,13 @@ int LlamaRuntime::prefill_block(int seq, const uint32_t *tokens, int rows, int b
     ESP_HIP_TRY(hipStreamSynchronize(s));   // the host vectors go out of scope
     ESP_HIP_TRY(launch_embed(embedding_, embedding_f16_, d_tokens_, rows, d, hidden_, s));
     (void)ad; (void)kd; (void)hd; (void)kv16;
-    return enqueue_layers_matrix(rows);
+    return enqueue_layers_matrix(rows, true);
 }
 
 // The layer loop over `rows` rows whose embeddings sit in hidden_ and whose (position, sequence) sit in
-// d_pos_/d_seq_, every projection as one dequant-fused MFMA GEMM.
-int LlamaRuntime::enqueue_layers_matrix(int rows) {
+// d_pos_/d_seq_, every projection as one dequant-fused MFMA GEMM.  Rows that are one sequence at consecutive positions
+// (a prompt block) take the matrix-core attention kernel, others the single-query one.
+int LlamaRuntime::enqueue_layers_matrix(int rows, bool one_sequence_consecutive) {
     hipStream_t s = context().stream;
     const int d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
     const bool kv16 = c_.kv_format == FMT_F16;
@@ -674,7 +677,8 @@ int LlamaRuntime::enqueue_layers_matrix(int rows) {
         aa.q = q_; aa.k_cache = L.k_cache; aa.v_cache = L.v_cache; aa.cache_seq_stride = cache_seq_stride;
         aa.n_head = c_.n_head; aa.n_kv_head = c_.n_kv_head; aa.head_dim = c_.head_dim; aa.max_seq = c_.max_seq;
         aa.pos = d_pos_; aa.seq = d_seq_; aa.ctx_f16 = ctx_; aa.split_scratch = attn_scratch_;
-        ESP_HIP_TRY(launch_attention(aa, rows, kv16, s));
+        if (one_sequence_consecutive && prompt_attention_) ESP_HIP_TRY(launch_attention_prompt(aa, rows, kv16, s));
+        else ESP_HIP_TRY(launch_attention(aa, rows, kv16, s));
         g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_;
         ESP_HIP_TRY(launch_gemm(g, s));
         ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_ffn, c_.norm_eps, rows, d, xn_, nullptr, s));

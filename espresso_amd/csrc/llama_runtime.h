@@ -107,7 +107,7 @@ class LlamaRuntime {
     // embedded: hidden_ already holds the rows' embeddings; final_out: where the last layer writes (default hidden_)
     int enqueue_trunk(int rows, bool embedded = false, float *final_out = nullptr);
     int prefill_block(int seq, const uint32_t *tokens, int rows, int base);
-    int enqueue_layers_matrix(int rows);
+    int enqueue_layers_matrix(int rows, bool one_sequence_consecutive = false);
     bool matrix_prefill_supported() const;
     bool wo_merges_attention(const Layer &L, int rows) const;
     int capture_step_graph(int seq);
@@ -141,6 +141,7 @@ class LlamaRuntime {
     bool merged_attention_ = true;
     TrunkLayer *trunk_layers_ = nullptr;   // device table, set when the fused trunk kernel covers this model
     unsigned *trunk_sync_ = nullptr;
+    bool prompt_attention_ = false;   // prompt blocks run attention on the matrix cores
     float *gemm_workspace_ = nullptr;
 
     struct TimedLaunch { int kernel_class; hipEvent_t start, stop; };

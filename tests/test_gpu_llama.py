@@ -244,6 +244,34 @@ def test_matrix_prefill_matches_oracle_and_per_token_path(llama, fmt, count, kv_
         assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,kv_fp16,count", [
+    (2, 2, 128, True, 75), (4, 1, 128, False, 530), (4, 1, 128, True, 97), (4, 4, 64, False, 64), (4, 1, 64, True, 33),
+])
+def test_prompt_block_attention_on_the_matrix_cores(llama, heads, kv_heads, head_dim, kv_fp16, count):
+    """Prompt blocks run causal attention as MFMA tiles (32 rows x 32 keys) for head sizes 64 / 128 and 1, 2 or 4 query
+    heads per KV head: ragged last tiles, a prompt longer than one 512-row block, both cache types.  The state it leaves
+    agrees with the oracle's token-by-token walk and with the per-token GPU path."""
+    cfg = dict(TINY, n_head=heads, n_kv_head=kv_heads, head_dim=head_dim, max_seq=count + 8, vocab=512)
+    o, g = make_pair(llama, cfg, orc.FMT_Q8_0, seed=900 + count, std=0.08, kv_fp16=kv_fp16, norm_jitter=0.05)
+    prompt = np.random.default_rng(count).integers(0, 512, count).tolist()
+    o.prefill(prompt)
+    g.prefill(prompt)
+    ho, hg = o.last_hidden(), g.last_hidden()
+    scale = max(1.0, np.abs(ho).max())
+    assert np.abs(ho - hg).max() <= 4e-3 * scale, np.abs(ho - hg).max()
+    assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
+    llama.set_matrix_prefill(g, False)
+    g.reset()
+    g.prefill(prompt)
+    assert np.abs(g.last_hidden() - hg).max() <= 4e-3 * scale
+    llama.set_matrix_prefill(g, True)
+    # the cache the block left behind serves the single-query kernels of the decode steps
+    for _ in range(4):
+        t = o.select_greedy()
+        o.advance(t); g.advance(t)
+        assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
+
+
 def _batch_pair(llama, kw, fmt, seed, n_seq, std=0.08):
     ocfg = orc.LlamaConfig(gemv_inputs_fp16=True, **kw)
     w = mu.random_weights(ocfg, seed, std=std, norm_jitter=0.05)
