@@ -245,7 +245,8 @@ def test_matrix_prefill_matches_oracle_and_per_token_path(llama, fmt, count, kv_
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,kv_fp16,count", [
-    (2, 2, 128, True, 75), (4, 1, 128, False, 530), (4, 1, 128, True, 97), (4, 4, 64, False, 64), (4, 1, 64, True, 33),
+    (2, 2, 128, True, 75), (4, 1, 128, False, 530), (4, 1, 128, True, 97), (4, 2, 128, False, 40), (4, 4, 64, False, 64),
+    (4, 1, 64, True, 33),
 ])
 def test_prompt_block_attention_on_the_matrix_cores(llama, heads, kv_heads, head_dim, kv_fp16, count):
     """Prompt blocks run causal attention as MFMA tiles (32 rows x 32 keys) for head sizes 64 / 128 and 1, 2 or 4 query
