@@ -24,6 +24,7 @@
 //     adds the partial sums in split order (deterministic, no atomics).
 #include "../common.h"
 #include <atomic>
+#include <type_traits>
 
 namespace esp {
 namespace {
