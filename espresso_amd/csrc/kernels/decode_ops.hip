@@ -423,8 +423,8 @@ __global__ __launch_bounds__(HD) void attention_merge_kernel(AttentionArgs a, in
 // once per row, this one reads a key tile once per 32 rows.
 // grid (KV heads, tiles of 32 rows); wavefront g of a workgroup serves query head kvh * G + g, so the G heads that share
 // a KV head share the value tiles.  Per tile of 32 keys:
-//   * S^T = K Q^T: keys are the A rows (a lane loads eight consecutive dims of its key straight from the cache, the next
-//     tile's while this one is computed), queries the B columns (fragments kept in registers); a lane's 16 accumulators are
+//   * S^T = K Q^T: keys are the A rows (a lane loads eight consecutive dims of its key straight from the cache, two
+//     tiles ahead), queries the B columns (fragments kept in registers); a lane's 16 accumulators are
 //     16 keys of ONE query, so the row maximum and sum of the online softmax are in-lane plus one exchange with lane ^ 32;
 //   * O^T += V^T P: the probabilities a lane holds are already a B fragment (column = its query, k slots = its keys), and
 //     the A operand is the value tile transposed in LDS (written once per workgroup, double-buffered: one barrier per tile),
@@ -475,8 +475,7 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
     };
     // value tile: piece = (key, group of eight dims); consecutive lanes take consecutive keys so that the transposed
     // two-byte LDS writes of a wavefront spread over the banks
-    attn_half8 vreg[VP];
-    auto load_v = [&](int t0) {
+    auto load_v = [&](int t0, attn_half8 (&vreg)[VP]) {
 #pragma unroll
         for (int i = 0; i < VP; i++) {
             const int piece = tid + i * THREADS, key = piece & 31, dg = piece >> 5;
@@ -489,7 +488,7 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
             }
         }
     };
-    auto store_v = [&](int buf) {
+    auto store_v = [&](int buf, const attn_half8 (&vreg)[VP]) {
 #pragma unroll
         for (int i = 0; i < VP; i++) {
             const int piece = tid + i * THREADS, key = piece & 31, dg = piece >> 5;
@@ -506,15 +505,18 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
     float mx = -INFINITY, l = 0.0f;
     const int qpos = pos0 + col;
 
-    attn_half8 kf[KS];
+    // Keys and values are fetched two tiles ahead: one tile of arithmetic is shorter than a trip to memory.
+    attn_half8 kf[KS], k1[KS], k2[KS], v1[VP], v2[VP];
     load_k(0, kf);
-    load_v(0);
-    store_v(0);
+    load_v(0, v1);
+    store_v(0, v1);
+    load_k(32, k1);      // tiles beyond t_max are clamped to it, in bounds and never used
+    load_v(32, v1);
     __syncthreads();
     for (int t0 = 0, buf = 0; t0 <= t_max; t0 += 32, buf ^= 1) {
         const bool more = t0 + 32 <= t_max;
-        attn_half8 kn[KS];
-        if (more) { load_k(t0 + 32, kn); load_v(t0 + 32); }
+        load_k(t0 + 64, k2);
+        load_v(t0 + 64, v2);
         attn_floatx16 sc;
 #pragma unroll
         for (int r = 0; r < 16; r++) sc[r] = 0.0f;
@@ -555,11 +557,11 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
                 o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[j], o[mt], 0, 0, 0);
             }
         }
-        if (more) {
-            store_v(buf ^ 1);
+        if (more) store_v(buf ^ 1, v1);
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) kf[ks] = kn[ks];
-        }
+        for (int ks = 0; ks < KS; ks++) { kf[ks] = k1[ks]; k1[ks] = k2[ks]; }
+#pragma unroll
+        for (int i = 0; i < VP; i++) v1[i] = v2[i];
         __syncthreads();
     }
     l += __shfl_xor(l, 32);
