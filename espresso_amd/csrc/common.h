@@ -97,6 +97,9 @@ struct GemmParams {
     int rows = 0;
     float *workspace = nullptr;       // split-K partial sums for short row counts (optional)
     size_t workspace_floats = 0;
+    // optional fp16 [rows][w.rows / 2]: silu(y[2i]) * y[2i + 1] for a matrix whose rows are (gate, up) pairs; y is then
+    // scratch (written only when the SwiGLU could not be done in the GEMM's own epilogue)
+    uint16_t *swiglu_out = nullptr;
 };
 
 // kernels/gemv.hip

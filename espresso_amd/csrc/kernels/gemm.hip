@@ -23,6 +23,7 @@
 //   * when the (n, m) grid is too small to fill the chip, K is split over grid.y and a small kernel
 //     adds the partial sums in split order (deterministic, no atomics).
 #include "../common.h"
+#include "decode_ops.h"
 #include <atomic>
 #include <type_traits>
 
@@ -49,6 +50,7 @@ struct GemmArgs {
     const float *residual;  // [M][N] or null
     float *partial;         // [splits][M][N] when gridDim.y > 1
     int tiles_per_split;
+    uint16_t *swiglu_out;   // tile kernel without split-K only: fp16 [M][N / 2] instead of y
 };
 
 __device__ __forceinline__ h2 as_h2(u32 v) { return __builtin_bit_cast(h2, v); }
@@ -299,6 +301,32 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs a) {
     }
 
     // accumulator r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32 x 32 tile
+    if (a.swiglu_out) {   // rows of W are (gate, up) pairs: even lanes hold gate, their right neighbours up (:6825-6827, :6337)
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const int n = n0 + (wn * TN + j) * 32 + (lane & 31);
+                // a pair of lanes holds (gate, up) of one unit for 16 rows; the even lane finishes the even accumulators, the
+                // odd lane the odd ones, so that no lane idles through the tanh
+                const bool odd = lane & 1;
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    const float a0 = acc[i][j][2 * k], a1 = acc[i][j][2 * k + 1];
+                    const float p0 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a0), 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+                    const float p1 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a1), 0xB1, 0xF, 0xF, false));
+                    const float g = odd ? p1 : a0, u = odd ? a1 : p0;
+                    const int r = 2 * k + (odd ? 1 : 0);
+                    const int m = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (m < a.M && (n | 1) < a.N) {
+                        const float hg = __fmul_rn(0.5f, g);
+                        const float silu = __fmul_rn(hg, __fadd_rn(1.0f, tanhf(hg)));
+                        a.swiglu_out[(size_t)m * (a.N / 2) + n / 2] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(silu, u));
+                    }
+                }
+            }
+        return;
+    }
     const bool split = gridDim.y > 1;
     float *out = split ? a.partial + (size_t)blockIdx.y * a.M * a.N : a.y;
 #pragma unroll
@@ -752,8 +780,10 @@ int choose_splits(int blocks, int units, int min_units, int target, const GemmAr
     return splits;
 }
 
+// `swiglu_out` (may be null) is handed to the tile kernel when it runs without split-K; *fused tells the caller.
 template <int FMT>
-hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, hipStream_t stream) {
+hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, uint16_t *swiglu_out, bool *fused, hipStream_t stream) {
+    *fused = false;
     const int n_blocks = (a.N + NT - 1) / NT;
     a.partial = workspace;
     hipError_t e;
@@ -802,6 +832,7 @@ hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, 
     splits = choose_splits(n_blocks * ((a.M + mt - 1) / mt), tiles, 8, 1024, a, workspace_floats);
     a.tiles_per_split = ((tiles + splits - 1) / splits + 3) & ~3;   // every split starts on a multiple of four tiles
     splits = (tiles + a.tiles_per_split - 1) / a.tiles_per_split;
+    if (splits == 1 && swiglu_out && a.N % 2 == 0) { a.swiglu_out = swiglu_out; *fused = true; }
     if (mt == 32) e = launch_tile<FMT, 1, 4, 1, 1, 4>(a, splits, stream);
     else if (mt == 64) e = launch_tile<FMT, 1, 4, 2, 1, 4>(a, splits, stream);
     else e = launch_tile<FMT, 2, 2, 2, 2, 2>(a, splits, stream);
@@ -818,13 +849,18 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t stream) {
     GemmArgs a{};
     a.qs = w.qs; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.N = w.rows; a.K = w.cols; a.M = p.rows;
     a.x = p.x; a.y = p.y; a.residual = p.residual;
+    bool fused = false;
+    hipError_t e;
     switch (w.format) {
-    case FMT_Q4_K: return launch_format<FMT_Q4_K>(a, p.workspace, p.workspace_floats, stream);
-    case FMT_Q4_0: return launch_format<FMT_Q4_0>(a, p.workspace, p.workspace_floats, stream);
-    case FMT_Q8_0: return launch_format<FMT_Q8_0>(a, p.workspace, p.workspace_floats, stream);
-    case FMT_F16: return launch_format<FMT_F16>(a, p.workspace, p.workspace_floats, stream);
+    case FMT_Q4_K: e = launch_format<FMT_Q4_K>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, stream); break;
+    case FMT_Q4_0: e = launch_format<FMT_Q4_0>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, stream); break;
+    case FMT_Q8_0: e = launch_format<FMT_Q8_0>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, stream); break;
+    case FMT_F16: e = launch_format<FMT_F16>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, stream); break;
     default: return hipErrorInvalidValue;   // fp32 matrices stay on the GEMV path
     }
+    if (e != hipSuccess || !p.swiglu_out || fused) return e;
+    if (w.rows % 2 != 0 || p.residual) return hipErrorInvalidValue;
+    return launch_swiglu(p.y, p.rows, w.rows / 2, p.swiglu_out, stream);
 }
 
 }  // namespace esp

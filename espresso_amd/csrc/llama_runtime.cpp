@@ -682,9 +682,9 @@ int LlamaRuntime::enqueue_layers_matrix(int rows, bool one_sequence_consecutive)
         g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_;
         ESP_HIP_TRY(launch_gemm(g, s));
         ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_ffn, c_.norm_eps, rows, d, xn_, nullptr, s));
-        g.w = L.w13; g.x = xn_; g.y = gu_; g.residual = nullptr;
+        g.w = L.w13; g.x = xn_; g.y = gu_; g.residual = nullptr; g.swiglu_out = act_;   // SwiGLU in the GEMM's epilogue where it can be
         ESP_HIP_TRY(launch_gemm(g, s));
-        ESP_HIP_TRY(launch_swiglu(gu_, rows, hd, act_, s));
+        g.swiglu_out = nullptr;
         g.w = L.w2; g.x = act_; g.y = hidden_; g.residual = hidden_;
         ESP_HIP_TRY(launch_gemm(g, s));
     }

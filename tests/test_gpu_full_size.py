@@ -109,6 +109,26 @@ def test_8b_shaped_layer_and_head_match_oracle(mods):
     print(f"8B-shaped layer + head: worst logit difference {worst:.2e}")
     g.close()
 
+def test_8b_shaped_layer_prompt_block_matches_oracle(mods):
+    """A 160-token prompt through one layer of the 8B shape: the block path at its real sizes (two row tiles of the MFMA
+    GEMM, gate|up without split-K so that SwiGLU runs in the GEMM's epilogue, causal attention on the matrix cores with a
+    ragged last tile) against the oracle's token-by-token walk."""
+    ll, ops, syn = mods
+    cfg = ll.MultiModelConfig(**dict(syn.LLAMA3_8B, n_layer=1, max_seq=176))
+    g, packed = syn.build_runtime(cfg, orc.FMT_Q4_K, seed=21, kv_format=orc.FMT_F16, keep_packed=True)
+    o = oracle_from_packed(cfg, packed, orc.FMT_Q4_K, 1, True, 176)
+    prompt = np.random.default_rng(160).integers(0, cfg.vocab, 160).astype(np.uint32)
+    o.prefill([int(t) for t in prompt])
+    g.prefill(prompt)
+    ho, hg = o.last_hidden(), g.last_hidden()
+    assert np.abs(ho - hg).max() <= 4e-3 * max(1.0, np.abs(ho).max()), np.abs(ho - hg).max()
+    assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
+    ll.set_matrix_prefill(g, False)
+    g.reset()
+    g.prefill(prompt)
+    assert np.abs(g.last_hidden() - hg).max() <= 4e-3 * max(1.0, np.abs(ho).max())
+    g.close()
+
 
 def test_8b_arch_whole_model_invariants(mods):
     """32 layers, Q4_K, fp16 KV: properties that hold by construction and need no CPU run."""
