@@ -100,6 +100,9 @@ struct GemmParams {
     // optional fp16 [rows][w.rows / 2]: silu(y[2i]) * y[2i + 1] for a matrix whose rows are (gate, up) pairs; y is then
     // scratch (written only when the SwiGLU could not be done in the GEMM's own epilogue)
     uint16_t *swiglu_out = nullptr;
+    // optional: when the GEMM runs split-K, leave the partial sums [splits][rows][w.rows] in `workspace` for the caller's
+    // next kernel to add (launch_rmsnorm_reduce) and report the split count here; 1 = y is complete
+    int *deferred_splits = nullptr;
 };
 
 // kernels/gemv.hip

@@ -53,6 +53,11 @@ int attention_split_count(int max_seq, int head_dim);
 hipError_t launch_embed(const void *table, bool table_is_f16, const int *tokens, int rows, int d, float *hidden, hipStream_t s);
 hipError_t launch_rmsnorm(const float *x, const float *w, float eps, int rows, int d, uint16_t *out_f16,
                           unsigned long long *argmax_cells, hipStream_t s);
+// RMSNorm of rows that are still split-K partial sums [splits][rows][d] (`plane` = rows * d floats apart): adds them in
+// split order (+ residual), writes the sums to y and the normalised fp16 rows to out_f16.  d % 4 == 0, d <= 8192.
+bool rmsnorm_reduce_supported(int d);
+hipError_t launch_rmsnorm_reduce(const float *partial, int splits, size_t plane, const float *residual, float *y, const float *w, float eps,
+                                 int rows, int d, uint16_t *out_f16, hipStream_t s);
 hipError_t launch_qkv_post(const QkvPostArgs &a, int rows, bool kv_f16, hipStream_t s);
 hipError_t launch_attention(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s);
 // Causal attention of `rows` rows that are ONE sequence at consecutive positions (a prompt block), on the matrix cores.

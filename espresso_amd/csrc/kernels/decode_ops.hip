@@ -184,6 +184,54 @@ __global__ void qkv_post_kernel(QkvPostArgs a) {
     }
 }
 
+// rmsnorm_kernel for a row whose values are still split-K partial sums of a GEMM: x = (residual +) partial[0] + partial[1]
+// + ... in split order (the sum gemm_reduce_kernel forms), written to y, then normalised as above.  One workgroup per row,
+// d a multiple of four and at most 8192.
+__global__ __launch_bounds__(kBlock) void rmsnorm_reduce_kernel(const float *partial, int splits, size_t plane, const float *residual, float *y,
+                                                                const float *w, float eps, int d, uint16_t *out_f16) {
+    __shared__ float scratch[16];
+    const int m = blockIdx.x;
+    constexpr int kVec = 8;
+    const int n4 = d / 4;
+    const float4 *w4 = reinterpret_cast<const float4 *>(w);
+    float4 v[kVec], g[kVec];
+#pragma unroll
+    for (int k = 0; k < kVec; k++) {
+        const int i = threadIdx.x + k * kBlock;
+        v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+        g[k] = v[k];
+        if (i < n4) {
+            const size_t o = (size_t)m * n4 + i;
+            float4 s = reinterpret_cast<const float4 *>(partial)[o];
+            for (int sp = 1; sp < splits; sp++) {
+                const float4 t = reinterpret_cast<const float4 *>(partial + (size_t)sp * plane)[o];
+                s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+            }
+            if (residual) {
+                const float4 r = reinterpret_cast<const float4 *>(residual)[o];
+                s.x = r.x + s.x; s.y = r.y + s.y; s.z = r.z + s.z; s.w = r.w + s.w;
+            }
+            reinterpret_cast<float4 *>(y)[o] = s;
+            v[k] = s;
+            g[k] = w4[i];
+        }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kVec; k++) s += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+    const float inv = 1.0f / sqrtf(block_sum(s, scratch) / (float)d + eps);
+#pragma unroll
+    for (int k = 0; k < kVec; k++) {
+        const int i = threadIdx.x + k * kBlock;
+        if (i < n4) {
+            uint2 o;
+            o.x = to_half_bits(__fmul_rn(__fmul_rn(v[k].x, inv), g[k].x)) | ((uint32_t)to_half_bits(__fmul_rn(__fmul_rn(v[k].y, inv), g[k].y)) << 16);
+            o.y = to_half_bits(__fmul_rn(__fmul_rn(v[k].z, inv), g[k].z)) | ((uint32_t)to_half_bits(__fmul_rn(__fmul_rn(v[k].w, inv), g[k].w)) << 16);
+            reinterpret_cast<uint2 *>(out_f16 + (size_t)m * d)[i] = o;
+        }
+    }
+}
+
 // Single-query attention over the visible prefix of one sequence's KV cache (:6774-6823): the
 // general kernel, one workgroup per (head, row), any head size.  Scores use the reference's exact
 // per-token sum (dims ascending, separate multiply and add); the softmax sums and the value sums
@@ -968,6 +1016,15 @@ hipError_t launch_attention_partials(const AttentionArgs &a, int rows, bool kv_f
         if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<64, true, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
         else hipLaunchKernelGGL((attention_partial_kernel<64, false, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
     }
+    return hipGetLastError();
+}
+
+bool rmsnorm_reduce_supported(int d) { return d % 4 == 0 && d <= 8 * 4 * kBlock; }
+
+hipError_t launch_rmsnorm_reduce(const float *partial, int splits, size_t plane, const float *residual, float *y, const float *w, float eps,
+                                 int rows, int d, uint16_t *out_f16, hipStream_t s) {
+    if (!rmsnorm_reduce_supported(d) || splits < 1 || plane % 4 != 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(rmsnorm_reduce_kernel, dim3(rows), dim3(kBlock), 0, s, partial, splits, plane, residual, y, w, eps, d, out_f16);
     return hipGetLastError();
 }
 

@@ -782,8 +782,14 @@ int choose_splits(int blocks, int units, int min_units, int target, const GemmAr
 
 // `swiglu_out` (may be null) is handed to the tile kernel when it runs without split-K; *fused tells the caller.
 template <int FMT>
-hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, uint16_t *swiglu_out, bool *fused, hipStream_t stream) {
+hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, uint16_t *swiglu_out, bool *fused, int *deferred_splits, hipStream_t stream) {
     *fused = false;
+    // split-K partial sums are added by gemm_reduce_kernel, or left to the caller's next kernel when it asked for that
+    auto finish = [&](hipError_t err, int used_splits) {
+        if (err != hipSuccess || used_splits == 1) return err;
+        if (deferred_splits) { *deferred_splits = used_splits; return hipSuccess; }
+        return launch_reduce(a, used_splits, stream);
+    };
     const int n_blocks = (a.N + NT - 1) / NT;
     a.partial = workspace;
     hipError_t e;
@@ -822,7 +828,7 @@ hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, 
             if (a.M <= 32) hipLaunchKernelGGL((gemm_skinny_kernel<FMT, 1, 2>), grid, dim3(kThreads), 0, stream, a);
             else hipLaunchKernelGGL((gemm_skinny_kernel<FMT, 2, 2>), grid, dim3(kThreads), 0, stream, a);
             e = hipGetLastError();
-            return e != hipSuccess || splits == 1 ? e : launch_reduce(a, splits, stream);
+            return finish(e, splits);
         }
     }
     const int tiles = a.K / KT;
@@ -836,7 +842,7 @@ hipError_t launch_format(GemmArgs a, float *workspace, size_t workspace_floats, 
     if (mt == 32) e = launch_tile<FMT, 1, 4, 1, 1, 4>(a, splits, stream);
     else if (mt == 64) e = launch_tile<FMT, 1, 4, 2, 1, 4>(a, splits, stream);
     else e = launch_tile<FMT, 2, 2, 2, 2, 2>(a, splits, stream);
-    return e != hipSuccess || splits == 1 ? e : launch_reduce(a, splits, stream);
+    return finish(e, splits);
 }
 
 }  // namespace
@@ -851,11 +857,12 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t stream) {
     a.x = p.x; a.y = p.y; a.residual = p.residual;
     bool fused = false;
     hipError_t e;
+    if (p.deferred_splits) *p.deferred_splits = 1;
     switch (w.format) {
-    case FMT_Q4_K: e = launch_format<FMT_Q4_K>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, stream); break;
-    case FMT_Q4_0: e = launch_format<FMT_Q4_0>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, stream); break;
-    case FMT_Q8_0: e = launch_format<FMT_Q8_0>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, stream); break;
-    case FMT_F16: e = launch_format<FMT_F16>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, stream); break;
+    case FMT_Q4_K: e = launch_format<FMT_Q4_K>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, p.deferred_splits, stream); break;
+    case FMT_Q4_0: e = launch_format<FMT_Q4_0>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, p.deferred_splits, stream); break;
+    case FMT_Q8_0: e = launch_format<FMT_Q8_0>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, p.deferred_splits, stream); break;
+    case FMT_F16: e = launch_format<FMT_F16>(a, p.workspace, p.workspace_floats, p.swiglu_out, &fused, p.deferred_splits, stream); break;
     default: return hipErrorInvalidValue;   // fp32 matrices stay on the GEMV path
     }
     if (e != hipSuccess || !p.swiglu_out || fused) return e;

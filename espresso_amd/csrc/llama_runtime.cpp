@@ -663,8 +663,22 @@ int LlamaRuntime::enqueue_layers_matrix(int rows, bool one_sequence_consecutive)
     const size_t cache_seq_stride = (size_t)kd * c_.max_seq;
     GemmParams g;
     g.rows = rows; g.workspace = gemm_workspace_; g.workspace_floats = kGemmWorkspaceFloats;
-    for (Layer &L : layers_) {
-        ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_att, c_.norm_eps, rows, d, xn_, nullptr, s));
+    // The RMSNorm that follows a projection with a residual reads that projection's result; when the GEMM ran split-K the
+    // norm kernel adds the partial sums itself (one launch instead of reduce + norm).
+    const bool fuse_norm = rmsnorm_reduce_supported(d);
+    auto project_and_norm = [&](const float *norm_w) -> int {   // g is set up for a GEMM into hidden_ with hidden_ as residual
+        int splits = 1;
+        g.deferred_splits = norm_w && fuse_norm ? &splits : nullptr;
+        ESP_HIP_TRY(launch_gemm(g, s));
+        g.deferred_splits = nullptr;
+        if (!norm_w) return ESP_OK;
+        if (splits > 1) ESP_HIP_TRY(launch_rmsnorm_reduce(gemm_workspace_, splits, (size_t)rows * d, hidden_, hidden_, norm_w, c_.norm_eps, rows, d, xn_, s));
+        else ESP_HIP_TRY(launch_rmsnorm(hidden_, norm_w, c_.norm_eps, rows, d, xn_, nullptr, s));
+        return ESP_OK;
+    };
+    ESP_HIP_TRY(launch_rmsnorm(hidden_, layers_.front().rms_att, c_.norm_eps, rows, d, xn_, nullptr, s));
+    for (size_t li = 0; li < layers_.size(); li++) {
+        Layer &L = layers_[li];
         g.w = L.wqkv; g.x = xn_; g.y = qkv_; g.residual = nullptr;
         ESP_HIP_TRY(launch_gemm(g, s));
         QkvPostArgs qa{};
@@ -680,13 +694,12 @@ int LlamaRuntime::enqueue_layers_matrix(int rows, bool one_sequence_consecutive)
         if (one_sequence_consecutive && prompt_attention_) ESP_HIP_TRY(launch_attention_prompt(aa, rows, kv16, s));
         else ESP_HIP_TRY(launch_attention(aa, rows, kv16, s));
         g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_;
-        ESP_HIP_TRY(launch_gemm(g, s));
-        ESP_HIP_TRY(launch_rmsnorm(hidden_, L.rms_ffn, c_.norm_eps, rows, d, xn_, nullptr, s));
+        { int rc = project_and_norm(L.rms_ffn); if (rc != ESP_OK) return rc; }
         g.w = L.w13; g.x = xn_; g.y = gu_; g.residual = nullptr; g.swiglu_out = act_;   // SwiGLU in the GEMM's epilogue where it can be
         ESP_HIP_TRY(launch_gemm(g, s));
         g.swiglu_out = nullptr;
         g.w = L.w2; g.x = act_; g.y = hidden_; g.residual = hidden_;
-        ESP_HIP_TRY(launch_gemm(g, s));
+        { int rc = project_and_norm(li + 1 < layers_.size() ? layers_[li + 1].rms_att : nullptr); if (rc != ESP_OK) return rc; }
     }
     (void)ad;
     return ESP_OK;
