@@ -30,6 +30,10 @@ struct QkvPostArgs {
     void *k_cache;          // this layer: [seq][max_seq][kvDim]
     void *v_cache;          // this layer: [seq][max_seq][kvDim]
     size_t cache_seq_stride;  // elements per sequence (kvDim * max_seq)
+    // `qkv` may still be the split-K partial sums of its GEMM: `splits` planes, `plane` floats apart, added in split order
+    // on load (0 or 1: qkv is complete)
+    int splits;
+    size_t plane;
 };
 
 struct AttentionArgs {

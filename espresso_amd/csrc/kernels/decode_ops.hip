@@ -138,11 +138,16 @@ __global__ void qkv_post_kernel(QkvPostArgs a) {
     const size_t seq_base = (size_t)a.seq[m] * a.cache_seq_stride;
     const int j = threadIdx.x;  // pair index; blockDim.x is `half` rounded up to whole wavefronts
     const bool live = j < half;
+    auto value = [&](const float *p) {   // the GEMM's result, or the sum of its split-K partial sums in split order
+        float s = p[0];
+        for (int sp = 1; sp < a.splits; sp++) s += p[(size_t)sp * a.plane];
+        return s;
+    };
     if (slot < nh + nkv) {
         const bool is_q = slot < nh;
         const int h = is_q ? slot : slot - nh;
         const float *src = row + (is_q ? 0 : ad) + (size_t)h * a.head_dim;
-        float v0 = live ? src[2 * j] : 0.0f, v1 = live ? src[2 * j + 1] : 0.0f;
+        float v0 = live ? value(src + 2 * j) : 0.0f, v1 = live ? value(src + 2 * j + 1) : 0.0f;
         const float *norm_w = is_q ? a.q_norm : a.k_norm;
         if (norm_w) {
             const float sum_sq = block_sum(v0 * v0 + v1 * v1, scratch);
@@ -178,8 +183,9 @@ __global__ void qkv_post_kernel(QkvPostArgs a) {
         const float *src = row + ad + kd + (size_t)h * a.head_dim;
         const size_t c0 = seq_base + (size_t)pos * kd + (size_t)h * a.head_dim;
         for (int i = j; i < a.head_dim; i += blockDim.x) {
-            if (KV_F16) reinterpret_cast<uint16_t *>(a.v_cache)[c0 + i] = to_half_bits(src[i]);
-            else reinterpret_cast<float *>(a.v_cache)[c0 + i] = src[i];
+            const float v = value(src + i);
+            if (KV_F16) reinterpret_cast<uint16_t *>(a.v_cache)[c0 + i] = to_half_bits(v);
+            else reinterpret_cast<float *>(a.v_cache)[c0 + i] = v;
         }
     }
 }

@@ -679,10 +679,13 @@ int LlamaRuntime::enqueue_layers_matrix(int rows, bool one_sequence_consecutive)
     ESP_HIP_TRY(launch_rmsnorm(hidden_, layers_.front().rms_att, c_.norm_eps, rows, d, xn_, nullptr, s));
     for (size_t li = 0; li < layers_.size(); li++) {
         Layer &L = layers_[li];
-        g.w = L.wqkv; g.x = xn_; g.y = qkv_; g.residual = nullptr;
+        int qkv_splits = 1;   // split-K partial sums of q|k|v are added by the kernel that applies norm / RoPE and writes the caches
+        g.w = L.wqkv; g.x = xn_; g.y = qkv_; g.residual = nullptr; g.deferred_splits = &qkv_splits;
         ESP_HIP_TRY(launch_gemm(g, s));
+        g.deferred_splits = nullptr;
         QkvPostArgs qa{};
-        qa.qkv = qkv_; qa.q_norm = L.q_norm; qa.k_norm = L.k_norm; qa.norm_eps = c_.norm_eps;
+        qa.qkv = qkv_splits > 1 ? gemm_workspace_ : qkv_; qa.splits = qkv_splits; qa.plane = (size_t)rows * (ad + 2 * kd);
+        qa.q_norm = L.q_norm; qa.k_norm = L.k_norm; qa.norm_eps = c_.norm_eps;
         qa.n_head = c_.n_head; qa.n_kv_head = c_.n_kv_head; qa.head_dim = c_.head_dim; qa.max_seq = c_.max_seq;
         qa.rope_cos = rope_cos_; qa.rope_sin = rope_sin_; qa.pos = d_pos_; qa.seq = d_seq_;
         qa.q_out = q_; qa.k_cache = L.k_cache; qa.v_cache = L.v_cache; qa.cache_seq_stride = cache_seq_stride;
