@@ -130,11 +130,7 @@ def _declare_llama(L: C.CDLL) -> None:
     L.esp_synth_weights.argtypes = [i32, C.c_uint64, C.c_float, sz, vp]
     L.esp_llama_set_graph_replay.restype = i32
     L.esp_llama_set_graph_replay.argtypes = [vp, i32]
-    L.esp_llama_set_fused_trunk.restype = i32
-    L.esp_llama_set_fused_trunk.argtypes = [vp, i32]
     L.esp_llama_set_merged_attention.restype = i32
     L.esp_llama_set_merged_attention.argtypes = [vp, i32]
-    L.esp_llama_fused_trunk_status.restype = i32
-    L.esp_llama_fused_trunk_status.argtypes = [vp, C.POINTER(i32), C.POINTER(C.c_uint)]
     L.esp_llama_set_matrix_prefill.restype = i32
     L.esp_llama_set_matrix_prefill.argtypes = [vp, i32]

@@ -153,25 +153,10 @@ int esp_llama_set_graph_replay(ESPLlamaRuntime *runtime, int enabled) {
     return ESP_OK;
 }
 
-int esp_llama_set_fused_trunk(ESPLlamaRuntime *runtime, int enabled) {
-    if (!runtime || !runtime->rt) return fail(ESP_ERR_INVALID_ARGUMENT, "set_fused_trunk: null runtime");
-    runtime->rt->set_fused_trunk(enabled != 0);
-    return ESP_OK;
-}
-
 int esp_llama_set_merged_attention(ESPLlamaRuntime *runtime, int enabled) {
     if (!runtime || !runtime->rt) return fail(ESP_ERR_INVALID_ARGUMENT, "set_merged_attention: null runtime");
     runtime->rt->set_merged_attention(enabled != 0);
     return runtime->rt->merged_attention_in_use() ? 1 : 0;
-}
-
-int esp_llama_fused_trunk_status(ESPLlamaRuntime *runtime, int *active, unsigned *barrier_timeouts) {
-    if (!runtime || !runtime->rt) return fail(ESP_ERR_INVALID_ARGUMENT, "fused_trunk_status: null runtime");
-    if (active) *active = runtime->rt->fused_trunk_active() ? 1 : 0;
-    unsigned n = 0;
-    int rc = runtime->rt->fused_trunk_timeouts(&n);
-    if (barrier_timeouts) *barrier_timeouts = n;
-    return rc;
 }
 
 int esp_llama_set_matrix_prefill(ESPLlamaRuntime *runtime, int enabled) {

@@ -71,8 +71,6 @@ LlamaRuntime::~LlamaRuntime() {
     free_device(d_visible_); free_device(d_log_); free_device(d_log_count_);
     free_device(attn_scratch_);
     free_device(gemm_workspace_);
-    free_device(trunk_layers_);
-    free_device(trunk_sync_);
     free_device(argmax_scratch_.part_value); free_device(argmax_scratch_.part_index);
     for (hipGraphExec_t g : step_graphs_) if (g) (void)hipGraphExecDestroy(g);
     for (TimedLaunch &t : timed_) { (void)hipEventDestroy(t.start); (void)hipEventDestroy(t.stop); }
@@ -128,10 +126,9 @@ int LlamaRuntime::collect_kernel_times(double total_us[K_CLASS_COUNT], long laun
 // two events: back-to-back dependent launches at the real shapes over the real weights, which no cache can hold
 // across a round.  The epilogues write into the step's buffers, so sequence state is garbage afterwards.
 // The decode step (one or two rows) runs attention as a single launch that leaves per-head partial states, and
-// the wo GEMV merges them while staging, when the head size and the matrix allow it.  The fused trunk keeps the
-// split-and-merge arithmetic it is compared with.
+// the wo GEMV merges them while staging, when the head size and the matrix allow it.
 bool LlamaRuntime::wo_merges_attention(const Layer &L, int rows) const {
-    return merged_attention_ && !fused_trunk_active() && c_.n_head % c_.n_kv_head == 0 && rows <= 2 &&
+    return merged_attention_ && c_.n_head % c_.n_kv_head == 0 && rows <= 2 &&
            L.wo.cols == c_.attention_dim() && gemv_merges_attention_partials(L.wo, rows, c_.head_dim);
 }
 
@@ -402,21 +399,8 @@ int LlamaRuntime::finalize() {
     }
     if ((rc = device_alloc(&gemm_workspace_, kGemmWorkspaceFloats)) != ESP_OK) return rc;
     {
-        bool all_q4k = true;
-        for (const Layer &L : layers_)
-            all_q4k = all_q4k && L.wqkv.format == FMT_Q4_K && L.wo.format == FMT_Q4_K && L.w13.format == FMT_Q4_K && L.w2.format == FMT_Q4_K && !L.q_norm;
         const char *pa = getenv("ESPRESSO_HIP_PROMPT_ATTENTION");   // "0": prompt blocks keep the single-query attention kernel
         prompt_attention_ = attention_prompt_supported(c_.n_head, c_.n_kv_head, c_.head_dim) && !(pa && pa[0] == '0');
-        const char *env = getenv("ESPRESSO_HIP_FUSED_TRUNK");
-        fused_trunk_ = env && env[0] == '1';   // measured slower than the separate kernels: opt-in
-        if (all_q4k && trunk_kernel_supports(d, hd, c_.head_dim, c_.n_head, c_.n_kv_head)) {
-            std::vector<TrunkLayer> table;
-            for (const Layer &L : layers_) table.push_back(TrunkLayer{L.wqkv.qs, L.wo.qs, L.w13.qs, L.w2.qs, L.rms_att, L.rms_ffn, L.k_cache, L.v_cache});
-            if ((rc = device_alloc(&trunk_layers_, table.size())) != ESP_OK) return rc;
-            ESP_HIP_TRY(hipMemcpy(trunk_layers_, table.data(), table.size() * sizeof(TrunkLayer), hipMemcpyHostToDevice));
-            if ((rc = device_alloc(&trunk_sync_, (size_t)kTrunkSyncWords)) != ESP_OK) return rc;
-            ESP_HIP_TRY(hipMemset(trunk_sync_, 0, kTrunkSyncWords * sizeof(unsigned)));
-        }
     }
     finalized_ = true;
     return reset();
@@ -475,16 +459,6 @@ int LlamaRuntime::enqueue_trunk(int M, bool embedded, float *final_out) {
     }
     // more than two rows (batched sequences, batched verify): one pass over the weights on the matrix cores
     if (M > 2 && matrix_prefill_ && matrix_prefill_supported()) return enqueue_layers_matrix(M);
-    if (M == 1 && fused_trunk_active() && !timing_enabled_) {
-        TrunkArgs t{};
-        t.layers = trunk_layers_; t.n_layer = c_.n_layer; t.hidden = hidden_; t.q = q_; t.ctx = ctx_; t.act = act_;
-        t.attn_scratch = attn_scratch_; t.rope_cos = rope_cos_; t.rope_sin = rope_sin_; t.pos = d_pos_; t.seq = d_seq_;
-        t.n_head = c_.n_head; t.n_kv_head = c_.n_kv_head; t.max_seq = c_.max_seq; t.kv_f16 = kv16 ? 1 : 0;
-        t.cache_seq_stride = (size_t)kd * c_.max_seq; t.norm_eps = c_.norm_eps; t.sync = trunk_sync_;
-        t.splits = attention_split_count(c_.max_seq, c_.head_dim);
-        ESP_HIP_TRY(launch_trunk_kernel(t, d, hd, s));
-        return ESP_OK;
-    }
     for (Layer &L : layers_) {
         // both RMSNorms of the layer run inside the staging of the GEMV that consumes them
         GemvParams g;
@@ -547,36 +521,10 @@ int LlamaRuntime::enqueue_trunk(int M, bool embedded, float *final_out) {
     return ESP_OK;
 }
 
-void LlamaRuntime::set_fused_trunk(bool enabled) {
-    if (enabled == fused_trunk_) return;
-    fused_trunk_ = enabled;
-    for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }   // captured with the other path
-}
-
 void LlamaRuntime::set_merged_attention(bool enabled) {
     if (enabled == merged_attention_) return;
     merged_attention_ = enabled;
     for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }   // captured with the other path
-}
-
-// A barrier of the fused trunk kernel that timed out means its results are garbage: fail loudly and fall
-// back to the separate kernels for the rest of the runtime's life.
-int LlamaRuntime::check_fused_trunk() {
-    if (!fused_trunk_active()) return ESP_OK;
-    unsigned n = 0;
-    int rc = fused_trunk_timeouts(&n);
-    if (rc != ESP_OK) return rc;
-    if (n == 0) return ESP_OK;
-    fused_trunk_ = false;
-    for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
-    return fail(ESP_ERR_LAUNCH_FAILED, "fused trunk kernel: %u barrier time-outs; its output is invalid (fused path disabled)", n);
-}
-
-int LlamaRuntime::fused_trunk_timeouts(unsigned *out) {
-    *out = 0;
-    if (!trunk_sync_) return ESP_OK;
-    ESP_HIP_TRY(trunk_kernel_timeouts(trunk_sync_, context().stream, out));
-    return ESP_OK;
 }
 
 int LlamaRuntime::keep_row(int row, int seq) {
@@ -738,7 +686,6 @@ int LlamaRuntime::select_greedy(int seq, uint32_t *token) {
     int t = 0;
     ESP_HIP_TRY(hipMemcpyAsync(&t, d_out_tokens_, sizeof(int), hipMemcpyDeviceToHost, context().stream));
     ESP_HIP_TRY(hipStreamSynchronize(context().stream));
-    if ((rc = check_fused_trunk()) != ESP_OK) return rc;
     *token = (uint32_t)t;
     return ESP_OK;
 }
@@ -763,16 +710,7 @@ int LlamaRuntime::capture_step_graph(int seq) {
     ESP_HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
     int rc = ESP_OK;
     float *kept = last_hidden_ + (size_t)seq * c_.d_model;
-    if (fused_trunk_active()) {
-        rc = run_head(kept, 1);
-        if (rc == ESP_OK) {
-            hipError_t e = launch_greedy_feed(d_out_tokens_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_, d_log_count_,
-                                              c_.max_seq, s);
-            if (e != hipSuccess) rc = fail_hip(e, "greedy_feed");
-        }
-        if (rc == ESP_OK) rc = enqueue_trunk(1);
-        if (rc == ESP_OK) rc = keep_row(0, seq);
-    } else {
+    {
         // head GEMV, argmax slices, then one launch that picks the token, feeds it and fetches its embedding; the
         // last layer writes the new hidden state where the next step's head reads it: 3 + 5 per layer launches
         GemvParams g;
@@ -830,7 +768,6 @@ int LlamaRuntime::continue_greedy(int seq, int steps, uint32_t *out_tokens) {
     std::vector<int> log(steps);
     ESP_HIP_TRY(hipMemcpyAsync(log.data(), d_log_, sizeof(int) * steps, hipMemcpyDeviceToHost, s));
     ESP_HIP_TRY(hipStreamSynchronize(s));
-    if ((rc = check_fused_trunk()) != ESP_OK) return rc;
     visible_[seq] += steps;
     if (out_tokens) for (int i = 0; i < steps; i++) out_tokens[i] = (uint32_t)log[i];
     return ESP_OK;

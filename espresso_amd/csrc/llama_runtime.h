@@ -7,7 +7,6 @@
 
 #include "context.h"
 #include "kernels/decode_ops.h"
-#include "kernels/layer_kernel.h"
 
 namespace esp {
 
@@ -67,16 +66,10 @@ class LlamaRuntime {
     void set_use_graph(bool enabled) { use_graph_ = enabled; }
     // Prompts of kMatrixPrefillMinTokens or more run in blocks through the MFMA kernels (default on).
     void set_matrix_prefill(bool enabled) { matrix_prefill_ = enabled; }
-    // Batch-1 steps of an all-Q4_K model whose shape the fused trunk kernel covers run the whole layer
-    // stack as one persistent launch (default on where supported).
-    void set_fused_trunk(bool enabled);
-    bool fused_trunk_active() const { return fused_trunk_ && trunk_layers_ != nullptr; }
     // Decode steps of one or two rows: attention as one launch that leaves partial states, merged by the wo GEMV
     // (on by default where the shapes allow); off = the split kernel plus the merge kernel.
     void set_merged_attention(bool enabled);
     bool merged_attention_in_use() const { return !layers_.empty() && wo_merges_attention(layers_[0], 1); }
-    int fused_trunk_timeouts(unsigned *out);
-    int check_fused_trunk();
     int read_last_hidden(int seq, float *out);
     int read_logits(int seq, float *out);         // runs the head on the kept hidden state
 
@@ -137,10 +130,7 @@ class LlamaRuntime {
     ArgmaxScratch argmax_scratch_;
     float *attn_scratch_ = nullptr;
     bool matrix_prefill_ = true;
-    bool fused_trunk_ = true;
     bool merged_attention_ = true;
-    TrunkLayer *trunk_layers_ = nullptr;   // device table, set when the fused trunk kernel covers this model
-    unsigned *trunk_sync_ = nullptr;
     bool prompt_attention_ = false;   // prompt blocks run attention on the matrix cores
     float *gemm_workspace_ = nullptr;
 

@@ -182,24 +182,12 @@ def set_graph_replay(rt: LlamaRuntime, enabled: bool) -> None:
     _lib.check(rt._L.esp_llama_set_graph_replay(rt._h, int(enabled)))
 
 
-def set_fused_trunk(rt: LlamaRuntime, enabled: bool) -> None:
-    _lib.check(rt._L.esp_llama_set_fused_trunk(rt._h, int(enabled)))
-
-
 def set_merged_attention(rt: LlamaRuntime, enabled: bool) -> bool:
     """Returns whether the one-launch attention merged by the wo GEMV is in use after the call."""
     r = rt._L.esp_llama_set_merged_attention(rt._h, int(enabled))
     if r < 0:
         _lib.check(r)
     return bool(r)
-
-
-def fused_trunk_status(rt: LlamaRuntime) -> tuple[bool, int]:
-    """(fused trunk kernel in use, barrier time-outs so far)."""
-    import ctypes as C
-    active, timeouts = C.c_int(0), C.c_uint(0)
-    _lib.check(rt._L.esp_llama_fused_trunk_status(rt._h, C.byref(active), C.byref(timeouts)))
-    return bool(active.value), int(timeouts.value)
 
 
 def set_matrix_prefill(rt: LlamaRuntime, enabled: bool) -> None:

@@ -214,17 +214,6 @@ int esp_llama_set_graph_replay(ESPLlamaRuntime *runtime, int enabled);
  * reference's token-by-token walk (RealModelInferenceEngine.swift:6365-6375).  enabled = 0 restores the
  * per-token path, whose arithmetic keeps the dequantised weights in fp32.  Default: enabled. */
 int esp_llama_set_matrix_prefill(ESPLlamaRuntime *runtime, int enabled);
-/* The layer loop of forwardToken (RealModelInferenceEngine.swift:6221-6347) as ONE persistent launch per
- * batch-1 step, with grid-wide barriers between the five phases of a layer instead of kernel boundaries.
- * Available for all-Q4_K models of the Llama-3-8B shape (d 4096, FFN 14336, head_dim 128, 4 query heads
- * per KV head).  Bit-identical to the separate kernels but measured slower on MI355X (2.34 ms against
- * 1.78 ms per token), so it is OFF unless enabled here or with ESPRESSO_HIP_FUSED_TRUNK=1.  Every spin in
- * it is bounded; a barrier that times out makes the next synchronising call fail with
- * ESP_ERR_LAUNCH_FAILED and switches the runtime back to the separate kernels.
- * status: active = 1 when the fused path is in use. */
-int esp_llama_set_fused_trunk(ESPLlamaRuntime *runtime, int enabled);
-int esp_llama_fused_trunk_status(ESPLlamaRuntime *runtime, int *active, unsigned *barrier_timeouts);
-
 /* Decode steps of one or two rows run attention (decodeContextFromCaches, :6774-6823) as one launch that leaves
  * per-head partial softmax states, and the wo GEMV merges them while it stages its input, where the shapes allow
  * (head size 128, Q4_K wo of 2048 or 4096 columns).  enabled = 0 restores the split kernel plus the merge kernel
