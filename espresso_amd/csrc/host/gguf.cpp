@@ -161,16 +161,40 @@ bool GGUFLoader::getString(const std::string &key, std::string *out) const {
     return true;
 }
 
+// Element count of a tensor, or 0 when the dimensions are empty, contain a zero or overflow 2^40 elements (a
+// malformed or hostile file): every size derived from it stays far inside 64 bits.
+static uint64_t checked_elements(const GGUFTensorInfo &t) {
+    constexpr uint64_t kMaxElements = (uint64_t)1 << 40;
+    if (t.dims.empty()) return 0;
+    uint64_t n = 1;
+    for (uint64_t d : t.dims) {
+        if (d == 0 || d > kMaxElements || n > kMaxElements / d) return 0;
+        n *= d;
+    }
+    return n;
+}
+
 bool GGUFLoader::readTensor(const GGUFTensorInfo &t, std::vector<uint8_t> *out, std::string *error) const {
-    const size_t bytes = tensorBytes(t.type, t.elements());
+    const uint64_t elements = checked_elements(t);
+    if (!elements) { if (error) *error = "tensor " + t.name + " has an empty or oversized shape"; return false; }
+    const size_t bytes = tensorBytes(t.type, elements);
     if (!bytes) { if (error) *error = "tensor " + t.name + " has unsupported ggml type " + std::to_string(t.type); return false; }
-    if (data_start_ + t.offset + bytes > file_size_) { if (error) *error = "tensor " + t.name + " runs past the end of the file"; return false; }
+    // offset <= file_size - data_start - bytes, written so that nothing can wrap
+    if (data_start_ > file_size_ || bytes > file_size_ - data_start_ || t.offset > file_size_ - data_start_ - bytes) {
+        if (error) *error = "tensor " + t.name + " runs past the end of the file";
+        return false;
+    }
     FILE *f = std::fopen(path_.c_str(), "rb");
     if (!f) { if (error) *error = "cannot reopen " + path_; return false; }
-    out->resize(bytes);
-    bool ok = std::fseek(f, (long)(data_start_ + t.offset), SEEK_SET) == 0 && std::fread(out->data(), 1, bytes, f) == bytes;
+    bool ok = false;
+    try {
+        out->resize(bytes);
+        ok = fseeko(f, (off_t)(data_start_ + t.offset), SEEK_SET) == 0 && std::fread(out->data(), 1, bytes, f) == bytes;
+        if (!ok && error) *error = "short read of tensor " + t.name;
+    } catch (const std::bad_alloc &) {
+        if (error) *error = "tensor " + t.name + " does not fit in memory";
+    }
     std::fclose(f);
-    if (!ok && error) *error = "short read of tensor " + t.name;
     return ok;
 }
 
@@ -215,8 +239,13 @@ namespace {
 
 // fp32 values of a tensor stored as F32 / F16 / BF16 / a supported quantised type (decoded on the GPU)
 int tensor_to_float(const GGUFTensorInfo &t, const std::vector<uint8_t> &raw, std::vector<float> *out) {
-    const size_t n = (size_t)t.elements();
-    out->resize(n);
+    const size_t n = (size_t)checked_elements(t);
+    if (!n || raw.size() != GGUFLoader::tensorBytes(t.type, n)) return fail(ESP_ERR_INVALID_ARGUMENT, "tensor %s: byte count does not match its shape", t.name.c_str());
+    try {
+        out->resize(n);
+    } catch (const std::bad_alloc &) {
+        return fail(ESP_ERR_OUT_OF_MEMORY, "tensor %s does not fit in memory", t.name.c_str());
+    }
     switch (t.type) {
     case GGML_F32: std::memcpy(out->data(), raw.data(), n * 4); return ESP_OK;
     case GGML_BF16:
@@ -270,16 +299,28 @@ int GGUFModelLoader::prepare(const std::string &ggufPath, const std::string &out
     if (!makeDirectories(joinPath(outputDir, "embeddings"))) return fail(ESP_ERR_IO, "cannot create %s", outputDir.c_str());
 
     int count = 0;
+    const int64_t d_ = c.dModel, ad_ = (int64_t)c.nHead * c.headDim, kd_ = (int64_t)c.nKVHead * c.headDim, hd_ = c.hiddenDim;
     // name in the GGUF file -> path under the weight directory, matrix?, q/k head count for the re-order
-    auto convert = [&](const std::string &gguf_name, const std::string &rel, bool matrix, int qk_heads, bool optional) -> int {
+    // `rows` x `cols` is the shape the configuration implies (cols = ne[0], the innermost dimension; vectors: rows = 1)
+    auto convert = [&](const std::string &gguf_name, const std::string &rel, bool matrix, int qk_heads, bool optional, int64_t rows,
+                       int64_t cols) -> int {
         const GGUFTensorInfo *t = g.find(gguf_name);
         if (!t) return optional ? ESP_OK : fail(ESP_ERR_INVALID_ARGUMENT, "GGUF file lacks tensor %s", gguf_name.c_str());
+        const bool shape_ok = matrix ? t->dims.size() == 2 && t->dims[0] == (uint64_t)cols && t->dims[1] == (uint64_t)rows
+                                     : !t->dims.empty() && t->dims[0] == (uint64_t)cols && checked_elements(*t) == (uint64_t)cols;
+        if (!shape_ok || rows <= 0 || cols <= 0)
+            return fail(ESP_ERR_INVALID_ARGUMENT, "tensor %s does not have the shape [%lld, %lld] the model configuration implies", gguf_name.c_str(),
+                        (long long)rows, (long long)cols);
         std::vector<uint8_t> raw;
         std::string e;
         if (!g.readTensor(*t, &raw, &e)) return fail(ESP_ERR_UNSUPPORTED, "%s", e.c_str());
         const std::string path = joinPath(outputDir, rel);
-        if (matrix && t->dims.size() == 2 && qk_heads > 0 && undo_interleave)
-            undo_qk_interleave(raw, qk_heads, c.headDim, raw.size() / (size_t)t->dims[1]);
+        if (matrix && qk_heads > 0 && undo_interleave) {
+            // rows == qk_heads * headDim was checked against the file above; whole blocks per row
+            if (rows != (int64_t)qk_heads * c.headDim || raw.size() % (size_t)rows != 0)
+                return fail(ESP_ERR_INVALID_ARGUMENT, "tensor %s: %lld rows are not %d heads of %d", gguf_name.c_str(), (long long)rows, qk_heads, c.headDim);
+            undo_qk_interleave(raw, qk_heads, c.headDim, raw.size() / (size_t)rows);
+        }
         const bool quantised = t->type == GGML_Q4_0 || t->type == GGML_Q8_0 || t->type == GGML_Q4_K;
         const bool is_embedding = rel == "embeddings/token.bin";
         if (matrix && quantised && !is_embedding) {
@@ -305,10 +346,10 @@ int GGUFModelLoader::prepare(const std::string &ggufPath, const std::string &out
         return ESP_OK;
     };
 
-    if ((rc = convert("token_embd.weight", "embeddings/token.bin", true, 0, false)) != ESP_OK) return rc;
-    if ((rc = convert("output_norm.weight", "rms_final.bin", false, 0, false)) != ESP_OK) return rc;
+    if ((rc = convert("token_embd.weight", "embeddings/token.bin", true, 0, false, c.vocab, d_)) != ESP_OK) return rc;
+    if ((rc = convert("output_norm.weight", "rms_final.bin", false, 0, false, 1, d_)) != ESP_OK) return rc;
     if (g.find("output.weight")) {
-        if ((rc = convert("output.weight", "lm_head.bin", true, 0, false)) != ESP_OK) return rc;
+        if ((rc = convert("output.weight", "lm_head.bin", true, 0, false, c.vocab, d_)) != ESP_OK) return rc;
     } else {
         // tied head: lm_head is the token embedding (materializeTiedLMHeadIfNeeded, :224-263); quantised
         // embeddings keep their packed bytes as the head's packed sidecar
@@ -329,17 +370,17 @@ int GGUFModelLoader::prepare(const std::string &ggufPath, const std::string &out
     for (int l = 0; l < c.nLayer; l++) {
         const std::string b = "blk." + std::to_string(l) + ".", d = "layers/" + std::to_string(l) + "/";
         if (!makeDirectories(joinPath(outputDir, "layers/" + std::to_string(l)))) return fail(ESP_ERR_IO, "cannot create layer directory");
-        if ((rc = convert(b + "attn_norm.weight", d + "rms_att.bin", false, 0, false)) != ESP_OK) return rc;
-        if ((rc = convert(b + "attn_q.weight", d + "wq.bin", true, c.nHead, false)) != ESP_OK) return rc;
-        if ((rc = convert(b + "attn_k.weight", d + "wk.bin", true, c.nKVHead, false)) != ESP_OK) return rc;
-        if ((rc = convert(b + "attn_v.weight", d + "wv.bin", true, 0, false)) != ESP_OK) return rc;
-        if ((rc = convert(b + "attn_output.weight", d + "wo.bin", true, 0, false)) != ESP_OK) return rc;
-        if ((rc = convert(b + "ffn_norm.weight", d + "rms_ffn.bin", false, 0, false)) != ESP_OK) return rc;
-        if ((rc = convert(b + "ffn_gate.weight", d + "w1.bin", true, 0, false)) != ESP_OK) return rc;
-        if ((rc = convert(b + "ffn_down.weight", d + "w2.bin", true, 0, false)) != ESP_OK) return rc;
-        if ((rc = convert(b + "ffn_up.weight", d + "w3.bin", true, 0, false)) != ESP_OK) return rc;
-        if ((rc = convert(b + "attn_q_norm.weight", d + "q_norm.bin", false, 0, true)) != ESP_OK) return rc;
-        if ((rc = convert(b + "attn_k_norm.weight", d + "k_norm.bin", false, 0, true)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_norm.weight", d + "rms_att.bin", false, 0, false, 1, d_)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_q.weight", d + "wq.bin", true, c.nHead, false, ad_, d_)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_k.weight", d + "wk.bin", true, c.nKVHead, false, kd_, d_)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_v.weight", d + "wv.bin", true, 0, false, kd_, d_)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_output.weight", d + "wo.bin", true, 0, false, d_, ad_)) != ESP_OK) return rc;
+        if ((rc = convert(b + "ffn_norm.weight", d + "rms_ffn.bin", false, 0, false, 1, d_)) != ESP_OK) return rc;
+        if ((rc = convert(b + "ffn_gate.weight", d + "w1.bin", true, 0, false, hd_, d_)) != ESP_OK) return rc;
+        if ((rc = convert(b + "ffn_down.weight", d + "w2.bin", true, 0, false, d_, hd_)) != ESP_OK) return rc;
+        if ((rc = convert(b + "ffn_up.weight", d + "w3.bin", true, 0, false, hd_, d_)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_q_norm.weight", d + "q_norm.bin", false, 0, true, 1, c.headDim)) != ESP_OK) return rc;
+        if ((rc = convert(b + "attn_k_norm.weight", d + "k_norm.bin", false, 0, true, 1, c.headDim)) != ESP_OK) return rc;
     }
     if (count == 0) return fail(ESP_ERR_INVALID_ARGUMENT, "no tensors converted");
     const std::string meta = metadataJSON(c);
@@ -353,7 +394,7 @@ int GGUFModelLoader::prepare(const std::string &ggufPath, const std::string &out
 // ---- prepared-artifact cache ------------------------------------------------------------------------
 namespace {
 
-constexpr int kPreparedArtifactCacheVersion = 1;
+constexpr int kPreparedArtifactCacheVersion = 2;   // 2: the converter options below are part of the key
 const char *const kManifestFileName = "prepare-manifest.json";
 const char *const kCacheMarkerFileName = ".espresso-gguf-cache-artifact";
 // converterCacheEnvironmentKeys (:29-36)
@@ -432,7 +473,11 @@ std::string cachePayloadJSON(const std::string &path, uint64_t size, double mtim
     }
     char num[64];
     std::snprintf(num, sizeof(num), "%.9f", mtime);
-    j += "},\"fileSize\":" + std::to_string(size) + ",\"ggufPath\":" + jsonString(path) + ",\"modificationTime\":" + num + ",\"selectedSidecars\":[";
+    // the options of this build's converter that change what is written (they are not in the reference's payload)
+    j += std::string("},\"emitDequantizedBlobs\":") + (o.emitDequantizedBlobs ? "true" : "false") + ",\"emitFloat32Sidecars\":" +
+         (o.emitFloat32Sidecars ? "true" : "false");
+    j += ",\"fileSize\":" + std::to_string(size) + ",\"ggufPath\":" + jsonString(path) + ",\"modificationTime\":" + num + ",\"qkLayout\":" + std::to_string(o.qkLayout) +
+         ",\"selectedSidecars\":[";
     first = true;
     if (o.exactFloat32SidecarMode == ExactFloat32SidecarMode::selected)
         for (const std::string &n : o.selectedSidecars) {   // std::set: sorted
@@ -541,7 +586,11 @@ int GGUFModelLoader::prepare(const std::string &ggufPath, const PrepareOptions &
         outputDir = joinPath(std::filesystem::temp_directory_path().string(), "espresso_gguf_" + randomSuffix());
     }
     PreparedModel pm;
-    const int rc = prepare(path, outputDir, options, &pm);
+    // The one converter switch of the reference's environment that this converter has a counterpart for: it forces the
+    // Q/K row re-order whatever the architecture says (the value is part of the cache key through converterEnvironment).
+    PrepareOptions effective = options;
+    if (effective.qkLayout < 0 && isEnabled(lookup(environment, "ESPRESSO_FORCE_QK_INVERSE_INTERLEAVE"))) effective.qkLayout = 1;
+    const int rc = prepare(path, outputDir, effective, &pm);
     if (rc != ESP_OK) {
         std::filesystem::remove_all(outputDir, ec);   // shouldCleanupOnFailure (:399-403)
         return rc;

@@ -28,25 +28,26 @@ def _value(v) -> bytes:
 
 
 def write_gguf(path, metadata: dict, tensors: list, alignment: int = 32, version: int = 3):
-    """tensors: [(name, ggml_type, (rows, cols) or (n,), raw_bytes)]"""
+    """tensors: [(name, ggml_type, (rows, cols) or (n,), raw_bytes[, offset written instead of the real one])]"""
     out = bytearray(struct.pack("<IIQQ", 0x46554747, version, len(tensors), len(metadata)))
     for k, v in metadata.items():
         out += _s(k) + _value(v)
     offset = 0
-    for name, gtype, shape, raw in tensors:
+    for name, gtype, shape, raw, *forced_offset in tensors:
         dims = list(reversed(shape))                      # ne[0] is the innermost dimension
         out += _s(name) + struct.pack("<I", len(dims)) + b"".join(struct.pack("<Q", d) for d in dims)
-        out += struct.pack("<IQ", gtype, offset)
+        out += struct.pack("<IQ", gtype, forced_offset[0] if forced_offset else offset)
         offset += (len(raw) + alignment - 1) // alignment * alignment
     out += b"\0" * ((-len(out)) % alignment)
-    for _, _, _, raw in tensors:
+    for _, _, _, raw, *_ in tensors:
         out += bytes(raw) + b"\0" * ((-len(raw)) % alignment)
     open(path, "wb").write(bytes(out))
 
 
-def gguf_model(path, kw, w, arch, matrix_fmt, tied=False, interleave_qk=True):
+def gguf_model(path, kw, w, arch, matrix_fmt, tied=False, interleave_qk=True, mutate=None):
     """Writes a llama-family GGUF file the way llama.cpp's converter lays it out; returns the fp32 values
-    (in the half-split row order the decoder uses) that the packed tensors decode to."""
+    (in the half-split row order the decoder uses) that the packed tensors decode to.  `mutate` may rewrite the tensor
+    list (malformed files for the loader's error paths)."""
     hd, half = kw["head_dim"], kw["head_dim"] // 2
 
     def gguf_rows(a, heads):   # stored row (h, j, s) <- half-split row (h, s, j)
@@ -94,5 +95,5 @@ def gguf_model(path, kw, w, arch, matrix_fmt, tied=False, interleave_qk=True):
                 tensors.append((f"blk.{l}.{g}.weight", 0, a.shape, a.astype("<f4").tobytes()))
                 S[k] = a
         seen["layers"].append(S)
-    write_gguf(path, meta, tensors)
+    write_gguf(path, meta, mutate(tensors) if mutate else tensors)
     return seen

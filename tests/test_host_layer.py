@@ -285,7 +285,7 @@ def test_prepare_through_the_artifact_cache(tmp_path):
     assert wdir == str(root / key) and count == 3 + 9 and cfg.d_model == 64
     manifest = json.load(open(os.path.join(wdir, "prepare-manifest.json")))
     assert manifest["tensorCount"] == count and manifest["ggufPath"] == path and manifest["sidecarMode"] == "automatic"
-    assert manifest["fileSize"] == os.path.getsize(path) and manifest["version"] == 1
+    assert manifest["fileSize"] == os.path.getsize(path) and manifest["version"] == 2
     assert os.path.exists(os.path.join(wdir, ".espresso-gguf-cache-artifact"))
     # a second prepare returns the cached directory untouched (a file planted in it survives), and cleanup keeps it
     open(os.path.join(wdir, "planted"), "w").close()
@@ -318,6 +318,47 @@ def test_prepare_through_the_artifact_cache(tmp_path):
     with pytest.raises(lib.EspressoError):
         eng.gguf_prepare_cached(str(bad), opts)
     assert not os.path.exists(str(root / eng.gguf_artifact_cache_key(str(bad), opts)))
+
+
+def test_cache_key_tracks_the_converter_options_and_malformed_tensors_are_refused(tmp_path):
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import model_util as mu
+    from gguf_writer import gguf_model
+    kw = dict(n_layer=1, n_head=2, n_kv_head=1, d_model=64, head_dim=32, hidden_dim=256, vocab=256, max_seq=16)
+    w = mu.random_weights(orc.LlamaConfig(**kw), 5, std=0.08)
+    path = str(tmp_path / "m.gguf")
+    gguf_model(path, kw, w, "llama", orc.FMT_Q8_0)
+    opts = eng.PrepareOptions(cache_root=str(tmp_path / "cache"))
+    # the same file prepared with the Q/K rows re-ordered and as stored: two cache entries, different wq bytes
+    _, undone, _ = eng.gguf_prepare_cached(path, opts, qk_layout=1)
+    _, stored, _ = eng.gguf_prepare_cached(path, opts, qk_layout=0)
+    assert undone != stored
+    wq = [open(os.path.join(d, "layers/0/wq.q8_0.bin"), "rb").read() for d in (undone, stored)]
+    assert len(wq[0]) == len(wq[1]) and wq[0] != wq[1]
+    assert open(os.path.join(undone, "layers/0/wv.q8_0.bin"), "rb").read() == open(os.path.join(stored, "layers/0/wv.q8_0.bin"), "rb").read()
+    # the converter switch of the environment forces the re-order (same bytes as qk_layout=1, an entry of its own)
+    _, forced, _ = eng.gguf_prepare_cached(path, opts, {"ESPRESSO_FORCE_QK_INVERSE_INTERLEAVE": "1"}, qk_layout=-1)
+    assert forced not in (undone, stored)
+    assert open(os.path.join(forced, "layers/0/wq.q8_0.bin"), "rb").read() == wq[0]
+    # so does the sidecar switch (the dequantised-blob switch needs the GPU and is covered by the engine tests)
+    _, bare, _ = eng.gguf_prepare_cached(path, opts, emit_float32_sidecars=False, qk_layout=1)
+    assert bare != undone and not os.path.exists(os.path.join(bare, "rms_final.float32.bin"))
+
+    # malformed files: an attn_q with the wrong number of rows, a zero dimension, an offset that wraps 64 bits
+    def reshape_q(shape):
+        def go(tensors):
+            return [(n, t, shape if n == "blk.0.attn_q.weight" else s, raw) for n, t, s, raw in tensors]
+        return go
+    for i, shape in enumerate([(32, 64), (64, 32), (0, 64), (2 ** 62, 2 ** 62)]):
+        bad = str(tmp_path / f"bad{i}.gguf")
+        gguf_model(bad, kw, w, "llama", orc.FMT_Q8_0, mutate=reshape_q(shape))
+        with pytest.raises(lib.EspressoError, match="shape"):
+            eng.gguf_prepare(bad, str(tmp_path / f"out{i}"))
+    far = str(tmp_path / "far.gguf")
+    gguf_model(far, kw, w, "llama", orc.FMT_Q8_0, mutate=lambda ts: [t + (2 ** 64 - 64,) if t[0] == "blk.0.ffn_up.weight" else t for t in ts])
+    with pytest.raises(lib.EspressoError, match="past the end"):
+        eng.gguf_prepare(far, str(tmp_path / "out_far"))
 
 
 # ---- ModelRegistry (Tests/ModelSupportTests/ModelConfigTests.swift:5-52) and ClassifierStrategy.select
