@@ -52,6 +52,7 @@ enum Epilogue : int {
     EPI_ADD_RESIDUAL = 1,  // y[b][r] = residual[b][r] + acc
     EPI_SWIGLU_F16 = 2,    // rows interleaved (gate_i, up_i): out_f16[b][i] = fp16(silu(gate_i) * up_i)
     EPI_QKV_ROPE = 3,      // fused q|k|v rows: RoPE, q -> q_out, k/v -> KV caches
+    EPI_ARGMAX = 4,        // output head: no logits are stored; every workgroup leaves (largest row sum, lowest row index holding it)
 };
 
 // Destination of the fused q|k|v GEMV (EPI_QKV_ROPE).  The matrix rows are q and k as RoPE pairs
@@ -82,6 +83,12 @@ struct GemvParams {
     const float *residual = nullptr;
     uint16_t *out_f16 = nullptr;  // EPI_SWIGLU_F16: [batch][rows/2]
     QkvEpilogue qkv;              // EPI_QKV_ROPE
+    // EPI_ARGMAX: per-workgroup partial results, [batch][*argmax_blocks] (value, index) pairs; `argmax_capacity` slots per
+    // batch row are available and the launch fails if the kernel's grid is larger.  *argmax_blocks receives the grid size.
+    float *argmax_value = nullptr;
+    int *argmax_index = nullptr;
+    int argmax_capacity = 0;
+    int *argmax_blocks = nullptr;
     int batch = 1;
     int epilogue = EPI_STORE_F32;
     // optional (batch <= 2): events that take the kernel's own start and end times
@@ -112,6 +119,9 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
 #define ESP_ATTENTION_HEAD_SPLITS 4
 #endif
 constexpr int kAttentionHeadSplits = ESP_ATTENTION_HEAD_SPLITS;
+// True when launch_gemv has the EPI_ARGMAX epilogue for this matrix (every format; Q4_K rows of 8192 or more columns, which
+// several wavefronts share, keep the separate argmax launches).
+bool gemv_supports_argmax(const DeviceMatrix &w);
 // True when launch_gemv can take its input as attention partial states (batch <= 2, head size 64 or 128).
 bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch, int head_dim);
 // kernels/gemm.hip

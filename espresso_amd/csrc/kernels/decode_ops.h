@@ -89,6 +89,12 @@ hipError_t launch_greedy_feed(const int *next_token, int seq, int *visible, int 
 hipError_t launch_greedy_step_tail(const float *logits, int vocab, int *out_token, const ArgmaxScratch &scratch, int seq, int *visible,
                                    int *tokens, int *pos, int *seqs, int *log, int *log_count, int log_capacity, const void *table,
                                    bool table_is_f16, int d, float *hidden, hipStream_t s);
+// The same two steps for a head GEMV that left one (value, index) pair per workgroup instead of logits (EPI_ARGMAX):
+// `blocks` pairs per row in scratch, rows `blocks` apart.
+hipError_t launch_argmax_final(const ArgmaxScratch &scratch, int blocks, int rows, int *out_token, hipStream_t s);
+hipError_t launch_greedy_tail(const ArgmaxScratch &scratch, int blocks, int *out_token, int seq, int *visible, int *tokens, int *pos, int *seqs,
+                              int *log, int *log_count, int log_capacity, const void *table, bool table_is_f16, int d, float *hidden,
+                              hipStream_t s);
 hipError_t launch_set_ints(int *dst0, int v0, int *dst1, int v1, hipStream_t s);
 hipError_t launch_copy_rows(const float *src, float *dst, int rows, int d, hipStream_t s);
 

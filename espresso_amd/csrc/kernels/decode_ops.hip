@@ -1049,6 +1049,23 @@ hipError_t launch_argmax(const float *logits, int rows, int vocab, int *out_toke
     return hipGetLastError();
 }
 
+hipError_t launch_argmax_final(const ArgmaxScratch &scratch, int blocks, int rows, int *out_token, hipStream_t s) {
+    if (!scratch.part_value || !scratch.part_index || blocks < 1 || rows < 1) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(kBlock), 0, s, scratch.part_value, scratch.part_index, blocks, out_token,
+                       static_cast<float *>(nullptr));
+    return hipGetLastError();
+}
+
+hipError_t launch_greedy_tail(const ArgmaxScratch &scratch, int blocks, int *out_token, int seq, int *visible, int *tokens, int *pos, int *seqs,
+                              int *log, int *log_count, int log_capacity, const void *table, bool table_is_f16, int d, float *hidden,
+                              hipStream_t s) {
+    if (!scratch.part_value || !scratch.part_index || blocks < 1) return hipErrorInvalidValue;
+    GreedyTailArgs a{scratch.part_value, scratch.part_index, blocks, out_token, seq, visible, tokens, pos, seqs, log, log_count, log_capacity,
+                     table, table_is_f16 ? 1 : 0, d, hidden};
+    hipLaunchKernelGGL(greedy_tail_kernel, dim3(1), dim3(kBlock), 0, s, a);
+    return hipGetLastError();
+}
+
 hipError_t launch_greedy_step_tail(const float *logits, int vocab, int *out_token, const ArgmaxScratch &scratch, int seq, int *visible,
                                    int *tokens, int *pos, int *seqs, int *log, int *log_count, int log_capacity, const void *table,
                                    bool table_is_f16, int d, float *hidden, hipStream_t s) {

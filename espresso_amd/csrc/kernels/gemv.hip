@@ -99,7 +99,36 @@ struct KernelArgs {
     // while staging (x and norm_x unused): [batch][cols / head_dim heads][kMergeSplits][head_dim values, m, l, 2 pad]
     const float *merge_partials;
     int merge_head_dim;
+    // EPI_ARGMAX: one (value, index) pair per workgroup and batch row, [batch][gridDim.x]
+    float *part_value;
+    int *part_index;
 };
+
+// First-max rule of the reference's output head (RealModelInferenceEngine.swift:8219-8275, neon_convert.c:36-101): a larger
+// value wins, equal values keep the lower index, NaN never wins.
+__device__ __forceinline__ void argmax_take(float &best, int &best_i, float v, int i) {
+    if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+}
+// The workgroup's result from one candidate per wavefront and batch row (lane 0 of each wavefront holds it).
+// Every thread of the workgroup must call this.  `bv` / `bi`: kWaves * B entries of LDS nobody else uses.
+template <int B>
+__device__ __forceinline__ void argmax_workgroup(const KernelArgs &a, const float (&best)[B], const int (&best_i)[B], float *bv, int *bi) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+#pragma unroll
+        for (int b = 0; b < B; b++) { bv[b * kWaves + wave] = best[b]; bi[b * kWaves + wave] = best_i[b]; }
+    }
+    __syncthreads();
+    if (threadIdx.x < B) {
+        const int b = threadIdx.x;
+        float v = bv[b * kWaves];
+        int i = bi[b * kWaves];
+#pragma unroll
+        for (int w = 1; w < kWaves; w++) argmax_take(v, i, bv[b * kWaves + w], bi[b * kWaves + w]);
+        a.part_value[(size_t)b * gridDim.x + blockIdx.x] = v;
+        a.part_index[(size_t)b * gridDim.x + blockIdx.x] = i;
+    }
+}
 
 // ---- attention context merged from per-split partial states -------------------------------------------
 // The arithmetic of attention_merge_kernel: M = max m, f = exp(m - M) (0 for an empty split), L = fma(l, f, L),
@@ -329,7 +358,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const uint8_t *qs, const
         __syncthreads();
     }
 
-    if (row0 >= a.rows) return;
+    if (row0 >= a.rows && a.epilogue != EPI_ARGMAX) return;   // (the arg-max epilogue ends with a workgroup barrier)
 
     float acc[R][B];
 #pragma unroll
@@ -437,6 +466,21 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const uint8_t *qs, const
         for (int b = 0; b < B; b++) acc[r][b] = wave_sum(acc[r][b]);
 
     static_assert(R == 2, "the epilogues work on row pairs");
+    if (a.epilogue == EPI_ARGMAX) {
+        __shared__ float bv[B * kWaves];
+        __shared__ int bi[B * kWaves];
+        float best[B];
+        int best_i[B];
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+            best[b] = -INFINITY;
+            best_i[b] = 0x7FFFFFFF;
+            if (row0 < a.rows) argmax_take(best[b], best_i[b], acc[0][b], row0);
+            if (row0 + 1 < a.rows) argmax_take(best[b], best_i[b], acc[1][b], row0 + 1);
+        }
+        argmax_workgroup<B>(a, best, best_i, bv, bi);
+        return;
+    }
     if (lane == 0) {
         float va[B], vb[B];
 #pragma unroll
@@ -620,6 +664,11 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
         }
     };
 
+    float best[B];     // EPI_ARGMAX (TEAM == 1): the wavefront's running first maximum, valid in lane 0
+    int best_i[B];
+#pragma unroll
+    for (int b = 0; b < B; b++) { best[b] = -INFINITY; best_i[b] = 0x7FFFFFFF; }
+
     auto process = [&](const Q4KItem (&buf)[PASSES], int pair, int round) {
         float acc_a[B], acc_b[B];
 #pragma unroll
@@ -647,7 +696,15 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
             }
         }
         if constexpr (TEAM == 1) {
-            if (pair < npairs && lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
+            if (a.epilogue == EPI_ARGMAX) {
+                if (pair < npairs) {
+#pragma unroll
+                    for (int b = 0; b < B; b++) {
+                        argmax_take(best[b], best_i[b], acc_a[b], 2 * pair);
+                        if (2 * pair + 1 < a.rows) argmax_take(best[b], best_i[b], acc_b[b], 2 * pair + 1);
+                    }
+                }
+            } else if (pair < npairs && lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
         } else {
             float *slot = red + (size_t)(deferred ? round : (round & 1)) * kWaves * 2 * B;
             if (lane == 0) {
@@ -682,6 +739,9 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
             process(buf1, pair, j + 1);
             pair = next;
         }
+    }
+    if constexpr (TEAM == 1) {
+        if (a.epilogue == EPI_ARGMAX) argmax_workgroup<B>(a, best, best_i, red, reinterpret_cast<int *>(red + B * kWaves));
     }
     if constexpr (TEAM > 1) {
         if (deferred) {
@@ -756,14 +816,33 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_generic_kernel(const uint8_
         acc_a[b] = wave_sum(acc_a[b]);
         acc_b[b] = wave_sum(acc_b[b]);
     }
+    if (a.epilogue == EPI_ARGMAX) {
+        __shared__ float bv[B * kWaves];
+        __shared__ int bi[B * kWaves];
+        float best[B];
+        int best_i[B];
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+            best[b] = -INFINITY;
+            best_i[b] = 0x7FFFFFFF;
+            if (2 * pair < a.rows) argmax_take(best[b], best_i[b], acc_a[b], 2 * pair);
+            if (2 * pair + 1 < a.rows) argmax_take(best[b], best_i[b], acc_b[b], 2 * pair + 1);
+        }
+        argmax_workgroup<B>(a, best, best_i, bv, bi);
+        return;
+    }
     if (lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
 }
 
 // Launch through the extension entry point when the caller gave the launch a pair of events of its own: they
 // take the kernel's own start and end times (what a kernel trace reports), without the gaps between launches.
 static thread_local hipEvent_t tl_start_event = nullptr, tl_stop_event = nullptr;
+static thread_local int tl_argmax_capacity = 0;   // EPI_ARGMAX: slots per batch row the caller provided
+static thread_local unsigned tl_last_grid = 0;    // workgroups of the most recent launch
 template <typename K, typename... Args>
 inline void launch_kernel(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args... args) {
+    tl_last_grid = grid.x;
+    if (tl_argmax_capacity > 0 && grid.x > (unsigned)tl_argmax_capacity) return;   // the caller reports the shortfall
     if (tl_start_event && tl_stop_event) hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, stream, tl_start_event, tl_stop_event, 0, args...);
     else hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
 }
@@ -892,6 +971,10 @@ bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch, int head_d
     return true;
 }
 
+bool gemv_supports_argmax(const DeviceMatrix &w) {
+    return !(w.format == FMT_Q4_K && (w.cols == 8192 || w.cols == 11008 || w.cols == 14336));
+}
+
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     const DeviceMatrix &w = p.w;
     if (!w.qs || (!p.x && !p.norm_x && !p.merge_partials) || (p.norm_x && !p.norm_w) || w.rows <= 0 || w.cols <= 0 || p.batch <= 0) return hipErrorInvalidValue;
@@ -899,6 +982,8 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     if ((p.epilogue == EPI_STORE_F32 || p.epilogue == EPI_ADD_RESIDUAL) && !p.y) return hipErrorInvalidValue;
     if (p.epilogue == EPI_ADD_RESIDUAL && !p.residual) return hipErrorInvalidValue;
     if (p.epilogue == EPI_SWIGLU_F16 && (!p.out_f16 || w.rows % 2 != 0)) return hipErrorInvalidValue;
+    if (p.epilogue == EPI_ARGMAX && (!p.argmax_value || !p.argmax_index || p.argmax_capacity <= 0 || p.batch > 2 || !gemv_supports_argmax(w)))
+        return hipErrorInvalidValue;
     if (p.epilogue == EPI_QKV_ROPE) {
         const QkvEpilogue &q = p.qkv;
         if (!q.rope_cos || !q.rope_sin || !q.pos || !q.seq || !q.q_out || !q.k_cache || !q.v_cache || q.head_dim % 2 != 0 ||
@@ -914,6 +999,10 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         EventScope(hipEvent_t a, hipEvent_t b) { tl_start_event = a; tl_stop_event = b; }
         ~EventScope() { tl_start_event = tl_stop_event = nullptr; }
     } scope(p.batch <= 2 ? p.start_event : nullptr, p.batch <= 2 ? p.stop_event : nullptr);
+    struct CapacityScope {
+        explicit CapacityScope(int n) { tl_argmax_capacity = n; }
+        ~CapacityScope() { tl_argmax_capacity = 0; }
+    } capacity(p.epilogue == EPI_ARGMAX ? p.argmax_capacity : 0);
     // batches beyond 2 run as successive pairs (each pair re-reads the weights)
     for (int b0 = 0; b0 < p.batch; b0 += 2) {
         const int nb = p.batch - b0 >= 2 ? 2 : 1;
@@ -926,6 +1015,8 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         a.residual = p.residual ? p.residual + (size_t)b0 * w.rows : nullptr;
         a.out_f16 = p.out_f16 ? p.out_f16 + (size_t)b0 * (w.rows / 2) : nullptr;
         a.qkv = p.qkv;
+        a.part_value = p.argmax_value;
+        a.part_index = p.argmax_index;
         if (p.epilogue == EPI_QKV_ROPE) {
             a.qkv.pos += b0;
             a.qkv.seq += b0;
@@ -945,6 +1036,10 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         default: e = hipErrorInvalidValue;
         }
         if (e != hipSuccess) return e;
+        if (p.epilogue == EPI_ARGMAX) {
+            if (p.argmax_blocks) *p.argmax_blocks = (int)tl_last_grid;
+            if (tl_last_grid > (unsigned)p.argmax_capacity) return hipErrorInvalidValue;   // nothing was launched
+        }
     }
     return hipSuccess;
 }

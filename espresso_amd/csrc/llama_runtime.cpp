@@ -160,7 +160,13 @@ int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us
             g.w = L->w13; g.norm_x = hidden_; g.norm_w = L->rms_ffn; g.norm_eps = c_.norm_eps; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
             break;
         case K_DOWN: g.w = L->w2; g.x = act_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL; break;
-        default: g.w = lm_head_; g.norm_x = hidden_; g.norm_w = final_norm_; g.norm_eps = c_.norm_eps; g.y = logits_; g.epilogue = EPI_STORE_F32; break;
+        default:
+            g.w = lm_head_; g.norm_x = hidden_; g.norm_w = final_norm_; g.norm_eps = c_.norm_eps; g.y = logits_; g.epilogue = EPI_STORE_F32;
+            if (head_fuses_argmax()) {   // what a greedy step launches
+                g.y = nullptr; g.epilogue = EPI_ARGMAX;
+                g.argmax_value = argmax_scratch_.part_value; g.argmax_index = argmax_scratch_.part_index; g.argmax_capacity = head_partial_capacity_;
+            }
+            break;
         }
         return launch_gemv(g, s);
     };
@@ -209,7 +215,7 @@ size_t LlamaRuntime::kernel_bytes(int kernel_class) const {
     case K_WO: return io(L.wo);
     case K_GATE_UP: return io(L.w13);
     case K_DOWN: return io(L.w2);
-    case K_HEAD: return io(lm_head_);
+    case K_HEAD: return io(lm_head_) - (head_fuses_argmax() ? (size_t)lm_head_.rows * 4 : 0);   // the fused head stores no logits
     default: return 0;
     }
 }
@@ -391,8 +397,11 @@ int LlamaRuntime::finalize() {
     if ((rc = device_alloc(&d_log_, (size_t)c_.max_seq)) != ESP_OK) return rc;
     if ((rc = device_alloc(&d_log_count_, 1)) != ESP_OK) return rc;
     step_graphs_.assign(c_.max_sequences, nullptr);
-    if ((rc = device_alloc(&argmax_scratch_.part_value, (size_t)kArgmaxScratchSlots)) != ESP_OK) return rc;
-    if ((rc = device_alloc(&argmax_scratch_.part_index, (size_t)kArgmaxScratchSlots)) != ESP_OK) return rc;
+    // one (value, index) pair per workgroup of the head GEMV and row: a workgroup owns eight rows, or the grid is persistent
+    head_partial_capacity_ = (c_.vocab + 7) / 8 > 4096 ? (c_.vocab + 7) / 8 : 4096;
+    const size_t argmax_slots = (size_t)2 * head_partial_capacity_ > (size_t)kArgmaxScratchSlots ? (size_t)2 * head_partial_capacity_ : (size_t)kArgmaxScratchSlots;
+    if ((rc = device_alloc(&argmax_scratch_.part_value, argmax_slots)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&argmax_scratch_.part_index, argmax_slots)) != ESP_OK) return rc;
     {
         const size_t per_row = (size_t)c_.n_kv_head * kAttentionMaxSplits * (c_.n_head / c_.n_kv_head) * (c_.head_dim + 2);
         if ((rc = device_alloc(&attn_scratch_, R * per_row)) != ESP_OK) return rc;
@@ -401,6 +410,8 @@ int LlamaRuntime::finalize() {
     {
         const char *pa = getenv("ESPRESSO_HIP_PROMPT_ATTENTION");   // "0": prompt blocks keep the single-query attention kernel
         prompt_attention_ = attention_prompt_supported(c_.n_head, c_.n_kv_head, c_.head_dim) && !(pa && pa[0] == '0');
+        const char *fh = getenv("ESPRESSO_HIP_FUSED_HEAD_ARGMAX");   // "0": the head stores logits and separate launches pick the token
+        fused_head_argmax_ = !(fh && fh[0] == '0');
     }
     finalized_ = true;
     return reset();
@@ -656,8 +667,22 @@ int LlamaRuntime::enqueue_layers_matrix(int rows, bool one_sequence_consecutive)
     return ESP_OK;
 }
 
-int LlamaRuntime::run_head(const float *hidden_rows, int count) {
+int LlamaRuntime::run_head(const float *hidden_rows, int count, bool want_logits) {
     hipStream_t s = context().stream;
+    if (count <= 2 && !want_logits && head_fuses_argmax()) {
+        // final RMSNorm in the staging, first-max arg-max in the epilogue: no logits are written (:8219-8275)
+        GemvParams g;
+        int blocks = 0;
+        g.w = lm_head_; g.norm_x = hidden_rows; g.norm_w = final_norm_; g.norm_eps = c_.norm_eps; g.batch = count; g.epilogue = EPI_ARGMAX;
+        g.argmax_value = argmax_scratch_.part_value; g.argmax_index = argmax_scratch_.part_index; g.argmax_capacity = head_partial_capacity_;
+        g.argmax_blocks = &blocks;
+        int rc;
+        if ((rc = time_begin(K_HEAD)) != ESP_OK) return rc;
+        ESP_HIP_TRY(launch_gemv(g, s));
+        if ((rc = time_end()) != ESP_OK) return rc;
+        ESP_HIP_TRY(launch_argmax_final(argmax_scratch_, blocks, count, d_out_tokens_, s));
+        return ESP_OK;
+    }
     if (count > 2 && matrix_prefill_ && lm_head_.format != FMT_F32 && lm_head_.cols % 64 == 0) {
         // batched rows: final RMSNorm, then the head as one MFMA GEMM
         ESP_HIP_TRY(launch_rmsnorm(hidden_rows, final_norm_, c_.norm_eps, count, c_.d_model, xn_, nullptr, s));
@@ -711,15 +736,28 @@ int LlamaRuntime::capture_step_graph(int seq) {
     int rc = ESP_OK;
     float *kept = last_hidden_ + (size_t)seq * c_.d_model;
     {
-        // head GEMV, argmax slices, then one launch that picks the token, feeds it and fetches its embedding; the
-        // last layer writes the new hidden state where the next step's head reads it: 3 + 5 per layer launches
+        // head GEMV with the arg-max in its epilogue, then one launch that picks the token among the workgroups' candidates,
+        // feeds it and fetches its embedding; the last layer writes the new hidden state where the next step's head reads
+        // it: 2 + 5 per layer launches (3 + 5 per layer when the head has to store its logits)
         GemvParams g;
-        g.w = lm_head_; g.norm_x = kept; g.norm_w = final_norm_; g.norm_eps = c_.norm_eps;
-        g.y = logits_; g.batch = 1; g.epilogue = EPI_STORE_F32;
-        hipError_t e = launch_gemv(g, s);
-        if (e == hipSuccess)
-            e = launch_greedy_step_tail(logits_, c_.vocab, d_out_tokens_, argmax_scratch_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_,
-                                        d_log_count_, c_.max_seq, embedding_, embedding_f16_, c_.d_model, hidden_, s);
+        g.w = lm_head_; g.norm_x = kept; g.norm_w = final_norm_; g.norm_eps = c_.norm_eps; g.batch = 1;
+        hipError_t e;
+        if (head_fuses_argmax()) {
+            int blocks = 0;
+            g.epilogue = EPI_ARGMAX;
+            g.argmax_value = argmax_scratch_.part_value; g.argmax_index = argmax_scratch_.part_index; g.argmax_capacity = head_partial_capacity_;
+            g.argmax_blocks = &blocks;
+            e = launch_gemv(g, s);
+            if (e == hipSuccess)
+                e = launch_greedy_tail(argmax_scratch_, blocks, d_out_tokens_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_, d_log_count_,
+                                       c_.max_seq, embedding_, embedding_f16_, c_.d_model, hidden_, s);
+        } else {
+            g.y = logits_; g.epilogue = EPI_STORE_F32;
+            e = launch_gemv(g, s);
+            if (e == hipSuccess)
+                e = launch_greedy_step_tail(logits_, c_.vocab, d_out_tokens_, argmax_scratch_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_,
+                                            d_log_count_, c_.max_seq, embedding_, embedding_f16_, c_.d_model, hidden_, s);
+        }
         if (e != hipSuccess) rc = fail_hip(e, "greedy step head");
         if (rc == ESP_OK) rc = enqueue_trunk(1, true, kept);
     }
@@ -783,7 +821,7 @@ int LlamaRuntime::read_last_hidden(int seq, float *out) {
 
 int LlamaRuntime::read_logits(int seq, float *out) {
     if (!finalized_ || seq < 0 || seq >= c_.max_sequences || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "read_logits");
-    int rc = run_head(last_hidden_ + (size_t)seq * c_.d_model, 1);
+    int rc = run_head(last_hidden_ + (size_t)seq * c_.d_model, 1, true);
     if (rc != ESP_OK) return rc;
     ESP_HIP_TRY(hipMemcpyAsync(out, logits_, (size_t)c_.vocab * 4, hipMemcpyDeviceToHost, context().stream));
     ESP_HIP_TRY(hipStreamSynchronize(context().stream));

@@ -96,7 +96,10 @@ class LlamaRuntime {
         void *k_cache = nullptr, *v_cache = nullptr;
     };
     int upload_vector(const HostTensor &t, size_t count, float **out, const char *what);
-    int run_head(const float *hidden_rows, int count);
+    // want_logits: the full-vocabulary logits are needed in logits_ (otherwise one or two rows take the head whose
+    // epilogue is the arg-max and store none)
+    int run_head(const float *hidden_rows, int count, bool want_logits = false);
+    bool head_fuses_argmax() const { return fused_head_argmax_ && gemv_supports_argmax(lm_head_); }
     // embedded: hidden_ already holds the rows' embeddings; final_out: where the last layer writes (default hidden_)
     int enqueue_trunk(int rows, bool embedded = false, float *final_out = nullptr);
     int prefill_block(int seq, const uint32_t *tokens, int rows, int base);
@@ -128,6 +131,8 @@ class LlamaRuntime {
     std::vector<hipGraphExec_t> step_graphs_;
     int *d_visible_ = nullptr, *d_log_ = nullptr, *d_log_count_ = nullptr;
     ArgmaxScratch argmax_scratch_;
+    int head_partial_capacity_ = 0;      // (value, index) slots per row for the head's per-workgroup candidates
+    bool fused_head_argmax_ = true;      // ESPRESSO_HIP_FUSED_HEAD_ARGMAX=0: head GEMV stores logits, separate arg-max launches
     float *attn_scratch_ = nullptr;
     bool matrix_prefill_ = true;
     bool merged_attention_ = true;

@@ -199,11 +199,47 @@ def test_config4_8b_512_token_block_then_decode_past_512(llama):
     h_walk = rt.last_hidden()
     scale = max(1.0, float(np.abs(h_walk).max()))
     diff = float(np.abs(h_walk - h_block).max())
-    print(f"8B 512-token prompt: block vs token walk last-hidden difference {diff:.3e} (scale {scale:.2f})")
-    assert diff <= 2e-2 * scale
     walk_logits = rt.logits()
     ll.set_matrix_prefill(rt, True)
     rt.reset(); rt.prefill(prompt)
-    assert np.abs(rt.logits() - walk_logits).max() <= LOGIT_TOL
+    logit_diff = float(np.abs(rt.logits() - walk_logits).max())
+    print(f"8B 512-token prompt: block vs token walk last-hidden difference {diff:.3e} (scale {scale:.2f}), logits {logit_diff:.3e}")
+    # Two GPU paths, not GPU against oracle: the block path feeds the matrix cores fp16 operands (each dequantised weight
+    # rounded to fp16 once, q and the softmax weights in fp16), the token walk keeps fp32 weights and fp32 q.  A relative
+    # 2^-11 per weight grows as a random walk over 128 projections to just under one percent of the residual stream; the
+    # oracle cannot walk 512 tokens through 32 layers of this width inside a test (the next test pins the block path
+    # against it on a shorter stack).
+    assert diff <= 1.5e-2 * scale
+    assert logit_diff <= 1e-1
     ll.set_graph_replay(rt, True)
     rt.close()
+
+
+def test_config4_8b_width_512_token_block_against_the_oracle(llama):
+    """The full 512-row block at the 8B width against the ORACLE in the reference's default arithmetic (fp32 activations),
+    on a stack the oracle can walk inside a test: 2 layers, Q4_K, fp16 KV, the 128256-row head.  Then six decode steps at
+    context 512+ (single-query attention over the block's cache, fused head)."""
+    import espresso_amd.synthetic as syn
+    from test_gpu_full_size import oracle_from_packed
+    ll = llama
+    cfg = ll.MultiModelConfig(**dict(syn.LLAMA3_8B, n_layer=2, max_seq=528))
+    g, packed = syn.build_runtime(cfg, orc.FMT_Q4_K, seed=23, kv_format=orc.FMT_F16, keep_packed=True)
+    o = oracle_from_packed(cfg, packed, orc.FMT_Q4_K, 2, True, 528, gemv_inputs_fp16=False)
+    prompt = np.random.default_rng(77).integers(0, cfg.vocab, 512).astype(np.uint32)
+    o.prefill([int(t) for t in prompt])
+    g.prefill(prompt)
+    ho, hg = o.last_hidden(), g.last_hidden()
+    scale = max(1.0, float(np.abs(ho).max()))
+    worst = float(np.abs(o.logits() - g.logits()).max())
+    print(f"8B width, 2 layers, 512-token block vs oracle (fp32 activations): hidden {np.abs(ho - hg).max():.3e} (scale {scale:.2f}), logits {worst:.3e}")
+    assert np.abs(ho - hg).max() <= 4e-3 * scale
+    assert worst <= LOGIT_TOL
+    for _ in range(6):
+        tok = o.select_greedy()
+        if o.top2_margin() > 5e-3:
+            assert g.select_greedy() == tok
+        o.advance(tok); g.advance(tok)
+        worst = max(worst, float(np.abs(o.logits() - g.logits()).max()))
+    print(f"  after six decode steps at context 512+: worst logit difference {worst:.3e}")
+    assert worst <= LOGIT_TOL
+    g.close()

@@ -63,10 +63,10 @@ def test_full_size_weight_gemv_matches_oracle(mods, name, rows, cols):
     mat.close()
 
 
-def oracle_from_packed(cfg, packed, fmt, n_layer, kv_fp16, max_seq):
+def oracle_from_packed(cfg, packed, fmt, n_layer, kv_fp16, max_seq, gemv_inputs_fp16=True):
     ocfg = orc.LlamaConfig(n_layer=n_layer, n_head=cfg.n_head, n_kv_head=cfg.n_kv_head, d_model=cfg.d_model, head_dim=cfg.head_dim,
                            hidden_dim=cfg.hidden_dim, vocab=cfg.vocab, max_seq=max_seq, norm_eps=cfg.norm_eps, rope_theta=cfg.rope_theta,
-                           gemv_inputs_fp16=True, kv_fp16=kv_fp16)
+                           gemv_inputs_fp16=gemv_inputs_fp16, kv_fp16=kv_fp16)
     shapes = {"wq": (cfg.attention_dim, cfg.d_model), "wk": (cfg.kv_dim, cfg.d_model), "wv": (cfg.kv_dim, cfg.d_model),
               "wo": (cfg.d_model, cfg.attention_dim), "w1": (cfg.hidden_dim, cfg.d_model), "w3": (cfg.hidden_dim, cfg.d_model),
               "w2": (cfg.d_model, cfg.hidden_dim)}
