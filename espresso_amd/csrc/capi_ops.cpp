@@ -10,6 +10,31 @@
 
 using namespace esp;
 
+// ---- scratch of the entry point that allocates nothing (esp_gemv_device_noalloc) ---------------------------
+// Split-K partial sums of the matrix-core kernels, [splits][batch][rows] floats, live in a file-scope device array
+// instead of a hipMalloc'ed workspace.  The array's name is a host-side stand-in, not a device address: the
+// address comes from hipGetSymbolAddress, once per device, at library set-up, and only that pointer is handed
+// to kernels.  Every GPU holds its own 16 MiB copy until the process ends.
+namespace {
+constexpr size_t kNoAllocScratchFloats = (size_t)4 << 20;
+constexpr int kNoAllocMaxBatch = 64;
+constexpr int kNoAllocMaxDevices = 16;
+static __device__ __align__(256) float scratch[kNoAllocScratchFloats];
+float *g_scratch_ptr[kNoAllocMaxDevices] = {};
+}  // namespace
+
+namespace esp {
+int noalloc_setup(int device) {
+    if (device < 0 || device >= kNoAllocMaxDevices) return fail(ESP_ERR_INVALID_ARGUMENT, "device %d outside 0..%d", device, kNoAllocMaxDevices - 1);
+    if (g_scratch_ptr[device]) return ESP_OK;
+    float *ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));   // `device` is the current device here
+    if (e != hipSuccess || !ptr) return fail_hip(e == hipSuccess ? hipErrorInvalidSymbol : e, "hipGetSymbolAddress(scratch)");
+    g_scratch_ptr[device] = ptr;
+    return ESP_OK;
+}
+}  // namespace esp
+
 extern "C" {
 
 int esp_init(void) { return ensure_init(); }
@@ -130,6 +155,34 @@ int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y
     if (d_res) (void)hipFree(d_res);
     if (d_ws) (void)hipFree(d_ws);
     return e == hipSuccess ? ESP_OK : fail_hip(e, "gemv");
+}
+
+int esp_gemv_device_noalloc(const ESPMatrix *matrix, const uint16_t *x_f16_device, int batch, float *y_device,
+                            const float *residual_device_or_null) {
+    if (!matrix || !x_f16_device || !y_device) return fail(ESP_ERR_INVALID_ARGUMENT, "gemv_device_noalloc: null pointer");
+    if (batch <= 0 || batch > kNoAllocMaxBatch)
+        return fail(ESP_ERR_OUT_OF_RANGE, "gemv_device_noalloc: batch %d outside 1..%d", batch, kNoAllocMaxBatch);
+    int rc = ensure_init();   // allocates nothing once the library is initialised
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    const DeviceMatrix &m = matrix->m;
+    float *workspace = c.device >= 0 && c.device < kNoAllocMaxDevices ? g_scratch_ptr[c.device] : nullptr;
+    if (!workspace) return fail(ESP_ERR_LAUNCH_FAILED, "gemv_device_noalloc: no scratch address for device %d", c.device);
+    if (use_gemm(m, batch) && (size_t)2 * batch * m.rows > kNoAllocScratchFloats)
+        return fail(ESP_ERR_OUT_OF_RANGE, "gemv_device_noalloc: batch %d x %d rows needs %zu floats of split-K scratch for two splits, the fixed scratch holds %zu",
+                    batch, m.rows, (size_t)2 * batch * m.rows, kNoAllocScratchFloats);
+    // Partial planes are written whole by every split before they are added: nothing has to start at zero.
+    hipError_t e;
+    if (use_gemm(m, batch)) {
+        GemmParams g;
+        g.w = m; g.x = x_f16_device; g.y = y_device; g.residual = residual_device_or_null; g.rows = batch;
+        g.workspace = workspace; g.workspace_floats = kNoAllocScratchFloats;
+        e = launch_gemm(g, c.stream);
+    } else {
+        e = run_matvec(m, x_f16_device, batch, y_device, residual_device_or_null, nullptr, c.stream);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "gemv_device_noalloc");
 }
 
 int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int rotate,

@@ -48,6 +48,10 @@ int ensure_init() {
     ESP_HIP_TRY(hipGetDeviceProperties(&g_context.props, 0));
     ESP_HIP_TRY(hipStreamCreateWithFlags(&g_context.stream, hipStreamNonBlocking));
     g_context.device = 0;
+    {
+        const int rc = noalloc_setup(0);
+        if (rc != ESP_OK) return rc;
+    }
     g_context.ready = true;
     return ESP_OK;
 }

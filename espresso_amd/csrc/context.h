@@ -43,6 +43,10 @@ int device_alloc(T **out, size_t count) {
     return ESP_OK;
 }
 
+// Looks up the device address of the fixed scratch array of esp_gemv_device_noalloc for `device`, which must be the
+// current device (capi_ops.cpp; called once from ensure_init).
+int noalloc_setup(int device);
+
 // Uploads GGUF-layout blocks (host memory) into a DeviceMatrix laid out for the GEMV kernels.
 int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, DeviceMatrix *out);
 void matrix_release(DeviceMatrix *m);

@@ -79,6 +79,15 @@ int esp_matrix_dequantize(const ESPMatrix *matrix, float *out);
  * batch 1 and 2 run the wave-per-row-pair GEMV; batch > 2 (prompt blocks, batched verify; any count) runs
  * the dequant-fused MFMA kernel, which rounds each dequantised weight to fp16 once (the GEMV does not). */
 int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y, const float *residual);
+/* esp_gemv for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  x, y and residual are DEVICE pointers
+ * (fp16 [batch][cols], fp32 [batch][rows], fp32 [batch][rows] or NULL); the call makes no hipMalloc / hipFree: the
+ * split-K partial sums of the matrix-core kernels (batch > 2) live in a fixed 16 MiB array inside the library, one
+ * copy per GPU, held until the process ends.  Limits: batch 1..64 and, for batch > 2, 2 * batch * rows <= 4 Mi floats;
+ * beyond them the call fails with ESP_ERR_OUT_OF_RANGE.  Synchronous like esp_gemv.  All calls on a GPU share that
+ * GPU's array: calls that overlap on one GPU race. */
+int esp_gemv_device_noalloc(const ESPMatrix *matrix, const uint16_t *x_f16_device, int batch, float *y_device,
+                            const float *residual_device_or_null);
 /* Times the GEMV kernel alone on buffers already resident in HBM: `warmup` untimed launches, then
  * `iters` launches bracketed by HIP events on the library stream.  Reports the mean and the best
  * per-launch time in microseconds.  rotate > 1 cycles through that many copies of the matrix so
