@@ -113,7 +113,7 @@ int esp_matrix_dequantize(const ESPMatrix *matrix, float *out) {
 
 namespace {
 // More than two rows of activations go to the matrix-core kernel (fp32 matrices stay on the GEMV path).
-bool use_gemm(const DeviceMatrix &m, int batch) { return batch > 2 && m.format != FMT_F32 && m.cols % 64 == 0; }
+bool use_gemm(const DeviceMatrix &m, int batch) { return batch > 2 && m.format != FMT_F32 && m.cols % 64 == 0 && !gemv_takes_rows(m, batch); }
 constexpr size_t kGemmWorkspaceFloats = (size_t)8 << 20;   // 32 MiB of split-K partial sums
 
 hipError_t run_matvec(const DeviceMatrix &m, const uint16_t *d_x, int batch, float *d_y, const float *d_res, float *workspace, hipStream_t s) {
@@ -202,9 +202,12 @@ int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int
     std::vector<hipEvent_t> marks;
     hipError_t e = hipSuccess;
     rc = ESP_OK;
+    const size_t tiled_bytes = m.tiled ? (size_t)((m.rows + 15) / 16) * (m.cols / 256) * 2304 : 0;
     for (int i = 1; i < rotate && rc == ESP_OK; i++) {
-        copies[i].qs = nullptr; copies[i].scales = nullptr;
+        copies[i].qs = nullptr; copies[i].scales = nullptr; copies[i].tiled = nullptr;
         rc = device_alloc(&copies[i].qs, qs_bytes);
+        if (rc == ESP_OK && tiled_bytes) rc = device_alloc(&copies[i].tiled, tiled_bytes);
+        if (rc == ESP_OK && tiled_bytes) e = hipMemcpyAsync(copies[i].tiled, m.tiled, tiled_bytes, hipMemcpyDeviceToDevice, c.stream);
         if (rc == ESP_OK && sc_count) rc = device_alloc(&copies[i].scales, sc_count);
         if (rc == ESP_OK) e = hipMemcpyAsync(copies[i].qs, m.qs, qs_bytes, hipMemcpyDeviceToDevice, c.stream);
         if (rc == ESP_OK && e == hipSuccess && sc_count)
@@ -256,7 +259,11 @@ int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int
         if (e != hipSuccess) rc = fail_hip(e, "gemv_time");
     }
     for (auto ev : marks) if (ev) (void)hipEventDestroy(ev);
-    for (int i = 1; i < rotate; i++) { if (copies[i].qs) (void)hipFree(copies[i].qs); if (copies[i].scales) (void)hipFree(copies[i].scales); }
+    for (int i = 1; i < rotate; i++) {
+        if (copies[i].qs) (void)hipFree(copies[i].qs);
+        if (copies[i].scales) (void)hipFree(copies[i].scales);
+        if (copies[i].tiled) (void)hipFree(copies[i].tiled);
+    }
     if (d_x) (void)hipFree(d_x);
     if (d_y) (void)hipFree(d_y);
     if (d_ws) (void)hipFree(d_ws);
@@ -334,6 +341,10 @@ int esp_int4_classifier_matvec_argmax(ESPInt4Classifier *h, const float *input, 
     if (e == hipSuccess && index) e = hipMemcpyAsync(index, h->token, sizeof(int), hipMemcpyDeviceToHost, c.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
     return e == hipSuccess ? ESP_OK : fail_hip(e, "int4_classifier");
+}
+
+int esp_set_tuning(const char *key, int value) {
+    return gemv_set_tuning(key, value) ? ESP_OK : fail(ESP_ERR_INVALID_ARGUMENT, "set_tuning: unknown key %s", key ? key : "(null)");
 }
 
 int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s) {

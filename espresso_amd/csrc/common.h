@@ -40,6 +40,9 @@ struct DeviceMatrix {
     int rows = 0, cols = 0;
     uint8_t *qs = nullptr;
     uint16_t *scales = nullptr;
+    // Q4_K only: a second copy of the same super-blocks tiled by (block of sixteen rows, super-block) for the matrix-core
+    // GEMV (layout: kernels/gemv.hip); rows padded to a multiple of sixteen with zero blocks.  Null when not built.
+    uint8_t *tiled = nullptr;
     size_t qs_row_bytes = 0;
     size_t bytes() const {  // algorithmic bytes: what one GEMV must read
         return (size_t)rows * qs_row_bytes + (scales ? (size_t)rows * (cols / 32) * 2 : 0);
@@ -119,6 +122,11 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
 #define ESP_ATTENTION_HEAD_SPLITS 4
 #endif
 constexpr int kAttentionHeadSplits = ESP_ATTENTION_HEAD_SPLITS;
+// Kernel-selection switches (also read from the environment at first use): "q4k_mfma" (ESPRESSO_HIP_Q4K_MFMA) and
+// "q4k_mfma_ks" (ESPRESSO_HIP_Q4K_MFMA_KS).  False for an unknown key.
+bool gemv_set_tuning(const char *key, int value);
+// True when launch_gemv handles `batch` rows without re-reading the weights per pair of rows (always for one or two rows).
+bool gemv_takes_rows(const DeviceMatrix &w, int batch);
 // True when launch_gemv has the EPI_ARGMAX epilogue for this matrix (every format; Q4_K rows of 8192 or more columns, which
 // several wavefronts share, keep the separate argmax launches).
 bool gemv_supports_argmax(const DeviceMatrix &w);
@@ -131,6 +139,8 @@ hipError_t launch_dequant(int format, const uint8_t *blocks, size_t elems, float
 // GGUF-layout blocks -> DeviceMatrix planes (device to device)
 hipError_t launch_repack(int format, const uint8_t *blocks, int rows, int cols, const DeviceMatrix &dst,
                          hipStream_t stream);
+// Q4_K super-blocks, row-major [rows][cols / 256][144 bytes] -> the tiled copy ((rows + 15) / 16 * cols / 256 tiles of 2304 bytes)
+hipError_t launch_q4k_tile(const uint8_t *blocks, int rows, int cols, uint8_t *tiled, hipStream_t stream);
 // DeviceMatrix -> fp32 [rows][cols] (used to check the planes carry the same bits)
 hipError_t launch_dequant_matrix(const DeviceMatrix &m, float *out, hipStream_t stream);
 

@@ -93,6 +93,12 @@ int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, Devic
         (void)hipFree(staging);
     } else {
         e = hipMemcpyAsync(m.qs, gguf_blocks, src_bytes, hipMemcpyHostToDevice, c.stream);
+        // Q4_K matrices of the widths the matrix-core GEMV is built for also get the tiled copy it reads
+        if (e == hipSuccess && format == FMT_Q4_K && (cols == 4096 || cols == 14336)) {
+            const size_t tiled_bytes = (size_t)((rows + 15) / 16) * (cols / 256) * 2304;
+            if ((rc = device_alloc(&m.tiled, tiled_bytes)) != ESP_OK) { matrix_release(&m); return rc; }
+            e = launch_q4k_tile(m.qs, rows, cols, m.tiled, c.stream);
+        }
         if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
     }
     if (e != hipSuccess) { matrix_release(&m); return fail_hip(e, "matrix upload"); }
@@ -103,6 +109,7 @@ int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, Devic
 void matrix_release(DeviceMatrix *m) {
     if (m->qs) (void)hipFree(m->qs);
     if (m->scales) (void)hipFree(m->scales);
+    if (m->tiled) (void)hipFree(m->tiled);
     *m = DeviceMatrix{};
 }
 

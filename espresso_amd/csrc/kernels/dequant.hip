@@ -108,6 +108,27 @@ __global__ void dequant_planes_q4_0_kernel(const uint8_t *qs, const uint16_t *sc
     out[i] = __fmul_rn((float)(n - 8), d);
 }
 
+// One thread per 16-byte piece of the tiled copy: tile (rb, sb) = sixteen headers, then piece (g, n) first halves, then
+// second halves (see the matrix-core GEMV).  Rows past the matrix are zero blocks.
+__global__ void q4k_tile_kernel(const uint8_t *blocks, int rows, int nsb, size_t pieces, uint8_t *tiled) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= pieces) return;
+    const size_t tile = i / 144;
+    const int p = (int)(i - tile * 144);
+    const int rb = (int)(tile / nsb), sb = (int)(tile - (size_t)rb * nsb);
+    int n, src;           // row inside the block, byte offset inside the 144-byte super-block
+    if (p < 16) { n = p; src = 0; }
+    else {
+        const int q = p - 16, half = q >> 6, gn = q & 63;   // piece (g, n) of half `half`
+        n = gn & 15;
+        src = 16 + 32 * (gn >> 4) + 16 * half;
+    }
+    const int row = rb * 16 + n;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (row < rows) v = *reinterpret_cast<const uint4 *>(blocks + ((size_t)row * nsb + sb) * 144 + src);
+    *reinterpret_cast<uint4 *>(tiled + i * 16) = v;
+}
+
 inline dim3 grid_for(size_t n, int threads) { return dim3((unsigned)((n + threads - 1) / threads)); }
 
 }  // namespace
@@ -149,6 +170,14 @@ hipError_t launch_repack(int format, const uint8_t *blocks, int rows, int cols, 
     }
     default: return hipErrorInvalidValue;
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_q4k_tile(const uint8_t *blocks, int rows, int cols, uint8_t *tiled, hipStream_t stream) {
+    if (!blocks || !tiled || rows <= 0 || cols <= 0 || cols % 256 != 0) return hipErrorInvalidValue;
+    const int nsb = cols / 256;
+    const size_t pieces = (size_t)((rows + 15) / 16) * nsb * 144;
+    hipLaunchKernelGGL(q4k_tile_kernel, grid_for(pieces, 256), dim3(256), 0, stream, blocks, rows, nsb, pieces, tiled);
     return hipGetLastError();
 }
 

@@ -29,6 +29,7 @@
 // workgroups that were dispatched first (they get their first weights first and stay ahead).
 #include <cstdlib>
 
+#include <string>
 #include <type_traits>
 
 #include "../common.h"
@@ -85,6 +86,7 @@ struct KernelArgs {
     QkvEpilogue qkv;
     uint16_t *out_f16;
     const uint8_t *qs;
+    const uint8_t *tiled;     // Q4_K: the copy tiled by (sixteen rows, super-block), or null
     const uint16_t *scales;
     size_t qs_row_bytes;
     int rows, cols;
@@ -501,7 +503,14 @@ __device__ __forceinline__ void q4k_stage_x(const KernelArgs &a, int cols, int x
 
 // cols = 64 * IPR: every load of the row is issued before the first use, so staging costs one memory
 // round trip (two with the fused RMSNorm: values, then nothing else - the weights ride along).
-template <int B, int IPR, bool NORM>
+// NATURAL: the LDS layout of the matrix-core kernel (q4k_store_group_natural) instead of the transposed one.
+template <bool NATURAL>
+__device__ __forceinline__ void q4k_store(const uint4 &v, int b, int g, int cols, int xstride, uint4 *xs4, float *xsum) {
+    if constexpr (NATURAL) q4k_store_group_natural(v, b, g, cols, xs4, xsum);
+    else q4k_store_group(v, b, g, cols, xstride, xs4, xsum);
+}
+
+template <int B, int IPR, bool NORM, bool NATURAL = false>
 struct Q4KStage {
     static_assert(IPR % 4 == 0, "whole super-blocks per row");
     static constexpr int GROUPS = IPR * 8, K = (GROUPS + kThreads - 1) / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1;
@@ -554,14 +563,14 @@ struct Q4KStage {
 #pragma unroll
                 for (int k = 0; k < K; k++)
                     if (FULL || tid + k * kThreads < GROUPS)
-                        q4k_store_group(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
+                        q4k_store<NATURAL>(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
             }
         } else {
 #pragma unroll
             for (int b = 0; b < B; b++)
 #pragma unroll
                 for (int k = 0; k < K; k++)
-                    if (FULL || tid + k * kThreads < GROUPS) q4k_store_group(v[b][k], b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
+                    if (FULL || tid + k * kThreads < GROUPS) q4k_store<NATURAL>(v[b][k], b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
         }
     }
 };
@@ -569,7 +578,7 @@ struct Q4KStage {
 // Staging of the persistent kernel when its input is the attention context left as partial states (merge_group
 // above).  Row 0's loads are issued with issue(), before the first weight loads; further rows take one more
 // round trip each inside finish().
-template <int B, int IPR>
+template <int B, int IPR, bool NATURAL = false>
 struct Q4KMergeStage {
     static constexpr int GROUPS = IPR * 8, K = GROUPS / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1;
     static_assert(GROUPS % kThreads == 0, "whole groups per thread");
@@ -582,7 +591,7 @@ struct Q4KMergeStage {
     }
     __device__ __forceinline__ void store_row(int b, uint4 *xs4, float *xsum) {
 #pragma unroll
-        for (int k = 0; k < K; k++) q4k_store_group(merge_group(ml[k], a0[k], a1[k]), b, threadIdx.x + k * kThreads, cols, XSTRIDE, xs4, xsum);
+        for (int k = 0; k < K; k++) q4k_store<NATURAL>(merge_group(ml[k], a0[k], a1[k]), b, threadIdx.x + k * kThreads, cols, XSTRIDE, xs4, xsum);
     }
     __device__ __forceinline__ void issue(const KernelArgs &a) { load_row(a, 0); }
     __device__ __forceinline__ void finish(const KernelArgs &a, uint4 *xs4, float *xsum, float *) {
@@ -834,6 +843,306 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_generic_kernel(const uint8_
     if (lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// Q4_K GEMV on the matrix cores: up to four activation rows for the price of one.
+//
+// v_mfma_f32_16x16x32_f16 computes D[i][j] += sum_k A[i][k] B[k][j] with lane l supplying A[l % 16][8 (l / 16) ..+7] and
+// B[8 (l / 16) ..+7][l % 16], and holding D[4 (l / 16) + r][l % 16], r = 0..3.  Here j is a weight row: a wavefront owns
+// sixteen consecutive rows, and lane (n = l % 16, g = l / 16) works on chunk g (64 weights: sub-blocks 2g in the low
+// nibbles, 2g + 1 in the high ones) of every super-block of row n.  The nibbles go into the B operand under an fp16
+// exponent (64 + n/16, 4 + n/16), exactly as in the dot-product kernels.  The four lane groups of one instruction hold
+// four different sub-blocks, whose scales differ, so their products must not meet in one sum: the sixteen i are used as
+// 4 lane groups x 4 activation rows, and slot i = 4 g + b carries activation row b in lane group g ONLY (zeros in the
+// other three groups).  D[4 g + b][n] is then the sum over lane group g's eight weights alone, and it lands in lane
+// (n, g) - the lane that loaded those weights and holds their super-block header.  Four instructions cover a
+// sub-block; scale, minimum and the exponent offsets are folded per lane as in q4k_item_dots.  Only 4 * NB lanes of an A
+// operand are not zero: those read the staged activations from LDS, the others read a block of zeros with the same
+// offsets.  The vector ALU is left with the nibble masks and the scale arithmetic (about one operation per weight
+// whatever the number of activation rows); the dot products cost it nothing, and a row's sum needs no reduction over
+// the wavefront because a lane keeps adding to its own row.
+//
+// The weights come from the matrix's TILED copy (DeviceMatrix::tiled): a tile is (block of sixteen rows, super-block),
+// 2304 bytes: sixteen 16-byte headers, then piece (g, n) = the first sixteen bytes of chunk g of row n at 256 + 16 (16 g
+// + n), then the second sixteen bytes at 1280 + 16 (16 g + n).  A wavefront's three loads of a step are then three
+// contiguous runs (256 B, 1 KiB, 1 KiB); from the row-major GGUF layout the same lanes would touch sixteen different
+// cache lines per quarter wavefront, which measures 25 % slower.  Rows are padded to a multiple of sixteen with zero
+// blocks (d = dmin = 0), so no load is clamped.
+//
+// Work: a workgroup of WAVES wavefronts takes WAVES / KS blocks of sixteen rows per round, KS wavefronts sharing a block
+// and splitting its super-blocks between them; their partial sums meet in LDS after the last round (one barrier).  The
+// grid is persistent; DEPTH super-block steps of packed weights are in flight per wavefront, across rounds.
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+constexpr int kMfmaRounds = 4;   // rounds whose partial sums have an LDS slot of their own (KS > 1)
+
+// Sum over the workgroup's WAVES wavefronts, added in wavefront order; `red` holds WAVES floats.
+template <int WAVES>
+__device__ __forceinline__ float workgroup_sum_waves(float v, float *red) {
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = red[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; w++) t += red[w];
+    return t;
+}
+
+// Activations of a row (fp16 as given, RMSNorm fused, or attention states merged) into LDS for the matrix-core kernel:
+// every load is issued before the first use, as in Q4KStage; THREADS threads take groups tid, tid + THREADS, ...
+template <int NB, int IPR, int THREADS, int MODE>
+struct MfmaStage {
+    static constexpr int GROUPS = IPR * 8, K = (GROUPS + THREADS - 1) / THREADS, cols = IPR * 64, WAVES = THREADS / 64;
+    static constexpr bool FULL = GROUPS % THREADS == 0;
+    float4 v0[MODE == 1 ? NB : 1][K], v1[MODE == 1 ? NB : 1][K], g0[K], g1[K];
+    uint4 v[MODE == 0 ? NB : 1][K];
+    float4 a0[MODE == 2 ? K : 1][kMergeSplits], a1[MODE == 2 ? K : 1][kMergeSplits];
+    float2 ml[MODE == 2 ? K : 1][kMergeSplits];
+
+    __device__ __forceinline__ int group(int k) const { return FULL || (int)threadIdx.x + k * THREADS < GROUPS ? (int)threadIdx.x + k * THREADS : 0; }
+    __device__ __forceinline__ bool mine(int k) const { return FULL || (int)threadIdx.x + k * THREADS < GROUPS; }
+
+    __device__ __forceinline__ void load_merge_row(const KernelArgs &a, int b) {
+#pragma unroll
+        for (int k = 0; k < K; k++) merge_group_load(a, b, group(k), cols, ml[k], a0[k], a1[k]);
+    }
+    __device__ __forceinline__ void issue(const KernelArgs &a) {
+        if constexpr (MODE == 1) {
+            const float4 *w4 = reinterpret_cast<const float4 *>(a.norm_w);
+            const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int k = 0; k < K; k++) {
+                const int g = group(k);
+                g0[k] = w4[2 * g];
+                g1[k] = w4[2 * g + 1];
+#pragma unroll
+                for (int b = 0; b < NB; b++) {
+                    const float4 *x4 = reinterpret_cast<const float4 *>(a.norm_x + (size_t)b * cols);
+                    v0[b][k] = x4[2 * g];
+                    v1[b][k] = x4[2 * g + 1];
+                    if (!mine(k)) v0[b][k] = v1[b][k] = zero;
+                }
+            }
+        } else if constexpr (MODE == 2) {
+            load_merge_row(a, 0);
+        } else {
+#pragma unroll
+            for (int b = 0; b < NB; b++)
+#pragma unroll
+                for (int k = 0; k < K; k++) v[b][k] = reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + group(k)];
+        }
+    }
+    __device__ __forceinline__ void finish(const KernelArgs &a, uint4 *xs4, float *xsum, float *red) {
+        if constexpr (MODE == 1) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                float s = 0.0f;
+#pragma unroll
+                for (int k = 0; k < K; k++) s += sum_squares(v0[b][k], v1[b][k]);
+                const float inv = 1.0f / sqrtf(workgroup_sum_waves<WAVES>(s, red + b * WAVES) / (float)cols + a.norm_eps);
+#pragma unroll
+                for (int k = 0; k < K; k++)
+                    if (mine(k)) q4k_store_group_natural(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, group(k), cols, xs4, xsum);
+            }
+        } else if constexpr (MODE == 2) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                if (b > 0) load_merge_row(a, b);
+#pragma unroll
+                for (int k = 0; k < K; k++)
+                    if (mine(k)) q4k_store_group_natural(merge_group(ml[k], a0[k], a1[k]), b, group(k), cols, xs4, xsum);
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < NB; b++)
+#pragma unroll
+                for (int k = 0; k < K; k++)
+                    if (mine(k)) q4k_store_group_natural(v[b][k], b, group(k), cols, xs4, xsum);
+        }
+    }
+};
+
+constexpr size_t kQ4KTileBytes = 2304;
+
+template <int NB, int IPR, int WAVES, int KS, int MODE>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t *tiled, const void *activations, const float *norm_w, int rows, int iters,
+                                                                   int workgroups, float norm_eps, KernelArgs rest) {
+    KernelArgs a = rest;
+    a.rows = rows;
+    if constexpr (MODE == 1) { a.norm_x = static_cast<const float *>(activations); a.norm_w = norm_w; a.norm_eps = norm_eps; }
+    else if constexpr (MODE == 2) a.merge_partials = static_cast<const float *>(activations);
+    else a.x = static_cast<const uint16_t *>(activations);
+    constexpr int THREADS = WAVES * 64, cols = IPR * 64, NSB = IPR / 4, S = NSB / KS, RB = WAVES / KS, GROUPS = cols / 8;
+    constexpr int DEPTH = S % 4 == 0 ? 4 : (S % 7 == 0 ? 7 : (S % 2 == 0 ? 2 : 1));   // divides S: a step's slot in the ring is a constant
+    static_assert(NSB % KS == 0 && WAVES % KS == 0 && NB >= 1 && NB <= 4, "whole super-blocks per wavefront");
+    extern __shared__ uint4 smem_raw[];
+    uint4 *xs4 = smem_raw;                                        // [NB][GROUPS] groups of eight fp16, (0,2,1,3) order inside fours
+    uint4 *zero4 = xs4 + (size_t)NB * GROUPS;                     // eight groups of zeros
+    float *xsum = reinterpret_cast<float *>(zero4 + 8);           // [NB][cols / 32]
+    float *red = xsum + (size_t)NB * (cols / 32);                 // [kMfmaRounds][WAVES][NB][16]   (KS > 1)
+    float *misc = red + (KS > 1 ? kMfmaRounds * WAVES * NB * 16 : 0);   // [NB][WAVES] norm sums, later [2][NB][WAVES] arg-max candidates
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, g = lane >> 4, ks = wave % KS, team = wave / KS;
+    const int row_blocks = (a.rows + 15) >> 4;
+    const Q4KLane L = q4k_chunk_constants(g);
+    // constants of the nibble trick, hidden from the optimiser so that (w & mask) | magic stays one v_and_or_b32
+    u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x54005400u, magic_hi = 0x44004400u;
+    asm volatile("" : "+s"(mask_lo), "+s"(mask_hi));
+    asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
+
+    // ---- packed weights: step f of this wavefront = (round f / S, super-block ks * S + f % S of its row block) ----
+    const int total_steps = iters * S;
+    auto block_of = [&](int round) { return (round * workgroups + (int)blockIdx.x) * RB + team; };
+    auto load_step = [&](int f) {
+        Q4KItem it;
+        const int round = f / S, step = f - round * S;
+        const int rb = block_of(round) < row_blocks ? block_of(round) : row_blocks - 1;   // blocks past the end repeat the last one; never stored
+        const uint8_t *tp = tiled + ((size_t)rb * NSB + (ks * S + step)) * kQ4KTileBytes;
+        it.hdr = *reinterpret_cast<const uint4 *>(tp + 16 * n);
+        it.q0 = *reinterpret_cast<const uint4 *>(tp + 256 + 16 * lane);
+        it.q1 = *reinterpret_cast<const uint4 *>(tp + 1280 + 16 * lane);
+        return it;
+    };
+
+    MfmaStage<NB, IPR, THREADS, MODE> stage;
+    stage.issue(a);
+    Q4KItem ring[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++)
+        if (d < total_steps) ring[d] = load_step(d);
+    if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
+    stage.finish(a, xs4, xsum, misc);
+    __syncthreads();
+
+    // ---- the A operand: slot i = lane % 16 carries activation row i % 4 in lane group i / 4 only ----
+    const int slot = lane & 15;
+    const bool feeds = (slot >> 2) == g && (slot & 3) < NB;
+    const uint4 *a_base = feeds ? xs4 + (size_t)(slot & 3) * GROUPS + 32 * (ks * S) + 8 * g : zero4;
+    const int a_stride = feeds ? 32 : 0;                           // groups per super-block step
+    const float *xsum_base = xsum + 8 * (ks * S) + 2 * g;
+
+    float v[NB];
+    auto step_compute = [&](const Q4KItem &it, int i) {            // i: step inside the round (a constant where unrolled)
+        const uint4 *ap = a_base + i * a_stride;
+        const u32 qd[8] = {it.q0.x, it.q0.y, it.q0.z, it.q0.w, it.q1.x, it.q1.y, it.q1.z, it.q1.w};
+        floatx4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const u32 w0 = qd[2 * jj], w1 = qd[2 * jj + 1];
+            const uint4 pl = make_uint4((w0 & mask_lo) | magic_lo, ((w0 >> 8) & mask_lo) | magic_lo, (w1 & mask_lo) | magic_lo, ((w1 >> 8) & mask_lo) | magic_lo);
+            const uint4 ph = make_uint4((w0 & mask_hi) | magic_hi, ((w0 >> 8) & mask_hi) | magic_hi, (w1 & mask_hi) | magic_hi, ((w1 >> 8) & mask_hi) | magic_hi);
+            lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[jj]), __builtin_bit_cast(half8, pl), lo, 0, 0, 0);
+            hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[4 + jj]), __builtin_bit_cast(half8, ph), hi, 0, 0, 0);
+        }
+        // 6-bit (scale, min) of sub-blocks 2g and 2g + 1, as in q4k_item_dots
+        const u32 src_sc = L.upper ? it.hdr.w : it.hdr.y, src_min = L.upper ? it.hdr.w : it.hdr.z;
+        const u32 scp = ((src_sc >> L.sh_sc) & L.mask_low) | ((it.hdr.y >> L.sh_top) & L.mask_top);
+        const u32 mp = ((src_min >> L.sh_min) & L.mask_low) | ((it.hdr.z >> L.sh_top) & L.mask_top);
+        const float sc_lo = (float)(scp & 0xFFu), sc_hi = (float)((scp >> 8) & 0xFFu);
+        const float m_lo = (float)(mp & 0xFFu), m_hi = (float)((mp >> 8) & 0xFFu);
+        const float d16 = 16.0f * half_bits_to_float(it.hdr.x & 0xFFFFu), dmin = half_bits_to_float(it.hdr.x >> 16);
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const float2 xsp = *reinterpret_cast<const float2 *>(xsum_base + (size_t)b * (cols >> 5) + 8 * i);
+            const float nx_lo = lo[b] - 64.0f * xsp.x, nx_hi = hi[b] - 4.0f * xsp.y;
+            v[b] += d16 * (sc_lo * nx_lo + sc_hi * nx_hi) - dmin * (m_lo * xsp.x + m_hi * xsp.y);
+        }
+    };
+
+    // rows n = 2q, 2q + 1 of a block are a pair: the even lane of each pair among lanes 0..15 runs the epilogue.  The
+    // arg-max epilogue keeps a running first maximum per lane instead (rows only grow from round to round).
+    float best[NB];
+    int best_i[NB];
+#pragma unroll
+    for (int b = 0; b < NB; b++) { best[b] = -INFINITY; best_i[b] = 0x7FFFFFFF; }
+    auto finish_block = [&](int rb, float (&sum)[NB]) {            // sum[b]: the row's total, valid in lanes 0..15
+        if (a.epilogue == EPI_ARGMAX) {
+            const int row = rb * 16 + lane;
+            if (lane < 16 && row < a.rows) {
+#pragma unroll
+                for (int b = 0; b < NB; b++) argmax_take(best[b], best_i[b], sum[b], row);
+            }
+            return;
+        }
+        float other[NB];
+#pragma unroll
+        for (int b = 0; b < NB; b++) other[b] = dpp_term<0xB1, 0xF>(sum[b]);   // the neighbouring lane's row
+        if (lane < 16 && (lane & 1) == 0 && rb < row_blocks) pair_epilogue<NB>(a, rb * 8 + (lane >> 1), sum, other);
+    };
+
+    for (int round = 0; round < iters; round++) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) v[b] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < S; i++) {
+            const Q4KItem it = ring[i % DEPTH];
+            const int next = round * S + i + DEPTH;
+            if (next < total_steps) ring[i % DEPTH] = load_step(next);
+            step_compute(it, i);
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) {          // the four lane groups of a row: every lane ends up with the row's share
+            v[b] += __shfl_xor(v[b], 16);
+            v[b] += __shfl_xor(v[b], 32);
+        }
+        if constexpr (KS == 1) {
+            finish_block(block_of(round), v);
+        } else {
+            float *slot_base = red + ((size_t)(round % kMfmaRounds) * WAVES + wave) * NB * 16;
+            if (lane < 16) {
+#pragma unroll
+                for (int b = 0; b < NB; b++) slot_base[b * 16 + lane] = v[b];
+            }
+        }
+    }
+
+    if constexpr (KS > 1) {
+        __syncthreads();
+        // wavefront ks == 0 of each team adds the team's shares (wavefront order, lane groups in order) and finishes its blocks
+        if (ks == 0) {
+            for (int round = 0; round < iters; round++) {
+                float sum[NB];
+#pragma unroll
+                for (int b = 0; b < NB; b++) {
+                    float t = 0.0f;
+                    if (lane < 16) {
+#pragma unroll
+                        for (int w = 0; w < KS; w++) t += red[((size_t)(round % kMfmaRounds) * WAVES + wave + w) * NB * 16 + b * 16 + lane];
+                    }
+                    sum[b] = t;
+                }
+                finish_block(block_of(round), sum);
+            }
+        }
+    }
+
+    if (a.epilogue == EPI_ARGMAX) {
+        // lanes 0..15 of the finishing wavefronts hold candidates: first within the wavefront, then over the workgroup
+        float *cv = misc;
+        int *ci = reinterpret_cast<int *>(misc + NB * WAVES);
+        __syncthreads();   // misc was the norm's scratch
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+#pragma unroll
+            for (int off = 8; off >= 1; off >>= 1) {
+                const float ov = __shfl_xor(best[b], off);
+                const int oi = __shfl_xor(best_i[b], off);
+                argmax_take(best[b], best_i[b], ov, oi);
+            }
+            if (lane == 0) { cv[b * WAVES + wave] = ks == 0 ? best[b] : -INFINITY; ci[b * WAVES + wave] = ks == 0 ? best_i[b] : 0x7FFFFFFF; }
+        }
+        __syncthreads();
+        if (tid < NB) {
+            float bv = cv[tid * WAVES];
+            int bi = ci[tid * WAVES];
+#pragma unroll
+            for (int w = 1; w < WAVES; w++) argmax_take(bv, bi, cv[tid * WAVES + w], ci[tid * WAVES + w]);
+            a.part_value[(size_t)tid * gridDim.x + blockIdx.x] = bv;
+            a.part_index[(size_t)tid * gridDim.x + blockIdx.x] = bi;
+        }
+    }
+}
+
 // Launch through the extension entry point when the caller gave the launch a pair of events of its own: they
 // take the kernel's own start and end times (what a kernel trace reports), without the gaps between launches.
 static thread_local hipEvent_t tl_start_event = nullptr, tl_stop_event = nullptr;
@@ -909,11 +1218,110 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     return hipGetLastError();
 }
 
+
+// The matrix-core Q4_K GEMV: ESPRESSO_HIP_Q4K_MFMA = 0 never, 1 wherever an instantiation exists, unset: the default table below.
+// The matrix-core Q4_K GEMV.  "q4k_mfma" (ESPRESSO_HIP_Q4K_MFMA): 0 never, 1 wherever an instantiation exists, -1 the
+// default (activation batches of two and more rows).  "q4k_mfma_ks" / "q4k_mfma_waves" override the table below.
+int g_q4k_mfma_mode = -2, g_q4k_mfma_split = -2, g_q4k_mfma_waves = -2;   // -2: not read from the environment yet
+int env_int(const char *name, int fallback) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : fallback;
+}
+int q4k_mfma_mode() {
+    if (g_q4k_mfma_mode == -2) g_q4k_mfma_mode = env_int("ESPRESSO_HIP_Q4K_MFMA", -1);
+    return g_q4k_mfma_mode;
+}
+int q4k_mfma_split() {
+    if (g_q4k_mfma_split == -2) g_q4k_mfma_split = env_int("ESPRESSO_HIP_Q4K_MFMA_KS", 0);
+    return g_q4k_mfma_split;
+}
+int q4k_mfma_waves() {
+    if (g_q4k_mfma_waves == -2) g_q4k_mfma_waves = env_int("ESPRESSO_HIP_Q4K_MFMA_WAVES", 0);
+    return g_q4k_mfma_waves;
+}
+
+template <int NB, int IPR, int WAVES, int KS, int MODE>
+hipError_t launch_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
+    constexpr int RB = WAVES / KS, cols = IPR * 64, THREADS = WAVES * 64;
+    *launched = false;
+    const size_t lds = ((size_t)NB * (cols / 8) + 8) * 16 + (size_t)NB * (cols / 32) * 4 + (KS > 1 ? (size_t)kMfmaRounds * WAVES * NB * 16 * 4 : 0) +
+                       (size_t)2 * NB * WAVES * 4;
+    if (lds > 160 * 1024) return hipSuccess;   // not launched
+    auto kernel = gemv_q4k_mfma_kernel<NB, IPR, WAVES, KS, MODE>;
+    static size_t configured_lds = 0;
+    hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
+    if (e != hipSuccess) return e;
+    static int resident_per_cu = 0;
+    if (resident_per_cu == 0) {
+        int n = 0;
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, THREADS, lds);
+        if (e != hipSuccess) return e;
+        const int limit = q4k_wgs_per_cu();
+        resident_per_cu = n < 1 ? 1 : (n > limit ? limit : n);
+    }
+    const int row_blocks = (a.rows + 15) / 16;
+    const int want = (row_blocks + RB - 1) / RB;
+    const int cap = compute_units() * resident_per_cu;
+    // every workgroup runs the same number of rounds: the grid is the smallest that needs no more rounds than the chip-filling one
+    int iters = (want + cap - 1) / cap;
+    const int grid = (want + iters - 1) / iters;
+    iters = (want + grid - 1) / grid;
+    if (KS > 1 && iters > kMfmaRounds) return hipSuccess;   // not launched: the caller takes the other kernel
+    const void *activations = MODE == 1 ? static_cast<const void *>(a.norm_x) : MODE == 2 ? static_cast<const void *>(a.merge_partials) : static_cast<const void *>(a.x);
+    launch_kernel(kernel, dim3(grid), dim3(THREADS), lds, stream, a.tiled, activations, a.norm_w, a.rows, iters, grid, a.norm_eps, a);
+    *launched = true;
+    return hipGetLastError();
+}
+
+// Picks the instantiation; *launched stays false when there is none for this shape.
+template <int NB>
+hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
+    *launched = false;
+    if (!a.tiled) return hipSuccess;
+    const int mode = a.merge_partials ? 2 : a.norm_x ? 1 : 0;
+    int waves = q4k_mfma_waves(), ks = q4k_mfma_split();
+    if (a.cols == 4096) {
+        if (waves == 0) waves = a.rows <= 8192 ? 8 : 4;
+        if (ks == 0) ks = a.rows <= 8192 ? 8 : 2;
+        if (ks > waves) ks = waves;
+#define ESP_MFMA_CASE(W_, KS_)                                                                                   \
+        if (waves == W_ && ks == KS_) {                                                                          \
+            if (mode == 0) return launch_q4k_mfma<NB, 64, W_, KS_, 0>(a, stream, launched);                       \
+            if (mode == 1) return launch_q4k_mfma<NB, 64, W_, KS_, 1>(a, stream, launched);                       \
+            if constexpr (NB <= 2) return launch_q4k_mfma<NB, 64, W_, KS_, 2>(a, stream, launched);               \
+        }
+        ESP_MFMA_CASE(4, 1)
+        ESP_MFMA_CASE(4, 2)
+        ESP_MFMA_CASE(4, 4)
+        ESP_MFMA_CASE(8, 4)
+        ESP_MFMA_CASE(8, 8)
+        ESP_MFMA_CASE(16, 8)
+        ESP_MFMA_CASE(16, 16)
+#undef ESP_MFMA_CASE
+        return hipSuccess;
+    }
+    if (a.cols == 14336 && mode == 0) {
+        if (waves == 0) waves = 8;
+        if (ks == 0) ks = 8;
+        if (waves == 4 && ks == 4) return launch_q4k_mfma<NB, 224, 4, 4, 0>(a, stream, launched);
+        if (waves == 8 && ks == 4) return launch_q4k_mfma<NB, 224, 8, 4, 0>(a, stream, launched);
+        if (waves == 8 && ks == 8) return launch_q4k_mfma<NB, 224, 8, 8, 0>(a, stream, launched);
+        if (waves == 16 && ks == 8) return launch_q4k_mfma<NB, 224, 16, 8, 0>(a, stream, launched);
+        return hipSuccess;
+    }
+    return hipSuccess;
+}
+
 // Column counts with a compile-time instantiation of the persistent kernel (items per row, wavefronts per
 // row pair): the model widths and FFN sizes of the llama family (2048, 4096, 8192; 11008, 14336).
 template <int B>
 hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     const bool norm = a.norm_x != nullptr;
+    if (q4k_mfma_mode() == 1 || (q4k_mfma_mode() < 0 && B >= 2)) {
+        bool launched = false;
+        const hipError_t e = try_q4k_mfma<B>(a, stream, &launched);
+        if (e != hipSuccess || launched) return e;
+    }
     if (a.merge_partials && a.cols == 2048) return launch_q4k_persistent<B, 32, 1, 2>(a, stream);
     if (a.merge_partials && a.cols == 4096) return launch_q4k_persistent<B, 64, 1, 2>(a, stream);
     if (!a.merge_partials) switch (a.cols) {
@@ -971,6 +1379,19 @@ bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch, int head_d
     return true;
 }
 
+bool gemv_set_tuning(const char *key, int value) {
+    const std::string k = key ? key : "";
+    if (k == "q4k_mfma") { g_q4k_mfma_mode = value; return true; }
+    if (k == "q4k_mfma_ks") { g_q4k_mfma_split = value; return true; }
+    if (k == "q4k_mfma_waves") { g_q4k_mfma_waves = value; return true; }
+    return false;
+}
+
+bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
+    if (batch <= 2) return true;
+    return batch <= 8 && w.format == FMT_Q4_K && w.tiled && q4k_mfma_mode() != 0 && (w.cols == 4096 || w.cols == 14336);
+}
+
 bool gemv_supports_argmax(const DeviceMatrix &w) {
     return !(w.format == FMT_Q4_K && (w.cols == 8192 || w.cols == 11008 || w.cols == 14336));
 }
@@ -1003,11 +1424,12 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         explicit CapacityScope(int n) { tl_argmax_capacity = n; }
         ~CapacityScope() { tl_argmax_capacity = 0; }
     } capacity(p.epilogue == EPI_ARGMAX ? p.argmax_capacity : 0);
-    // batches beyond 2 run as successive pairs (each pair re-reads the weights)
-    for (int b0 = 0; b0 < p.batch; b0 += 2) {
-        const int nb = p.batch - b0 >= 2 ? 2 : 1;
+    // batches beyond 2 run as successive pairs (each pair re-reads the weights); the matrix-core Q4_K kernel takes four rows at once
+    const bool fours = p.batch > 2 && gemv_takes_rows(w, p.batch) && !p.merge_partials;
+    for (int b0 = 0, nb = 0; b0 < p.batch; b0 += nb) {
+        nb = fours && p.batch - b0 >= 4 ? 4 : p.batch - b0 >= 2 ? 2 : 1;
         KernelArgs a;
-        a.qs = w.qs; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.rows = w.rows; a.cols = w.cols;
+        a.qs = w.qs; a.tiled = w.tiled; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.rows = w.rows; a.cols = w.cols;
         a.x = p.x ? p.x + (size_t)b0 * w.cols : nullptr;
         a.merge_partials = p.merge_partials;   // batch <= 2 here: one launch
         a.merge_head_dim = p.merge_head_dim;
@@ -1028,7 +1450,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         a.norm_eps = p.norm_eps;
         hipError_t e;
         switch (w.format) {
-        case FMT_Q4_K: e = nb == 1 ? launch_q4k<1>(a, stream) : launch_q4k<2>(a, stream); break;
+        case FMT_Q4_K: e = nb == 1 ? launch_q4k<1>(a, stream) : nb == 2 ? launch_q4k<2>(a, stream) : launch_q4k<4>(a, stream); break;
         case FMT_Q4_0: e = launch_fmt<FMT_Q4_0>(a, nb, stream); break;
         case FMT_Q8_0: e = launch_fmt<FMT_Q8_0>(a, nb, stream); break;
         case FMT_F16: e = launch_fmt<FMT_F16>(a, nb, stream); break;

@@ -108,9 +108,12 @@ struct Q4KLane {   // per-lane constants of the scale unpacking
     u32 magic_lo, magic_hi;   // kept in vector registers for v_and_or_b32
 };
 
-__device__ __forceinline__ Q4KLane q4k_lane_constants(int lane) {
+__device__ __forceinline__ Q4KLane q4k_chunk_constants(int c);
+__device__ __forceinline__ Q4KLane q4k_lane_constants(int lane) { return q4k_chunk_constants(lane & 3); }
+// c = which 64-weight chunk of a super-block the lane works on (0..3)
+__device__ __forceinline__ Q4KLane q4k_chunk_constants(int c) {
     Q4KLane L;
-    const int c = lane & 3, sh = (c & 1) * 16;
+    const int sh = (c & 1) * 16;
     L.upper = c >= 2;
     L.sh_sc = sh;
     L.sh_min = L.upper ? sh + 4 : sh;
@@ -166,6 +169,16 @@ __device__ __forceinline__ void q4k_store_group(const uint4 &v, int b, int g, in
     float s = ((float)as_h2(v.x).x + (float)as_h2(v.x).y) + ((float)as_h2(v.y).x + (float)as_h2(v.y).y) +
               ((float)as_h2(v.z).x + (float)as_h2(v.z).y) + ((float)as_h2(v.w).x + (float)as_h2(v.w).y);
     s += dpp_term<0xB1, 0xF>(s);   // the four lanes of a quad hold the four groups of one 32
+    s += dpp_term<0x4E, 0xF>(s);
+    if ((threadIdx.x & 3) == 0) xsum[(size_t)b * (cols >> 5) + (g >> 2)] = s;
+}
+
+// The same for the matrix-core GEMV: groups of eight in their natural places, [b][cols / 8], sums of each 32 alongside.
+__device__ __forceinline__ void q4k_store_group_natural(const uint4 &v, int b, int g, int cols, uint4 *xs4, float *xsum) {
+    xs4[(size_t)b * (cols >> 3) + g] = swap_middle(v);
+    float s = ((float)as_h2(v.x).x + (float)as_h2(v.x).y) + ((float)as_h2(v.y).x + (float)as_h2(v.y).y) +
+              ((float)as_h2(v.z).x + (float)as_h2(v.z).y) + ((float)as_h2(v.w).x + (float)as_h2(v.w).y);
+    s += dpp_term<0xB1, 0xF>(s);
     s += dpp_term<0x4E, 0xF>(s);
     if ((threadIdx.x & 3) == 0) xsum[(size_t)b * (cols >> 5) + (g >> 2)] = s;
 }

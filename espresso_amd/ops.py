@@ -127,6 +127,14 @@ class Int4Classifier:
             pass
 
 
+def set_tuning(key: str, value: int) -> None:
+    """Kernel-selection switch (esp_set_tuning)."""
+    L = _lib.load_library()
+    L.esp_set_tuning.restype = C.c_int
+    L.esp_set_tuning.argtypes = [C.c_char_p, C.c_int]
+    _lib.check(L.esp_set_tuning(key.encode(), value))
+
+
 def hbm_read_probe(nbytes: int = 1 << 30, iters: int = 10) -> float:
     """GB/s a plain streaming-read kernel reaches over `nbytes` of HBM."""
     L = _lib.load_library()

@@ -108,6 +108,12 @@ void esp_int4_classifier_free(ESPInt4Classifier *classifier);
 int esp_int4_classifier_export(const ESPInt4Classifier *classifier, uint8_t *packed, float *scales, float *biases);
 int esp_int4_classifier_matvec_argmax(ESPInt4Classifier *classifier, const float *input, float *logits_or_null, int *index_or_null);
 
+/* Kernel-selection switches for measurements and tests (no counterpart in the reference); the same switches are read from
+ * the environment when first needed.  "q4k_mfma" (ESPRESSO_HIP_Q4K_MFMA): 1 = Q4_K GEMVs of 4096 / 14336 columns run on the
+ * matrix cores (one to eight activation rows per pass over the weights), 0 = never, -1 = the library's own choice.
+ * "q4k_mfma_ks" (ESPRESSO_HIP_Q4K_MFMA_KS): wavefronts that share a block of sixteen rows, 1 / 2 / 4, 0 = by shape.
+ * Runtimes that captured a step graph keep the kernels they captured. */
+int esp_set_tuning(const char *key, int value);
 /* Measurement aid with no counterpart in the reference: a kernel that only streams `bytes` (>= 1 MiB, a
  * multiple of 16) from HBM with 128-bit loads, `iters` times; reports GB/s.  bench.py prints it next to the
  * GEMV bandwidth so that fractions of the published peak can be read against what a plain reader gets. */

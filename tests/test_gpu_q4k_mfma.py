@@ -1,0 +1,102 @@
+"""The Q4_K GEMV that runs on the matrix cores (one to eight activation rows per pass over the weights), against the
+oracle's matvec on the dequantised weights and against the dot-product kernels, stand-alone and inside the decoder."""
+import numpy as np
+import pytest
+
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mods():
+    import espresso_amd.llama as ll
+    import espresso_amd.ops as ops
+    import espresso_amd.synthetic as syn
+    ops.init()
+    yield ll, ops, syn
+    ops.set_tuning("q4k_mfma", -1)
+    ops.set_tuning("q4k_mfma_waves", 0)
+    ops.set_tuning("q4k_mfma_ks", 0)
+
+
+def q4k_matrix(ops, rows, cols, seed):
+    w = np.random.default_rng(seed).normal(0, 0.02, (rows, cols)).astype(np.float32)
+    blocks = orc.quantize(orc.FMT_Q4_K, w)
+    return ops.Matrix(orc.FMT_Q4_K, blocks, rows, cols), orc.dequantize(orc.FMT_Q4_K, blocks, rows * cols).reshape(rows, cols)
+
+
+@pytest.mark.parametrize("rows,cols", [(16, 4096), (1000, 4096), (4096, 4096), (6144, 4096), (28672, 4096), (130, 14336), (4096, 14336)])
+def test_matches_oracle_and_dot_product_kernels(mods, rows, cols):
+    ll, ops, syn = mods
+    mat, deq = q4k_matrix(ops, rows, cols, rows + cols)
+    rng = np.random.default_rng(rows)
+    scale = np.abs(deq).max() * np.sqrt(cols)
+    for batch in (1, 2, 3, 4, 8):
+        x = rng.normal(0, 1, (batch, cols)).astype(np.float16)
+        res = rng.normal(0, 1, (batch, rows)).astype(np.float32)
+        want = np.stack([orc.matvec(deq, x[b].astype(np.float32)) for b in range(batch)])
+        ops.set_tuning("q4k_mfma", 0)
+        base = mat.gemv(x) if batch <= 2 else None
+        for waves, ks in (((0, 0), (4, 1), (4, 2), (4, 4), (8, 4), (8, 8), (16, 8), (16, 16)) if cols == 4096 else ((0, 0), (4, 4), (8, 4), (16, 8))):
+            ops.set_tuning("q4k_mfma", 1)
+            ops.set_tuning("q4k_mfma_waves", waves)
+            ops.set_tuning("q4k_mfma_ks", ks)
+            y = mat.gemv(x)
+            # exact products, fp32 sums: only the order of additions differs from the oracle's
+            assert np.abs(y - want).max() <= 2e-5 * scale + 1e-6, (batch, ks, np.abs(y - want).max())
+            if base is not None:
+                assert np.abs(y - base).max() <= 2e-5 * scale + 1e-6
+            assert np.array_equal(mat.gemv(x).view(np.uint32), y.view(np.uint32))      # deterministic
+            yr = mat.gemv(x, res)
+            assert np.abs(yr - (want + res)).max() <= 2e-5 * scale + 1e-5
+    # one-hot activations read columns of the dequantised matrix back, in every slot of a four-row pass
+    ops.set_tuning("q4k_mfma", 1)
+    ops.set_tuning("q4k_mfma_waves", 0)
+    ops.set_tuning("q4k_mfma_ks", 0)
+    for j in (0, 7, 31, 32, 255, 256, cols - 1):
+        x = np.zeros((4, cols), np.float16)
+        x[0, j] = 1.0; x[1, (j + 1) % cols] = 1.0; x[2, (j + 33) % cols] = 2.0; x[3, cols - 1 - j] = -1.0
+        y = mat.gemv(x)
+        for b, (col, f) in enumerate([(j, 1.0), ((j + 1) % cols, 1.0), ((j + 33) % cols, 2.0), (cols - 1 - j, -1.0)]):
+            assert np.abs(y[b] - f * deq[:, col]).max() <= 1e-6 * max(1.0, np.abs(deq[:, col]).max()) + 1e-7, (j, b)
+    mat.close()
+
+
+@pytest.mark.parametrize("waves,ks", [(0, 0), (4, 1), (16, 16)])
+def test_decoder_with_matrix_core_gemvs_matches_oracle(mods, waves, ks):
+    """One layer of the 8B shape: fused RMSNorm staging, RoPE / KV-write, SwiGLU and residual epilogues, attention states merged
+    in the wo GEMV - all through the matrix-core kernel - against the oracle, then the two-row verify step."""
+    from test_gpu_full_size import oracle_from_packed
+    ll, ops, syn = mods
+    ops.set_tuning("q4k_mfma", 1)
+    ops.set_tuning("q4k_mfma_waves", waves)
+    ops.set_tuning("q4k_mfma_ks", ks)
+    cfg = ll.MultiModelConfig(**dict(syn.LLAMA3_8B, n_layer=1, max_seq=48))
+    g, packed = syn.build_runtime(cfg, orc.FMT_Q4_K, seed=9, kv_format=orc.FMT_F16, keep_packed=True)
+    o = oracle_from_packed(cfg, packed, orc.FMT_Q4_K, 1, True, 48)
+    prompt = [1, 128255, 777, 64000, 5, 90210, 31337, 2]
+    o.prefill(prompt)
+    g.prefill(np.asarray(prompt, np.uint32))
+    for step in range(5):
+        ho, hg = o.last_hidden(), g.last_hidden()
+        assert np.abs(ho - hg).max() <= 2e-3 * max(1.0, np.abs(ho).max())
+        assert np.abs(o.logits() - g.logits()).max() <= 2e-2
+        tok = o.select_greedy()
+        if o.top2_margin() > 1e-3:
+            assert g.select_greedy() == tok
+        o.advance(tok); g.advance(tok)
+    # graph replay and the two-token loop (two-row passes) give the plain stream
+    plain = g.generate(prompt, 24)[0]
+    ops.set_tuning("q4k_mfma", 0)
+    reference_kernels = syn.build_runtime(cfg, orc.FMT_Q4_K, seed=9, kv_format=orc.FMT_F16)[0]
+    want = reference_kernels.generate(prompt, 24)[0]
+    ops.set_tuning("q4k_mfma", 1)
+    twin = syn.build_runtime(cfg, orc.FMT_Q4_K, seed=9, kv_format=orc.FMT_F16)[0]
+    got, st = ll.generate_two_token(g, twin, prompt, 24)
+    assert got == plain
+    margin_ok = o.generate(prompt, 24, with_margin=True)[1] > 1e-3
+    if margin_ok:
+        assert plain == want
+    for r in (g, twin, reference_kernels):
+        r.close()
