@@ -874,7 +874,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_generic_kernel(const uint8_
 // grid is persistent; DEPTH super-block steps of packed weights are in flight per wavefront, across rounds.
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
-constexpr int kMfmaRounds = 4;   // rounds whose partial sums have an LDS slot of their own (KS > 1)
+constexpr int kMfmaRounds = 8;   // rounds whose partial sums have an LDS slot of their own (KS > 1)
 
 // Sum over the workgroup's WAVES wavefronts, added in wavefront order; `red` holds WAVES floats.
 template <int WAVES>
@@ -1281,9 +1281,16 @@ hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
     const int mode = a.merge_partials ? 2 : a.norm_x ? 1 : 0;
     int waves = q4k_mfma_waves(), ks = q4k_mfma_split();
     if (a.cols == 4096) {
-        if (waves == 0) waves = a.rows <= 8192 ? 8 : 4;
-        if (ks == 0) ks = a.rows <= 8192 ? 8 : 2;
-        if (ks > waves) ks = waves;
+        // measured on the Llama-3-8B shapes (kernel duration / back-to-back, microseconds, one activation row):
+        //   4096 rows: 16 x 16 5.5 / 6.1, 8 x 8 5.8 / 6.5;  6144 rows: 8 x 8 6.3 / 7.0, 16 x 16 6.4 / 7.2;
+        //   28672 rows: 8 x 8 13.8 / 15.4, 4 x 2 14.7 / 15.8; with two rows and more the long matrices prefer 4 x 2
+        if (waves == 0 && ks == 0) {
+            if (a.rows <= 4096) waves = ks = 16;
+            else if (a.rows <= 8192 || NB == 1) waves = ks = 8;
+            else { waves = 4; ks = 2; }
+        }
+        if (waves == 0) waves = 8;
+        if (ks == 0 || ks > waves) ks = waves;
 #define ESP_MFMA_CASE(W_, KS_)                                                                                   \
         if (waves == W_ && ks == KS_) {                                                                          \
             if (mode == 0) return launch_q4k_mfma<NB, 64, W_, KS_, 0>(a, stream, launched);                       \
@@ -1317,7 +1324,9 @@ hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
 template <int B>
 hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     const bool norm = a.norm_x != nullptr;
-    if (q4k_mfma_mode() == 1 || (q4k_mfma_mode() < 0 && B >= 2)) {
+    // By default the matrix-core kernel takes two rows and more, and single rows of the 4096-column matrices except the
+    // output head (for the head and for 14336 columns the dot-product kernel measures the same or better at one row).
+    if (q4k_mfma_mode() == 1 || (q4k_mfma_mode() < 0 && (B >= 2 || (a.cols == 4096 && a.rows <= 65536)))) {
         bool launched = false;
         const hipError_t e = try_q4k_mfma<B>(a, stream, &launched);
         if (e != hipSuccess || launched) return e;
