@@ -974,7 +974,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
     else a.x = static_cast<const uint16_t *>(activations);
     constexpr int THREADS = WAVES * 64, cols = IPR * 64, NSB = IPR / 4, S = NSB / KS, RB = WAVES / KS, GROUPS = cols / 8;
     constexpr int DEPTH = S % 4 == 0 ? 4 : (S % 7 == 0 ? 7 : (S % 2 == 0 ? 2 : 1));   // divides S: a step's slot in the ring is a constant
-    static_assert(NSB % KS == 0 && WAVES % KS == 0 && NB >= 1 && NB <= 4, "whole super-blocks per wavefront");
+    constexpr int SETS = (NB + 3) / 4;   // activation rows 4 s .. 4 s + 3 ride in the slots of A operand set s; every set meets the same B operand
+    static_assert(NSB % KS == 0 && WAVES % KS == 0 && NB >= 1 && NB <= 8, "whole super-blocks per wavefront");
     extern __shared__ uint4 smem_raw[];
     uint4 *xs4 = smem_raw;                                        // [NB][GROUPS] groups of eight fp16, (0,2,1,3) order inside fours
     uint4 *zero4 = xs4 + (size_t)NB * GROUPS;                     // eight groups of zeros
@@ -1016,23 +1017,37 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
 
     // ---- the A operand: slot i = lane % 16 carries activation row i % 4 in lane group i / 4 only ----
     const int slot = lane & 15;
-    const bool feeds = (slot >> 2) == g && (slot & 3) < NB;
-    const uint4 *a_base = feeds ? xs4 + (size_t)(slot & 3) * GROUPS + 32 * (ks * S) + 8 * g : zero4;
-    const int a_stride = feeds ? 32 : 0;                           // groups per super-block step
+    const uint4 *a_base[SETS];
+    int a_stride[SETS];                                            // groups per super-block step
+#pragma unroll
+    for (int set = 0; set < SETS; set++) {
+        const bool feeds = (slot >> 2) == g && 4 * set + (slot & 3) < NB;
+        a_base[set] = feeds ? xs4 + (size_t)(4 * set + (slot & 3)) * GROUPS + 32 * (ks * S) + 8 * g : zero4;
+        a_stride[set] = feeds ? 32 : 0;
+    }
     const float *xsum_base = xsum + 8 * (ks * S) + 2 * g;
 
     float v[NB];
     auto step_compute = [&](const Q4KItem &it, int i) {            // i: step inside the round (a constant where unrolled)
-        const uint4 *ap = a_base + i * a_stride;
+        const uint4 *ap[SETS];
+        floatx4 lo[SETS], hi[SETS];
+#pragma unroll
+        for (int set = 0; set < SETS; set++) {
+            ap[set] = a_base[set] + i * a_stride[set];
+            lo[set] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            hi[set] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
         const u32 qd[8] = {it.q0.x, it.q0.y, it.q0.z, it.q0.w, it.q1.x, it.q1.y, it.q1.z, it.q1.w};
-        floatx4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
             const u32 w0 = qd[2 * jj], w1 = qd[2 * jj + 1];
             const uint4 pl = make_uint4((w0 & mask_lo) | magic_lo, ((w0 >> 8) & mask_lo) | magic_lo, (w1 & mask_lo) | magic_lo, ((w1 >> 8) & mask_lo) | magic_lo);
             const uint4 ph = make_uint4((w0 & mask_hi) | magic_hi, ((w0 >> 8) & mask_hi) | magic_hi, (w1 & mask_hi) | magic_hi, ((w1 >> 8) & mask_hi) | magic_hi);
-            lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[jj]), __builtin_bit_cast(half8, pl), lo, 0, 0, 0);
-            hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[4 + jj]), __builtin_bit_cast(half8, ph), hi, 0, 0, 0);
+#pragma unroll
+            for (int set = 0; set < SETS; set++) {
+                lo[set] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[set][jj]), __builtin_bit_cast(half8, pl), lo[set], 0, 0, 0);
+                hi[set] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[set][4 + jj]), __builtin_bit_cast(half8, ph), hi[set], 0, 0, 0);
+            }
         }
         // 6-bit (scale, min) of sub-blocks 2g and 2g + 1, as in q4k_item_dots
         const u32 src_sc = L.upper ? it.hdr.w : it.hdr.y, src_min = L.upper ? it.hdr.w : it.hdr.z;
@@ -1044,7 +1059,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             const float2 xsp = *reinterpret_cast<const float2 *>(xsum_base + (size_t)b * (cols >> 5) + 8 * i);
-            const float nx_lo = lo[b] - 64.0f * xsp.x, nx_hi = hi[b] - 4.0f * xsp.y;
+            const float nx_lo = lo[b >> 2][b & 3] - 64.0f * xsp.x, nx_hi = hi[b >> 2][b & 3] - 4.0f * xsp.y;
             v[b] += d16 * (sc_lo * nx_lo + sc_hi * nx_hi) - dmin * (m_lo * xsp.x + m_hi * xsp.y);
         }
     };
@@ -1284,9 +1299,10 @@ hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
         // measured on the Llama-3-8B shapes (kernel duration / back-to-back, microseconds, one activation row):
         //   4096 rows: 16 x 16 5.5 / 6.1, 8 x 8 5.8 / 6.5;  6144 rows: 8 x 8 6.3 / 7.0, 16 x 16 6.4 / 7.2;
         //   28672 rows: 8 x 8 13.8 / 15.4, 4 x 2 14.7 / 15.8; with two rows and more the long matrices prefer 4 x 2
+        //   two rows: 14336 rows 8 x 8 9.8, 4 x 2 10.0; 28672 rows 4 x 2 16.4, 8 x 8 17.6.  Eight rows: 4096 rows 8 x 8 8.7, 16 x 16 10.9
         if (waves == 0 && ks == 0) {
-            if (a.rows <= 4096) waves = ks = 16;
-            else if (a.rows <= 8192 || NB == 1) waves = ks = 8;
+            if (a.rows <= 4096 && NB <= 4) waves = ks = 16;
+            else if (a.rows <= 16384 || NB == 1) waves = ks = 8;
             else { waves = 4; ks = 2; }
         }
         if (waves == 0) waves = 8;
@@ -1398,7 +1414,10 @@ bool gemv_set_tuning(const char *key, int value) {
 
 bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
     if (batch <= 2) return true;
-    return batch <= 8 && w.format == FMT_Q4_K && w.tiled && q4k_mfma_mode() != 0 && (w.cols == 4096 || w.cols == 14336);
+    // (eight rows of 14336 columns do not fit the kernel's LDS staging in one pass and stay on the nibble-B GEMM kernel)
+    // and so do five to eight rows of the long 4096-column matrices, where that kernel measures faster: 15.3 against 17.1 us at 14336 rows)
+    if (w.format != FMT_Q4_K || !w.tiled || q4k_mfma_mode() == 0 || batch > 8) return false;
+    return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (w.cols == 4096 && w.rows <= 8192);
 }
 
 bool gemv_supports_argmax(const DeviceMatrix &w) {
@@ -1436,7 +1455,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     // batches beyond 2 run as successive pairs (each pair re-reads the weights); the matrix-core Q4_K kernel takes four rows at once
     const bool fours = p.batch > 2 && gemv_takes_rows(w, p.batch) && !p.merge_partials;
     for (int b0 = 0, nb = 0; b0 < p.batch; b0 += nb) {
-        nb = fours && p.batch - b0 >= 4 ? 4 : p.batch - b0 >= 2 ? 2 : 1;
+        nb = fours && p.batch - b0 == 8 ? 8 : fours && p.batch - b0 >= 4 ? 4 : p.batch - b0 >= 2 ? 2 : 1;
         KernelArgs a;
         a.qs = w.qs; a.tiled = w.tiled; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.rows = w.rows; a.cols = w.cols;
         a.x = p.x ? p.x + (size_t)b0 * w.cols : nullptr;
@@ -1459,7 +1478,13 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         a.norm_eps = p.norm_eps;
         hipError_t e;
         switch (w.format) {
-        case FMT_Q4_K: e = nb == 1 ? launch_q4k<1>(a, stream) : nb == 2 ? launch_q4k<2>(a, stream) : launch_q4k<4>(a, stream); break;
+        case FMT_Q4_K:
+            if (nb == 8) {   // only the matrix-core kernel takes eight rows
+                bool launched = false;
+                e = try_q4k_mfma<8>(a, stream, &launched);
+                if (e == hipSuccess && !launched) e = hipErrorInvalidValue;
+            } else e = nb == 1 ? launch_q4k<1>(a, stream) : nb == 2 ? launch_q4k<2>(a, stream) : launch_q4k<4>(a, stream);
+            break;
         case FMT_Q4_0: e = launch_fmt<FMT_Q4_0>(a, nb, stream); break;
         case FMT_Q8_0: e = launch_fmt<FMT_Q8_0>(a, nb, stream); break;
         case FMT_F16: e = launch_fmt<FMT_F16>(a, nb, stream); break;
