@@ -97,7 +97,7 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
     full = name == "stories-6l-q8_0"
     n_layer = cfg.n_layer if full else 1
     ocfg = orc.LlamaConfig(n_layer=n_layer, n_head=cfg.n_head, n_kv_head=cfg.n_kv_head, d_model=cfg.d_model,
-                           head_dim=cfg.head_dim, hidden_dim=cfg.hidden_dim, vocab=cfg.vocab, max_seq=64 if not full else cfg.max_seq,
+                           head_dim=cfg.head_dim, hidden_dim=cfg.hidden_dim, vocab=cfg.vocab, max_seq=len(gpu["prompt"]) + 16 if not full else cfg.max_seq,
                            norm_eps=cfg.norm_eps, rope_theta=cfg.rope_theta, gemv_inputs_fp16=True, kv_fp16=w["kv"] == "f16")
     rt = orc.LlamaRuntime(ocfg)
     n = cfg.vocab * cfg.d_model
@@ -125,8 +125,12 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
         return {"value": n_tok / dt, "unit": "tok/s", "cores": 1, "kind": "port",
                 "sample": f"whole model, {n_tok} greedy tokens after the same {len(prompt)}-token prompt; "
                           f"tokens identical to the GPU run: {same}"}
-    # bounded sample of the 8B shape: layer 0 alone plus the LM head
-    rt.prefill(prompt[:8].tolist())
+    # bounded sample of the 8B shape: layer 0 alone plus the LM head, at the benchmark's context (the prompt is walked through
+    # the one layer first, so the timed tokens attend over 512+ cached positions as the GPU's do)
+    ctx = len(prompt)
+    t0 = time.perf_counter()
+    rt.prefill(prompt.tolist())
+    t_prefill = time.perf_counter() - t0
     n_tok = 6
     t_layer = t_head = 0.0
     for i in range(n_tok):
@@ -135,43 +139,44 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
     t_layer /= n_tok; t_head /= n_tok
     est = 1.0 / (cfg.n_layer * t_layer + t_head)
     return {"value": est, "unit": "tok/s", "cores": 1, "kind": "port",
-            "sample": f"layer 0 of {cfg.n_layer} ({t_layer * 1e3:.0f} ms/token) and the LM head ({t_head * 1e3:.0f} ms/token), "
-                      f"{n_tok} tokens at context <= 16, extrapolated to {cfg.n_layer} layers (attention at the benchmark's "
-                      f"context not included)"}
+            "sample": f"layer 0 of {cfg.n_layer} ({t_layer * 1e3:.0f} ms/token incl. attention over {ctx}+ cached tokens) and the LM head "
+                      f"({t_head * 1e3:.0f} ms/token), {n_tok} decode tokens after the {ctx}-token prompt was walked through that layer "
+                      f"({t_prefill:.1f} s), extrapolated to {cfg.n_layer} layers"}
 
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # workload (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors kernels of known size in the same runs gave);
 # the runs and the per-kernel table are in profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt.
 MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66569318}
+TRAFFIC_SOURCE = "profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload; not measured in this run)"
 
 
 # BASELINE.json configs[2]: weight-GEMV microbenchmark at the Llama-3-8B layer shapes
 MICRO_SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
 
 
-def run_microbench() -> dict:
+def run_microbench(shapes=None, formats=("q4_k", "q4_0"), batches=(1, 2, 4, 8), launches=100) -> dict:
     """Isolated dequant-GEMV (batch 1, 2: wave-per-row-pair kernel; batch 8: MFMA kernel) for Q4_K and Q4_0, weights
     rotated through enough copies that no launch finds them in the last-level cache."""
     import espresso_amd.ops as ops
     from espresso_amd import _lib
     rows_out = []
-    for name in ("q4_k", "q4_0"):
+    for name in formats:
         fmt = _lib.FORMAT_NAMES[name]
-        for rows, cols in MICRO_SHAPES:
+        for rows, cols in (shapes or MICRO_SHAPES):
             blocks = ops.synth_weights(fmt, 7 + rows + cols, 0.02, rows * cols)
             m = ops.Matrix(fmt, blocks, rows, cols)
             rotate = max(2, min(64, int(600e6 // m.bytes) + 1))
-            for batch in (1, 2, 8):
-                t = m.time_gemv(batch, 10, 100, rotate)
+            for batch in batches:
+                t = m.time_gemv(batch, 10, launches, rotate)
                 nbytes = m.bytes + batch * cols * 2 + batch * rows * 4
                 rows_out.append({"format": name, "rows": rows, "cols": cols, "batch": batch, "mean_us": round(t["mean_us"], 2),
                                  "gbps": round(nbytes / t["mean_us"] / 1e3, 1), "frac_hbm_peak": round(nbytes / t["mean_us"] / 1e3 / HBM_PEAK_GBPS, 3),
                                  "bytes": nbytes})
             m.close()
     return {"metric": "dequant-GEMV HBM GB/s (Llama-3-8B layer shapes)", "unit": "GB/s", "n_gpus": 1, "data": "synthetic",
-            "how": "mean of 100 back-to-back launches between two HIP events after 10 warm-up launches; weights rotate "
-                   "through copies totalling > 600 MB so every launch reads HBM",
+            "how": f"mean of {launches} back-to-back launches between two HIP events after 10 warm-up launches; weights rotate "
+                   "through copies totalling > 600 MB so every launch reads HBM; each mean includes the ~4 us a dependent launch costs",
             "results": rows_out}
 
 
@@ -196,6 +201,13 @@ def run_two_token(steps: int) -> dict:
     t0 = time.perf_counter()
     plain, _ = target.generate(prompts[0], n)
     dt_plain = time.perf_counter() - t0
+    # the target as its own draft: every proposal is accepted, the ceiling of the scheme (two tokens per verify pass)
+    twin, _ = syn.build_runtime(tcfg, _lib.FORMAT_F16, seed=1)
+    ll.generate_two_token(target, twin, prompts[0], 8)
+    t0 = time.perf_counter()
+    twin_tokens, twin_stats = ll.generate_two_token(target, twin, prompts[0], n)
+    dt_twin = time.perf_counter() - t0
+    twin.close()
     batch = {}
     for label, d in (("plain_greedy", None), ("two_token", draft)):
         target.reset(); draft.reset()
@@ -210,14 +222,57 @@ def run_two_token(steps: int) -> dict:
                        "accepted_future_tokens_per_pass": stats["accepted_total"] / max(stats["passes"], 1),
                        "committed_exact_tokens_per_pass": stats["committed_total"] / max(stats["passes"], 1),
                        "stream_identical_to_plain_greedy": tokens == plain[:len(tokens)],
-                       "plain_greedy_tok_s": len(plain) / dt_plain},
+                       "plain_greedy_tok_s": len(plain) / dt_plain,
+                       "target_as_its_own_draft": {"tok_s": len(twin_tokens) / dt_twin, "passes": twin_stats["passes"],
+                                                   "accepted_future_tokens_per_pass": twin_stats["accepted_total"] / max(twin_stats["passes"], 1),
+                                                   "stream_identical_to_plain_greedy": twin_tokens == plain[:len(twin_tokens)]}},
             "batch16": {"tok_s": batch["two_token"]["tok_s"], "passes": b2["passes"],
                         "accepted_future_tokens_per_pass_per_sequence": b2["accepted_total"] / max(b2["passes"], 1) / 16,
                         "committed_exact_tokens_per_pass_per_sequence": b2["committed_total"] / max(b2["passes"], 1) / 16,
                         "streams_identical_to_plain_greedy": batch["two_token"]["tokens"] == batch["plain_greedy"]["tokens"],
                         "plain_greedy_tok_s": batch["plain_greedy"]["tok_s"]},
-            "note": "a random-init draft almost never agrees with a random-init target, so acceptance is ~0 and the two-token "
-                    "figures are the cost of drafting and verifying; tok/s counts decode only (prefill excluded), whole batch"}
+            "note": "a random-init draft almost never agrees with a random-init target, so acceptance is ~0 and those two-token "
+                    "figures are the cost of drafting and verifying; the target as its own draft accepts every proposal and shows the "
+                    "ceiling; tok/s counts decode only (prefill excluded), whole batch"}
+
+
+def run_stamps() -> dict:
+    """Where the time of one Q4_K GEMV launch goes: every wavefront of the last of eight back-to-back launches records
+    100 MHz wall-clock stamps at its start, after the activations are staged, after its first weights were consumed and
+    at its end.  Percentiles over the wavefronts, in microseconds from the first wavefront's start."""
+    import espresso_amd.ops as ops
+    from espresso_amd import _lib
+    fmt = _lib.FORMAT_NAMES["q4_k"]
+    out = []
+    for name, rows, cols in (("q|k|v", 6144, 4096), ("wo", 4096, 4096), ("gate|up", 28672, 4096), ("down", 4096, 14336)):
+        m = ops.Matrix(fmt, ops.synth_weights(fmt, 7 + rows + cols, 0.02, rows * cols), rows, cols)
+        for kernel, mode in (("dot-product", 0), ("matrix-core", 1)):
+            ops.set_tuning("q4k_mfma", mode)
+            st = ops.gemv_stamps(m, 1, 8).astype(np.float64)
+            t = (st - st[:, 0].min()) / 100.0           # microseconds
+            pct = lambda col: [round(float(np.percentile(t[:, col], q)), 2) for q in (0, 50, 90, 100)]
+            out.append({"matrix": name, "rows": rows, "cols": cols, "kernel": kernel, "wavefronts": int(len(t)),
+                        "start_us_min_p50_p90_max": pct(0), "staged_us": pct(1), "first_weights_consumed_us": pct(2), "end_us": pct(3),
+                        "per_wavefront_busy_us_p50": round(float(np.median(t[:, 3] - t[:, 0])), 2)})
+        ops.set_tuning("q4k_mfma", -1)
+        m.close()
+    return {"metric": "per-wavefront stamps of one Q4_K GEMV launch (Llama-3-8B shapes, one activation row, fp16 activations given)",
+            "unit": "us", "n_gpus": 1, "results": out}
+
+
+def reader_ceiling(bytes_per_launch: int, gemv_back_to_back_us: float) -> dict:
+    """A kernel with the persistent Q4_K GEMV's grid and loads that only reads: one launch's worth of bytes per launch
+    (rotating buffers, back to back) and 1 GiB per launch (the steady state)."""
+    import espresso_amd.ops as ops
+    pair = 4608                                        # two rows of 4096 columns
+    n = bytes_per_launch // pair * pair
+    one = ops.hbm_read_probe_pairs(n, pair, 768, max(2, int(1.2e9 // n)), 128)
+    big = ops.hbm_read_probe_pairs((1 << 30) // pair * pair, pair, 768, 2, 8)
+    return {"bytes_per_launch": n, "mean_us": round(one["mean_us"], 2), "gbps": round(one["gbps"], 1),
+            "gemv_back_to_back_over_reader": round(gemv_back_to_back_us / one["mean_us"], 3),
+            "steady_state_gbps_1gib_launch": round(big["gbps"], 1),
+            "note": "same grid (768 workgroups of 4 wavefronts), same 128-bit loads two row pairs deep, no arithmetic, staging or "
+                    "epilogue; back-to-back dependent launches over buffers that rotate through > 1 GB"}
 
 
 def main() -> None:
@@ -232,6 +287,7 @@ def main() -> None:
                     help="launch kernels one at a time instead of replaying the captured per-token HIP graph "
                          "(for rocprofv3 kernel traces)")
     ap.add_argument("--microbench", action="store_true", help="weight-GEMV microbenchmark (Q4_K / Q4_0, batch 1, 2, 8) instead of decode")
+    ap.add_argument("--stamps", action="store_true", help="per-wavefront time stamps inside one Q4_K GEMV launch, per decode shape and kernel")
     ap.add_argument("--two-token", action="store_true", help="exact two-token draft/verify decode on the 6-layer model instead of plain decode")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -243,6 +299,9 @@ def main() -> None:
         return
     if args.two_token:
         print(json.dumps(run_two_token(args.steps or 240)))
+        return
+    if args.stamps:
+        print(json.dumps(run_stamps()))
         return
     w = WORKLOADS[args.workload]
     steps = args.steps if args.steps is not None else w["decode"]
@@ -270,6 +329,7 @@ def main() -> None:
                    "token_bytes_over_hbm_peak_tok_s": HBM_PEAK_GBPS * 1e9 / gpu["weight_bytes"]},
         "roofline": {"bound": "hbm", "kernel": f"dequant-GEMV {dominant}", "achieved": d["gbps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": d["gbps"] / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get((args.workload, dominant)),
+                     "traffic_source": TRAFFIC_SOURCE if (args.workload, dominant) in MEASURED_TRAFFIC else None,
                      "bytes_per_launch": d["bytes_per_launch"], "mean_launch_us": d["kernel_us"], "launches_timed": 8 * (1 if dominant == "head" else n_layer),
                      "all_gemv_gbps": gemv_bytes / gemv_us / 1e3 if gemv_us else 0.0,
                      "all_gemv_frac": gemv_bytes / gemv_us / 1e3 / HBM_PEAK_GBPS if gemv_us else 0.0,
@@ -283,6 +343,7 @@ def main() -> None:
                             "decode pass; each mean includes what a pair costs by itself (event_pair_us)",
                      "kernel_us": {k: round(x, 2) for k, x in gpu["kernel_us"].items()},
                      "event_pair_us": round(pair_us, 2), "back_to_back_us": {k: round(x, 2) for k, x in gpu["b2b_us"].items()},
+                     "reader_same_grid": reader_ceiling(d["bytes_per_launch"], gpu["b2b_us"][dominant]),
                      "plain_read_kernel_gbps": round(ops.hbm_read_probe(1 << 30, 10), 1),
                      "plain_read_kernel_note": "a kernel that only streams 1 GiB with 128-bit loads, same process: the ceiling "
                                                "the memory system gives the simplest reader, to read `frac` against"},
@@ -296,6 +357,7 @@ def main() -> None:
     gpu["rt"].close()
     del gpu
     if not args.no_secondary:
+        secondary = {}
         other = "stories-6l-q8_0" if args.workload == "llama3-8b-q4k" else None
         if other:
             ow = WORKLOADS[other]
@@ -304,11 +366,18 @@ def main() -> None:
             sec = {"metric": "decode tok/s bs1 (6L d768 Q8_0)", "value": osteps / g2["elapsed"], "unit": "tok/s",
                    "steps": osteps, "ms_per_step": g2["elapsed"] / osteps * 1e3, "workload": other,
                    "weight_bytes_per_token": g2["weight_bytes"],
+                   "frac_hbm_peak_whole_token": g2["weight_bytes"] / (g2["elapsed"] / osteps) / 1e9 / HBM_PEAK_GBPS,
                    "per_kernel": {k: {"mean_us": round(v["mean_us"], 2), "gbps": round(v["gbps"], 1)} for k, v in g2["kernel_times"].items()},
                    "per_kernel_note": "raw HIP-event means, event-pair overhead (see event_pair) included"}
             if not args.no_cpu_baseline:
                 sec["cpu_baseline"] = cpu_baseline(other, g2)
-            result["secondary"] = sec
+            g2["rt"].close()
+            del g2
+            secondary[other] = sec
+        # BASELINE.json configs[2] (the two largest shapes; --microbench prints all four) and configs[4]
+        secondary["gemv_microbench"] = run_microbench(shapes=[(14336, 4096), (4096, 14336)], launches=50)
+        secondary["two_token"] = run_two_token(240)
+        result["secondary"] = secondary
     print(json.dumps(result))
 
 

@@ -343,6 +343,37 @@ int esp_int4_classifier_matvec_argmax(ESPInt4Classifier *h, const float *input, 
     return e == hipSuccess ? ESP_OK : fail_hip(e, "int4_classifier");
 }
 
+int esp_gemv_stamps(const ESPMatrix *matrix, int batch, int launches, uint64_t *out_stamps, int capacity_wavefronts, int *out_wavefronts) {
+    if (!matrix || batch < 1 || batch > 2 || launches < 1 || !out_stamps || capacity_wavefronts < 1 || !out_wavefronts)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "gemv_stamps: bad argument");
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    const DeviceMatrix &m = matrix->m;
+    if (m.format != FMT_Q4_K) return fail(ESP_ERR_UNSUPPORTED, "gemv_stamps: the stamped kernels are the persistent Q4_K ones");
+    uint16_t *d_x = nullptr;
+    float *d_y = nullptr;
+    unsigned long long *d_s = nullptr;
+    const size_t words = (size_t)capacity_wavefronts * 4;
+    if ((rc = device_alloc(&d_x, (size_t)batch * m.cols)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_y, (size_t)batch * m.rows)) != ESP_OK) { (void)hipFree(d_x); return rc; }
+    if ((rc = device_alloc(&d_s, words)) != ESP_OK) { (void)hipFree(d_x); (void)hipFree(d_y); return rc; }
+    hipError_t e = hipMemsetAsync(d_x, 0x3c, (size_t)batch * m.cols * 2, c.stream);
+    GemvParams p;
+    p.w = m; p.x = d_x; p.y = d_y; p.batch = batch; p.epilogue = EPI_STORE_F32;
+    for (int i = 0; i + 1 < launches && e == hipSuccess; i++) e = launch_gemv(p, c.stream);   // warm: back to back, the last one is stamped
+    if (e == hipSuccess) e = hipMemsetAsync(d_s, 0, words * 8, c.stream);
+    p.stamps = d_s;
+    if (e == hipSuccess) e = launch_gemv(p, c.stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(out_stamps, d_s, words * 8, hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+    int n = 0;
+    if (e == hipSuccess) for (n = 0; n < capacity_wavefronts && out_stamps[(size_t)n * 4] != 0; n++) {}
+    *out_wavefronts = n;
+    (void)hipFree(d_x); (void)hipFree(d_y); (void)hipFree(d_s);
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "gemv_stamps");
+}
+
 int esp_set_tuning(const char *key, int value) {
     return gemv_set_tuning(key, value) ? ESP_OK : fail(ESP_ERR_INVALID_ARGUMENT, "set_tuning: unknown key %s", key ? key : "(null)");
 }
@@ -372,6 +403,39 @@ int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s) {
     if (t1) (void)hipEventDestroy(t1);
     (void)hipFree(buf); (void)hipFree(sink);
     return e == hipSuccess ? ESP_OK : fail_hip(e, "hbm_read_probe");
+}
+
+int esp_hbm_read_probe_pairs(size_t bytes_per_launch, int pair_bytes, int workgroups, int copies, int launches, double *mean_us, double *gb_per_s) {
+    if (bytes_per_launch < 4096 || pair_bytes <= 0 || pair_bytes % 16 != 0 || bytes_per_launch % (size_t)pair_bytes != 0 || workgroups <= 0 ||
+        copies < 1 || launches < 1 || !mean_us || !gb_per_s)
+        return fail(ESP_ERR_INVALID_ARGUMENT, "hbm_read_probe_pairs: bad argument");
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    uint8_t *buf = nullptr;
+    unsigned *sink = nullptr;
+    if ((rc = device_alloc(&buf, bytes_per_launch * copies)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&sink, (size_t)4)) != ESP_OK) { (void)hipFree(buf); return rc; }
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    hipError_t e = hipMemsetAsync(buf, 1, bytes_per_launch * copies, c.stream);
+    if (e == hipSuccess) e = hipEventCreate(&t0);
+    if (e == hipSuccess) e = hipEventCreate(&t1);
+    auto launch = [&](int i) { return launch_stream_read_pairs(buf + (size_t)(i % copies) * bytes_per_launch, bytes_per_launch, pair_bytes, workgroups, sink, c.stream); };
+    for (int i = 0; i < copies && e == hipSuccess; i++) e = launch(i);
+    if (e == hipSuccess) e = hipEventRecord(t0, c.stream);
+    for (int i = 0; i < launches && e == hipSuccess; i++) e = launch(i);
+    if (e == hipSuccess) e = hipEventRecord(t1, c.stream);
+    if (e == hipSuccess) e = hipEventSynchronize(t1);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+    if (e == hipSuccess && ms > 0.0f) {
+        *mean_us = (double)ms * 1e3 / launches;
+        *gb_per_s = (double)bytes_per_launch * launches / (ms * 1e-3) / 1e9;
+    }
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
+    (void)hipFree(buf); (void)hipFree(sink);
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "hbm_read_probe_pairs");
 }
 
 }  // extern "C"

@@ -92,6 +92,8 @@ struct GemvParams {
     int *argmax_index = nullptr;
     int argmax_capacity = 0;
     int *argmax_blocks = nullptr;
+    // measurement only: device buffer of four wall-clock stamps (100 MHz) per wavefront of the launch (persistent Q4_K kernels)
+    unsigned long long *stamps = nullptr;
     int batch = 1;
     int epilogue = EPI_STORE_F32;
     // optional (batch <= 2): events that take the kernel's own start and end times
@@ -150,6 +152,8 @@ hipError_t launch_int4_matvec(const uint8_t *packed, const float *scales, const 
 
 // kernels/probe.hip — plain streaming read of `bytes` (a multiple of 16)
 hipError_t launch_stream_read(const void *src, size_t bytes, unsigned *sink, hipStream_t stream);
+// the same with the persistent Q4_K GEMV's grid and loads: `grid` workgroups of four wavefronts over pairs of rows of `pair_bytes`
+hipError_t launch_stream_read_pairs(const void *src, size_t bytes, int pair_bytes, int grid, unsigned *sink, hipStream_t stream);
 
 // kernels/synth.hip — seeded N(0, std) weights quantised into GGUF-layout blocks on the GPU
 hipError_t launch_synth(int format, uint64_t seed, float std_dev, size_t elems, uint8_t *out, hipStream_t stream);

@@ -104,7 +104,14 @@ struct KernelArgs {
     // EPI_ARGMAX: one (value, index) pair per workgroup and batch row, [batch][gridDim.x]
     float *part_value;
     int *part_index;
+    // measurement only (null otherwise): four 100 MHz wall-clock stamps per wavefront, [wavefront][4] =
+    // start, activations staged, first weights consumed, end
+    unsigned long long *stamps;
 };
+__device__ __forceinline__ void stamp(const KernelArgs &a, int which) {
+    if (a.stamps && (threadIdx.x & 63) == 0)
+        a.stamps[((size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 4 + which] = wall_clock64();
+}
 
 // First-max rule of the reference's output head (RealModelInferenceEngine.swift:8219-8275, neon_convert.c:36-101): a larger
 // value wins, equal values keep the lower index, NaN never wins.
@@ -733,14 +740,17 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
     typename std::conditional<MODE == 2, Q4KMergeStage<B, MODE == 2 ? IPR : 32>, Q4KStage<B, IPR, MODE == 1>>::type stage;
     const int first_pair = blockIdx.x * TEAMS + wave / TEAM;
     int pair = first_pair;
+    stamp(a, 0);
     stage.issue(a);
     if (pair < npairs) load_pair(pair, buf0);
     stage.finish(a, xs4, xsum, norm_red);
     __syncthreads();
+    stamp(a, 1);
     for (int j = 0; j < iters; j += 2) {
         int next = pair + n_teams;
         if (next < npairs) load_pair(next, buf1);
         process(buf0, pair, j);
+        if (j == 0) stamp(a, 2);
         pair = next;
         if (j + 1 < iters) {
             next = pair + n_teams;
@@ -749,6 +759,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
             pair = next;
         }
     }
+    stamp(a, 3);
     if constexpr (TEAM == 1) {
         if (a.epilogue == EPI_ARGMAX) argmax_workgroup<B>(a, best, best_i, red, reinterpret_cast<int *>(red + B * kWaves));
     }
@@ -992,6 +1003,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
     asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
 
     // ---- packed weights: step f of this wavefront = (round f / S, super-block ks * S + f % S of its row block) ----
+    // The last round is ragged and goes to the workgroups with the lowest indices: they are dispatched first, get their first
+    // weights first (the opening burst of loads is served roughly in order) and stay ahead to the end, so one round more for
+    // them evens the finish.
+    {
+        const int units = (row_blocks + RB - 1) / RB;   // a unit = the RB row blocks a workgroup takes per round
+        iters = (units - (int)blockIdx.x + workgroups - 1) / workgroups;
+        if (iters < 0) iters = 0;
+    }
     const int total_steps = iters * S;
     auto block_of = [&](int round) { return (round * workgroups + (int)blockIdx.x) * RB + team; };
     auto load_step = [&](int f) {
@@ -1005,6 +1024,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
         return it;
     };
 
+    stamp(a, 0);
     MfmaStage<NB, IPR, THREADS, MODE> stage;
     stage.issue(a);
     Q4KItem ring[DEPTH];
@@ -1014,6 +1034,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
     if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
     stage.finish(a, xs4, xsum, misc);
     __syncthreads();
+    stamp(a, 1);
 
     // ---- the A operand: slot i = lane % 16 carries activation row i % 4 in lane group i / 4 only ----
     const int slot = lane & 15;
@@ -1094,6 +1115,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
             const int next = round * S + i + DEPTH;
             if (next < total_steps) ring[i % DEPTH] = load_step(next);
             step_compute(it, i);
+            if (a.stamps && round == 0 && i == 0) { if (v[0] != 12345.678f) stamp(a, 2); }   // after the first weights were needed
         }
 #pragma unroll
         for (int b = 0; b < NB; b++) {          // the four lane groups of a row: every lane ends up with the row's share
@@ -1131,6 +1153,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
         }
     }
 
+    stamp(a, 3);
     if (a.epilogue == EPI_ARGMAX) {
         // lanes 0..15 of the finishing wavefronts hold candidates: first within the wavefront, then over the workgroup
         float *cv = misc;
@@ -1237,6 +1260,7 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
 // The matrix-core Q4_K GEMV: ESPRESSO_HIP_Q4K_MFMA = 0 never, 1 wherever an instantiation exists, unset: the default table below.
 // The matrix-core Q4_K GEMV.  "q4k_mfma" (ESPRESSO_HIP_Q4K_MFMA): 0 never, 1 wherever an instantiation exists, -1 the
 // default (activation batches of two and more rows).  "q4k_mfma_ks" / "q4k_mfma_waves" override the table below.
+int g_q4k_mfma_ragged = 1;
 int g_q4k_mfma_mode = -2, g_q4k_mfma_split = -2, g_q4k_mfma_waves = -2;   // -2: not read from the environment yet
 int env_int(const char *name, int fallback) {
     const char *e = getenv(name);
@@ -1277,9 +1301,10 @@ hipError_t launch_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launch
     const int row_blocks = (a.rows + 15) / 16;
     const int want = (row_blocks + RB - 1) / RB;
     const int cap = compute_units() * resident_per_cu;
-    // every workgroup runs the same number of rounds: the grid is the smallest that needs no more rounds than the chip-filling one
+    // "q4k_mfma_ragged" 0: every workgroup runs the same number of rounds (the smallest grid that needs no more rounds than the
+    // chip-filling one); 1 (default): the grid fills the chip and the ragged last round goes to the first workgroups
     int iters = (want + cap - 1) / cap;
-    const int grid = (want + iters - 1) / iters;
+    int grid = g_q4k_mfma_ragged ? (want < cap ? want : cap) : (want + iters - 1) / iters;
     iters = (want + grid - 1) / grid;
     if (KS > 1 && iters > kMfmaRounds) return hipSuccess;   // not launched: the caller takes the other kernel
     const void *activations = MODE == 1 ? static_cast<const void *>(a.norm_x) : MODE == 2 ? static_cast<const void *>(a.merge_partials) : static_cast<const void *>(a.x);
@@ -1409,6 +1434,7 @@ bool gemv_set_tuning(const char *key, int value) {
     if (k == "q4k_mfma") { g_q4k_mfma_mode = value; return true; }
     if (k == "q4k_mfma_ks") { g_q4k_mfma_split = value; return true; }
     if (k == "q4k_mfma_waves") { g_q4k_mfma_waves = value; return true; }
+    if (k == "q4k_mfma_ragged") { g_q4k_mfma_ragged = value; return true; }
     return false;
 }
 
@@ -1467,6 +1493,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         a.qkv = p.qkv;
         a.part_value = p.argmax_value;
         a.part_index = p.argmax_index;
+        a.stamps = p.stamps;
         if (p.epilogue == EPI_QKV_ROPE) {
             a.qkv.pos += b0;
             a.qkv.seq += b0;

@@ -127,6 +127,17 @@ class Int4Classifier:
             pass
 
 
+def gemv_stamps(m: "Matrix", batch: int = 1, launches: int = 8, capacity: int = 16384) -> np.ndarray:
+    """[wavefronts][4] wall-clock stamps (100 MHz ticks: start, staged, first weights consumed, end) of one Q4_K GEMV launch."""
+    L = _lib.load_library()
+    L.esp_gemv_stamps.restype = C.c_int
+    L.esp_gemv_stamps.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_int)]
+    out = np.zeros((capacity, 4), dtype=np.uint64)
+    n = C.c_int(0)
+    _lib.check(L.esp_gemv_stamps(m._h, batch, launches, _ptr(out), capacity, C.byref(n)))
+    return out[:n.value]
+
+
 def set_tuning(key: str, value: int) -> None:
     """Kernel-selection switch (esp_set_tuning)."""
     L = _lib.load_library()
@@ -143,6 +154,16 @@ def hbm_read_probe(nbytes: int = 1 << 30, iters: int = 10) -> float:
     out = C.c_double(0)
     _lib.check(L.esp_hbm_read_probe(nbytes, iters, C.byref(out)))
     return out.value
+
+
+def hbm_read_probe_pairs(bytes_per_launch: int, pair_bytes: int = 4608, workgroups: int = 768, copies: int = 16, launches: int = 64) -> dict:
+    """Mean microseconds and GB/s of a reader with the persistent Q4_K GEMV's grid and loads over `bytes_per_launch` per launch."""
+    L = _lib.load_library()
+    L.esp_hbm_read_probe_pairs.restype = C.c_int
+    L.esp_hbm_read_probe_pairs.argtypes = [C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
+    us, gbps = C.c_double(0), C.c_double(0)
+    _lib.check(L.esp_hbm_read_probe_pairs(bytes_per_launch, pair_bytes, workgroups, copies, launches, C.byref(us), C.byref(gbps)))
+    return {"mean_us": us.value, "gbps": gbps.value}
 
 
 def synth_weights(fmt: int, seed: int, std: float, elements: int) -> np.ndarray:

@@ -108,6 +108,10 @@ void esp_int4_classifier_free(ESPInt4Classifier *classifier);
 int esp_int4_classifier_export(const ESPInt4Classifier *classifier, uint8_t *packed, float *scales, float *biases);
 int esp_int4_classifier_matvec_argmax(ESPInt4Classifier *classifier, const float *input, float *logits_or_null, int *index_or_null);
 
+/* Measurement aid (no counterpart in the reference): runs the Q4_K GEMV `launches` times back to back and has every wavefront
+ * of the last launch record four 100 MHz wall-clock stamps: start, activations staged, first weights consumed, end.
+ * out_stamps receives [wavefront][4]; *out_wavefronts how many wavefronts wrote (at most capacity_wavefronts). */
+int esp_gemv_stamps(const ESPMatrix *matrix, int batch, int launches, uint64_t *out_stamps, int capacity_wavefronts, int *out_wavefronts);
 /* Kernel-selection switches for measurements and tests (no counterpart in the reference); the same switches are read from
  * the environment when first needed.  "q4k_mfma" (ESPRESSO_HIP_Q4K_MFMA): 1 = Q4_K GEMVs of 4096 / 14336 columns run on the
  * matrix cores (one to eight activation rows per pass over the weights), 0 = never, -1 = the library's own choice.
@@ -118,6 +122,13 @@ int esp_set_tuning(const char *key, int value);
  * multiple of 16) from HBM with 128-bit loads, `iters` times; reports GB/s.  bench.py prints it next to the
  * GEMV bandwidth so that fractions of the published peak can be read against what a plain reader gets. */
 int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s);
+/* The ceiling for ONE GEMV launch: a kernel with the persistent Q4_K GEMV's grid (`workgroups` of four wavefronts) and its
+ * loads (a wavefront takes pairs of rows of `pair_bytes`, the next pair's 128-bit loads in flight while the current one is
+ * consumed) that does nothing else, launched back to back `launches` times over `copies` buffers of `bytes_per_launch` in
+ * turn (so that no launch finds its bytes in a cache).  Reports the mean time per launch, which includes what a dependent
+ * launch costs on this machine, and the resulting GB/s. */
+int esp_hbm_read_probe_pairs(size_t bytes_per_launch, int pair_bytes, int workgroups, int copies, int launches, double *mean_us,
+                             double *gb_per_s);
 
 /* ---- llama decoder state resident on the GPU -------------------------------------------- *
  * Replaces CPUExactLlamaRuntime (Sources/RealModelInference/RealModelInferenceEngine.swift:548-850):
