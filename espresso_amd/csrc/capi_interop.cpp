@@ -1,7 +1,9 @@
 // C ABI: kernel handles and surfaces in the call shape of the reference's ANEInterop module
 // (Sources/ANEInterop/include/ane_interop.h).  See the header for the contract of every function.
 #include <atomic>
+#include <cmath>
 #include <cstring>
+#include <initializer_list>
 #include <map>
 #include <sstream>
 #include <string>
@@ -71,7 +73,7 @@ bool slice_ok(const ESPSurface *s, int ch_off, int channels, int spatial, int in
     return region_ok(s, ch_off, channels, spatial) && index >= 0 && index < spatial;
 }
 
-enum KernelKind { KIND_GEMV, KIND_CLASSIFIER, KIND_FFN };
+enum KernelKind { KIND_GEMV, KIND_CLASSIFIER, KIND_FFN, KIND_QKV, KIND_PROJECTION };
 
 std::string trim(const std::string &s) {
     size_t a = s.find_first_not_of(" \t\r"), b = s.find_last_not_of(" \t\r");
@@ -125,7 +127,7 @@ WeightBytes payload_of(WeightBytes w) {
 
 struct ESPHandle {
     int kind = KIND_GEMV;
-    int lanes = 1, spatial = 1, rows = 0, cols = 0, dim = 0, hidden = 0, vocab = 0;
+    int lanes = 1, spatial = 1, rows = 0, cols = 0, dim = 0, hidden = 0, vocab = 0, q_dim = 0, kv_dim = 0;
     float norm_eps = 1e-5f;
     DeviceMatrix w, w13, w2, classifier;
     float *norm = nullptr;
@@ -288,6 +290,42 @@ ESPHandle *esp_interop_compile(const uint8_t *program, size_t program_len, const
         want_in = {(size_t)h->dim * h->spatial * 2};
         want_out = {(size_t)h->dim * h->spatial * 2};
         h->rows = h->dim; h->cols = h->dim;
+    } else if (kind == "decode_qkv") {
+        // decodeQKVOnly (DecodeAttentionQKVGenerator.swift:86-131; outputs k @ 0, q @ 1, v @ 2, DecodeForwardPass.swift:374-377):
+        // rmsnorm, then the three projections; RoPE, the KV-cache update and attention are separate calls, as in the reference
+        h->kind = KIND_QKV;
+        h->dim = get_int("dim", 0); h->q_dim = get_int("q_dim", h->dim); h->kv_dim = get_int("kv_dim", h->dim);
+        WeightBytes *g = need("rms_att"), *wq = need("wq"), *wk = need("wk"), *wv = need("wv");
+        if (format < 0 || h->dim <= 0 || h->q_dim <= 0 || h->kv_dim <= 0 || !g || !wq || !wk || !wv)
+            return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: decode_qkv needs format, dim, rms_att, wq, wk and wv%s");
+        rc = upload_norm(*g, h->dim, &h->norm);
+        if (rc == ESP_OK) {
+            const size_t rb = format_bytes(format, (size_t)h->dim);
+            WeightBytes pq = format == FMT_F16 ? payload_of(*wq) : *wq, pk = format == FMT_F16 ? payload_of(*wk) : *wk, pv = format == FMT_F16 ? payload_of(*wv) : *wv;
+            if (pq.len != rb * h->q_dim || pk.len != rb * h->kv_dim || pv.len != rb * h->kv_dim) rc = fail(ESP_ERR_INVALID_ARGUMENT, "wq/wk/wv byte counts do not match their shapes");
+            else {
+                std::vector<uint8_t> fused(rb * (size_t)(h->q_dim + 2 * h->kv_dim));   // rows: q, then k, then v
+                std::memcpy(fused.data(), pq.data, pq.len);
+                std::memcpy(fused.data() + pq.len, pk.data, pk.len);
+                std::memcpy(fused.data() + pq.len + pk.len, pv.data, pv.len);
+                rc = matrix_upload(format, fused.data(), h->q_dim + 2 * h->kv_dim, h->dim, &h->w);
+            }
+        }
+        want_in = {(size_t)h->dim * h->spatial * 2};
+        want_out = {(size_t)h->kv_dim * h->spatial * 2, (size_t)h->q_dim * h->spatial * 2, (size_t)h->kv_dim * h->spatial * 2};
+        h->rows = h->q_dim + 2 * h->kv_dim; h->cols = h->dim;
+    } else if (kind == "decode_projection") {
+        // decodeProjection: out = residual + Wo * context; input 0 = the attention context, input 1 = the residual, which the
+        // reference rebinds to the layer's input surface (DecodeForwardPass.swift:383,396)
+        h->kind = KIND_PROJECTION;
+        h->dim = get_int("dim", 0); h->q_dim = get_int("q_dim", h->dim);
+        WeightBytes *wo = need("wo");
+        if (format < 0 || h->dim <= 0 || h->q_dim <= 0 || !wo)
+            return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: decode_projection needs format, dim and wo%s");
+        rc = upload_matrix(*wo, format, h->dim, h->q_dim, &h->w);
+        want_in = {(size_t)h->q_dim * h->spatial * 2, (size_t)h->dim * h->spatial * 2};
+        want_out = {(size_t)h->dim * h->spatial * 2};
+        h->rows = h->dim; h->cols = h->q_dim;
     } else {
         return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_COMPILER_FAILURE, "compile: unknown kernel kind %s", kind.c_str());
     }
@@ -300,7 +338,7 @@ ESPHandle *esp_interop_compile(const uint8_t *program, size_t program_len, const
         if (output_sizes[i] != want_out[i]) return compile_fail(h, ESP_INTEROP_COMPILE_ERROR_INVALID_ARGUMENTS, "compile: output surface size does not match channels x spatial x 2%s");
     for (size_t b : want_in) h->inputs.push_back(esp_interop_create_surface(b));
     for (size_t b : want_out) h->outputs.push_back(esp_interop_create_surface(b));
-    const size_t widest = (size_t)std::max(std::max(h->rows, h->cols), std::max(h->hidden, h->vocab));
+    const size_t widest = (size_t)std::max(std::max(std::max(h->rows, h->cols), std::max(h->hidden, h->vocab)), std::max(h->dim, h->q_dim));
     bool ok = device_alloc(&h->x16, (size_t)h->lanes * widest) == ESP_OK && device_alloc(&h->act16, (size_t)h->lanes * widest) == ESP_OK &&
               device_alloc(&h->x32, (size_t)h->lanes * widest) == ESP_OK && device_alloc(&h->y32, (size_t)h->lanes * widest) == ESP_OK &&
               hipEventCreate(&h->ev0) == hipSuccess && hipEventCreate(&h->ev1) == hipSuccess;
@@ -336,6 +374,20 @@ bool esp_interop_eval(ESPHandle *h) {
         if (e == hipSuccess) e = launch_gemv(g, s);
         if (e == hipSuccess) e = launch_scatter_columns(h->y32, h->vocab, h->spatial, h->lanes, out0, s);
         if (e == hipSuccess) e = launch_row_max(h->y32, h->vocab, h->spatial, h->lanes, reinterpret_cast<uint16_t *>(h->outputs[1]->device), s);
+    } else if (e == hipSuccess && h->kind == KIND_QKV) {
+        e = launch_gather_columns(in0, h->dim, h->spatial, h->lanes, nullptr, h->x32, s);
+        g.w = h->w; g.norm_x = h->x32; g.norm_w = h->norm; g.norm_eps = h->norm_eps; g.y = h->y32; g.epilogue = EPI_STORE_F32;
+        if (e == hipSuccess) e = launch_gemv(g, s);
+        const int stride = h->q_dim + 2 * h->kv_dim;
+        if (e == hipSuccess) e = launch_scatter_columns_strided(h->y32 + h->q_dim, stride, h->kv_dim, h->spatial, h->lanes, out0, s);                         // k @ 0
+        if (e == hipSuccess) e = launch_scatter_columns_strided(h->y32, stride, h->q_dim, h->spatial, h->lanes, reinterpret_cast<uint16_t *>(h->outputs[1]->device), s);   // q @ 1
+        if (e == hipSuccess) e = launch_scatter_columns_strided(h->y32 + h->q_dim + h->kv_dim, stride, h->kv_dim, h->spatial, h->lanes, reinterpret_cast<uint16_t *>(h->outputs[2]->device), s);   // v @ 2
+    } else if (e == hipSuccess && h->kind == KIND_PROJECTION) {
+        e = launch_gather_columns(in0, h->q_dim, h->spatial, h->lanes, h->x16, nullptr, s);
+        if (e == hipSuccess) e = launch_gather_columns(reinterpret_cast<const uint16_t *>(h->inputs[1]->device), h->dim, h->spatial, h->lanes, nullptr, h->x32, s);
+        g.w = h->w; g.x = h->x16; g.y = h->y32; g.residual = h->x32; g.epilogue = EPI_ADD_RESIDUAL;
+        if (e == hipSuccess) e = launch_gemv(g, s);
+        if (e == hipSuccess) e = launch_scatter_columns(h->y32, h->dim, h->spatial, h->lanes, out0, s);
     } else if (e == hipSuccess) {
         e = launch_gather_columns(in0, h->dim, h->spatial, h->lanes, nullptr, h->x32, s);
         g.w = h->w13; g.norm_x = h->x32; g.norm_w = h->norm; g.norm_eps = h->norm_eps; g.out_f16 = h->act16; g.epilogue = EPI_SWIGLU_F16;
@@ -489,6 +541,189 @@ bool esp_interop_io_argmax_batch_fp16_spatial(ESPSurfaceRef surface, int ch_off,
     const uint16_t *s = shadow_for_read(surface);
     if (!s) return false;
     for (int i = 0; i < stream_count; i++) esp_interop_argmax_f16_strided(s + (size_t)ch_off * spatial + i, channels, spatial, &out_indices[i], &out_values[i]);
+    return true;
+}
+
+// ---- what the reference's hybrid decode does between its kernel evaluations, on surfaces resident in HBM ----
+namespace {
+bool surfaces_on_device(std::initializer_list<ESPSurface *> list) {
+    for (ESPSurface *s : list) if (!s || !surface_to_device(s)) return false;
+    return true;
+}
+void written_on_device(ESPSurface *s) { s->device_valid = true; s->host_valid = false; }
+bool finish(hipError_t e, const char *what) {
+    if (e == hipSuccess) e = hipStreamSynchronize(context().stream);
+    if (e != hipSuccess) { fail_hip(e, what); return false; }
+    return true;
+}
+}  // namespace
+
+bool esp_interop_rope_decode(ESPSurfaceRef q, ESPSurfaceRef k, int n_heads, int n_kv_heads, int head_dim, int position, float theta, int lane_spatial) {
+    if (n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || head_dim % 2 != 0 || position < 0 || lane_spatial <= 0 ||
+        !region_ok(q, 0, n_heads * head_dim, lane_spatial) || !region_ok(k, 0, n_kv_heads * head_dim, lane_spatial) || !surfaces_on_device({q, k}))
+        return false;
+    const hipError_t e = launch_surface_rope(reinterpret_cast<uint16_t *>(q->device), reinterpret_cast<uint16_t *>(k->device), n_heads, n_kv_heads, head_dim,
+                                             position, theta, lane_spatial, context().stream);
+    written_on_device(q); written_on_device(k);
+    return finish(e, "rope_decode");
+}
+
+bool esp_interop_kv_cache_scatter(ESPSurfaceRef k_src, ESPSurfaceRef v_src, ESPSurfaceRef k_cache, ESPSurfaceRef v_cache, int kv_dim, int token_index,
+                                  int cache_stride, int lane_spatial) {
+    if (kv_dim <= 0 || lane_spatial <= 0 || !slice_ok(k_cache, 0, kv_dim, cache_stride, token_index) || !slice_ok(v_cache, 0, kv_dim, cache_stride, token_index) ||
+        !region_ok(k_src, 0, kv_dim, lane_spatial) || !region_ok(v_src, 0, kv_dim, lane_spatial) || !surfaces_on_device({k_src, v_src, k_cache, v_cache}))
+        return false;
+    const hipError_t e = launch_surface_kv_scatter(reinterpret_cast<const uint16_t *>(k_src->device), reinterpret_cast<const uint16_t *>(v_src->device),
+                                                   reinterpret_cast<uint16_t *>(k_cache->device), reinterpret_cast<uint16_t *>(v_cache->device), kv_dim,
+                                                   token_index, cache_stride, lane_spatial, context().stream);
+    written_on_device(k_cache); written_on_device(v_cache);
+    return finish(e, "kv_cache_scatter");
+}
+
+bool esp_interop_decode_sdpa(ESPSurfaceRef q, ESPSurfaceRef k_cache, ESPSurfaceRef v_cache, ESPSurfaceRef context_surface, int heads, int kv_heads, int head_dim,
+                             int visible_tokens, int token_base, int cache_stride, int lane_spatial) {
+    if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim <= 0 || visible_tokens <= 0 || token_base < 0 || lane_spatial <= 0 ||
+        token_base + visible_tokens > cache_stride || !region_ok(q, 0, heads * head_dim, lane_spatial) ||
+        !region_ok(context_surface, 0, heads * head_dim, lane_spatial) || !region_ok(k_cache, 0, kv_heads * head_dim, cache_stride) ||
+        !region_ok(v_cache, 0, kv_heads * head_dim, cache_stride) || !surfaces_on_device({q, k_cache, v_cache, context_surface}))
+        return false;
+    const hipError_t e = launch_surface_sdpa(reinterpret_cast<const uint16_t *>(q->device), reinterpret_cast<const uint16_t *>(k_cache->device),
+                                             reinterpret_cast<const uint16_t *>(v_cache->device), reinterpret_cast<uint16_t *>(context_surface->device), heads,
+                                             kv_heads, head_dim, visible_tokens, token_base, cache_stride, lane_spatial, context().stream);
+    written_on_device(context_surface);
+    return finish(e, "decode_sdpa");
+}
+
+// ---- the remaining surface I/O variants of ane_interop.h ----
+void esp_interop_gather_f16_to_f32(float *dst, const void *src, int count, int stride) {
+    const uint16_t *s = static_cast<const uint16_t *>(src);
+    for (int i = 0; i < count; i++) dst[i] = half_to_float(s[(size_t)i * stride]);
+}
+void esp_interop_scatter_f32_to_f16(void *dst, const float *src, int count, int stride) {
+    uint16_t *d = static_cast<uint16_t *>(dst);
+    for (int i = 0; i < count; i++) d[(size_t)i * stride] = float_to_half_rne(src[i]);
+}
+
+bool esp_interop_io_copy_two_fp16_spatial_slices(ESPSurfaceRef dst0, int dst0_ch_off, int dst0_index, int dst0_spatial, ESPSurfaceRef src0, int src0_ch_off,
+                                                 int src0_index, int src0_spatial, ESPSurfaceRef dst1, int dst1_ch_off, int dst1_index, int dst1_spatial,
+                                                 ESPSurfaceRef src1, int src1_ch_off, int src1_index, int src1_spatial, int channels) {
+    // both pairs are checked before either is touched
+    if (!slice_ok(dst0, dst0_ch_off, channels, dst0_spatial, dst0_index) || !slice_ok(src0, src0_ch_off, channels, src0_spatial, src0_index) ||
+        !slice_ok(dst1, dst1_ch_off, channels, dst1_spatial, dst1_index) || !slice_ok(src1, src1_ch_off, channels, src1_spatial, src1_index))
+        return false;
+    return esp_interop_io_copy_fp16_spatial_slice(dst0, dst0_ch_off, dst0_index, dst0_spatial, src0, src0_ch_off, src0_index, src0_spatial, channels) &&
+           esp_interop_io_copy_fp16_spatial_slice(dst1, dst1_ch_off, dst1_index, dst1_spatial, src1, src1_ch_off, src1_index, src1_spatial, channels);
+}
+
+bool esp_interop_io_argmax_fp16_spatial_slice_with_hint(ESPSurfaceRef surface, int ch_off, int index, int spatial, int channels, ESPSurfaceRef hint_surface,
+                                                        int hint_index, int hint_spatial, int *out_index, float *out_value) {
+    if (channels <= 0 || !slice_ok(surface, ch_off, channels, spatial, index) || !slice_ok(hint_surface, 0, 1, hint_spatial, hint_index)) return false;
+    const uint16_t *s = shadow_for_read(surface), *hint = shadow_for_read(hint_surface);
+    if (!s || !hint) return false;
+    // the hint is the column's maximum (the classifier kernel's reduce_max output): the first channel that equals it is the
+    // first maximum; a hint that matches nothing falls back to the full scan
+    const uint16_t want = hint[hint_index];
+    for (int c = 0; c < channels; c++)
+        if (s[(size_t)(ch_off + c) * spatial + index] == want) {
+            if (out_index) *out_index = c;
+            if (out_value) *out_value = half_to_float(want);
+            return true;
+        }
+    esp_interop_argmax_f16_strided(s + (size_t)ch_off * spatial + index, channels, spatial, out_index, out_value);
+    return true;
+}
+
+bool esp_interop_io_write_fp16_at_batched(ESPSurfaceRef surface, const int *channel_offsets, const float *const *sources, const int *channels, int region_count,
+                                          int spatial) {
+    if (!channel_offsets || !sources || !channels || region_count < 0) return false;
+    for (int r = 0; r < region_count; r++) if (!sources[r] || !region_ok(surface, channel_offsets[r], channels[r], spatial)) return false;
+    for (int r = 0; r < region_count; r++) if (!esp_interop_io_write_fp16_at(surface, channel_offsets[r], sources[r], channels[r], spatial)) return false;
+    return true;
+}
+
+bool esp_interop_io_copy_batched(ESPSurfaceRef dst, ESPSurfaceRef src, const int *dst_channel_offsets, const int *src_channel_offsets, const int *channels,
+                                 int region_count, int spatial) {
+    if (!dst_channel_offsets || !src_channel_offsets || !channels || region_count < 0) return false;
+    for (int r = 0; r < region_count; r++)
+        if (!region_ok(dst, dst_channel_offsets[r], channels[r], spatial) || !region_ok(src, src_channel_offsets[r], channels[r], spatial)) return false;
+    for (int r = 0; r < region_count; r++) if (!esp_interop_io_copy(dst, dst_channel_offsets[r], src, src_channel_offsets[r], channels[r], spatial)) return false;
+    return true;
+}
+
+bool esp_interop_io_copy_multi_src(ESPSurfaceRef dst, const ESPSurfaceRef *sources, const int *dst_channel_offsets, const int *src_channel_offsets,
+                                   const int *channels, int region_count, int spatial) {
+    if (!sources || !dst_channel_offsets || !src_channel_offsets || !channels || region_count < 0) return false;
+    for (int r = 0; r < region_count; r++)
+        if (!region_ok(dst, dst_channel_offsets[r], channels[r], spatial) || !region_ok(sources[r], src_channel_offsets[r], channels[r], spatial)) return false;
+    for (int r = 0; r < region_count; r++)
+        if (!esp_interop_io_copy(dst, dst_channel_offsets[r], sources[r], src_channel_offsets[r], channels[r], spatial)) return false;
+    return true;
+}
+
+// The channel range is split into n_blocks parts that are scanned independently and merged in channel order, so the result
+// is the serial scan's: lowest index on ties (surface_io.c:689-700).  (The reference runs the parts on separate cores.)
+bool esp_interop_io_argmax_batch_fp16_spatial_parallel(ESPSurfaceRef surface, int ch_off, int spatial, int channels, int stream_count, int *out_indices,
+                                                       float *out_values, int n_blocks) {
+    if (!out_indices || !out_values || stream_count < 0 || stream_count > spatial || channels <= 0 || !region_ok(surface, ch_off, channels, spatial)) return false;
+    const uint16_t *s = shadow_for_read(surface);
+    if (!s) return false;
+    if (n_blocks < 1) n_blocks = 1;
+    if (n_blocks > channels) n_blocks = channels;
+    const int per = (channels + n_blocks - 1) / n_blocks;
+    for (int i = 0; i < stream_count; i++) {
+        int best = 0;
+        float bv = -INFINITY;
+        bool any = false;
+        for (int b = 0; b < n_blocks; b++) {
+            const int lo = b * per, hi = lo + per < channels ? lo + per : channels;
+            if (lo >= hi) break;
+            int bi = 0;
+            float v = 0.0f;
+            esp_interop_argmax_f16_strided(s + (size_t)(ch_off + lo) * spatial + i, hi - lo, spatial, &bi, &v);
+            if (!any || v > bv) { bv = v; best = lo + bi; any = true; }   // strict >: an earlier block keeps a tie
+        }
+        out_indices[i] = best;
+        out_values[i] = bv;
+    }
+    return true;
+}
+bool esp_interop_io_argmax_batch_fp16_spatial_nolock(ESPSurfaceRef surface, int ch_off, int spatial, int channels, int stream_count, int *out_indices,
+                                                     float *out_values, int n_blocks) {
+    // "assumes the surface is already coherent": the host shadow is read as it is when it is current, else it is fetched
+    return esp_interop_io_argmax_batch_fp16_spatial_parallel(surface, ch_off, spatial, channels, stream_count, out_indices, out_values, n_blocks);
+}
+
+// ane_interop_fused_expansion_argmax_fp16 (surface_io.c:1438-1520, :1521-1700): logit[c][s] = sum_k proj[g * cpg + k][s] * w[c][k] with
+// g = c / (vocab / groups), accumulated in fp16 with a fused multiply-add per term as the NEON code does, strict > across
+// channels.  The same argument checks: vocab <= 65535, spatial a multiple of 8, bottleneck and vocab multiples of groups.
+bool esp_interop_fused_expansion_argmax_fp16(ESPSurfaceRef proj_surface, int proj_ch_off, int spatial, int bottleneck, int groups,
+                                             const void *expansion_weights_fp16, int vocab_size, int stream_count, int *out_indices, float *out_values,
+                                             int n_blocks) {
+    (void)n_blocks;   // the partition only spreads work over cores in the reference; the result does not depend on it
+    if (!proj_surface || !expansion_weights_fp16 || !out_indices || !out_values) return false;
+    if (proj_ch_off < 0 || spatial <= 0 || bottleneck <= 0 || groups <= 0 || vocab_size <= 0) return false;
+    if (stream_count <= 0 || stream_count > spatial || vocab_size > 65535) return false;
+    if (spatial > 32768 || spatial % 8 != 0 || bottleneck % groups != 0 || vocab_size % groups != 0) return false;
+    if (!region_ok(proj_surface, proj_ch_off, bottleneck, spatial)) return false;
+    const uint16_t *proj = shadow_for_read(proj_surface);
+    if (!proj) return false;
+    const _Float16 *w = static_cast<const _Float16 *>(expansion_weights_fp16);
+    const int cpg = bottleneck / groups, ch_per_group = vocab_size / groups;
+    for (int s = 0; s < stream_count; s++) {
+        _Float16 best = (_Float16)(-65504.0f);
+        int best_i = 0;
+        for (int c = 0; c < vocab_size; c++) {
+            const int g = c / ch_per_group;
+            _Float16 acc = (_Float16)0.0f;
+            for (int k = 0; k < cpg; k++) {
+                const _Float16 p = __builtin_bit_cast(_Float16, proj[(size_t)(proj_ch_off + g * cpg + k) * spatial + s]);
+                acc = (_Float16)((double)w[(size_t)c * cpg + k] * (double)p + (double)acc);   // one rounding per term: fp16 fused multiply-add
+            }
+            if (acc > best) { best = acc; best_i = c; }
+        }
+        out_indices[s] = best_i;
+        out_values[s] = (float)best;
+    }
     return true;
 }
 

@@ -26,6 +26,73 @@ __global__ void scatter_columns_kernel(const float *in, int channels, int spatia
     surface[(size_t)c * spatial + l] = f2h(in[(size_t)l * channels + c]);
 }
 
+__global__ void scatter_columns_strided_kernel(const float *in, int in_stride, int channels, int spatial, int lanes, uint16_t *surface) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, l = blockIdx.y;
+    if (c >= channels || l >= lanes) return;
+    surface[(size_t)c * spatial + l] = f2h(in[(size_t)l * in_stride + c]);
+}
+
+// rope_decode (MetalAttentionKernel.swift:1756-1795): pairs (d, d + headDim/2), freq = theta^(-pair / half), fp16 in and out
+__global__ void surface_rope_kernel(uint16_t *q, uint16_t *k, int n_heads, int n_kv_heads, int head_dim, int position, float theta, int lane_stride) {
+    const int pair = blockIdx.x * blockDim.x + threadIdx.x, head = blockIdx.y, half = head_dim / 2;
+    if (pair >= half) return;
+    const float freq = powf(theta, -(float)pair / (float)half);
+    const float angle = (float)position * freq;
+    const float c = cosf(angle), sn = sinf(angle);
+    auto rotate = [&](uint16_t *t) {
+        const size_t i0 = (size_t)(head * head_dim + pair) * lane_stride, i1 = (size_t)(head * head_dim + pair + half) * lane_stride;
+        const float v0 = h2f(t[i0]), v1 = h2f(t[i1]);
+        t[i0] = f2h(__fsub_rn(__fmul_rn(v0, c), __fmul_rn(v1, sn)));
+        t[i1] = f2h(__fadd_rn(__fmul_rn(v0, sn), __fmul_rn(v1, c)));
+    };
+    if (head < n_heads) rotate(q);
+    if (head < n_kv_heads) rotate(k);
+}
+
+__global__ void surface_kv_scatter_kernel(const uint16_t *k_src, const uint16_t *v_src, uint16_t *k_cache, uint16_t *v_cache, int kv_dim, int token_index,
+                                          int cache_stride, int lane_stride) {
+    const int ch = blockIdx.x * blockDim.x + threadIdx.x;
+    if (ch >= kv_dim) return;
+    k_cache[(size_t)ch * cache_stride + token_index] = k_src[(size_t)ch * lane_stride];
+    v_cache[(size_t)ch * cache_stride + token_index] = v_src[(size_t)ch * lane_stride];
+}
+
+// fused_decode_sdpa (MetalAttentionKernel.swift:1824-1886): one workgroup per query head; scores over the visible tokens in
+// LDS, max-subtracted softmax, weighted sum of V per channel.  kvHead = head / (heads / kvHeads).
+__global__ __launch_bounds__(256) void surface_sdpa_kernel(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *context, int heads,
+                                                           int kv_heads, int head_dim, int visible, int token_base, int cache_stride, int lane_stride) {
+    extern __shared__ float scores[];   // [visible] + 256 for the reductions
+    float *red = scores + visible;
+    const int head = blockIdx.x, tid = threadIdx.x, kv_head = head / (heads / kv_heads);
+    const float scale = 1.0f / sqrtf((float)head_dim);
+    for (int t = tid; t < visible; t += 256) {
+        float dot = 0.0f;
+        for (int d = 0; d < head_dim; d++)
+            dot += h2f(q[(size_t)(head * head_dim + d) * lane_stride]) * h2f(k_cache[(size_t)(kv_head * head_dim + d) * cache_stride + token_base + t]);
+        scores[t] = dot * scale;
+    }
+    __syncthreads();
+    float m = -INFINITY;
+    for (int t = tid; t < visible; t += 256) m = fmaxf(m, scores[t]);
+    red[tid] = m;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) { if (tid < s) red[tid] = fmaxf(red[tid], red[tid + s]); __syncthreads(); }
+    m = red[0];
+    __syncthreads();
+    float sum = 0.0f;
+    for (int t = tid; t < visible; t += 256) { const float e = expf(scores[t] - m); scores[t] = e; sum += e; }
+    red[tid] = sum;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) { if (tid < s) red[tid] += red[tid + s]; __syncthreads(); }
+    const float inv = red[0] > 0.0f ? 1.0f / red[0] : 0.0f;
+    for (int d = tid; d < head_dim; d += 256) {
+        const uint16_t *v = v_cache + (size_t)(kv_head * head_dim + d) * cache_stride + token_base;
+        float acc = 0.0f;
+        for (int t = 0; t < visible; t++) acc += (scores[t] * inv) * h2f(v[t]);
+        context[(size_t)(head * head_dim + d) * lane_stride] = f2h(acc);
+    }
+}
+
 // surface[l] = fp16(max_c in[l][c]) — the reduce_max output of the classifier kernel
 __global__ __launch_bounds__(256) void row_max_kernel(const float *in, int channels, int spatial, uint16_t *surface) {
     __shared__ float red[256];
@@ -50,6 +117,29 @@ hipError_t launch_gather_columns(const uint16_t *surface, int channels, int spat
 }
 hipError_t launch_scatter_columns(const float *in, int channels, int spatial, int lanes, uint16_t *surface, hipStream_t s) {
     hipLaunchKernelGGL(scatter_columns_kernel, dim3((channels + 255) / 256, lanes), dim3(256), 0, s, in, channels, spatial, lanes, surface);
+    return hipGetLastError();
+}
+hipError_t launch_scatter_columns_strided(const float *in, int in_stride, int channels, int spatial, int lanes, uint16_t *surface, hipStream_t s) {
+    hipLaunchKernelGGL(scatter_columns_strided_kernel, dim3((channels + 255) / 256, lanes), dim3(256), 0, s, in, in_stride, channels, spatial, lanes, surface);
+    return hipGetLastError();
+}
+hipError_t launch_surface_rope(uint16_t *q, uint16_t *k, int n_heads, int n_kv_heads, int head_dim, int position, float theta, int lane_stride, hipStream_t s) {
+    const int half = head_dim / 2, heads = n_heads > n_kv_heads ? n_heads : n_kv_heads;
+    hipLaunchKernelGGL(surface_rope_kernel, dim3((half + 63) / 64, heads), dim3(64), 0, s, q, k, n_heads, n_kv_heads, head_dim, position, theta, lane_stride);
+    return hipGetLastError();
+}
+hipError_t launch_surface_kv_scatter(const uint16_t *k_src, const uint16_t *v_src, uint16_t *k_cache, uint16_t *v_cache, int kv_dim, int token_index,
+                                     int cache_stride, int lane_stride, hipStream_t s) {
+    hipLaunchKernelGGL(surface_kv_scatter_kernel, dim3((kv_dim + 255) / 256), dim3(256), 0, s, k_src, v_src, k_cache, v_cache, kv_dim, token_index, cache_stride,
+                       lane_stride);
+    return hipGetLastError();
+}
+hipError_t launch_surface_sdpa(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *context, int heads, int kv_heads, int head_dim,
+                               int visible_tokens, int token_base, int cache_stride, int lane_stride, hipStream_t s) {
+    const size_t lds = ((size_t)visible_tokens + 256) * 4;
+    if (lds > 64 * 1024) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(surface_sdpa_kernel, dim3(heads), dim3(256), lds, s, q, k_cache, v_cache, context, heads, kv_heads, head_dim, visible_tokens, token_base,
+                       cache_stride, lane_stride);
     return hipGetLastError();
 }
 hipError_t launch_row_max(const float *in, int channels, int spatial, int lanes, uint16_t *surface, hipStream_t s) {

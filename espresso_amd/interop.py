@@ -57,6 +57,19 @@ def _L() -> C.CDLL:
         "esp_interop_io_write_fp16_at": (b, [vp, i32, vp, i32, i32]),
         "esp_interop_io_write_embedding_batch_fp16": (b, [vp, i32, i32, vp, i32, i32, vp, i32]),
         "esp_interop_io_argmax_batch_fp16_spatial": (b, [vp, i32, i32, i32, i32, ip, fp]),
+        "esp_interop_io_copy_two_fp16_spatial_slices": (b, [vp, i32, i32, i32, vp, i32, i32, i32, vp, i32, i32, i32, vp, i32, i32, i32, i32]),
+        "esp_interop_io_argmax_fp16_spatial_slice_with_hint": (b, [vp, i32, i32, i32, i32, vp, i32, i32, ip, fp]),
+        "esp_interop_io_write_fp16_at_batched": (b, [vp, ip, C.POINTER(vp), ip, i32, i32]),
+        "esp_interop_io_copy_batched": (b, [vp, vp, ip, ip, ip, i32, i32]),
+        "esp_interop_io_copy_multi_src": (b, [vp, C.POINTER(vp), ip, ip, ip, i32, i32]),
+        "esp_interop_io_argmax_batch_fp16_spatial_parallel": (b, [vp, i32, i32, i32, i32, ip, fp, i32]),
+        "esp_interop_io_argmax_batch_fp16_spatial_nolock": (b, [vp, i32, i32, i32, i32, ip, fp, i32]),
+        "esp_interop_fused_expansion_argmax_fp16": (b, [vp, i32, i32, i32, i32, vp, i32, i32, ip, fp, i32]),
+        "esp_interop_gather_f16_to_f32": (None, [vp, vp, i32, i32]),
+        "esp_interop_scatter_f32_to_f16": (None, [vp, vp, i32, i32]),
+        "esp_interop_rope_decode": (b, [vp, vp, i32, i32, i32, i32, C.c_float, i32]),
+        "esp_interop_kv_cache_scatter": (b, [vp, vp, vp, vp, i32, i32, i32, i32]),
+        "esp_interop_decode_sdpa": (b, [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32]),
         "esp_interop_io_lock_write": (b, [vp]),
         "esp_interop_io_unlock_write": (b, [vp]),
         "esp_interop_io_lock_read": (b, [vp]),
@@ -184,6 +197,123 @@ class SurfaceIO:
         val = (C.c_float * max(streamCount, 1))()
         _ok(_L().esp_interop_io_argmax_batch_fp16_spatial(from_.ref, channelOffset, spatial, channels, streamCount, idx, val), "argmaxBatchFP16Spatial")
         return list(idx[:streamCount]), list(val[:streamCount])
+
+
+    @staticmethod
+    def copyTwoFP16SpatialSlices(dst0: Surface, dst0ChannelOffset: int, dst0SpatialIndex: int, dst0Spatial: int, src0: Surface, src0ChannelOffset: int,
+                                 src0SpatialIndex: int, src0Spatial: int, dst1: Surface, dst1ChannelOffset: int, dst1SpatialIndex: int, dst1Spatial: int,
+                                 src1: Surface, src1ChannelOffset: int, src1SpatialIndex: int, src1Spatial: int, channels: int) -> None:
+        """SurfaceIO.swift:285-339."""
+        _ok(_L().esp_interop_io_copy_two_fp16_spatial_slices(
+            dst0.ref, dst0ChannelOffset, dst0SpatialIndex, dst0Spatial, src0.ref, src0ChannelOffset, src0SpatialIndex, src0Spatial,
+            dst1.ref, dst1ChannelOffset, dst1SpatialIndex, dst1Spatial, src1.ref, src1ChannelOffset, src1SpatialIndex, src1Spatial, channels),
+            "copyTwoFP16SpatialSlices")
+
+    @staticmethod
+    def argmaxFP16SpatialSliceWithHint(from_: Surface, channelOffset: int, spatialIndex: int, spatial: int, channels: int, hint: Surface,
+                                       hintSpatialIndex: int, hintSpatial: int) -> tuple[int, float]:
+        """SurfaceIO.swift:433-474: the hint surface holds the column's maximum (the classifier kernel's second output)."""
+        idx, val = C.c_int(-1), C.c_float(0)
+        _ok(_L().esp_interop_io_argmax_fp16_spatial_slice_with_hint(from_.ref, channelOffset, spatialIndex, spatial, channels, hint.ref, hintSpatialIndex,
+                                                                   hintSpatial, C.byref(idx), C.byref(val)), "argmaxFP16SpatialSliceWithHint")
+        return idx.value, val.value
+
+    @staticmethod
+    def writeFP16AtBatched(to: Surface, spatial: int, regions) -> None:
+        """regions: (channelOffset, data, channels) triples (SurfaceIO.swift:190-229); all are checked before any is written."""
+        keep = [np.ascontiguousarray(d, dtype=np.float32) for _, d, _ in regions]
+        n = len(regions)
+        offs = (C.c_int * max(n, 1))(*[r[0] for r in regions])
+        chans = (C.c_int * max(n, 1))(*[r[2] for r in regions])
+        for a, (_, _, ch) in zip(keep, regions):
+            if a.size != ch * spatial:
+                raise SurfaceIOError("writeFP16AtBatched: data size does not match channels x spatial")
+        srcs = (C.c_void_p * max(n, 1))(*[a.ctypes.data for a in keep])
+        _ok(_L().esp_interop_io_write_fp16_at_batched(to.ref, offs, srcs, chans, n, spatial), "writeFP16AtBatched")
+
+    @staticmethod
+    def copyFP16Batched(dst: Surface, src: Surface, spatial: int, regions) -> None:
+        """regions: (dstChannelOffset, srcChannelOffset, channels) triples (SurfaceIO.swift:672-716)."""
+        n = len(regions)
+        d = (C.c_int * max(n, 1))(*[r[0] for r in regions])
+        s = (C.c_int * max(n, 1))(*[r[1] for r in regions])
+        c = (C.c_int * max(n, 1))(*[r[2] for r in regions])
+        _ok(_L().esp_interop_io_copy_batched(dst.ref, src.ref, d, s, c, n, spatial), "copyFP16Batched")
+
+    @staticmethod
+    def copyFP16FromMultipleSources(dst: Surface, spatial: int, regions) -> None:
+        """regions: (source, dstChannelOffset, srcChannelOffset, channels) (SurfaceIO.swift:783-828)."""
+        n = len(regions)
+        srcs = (C.c_void_p * max(n, 1))(*[r[0].ref for r in regions])
+        d = (C.c_int * max(n, 1))(*[r[1] for r in regions])
+        s = (C.c_int * max(n, 1))(*[r[2] for r in regions])
+        c = (C.c_int * max(n, 1))(*[r[3] for r in regions])
+        _ok(_L().esp_interop_io_copy_multi_src(dst.ref, srcs, d, s, c, n, spatial), "copyFP16FromMultipleSources")
+
+    @staticmethod
+    def _argmax_blocks(fn, what, from_, channelOffset, spatial, channels, streamCount, nBlocks):
+        idx = (C.c_int * max(streamCount, 1))()
+        val = (C.c_float * max(streamCount, 1))()
+        _ok(fn(from_.ref, channelOffset, spatial, channels, streamCount, idx, val, nBlocks), what)
+        return list(idx[:streamCount]), list(val[:streamCount])
+
+    @staticmethod
+    def argmaxBatchFP16SpatialParallel(from_: Surface, channelOffset: int, spatial: int, channels: int, streamCount: int, nBlocks: int = 4):
+        """SurfaceIO.swift:542-578."""
+        return SurfaceIO._argmax_blocks(_L().esp_interop_io_argmax_batch_fp16_spatial_parallel, "argmaxBatchFP16SpatialParallel", from_, channelOffset,
+                                        spatial, channels, streamCount, nBlocks)
+
+    @staticmethod
+    def argmaxBatchFP16SpatialNolock(from_: Surface, channelOffset: int, spatial: int, channels: int, streamCount: int, nBlocks: int = 4):
+        """SurfaceIO.swift:580-615."""
+        return SurfaceIO._argmax_blocks(_L().esp_interop_io_argmax_batch_fp16_spatial_nolock, "argmaxBatchFP16SpatialNolock", from_, channelOffset,
+                                        spatial, channels, streamCount, nBlocks)
+
+    @staticmethod
+    def fusedExpansionArgmax(projSurface: Surface, projChannelOffset: int, spatial: int, bottleneck: int, groups: int, expansionWeights, vocabSize: int,
+                             streamCount: int, nBlocks: int = 4):
+        """SurfaceIO.swift:617-670; expansionWeights: fp16 bits [vocab, bottleneck / groups]."""
+        w = np.ascontiguousarray(expansionWeights, dtype=np.uint16)
+        if groups <= 0 or bottleneck % groups != 0 or w.size != vocabSize * (bottleneck // groups):
+            raise SurfaceIOError("fusedExpansionArgmax: weight count does not match vocab x bottleneck / groups")
+        idx = (C.c_int * max(streamCount, 1))()
+        val = (C.c_float * max(streamCount, 1))()
+        _ok(_L().esp_interop_fused_expansion_argmax_fp16(projSurface.ref, projChannelOffset, spatial, bottleneck, groups, _ptr(w), vocabSize, streamCount,
+                                                         idx, val, nBlocks), "fusedExpansionArgmax")
+        return list(idx[:streamCount]), list(val[:streamCount])
+
+
+def gather_f16_to_f32(bits, count: int, stride: int) -> np.ndarray:
+    a = np.ascontiguousarray(bits, dtype=np.uint16)
+    assert count == 0 or (count - 1) * stride < a.size
+    out = np.empty(count, dtype=np.float32)
+    _L().esp_interop_gather_f16_to_f32(_ptr(out), _ptr(a), count, stride)
+    return out
+
+
+def scatter_f32_to_f16(dst_bits: np.ndarray, values, stride: int) -> None:
+    v = np.ascontiguousarray(values, dtype=np.float32)
+    assert dst_bits.dtype == np.uint16 and dst_bits.flags.c_contiguous and (v.size == 0 or (v.size - 1) * stride < dst_bits.size)
+    _L().esp_interop_scatter_f32_to_f16(_ptr(dst_bits), _ptr(v), v.size, stride)
+
+
+def rope_decode(q: Surface, k: Surface, nHeads: int, nKVHeads: int, headDim: int, position: int, theta: float, laneSpatial: int) -> None:
+    """rope_decode of the hybrid decode path (MetalAttentionKernel.swift:1756-1795) on surfaces resident on the device."""
+    if not _L().esp_interop_rope_decode(q.ref, k.ref, nHeads, nKVHeads, headDim, position, theta, laneSpatial):
+        raise ANEError("evaluationFailed", "rope_decode: " + _lib.last_error())
+
+
+def kv_cache_scatter(kSrc: Surface, vSrc: Surface, kCache: Surface, vCache: Surface, kvDim: int, tokenIndex: int, cacheStride: int, laneSpatial: int) -> None:
+    """kv_cache_scatter (MetalAttentionKernel.swift:1805-1820)."""
+    if not _L().esp_interop_kv_cache_scatter(kSrc.ref, vSrc.ref, kCache.ref, vCache.ref, kvDim, tokenIndex, cacheStride, laneSpatial):
+        raise ANEError("evaluationFailed", "kv_cache_scatter: " + _lib.last_error())
+
+
+def decode_sdpa(q: Surface, kCache: Surface, vCache: Surface, context: Surface, heads: int, kvHeads: int, headDim: int, visibleTokens: int, tokenBase: int,
+                cacheStride: int, laneSpatial: int) -> None:
+    """fused_decode_sdpa (MetalAttentionKernel.swift:1824-1886)."""
+    if not _L().esp_interop_decode_sdpa(q.ref, kCache.ref, vCache.ref, context.ref, heads, kvHeads, headDim, visibleTokens, tokenBase, cacheStride, laneSpatial):
+        raise ANEError("evaluationFailed", "decode_sdpa: " + _lib.last_error())
 
 
 def cvt_f32_to_f16(values) -> np.ndarray:

@@ -590,7 +590,7 @@ size_t esp_surface_bytes(ESPSurfaceRef surface);                 /* IOSurfaceGet
 /* ane_interop_compile (:24-28).  `program` is a text description of one HIP kernel set instead of MIL
  * text: "key: value" lines, e.g.
  *     program: espresso.hip/1
- *     kernel: gemv            (gemv | rmsnorm_classifier | decode_ffn)
+ *     kernel: gemv            (gemv | rmsnorm_classifier | decode_ffn | decode_qkv | decode_projection)
  *     format: q8_0            (f32 | f16 | q4_0 | q8_0 | q4_k; weight matrices)
  *     rows: 768  cols: 768    (gemv)   dim / hidden (decode_ffn)   dim / vocab (rmsnorm_classifier)
  *     spatial: 32             (surface width S; a decode token lives in column 0, DecodeKernelSet.swift:10)
@@ -601,7 +601,13 @@ size_t esp_surface_bytes(ESPSurfaceRef surface);                 /* IOSurfaceGet
  * blocks of `format`, or a BLOBFILE when format is f16; norm vectors are BLOBFILEs.  The bytes are copied
  * during the call.  Surfaces: gemv in [cols,S] -> out [rows,S]; rmsnorm_classifier in [dim,S] -> logits
  * [vocab,S], max [1,S] (GenerationRMSNormClassifierGenerator.swift:27-63); decode_ffn in [dim,S] -> [dim,S]
- * computing x + W2(silu(W1 n) * W3 n), n = rmsnorm(x) (DecodeFFNGenerator.swift:40-91). */
+ * computing x + W2(silu(W1 n) * W3 n), n = rmsnorm(x) (DecodeFFNGenerator.swift:40-91).
+ * decode_qkv (dim, q_dim, kv_dim; weights rms_att, wq, wk, wv): in [dim,S] -> k [kv_dim,S] @ 0, q [q_dim,S] @ 1, v [kv_dim,S] @ 2,
+ * the output order of the reference's decodeQKVOnly kernel (DecodeForwardPass.swift:374-377; DecodeAttentionQKVGenerator.swift:86-131):
+ * rmsnorm and the three projections, no RoPE.  decode_projection (dim, q_dim; weight wo): context [q_dim,S] @ 0 and residual
+ * [dim,S] @ 1 -> residual + Wo context [dim,S]; the reference rebinds input 1 to the layer's input surface
+ * (DecodeForwardPass.swift:383,396).  Together with decode_ffn and the three calls below these run one layer of
+ * HybridDecodeKernelSet (Sources/ANERuntime/HybridDecodeKernelSet.swift:30-56) handle by handle. */
 ESPHandle *esp_interop_compile(const uint8_t *program, size_t program_len,
                                const char **weight_paths, const uint8_t **weight_datas,
                                const size_t *weight_lens, int weight_count,
@@ -622,11 +628,25 @@ uint64_t esp_interop_last_hw_execution_time_ns(ESPHandle *handle);          /* :
 bool esp_interop_has_perf_stats(ESPHandle *handle);                         /* :43 */
 bool esp_interop_rebind_input(ESPHandle *handle, int index, ESPSurfaceRef new_surface);   /* :50 */
 
+/* Between the kernel evaluations of a hybrid decode layer the reference runs Metal kernels on the same surfaces
+ * (Sources/Espresso/MetalAttentionKernel.swift); these are their counterparts on surfaces resident in HBM, synchronous:
+ *   rope_decode       :1756-1795  half-split RoPE in place on lane 0 of q [heads*D, S] and k [kvHeads*D, S]
+ *   kv_cache_scatter  :1805-1820  lane 0 of k / v into column token_index of the caches [kvDim, cacheStride]
+ *   decode_sdpa       :1824-1886  fused_decode_sdpa: softmax(q K / sqrt(D)) V over columns token_base .. +visible of the caches into
+ *                                 lane 0 of the context surface [heads*D, S] (fp16; kvHead = head / (heads / kvHeads)) */
+bool esp_interop_rope_decode(ESPSurfaceRef q, ESPSurfaceRef k, int n_heads, int n_kv_heads, int head_dim, int position, float theta, int lane_spatial);
+bool esp_interop_kv_cache_scatter(ESPSurfaceRef k_src, ESPSurfaceRef v_src, ESPSurfaceRef k_cache, ESPSurfaceRef v_cache, int kv_dim, int token_index,
+                                  int cache_stride, int lane_spatial);
+bool esp_interop_decode_sdpa(ESPSurfaceRef q, ESPSurfaceRef k_cache, ESPSurfaceRef v_cache, ESPSurfaceRef context, int heads, int kv_heads, int head_dim,
+                             int visible_tokens, int token_base, int cache_stride, int lane_spatial);
+
 void esp_interop_cvt_f32_to_f16(void *dst, const float *src, int count);    /* :143, round to nearest even */
 void esp_interop_cvt_f16_to_f32(float *dst, const void *src, int count);    /* :144 */
 /* First-max argmax over fp16 values: lowest index wins ties (:146-156, neon_convert.c:36-101). */
 void esp_interop_argmax_f16(const void *src, int count, int *out_index, float *out_value);
 void esp_interop_argmax_f16_strided(const void *src, int count, int stride, int *out_index, float *out_value);
+void esp_interop_gather_f16_to_f32(float *dst, const void *src, int count, int stride);      /* :160 */
+void esp_interop_scatter_f32_to_f16(void *dst, const float *src, int count, int stride);     /* :165 */
 
 /* Surface I/O (:168-348): fp32 on the caller's side, fp16 on the surface; all return false on a
  * range error instead of touching memory. */
@@ -649,6 +669,28 @@ bool esp_interop_io_write_embedding_batch_fp16(ESPSurfaceRef surface, int ch_off
                                                int vocab_size, int dim, const uint16_t *token_ids, int stream_count);      /* :270 */
 bool esp_interop_io_argmax_batch_fp16_spatial(ESPSurfaceRef surface, int ch_off, int spatial, int channels, int stream_count,
                                               int *out_indices, float *out_values);                                        /* :282 */
+bool esp_interop_io_copy_two_fp16_spatial_slices(ESPSurfaceRef dst0, int dst0_ch_off, int dst0_spatial_index, int dst0_spatial, ESPSurfaceRef src0,
+                                                 int src0_ch_off, int src0_spatial_index, int src0_spatial, ESPSurfaceRef dst1, int dst1_ch_off,
+                                                 int dst1_spatial_index, int dst1_spatial, ESPSurfaceRef src1, int src1_ch_off, int src1_spatial_index,
+                                                 int src1_spatial, int channels);                                              /* :184 */
+bool esp_interop_io_argmax_fp16_spatial_slice_with_hint(ESPSurfaceRef surface, int ch_off, int spatial_index, int spatial, int channels,
+                                                        ESPSurfaceRef hint_surface, int hint_spatial_index, int hint_spatial, int *out_index,
+                                                        float *out_value);                                                    /* :224 */
+bool esp_interop_io_write_fp16_at_batched(ESPSurfaceRef surface, const int *channel_offsets, const float *const *sources, const int *channels,
+                                          int region_count, int spatial);                                                     /* :246 */
+bool esp_interop_io_copy_batched(ESPSurfaceRef dst, ESPSurfaceRef src, const int *dst_channel_offsets, const int *src_channel_offsets,
+                                 const int *channels, int region_count, int spatial);                                         /* :252 */
+bool esp_interop_io_copy_multi_src(ESPSurfaceRef dst, const ESPSurfaceRef *sources, const int *dst_channel_offsets, const int *src_channel_offsets,
+                                   const int *channels, int region_count, int spatial);                                       /* :259 */
+bool esp_interop_io_argmax_batch_fp16_spatial_parallel(ESPSurfaceRef surface, int ch_off, int spatial, int channels, int stream_count,
+                                                       int *out_indices, float *out_values, int n_blocks);                    /* :294 */
+bool esp_interop_io_argmax_batch_fp16_spatial_nolock(ESPSurfaceRef surface, int ch_off, int spatial, int channels, int stream_count,
+                                                     int *out_indices, float *out_values, int n_blocks);                      /* :306 */
+/* :320; the factored output head's expansion + argmax on the host: fp16 fused multiply-adds in channel order, first maximum,
+ * vocab <= 65535, spatial a multiple of 8 (surface_io.c:1438-1700).  Parity unpinned: the reference holds no vector for it. */
+bool esp_interop_fused_expansion_argmax_fp16(ESPSurfaceRef proj_surface, int proj_ch_off, int spatial, int bottleneck, int groups,
+                                             const void *expansion_weights_fp16, int vocab_size, int stream_count, int *out_indices,
+                                             float *out_values, int n_blocks);
 bool esp_interop_io_lock_write(ESPSurfaceRef surface);                                                                     /* :335 */
 bool esp_interop_io_unlock_write(ESPSurfaceRef surface);
 bool esp_interop_io_lock_read(ESPSurfaceRef surface);

@@ -146,3 +146,135 @@ def test_compile_errors_eval_failure_hook_and_rebind(io):
     with pytest.raises(io.ANEError):
         k.rebindInput(0, io.Surface.create(64))                      # wrong size
     k.free()
+
+
+def test_decode_qkv_outputs_k_q_v_in_the_reference_order(io):
+    """decodeQKVOnly's outputs are k @ 0, q @ 1, v @ 2 (DecodeForwardPass.swift:374-377); grouped-query shapes."""
+    dim, q_dim, kv_dim, spatial, lanes = 512, 512, 128, 32, 2
+    rng = np.random.default_rng(41)
+    bq, wq = _matrix("q4_k", q_dim, dim, rng)
+    bk, wk = _matrix("q4_k", kv_dim, dim, rng)
+    bv, wv = _matrix("q4_k", kv_dim, dim, rng)
+    gamma = (1.0 + rng.normal(0, 0.1, dim)).astype(np.float32)
+    k = io.ANEKernel(io.program_text("decode_qkv", "q4_k", spatial, lanes, dim=dim, q_dim=q_dim, kv_dim=kv_dim),
+                     [("@model_path/weights/rms_att.bin", orc.blob_build(gamma)), ("@model_path/weights/wq.bin", bq),
+                      ("@model_path/weights/wk.bin", bk), ("@model_path/weights/wv.bin", bv)],
+                     [dim * spatial * 2], [kv_dim * spatial * 2, q_dim * spatial * 2, kv_dim * spatial * 2])
+    x = rng.normal(0, 1, (dim, spatial)).astype(np.float32)
+    io.SurfaceIO.writeFP16(k.inputSurface(0), x, dim, spatial)
+    k.eval()
+    for out_index, w, rows in ((0, wk, kv_dim), (1, wq, q_dim), (2, wv, kv_dim)):
+        got = io.SurfaceIO.readFP16(k.outputSurface(out_index), 0, rows, spatial)
+        for lane in range(lanes):
+            n = _f16(orc.rmsnorm(_f16(x[:, lane]), _f16(gamma), 1e-5))
+            _fp16_close(got[:, lane], orc.matvec(w, n), extra=1e-3)
+        assert np.all(got[:, lanes:] == 0)
+    with pytest.raises(io.ANEError, match="invalidArguments"):      # the surfaces in q, k, v order are not what the kernel has
+        io.ANEKernel(io.program_text("decode_qkv", "q4_k", spatial, lanes, dim=dim, q_dim=q_dim, kv_dim=kv_dim),
+                     [("rms_att.bin", orc.blob_build(gamma)), ("wq.bin", bq), ("wk.bin", bk), ("wv.bin", bv)],
+                     [dim * spatial * 2], [q_dim * spatial * 2, kv_dim * spatial * 2, kv_dim * spatial * 2])
+    k.free()
+
+
+def test_rope_scatter_and_sdpa_on_surfaces_match_the_oracle(io):
+    """rope_decode, kv_cache_scatter and fused_decode_sdpa (MetalAttentionKernel.swift:1756-1886) on channel-first surfaces."""
+    heads, kv_heads, hd, lane, stride = 8, 2, 64, 32, 48
+    q_dim, kv_dim = heads * hd, kv_heads * hd
+    rng = np.random.default_rng(42)
+    q, kk = io.Surface.create(q_dim * lane * 2), io.Surface.create(kv_dim * lane * 2)
+    v = io.Surface.create(kv_dim * lane * 2)
+    kc, vc, ctx = io.Surface.create(kv_dim * stride * 2), io.Surface.create(kv_dim * stride * 2), io.Surface.create(q_dim * lane * 2)
+    k_rows, v_rows = [], []
+    for pos in range(37):
+        qv, kv_, vv = (rng.normal(0, 1, n).astype(np.float32) for n in (q_dim, kv_dim, kv_dim))
+        io.SurfaceIO.writeFP16SpatialSlice(q, 0, 0, lane, qv, q_dim)
+        io.SurfaceIO.writeFP16SpatialSlice(kk, 0, 0, lane, kv_, kv_dim)
+        io.SurfaceIO.writeFP16SpatialSlice(v, 0, 0, lane, vv, kv_dim)
+        io.rope_decode(q, kk, heads, kv_heads, hd, pos, 10000.0, lane)
+        q_rot = io.SurfaceIO.readFP16SpatialSlice(q, 0, 0, lane, q_dim)
+        k_rot = io.SurfaceIO.readFP16SpatialSlice(kk, 0, 0, lane, kv_dim)
+        _fp16_close(q_rot, orc.rope_half_split(_f16(qv), heads, hd, pos, 10000.0), extra=2e-3)
+        _fp16_close(k_rot, orc.rope_half_split(_f16(kv_), kv_heads, hd, pos, 10000.0), extra=2e-3)
+        io.kv_cache_scatter(kk, v, kc, vc, kv_dim, pos, stride, lane)
+        k_rows.append(k_rot); v_rows.append(_f16(vv))
+        assert np.array_equal(io.SurfaceIO.readFP16SpatialSlice(kc, 0, pos, stride, kv_dim), k_rot)
+        assert np.array_equal(io.SurfaceIO.readFP16SpatialSlice(vc, 0, pos, stride, kv_dim), _f16(vv))
+        if pos in (0, 1, 17, 36):
+            io.decode_sdpa(q, kc, vc, ctx, heads, kv_heads, hd, pos + 1, 0, stride, lane)
+            got = io.SurfaceIO.readFP16SpatialSlice(ctx, 0, 0, lane, q_dim)
+            K, V = np.stack(k_rows), np.stack(v_rows)                     # [tokens, kv_dim]
+            want = np.empty(q_dim, np.float32)
+            for h in range(heads):
+                g = h // (heads // kv_heads)
+                sc = (K[:, g * hd:(g + 1) * hd] @ q_rot[h * hd:(h + 1) * hd]) / np.sqrt(np.float32(hd))
+                p = np.exp(sc - sc.max()); p /= p.sum()
+                want[h * hd:(h + 1) * hd] = p @ V[:, g * hd:(g + 1) * hd]
+            _fp16_close(got, want, extra=1e-3)
+    # a window that starts past column 0: tokens 30..36 only
+    io.decode_sdpa(q, kc, vc, ctx, heads, kv_heads, hd, 7, 30, stride, lane)
+    got = io.SurfaceIO.readFP16SpatialSlice(ctx, 0, 0, lane, q_dim)
+    K, V = np.stack(k_rows[30:]), np.stack(v_rows[30:])
+    sc = (K[:, :hd] @ q_rot[:hd]) / np.sqrt(np.float32(hd))
+    p = np.exp(sc - sc.max()); p /= p.sum()
+    _fp16_close(got[:hd], p @ V[:, :hd], extra=1e-3)
+    with pytest.raises(io.ANEError):
+        io.decode_sdpa(q, kc, vc, ctx, heads, kv_heads, hd, 20, 30, stride, lane)      # window runs past the cache
+    with pytest.raises(io.ANEError):
+        io.kv_cache_scatter(kk, v, kc, vc, kv_dim, stride, stride, lane)               # token index past the cache
+    with pytest.raises(io.ANEError):
+        io.rope_decode(q, kk, heads + 1, kv_heads, hd, 0, 10000.0, lane)               # more heads than the surface holds
+
+
+@pytest.mark.parametrize("name,shape", [
+    ("q8_0", dict(n_layer=1, n_head=12, n_kv_head=12, d_model=768, head_dim=64, hidden_dim=2048, vocab=2048, max_seq=64)),
+    ("q4_k", dict(n_layer=1, n_head=8, n_kv_head=2, d_model=512, head_dim=64, hidden_dim=1024, vocab=1024, max_seq=64, rope_theta=500000.0)),
+])
+def test_one_layer_handle_by_handle_matches_the_runtime(io, name, shape):
+    """The hybrid decode layer as the reference's DecodeForwardPass runs it (DecodeForwardPass.swift:360-400): decodeQKVOnly,
+    rope_decode, kv_cache_scatter, fused_decode_sdpa, decodeProjection with the residual rebound to the layer input, decodeFFN;
+    hidden state after every token against the runtime's own decode step.  The handles round q, k, v, the attention context
+    and both residual sums to fp16 on their surfaces, the runtime keeps fp32: the tolerance is that rounding."""
+    import espresso_amd.llama as ll
+    import espresso_amd.synthetic as syn
+    cfg = ll.MultiModelConfig(**shape)
+    rt, packed = syn.build_runtime(cfg, FMT[name], seed=23, kv_format=orc.FMT_F16, keep_packed=True)
+    lw = packed["layers"][0]
+    dim, q_dim, kv_dim, hidden = cfg.d_model, cfg.n_head * cfg.head_dim, cfg.n_kv_head * cfg.head_dim, cfg.hidden_dim
+    spatial, stride = 32, cfg.max_seq
+    norm = lambda key: orc.blob_build(np.frombuffer(bytes(lw[key]), np.float16).astype(np.float32))
+    path = lambda stem: f"@model_path/weights/{stem}.bin"
+    qkv = io.ANEKernel(io.program_text("decode_qkv", name, spatial, 1, dim=dim, q_dim=q_dim, kv_dim=kv_dim),
+                       [(path("rms_att"), norm("rms_att")), (path("wq"), bytes(lw["wq"])), (path("wk"), bytes(lw["wk"])), (path("wv"), bytes(lw["wv"]))],
+                       [dim * spatial * 2], [kv_dim * spatial * 2, q_dim * spatial * 2, kv_dim * spatial * 2])
+    proj = io.ANEKernel(io.program_text("decode_projection", name, spatial, 1, dim=dim, q_dim=q_dim), [(path("wo"), bytes(lw["wo"]))],
+                        [q_dim * spatial * 2, dim * spatial * 2], [dim * spatial * 2])
+    ffn = io.ANEKernel(io.program_text("decode_ffn", name, spatial, 1, dim=dim, hidden=hidden),
+                       [(path("rms_ffn"), norm("rms_ffn")), (path("w1"), bytes(lw["w1"])), (path("w3"), bytes(lw["w3"])), (path("w2"), bytes(lw["w2"]))],
+                       [dim * spatial * 2], [dim * spatial * 2])
+    x_in = qkv.inputSurface(0)
+    k_out, q_out, v_out = qkv.outputSurface(0), qkv.outputSurface(1), qkv.outputSurface(2)
+    k_cache, v_cache = io.Surface.create(kv_dim * stride * 2), io.Surface.create(kv_dim * stride * 2)
+    proj.rebindInput(1, x_in)                         # the residual is the layer's input surface
+    ffn.rebindInput(0, proj.outputSurface(0))
+    ctx, out = proj.inputSurface(0), ffn.outputSurface(0)
+    emb = np.frombuffer(bytes(packed["embedding"]), np.float16).reshape(cfg.vocab, dim).astype(np.float32)
+    rng = np.random.default_rng(7)
+    worst = 0.0
+    for pos, token in enumerate(rng.integers(0, cfg.vocab, 40).tolist()):
+        io.SurfaceIO.writeFP16SpatialSlice(x_in, 0, 0, spatial, emb[token], dim)
+        qkv.eval()
+        io.rope_decode(q_out, k_out, cfg.n_head, cfg.n_kv_head, cfg.head_dim, pos, cfg.rope_theta, spatial)
+        io.kv_cache_scatter(k_out, v_out, k_cache, v_cache, kv_dim, pos, stride, spatial)
+        io.decode_sdpa(q_out, k_cache, v_cache, ctx, cfg.n_head, cfg.n_kv_head, cfg.head_dim, pos + 1, 0, stride, spatial)
+        proj.eval()
+        ffn.eval()
+        got = io.SurfaceIO.readFP16SpatialSlice(out, 0, 0, spatial, dim)
+        rt.advance(token)
+        want = rt.last_hidden()
+        scale = float(np.abs(want).max())
+        worst = max(worst, float(np.abs(got - want).max()) / scale)
+        assert np.all(np.abs(got - want) <= 2.0 ** -9 * scale + 1e-5), (pos, float(np.abs(got - want).max()), scale)
+    print(f"\n  {name}: worst |handles - runtime| / max|hidden| over 40 tokens = {worst:.2e}")
+    for kernel in (qkv, proj, ffn):
+        kernel.free()
+    rt.close()

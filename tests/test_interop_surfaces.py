@@ -199,3 +199,133 @@ def test_retain_release_counts():
     L.esp_surface_release(ref)
     assert L.esp_surface_bytes(ref) == 32        # still alive after one of two releases
     L.esp_surface_release(ref)
+
+
+def test_two_slice_copy_checks_both_pairs_before_touching_either():   # SurfaceIO.swift:285-339
+    channels = 6
+    k_src, v_src = Surface.create(channels * 4 * 2), Surface.create(channels * 4 * 2)
+    k_dst, v_dst = Surface.create(channels * 16 * 2), Surface.create(channels * 16 * 2)
+    rng = np.random.default_rng(21)
+    k, v = rng.normal(0, 1, (channels, 4)).astype(np.float32), rng.normal(0, 1, (channels, 4)).astype(np.float32)
+    SurfaceIO.writeFP16(k_src, k, channels, 4)
+    SurfaceIO.writeFP16(v_src, v, channels, 4)
+    SurfaceIO.copyTwoFP16SpatialSlices(k_dst, 0, 9, 16, k_src, 0, 2, 4, v_dst, 0, 9, 16, v_src, 0, 1, 4, channels)
+    assert np.array_equal(SurfaceIO.readFP16SpatialSlice(k_dst, 0, 9, 16, channels), k[:, 2].astype(np.float16).astype(np.float32))
+    assert np.array_equal(SurfaceIO.readFP16SpatialSlice(v_dst, 0, 9, 16, channels), v[:, 1].astype(np.float16).astype(np.float32))
+    with pytest.raises(io.SurfaceIOError):          # the second pair is out of range: the first must stay untouched
+        SurfaceIO.copyTwoFP16SpatialSlices(k_dst, 0, 3, 16, k_src, 0, 0, 4, v_dst, 0, 16, 16, v_src, 0, 0, 4, channels)
+    assert np.all(SurfaceIO.readFP16SpatialSlice(k_dst, 0, 3, 16, channels) == 0)
+
+
+def test_batched_writes_and_copies_are_all_or_nothing():   # SurfaceIO.swift:190-229, :672-716, :783-828
+    channels, spatial = 12, 4
+    s, t, u = (Surface.create(channels * spatial * 2) for _ in range(3))
+    a, b = np.arange(2 * spatial, dtype=np.float32) + 1, -(np.arange(3 * spatial, dtype=np.float32) + 1)
+    SurfaceIO.writeFP16AtBatched(s, spatial, [(1, a, 2), (7, b, 3)])
+    got = SurfaceIO.readFP16(s, 0, channels, spatial)
+    assert np.array_equal(got[1:3].ravel(), a) and np.array_equal(got[7:10].ravel(), b)
+    assert np.all(got[0] == 0) and np.all(got[3:7] == 0) and np.all(got[10:] == 0)
+    with pytest.raises(io.SurfaceIOError):          # second region runs past the surface: nothing is written
+        SurfaceIO.writeFP16AtBatched(t, spatial, [(0, a, 2), (10, b, 3)])
+    assert np.all(SurfaceIO.readFP16(t, 0, channels, spatial) == 0)
+    SurfaceIO.copyFP16Batched(t, s, spatial, [(0, 7, 3), (5, 1, 2)])
+    got_t = SurfaceIO.readFP16(t, 0, channels, spatial)
+    assert np.array_equal(got_t[0:3], got[7:10]) and np.array_equal(got_t[5:7], got[1:3]) and np.all(got_t[3:5] == 0) and np.all(got_t[7:] == 0)
+    with pytest.raises(io.SurfaceIOError):
+        SurfaceIO.copyFP16Batched(u, s, spatial, [(0, 7, 3), (11, 1, 2)])
+    assert np.all(SurfaceIO.readFP16(u, 0, channels, spatial) == 0)
+    SurfaceIO.copyFP16FromMultipleSources(u, spatial, [(s, 0, 1, 2), (t, 4, 0, 3), (s, 9, 7, 3)])
+    got_u = SurfaceIO.readFP16(u, 0, channels, spatial)
+    assert np.array_equal(got_u[0:2], got[1:3]) and np.array_equal(got_u[4:7], got_t[0:3]) and np.array_equal(got_u[9:12], got[7:10])
+    with pytest.raises(io.SurfaceIOError):
+        SurfaceIO.copyFP16FromMultipleSources(u, spatial, [(s, 0, 1, 2), (t, 4, 11, 3)])
+    SurfaceIO.copyFP16Batched(u, s, spatial, [])    # empty region lists are no-ops (SurfaceIO.swift:676, :787)
+    SurfaceIO.copyFP16FromMultipleSources(u, spatial, [])
+
+
+def test_block_partitioned_argmax_is_the_serial_first_maximum():   # surface_io.c:689-700; SurfaceIO.swift:542-615
+    channels, spatial, streams = 1003, 8, 5
+    rng = np.random.default_rng(33)
+    x = rng.normal(0, 1, (channels, spatial)).astype(np.float32)
+    x[[250, 251, 600], 0] = 9.0                     # ties across every block boundary of the partitions below
+    x[[1002, 17], 1] = 7.5                          # the first and the last block
+    x[:, 2] = -3.0                                  # all equal: channel 0
+    x[:, 3] = -65504.0                              # the lowest finite value everywhere
+    s = Surface.create((channels + 4) * spatial * 2)
+    SurfaceIO.writeFP16At(s, 4, x, channels, spatial)
+    serial = SurfaceIO.argmaxBatchFP16Spatial(s, 4, spatial, channels, streams)
+    assert serial[0][:4] == [250, 17, 0, 0] and serial[1][:4] == [9.0, 7.5, -3.0, -65504.0]
+    for blocks in (1, 2, 3, 4, 7, 8, 16, 1003, 5000):
+        assert SurfaceIO.argmaxBatchFP16SpatialParallel(s, 4, spatial, channels, streams, blocks) == serial
+        assert SurfaceIO.argmaxBatchFP16SpatialNolock(s, 4, spatial, channels, streams, blocks) == serial
+    with pytest.raises(io.SurfaceIOError):
+        SurfaceIO.argmaxBatchFP16SpatialParallel(s, 4, spatial, channels + 1, streams, 4)
+    with pytest.raises(io.SurfaceIOError):
+        SurfaceIO.argmaxBatchFP16SpatialParallel(s, 4, spatial, channels, spatial + 1, 4)
+
+
+def test_argmax_with_hint_is_the_first_maximum_and_survives_a_wrong_hint():   # SurfaceIO.swift:433-474
+    channels, spatial = 300, 4
+    rng = np.random.default_rng(34)
+    x = rng.normal(0, 1, (channels, spatial)).astype(np.float32)
+    x[[40, 200], 1] = 6.0
+    s, hint = Surface.create(channels * spatial * 2), Surface.create(spatial * 2)
+    SurfaceIO.writeFP16(s, x, channels, spatial)
+    SurfaceIO.writeFP16(hint, x.astype(np.float16).astype(np.float32).max(axis=0), 1, spatial)
+    for lane in range(spatial):
+        assert SurfaceIO.argmaxFP16SpatialSliceWithHint(s, 0, lane, spatial, channels, hint, lane, spatial) == SurfaceIO.argmaxFP16SpatialSlice(s, 0, lane, spatial, channels)
+    assert SurfaceIO.argmaxFP16SpatialSliceWithHint(s, 0, 1, spatial, channels, hint, 1, spatial) == (40, 6.0)
+    # a hint that matches no channel (lane 1's maximum used for lane 0) still gives the scan's answer
+    assert SurfaceIO.argmaxFP16SpatialSliceWithHint(s, 0, 0, spatial, channels, hint, 1, spatial) == SurfaceIO.argmaxFP16SpatialSlice(s, 0, 0, spatial, channels)
+    with pytest.raises(io.SurfaceIOError):
+        SurfaceIO.argmaxFP16SpatialSliceWithHint(s, 0, 0, spatial, channels, hint, spatial, spatial)
+
+
+def test_strided_gather_and_scatter_convert_like_the_contiguous_routines():   # ane_interop.h:160, :165
+    rng = np.random.default_rng(35)
+    x = rng.normal(0, 2, 96).astype(np.float32)
+    bits = io.cvt_f32_to_f16(x)
+    assert np.array_equal(io.gather_f16_to_f32(bits, 12, 8), io.cvt_f16_to_f32(bits[::8]))
+    dst = np.full(96, 0x7BFF, np.uint16)
+    io.scatter_f32_to_f16(dst, x[:12], 8)
+    assert np.array_equal(dst[::8], io.cvt_f32_to_f16(x[:12]))
+    untouched = np.ones(96, bool); untouched[::8] = False
+    assert np.all(dst[untouched] == 0x7BFF)
+
+
+def test_fused_expansion_argmax_follows_fp16_fused_multiply_adds():   # surface_io.c:1438-1700
+    """Parity unpinned against the reference (it holds no vector for this routine); pinned here against exact
+    fp16 arithmetic done in numpy: every term is one fused multiply-add rounded to fp16, terms in channel order."""
+    bottleneck, groups, vocab, spatial, streams = 32, 4, 96, 8, 3
+    cpg, per = bottleneck // groups, vocab // groups
+    rng = np.random.default_rng(36)
+    proj = rng.normal(0, 1, (bottleneck, spatial)).astype(np.float16)
+    w = rng.normal(0, 1, (vocab, cpg)).astype(np.float16)
+    w[50] = w[49]                                   # rows 49 and 50 (same group) tie exactly: 49 wins whenever they lead
+    s = Surface.create((bottleneck + 2) * spatial * 2)
+    SurfaceIO.writeFP16At(s, 2, proj.astype(np.float32), bottleneck, spatial)
+    want_i, want_v = [], []
+    for lane in range(streams):
+        logits = np.empty(vocab, np.float16)
+        for c in range(vocab):
+            g, acc = c // per, np.float16(0)
+            for k in range(cpg):
+                acc = np.float16(np.float64(w[c, k]) * np.float64(proj[g * cpg + k, lane]) + np.float64(acc))
+            logits[c] = acc
+        want_i.append(int(np.argmax(logits))); want_v.append(float(logits.max()))
+    got_i, got_v = SurfaceIO.fusedExpansionArgmax(s, 2, spatial, bottleneck, groups, w.view(np.uint16), vocab, streams)
+    assert got_i == want_i and got_v == want_v
+    # a one-hot projection selects one weight column: the winner is that column's largest entry within the group
+    onehot = np.zeros((bottleneck, spatial), np.float32); onehot[cpg * 2 + 3, 0] = 1.0
+    SurfaceIO.writeFP16At(s, 2, onehot, bottleneck, spatial)
+    col = w[2 * per:3 * per, 3].astype(np.float32)
+    i, v = SurfaceIO.fusedExpansionArgmax(s, 2, spatial, bottleneck, groups, w.view(np.uint16), vocab, 1)
+    if col.max() > 0:
+        assert i == [2 * per + int(np.argmax(col))] and v == [float(col.max())]
+    else:
+        assert v == [0.0]                             # every other group scores exactly 0
+    # the reference's argument checks
+    for bad in (dict(spatial=12), dict(vocab=65536 + 32), dict(groups=5), dict(streams=spatial + 1)):
+        sp, vc, gr, st = bad.get("spatial", spatial), bad.get("vocab", vocab), bad.get("groups", groups), bad.get("streams", streams)
+        idx, val = (C.c_int * 16)(), (C.c_float * 16)()
+        assert not io._L().esp_interop_fused_expansion_argmax_fp16(s.ref, 2, sp, bottleneck, gr, w.ctypes.data_as(C.c_void_p), vc, st, idx, val, 4)
