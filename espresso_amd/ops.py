@@ -127,15 +127,17 @@ class Int4Classifier:
             pass
 
 
-def gemv_stamps(m: "Matrix", batch: int = 1, launches: int = 8, capacity: int = 16384) -> np.ndarray:
-    """[wavefronts][4] wall-clock stamps (100 MHz ticks: start, staged, first weights consumed, end) of one Q4_K GEMV launch."""
+def gemv_stamps(m: "Matrix", batch: int = 1, launches: int = 8, capacity: int = 16384) -> tuple[np.ndarray, float]:
+    """([wavefronts][4] wall-clock stamps (100 MHz ticks: start, staged, first weights consumed, end), microseconds from
+    this launch's first wavefront start to the next launch's) of one Q4_K GEMV launch inside a back-to-back train over
+    copies of the matrix that exceed the caches."""
     L = _lib.load_library()
     L.esp_gemv_stamps.restype = C.c_int
-    L.esp_gemv_stamps.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_int)]
+    L.esp_gemv_stamps.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_double)]
     out = np.zeros((capacity, 4), dtype=np.uint64)
-    n = C.c_int(0)
-    _lib.check(L.esp_gemv_stamps(m._h, batch, launches, _ptr(out), capacity, C.byref(n)))
-    return out[:n.value]
+    n, us = C.c_int(0), C.c_double(0)
+    _lib.check(L.esp_gemv_stamps(m._h, batch, launches, _ptr(out), capacity, C.byref(n), C.byref(us)))
+    return out[:n.value], us.value
 
 
 def set_tuning(key: str, value: int) -> None:

@@ -108,10 +108,15 @@ void esp_int4_classifier_free(ESPInt4Classifier *classifier);
 int esp_int4_classifier_export(const ESPInt4Classifier *classifier, uint8_t *packed, float *scales, float *biases);
 int esp_int4_classifier_matvec_argmax(ESPInt4Classifier *classifier, const float *input, float *logits_or_null, int *index_or_null);
 
-/* Measurement aid (no counterpart in the reference): runs the Q4_K GEMV `launches` times back to back and has every wavefront
- * of the last launch record four 100 MHz wall-clock stamps: start, activations staged, first weights consumed, end.
- * out_stamps receives [wavefront][4]; *out_wavefronts how many wavefronts wrote (at most capacity_wavefronts). */
-int esp_gemv_stamps(const ESPMatrix *matrix, int batch, int launches, uint64_t *out_stamps, int capacity_wavefronts, int *out_wavefronts);
+/* Measurement aid (no counterpart in the reference): runs the Q4_K GEMV back to back over copies of the matrix that together
+ * exceed the caches (at least `launches` - 1 times and once through all copies: weights from HBM, code and activations warm,
+ * the state a decode step finds); every wavefront of one launch inside that train records four 100 MHz wall-clock stamps:
+ * start, activations staged, first weights consumed, end.  out_stamps receives [wavefront][4]; *out_wavefronts how many
+ * wavefronts wrote (at most capacity_wavefronts); *out_period_us (may be null) the time from the first wavefront start of
+ * that launch to the first wavefront start of the next one: the launch's share of the train, which exceeds its last
+ * wavefront's end by the time in which no wavefront of either kernel runs. */
+int esp_gemv_stamps(const ESPMatrix *matrix, int batch, int launches, uint64_t *out_stamps, int capacity_wavefronts, int *out_wavefronts,
+                    double *out_period_us);
 /* Kernel-selection switches for measurements and tests (no counterpart in the reference); the same switches are read from
  * the environment when first needed.  "q4k_mfma" (ESPRESSO_HIP_Q4K_MFMA): 1 = Q4_K GEMVs of 4096 / 14336 columns run on the
  * matrix cores (one to eight activation rows per pass over the weights), 0 = never, -1 = the library's own choice.
