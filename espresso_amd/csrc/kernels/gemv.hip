@@ -646,13 +646,17 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
     const int n_teams = workgroups * TEAMS, npairs = (a.rows + 1) / 2;
     const Q4KLane L = q4k_lane_constants(lane);
 
+    // Issued unconditionally, also for pairs past the end (those read the matrix's first 48 bytes, shared by every lane): a load
+    // under a branch makes the compiler wait for every load in flight wherever it needs one of them, which would tie the staging
+    // of the activations to the arrival of the first weights.
     auto load_pair = [&](int pair, Q4KItem (&buf)[PASSES]) {
+        const bool real = pair < npairs;
         const int row_a = 2 * pair < a.rows ? 2 * pair : a.rows - 1;   // clamped: loads stay inside the matrix
         const int row_b = 2 * pair + 1 < a.rows ? 2 * pair + 1 : a.rows - 1;
-        const uint8_t *base_a = a.qs + (size_t)row_a * a.qs_row_bytes, *base_b = a.qs + (size_t)row_b * a.qs_row_bytes;
+        const uint8_t *base_a = a.qs + (real ? (size_t)row_a * a.qs_row_bytes : 0), *base_b = a.qs + (real ? (size_t)row_b * a.qs_row_bytes : 0);
 #pragma unroll
         for (int p = 0; p < PASSES; p++) {
-            const int t = tl + p * TEAM_LANES, tt = t < TOTAL ? t : 0;
+            const int t = tl + p * TEAM_LANES, tt = t < TOTAL && real ? t : 0;
             const bool second = tt >= IPR;
             const int i = tt - (second ? IPR : 0);
             const uint8_t *bp = (second ? base_b : base_a) + (size_t)(i >> 2) * 144;
@@ -742,19 +746,19 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
     int pair = first_pair;
     stamp(a, 0);
     stage.issue(a);
-    if (pair < npairs) load_pair(pair, buf0);
+    load_pair(pair, buf0);
     stage.finish(a, xs4, xsum, norm_red);
     __syncthreads();
     stamp(a, 1);
     for (int j = 0; j < iters; j += 2) {
         int next = pair + n_teams;
-        if (next < npairs) load_pair(next, buf1);
+        load_pair(next, buf1);
         process(buf0, pair, j);
         if (j == 0) stamp(a, 2);
         pair = next;
         if (j + 1 < iters) {
             next = pair + n_teams;
-            if (next < npairs) load_pair(next, buf0);
+            load_pair(next, buf0);
             process(buf1, pair, j + 1);
             pair = next;
         }
@@ -1013,14 +1017,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
     }
     const int total_steps = iters * S;
     auto block_of = [&](int round) { return (round * workgroups + (int)blockIdx.x) * RB + team; };
+    // Every load of the ring is issued unconditionally: a load under a branch makes the compiler wait for all loads in flight
+    // wherever it needs any of them (it cannot count what was issued), which would tie the staging of the activations and every
+    // step of the ring to the arrival of the newest weights.  Steps past the end read sixteen bytes that every lane shares.
     auto load_step = [&](int f) {
         Q4KItem it;
+        const bool real = f < total_steps;
         const int round = f / S, step = f - round * S;
         const int rb = block_of(round) < row_blocks ? block_of(round) : row_blocks - 1;   // blocks past the end repeat the last one; never stored
-        const uint8_t *tp = tiled + ((size_t)rb * NSB + (ks * S + step)) * kQ4KTileBytes;
-        it.hdr = *reinterpret_cast<const uint4 *>(tp + 16 * n);
-        it.q0 = *reinterpret_cast<const uint4 *>(tp + 256 + 16 * lane);
-        it.q1 = *reinterpret_cast<const uint4 *>(tp + 1280 + 16 * lane);
+        const uint8_t *tp = real ? tiled + ((size_t)rb * NSB + (ks * S + step)) * kQ4KTileBytes : tiled;
+        const int spread = real ? 16 : 0;
+        it.hdr = *reinterpret_cast<const uint4 *>(tp + spread * n);
+        it.q0 = *reinterpret_cast<const uint4 *>(tp + (real ? 256 : 0) + spread * lane);
+        it.q1 = *reinterpret_cast<const uint4 *>(tp + (real ? 1280 : 0) + spread * lane);
         return it;
     };
 
@@ -1029,8 +1038,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
     stage.issue(a);
     Q4KItem ring[DEPTH];
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++)
-        if (d < total_steps) ring[d] = load_step(d);
+    for (int d = 0; d < DEPTH; d++) ring[d] = load_step(d);
     if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
     stage.finish(a, xs4, xsum, misc);
     __syncthreads();
@@ -1112,8 +1120,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
 #pragma unroll
         for (int i = 0; i < S; i++) {
             const Q4KItem it = ring[i % DEPTH];
-            const int next = round * S + i + DEPTH;
-            if (next < total_steps) ring[i % DEPTH] = load_step(next);
+            ring[i % DEPTH] = load_step(round * S + i + DEPTH);
             step_compute(it, i);
             if (a.stamps && round == 0 && i == 0) { if (v[0] != 12345.678f) stamp(a, 2); }   // after the first weights were needed
         }
