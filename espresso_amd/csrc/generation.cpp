@@ -8,6 +8,81 @@ namespace esp {
 namespace {
 using Clock = std::chrono::steady_clock;
 double ms_since(Clock::time_point t0) { return std::chrono::duration<double, std::milli>(Clock::now() - t0).count(); }
+
+// One pass of the exact two-token loop with every decision on the device (TwoTokenState): the draft runs two rows (the row
+// it owes after an accepted pass and the current token, or the current token twice) and proposes; the target verifies
+// (current, proposed); the accept kernel emits, keeps the hidden row and writes the next pass's rows.  No host decision, so
+// the pass replays as a captured graph.
+int enqueue_two_token_pass(LlamaRuntime &full, LlamaRuntime &draft, TwoTokenState *state, int *log, int log_capacity) {
+    hipStream_t s = context().stream;
+    int rc;
+    if ((rc = draft.enqueue_device_rows(2)) != ESP_OK) return rc;
+    if ((rc = draft.enqueue_device_head(2)) != ESP_OK) return rc;
+    ESP_HIP_TRY(launch_two_token_verify_rows(state, draft.device_head_tokens(), full.device_row_tokens(), full.device_row_positions(), s));
+    if ((rc = full.enqueue_device_rows(2)) != ESP_OK) return rc;
+    if ((rc = full.enqueue_device_head(2)) != ESP_OK) return rc;
+    ESP_HIP_TRY(launch_two_token_accept(state, full.device_head_tokens(), log, log_capacity, full.device_hidden_rows(), full.device_last_hidden(0),
+                                        full.config().d_model, draft.device_row_tokens(), draft.device_row_positions(), s));
+    return ESP_OK;
+}
+
+// Runs passes on the device until the loop ends or a pass would need a host decision (fewer than two tokens of budget or two
+// positions of context left).  `state` comes in with the host loop's variables and goes out with them; log receives the
+// emitted tokens at their output indices.
+int run_two_token_passes_on_device(LlamaRuntime &full, LlamaRuntime &draft, TwoTokenState *state, std::vector<int> *log) {
+    hipStream_t s = context().stream;
+    TwoTokenState *d_state = nullptr;
+    int *d_log = nullptr;
+    hipGraphExec_t exec = nullptr;
+    const int capacity = state->budget + 2;
+    log->assign(capacity, 0);
+    int rc = device_alloc(&d_state, (size_t)1);
+    if (rc == ESP_OK) rc = device_alloc(&d_log, (size_t)capacity);
+    auto cleanup = [&](int code) {
+        if (exec) (void)hipGraphExecDestroy(exec);
+        if (d_state) (void)hipFree(d_state);
+        if (d_log) (void)hipFree(d_log);
+        return code;
+    };
+    if (rc != ESP_OK) return cleanup(rc);
+    auto hip = [&](hipError_t e, const char *what) { return e == hipSuccess ? ESP_OK : fail_hip(e, what); };
+    auto fetch = [&]() {
+        int r = hip(hipMemcpyAsync(state, d_state, sizeof(TwoTokenState), hipMemcpyDeviceToHost, s), "two-token state");
+        if (r == ESP_OK) r = hip(hipStreamSynchronize(s), "two-token pass");
+        return r;
+    };
+    StepRows rows{};
+    rows.count = 2;
+    rows.token[0] = rows.token[1] = state->current;
+    rows.pos[0] = rows.pos[1] = state->full_pos;
+    rows.seq[0] = rows.seq[1] = 0;
+    if ((rc = hip(hipMemcpyAsync(d_state, state, sizeof(TwoTokenState), hipMemcpyHostToDevice, s), "two-token state")) != ESP_OK) return cleanup(rc);
+    if ((rc = hip(launch_set_rows(rows, draft.device_row_tokens(), draft.device_row_positions(), draft.device_row_sequences(), s), "rows")) != ESP_OK) return cleanup(rc);
+    if ((rc = hip(launch_set_rows(rows, full.device_row_tokens(), full.device_row_positions(), full.device_row_sequences(), s), "rows")) != ESP_OK) return cleanup(rc);
+    // the first pass runs as plain launches: whatever a kernel configures on its first use happens outside the capture
+    if ((rc = enqueue_two_token_pass(full, draft, d_state, d_log, capacity)) != ESP_OK) return cleanup(rc);
+    if ((rc = fetch()) != ESP_OK) return cleanup(rc);
+    while (!state->done) {
+        if (!exec) {
+            hipGraph_t graph = nullptr;
+            if ((rc = hip(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture")) != ESP_OK) return cleanup(rc);
+            rc = enqueue_two_token_pass(full, draft, d_state, d_log, capacity);
+            const hipError_t e = hipStreamEndCapture(s, &graph);
+            if (rc == ESP_OK) rc = hip(e, "hipStreamEndCapture");
+            if (rc == ESP_OK) rc = hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+            if (graph) (void)hipGraphDestroy(graph);
+            if (rc != ESP_OK) return cleanup(rc);
+        }
+        // a pass emits one or two tokens: half of what is left can never overrun, and passes after the end change nothing
+        const int left = state->budget - state->emitted, chunk = left / 2 > 1 ? left / 2 : 1;
+        for (int i = 0; i < chunk; i++)
+            if ((rc = hip(hipGraphLaunch(exec, s), "hipGraphLaunch")) != ESP_OK) return cleanup(rc);
+        if ((rc = fetch()) != ESP_OK) return cleanup(rc);
+    }
+    rc = hip(hipMemcpyAsync(log->data(), d_log, sizeof(int) * capacity, hipMemcpyDeviceToHost, s), "two-token log");
+    if (rc == ESP_OK) rc = hip(hipStreamSynchronize(s), "two-token log");
+    return cleanup(rc);
+}
 }  // namespace
 
 int generate_greedy(LlamaRuntime &rt, const uint32_t *prompt, int prompt_count, int max_tokens,
@@ -107,6 +182,41 @@ int generate_two_token(LlamaRuntime &full, LlamaRuntime &draft, const uint32_t *
     emit(current);
     int all = prompt_count + 1;
     if ((eos >= 0 && current == (uint32_t)eos) || (int)out->size() >= eff || all >= max_seq) return finish();
+
+    // Full passes (two tokens of budget and two positions of context left) run on the device, one captured graph per pass and
+    // no host decision in between; what is left afterwards (at most one pass) takes the loop below.
+    if (full.graph_replay_enabled() && draft.graph_replay_enabled() && &full != &draft && eff - (int)out->size() >= 2 && all + 1 < max_seq) {
+        TwoTokenState ds{};
+        ds.current = (int)current; ds.full_pos = full.visible(0); ds.emitted = (int)out->size(); ds.budget = eff; ds.all = all;
+        ds.max_seq = max_seq; ds.eos = eos; ds.reference_accounting = reference_accounting ? 1 : 0;
+        std::vector<int> log;
+        const auto t_device = Clock::now();
+        const int first = ds.emitted;
+        if ((rc = run_two_token_passes_on_device(full, draft, &ds, &log)) != ESP_OK) return rc;
+        const double per_token = ms_since(t_device) / (ds.emitted - first > 0 ? ds.emitted - first : 1);
+        for (int i = first; i < ds.emitted; i++) {
+            out->push_back((uint32_t)log[i]);
+            if (timing) timing->token_latencies_ms.push_back(per_token);   // one measurement for all of them
+        }
+        t_emit = Clock::now();
+        st.passes += ds.passes; st.committed_total += ds.committed_total; st.accepted_total += ds.accepted_total;
+        st.reference_accepted_total += ds.reference_accepted_total;
+        all = ds.all;
+        current = (uint32_t)ds.current;
+        // both models as the host loop would have left them: the draft has consumed what the target has, less the row it owes
+        if ((rc = full.set_visible(0, ds.full_pos)) != ESP_OK) return rc;
+        if ((rc = draft.set_visible(0, ds.full_pos - (ds.accepted_prev ? 1 : 0))) != ESP_OK) return rc;
+        if ((rc = draft.keep_row(1, 0)) != ESP_OK) return rc;
+        if (ds.accepted_prev) {
+            if ((rc = draft.advance(0, (uint32_t)ds.proposed_prev)) != ESP_OK) return rc;
+            if (reference_accounting) {
+                uint32_t p1 = 0;
+                if ((rc = draft.select_greedy(0, &p1)) != ESP_OK) return rc;
+                if (p1 == (uint32_t)ds.exact1_prev) st.reference_accepted_total++;
+            }
+        }
+        if (ds.stopped) return finish();
+    }
 
     // Invariant: `current` is the last emitted token; neither model has consumed it yet.
     while ((int)out->size() < eff && all < max_seq) {

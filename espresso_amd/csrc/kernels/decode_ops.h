@@ -96,6 +96,28 @@ hipError_t launch_greedy_tail(const ArgmaxScratch &scratch, int blocks, int *out
                               int *log, int *log_count, int log_capacity, const void *table, bool table_is_f16, int d, float *hidden,
                               hipStream_t s);
 hipError_t launch_set_ints(int *dst0, int v0, int *dst1, int v1, hipStream_t s);
+
+// Device-resident state of the exact two-token loop over one sequence (generateIncrementalExactTwoTokenDraftLlama,
+// RealModelInferenceEngine.swift:6014-6190): what the host loop keeps in local variables, so that whole passes (draft step,
+// two-row verify step, acceptance) replay as one captured graph without a host decision in between.
+struct TwoTokenState {
+    int current;        // the last emitted token; neither model has consumed it yet
+    int full_pos;       // the target's visible token count
+    int accepted_prev;  // the pass before accepted its proposal: the draft still owes the row (proposed_prev, full_pos - 1)
+    int proposed_prev, exact1_prev;
+    int proposed;       // this pass's proposal (set between the draft step and the verify step)
+    int emitted, budget, all, max_seq, eos, reference_accounting;
+    int done;           // no further pass may run on the device (end of the loop, or a pass that needs a host decision)
+    int stopped;        // the loop itself is over (stop token, budget, context)
+    int passes, committed_total, accepted_total, reference_accepted_total;
+};
+// After the draft's two rows went through its head: the proposal becomes row 1 of the target's verify step; the draft's
+// successor of the row it owed is compared for the reference's accepted count.
+hipError_t launch_two_token_verify_rows(TwoTokenState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, hipStream_t s);
+// After the target's two rows went through its head: emits one or two tokens into log, keeps the matching hidden row of the
+// target (d floats from hidden_rows into last_hidden), advances the state and writes the draft's two rows of the next pass.
+hipError_t launch_two_token_accept(TwoTokenState *state, const int *target_head_tokens, int *log, int log_capacity, const float *hidden_rows,
+                                   float *last_hidden, int d, int *draft_tokens, int *draft_pos, hipStream_t s);
 hipError_t launch_copy_rows(const float *src, float *dst, int rows, int d, hipStream_t s);
 
 }  // namespace esp

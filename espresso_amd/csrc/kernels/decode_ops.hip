@@ -926,7 +926,76 @@ __global__ void copy_rows_kernel(const float *src, float *dst, int d) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < d; i += gridDim.x * blockDim.x) dst[(size_t)m * d + i] = src[(size_t)m * d + i];
 }
 
+// One thread: see launch_two_token_verify_rows.
+__global__ void two_token_verify_rows_kernel(TwoTokenState *st, const int *draft_head, int *tokens, int *pos) {
+    if (threadIdx.x != 0 || blockIdx.x != 0 || st->done) return;
+    // row 0 of the draft's step was the row it owed after an accepted pass: its successor is the reference's second
+    // comparison of that pass (:6156-6163)
+    if (st->accepted_prev && st->reference_accounting && draft_head[0] == st->exact1_prev) st->reference_accepted_total += 1;
+    const int proposed = draft_head[1];
+    st->proposed = proposed;
+    tokens[0] = st->current; pos[0] = st->full_pos;
+    tokens[1] = proposed;    pos[1] = st->full_pos + 1;
+}
+
+// Thread 0 runs one iteration of the reference loop's bookkeeping (:6109-6186), then the workgroup keeps the hidden row.
+__global__ __launch_bounds__(256) void two_token_accept_kernel(TwoTokenState *st, const int *head, int *log, int log_capacity, const float *hidden_rows,
+                                                                float *last_hidden, int d, int *draft_tokens, int *draft_pos) {
+    __shared__ int keep;
+    if (threadIdx.x == 0) {
+        keep = -1;
+        if (!st->done) {
+            const int e0 = head[0], e1 = head[1], proposed = st->proposed;
+            st->passes += 1;
+            if (st->emitted < log_capacity) log[st->emitted] = e0;
+            st->emitted += 1; st->all += 1; st->committed_total += 1;
+            if (st->reference_accounting && proposed == e0) st->reference_accepted_total += 1;
+            const bool stop0 = (st->eos >= 0 && e0 == st->eos) || st->emitted >= st->budget || st->all >= st->max_seq;
+            if (stop0 || proposed != e0) {
+                st->full_pos += 1; st->current = e0; st->accepted_prev = 0;
+                keep = 0;
+                if (stop0) { st->done = 1; st->stopped = 1; }
+            } else {
+                // the proposal was right: row 1 ran on the exact token, its column and its successor stand
+                st->accepted_total += 1; st->committed_total += 1;
+                st->full_pos += 2;
+                keep = 1;
+                if (st->emitted < log_capacity) log[st->emitted] = e1;
+                st->emitted += 1; st->all += 1; st->current = e1;
+                st->accepted_prev = 1; st->proposed_prev = proposed; st->exact1_prev = e1;
+                if (st->eos >= 0 && e1 == st->eos) { st->done = 1; st->stopped = 1; }
+            }
+            // the next pass runs here only if it is a full one: two tokens of budget and two positions of context left
+            if (!st->done && (st->budget - st->emitted < 2 || st->all + 1 >= st->max_seq || st->emitted >= st->budget || st->all >= st->max_seq)) st->done = 1;
+            if (!st->done) {
+                if (st->accepted_prev) {
+                    draft_tokens[0] = st->proposed_prev; draft_pos[0] = st->full_pos - 1;
+                    draft_tokens[1] = st->current;       draft_pos[1] = st->full_pos;
+                } else {   // nothing owed: both rows are the same row, which writes the same cache column twice
+                    draft_tokens[0] = draft_tokens[1] = st->current;
+                    draft_pos[0] = draft_pos[1] = st->full_pos;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (keep >= 0)
+        for (int i = threadIdx.x; i < d; i += 256) last_hidden[i] = hidden_rows[(size_t)keep * d + i];
+}
+
 }  // namespace
+
+hipError_t launch_two_token_verify_rows(TwoTokenState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, hipStream_t s) {
+    hipLaunchKernelGGL(two_token_verify_rows_kernel, dim3(1), dim3(64), 0, s, state, draft_head_tokens, target_tokens, target_pos);
+    return hipGetLastError();
+}
+
+hipError_t launch_two_token_accept(TwoTokenState *state, const int *target_head_tokens, int *log, int log_capacity, const float *hidden_rows,
+                                   float *last_hidden, int d, int *draft_tokens, int *draft_pos, hipStream_t s) {
+    hipLaunchKernelGGL(two_token_accept_kernel, dim3(1), dim3(256), 0, s, state, target_head_tokens, log, log_capacity, hidden_rows, last_hidden, d,
+                       draft_tokens, draft_pos);
+    return hipGetLastError();
+}
 
 hipError_t launch_embed(const void *table, bool table_is_f16, const int *tokens, int rows, int d, float *hidden, hipStream_t s) {
     hipLaunchKernelGGL(embed_kernel, dim3((d + 255) / 256, rows), dim3(256), 0, s, table, table_is_f16 ? 1 : 0, tokens, d, hidden);

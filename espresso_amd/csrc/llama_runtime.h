@@ -75,6 +75,18 @@ class LlamaRuntime {
 
     size_t weight_bytes_per_token() const { return weight_bytes_; }
 
+    // Steps whose rows (token, position, sequence) already sit in the device arrays below: generation loops that keep
+    // their decisions on the device enqueue these, also under stream capture.  Nothing here synchronises.
+    int *device_row_tokens() { return d_tokens_; }
+    int *device_row_positions() { return d_pos_; }
+    int *device_row_sequences() { return d_seq_; }
+    const int *device_head_tokens() const { return d_out_tokens_; }
+    const float *device_hidden_rows() const { return hidden_; }
+    float *device_last_hidden(int seq) { return last_hidden_ + (size_t)seq * c_.d_model; }
+    int enqueue_device_rows(int rows) { return enqueue_trunk(rows); }             // embedding, then every layer
+    int enqueue_device_head(int rows) { return run_head(hidden_, rows); }         // final norm, head, first-max arg-max per row
+    bool graph_replay_enabled() const { return use_graph_ && !timing_enabled_; }
+
     // Per-kernel timing with HIP events on the library stream.  While enabled, every launch of the
     // kernels below is bracketed by an event pair; collect_kernel_times() synchronises and adds the
     // elapsed times to the totals.
