@@ -147,7 +147,9 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # workload (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors kernels of known size in the same runs gave);
 # the runs and the per-kernel table are in profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt.
-MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66569318}
+MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66532352}
+# the same kernel's mean duration in the committed rocprofv3 kernel trace (a profiled run; 3-5 % slower than an unprofiled one)
+PROFILE_KERNEL_US = {("llama3-8b-q4k", "gate_up"): (14.25, "profiles/q4k_gemv_decode_llama3_8b_kernel_trace.txt")}
 TRAFFIC_SOURCE = "profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload; not measured in this run)"
 
 
@@ -360,6 +362,10 @@ def main() -> None:
         "roofline": {"bound": "hbm", "kernel": f"dequant-GEMV {dominant}", "achieved": d["gbps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": d["gbps"] / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get((args.workload, dominant)),
                      "traffic_source": TRAFFIC_SOURCE if (args.workload, dominant) in MEASURED_TRAFFIC else None,
+                     "profile": ({"mean_launch_us": PROFILE_KERNEL_US[(args.workload, dominant)][0],
+                                  "frac": d["bytes_per_launch"] / PROFILE_KERNEL_US[(args.workload, dominant)][0] / 1e3 / HBM_PEAK_GBPS,
+                                  "source": PROFILE_KERNEL_US[(args.workload, dominant)][1] + " (rocprofv3 --kernel-trace of the same command; not measured in this run)"}
+                                 if (args.workload, dominant) in PROFILE_KERNEL_US else None),
                      "bytes_per_launch": d["bytes_per_launch"], "mean_launch_us": d["kernel_us"], "launches_timed": 8 * (1 if dominant == "head" else n_layer),
                      "all_gemv_gbps": gemv_bytes / gemv_us / 1e3 if gemv_us else 0.0,
                      "all_gemv_frac": gemv_bytes / gemv_us / 1e3 / HBM_PEAK_GBPS if gemv_us else 0.0,
