@@ -193,7 +193,7 @@ struct RotatingCopies {
     int make(const DeviceMatrix &m, int rotate, hipStream_t stream) {
         copies.assign(rotate < 1 ? 1 : rotate, m);
         const size_t qs_bytes = (size_t)m.rows * m.qs_row_bytes, sc_count = m.scales ? (size_t)m.rows * (m.cols / 32) : 0;
-        const size_t tiled_bytes = m.tiled ? (size_t)((m.rows + 15) / 16) * (m.cols / 256) * 2304 : 0;
+        const size_t tiled_bytes = m.tiled_bytes();
         for (size_t i = 1; i < copies.size(); i++) { copies[i].qs = nullptr; copies[i].scales = nullptr; copies[i].tiled = nullptr; }
         for (size_t i = 1; i < copies.size(); i++) {
             int rc = device_alloc(&copies[i].qs, qs_bytes);

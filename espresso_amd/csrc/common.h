@@ -40,9 +40,13 @@ struct DeviceMatrix {
     int rows = 0, cols = 0;
     uint8_t *qs = nullptr;
     uint16_t *scales = nullptr;
-    // Q4_K only: a second copy of the same super-blocks tiled by (block of sixteen rows, super-block) for the matrix-core
-    // GEMV (layout: kernels/gemv.hip); rows padded to a multiple of sixteen with zero blocks.  Null when not built.
+    // Q4_K and Q4_0 matrices of 4096 or 14336 columns: a second copy tiled by (block of sixteen rows, 256 or 512 columns) for
+    // the matrix-core GEMV (layouts: kernels/gemv.hip); rows padded to a multiple of sixteen with zero blocks.  Null when not built.
     uint8_t *tiled = nullptr;
+    size_t tiled_bytes() const {
+        if (!tiled) return 0;
+        return format == FMT_Q4_K ? (size_t)((rows + 15) / 16) * (cols / 256) * 2304 : (size_t)((rows + 15) / 16) * (cols / 512) * 4608;
+    }
     size_t qs_row_bytes = 0;
     size_t bytes() const {  // algorithmic bytes: what one GEMV must read
         return (size_t)rows * qs_row_bytes + (scales ? (size_t)rows * (cols / 32) * 2 : 0);
@@ -143,6 +147,8 @@ hipError_t launch_repack(int format, const uint8_t *blocks, int rows, int cols, 
                          hipStream_t stream);
 // Q4_K super-blocks, row-major [rows][cols / 256][144 bytes] -> the tiled copy ((rows + 15) / 16 * cols / 256 tiles of 2304 bytes)
 hipError_t launch_q4k_tile(const uint8_t *blocks, int rows, int cols, uint8_t *tiled, hipStream_t stream);
+// Q4_0 planes -> the tiled copy ((rows + 15) / 16 * cols / 512 tiles of 4608 bytes)
+hipError_t launch_q40_tile(const uint8_t *qs, const uint16_t *scales, int rows, int cols, uint8_t *tiled, hipStream_t stream);
 // DeviceMatrix -> fp32 [rows][cols] (used to check the planes carry the same bits)
 hipError_t launch_dequant_matrix(const DeviceMatrix &m, float *out, hipStream_t stream);
 

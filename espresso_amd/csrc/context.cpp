@@ -89,6 +89,12 @@ int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, Devic
         if ((rc = device_alloc(&staging, src_bytes)) != ESP_OK) { matrix_release(&m); return rc; }
         e = hipMemcpyAsync(staging, gguf_blocks, src_bytes, hipMemcpyHostToDevice, c.stream);
         if (e == hipSuccess) e = launch_repack(format, staging, rows, cols, m, c.stream);
+        // Q4_0 matrices of the widths the matrix-core GEMV is built for also get the tiled copy it reads
+        if (e == hipSuccess && format == FMT_Q4_0 && (cols == 4096 || cols == 14336)) {
+            const size_t tiled_bytes = (size_t)((rows + 15) / 16) * (cols / 512) * 4608;
+            if ((rc = device_alloc(&m.tiled, tiled_bytes)) != ESP_OK) { (void)hipFree(staging); matrix_release(&m); return rc; }
+            e = launch_q40_tile(m.qs, m.scales, rows, cols, m.tiled, c.stream);
+        }
         if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
         (void)hipFree(staging);
     } else {

@@ -129,6 +129,31 @@ __global__ void q4k_tile_kernel(const uint8_t *blocks, int rows, int nsb, size_t
     *reinterpret_cast<uint4 *>(tiled + i * 16) = v;
 }
 
+// Q4_0 planes -> the tiled copy of the matrix-core GEMV: tile (rb, t) = sixteen rows x 512 columns = [j][lane] 16 bytes of nibbles
+// (lane (n, g) = g * 16 + n owns block 16 t + 4 j + g of row n), then [lane][j] fp16 scales.  320 threads per tile; rows past the
+// matrix are zero blocks with zero scales.
+__global__ void q40_tile_kernel(const uint8_t *qs, const uint16_t *scales, int rows, int tpr, size_t tiles, uint8_t *tiled) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t tile = i / 320;
+    if (tile >= tiles) return;
+    const int p = (int)(i - tile * 320);
+    const int rb = (int)(tile / tpr), t = (int)(tile - (size_t)rb * tpr);
+    uint8_t *dst = tiled + tile * 4608;
+    const int blocks_per_row = tpr * 16;
+    if (p < 256) {
+        const int j = p >> 6, lane = p & 63, g = lane >> 4, n = lane & 15, row = rb * 16 + n;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (row < rows) v = *reinterpret_cast<const uint4 *>(qs + ((size_t)row * blocks_per_row + 16 * t + 4 * j + g) * 16);
+        *reinterpret_cast<uint4 *>(dst + 1024 * j + 16 * lane) = v;
+    } else {
+        const int lane = p - 256, g = lane >> 4, n = lane & 15, row = rb * 16 + n;
+        uint16_t d[4] = {0, 0, 0, 0};
+        if (row < rows)
+            for (int j = 0; j < 4; j++) d[j] = scales[(size_t)row * blocks_per_row + 16 * t + 4 * j + g];
+        *reinterpret_cast<uint2 *>(dst + 4096 + 8 * lane) = make_uint2(d[0] | ((unsigned)d[1] << 16), d[2] | ((unsigned)d[3] << 16));
+    }
+}
+
 inline dim3 grid_for(size_t n, int threads) { return dim3((unsigned)((n + threads - 1) / threads)); }
 
 }  // namespace
@@ -178,6 +203,14 @@ hipError_t launch_q4k_tile(const uint8_t *blocks, int rows, int cols, uint8_t *t
     const int nsb = cols / 256;
     const size_t pieces = (size_t)((rows + 15) / 16) * nsb * 144;
     hipLaunchKernelGGL(q4k_tile_kernel, grid_for(pieces, 256), dim3(256), 0, stream, blocks, rows, nsb, pieces, tiled);
+    return hipGetLastError();
+}
+
+hipError_t launch_q40_tile(const uint8_t *qs, const uint16_t *scales, int rows, int cols, uint8_t *tiled, hipStream_t stream) {
+    if (!qs || !scales || !tiled || rows <= 0 || cols <= 0 || cols % 512 != 0) return hipErrorInvalidValue;
+    const int tpr = cols / 512;
+    const size_t tiles = (size_t)((rows + 15) / 16) * tpr;
+    hipLaunchKernelGGL(q40_tile_kernel, grid_for(tiles * 320, 320), dim3(320), 0, stream, qs, scales, rows, tpr, tiles, tiled);
     return hipGetLastError();
 }
 

@@ -905,7 +905,7 @@ __device__ __forceinline__ float workgroup_sum_waves(float v, float *red) {
 
 // Activations of a row (fp16 as given, RMSNorm fused, or attention states merged) into LDS for the matrix-core kernel:
 // every load is issued before the first use, as in Q4KStage; THREADS threads take groups tid, tid + THREADS, ...
-template <int NB, int IPR, int THREADS, int MODE>
+template <int NB, int IPR, int THREADS, int MODE, bool Q40 = false>
 struct MfmaStage {
     static constexpr int GROUPS = IPR * 8, K = (GROUPS + THREADS - 1) / THREADS, cols = IPR * 64, WAVES = THREADS / 64;
     static constexpr bool FULL = GROUPS % THREADS == 0;
@@ -957,7 +957,7 @@ struct MfmaStage {
                 const float inv = 1.0f / sqrtf(workgroup_sum_waves<WAVES>(s, red + b * WAVES) / (float)cols + a.norm_eps);
 #pragma unroll
                 for (int k = 0; k < K; k++)
-                    if (mine(k)) q4k_store_group_natural(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, group(k), cols, xs4, xsum);
+                    if (mine(k)) q4k_store_group_natural<Q40>(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, group(k), cols, xs4, xsum);
             }
         } else if constexpr (MODE == 2) {
 #pragma unroll
@@ -965,14 +965,14 @@ struct MfmaStage {
                 if (b > 0) load_merge_row(a, b);
 #pragma unroll
                 for (int k = 0; k < K; k++)
-                    if (mine(k)) q4k_store_group_natural(merge_group(ml[k], a0[k], a1[k]), b, group(k), cols, xs4, xsum);
+                    if (mine(k)) q4k_store_group_natural<Q40>(merge_group(ml[k], a0[k], a1[k]), b, group(k), cols, xs4, xsum);
             }
         } else {
 #pragma unroll
             for (int b = 0; b < NB; b++)
 #pragma unroll
                 for (int k = 0; k < K; k++)
-                    if (mine(k)) q4k_store_group_natural(v[b][k], b, group(k), cols, xs4, xsum);
+                    if (mine(k)) q4k_store_group_natural<Q40>(v[b][k], b, group(k), cols, xs4, xsum);
         }
     }
 };
@@ -1166,6 +1166,208 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
         float *cv = misc;
         int *ci = reinterpret_cast<int *>(misc + NB * WAVES);
         __syncthreads();   // misc was the norm's scratch
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+#pragma unroll
+            for (int off = 8; off >= 1; off >>= 1) {
+                const float ov = __shfl_xor(best[b], off);
+                const int oi = __shfl_xor(best_i[b], off);
+                argmax_take(best[b], best_i[b], ov, oi);
+            }
+            if (lane == 0) { cv[b * WAVES + wave] = ks == 0 ? best[b] : -INFINITY; ci[b * WAVES + wave] = ks == 0 ? best_i[b] : 0x7FFFFFFF; }
+        }
+        __syncthreads();
+        if (tid < NB) {
+            float bv = cv[tid * WAVES];
+            int bi = ci[tid * WAVES];
+#pragma unroll
+            for (int w = 1; w < WAVES; w++) argmax_take(bv, bi, cv[tid * WAVES + w], ci[tid * WAVES + w]);
+            a.part_value[(size_t)tid * gridDim.x + blockIdx.x] = bv;
+            a.part_index[(size_t)tid * gridDim.x + blockIdx.x] = bi;
+        }
+    }
+}
+
+
+// ---- Q4_0 on the matrix cores ---------------------------------------------------------------------------------------------------
+// The same scheme as gemv_q4k_mfma_kernel for Q4_0's 32-weight blocks.  The tiled copy holds, per (sixteen rows, 512 columns),
+// four kilobytes of nibbles as [j][lane] 16 bytes (lane (n, g) owns blocks 4 j + g, j = 0..3, of row n) and then [lane][j] fp16
+// scales: four contiguous 1 KB loads and one of 512 bytes per wavefront and tile.  The four MFMAs of a block (low and high nibbles
+// of its two byte halves) share the block's one scale and hence one accumulator: w = d (n - 8) = d (16 acc - 1032 Sx_first16 -
+// 72 Sx_last16) with the low nibbles read as 64 + n / 16 and the high ones as 4 + n / 16 (staged beside the activations per block).
+constexpr size_t kQ40TileBytes = 4608;
+// rounds whose partial sums have an LDS slot of their own (KS > 1): sixteen at 4096 columns (a 128256-row head needs eleven), eight
+// at 14336 columns, where four activation rows leave no room for more
+constexpr int q40_rounds(int tpr) { return tpr >= 28 ? 8 : 16; }
+struct Q40Item { uint4 q[4]; uint2 d; };
+
+template <int NB, int TPR, int WAVES, int KS, int MODE>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t *tiled, const void *activations, const float *norm_w, int rows, int iters,
+                                                                   int workgroups, float norm_eps, KernelArgs rest) {
+    KernelArgs a = rest;
+    a.rows = rows;
+    if constexpr (MODE == 1) { a.norm_x = static_cast<const float *>(activations); a.norm_w = norm_w; a.norm_eps = norm_eps; }
+    else if constexpr (MODE == 2) a.merge_partials = static_cast<const float *>(activations);
+    else a.x = static_cast<const uint16_t *>(activations);
+    constexpr int THREADS = WAVES * 64, cols = TPR * 512, IPR = cols / 64, S = TPR / KS, RB = WAVES / KS, GROUPS = cols / 8;
+    constexpr int DEPTH = S % 4 == 0 ? 4 : (S % 7 == 0 ? 7 : (S % 2 == 0 ? 2 : 1));   // divides S: a step's slot in the ring is a constant
+    constexpr int SETS = (NB + 3) / 4;
+    static_assert(TPR % KS == 0 && WAVES % KS == 0 && NB >= 1 && NB <= 8, "whole tiles per wavefront");
+    extern __shared__ uint4 smem_raw[];
+    uint4 *xs4 = smem_raw;                                        // [NB][GROUPS] groups of eight fp16, (0,2,1,3) order inside fours
+    uint4 *zero4 = xs4 + (size_t)NB * GROUPS;                     // eight groups of zeros
+    float *xsum = reinterpret_cast<float *>(zero4 + 8);           // [NB][cols / 32]: the offset term of every block
+    float *red = xsum + (size_t)NB * (cols / 32);                 // [q40_rounds(TPR)][WAVES][NB][16]   (KS > 1)
+    float *misc = red + (KS > 1 ? q40_rounds(TPR) * WAVES * NB * 16 : 0);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = lane >> 4, ks = wave % KS, team = wave / KS;
+    const int row_blocks = (a.rows + 15) >> 4;
+    u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x54005400u, magic_hi = 0x44004400u;
+    asm volatile("" : "+s"(mask_lo), "+s"(mask_hi));
+    asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
+
+    {
+        const int units = (row_blocks + RB - 1) / RB;
+        iters = (units - (int)blockIdx.x + workgroups - 1) / workgroups;   // ragged last round for the lowest workgroups
+        if (iters < 0) iters = 0;
+    }
+    const int total_steps = iters * S;
+    auto block_of = [&](int round) { return (round * workgroups + (int)blockIdx.x) * RB + team; };
+    auto load_step = [&](int f) {   // unconditional: steps past the end read bytes that every lane shares
+        Q40Item it;
+        const bool real = f < total_steps;
+        const int round = f / S, step = f - round * S;
+        const int rb = block_of(round) < row_blocks ? block_of(round) : row_blocks - 1;
+        const uint8_t *tp = real ? tiled + ((size_t)rb * TPR + (ks * S + step)) * kQ40TileBytes : tiled;
+        const int spread = real ? 16 : 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) it.q[j] = *reinterpret_cast<const uint4 *>(tp + (real ? 1024 * j : 0) + spread * lane);
+        it.d = *reinterpret_cast<const uint2 *>(tp + (real ? 4096 : 0) + (real ? 8 : 0) * lane);
+        return it;
+    };
+
+    stamp(a, 0);
+    MfmaStage<NB, IPR, THREADS, MODE, true> stage;
+    stage.issue(a);
+    Q40Item ring[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) ring[d] = load_step(d);
+    if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
+    stage.finish(a, xs4, xsum, misc);
+    __syncthreads();
+    stamp(a, 1);
+
+    // A operand: slot i = lane % 16 carries activation row i % 4 in lane group i / 4 only; group index of (tile step, j, fragment f)
+    // = 64 step + 16 j + 4 g + f
+    const int slot = lane & 15;
+    const uint4 *a_base[SETS];
+    int a_stride[SETS], a_jstride[SETS];
+#pragma unroll
+    for (int set = 0; set < SETS; set++) {
+        const bool feeds = (slot >> 2) == g && 4 * set + (slot & 3) < NB;
+        a_base[set] = feeds ? xs4 + (size_t)(4 * set + (slot & 3)) * GROUPS + 64 * (ks * S) + 4 * g : zero4;
+        a_stride[set] = feeds ? 64 : 0;
+        a_jstride[set] = feeds ? 16 : 0;
+    }
+    const float *xsum_base = xsum + 16 * (ks * S) + g;
+
+    float v[NB];
+    auto step_compute = [&](const Q40Item &it, int i) {
+        const u32 dw[2] = {it.d.x, it.d.y};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            floatx4 acc[SETS];
+#pragma unroll
+            for (int set = 0; set < SETS; set++) acc[set] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            const u32 w0 = it.q[j].x, w1 = it.q[j].y, w2 = it.q[j].z, w3 = it.q[j].w;
+            const uint4 pl0 = make_uint4((w0 & mask_lo) | magic_lo, ((w0 >> 8) & mask_lo) | magic_lo, (w1 & mask_lo) | magic_lo, ((w1 >> 8) & mask_lo) | magic_lo);
+            const uint4 pl1 = make_uint4((w2 & mask_lo) | magic_lo, ((w2 >> 8) & mask_lo) | magic_lo, (w3 & mask_lo) | magic_lo, ((w3 >> 8) & mask_lo) | magic_lo);
+            const uint4 ph0 = make_uint4((w0 & mask_hi) | magic_hi, ((w0 >> 8) & mask_hi) | magic_hi, (w1 & mask_hi) | magic_hi, ((w1 >> 8) & mask_hi) | magic_hi);
+            const uint4 ph1 = make_uint4((w2 & mask_hi) | magic_hi, ((w2 >> 8) & mask_hi) | magic_hi, (w3 & mask_hi) | magic_hi, ((w3 >> 8) & mask_hi) | magic_hi);
+#pragma unroll
+            for (int set = 0; set < SETS; set++) {
+                const uint4 *ap = a_base[set] + i * a_stride[set] + j * a_jstride[set];
+                acc[set] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[0]), __builtin_bit_cast(half8, pl0), acc[set], 0, 0, 0);
+                acc[set] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[1]), __builtin_bit_cast(half8, pl1), acc[set], 0, 0, 0);
+                acc[set] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[2]), __builtin_bit_cast(half8, ph0), acc[set], 0, 0, 0);
+                acc[set] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[3]), __builtin_bit_cast(half8, ph1), acc[set], 0, 0, 0);
+            }
+            const float d = half_bits_to_float((dw[j >> 1] >> (16 * (j & 1))) & 0xFFFFu);
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                const float c = xsum_base[(size_t)b * (cols >> 5) + 16 * i + 4 * j];
+                v[b] += d * (16.0f * acc[b >> 2][b & 3] - c);
+            }
+        }
+    };
+
+    float best[NB];
+    int best_i[NB];
+#pragma unroll
+    for (int b = 0; b < NB; b++) { best[b] = -INFINITY; best_i[b] = 0x7FFFFFFF; }
+    auto finish_block = [&](int rb, float (&sum)[NB]) {
+        if (a.epilogue == EPI_ARGMAX) {
+            const int row = rb * 16 + lane;
+            if (lane < 16 && row < a.rows) {
+#pragma unroll
+                for (int b = 0; b < NB; b++) argmax_take(best[b], best_i[b], sum[b], row);
+            }
+            return;
+        }
+        float other[NB];
+#pragma unroll
+        for (int b = 0; b < NB; b++) other[b] = dpp_term<0xB1, 0xF>(sum[b]);
+        if (lane < 16 && (lane & 1) == 0 && rb < row_blocks) pair_epilogue<NB>(a, rb * 8 + (lane >> 1), sum, other);
+    };
+
+    for (int round = 0; round < iters; round++) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) v[b] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < S; i++) {
+            const Q40Item it = ring[i % DEPTH];
+            ring[i % DEPTH] = load_step(round * S + i + DEPTH);
+            step_compute(it, i);
+            if (a.stamps && round == 0 && i == 0) { if (v[0] != 12345.678f) stamp(a, 2); }
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            v[b] += __shfl_xor(v[b], 16);
+            v[b] += __shfl_xor(v[b], 32);
+        }
+        if constexpr (KS == 1) {
+            finish_block(block_of(round), v);
+        } else {
+            float *slot_base = red + ((size_t)(round % q40_rounds(TPR)) * WAVES + wave) * NB * 16;
+            if (lane < 16) {
+#pragma unroll
+                for (int b = 0; b < NB; b++) slot_base[b * 16 + lane] = v[b];
+            }
+        }
+    }
+    if constexpr (KS > 1) {
+        __syncthreads();
+        if (ks == 0) {   // the team's shares in wavefront order, then the epilogue
+            for (int round = 0; round < iters; round++) {
+                float sum[NB];
+#pragma unroll
+                for (int b = 0; b < NB; b++) {
+                    float t = 0.0f;
+                    if (lane < 16) {
+#pragma unroll
+                        for (int w = 0; w < KS; w++) t += red[((size_t)(round % q40_rounds(TPR)) * WAVES + wave + w) * NB * 16 + b * 16 + lane];
+                    }
+                    sum[b] = t;
+                }
+                finish_block(block_of(round), sum);
+            }
+        }
+    }
+    stamp(a, 3);
+    if (a.epilogue == EPI_ARGMAX) {
+        float *cv = misc;
+        int *ci = reinterpret_cast<int *>(misc + NB * WAVES);
+        __syncthreads();
 #pragma unroll
         for (int b = 0; b < NB; b++) {
 #pragma unroll
@@ -1427,6 +1629,91 @@ hipError_t launch_fmt(const KernelArgs &a, int batch, hipStream_t stream) {
     return hipErrorInvalidValue;
 }
 
+
+template <int NB, int TPR, int WAVES, int KS, int MODE>
+hipError_t launch_q40_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
+    constexpr int RB = WAVES / KS, cols = TPR * 512, THREADS = WAVES * 64;
+    *launched = false;
+    const size_t lds = ((size_t)NB * (cols / 8) + 8) * 16 + (size_t)NB * (cols / 32) * 4 + (KS > 1 ? (size_t)q40_rounds(TPR) * WAVES * NB * 16 * 4 : 0) +
+                       (size_t)2 * NB * WAVES * 4;
+    if (lds > 160 * 1024) return hipSuccess;   // not launched
+    auto kernel = gemv_q40_mfma_kernel<NB, TPR, WAVES, KS, MODE>;
+    static size_t configured_lds = 0;
+    hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
+    if (e != hipSuccess) return e;
+    static int resident_per_cu = 0;
+    if (resident_per_cu == 0) {
+        int n = 0;
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, THREADS, lds);
+        if (e != hipSuccess) return e;
+        const int limit = q4k_wgs_per_cu();
+        resident_per_cu = n < 1 ? 1 : (n > limit ? limit : n);
+    }
+    const int row_blocks = (a.rows + 15) / 16;
+    const int want = (row_blocks + RB - 1) / RB;
+    const int cap = compute_units() * resident_per_cu;
+    const int grid = want < cap ? want : cap;
+    const int iters = (want + grid - 1) / grid;
+    if (KS > 1 && iters > q40_rounds(TPR)) return hipSuccess;   // not launched: the caller takes the other kernel
+    const void *activations = MODE == 1 ? static_cast<const void *>(a.norm_x) : MODE == 2 ? static_cast<const void *>(a.merge_partials) : static_cast<const void *>(a.x);
+    launch_kernel(kernel, dim3(grid), dim3(THREADS), lds, stream, a.tiled, activations, a.norm_w, a.rows, iters, grid, a.norm_eps, a);
+    *launched = true;
+    return hipGetLastError();
+}
+
+// "q40_mfma" (ESPRESSO_HIP_Q40_MFMA): 0 never, 1 wherever an instantiation exists, -1 the default (two and more activation rows,
+// and single rows of matrices with 2048 rows and more: 1024 x 4096 measures 3.7 against 3.3 us on the dot-product kernel).
+int g_q40_mfma_mode = -2;
+int q40_mfma_mode() {
+    if (g_q40_mfma_mode == -2) g_q40_mfma_mode = env_int("ESPRESSO_HIP_Q40_MFMA", -1);
+    return g_q40_mfma_mode;
+}
+
+template <int NB>
+hipError_t try_q40_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
+    *launched = false;
+    if (!a.tiled) return hipSuccess;
+    const int mode = a.merge_partials ? 2 : a.norm_x ? 1 : 0;
+    int waves = q4k_mfma_waves(), ks = q4k_mfma_split();
+    if (a.cols == 4096) {
+        // measured (us, one / two / four rows): 14336 rows 8 x 8 9.2 / 9.5 / 11.0, 8 x 4 9.4 / 9.9 / 11.4, 4 x 2 9.7 / 10.7 / 12.6;
+        // 28672 rows 13.6 / 14.3 / 16.1, 14.6 / 15.6 / 18.0, 16.3 / 17.5 / 20.5; the dot-product kernel 9.9 / 12.2 / 15.6 and 17.2 / 22.0 / 28.8
+        if (waves == 0) waves = 8;
+        if (ks == 0 || ks > waves) ks = waves;
+#define ESP_Q40_CASE(W_, KS_)                                                                                    \
+        if (waves == W_ && ks == KS_) {                                                                          \
+            if (mode == 0) return launch_q40_mfma<NB, 8, W_, KS_, 0>(a, stream, launched);                        \
+            if (mode == 1) return launch_q40_mfma<NB, 8, W_, KS_, 1>(a, stream, launched);                        \
+            if constexpr (NB <= 2) return launch_q40_mfma<NB, 8, W_, KS_, 2>(a, stream, launched);                \
+        }
+        ESP_Q40_CASE(4, 2)
+        ESP_Q40_CASE(8, 4)
+        ESP_Q40_CASE(8, 8)
+#undef ESP_Q40_CASE
+        return hipSuccess;
+    }
+    if (a.cols == 14336 && mode == 0) {
+        // 4096 rows: 14 x 14 10.5 / 11.4 / 13.7, 7 x 7 10.4 / 11.6 / 14.6; the dot-product kernel 10.8 / 14.2 / 25.1
+        if (waves == 0) waves = 14;
+        if (ks == 0) ks = waves == 8 ? 4 : waves;
+        if (waves == 7 && ks == 7) return launch_q40_mfma<NB, 28, 7, 7, 0>(a, stream, launched);
+        if (waves == 14 && ks == 14) return launch_q40_mfma<NB, 28, 14, 14, 0>(a, stream, launched);
+        if (waves == 14 && ks == 7) return launch_q40_mfma<NB, 28, 14, 7, 0>(a, stream, launched);
+        if (waves == 8 && ks == 4) return launch_q40_mfma<NB, 28, 8, 4, 0>(a, stream, launched);
+        return hipSuccess;
+    }
+    return hipSuccess;
+}
+
+template <int B>
+hipError_t launch_q40(const KernelArgs &a, hipStream_t stream) {
+    if (q40_mfma_mode() == 1 || (q40_mfma_mode() < 0 && (B >= 2 || a.rows >= 2048))) {
+        bool launched = false;
+        const hipError_t e = try_q40_mfma<B>(a, stream, &launched);
+        if (e != hipSuccess || launched) return e;
+    }
+    return launch_fmt<FMT_Q4_0>(a, B, stream);
+}
 }  // namespace
 
 bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch, int head_dim) {
@@ -1442,6 +1729,7 @@ bool gemv_set_tuning(const char *key, int value) {
     if (k == "q4k_mfma_ks") { g_q4k_mfma_split = value; return true; }
     if (k == "q4k_mfma_waves") { g_q4k_mfma_waves = value; return true; }
     if (k == "q4k_mfma_ragged") { g_q4k_mfma_ragged = value; return true; }
+    if (k == "q40_mfma") { g_q40_mfma_mode = value; return true; }
     return false;
 }
 
@@ -1449,6 +1737,7 @@ bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
     if (batch <= 2) return true;
     // (eight rows of 14336 columns do not fit the kernel's LDS staging in one pass and stay on the nibble-B GEMM kernel)
     // and so do five to eight rows of the long 4096-column matrices, where that kernel measures faster: 15.3 against 17.1 us at 14336 rows)
+    if (w.format == FMT_Q4_0) return w.tiled && q40_mfma_mode() != 0 && batch <= 4 && (w.cols == 4096 || w.cols == 14336);
     if (w.format != FMT_Q4_K || !w.tiled || q4k_mfma_mode() == 0 || batch > 8) return false;
     return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (w.cols == 4096 && w.rows <= 8192);
 }
@@ -1519,7 +1808,13 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
                 if (e == hipSuccess && !launched) e = hipErrorInvalidValue;
             } else e = nb == 1 ? launch_q4k<1>(a, stream) : nb == 2 ? launch_q4k<2>(a, stream) : launch_q4k<4>(a, stream);
             break;
-        case FMT_Q4_0: e = launch_fmt<FMT_Q4_0>(a, nb, stream); break;
+        case FMT_Q4_0:
+            if (nb == 4) {   // four rows only on the matrix cores; where that kernel declines the shape, two rows at a time
+                bool launched = false;
+                e = try_q40_mfma<4>(a, stream, &launched);
+                if (e == hipSuccess && !launched) { nb = 2; e = launch_q40<2>(a, stream); }
+            } else e = nb == 1 ? launch_q40<1>(a, stream) : launch_q40<2>(a, stream);
+            break;
         case FMT_Q8_0: e = launch_fmt<FMT_Q8_0>(a, nb, stream); break;
         case FMT_F16: e = launch_fmt<FMT_F16>(a, nb, stream); break;
         case FMT_F32: e = launch_fmt<FMT_F32>(a, nb, stream); break;

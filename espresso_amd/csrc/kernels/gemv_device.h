@@ -174,10 +174,14 @@ __device__ __forceinline__ void q4k_store_group(const uint4 &v, int b, int g, in
 }
 
 // The same for the matrix-core GEMV: groups of eight in their natural places, [b][cols / 8], sums of each 32 alongside.
+// Q40: the term that removes the nibble offsets of a Q4_0 block instead, 1032 x (sum of the first sixteen) + 72 x (sum of the last
+// sixteen): w = d (n - 8) with the low nibbles read as 64 + n / 16 and the high ones as 4 + n / 16.
+template <bool Q40 = false>
 __device__ __forceinline__ void q4k_store_group_natural(const uint4 &v, int b, int g, int cols, uint4 *xs4, float *xsum) {
     xs4[(size_t)b * (cols >> 3) + g] = swap_middle(v);
     float s = ((float)as_h2(v.x).x + (float)as_h2(v.x).y) + ((float)as_h2(v.y).x + (float)as_h2(v.y).y) +
               ((float)as_h2(v.z).x + (float)as_h2(v.z).y) + ((float)as_h2(v.w).x + (float)as_h2(v.w).y);
+    if constexpr (Q40) s *= (g & 2) ? 72.0f : 1032.0f;
     s += dpp_term<0xB1, 0xF>(s);
     s += dpp_term<0x4E, 0xF>(s);
     if ((threadIdx.x & 3) == 0) xsum[(size_t)b * (cols >> 5) + (g >> 2)] = s;
