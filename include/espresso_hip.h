@@ -120,7 +120,10 @@ int esp_gemv_stamps(const ESPMatrix *matrix, int batch, int launches, uint64_t *
 /* Kernel-selection switches for measurements and tests (no counterpart in the reference); the same switches are read from
  * the environment when first needed.  "q4k_mfma" (ESPRESSO_HIP_Q4K_MFMA): 1 = Q4_K GEMVs of 4096 / 14336 columns run on the
  * matrix cores (one to eight activation rows per pass over the weights), 0 = never, -1 = the library's own choice.
- * "q4k_mfma_ks" (ESPRESSO_HIP_Q4K_MFMA_KS): wavefronts that share a block of sixteen rows, 1 / 2 / 4, 0 = by shape.
+ * "q40_mfma" (ESPRESSO_HIP_Q40_MFMA): the same for Q4_0 (one to four rows).
+ * "q4k_mfma_ks" / "q4k_mfma_waves" (ESPRESSO_HIP_Q4K_MFMA_KS / _WAVES): wavefronts that share a block of sixteen rows and
+ * wavefronts per workgroup, 0 = by shape; combinations without a compiled kernel fall back to the dot-product kernels.
+ * "q4k_mfma_ragged": 0 = every workgroup runs the same number of rounds.
  * Runtimes that captured a step graph keep the kernels they captured. */
 int esp_set_tuning(const char *key, int value);
 /* Measurement aid with no counterpart in the reference: a kernel that only streams `bytes` (>= 1 MiB, a
