@@ -1483,6 +1483,11 @@ int q4k_mfma_split() {
     if (g_q4k_mfma_split == -2) g_q4k_mfma_split = env_int("ESPRESSO_HIP_Q4K_MFMA_KS", 0);
     return g_q4k_mfma_split;
 }
+int g_q4k_mfma_max_rows = -2;   // single activation rows: matrices with more rows stay on the dot-product kernel (0: no limit)
+int q4k_mfma_max_rows() {
+    if (g_q4k_mfma_max_rows == -2) g_q4k_mfma_max_rows = env_int("ESPRESSO_HIP_Q4K_MFMA_MAX_ROWS", 0);
+    return g_q4k_mfma_max_rows;
+}
 int q4k_mfma_waves() {
     if (g_q4k_mfma_waves == -2) g_q4k_mfma_waves = env_int("ESPRESSO_HIP_Q4K_MFMA_WAVES", 0);
     return g_q4k_mfma_waves;
@@ -1534,10 +1539,12 @@ hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
         //   4096 rows: 16 x 16 5.5 / 6.1, 8 x 8 5.8 / 6.5;  6144 rows: 8 x 8 6.3 / 7.0, 16 x 16 6.4 / 7.2;
         //   28672 rows: 8 x 8 13.8 / 15.4, 4 x 2 14.7 / 15.8; with two rows and more the long matrices prefer 4 x 2
         //   two rows: 14336 rows 8 x 8 9.8, 4 x 2 10.0; 28672 rows 4 x 2 16.4, 8 x 8 17.6.  Eight rows: 4096 rows 8 x 8 8.7, 16 x 16 10.9
+        //   second sweep (another box; one / two / four rows): 28672 rows 8 x 8 14.7 / 15.5 / 17.5, 4 x 2 15.9 / 16.6 / 19.9; 128256 rows
+        //   (the output head; splits of K decline it, too many rounds) 4 x 1 53.9 / 57.2 / 67.2, dot-product kernel 60.6 / 71.1 / 92.6
         if (waves == 0 && ks == 0) {
             if (a.rows <= 4096 && NB <= 4) waves = ks = 16;
-            else if (a.rows <= 16384 || NB == 1) waves = ks = 8;
-            else { waves = 4; ks = 2; }
+            else if (a.rows <= 32768) waves = ks = 8;
+            else { waves = 4; ks = 1; }
         }
         if (waves == 0) waves = 8;
         if (ks == 0 || ks > waves) ks = waves;
@@ -1574,9 +1581,9 @@ hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
 template <int B>
 hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     const bool norm = a.norm_x != nullptr;
-    // By default the matrix-core kernel takes two rows and more, and single rows of the 4096-column matrices except the
-    // output head (for the head and for 14336 columns the dot-product kernel measures the same or better at one row).
-    if (q4k_mfma_mode() == 1 || (q4k_mfma_mode() < 0 && (B >= 2 || (a.cols == 4096 && a.rows <= 65536)))) {
+    // By default the matrix-core kernel takes two rows and more, and single rows of the 4096-column matrices (for 14336 columns
+    // the dot-product kernel measures the same or better at one row).
+    if (q4k_mfma_mode() == 1 || (q4k_mfma_mode() < 0 && (B >= 2 || (a.cols == 4096 && (q4k_mfma_max_rows() <= 0 || a.rows <= q4k_mfma_max_rows()))))) {
         bool launched = false;
         const hipError_t e = try_q4k_mfma<B>(a, stream, &launched);
         if (e != hipSuccess || launched) return e;
@@ -1730,6 +1737,7 @@ bool gemv_set_tuning(const char *key, int value) {
     if (k == "q4k_mfma_waves") { g_q4k_mfma_waves = value; return true; }
     if (k == "q4k_mfma_ragged") { g_q4k_mfma_ragged = value; return true; }
     if (k == "q40_mfma") { g_q40_mfma_mode = value; return true; }
+    if (k == "q4k_mfma_max_rows") { g_q4k_mfma_max_rows = value; return true; }
     return false;
 }
 
