@@ -9,6 +9,40 @@ namespace {
 using Clock = std::chrono::steady_clock;
 double ms_since(Clock::time_point t0) { return std::chrono::duration<double, std::milli>(Clock::now() - t0).count(); }
 
+// A pass of a generation loop as a captured graph: the first pass runs as plain launches (whatever a kernel configures on its first
+// use happens outside the capture), later ones replay.
+struct PassGraph {
+    hipGraphExec_t exec = nullptr;
+    ~PassGraph() { if (exec) (void)hipGraphExecDestroy(exec); }
+    template <class Enqueue>
+    int capture(Enqueue enqueue) {
+        hipStream_t s = context().stream;
+        hipGraph_t graph = nullptr;
+        hipError_t e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+        if (e != hipSuccess) return fail_hip(e, "hipStreamBeginCapture");
+        int rc = enqueue();
+        e = hipStreamEndCapture(s, &graph);
+        if (rc == ESP_OK && e != hipSuccess) rc = fail_hip(e, "hipStreamEndCapture");
+        if (rc == ESP_OK && (e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0)) != hipSuccess) rc = fail_hip(e, "hipGraphInstantiate");
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
+    }
+    int launch(int times) {
+        for (int i = 0; i < times; i++) {
+            const hipError_t e = hipGraphLaunch(exec, context().stream);
+            if (e != hipSuccess) return fail_hip(e, "hipGraphLaunch");
+        }
+        return ESP_OK;
+    }
+};
+template <class T>
+struct DeviceArray {
+    T *p = nullptr;
+    ~DeviceArray() { if (p) (void)hipFree(p); }
+    int alloc(size_t count) { return device_alloc(&p, count); }
+};
+int hip_ok(hipError_t e, const char *what) { return e == hipSuccess ? ESP_OK : fail_hip(e, what); }
+
 // One pass of the exact two-token loop with every decision on the device (TwoTokenState): the draft runs two rows (the row
 // it owes after an accepted pass and the current token, or the current token twice) and proposes; the target verifies
 // (current, proposed); the accept kernel emits, keeps the hidden row and writes the next pass's rows.  No host decision, so
@@ -358,7 +392,39 @@ int generate_greedy_batch(LlamaRuntime &rt, const uint32_t *const *prompts, cons
             if ((rc = rt.select_greedy(s, &current[s])) != ESP_OK) return rc;
             (*out)[s].push_back(current[s]);
         }
-        for (int step = 1; step < eff; step++) {
+        int first_host_step = 1;
+        if (rt.graph_replay_enabled() && eff > 2) {
+            // every step but none of the decisions needs the host: rows feed themselves on the device, one graph per step
+            hipStream_t st = context().stream;
+            const int steps = eff - 1;
+            DeviceArray<int> d_log, d_step;
+            if ((rc = d_log.alloc((size_t)steps * n_seq)) != ESP_OK || (rc = d_step.alloc(1)) != ESP_OK) return rc;
+            StepRows rows{};
+            rows.count = n_seq;
+            for (int s = 0; s < n_seq; s++) { rows.token[s] = (int)current[s]; rows.pos[s] = rt.visible(s); rows.seq[s] = s; }
+            if ((rc = hip_ok(launch_set_rows(rows, rt.device_row_tokens(), rt.device_row_positions(), rt.device_row_sequences(), st), "rows")) != ESP_OK) return rc;
+            if ((rc = hip_ok(launch_set_ints(d_step.p, 0, nullptr, 0, st), "step")) != ESP_OK) return rc;
+            auto pass = [&]() {
+                int r = rt.enqueue_device_rows(n_seq);
+                if (r == ESP_OK) r = rt.enqueue_device_head(n_seq);
+                if (r == ESP_OK) r = hip_ok(launch_batch_greedy_feed(rt.device_head_tokens(), n_seq, rt.device_row_tokens(), rt.device_row_positions(), d_log.p,
+                                                                     d_step.p, steps, st), "feed");
+                return r;
+            };
+            PassGraph graph;
+            if ((rc = pass()) != ESP_OK) return rc;
+            if ((rc = graph.capture(pass)) != ESP_OK) return rc;
+            if ((rc = graph.launch(steps - 1)) != ESP_OK) return rc;
+            std::vector<int> log((size_t)steps * n_seq);
+            if ((rc = hip_ok(hipMemcpyAsync(log.data(), d_log.p, sizeof(int) * log.size(), hipMemcpyDeviceToHost, st), "log")) != ESP_OK) return rc;
+            if ((rc = hip_ok(hipStreamSynchronize(st), "greedy batch")) != ESP_OK) return rc;
+            for (int s = 0; s < n_seq; s++) {
+                for (int i = 0; i < steps; i++) (*out)[s].push_back((uint32_t)log[(size_t)i * n_seq + s]);
+                rt.set_visible(s, rt.visible(s) + steps);
+            }
+            first_host_step = eff;
+        }
+        for (int step = first_host_step; step < eff; step++) {
             StepRows rows{};
             rows.count = n_seq;
             for (int s = 0; s < n_seq; s++) { rows.token[s] = (int)current[s]; rows.pos[s] = rt.visible(s); rows.seq[s] = s; }
@@ -398,6 +464,66 @@ int generate_two_token_batch(LlamaRuntime &full, LlamaRuntime &draft, const uint
         for (int s = 0; s < n_seq; s++) {
             if ((rc = full.select_greedy(s, &current[s])) != ESP_OK) return rc;
             (*out)[s].push_back(current[s]);
+        }
+    }
+    if (full.graph_replay_enabled() && draft.graph_replay_enabled() && &full != &draft && eff > 2 && n_seq <= kMaxLoopSequences) {
+        // the passes run on the device: per-sequence variables in TwoTokenBatchState, rows 2 s and 2 s + 1 of both models belong to
+        // sequence s, a sequence whose budget is spent keeps replaying its last rows (which rewrite the same values)
+        hipStream_t strm = context().stream;
+        TwoTokenBatchState h{};
+        h.n_seq = n_seq; h.budget = eff;
+        StepRows rows{};
+        rows.count = 2 * n_seq;
+        for (int s = 0; s < n_seq; s++) {
+            h.current[s] = (int)current[s]; h.full_pos[s] = full.visible(s); h.emitted[s] = 1;
+            for (int k = 0; k < 2; k++) { rows.token[2 * s + k] = (int)current[s]; rows.pos[2 * s + k] = full.visible(s); rows.seq[2 * s + k] = s; }
+        }
+        DeviceArray<TwoTokenBatchState> d_state;
+        DeviceArray<int> d_log;
+        if ((rc = d_state.alloc(1)) != ESP_OK || (rc = d_log.alloc((size_t)n_seq * eff)) != ESP_OK) return rc;
+        if ((rc = hip_ok(hipMemcpyAsync(d_state.p, &h, sizeof(h), hipMemcpyHostToDevice, strm), "state")) != ESP_OK) return rc;
+        if ((rc = hip_ok(launch_set_rows(rows, draft.device_row_tokens(), draft.device_row_positions(), draft.device_row_sequences(), strm), "rows")) != ESP_OK) return rc;
+        if ((rc = hip_ok(launch_set_rows(rows, full.device_row_tokens(), full.device_row_positions(), full.device_row_sequences(), strm), "rows")) != ESP_OK) return rc;
+        auto pass = [&]() {
+            int r = draft.enqueue_device_rows(2 * n_seq);
+            if (r == ESP_OK) r = draft.enqueue_device_head(2 * n_seq);
+            if (r == ESP_OK) r = hip_ok(launch_two_token_batch_verify_rows(d_state.p, draft.device_head_tokens(), full.device_row_tokens(), full.device_row_positions(), strm), "verify rows");
+            if (r == ESP_OK) r = full.enqueue_device_rows(2 * n_seq);
+            if (r == ESP_OK) r = full.enqueue_device_head(2 * n_seq);
+            if (r == ESP_OK) r = hip_ok(launch_two_token_batch_accept(d_state.p, n_seq, full.device_head_tokens(), d_log.p, full.device_hidden_rows(), full.device_last_hidden(0),
+                                                                      full.config().d_model, draft.device_row_tokens(), draft.device_row_positions(), strm), "accept");
+            return r;
+        };
+        auto fetch = [&]() {
+            int r = hip_ok(hipMemcpyAsync(&h, d_state.p, sizeof(h), hipMemcpyDeviceToHost, strm), "state");
+            if (r == ESP_OK) r = hip_ok(hipStreamSynchronize(strm), "two-token batch pass");
+            return r;
+        };
+        auto fewest = [&]() { int m = h.emitted[0]; for (int s = 1; s < n_seq; s++) m = h.emitted[s] < m ? h.emitted[s] : m; return m; };
+        PassGraph graph;
+        if ((rc = pass()) != ESP_OK || (rc = fetch()) != ESP_OK) return rc;
+        while (fewest() < eff) {
+            if (!graph.exec && (rc = graph.capture(pass)) != ESP_OK) return rc;
+            const int left = eff - fewest();
+            if ((rc = graph.launch(left / 2 > 1 ? left / 2 : 1)) != ESP_OK || (rc = fetch()) != ESP_OK) return rc;
+        }
+        std::vector<int> log((size_t)n_seq * eff);
+        if ((rc = hip_ok(hipMemcpyAsync(log.data(), d_log.p, sizeof(int) * log.size(), hipMemcpyDeviceToHost, strm), "log")) != ESP_OK) return rc;
+        if ((rc = hip_ok(hipStreamSynchronize(strm), "two-token batch log")) != ESP_OK) return rc;
+        StepRows owed{};
+        for (int s = 0; s < n_seq; s++) {
+            for (int i = 1; i < eff; i++) (*out)[s].push_back((uint32_t)log[(size_t)s * eff + i]);
+            st.committed_total += h.committed[s]; st.accepted_total += h.accepted[s];
+            if ((rc = full.set_visible(s, h.full_pos[s])) != ESP_OK) return rc;
+            if ((rc = draft.set_visible(s, h.full_pos[s] - (h.accepted_prev[s] ? 1 : 0))) != ESP_OK) return rc;
+            if (h.accepted_prev[s]) {   // the row the draft still owes, as the host loop runs it at the end of an accepting pass
+                owed.token[owed.count] = h.proposed_prev[s]; owed.pos[owed.count] = draft.visible(s); owed.seq[owed.count] = s; owed.count++;
+            }
+        }
+        st.passes += h.passes;
+        if (owed.count > 0) {
+            if ((rc = draft.forward_rows(owed)) != ESP_OK) return rc;
+            for (int i = 0; i < owed.count; i++) draft.set_visible(owed.seq[i], owed.pos[i] + 1);
         }
     }
     auto active = [&](int s) { return (int)(*out)[s].size() < eff; };

@@ -116,6 +116,21 @@ struct TwoTokenState {
 hipError_t launch_two_token_verify_rows(TwoTokenState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, hipStream_t s);
 // After the target's two rows went through its head: emits one or two tokens into log, keeps the matching hidden row of the
 // target (d floats from hidden_rows into last_hidden), advances the state and writes the draft's two rows of the next pass.
+// The same loop over up to sixteen sequences in lock step (rows 2 s and 2 s + 1 of both models belong to sequence s), and the plain
+// greedy loop over several sequences: per-sequence variables in device memory, every pass one captured graph.
+constexpr int kMaxLoopSequences = kMaxStepRows / 2;
+struct TwoTokenBatchState {
+    int n_seq, budget, passes;
+    int current[kMaxLoopSequences], full_pos[kMaxLoopSequences], accepted_prev[kMaxLoopSequences], proposed_prev[kMaxLoopSequences];
+    int proposed[kMaxLoopSequences], can_two[kMaxLoopSequences], live[kMaxLoopSequences], emitted[kMaxLoopSequences];
+    int committed[kMaxLoopSequences], accepted[kMaxLoopSequences];
+};
+hipError_t launch_two_token_batch_verify_rows(TwoTokenBatchState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, hipStream_t s);
+// log: [n_seq][budget] tokens; last_hidden: [sequence][d]
+hipError_t launch_two_token_batch_accept(TwoTokenBatchState *state, int n_seq, const int *target_head_tokens, int *log, const float *hidden_rows,
+                                         float *last_hidden, int d, int *draft_tokens, int *draft_pos, hipStream_t s);
+// Greedy step of n sequences: the head's tokens become the next rows at the next positions and go to log[step][n].
+hipError_t launch_batch_greedy_feed(const int *head_tokens, int n, int *tokens, int *pos, int *log, int *step, int capacity_steps, hipStream_t s);
 hipError_t launch_two_token_accept(TwoTokenState *state, const int *target_head_tokens, int *log, int log_capacity, const float *hidden_rows,
                                    float *last_hidden, int d, int *draft_tokens, int *draft_pos, hipStream_t s);
 hipError_t launch_copy_rows(const float *src, float *dst, int rows, int d, hipStream_t s);

@@ -983,7 +983,97 @@ __global__ __launch_bounds__(256) void two_token_accept_kernel(TwoTokenState *st
         for (int i = threadIdx.x; i < d; i += 256) last_hidden[i] = hidden_rows[(size_t)keep * d + i];
 }
 
+// One thread per sequence: see launch_two_token_batch_verify_rows.
+__global__ void two_token_batch_verify_rows_kernel(TwoTokenBatchState *st, const int *draft_head, int *tokens, int *pos) {
+    const int s = threadIdx.x;
+    if (s >= st->n_seq) return;
+    const bool live = st->emitted[s] < st->budget;
+    st->live[s] = live ? 1 : 0;
+    if (!live) return;                       // finished: its rows stay what they were, the pass recomputes the same values
+    const int proposed = draft_head[2 * s + 1];
+    const bool can_two = st->budget - st->emitted[s] >= 2;
+    st->proposed[s] = proposed;
+    st->can_two[s] = can_two ? 1 : 0;
+    tokens[2 * s] = st->current[s];                            pos[2 * s] = st->full_pos[s];
+    tokens[2 * s + 1] = can_two ? proposed : st->current[s];   pos[2 * s + 1] = st->full_pos[s] + (can_two ? 1 : 0);
+}
+
+// One workgroup per sequence: thread 0 runs the sequence's bookkeeping, then the workgroup keeps its hidden row.
+__global__ __launch_bounds__(256) void two_token_batch_accept_kernel(TwoTokenBatchState *st, const int *head, int *log, const float *hidden_rows,
+                                                                      float *last_hidden, int d, int *draft_tokens, int *draft_pos) {
+    __shared__ int keep;
+    const int s = blockIdx.x;
+    if (threadIdx.x == 0) {
+        keep = -1;
+        if (s == 0) {
+            int any = 0;
+            for (int i = 0; i < st->n_seq; i++) any |= st->live[i];
+            if (any) st->passes += 1;
+        }
+        if (st->live[s]) {
+            const int e0 = head[2 * s], e1 = head[2 * s + 1], proposed = st->proposed[s];
+            int *out = log + (size_t)s * st->budget;
+            out[st->emitted[s]] = e0;
+            st->emitted[s] += 1; st->committed[s] += 1;
+            if (!(st->can_two[s] && proposed == e0)) {
+                st->full_pos[s] += 1; st->current[s] = e0; st->accepted_prev[s] = 0;
+                keep = 2 * s;
+            } else {
+                st->accepted[s] += 1; st->committed[s] += 1;
+                st->full_pos[s] += 2;
+                out[st->emitted[s]] = e1;
+                st->emitted[s] += 1; st->current[s] = e1;
+                st->accepted_prev[s] = 1; st->proposed_prev[s] = proposed;
+                keep = 2 * s + 1;
+            }
+            if (st->emitted[s] < st->budget) {   // the draft's rows of the next pass
+                if (st->accepted_prev[s]) {
+                    draft_tokens[2 * s] = st->proposed_prev[s]; draft_pos[2 * s] = st->full_pos[s] - 1;
+                    draft_tokens[2 * s + 1] = st->current[s];   draft_pos[2 * s + 1] = st->full_pos[s];
+                } else {
+                    draft_tokens[2 * s] = draft_tokens[2 * s + 1] = st->current[s];
+                    draft_pos[2 * s] = draft_pos[2 * s + 1] = st->full_pos[s];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (keep >= 0)
+        for (int i = threadIdx.x; i < d; i += 256) last_hidden[(size_t)s * d + i] = hidden_rows[(size_t)keep * d + i];
+}
+
+__global__ void batch_greedy_feed_kernel(const int *head_tokens, int n, int *tokens, int *pos, int *log, int *step, int capacity_steps) {
+    const int s = threadIdx.x, at = *step;
+    __syncthreads();
+    if (s < n) {
+        const int t = head_tokens[s];
+        tokens[s] = t;
+        pos[s] += 1;
+        if (at < capacity_steps) log[(size_t)at * n + s] = t;
+    }
+    if (s == 0) *step = at + 1;
+}
+
 }  // namespace
+
+hipError_t launch_two_token_batch_verify_rows(TwoTokenBatchState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, hipStream_t s) {
+    hipLaunchKernelGGL(two_token_batch_verify_rows_kernel, dim3(1), dim3(64), 0, s, state, draft_head_tokens, target_tokens, target_pos);
+    return hipGetLastError();
+}
+
+hipError_t launch_two_token_batch_accept(TwoTokenBatchState *state, int n_seq, const int *target_head_tokens, int *log, const float *hidden_rows,
+                                         float *last_hidden, int d, int *draft_tokens, int *draft_pos, hipStream_t s) {
+    if (n_seq < 1 || n_seq > kMaxLoopSequences) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(two_token_batch_accept_kernel, dim3(n_seq), dim3(256), 0, s, state, target_head_tokens, log, hidden_rows, last_hidden, d,
+                       draft_tokens, draft_pos);
+    return hipGetLastError();
+}
+
+hipError_t launch_batch_greedy_feed(const int *head_tokens, int n, int *tokens, int *pos, int *log, int *step, int capacity_steps, hipStream_t s) {
+    if (n < 1 || n > kMaxStepRows) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(batch_greedy_feed_kernel, dim3(1), dim3(64), 0, s, head_tokens, n, tokens, pos, log, step, capacity_steps);
+    return hipGetLastError();
+}
 
 hipError_t launch_two_token_verify_rows(TwoTokenState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, hipStream_t s) {
     hipLaunchKernelGGL(two_token_verify_rows_kernel, dim3(1), dim3(64), 0, s, state, draft_head_tokens, target_tokens, target_pos);

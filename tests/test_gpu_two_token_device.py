@@ -111,3 +111,44 @@ def test_stop_token_and_context_end_on_the_device(llama):
     tokens, _ = both_ways(llama, target, draft, prompt, 40)
     assert tokens == plain[:17 - len(prompt)]
     target.close(); draft.close()
+
+
+def build_batch(ll, packed, fmt, n_layer, max_seq, n_seq):
+    cfg = ll.MultiModelConfig(n_layer=n_layer, max_seq=max_seq, **BASE)
+    rt = ll.LlamaRuntime(cfg, max_sequences=n_seq)
+    ll.load_packed_weights(rt, dict(packed, layers=packed["layers"][:n_layer]), fmt)
+    return rt
+
+
+@pytest.mark.parametrize("n_seq", [1, 3, 16])
+def test_lock_step_loops_on_the_device_equal_the_host_loops(llama, n_seq):
+    """generate_batch (plain greedy and the exact two-token loop over several sequences): passes replayed as graphs with the
+    per-sequence variables on the device against the host-driven loops - the same streams, counters and visible counts."""
+    fmt = orc.FMT_Q8_0
+    rng = np.random.default_rng(n_seq)
+    prompts = [rng.integers(0, BASE["vocab"], int(rng.integers(3, 9))).astype(np.uint32) for _ in range(n_seq)]
+    for label, upper in (("never agrees", None), ("sometimes", 0.15), ("always", 0.0)):
+        if upper is None:
+            target = build_batch(llama, weights(fmt, 21, 3), fmt, 3, 64, n_seq)
+            draft = build_batch(llama, weights(fmt, 22, 1), fmt, 1, 64, n_seq)
+        else:
+            packed = weights(fmt, 23, 3, upper)
+            target, draft = build_batch(llama, packed, fmt, 3, 64, n_seq), build_batch(llama, packed, fmt, 1, 64, n_seq)
+        for budget in (1, 2, 3, 4, 9, 30):
+            runs = {}
+            for on_device in (True, False):
+                for d in (None, draft):
+                    llama.set_graph_replay(target, on_device)
+                    target.reset(); draft.reset()
+                    toks, st = llama.generate_batch(target, prompts, budget, draft=d)
+                    runs[(on_device, d is not None)] = (toks, (st["passes"], st["committed_total"], st["accepted_total"]),
+                                                        [target.visible(s) for s in range(n_seq)], [draft.visible(s) for s in range(n_seq)])
+            llama.set_graph_replay(target, True)
+            assert runs[(True, False)] == runs[(False, False)], (label, budget, "plain greedy")
+            assert runs[(True, True)] == runs[(False, True)], (label, budget, "two-token")
+            assert runs[(True, True)][0] == runs[(True, False)][0]                  # the exact loop gives the greedy streams
+            assert all(len(t) == budget for t in runs[(True, True)][0])
+            if label == "always" and budget == 30:
+                passes, committed, accepted = runs[(True, True)][1]
+                assert accepted == 14 * n_seq and committed == 29 * n_seq and passes == 15
+        target.close(); draft.close()
