@@ -1699,7 +1699,7 @@ hipError_t try_q40_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
 #undef ESP_Q40_CASE
         return hipSuccess;
     }
-    if (a.cols == 14336 && mode == 0) {
+    if constexpr (NB <= 4) if (a.cols == 14336 && mode == 0) {
         // 4096 rows: 14 x 14 10.5 / 11.4 / 13.7, 7 x 7 10.4 / 11.6 / 14.6; the dot-product kernel 10.8 / 14.2 / 25.1
         if (waves == 0) waves = 14;
         if (ks == 0) ks = waves == 8 ? 4 : waves;
@@ -1745,7 +1745,9 @@ bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
     if (batch <= 2) return true;
     // (eight rows of 14336 columns do not fit the kernel's LDS staging in one pass and stay on the nibble-B GEMM kernel)
     // and so do five to eight rows of the long 4096-column matrices, where that kernel measures faster: 15.3 against 17.1 us at 14336 rows)
-    if (w.format == FMT_Q4_0) return w.tiled && q40_mfma_mode() != 0 && batch <= 4 && (w.cols == 4096 || w.cols == 14336);
+    if (w.format == FMT_Q4_0)
+        // (five to eight rows: up to 8192 x 4096 8.7 against 10.7 us on the nibble-B kernel, at 14336 rows 18.9 against 17.1)
+        return w.tiled && q40_mfma_mode() != 0 && (batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (batch <= 8 && w.cols == 4096 && w.rows <= 8192));
     if (w.format != FMT_Q4_K || !w.tiled || q4k_mfma_mode() == 0 || batch > 8) return false;
     return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (w.cols == 4096 && w.rows <= 8192);
 }
@@ -1817,9 +1819,9 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
             } else e = nb == 1 ? launch_q4k<1>(a, stream) : nb == 2 ? launch_q4k<2>(a, stream) : launch_q4k<4>(a, stream);
             break;
         case FMT_Q4_0:
-            if (nb == 4) {   // four rows only on the matrix cores; where that kernel declines the shape, two rows at a time
+            if (nb >= 4) {   // four and eight rows only on the matrix cores; where that kernel declines the shape, two rows at a time
                 bool launched = false;
-                e = try_q40_mfma<4>(a, stream, &launched);
+                e = nb == 8 ? try_q40_mfma<8>(a, stream, &launched) : try_q40_mfma<4>(a, stream, &launched);
                 if (e == hipSuccess && !launched) { nb = 2; e = launch_q40<2>(a, stream); }
             } else e = nb == 1 ? launch_q40<1>(a, stream) : launch_q40<2>(a, stream);
             break;

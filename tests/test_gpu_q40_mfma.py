@@ -33,7 +33,7 @@ def test_matches_oracle_and_dot_product_kernel(mods, rows, cols):
     rng = np.random.default_rng(rows)
     scale = np.abs(deq).max() * np.sqrt(cols)
     variants = ((0, 0), (4, 2), (8, 4), (8, 8)) if cols == 4096 else ((0, 0), (7, 7), (14, 14), (14, 7), (8, 4))
-    for batch in (1, 2, 3, 4, 5):
+    for batch in (1, 2, 3, 4, 5, 8):
         x = rng.normal(0, 1, (batch, cols)).astype(np.float16)
         res = rng.normal(0, 1, (batch, rows)).astype(np.float32)
         want = np.stack([orc.matvec(deq, x[b].astype(np.float32)) for b in range(batch)])
@@ -45,9 +45,9 @@ def test_matches_oracle_and_dot_product_kernel(mods, rows, cols):
             ops.set_tuning("q4k_mfma_waves", waves)
             ops.set_tuning("q4k_mfma_ks", ks)
             y = mat.gemv(x)
-            # exact products, fp32 sums: only the order of additions differs from the oracle's (five rows and more take the
-            # MFMA GEMM kernels, whose weights are d (n - 8) rounded to fp16)
-            tol = (2e-5 if batch <= 4 else 3e-4) * scale
+            # exact products, fp32 sums: only the order of additions differs from the oracle's (five rows and more of the larger
+            # matrices take the MFMA GEMM kernels, whose weights are d (n - 8) rounded to fp16)
+            tol = (2e-5 if batch <= 4 or (cols == 4096 and rows <= 8192) else 3e-4) * scale
             assert np.abs(y - want).max() <= tol + 1e-6, (batch, waves, ks, float(np.abs(y - want).max()), scale)
             assert np.array_equal(mat.gemv(x).view(np.uint32), y.view(np.uint32))      # deterministic
             yr = mat.gemv(x, res)
