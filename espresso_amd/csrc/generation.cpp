@@ -134,18 +134,27 @@ int generate_greedy(LlamaRuntime &rt, const uint32_t *prompt, int prompt_count, 
 
     auto t_start = Clock::now(), t_emit = t_start;
     int all = prompt_count;
-    if (c.eos_token < 0 && eff > 1) {
-        // No stop token: the first eff-1 tokens need no host decision, so they run as graph replays with
-        // one synchronisation; the last token is selected but not advanced, as in the loop below.
+    if (eff > 1) {
+        // The first eff-1 tokens need no host decision (the step graph notices a stop token by itself), so they run as graph
+        // replays with a synchronisation at the end or every 32 tokens; the last token is selected but not advanced, as in the
+        // loop below.
         out->resize(eff - 1);
-        if ((rc = rt.continue_greedy(0, eff - 1, out->data())) != ESP_OK) return rc;
-        all += eff - 1;
-        if (timing) {
-            const double per_token = ms_since(t_start) / (eff - 1);
+        int produced = eff - 1;
+        if (c.eos_token < 0) rc = rt.continue_greedy(0, eff - 1, out->data());
+        else rc = rt.continue_greedy_until_stop(0, eff - 1, out->data(), &produced);
+        if (rc != ESP_OK) return rc;
+        out->resize(produced);
+        all += produced;
+        if (timing && produced > 0) {
+            const double per_token = ms_since(t_start) / produced;
             timing->first_token_latency_ms = per_token;
-            timing->token_latencies_ms.assign(eff - 1, per_token);   // one measurement for the whole run
+            timing->token_latencies_ms.assign(produced, per_token);   // one measurement for the whole run
         }
         t_emit = Clock::now();
+        if (produced > 0 && c.eos_token >= 0 && out->back() == (uint32_t)c.eos_token) {   // EOS is appended, then the loop ends (:6385-6388)
+            if (timing) timing->decode_ms = ms_since(t_start);
+            return ESP_OK;
+        }
     }
     while ((int)out->size() < eff) {
         uint32_t next = 0;

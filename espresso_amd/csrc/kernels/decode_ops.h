@@ -88,13 +88,15 @@ hipError_t launch_greedy_feed(const int *next_token, int seq, int *visible, int 
 // that reduces them, feeds the token as launch_greedy_feed does and writes its embedding row to hidden[0..d).
 hipError_t launch_greedy_step_tail(const float *logits, int vocab, int *out_token, const ArgmaxScratch &scratch, int seq, int *visible,
                                    int *tokens, int *pos, int *seqs, int *log, int *log_count, int log_capacity, const void *table,
-                                   bool table_is_f16, int d, float *hidden, hipStream_t s);
+                                   bool table_is_f16, int d, float *hidden, int eos, hipStream_t s);
 // The same two steps for a head GEMV that left one (value, index) pair per workgroup instead of logits (EPI_ARGMAX):
 // `blocks` pairs per row in scratch, rows `blocks` apart.
 hipError_t launch_argmax_final(const ArgmaxScratch &scratch, int blocks, int rows, int *out_token, hipStream_t s);
 hipError_t launch_greedy_tail(const ArgmaxScratch &scratch, int blocks, int *out_token, int seq, int *visible, int *tokens, int *pos, int *seqs,
                               int *log, int *log_count, int log_capacity, const void *table, bool table_is_f16, int d, float *hidden,
-                              hipStream_t s);
+                              int eos, hipStream_t s);
+// log_count points at three ints: tokens logged so far, stopped (set by the kernel when it emits the stop token `eos` while the third
+// int, set by the host, is non-zero), stop enabled.  A stopped sequence's replays emit nothing and recompute the row they computed last.
 hipError_t launch_set_ints(int *dst0, int v0, int *dst1, int v1, hipStream_t s);
 
 // Device-resident state of the exact two-token loop over one sequence (generateIncrementalExactTwoTokenDraftLlama,

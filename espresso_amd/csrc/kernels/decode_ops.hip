@@ -879,11 +879,12 @@ struct GreedyTailArgs {
     int nblk;
     int *out_token;
     int seq;
-    int *visible, *tokens, *pos, *seqs, *log, *log_count;
+    int *visible, *tokens, *pos, *seqs, *log, *log_count;   // log_count: [tokens logged, stopped, stop at the stop token (set by the host)]
     int log_capacity;
     const void *table;
     int table_is_f16, d;
     float *hidden;
+    int eos;
 };
 __global__ __launch_bounds__(kBlock) void greedy_tail_kernel(GreedyTailArgs a) {
     __shared__ float bv[kBlock];
@@ -896,17 +897,32 @@ __global__ __launch_bounds__(kBlock) void greedy_tail_kernel(GreedyTailArgs a) {
         if (better(v, idx, best, best_i)) { best = v; best_i = idx; }
     }
     argmax_block_reduce(best, best_i, bv, bi);
-    const int t = best_i == 0x7FFFFFFF ? 0 : best_i;
+    int t = best_i == 0x7FFFFFFF ? 0 : best_i;
+    __shared__ int feed;   // the token whose embedding the trunk after this kernel runs on
     if (threadIdx.x == 0) {
-        a.out_token[0] = t;
-        a.tokens[0] = t;
-        a.pos[0] = a.visible[a.seq];
-        a.seqs[0] = a.seq;
-        const int n = *a.log_count;
-        if (n < a.log_capacity) a.log[n] = t;
-        *a.log_count = n + 1;
-        a.visible[a.seq] += 1;
+        if (a.log_count[1]) {
+            // stopped in an earlier replay: nothing is emitted, and the trunk recomputes the row it computed last (same token, same
+            // position, same values), so replays past the stop change nothing
+            feed = a.tokens[0];
+        } else {
+            a.out_token[0] = t;
+            const int n = a.log_count[0];
+            if (n < a.log_capacity) a.log[n] = t;
+            a.log_count[0] = n + 1;
+            if (a.eos >= 0 && a.log_count[2] && t == a.eos) {   // the stop token is emitted, not consumed (:6385-6388)
+                a.log_count[1] = 1;
+                feed = a.tokens[0];
+            } else {
+                a.tokens[0] = t;
+                a.pos[0] = a.visible[a.seq];
+                a.seqs[0] = a.seq;
+                a.visible[a.seq] += 1;
+                feed = t;
+            }
+        }
     }
+    __syncthreads();
+    t = feed;
     const size_t row = (size_t)t * a.d;
     for (int i = threadIdx.x; i < a.d; i += kBlock)
         a.hidden[i] = a.table_is_f16 ? from_half_bits(reinterpret_cast<const uint16_t *>(a.table)[row + i])
@@ -1216,23 +1232,23 @@ hipError_t launch_argmax_final(const ArgmaxScratch &scratch, int blocks, int row
 }
 
 hipError_t launch_greedy_tail(const ArgmaxScratch &scratch, int blocks, int *out_token, int seq, int *visible, int *tokens, int *pos, int *seqs,
-                              int *log, int *log_count, int log_capacity, const void *table, bool table_is_f16, int d, float *hidden,
+                              int *log, int *log_count, int log_capacity, const void *table, bool table_is_f16, int d, float *hidden, int eos,
                               hipStream_t s) {
     if (!scratch.part_value || !scratch.part_index || blocks < 1) return hipErrorInvalidValue;
     GreedyTailArgs a{scratch.part_value, scratch.part_index, blocks, out_token, seq, visible, tokens, pos, seqs, log, log_count, log_capacity,
-                     table, table_is_f16 ? 1 : 0, d, hidden};
+                     table, table_is_f16 ? 1 : 0, d, hidden, eos};
     hipLaunchKernelGGL(greedy_tail_kernel, dim3(1), dim3(kBlock), 0, s, a);
     return hipGetLastError();
 }
 
 hipError_t launch_greedy_step_tail(const float *logits, int vocab, int *out_token, const ArgmaxScratch &scratch, int seq, int *visible,
                                    int *tokens, int *pos, int *seqs, int *log, int *log_count, int log_capacity, const void *table,
-                                   bool table_is_f16, int d, float *hidden, hipStream_t s) {
+                                   bool table_is_f16, int d, float *hidden, int eos, hipStream_t s) {
     if (!scratch.part_value || !scratch.part_index) return hipErrorInvalidValue;
     const int blocks = vocab < kArgmaxBlocks * kBlock ? (vocab + kBlock - 1) / kBlock : kArgmaxBlocks;
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(blocks, 1), dim3(kBlock), 0, s, logits, vocab, scratch.part_value, scratch.part_index);
     GreedyTailArgs a{scratch.part_value, scratch.part_index, blocks, out_token, seq, visible, tokens, pos, seqs, log, log_count, log_capacity,
-                     table, table_is_f16 ? 1 : 0, d, hidden};
+                     table, table_is_f16 ? 1 : 0, d, hidden, eos};
     hipLaunchKernelGGL(greedy_tail_kernel, dim3(1), dim3(kBlock), 0, s, a);
     return hipGetLastError();
 }

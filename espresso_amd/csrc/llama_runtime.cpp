@@ -395,7 +395,7 @@ int LlamaRuntime::finalize() {
     if ((rc = device_alloc(&d_out_tokens_, R)) != ESP_OK) return rc;
     if ((rc = device_alloc(&d_visible_, (size_t)c_.max_sequences)) != ESP_OK) return rc;
     if ((rc = device_alloc(&d_log_, (size_t)c_.max_seq)) != ESP_OK) return rc;
-    if ((rc = device_alloc(&d_log_count_, 1)) != ESP_OK) return rc;
+    if ((rc = device_alloc(&d_log_count_, 3)) != ESP_OK) return rc;   // tokens logged, stopped, stop enabled (greedy_tail_kernel)
     step_graphs_.assign(c_.max_sequences, nullptr);
     // one (value, index) pair per workgroup of the head GEMV and row: a workgroup owns eight rows, or the grid is persistent
     head_partial_capacity_ = (c_.vocab + 7) / 8 > 4096 ? (c_.vocab + 7) / 8 : 4096;
@@ -750,13 +750,13 @@ int LlamaRuntime::capture_step_graph(int seq) {
             e = launch_gemv(g, s);
             if (e == hipSuccess)
                 e = launch_greedy_tail(argmax_scratch_, blocks, d_out_tokens_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_, d_log_count_,
-                                       c_.max_seq, embedding_, embedding_f16_, c_.d_model, hidden_, s);
+                                       c_.max_seq, embedding_, embedding_f16_, c_.d_model, hidden_, c_.eos_token, s);
         } else {
             g.y = logits_; g.epilogue = EPI_STORE_F32;
             e = launch_gemv(g, s);
             if (e == hipSuccess)
                 e = launch_greedy_step_tail(logits_, c_.vocab, d_out_tokens_, argmax_scratch_, seq, d_visible_, d_tokens_, d_pos_, d_seq_, d_log_,
-                                            d_log_count_, c_.max_seq, embedding_, embedding_f16_, c_.d_model, hidden_, s);
+                                            d_log_count_, c_.max_seq, embedding_, embedding_f16_, c_.d_model, hidden_, c_.eos_token, s);
         }
         if (e != hipSuccess) rc = fail_hip(e, "greedy step head");
         if (rc == ESP_OK) rc = enqueue_trunk(1, true, kept);
@@ -802,12 +802,68 @@ int LlamaRuntime::continue_greedy(int seq, int steps, uint32_t *out_tokens) {
         if (steps == 0) return ESP_OK;
     }
     ESP_HIP_TRY(launch_set_ints(d_visible_ + seq, visible_[seq], d_log_count_, 0, s));
+    ESP_HIP_TRY(launch_set_ints(d_log_count_ + 1, 0, d_log_count_ + 2, 0, s));   // not stopped, and no stop at the stop token
     for (int i = 0; i < steps; i++) ESP_HIP_TRY(hipGraphLaunch(step_graphs_[seq], s));
     std::vector<int> log(steps);
     ESP_HIP_TRY(hipMemcpyAsync(log.data(), d_log_, sizeof(int) * steps, hipMemcpyDeviceToHost, s));
     ESP_HIP_TRY(hipStreamSynchronize(s));
     visible_[seq] += steps;
     if (out_tokens) for (int i = 0; i < steps; i++) out_tokens[i] = (uint32_t)log[i];
+    return ESP_OK;
+}
+
+// continue_greedy that ends with the stop token: the token is emitted and not consumed, as in the reference loop (:6385-6388).  The
+// replays run in chunks; the step graph itself notices the stop token, and replays after it change nothing.
+int LlamaRuntime::continue_greedy_until_stop(int seq, int steps, uint32_t *out_tokens, int *produced) {
+    if (!finalized_) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+    if (seq < 0 || seq >= c_.max_sequences || !out_tokens || !produced) return fail(ESP_ERR_OUT_OF_RANGE, "continue_greedy_until_stop(seq %d)", seq);
+    *produced = 0;
+    if (steps < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "steps must be >= 0");
+    if (visible_[seq] + steps > c_.max_seq)
+        return fail(ESP_ERR_OUT_OF_RANGE, "runtime position %d + %d steps exceeds context %d", visible_[seq], steps, c_.max_seq);
+    const int eos = c_.eos_token;
+    hipStream_t s = context().stream;
+    int rc;
+    auto eager_step = [&](bool *stopped) {
+        uint32_t t = 0;
+        int r = select_greedy(seq, &t);
+        if (r != ESP_OK) return r;
+        out_tokens[(*produced)++] = t;
+        *stopped = eos >= 0 && t == (uint32_t)eos;
+        return *stopped ? ESP_OK : advance(seq, t);
+    };
+    bool stopped = false;
+    if (!use_graph_ || timing_enabled_) {
+        while (*produced < steps && !stopped)
+            if ((rc = eager_step(&stopped)) != ESP_OK) return rc;
+        return ESP_OK;
+    }
+    if (steps > 0 && !step_graphs_[seq]) {   // one eager step first: it configures every kernel's LDS limit outside the capture
+        if ((rc = eager_step(&stopped)) != ESP_OK) return rc;
+        if (stopped) return ESP_OK;
+        if ((rc = capture_step_graph(seq)) != ESP_OK) return rc;
+    }
+    if (*produced >= steps) return ESP_OK;
+    const int first = *produced, want = steps - first;
+    ESP_HIP_TRY(launch_set_ints(d_visible_ + seq, visible_[seq], d_log_count_, 0, s));
+    ESP_HIP_TRY(launch_set_ints(d_log_count_ + 1, 0, d_log_count_ + 2, 1, s));
+    int state[2] = {0, 0};   // tokens logged, stopped
+    for (int launched = 0; launched < want && !state[1];) {
+        const int chunk = want - launched < 32 ? want - launched : 32;
+        for (int i = 0; i < chunk; i++) ESP_HIP_TRY(hipGraphLaunch(step_graphs_[seq], s));
+        launched += chunk;
+        ESP_HIP_TRY(hipMemcpyAsync(state, d_log_count_, sizeof(state), hipMemcpyDeviceToHost, s));
+        ESP_HIP_TRY(hipStreamSynchronize(s));
+    }
+    const int logged = state[0] < want ? state[0] : want;
+    std::vector<int> log(logged > 0 ? logged : 1);
+    if (logged > 0) {
+        ESP_HIP_TRY(hipMemcpyAsync(log.data(), d_log_, sizeof(int) * logged, hipMemcpyDeviceToHost, s));
+        ESP_HIP_TRY(hipStreamSynchronize(s));
+    }
+    for (int i = 0; i < logged; i++) out_tokens[first + i] = (uint32_t)log[i];
+    *produced = first + logged;
+    visible_[seq] += logged - (state[1] ? 1 : 0);   // every logged token was consumed, except a stop token
     return ESP_OK;
 }
 

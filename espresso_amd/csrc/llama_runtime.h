@@ -63,6 +63,9 @@ class LlamaRuntime {
     // `steps` greedy tokens from the sequence's current state (select, then advance, per token) as
     // replays of one captured HIP graph per token; the host synchronises once at the end.
     int continue_greedy(int seq, int steps, uint32_t *out_tokens);
+    // The same, ending early at the configuration's stop token: the stop token is emitted (it is the last of *produced tokens) and not
+    // consumed.  The step graph notices it on the device; the host looks once per 32 replays.
+    int continue_greedy_until_stop(int seq, int steps, uint32_t *out_tokens, int *produced);
     void set_use_graph(bool enabled) { use_graph_ = enabled; }
     // Prompts of kMatrixPrefillMinTokens or more run in blocks through the MFMA kernels (default on).
     void set_matrix_prefill(bool enabled) { matrix_prefill_ = enabled; }
