@@ -517,13 +517,14 @@ __device__ __forceinline__ void q4k_store(const uint4 &v, int b, int g, int cols
     else q4k_store_group(v, b, g, cols, xstride, xs4, xsum);
 }
 
-template <int B, int IPR, bool NORM, bool NATURAL = false>
+template <int B, int IPR, bool NORM, bool NATURAL = false, int THREADS = kThreads>
 struct Q4KStage {
+    static_assert(!NORM || THREADS == kThreads, "the fused RMSNorm adds four wavefronts' sums");
     static_assert(IPR % 4 == 0, "whole super-blocks per row");
-    static constexpr int GROUPS = IPR * 8, K = (GROUPS + kThreads - 1) / kThreads, cols = IPR * 64, XSTRIDE = IPR | 1;
+    static constexpr int GROUPS = IPR * 8, K = (GROUPS + THREADS - 1) / THREADS, cols = IPR * 64, XSTRIDE = IPR | 1;
     // Threads past the last group load group 0 and drop it: a guarded load becomes a branch, and
     // each branch waits for its own round trip to the L2, while clamped loads all issue at once.
-    static constexpr bool FULL = GROUPS % kThreads == 0;
+    static constexpr bool FULL = GROUPS % THREADS == 0;
     float4 v0[NORM ? B : 1][K], v1[NORM ? B : 1][K], g0[K], g1[K];   // NORM: fp32 values and norm weights
     uint4 v[NORM ? 1 : B][K];                                        // otherwise: fp16 values
 
@@ -536,8 +537,8 @@ struct Q4KStage {
             const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
             for (int k = 0; k < K; k++) {
-                const bool in = FULL || tid + k * kThreads < GROUPS;   // whole quads of lanes: GROUPS is a multiple of 32
-                const int g = in ? tid + k * kThreads : 0;
+                const bool in = FULL || tid + k * THREADS < GROUPS;   // whole quads of lanes: GROUPS is a multiple of 32
+                const int g = in ? tid + k * THREADS : 0;
                 g0[k] = w4[2 * g];
                 g1[k] = w4[2 * g + 1];
 #pragma unroll
@@ -553,7 +554,7 @@ struct Q4KStage {
             for (int b = 0; b < B; b++)
 #pragma unroll
                 for (int k = 0; k < K; k++)
-                    v[b][k] = reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + (FULL || tid + k * kThreads < GROUPS ? tid + k * kThreads : 0)];
+                    v[b][k] = reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + (FULL || tid + k * THREADS < GROUPS ? tid + k * THREADS : 0)];
         }
     }
 
@@ -569,15 +570,15 @@ struct Q4KStage {
                 const float inv = 1.0f / sqrtf(workgroup_sum(s, red + b * kWaves) / (float)cols + a.norm_eps);
 #pragma unroll
                 for (int k = 0; k < K; k++)
-                    if (FULL || tid + k * kThreads < GROUPS)
-                        q4k_store<NATURAL>(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
+                    if (FULL || tid + k * THREADS < GROUPS)
+                        q4k_store<NATURAL>(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, tid + k * THREADS, cols, XSTRIDE, xs4, xsum);
             }
         } else {
 #pragma unroll
             for (int b = 0; b < B; b++)
 #pragma unroll
                 for (int k = 0; k < K; k++)
-                    if (FULL || tid + k * kThreads < GROUPS) q4k_store<NATURAL>(v[b][k], b, tid + k * kThreads, cols, XSTRIDE, xs4, xsum);
+                    if (FULL || tid + k * THREADS < GROUPS) q4k_store<NATURAL>(v[b][k], b, tid + k * THREADS, cols, XSTRIDE, xs4, xsum);
         }
     }
 };
@@ -621,8 +622,10 @@ struct Q4KMergeStage {
 constexpr int kDeferredRounds = 16;   // rounds whose team reductions wait for one barrier at the end of the kernel
 
 // MODE: 0 = fp16 activations as given, 1 = RMSNorm fused into the staging, 2 = attention partial states merged in the staging.
-template <int B, int IPR, int TEAM, int MODE>
-__global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, const void *activations, const float *norm_w, int rows, int row_bytes,
+// WAVES: wavefronts per workgroup (more than four only with activations given as fp16, MODE 0, and TEAM > 1): the activations are
+// staged once per workgroup, so with eight wavefronts a long row's 28 KB of them are read by a third as many workgroups.
+template <int B, int IPR, int TEAM, int MODE, int WAVES = kWaves>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q4k_kernel(const uint8_t *qs, const void *activations, const float *norm_w, int rows, int row_bytes,
                                                             int iters, int workgroups, float norm_eps, KernelArgs rest) {
     // The arguments that the first loads need come as leading scalars: those can be preloaded into registers
     // with the wavefront's launch, where fields of a structure passed by value are fetched from memory first.
@@ -634,13 +637,14 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
     else if constexpr (MODE == 2) a.merge_partials = static_cast<const float *>(activations);
     else a.x = static_cast<const uint16_t *>(activations);
     constexpr int cols = IPR * 64, XSTRIDE = IPR | 1, TOTAL = 2 * IPR, TEAM_LANES = TEAM * 64;
-    constexpr int PASSES = (TOTAL + TEAM_LANES - 1) / TEAM_LANES, TEAMS = kWaves / TEAM;
-    static_assert(PASSES <= 2 && kWaves % TEAM == 0, "pick TEAM so that a lane holds at most two items per pair");
+    constexpr int PASSES = (TOTAL + TEAM_LANES - 1) / TEAM_LANES, TEAMS = WAVES / TEAM;
+    static_assert(WAVES == kWaves || (MODE == 0 && TEAM > 1), "more wavefronts: fp16 activations, teams");
+    static_assert(PASSES <= 2 && WAVES % TEAM == 0, "pick TEAM so that a lane holds at most two items per pair");
     extern __shared__ uint4 smem_raw[];
     uint4 *xs4 = smem_raw;                                                       // [B][8][XSTRIDE] x 8 fp16
     float *xsum = reinterpret_cast<float *>(smem_raw + (size_t)B * 8 * XSTRIDE);  // [B][cols/32]
-    float *red = xsum + (size_t)B * (cols / 32);                                  // [kDeferredRounds][kWaves][2 * B]
-    float *norm_red = red + kDeferredRounds * kWaves * 2 * B;                     // [B][kWaves]
+    float *red = xsum + (size_t)B * (cols / 32);                                  // [kDeferredRounds][WAVES][2 * B]
+    float *norm_red = red + kDeferredRounds * WAVES * 2 * B;                     // [B][kWaves]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tl = (wave % TEAM) * 64 + lane;
     const int n_teams = workgroups * TEAMS, npairs = (a.rows + 1) / 2;
@@ -726,7 +730,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
                 }
             } else if (pair < npairs && lane == 0) pair_epilogue<B>(a, pair, acc_a, acc_b);
         } else {
-            float *slot = red + (size_t)(deferred ? round : (round & 1)) * kWaves * 2 * B;
+            float *slot = red + (size_t)(deferred ? round : (round & 1)) * WAVES * 2 * B;
             if (lane == 0) {
 #pragma unroll
                 for (int b = 0; b < B; b++) { slot[wave * 2 * B + 2 * b] = acc_a[b]; slot[wave * 2 * B + 2 * b + 1] = acc_b[b]; }
@@ -741,7 +745,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
     };
 
     Q4KItem buf0[PASSES], buf1[PASSES];
-    typename std::conditional<MODE == 2, Q4KMergeStage<B, MODE == 2 ? IPR : 32>, Q4KStage<B, IPR, MODE == 1>>::type stage;
+    typename std::conditional<MODE == 2, Q4KMergeStage<B, MODE == 2 ? IPR : 32>, Q4KStage<B, IPR, MODE == 1, false, WAVES * 64>>::type stage;
     const int first_pair = blockIdx.x * TEAMS + wave / TEAM;
     int pair = first_pair;
     stamp(a, 0);
@@ -774,7 +778,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q4k_kernel(const uint8_t *qs, c
             const int p = first_pair + round * n_teams;
             if (round < iters && p < npairs) {
                 float sa[B], sb[B];
-                team_sum(red + (size_t)round * kWaves * 2 * B, sa, sb);
+                team_sum(red + (size_t)round * WAVES * 2 * B, sa, sb);
                 pair_epilogue<B>(a, p, sa, sb);
             }
         }
@@ -1431,11 +1435,11 @@ int compute_units() {
     return v;
 }
 
-template <int B, int IPR, int TEAM, int MODE>
+template <int B, int IPR, int TEAM, int MODE, int WAVES = kWaves>
 hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
-    constexpr int TEAMS = kWaves / TEAM;
-    const size_t lds = (size_t)B * 8 * (IPR | 1) * 16 + (size_t)B * (IPR * 2) * 4 + (size_t)(kDeferredRounds * kWaves * 2 * B + B * kWaves) * 4;
-    auto kernel = gemv_q4k_kernel<B, IPR, TEAM, MODE>;
+    constexpr int TEAMS = WAVES / TEAM;
+    const size_t lds = (size_t)B * 8 * (IPR | 1) * 16 + (size_t)B * (IPR * 2) * 4 + (size_t)(kDeferredRounds * WAVES * 2 * B + B * WAVES) * 4;
+    auto kernel = gemv_q4k_kernel<B, IPR, TEAM, MODE, WAVES>;
     static size_t configured_lds = 0;
     hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
     if (e != hipSuccess) return e;
@@ -1443,7 +1447,7 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     static int resident_per_cu = 0;
     if (resident_per_cu == 0) {
         int n = 0;
-        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, kThreads, lds);
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, WAVES * 64, lds);
         if (e != hipSuccess) return e;
         const int limit = q4k_wgs_per_cu();
         resident_per_cu = n < 1 ? 1 : (n > limit ? limit : n);
@@ -1461,7 +1465,7 @@ hipError_t launch_q4k_persistent(const KernelArgs &a, hipStream_t stream) {
     // ahead by one to three microseconds to the end: one pair less for the later workgroups evens the finish.
     const int iters = (npairs + grid * TEAMS - 1) / (grid * TEAMS);
     const void *activations = MODE == 1 ? static_cast<const void *>(a.norm_x) : MODE == 2 ? static_cast<const void *>(a.merge_partials) : static_cast<const void *>(a.x);
-    launch_kernel(kernel, dim3(grid), dim3(kThreads), lds, stream, a.qs, activations, a.norm_w, a.rows, (int)a.qs_row_bytes, iters, grid, a.norm_eps, a);
+    launch_kernel(kernel, dim3(grid), dim3(WAVES * 64), lds, stream, a.qs, activations, a.norm_w, a.rows, (int)a.qs_row_bytes, iters, grid, a.norm_eps, a);
     return hipGetLastError();
 }
 
@@ -1487,6 +1491,11 @@ int g_q4k_mfma_max_rows = -2;   // single activation rows: matrices with more ro
 int q4k_mfma_max_rows() {
     if (g_q4k_mfma_max_rows == -2) g_q4k_mfma_max_rows = env_int("ESPRESSO_HIP_Q4K_MFMA_MAX_ROWS", 0);
     return g_q4k_mfma_max_rows;
+}
+int g_q4k_long_row_waves = -2;   // wavefronts per workgroup of the dot-product kernel at 14336 columns: 8 (default) or 4
+int q4k_long_row_waves() {
+    if (g_q4k_long_row_waves == -2) g_q4k_long_row_waves = env_int("ESPRESSO_HIP_Q4K_LONG_ROW_WAVES", 8);
+    return g_q4k_long_row_waves;
 }
 int q4k_mfma_waves() {
     if (g_q4k_mfma_waves == -2) g_q4k_mfma_waves = env_int("ESPRESSO_HIP_Q4K_MFMA_WAVES", 0);
@@ -1595,7 +1604,17 @@ hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     case 4096: return norm ? launch_q4k_persistent<B, 64, 1, 1>(a, stream) : launch_q4k_persistent<B, 64, 1, 0>(a, stream);
     case 8192: return norm ? launch_q4k_persistent<B, 128, 2, 1>(a, stream) : launch_q4k_persistent<B, 128, 2, 0>(a, stream);
     case 11008: if (!norm) return launch_q4k_persistent<B, 172, 4, 0>(a, stream); break;
-    case 14336: if (!norm) return launch_q4k_persistent<B, 224, 4, 0>(a, stream); break;
+    case 14336:
+        if (!norm) {
+            // Eight wavefronts (two teams) per workgroup, one workgroup per compute unit: a workgroup stages the row's 28 KB of
+            // activations once, and with a third as many workgroups doing so the last of them has them 2.6 us after the launch
+            // instead of 6.3 us.  Measured in the 8B decode step: 9.3 against 10.2-10.6 us per launch, 704 against 690 tok/s;
+            // twelve and sixteen wavefronts, eight per team and two such workgroups per compute unit (at 128 registers) measure no better
+            // than four.  "q4k_long_row_waves" = 4 restores four wavefronts, three workgroups per compute unit.
+            if (q4k_long_row_waves() == 8) return launch_q4k_persistent<B, 224, 4, 0, 8>(a, stream);
+            return launch_q4k_persistent<B, 224, 4, 0>(a, stream);
+        }
+        break;
     default: break;
     }
     const size_t lds = (size_t)B * 8 * ((a.cols / 64) | 1) * 16 + (size_t)B * (a.cols / 32) * 4 + (size_t)B * kWaves * 4;
@@ -1738,6 +1757,7 @@ bool gemv_set_tuning(const char *key, int value) {
     if (k == "q4k_mfma_ragged") { g_q4k_mfma_ragged = value; return true; }
     if (k == "q40_mfma") { g_q40_mfma_mode = value; return true; }
     if (k == "q4k_mfma_max_rows") { g_q4k_mfma_max_rows = value; return true; }
+    if (k == "q4k_long_row_waves") { g_q4k_long_row_waves = value; return true; }
     return false;
 }
 
