@@ -147,9 +147,9 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # workload (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors kernels of known size in the same runs gave);
 # the runs and the per-kernel table are in profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt.
-MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66524697}
+MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66526737}
 # the same kernel's mean duration in the committed rocprofv3 kernel trace (a profiled run; 3-5 % slower than an unprofiled one)
-PROFILE_KERNEL_US = {("llama3-8b-q4k", "gate_up"): (14.40, "profiles/q4k_gemv_decode_llama3_8b_kernel_trace.txt")}
+PROFILE_KERNEL_US = {("llama3-8b-q4k", "gate_up"): (14.58, "profiles/q4k_gemv_decode_llama3_8b_kernel_trace.txt")}
 TRAFFIC_SOURCE = "profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload; not measured in this run)"
 
 
