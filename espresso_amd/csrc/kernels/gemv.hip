@@ -1040,9 +1040,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
     stamp(a, 0);
     MfmaStage<NB, IPR, THREADS, MODE> stage;
     stage.issue(a);
+    // AHEAD steps (of 2.3 KB per wavefront) are in flight per wavefront.  The ring has a slot per step of a round, up to seven (14336
+    // columns), so that a step's slot is a constant; but a compute unit's memory pipeline takes about 50-70 KB at once, and what is
+    // issued beyond that blocks the issuing wavefront - and with it the barrier below and the start of the arithmetic - until the
+    // first weights have arrived.  Measured in the 8B decode step (same box, alternating): one step ahead instead of two for the
+    // 4096-column kernels with eight wavefronts (two workgroups per compute unit: 37 KB in flight instead of 74) 723 against 711
+    // tok/s; three steps ahead instead of seven at 14336 columns (55 KB per compute unit instead of 129) 9.3 against 11.4 us per
+    // launch, two or four steps ahead measure the same or slightly worse.  Four-step rings stay full: they belong to four-wavefront
+    // workgroups (37 KB per workgroup), and the 128256-row head measures 54.3 us with four steps ahead, 57.0 with two, 67.3 with one.
+    constexpr int AHEAD = DEPTH == 2 ? 1 : DEPTH == 7 ? 3 : DEPTH;
     Q4KItem ring[DEPTH];
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) ring[d] = load_step(d);
+    for (int d = 0; d < AHEAD; d++) ring[d] = load_step(d);
     if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
     stage.finish(a, xs4, xsum, misc);
     __syncthreads();
@@ -1124,7 +1133,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
 #pragma unroll
         for (int i = 0; i < S; i++) {
             const Q4KItem it = ring[i % DEPTH];
-            ring[i % DEPTH] = load_step(round * S + i + DEPTH);
+            ring[(i + AHEAD) % DEPTH] = load_step(round * S + i + AHEAD);
             step_compute(it, i);
             if (a.stamps && round == 0 && i == 0) { if (v[0] != 12345.678f) stamp(a, 2); }   // after the first weights were needed
         }
@@ -1253,9 +1262,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t
     stamp(a, 0);
     MfmaStage<NB, IPR, THREADS, MODE, true> stage;
     stage.issue(a);
+    // steps in flight, as in gemv_q4k_mfma_kernel: with fourteen wavefronts a two-step ring filled up front has 129 KB on its
+    // way before the staging barrier (4096 x 14336: 10.5 / 11.4 / 13.7 us for one / two / four rows; one step ahead 8.7 / 9.8 / 12.1)
+    constexpr int AHEAD = DEPTH == 2 ? 1 : DEPTH;
     Q40Item ring[DEPTH];
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) ring[d] = load_step(d);
+    for (int d = 0; d < AHEAD; d++) ring[d] = load_step(d);
     if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
     stage.finish(a, xs4, xsum, misc);
     __syncthreads();
@@ -1330,7 +1342,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t
 #pragma unroll
         for (int i = 0; i < S; i++) {
             const Q40Item it = ring[i % DEPTH];
-            ring[i % DEPTH] = load_step(round * S + i + DEPTH);
+            ring[(i + AHEAD) % DEPTH] = load_step(round * S + i + AHEAD);
             step_compute(it, i);
             if (a.stamps && round == 0 && i == 0) { if (v[0] != 12345.678f) stamp(a, 2); }
         }
@@ -1492,9 +1504,10 @@ int q4k_mfma_max_rows() {
     if (g_q4k_mfma_max_rows == -2) g_q4k_mfma_max_rows = env_int("ESPRESSO_HIP_Q4K_MFMA_MAX_ROWS", 0);
     return g_q4k_mfma_max_rows;
 }
-int g_q4k_long_row_waves = -2;   // wavefronts per workgroup of the dot-product kernel at 14336 columns: 8 (default) or 4
+// one activation row at 14336 columns: 0 (default) = the matrix-core kernel, 8 or 4 = the dot-product kernel with that many wavefronts per workgroup
+int g_q4k_long_row_waves = -2;
 int q4k_long_row_waves() {
-    if (g_q4k_long_row_waves == -2) g_q4k_long_row_waves = env_int("ESPRESSO_HIP_Q4K_LONG_ROW_WAVES", 8);
+    if (g_q4k_long_row_waves == -2) g_q4k_long_row_waves = env_int("ESPRESSO_HIP_Q4K_LONG_ROW_WAVES", 0);
     return g_q4k_long_row_waves;
 }
 int q4k_mfma_waves() {
@@ -1590,9 +1603,12 @@ hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
 template <int B>
 hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     const bool norm = a.norm_x != nullptr;
-    // By default the matrix-core kernel takes two rows and more, and single rows of the 4096-column matrices (for 14336 columns
-    // the dot-product kernel measures the same or better at one row).
-    if (q4k_mfma_mode() == 1 || (q4k_mfma_mode() < 0 && (B >= 2 || (a.cols == 4096 && (q4k_mfma_max_rows() <= 0 || a.rows <= q4k_mfma_max_rows()))))) {
+    // By default the matrix-core kernel takes two rows and more, and single rows of the 4096- and 14336-column matrices (14336
+    // columns, 4096 rows, one row, in the 8B decode step: 8.3 us on the matrix cores with three steps in flight, 9.3 us on the
+    // eight-wavefront dot-product kernel below, which "q4k_long_row_waves" = 8 or 4 selects).
+    const bool one_row_on_the_matrix_cores = (a.cols == 4096 && (q4k_mfma_max_rows() <= 0 || a.rows <= q4k_mfma_max_rows())) ||
+                                             (a.cols == 14336 && q4k_long_row_waves() == 0);
+    if (q4k_mfma_mode() == 1 || (q4k_mfma_mode() < 0 && (B >= 2 || one_row_on_the_matrix_cores))) {
         bool launched = false;
         const hipError_t e = try_q4k_mfma<B>(a, stream, &launched);
         if (e != hipSuccess || launched) return e;
@@ -1610,8 +1626,8 @@ hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
             // activations once, and with a third as many workgroups doing so the last of them has them 2.6 us after the launch
             // instead of 6.3 us.  Measured in the 8B decode step: 9.3 against 10.2-10.6 us per launch, 704 against 690 tok/s;
             // twelve and sixteen wavefronts, eight per team and two such workgroups per compute unit (at 128 registers) measure no better
-            // than four.  "q4k_long_row_waves" = 4 restores four wavefronts, three workgroups per compute unit.
-            if (q4k_long_row_waves() == 8) return launch_q4k_persistent<B, 224, 4, 0, 8>(a, stream);
+            // than four.  "q4k_long_row_waves" = 4 selects four wavefronts, three workgroups per compute unit.
+            if (q4k_long_row_waves() != 4) return launch_q4k_persistent<B, 224, 4, 0, 8>(a, stream);
             return launch_q4k_persistent<B, 224, 4, 0>(a, stream);
         }
         break;

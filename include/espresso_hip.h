@@ -124,8 +124,8 @@ int esp_gemv_stamps(const ESPMatrix *matrix, int batch, int launches, uint64_t *
  * "q4k_mfma_ks" / "q4k_mfma_waves" (ESPRESSO_HIP_Q4K_MFMA_KS / _WAVES): wavefronts that share a block of sixteen rows and
  * wavefronts per workgroup, 0 = by shape; combinations without a compiled kernel fall back to the dot-product kernels.
  * "q4k_mfma_ragged": 0 = every workgroup runs the same number of rounds.
- * "q4k_long_row_waves" (ESPRESSO_HIP_Q4K_LONG_ROW_WAVES): wavefronts per workgroup of the dot-product kernel at 14336 columns, 8
- * (default: one workgroup per compute unit) or 4 (three per compute unit).
+ * "q4k_long_row_waves" (ESPRESSO_HIP_Q4K_LONG_ROW_WAVES): one activation row at 14336 columns: 0 (default) = the matrix-core
+ * kernel, 8 or 4 = the dot-product kernel with that many wavefronts per workgroup (one or three workgroups per compute unit).
  * Runtimes that captured a step graph keep the kernels they captured. */
 int esp_set_tuning(const char *key, int value);
 /* Measurement aid with no counterpart in the reference: a kernel that only streams `bytes` (>= 1 MiB, a
