@@ -147,9 +147,9 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # workload (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors kernels of known size in the same runs gave);
 # the runs and the per-kernel table are in profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt.
-MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66526737}
-# the same kernel's mean duration in the committed rocprofv3 kernel trace (a profiled run; 3-5 % slower than an unprofiled one)
-PROFILE_KERNEL_US = {("llama3-8b-q4k", "gate_up"): (14.58, "profiles/q4k_gemv_decode_llama3_8b_kernel_trace.txt")}
+MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66521607}
+# the same kernel's mean duration in the committed rocprofv3 kernel trace (a profiled run; 2-4 % slower than an unprofiled one)
+PROFILE_KERNEL_US = {("llama3-8b-q4k", "gate_up"): (13.88, "profiles/q4k_gemv_decode_llama3_8b_kernel_trace.txt")}
 TRAFFIC_SOURCE = "profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload; not measured in this run)"
 
 
@@ -361,6 +361,7 @@ def main() -> None:
     per_token = {"qkv": n_layer, "wo": n_layer, "gate_up": n_layer, "down": n_layer, "head": 1}
     gemv_us = sum(gpu["b2b_us"][k] * n for k, n in per_token.items())
     gemv_bytes = sum(kt[k]["bytes_per_launch"] * n for k, n in per_token.items())
+    gemv_kernel_us = sum(gpu["kernel_us"][k] * n for k, n in per_token.items())
     result = {
         "metric": "decode tok/s bs1 (%s)" % ("8B-arch Q4_K" if args.workload == "llama3-8b-q4k" else "6L d768 Q8_0"),
         "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
@@ -379,6 +380,9 @@ def main() -> None:
                      "bytes_per_launch": d["bytes_per_launch"], "mean_launch_us": d["kernel_us"], "launches_timed": 8 * (1 if dominant == "head" else n_layer),
                      "all_gemv_gbps": gemv_bytes / gemv_us / 1e3 if gemv_us else 0.0,
                      "all_gemv_frac": gemv_bytes / gemv_us / 1e3 / HBM_PEAK_GBPS if gemv_us else 0.0,
+                     "all_gemv_note": "a token's GEMV bytes over its GEMVs' back-to-back periods (kernel + the gap to the next launch); "
+                                      "all_gemv_frac_kernel_durations: over the kernels' own durations (kernel_us), as a kernel trace adds them up",
+                     "all_gemv_frac_kernel_durations": gemv_bytes / gemv_kernel_us / 1e3 / HBM_PEAK_GBPS if gemv_kernel_us else 0.0,
                      "per_kernel": {k: {"mean_us": round(v["mean_us"], 2), "gbps": round(v["gbps"], 1), "launches": v["launches"]}
                                     for k, v in kt.items()},
                      "how": "achieved/mean_launch_us: the dominant kernel launched for each layer's matrix in turn, 8 rounds on the "
