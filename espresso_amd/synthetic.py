@@ -18,9 +18,12 @@ def matrix_shapes(cfg: llama.MultiModelConfig) -> dict:
 
 def build_runtime(cfg: llama.MultiModelConfig, matrix_format: int, seed: int, std: float = 0.02,
                   kv_format: int = _lib.FORMAT_F32, max_sequences: int = 1, keep_packed: bool = False,
-                  head_format: int | None = None):
+                  head_format: int | None = None, zero_upper_outputs: bool = False):
     """Random-init model: every linear ~N(0, std) in `matrix_format`, embedding fp16 ~N(0, std), norm weights 1.
-    Returns (runtime, packed) where packed holds the GGUF-layout bytes when keep_packed is set."""
+    Returns (runtime, packed) where packed holds the GGUF-layout bytes when keep_packed is set.  Tensor seeds do not depend
+    on the layer count, so a model built with fewer layers from the same seed is a prefix of the deeper one.
+    zero_upper_outputs: wo and w2 of every layer above the first are all-zero blocks, i.e. those layers cost what they
+    always cost and add nothing to the residual stream: the model's tokens are those of its first layer alone."""
     rt = llama.LlamaRuntime(cfg, kv_format=kv_format, max_sequences=max_sequences)
     shapes = matrix_shapes(cfg)
     head_format = matrix_format if head_format is None else head_format
@@ -46,7 +49,10 @@ def build_runtime(cfg: llama.MultiModelConfig, matrix_format: int, seed: int, st
         put(l, "rms_ffn", llama.SLOT_RMS_FFN, _lib.FORMAT_F16, ones.view(np.uint8))
         for i, name in enumerate(_TENSORS):
             r, c = shapes[name]
-            data = ops.synth_weights(matrix_format, base + 16 * (l + 1) + i, std, r * c)
+            if zero_upper_outputs and l >= 1 and name in ("wo", "w2"):
+                data = np.zeros(ops.format_bytes(matrix_format, r * c), dtype=np.uint8)
+            else:
+                data = ops.synth_weights(matrix_format, base + 16 * (l + 1) + i, std, r * c)
             put(l, name, llama.LAYER_SLOTS[name], matrix_format, data)
     rt.finalize()
     return rt, packed
