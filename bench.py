@@ -346,18 +346,18 @@ def run_stamps() -> dict:
 
 
 def reader_ceiling(bytes_per_launch: int, gemv_back_to_back_us: float) -> dict:
-    """A kernel with the persistent Q4_K GEMV's grid and loads that only reads: one launch's worth of bytes per launch
+    """A kernel with the matrix-core Q4_K GEMV's grid and loads that only reads: one launch's worth of bytes per launch
     (rotating buffers, back to back) and 1 GiB per launch (the steady state)."""
     import espresso_amd.ops as ops
-    pair = 4608                                        # two rows of 4096 columns
+    pair = 2304                                        # one weight tile: sixteen rows x 256 columns
     n = bytes_per_launch // pair * pair
-    one = ops.hbm_read_probe_pairs(n, pair, 768, max(2, int(1.2e9 // n)), 128)
-    big = ops.hbm_read_probe_pairs((1 << 30) // pair * pair, pair, 768, 2, 8)
+    one = ops.hbm_read_probe_pairs(n, pair, 512, 8, max(2, int(1.2e9 // n)), 128)
+    big = ops.hbm_read_probe_pairs((1 << 30) // pair * pair, pair, 512, 8, 2, 8)
     return {"bytes_per_launch": n, "mean_us": round(one["mean_us"], 2), "gbps": round(one["gbps"], 1),
             "gemv_back_to_back_over_reader": round(gemv_back_to_back_us / one["mean_us"], 3),
             "steady_state_gbps_1gib_launch": round(big["gbps"], 1),
-            "note": "same grid (768 workgroups of 4 wavefronts), same 128-bit loads two row pairs deep, no arithmetic, staging or "
-                    "epilogue; back-to-back dependent launches over buffers that rotate through > 1 GB"}
+            "note": "same grid (512 workgroups of 8 wavefronts), same 128-bit loads one 2304-byte tile ahead per wavefront, no arithmetic, "
+                    "staging or epilogue; back-to-back dependent launches over buffers that rotate through > 1 GB"}
 
 
 def main() -> None:

@@ -444,8 +444,9 @@ int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s) {
     return e == hipSuccess ? ESP_OK : fail_hip(e, "hbm_read_probe");
 }
 
-int esp_hbm_read_probe_pairs(size_t bytes_per_launch, int pair_bytes, int workgroups, int copies, int launches, double *mean_us, double *gb_per_s) {
+int esp_hbm_read_probe_pairs(size_t bytes_per_launch, int pair_bytes, int workgroups, int wavefronts, int copies, int launches, double *mean_us, double *gb_per_s) {
     if (bytes_per_launch < 4096 || pair_bytes <= 0 || pair_bytes % 16 != 0 || bytes_per_launch % (size_t)pair_bytes != 0 || workgroups <= 0 ||
+        (wavefronts != 4 && wavefronts != 8) ||
         copies < 1 || launches < 1 || !mean_us || !gb_per_s)
         return fail(ESP_ERR_INVALID_ARGUMENT, "hbm_read_probe_pairs: bad argument");
     int rc = ensure_init();
@@ -459,7 +460,7 @@ int esp_hbm_read_probe_pairs(size_t bytes_per_launch, int pair_bytes, int workgr
     hipError_t e = hipMemsetAsync(buf, 1, bytes_per_launch * copies, c.stream);
     if (e == hipSuccess) e = hipEventCreate(&t0);
     if (e == hipSuccess) e = hipEventCreate(&t1);
-    auto launch = [&](int i) { return launch_stream_read_pairs(buf + (size_t)(i % copies) * bytes_per_launch, bytes_per_launch, pair_bytes, workgroups, sink, c.stream); };
+    auto launch = [&](int i) { return launch_stream_read_pairs(buf + (size_t)(i % copies) * bytes_per_launch, bytes_per_launch, pair_bytes, workgroups, wavefronts, sink, c.stream); };
     for (int i = 0; i < copies && e == hipSuccess; i++) e = launch(i);
     if (e == hipSuccess) e = hipEventRecord(t0, c.stream);
     for (int i = 0; i < launches && e == hipSuccess; i++) e = launch(i);

@@ -159,7 +159,7 @@ hipError_t launch_int4_matvec(const uint8_t *packed, const float *scales, const 
 // kernels/probe.hip — plain streaming read of `bytes` (a multiple of 16)
 hipError_t launch_stream_read(const void *src, size_t bytes, unsigned *sink, hipStream_t stream);
 // the same with the persistent Q4_K GEMV's grid and loads: `grid` workgroups of four wavefronts over pairs of rows of `pair_bytes`
-hipError_t launch_stream_read_pairs(const void *src, size_t bytes, int pair_bytes, int grid, unsigned *sink, hipStream_t stream);
+hipError_t launch_stream_read_pairs(const void *src, size_t bytes, int pair_bytes, int grid, int wavefronts, unsigned *sink, hipStream_t stream);
 
 // kernels/synth.hip — seeded N(0, std) weights quantised into GGUF-layout blocks on the GPU
 hipError_t launch_synth(int format, uint64_t seed, float std_dev, size_t elems, uint8_t *out, hipStream_t stream);

@@ -18,15 +18,15 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const uint4 *src, size
     if (acc == 0x12345678u) sink[0] = acc;   // keeps the loads alive; practically never true
 }
 
-// The same bytes read the way the persistent Q4_K GEMV reads them, and nothing else: workgroups of four wavefronts, a
-// wavefront takes pairs of rows (`pair_bytes` contiguous bytes) team, team + n_teams, ..., every lane issues its 128-bit
-// loads of the next pair before it consumes the current one.  What this kernel reaches for a launch of N bytes is the
-// ceiling for a GEMV launch over the same N bytes: same grid, same loads in flight, no arithmetic, no staging, no
-// epilogue.
+// The same bytes read the way the persistent Q4_K GEMVs read them, and nothing else: workgroups of four or eight wavefronts, a
+// wavefront takes items of `pair_bytes` contiguous bytes (a weight tile of the matrix-core kernel, a pair of rows of the
+// dot-product kernel) team, team + n_teams, ..., every lane issues its 128-bit loads of the next item before it consumes the
+// current one.  What this kernel reaches for a launch of N bytes is the ceiling for a GEMV launch over the same N bytes: same
+// grid, same loads in flight, no arithmetic, no staging, no epilogue.
 template <int PER_LANE>
-__global__ __launch_bounds__(256) void stream_read_pairs_kernel(const uint8_t *src, int pairs, int pair_bytes, unsigned *sink) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n16 = pair_bytes / 16;
-    const int n_teams = gridDim.x * 4;
+__global__ __launch_bounds__(512) void stream_read_pairs_kernel(const uint8_t *src, int pairs, int pair_bytes, unsigned *sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n16 = pair_bytes / 16, waves = blockDim.x >> 6;
+    const int n_teams = gridDim.x * waves;
     unsigned acc = 0;
     uint4 cur[PER_LANE], nxt[PER_LANE];
     auto load = [&](int pair, uint4 (&buf)[PER_LANE]) {
@@ -34,7 +34,7 @@ __global__ __launch_bounds__(256) void stream_read_pairs_kernel(const uint8_t *s
 #pragma unroll
         for (int k = 0; k < PER_LANE; k++) buf[k] = p[lane + 64 * k < n16 ? lane + 64 * k : n16 - 1];
     };
-    int pair = blockIdx.x * 4 + wave;
+    int pair = blockIdx.x * waves + wave;
     if (pair < pairs) load(pair, cur);
     for (; pair < pairs; pair += n_teams) {
         if (pair + n_teams < pairs) load(pair + n_teams, nxt);
@@ -48,12 +48,12 @@ __global__ __launch_bounds__(256) void stream_read_pairs_kernel(const uint8_t *s
 
 }  // namespace
 
-hipError_t launch_stream_read_pairs(const void *src, size_t bytes, int pair_bytes, int grid, unsigned *sink, hipStream_t stream) {
-    if (pair_bytes <= 0 || pair_bytes % 16 != 0 || bytes % pair_bytes != 0 || grid <= 0) return hipErrorInvalidValue;
+hipError_t launch_stream_read_pairs(const void *src, size_t bytes, int pair_bytes, int grid, int wavefronts, unsigned *sink, hipStream_t stream) {
+    if (pair_bytes <= 0 || pair_bytes % 16 != 0 || bytes % pair_bytes != 0 || grid <= 0 || (wavefronts != 4 && wavefronts != 8)) return hipErrorInvalidValue;
     const int pairs = (int)(bytes / pair_bytes), per_lane = (pair_bytes / 16 + 63) / 64;
     const uint8_t *p = static_cast<const uint8_t *>(src);
-    if (per_lane <= 5) hipLaunchKernelGGL(stream_read_pairs_kernel<5>, dim3(grid), dim3(256), 0, stream, p, pairs, pair_bytes, sink);
-    else if (per_lane <= 16) hipLaunchKernelGGL(stream_read_pairs_kernel<16>, dim3(grid), dim3(256), 0, stream, p, pairs, pair_bytes, sink);
+    if (per_lane <= 5) hipLaunchKernelGGL(stream_read_pairs_kernel<5>, dim3(grid), dim3(64 * wavefronts), 0, stream, p, pairs, pair_bytes, sink);
+    else if (per_lane <= 16) hipLaunchKernelGGL(stream_read_pairs_kernel<16>, dim3(grid), dim3(64 * wavefronts), 0, stream, p, pairs, pair_bytes, sink);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }

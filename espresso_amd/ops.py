@@ -158,13 +158,15 @@ def hbm_read_probe(nbytes: int = 1 << 30, iters: int = 10) -> float:
     return out.value
 
 
-def hbm_read_probe_pairs(bytes_per_launch: int, pair_bytes: int = 4608, workgroups: int = 768, copies: int = 16, launches: int = 64) -> dict:
-    """Mean microseconds and GB/s of a reader with the persistent Q4_K GEMV's grid and loads over `bytes_per_launch` per launch."""
+def hbm_read_probe_pairs(bytes_per_launch: int, pair_bytes: int = 2304, workgroups: int = 512, wavefronts: int = 8, copies: int = 16,
+                         launches: int = 64) -> dict:
+    """Mean microseconds and GB/s of a reader with a persistent Q4_K GEMV's grid and loads over `bytes_per_launch` per launch
+    (defaults: the matrix-core kernel's 512 workgroups of eight wavefronts, one 2304-byte tile ahead per wavefront)."""
     L = _lib.load_library()
     L.esp_hbm_read_probe_pairs.restype = C.c_int
-    L.esp_hbm_read_probe_pairs.argtypes = [C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
+    L.esp_hbm_read_probe_pairs.argtypes = [C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     us, gbps = C.c_double(0), C.c_double(0)
-    _lib.check(L.esp_hbm_read_probe_pairs(bytes_per_launch, pair_bytes, workgroups, copies, launches, C.byref(us), C.byref(gbps)))
+    _lib.check(L.esp_hbm_read_probe_pairs(bytes_per_launch, pair_bytes, workgroups, wavefronts, copies, launches, C.byref(us), C.byref(gbps)))
     return {"mean_us": us.value, "gbps": gbps.value}
 
 

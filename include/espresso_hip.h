@@ -132,12 +132,12 @@ int esp_set_tuning(const char *key, int value);
  * multiple of 16) from HBM with 128-bit loads, `iters` times; reports GB/s.  bench.py prints it next to the
  * GEMV bandwidth so that fractions of the published peak can be read against what a plain reader gets. */
 int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s);
-/* The ceiling for ONE GEMV launch: a kernel with the persistent Q4_K GEMV's grid (`workgroups` of four wavefronts) and its
- * loads (a wavefront takes pairs of rows of `pair_bytes`, the next pair's 128-bit loads in flight while the current one is
- * consumed) that does nothing else, launched back to back `launches` times over `copies` buffers of `bytes_per_launch` in
+/* The ceiling for ONE GEMV launch: a kernel with a persistent Q4_K GEMV's grid (`workgroups` of `wavefronts` = 4 or 8) and its
+ * loads (a wavefront takes items of `pair_bytes`, a 2304-byte weight tile of the matrix-core kernel or a pair of rows of the
+ * dot-product kernel, the next item's 128-bit loads in flight while the current one is consumed) that does nothing else, launched back to back `launches` times over `copies` buffers of `bytes_per_launch` in
  * turn (so that no launch finds its bytes in a cache).  Reports the mean time per launch, which includes what a dependent
  * launch costs on this machine, and the resulting GB/s. */
-int esp_hbm_read_probe_pairs(size_t bytes_per_launch, int pair_bytes, int workgroups, int copies, int launches, double *mean_us,
+int esp_hbm_read_probe_pairs(size_t bytes_per_launch, int pair_bytes, int workgroups, int wavefronts, int copies, int launches, double *mean_us,
                              double *gb_per_s);
 
 /* ---- llama decoder state resident on the GPU -------------------------------------------- *
