@@ -889,34 +889,54 @@ struct GreedyTailArgs {
 __global__ __launch_bounds__(kBlock) void greedy_tail_kernel(GreedyTailArgs a) {
     __shared__ float bv[kBlock];
     __shared__ int bi[kBlock];
+    // The loop state the bookkeeping below branches on is requested first, all of it at once: read where it is needed, its five
+    // words would be a chain of trips to memory behind the reduction (every replay finds them written by the replay before).
+    // (Through pointers the compiler must keep in vector registers: vector loads share a counter with the candidates' loads below and
+    // are in flight together with them, scalar loads would be waited for together with the kernel's arguments, before anything else.)
+    typedef const __attribute__((address_space(1))) int *global_ints;   // global, not generic: generic loads count as LDS traffic too
+    global_ints state = (global_ints)a.log_count, fed = (global_ints)a.tokens, vis = (global_ints)(a.visible + a.seq);
+    asm volatile("" : "+v"(state), "+v"(fed), "+v"(vis));
+    int logged = state[0], stopped = state[1], stop_armed = state[2];
+    int fed_before = fed[0], visible_before = vis[0];
     float best = -INFINITY;
     int best_i = 0x7FFFFFFF;
-    for (int i = threadIdx.x; i < a.nblk; i += kBlock) {
-        const float v = a.part_value[i];
-        const int idx = a.part_index[i];
-        if (better(v, idx, best, best_i)) { best = v; best_i = idx; }
-    }
+    auto take_four = [&](int i0) {   // four candidates per thread in flight; past the end candidate 0 again, which changes nothing
+        float v[4];
+        int idx[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = i0 + u * kBlock, j = i < a.nblk ? i : 0;
+            v[u] = a.part_value[j];
+            idx[u] = a.part_index[j];
+        }
+        __builtin_amdgcn_sched_barrier(0);   // every load is issued before the first comparison waits for one
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (better(v[u], idx[u], best, best_i)) { best = v[u]; best_i = idx[u]; }
+    };
+    take_four(threadIdx.x);   // outside the loop: a loop's entry would wait for the state loads above
+    for (int i0 = threadIdx.x + 4 * kBlock; i0 < a.nblk; i0 += 4 * kBlock) take_four(i0);
+    asm volatile("" : "+v"(logged), "+v"(stopped), "+v"(stop_armed), "+v"(fed_before), "+v"(visible_before));   // here at the latest
     argmax_block_reduce(best, best_i, bv, bi);
     int t = best_i == 0x7FFFFFFF ? 0 : best_i;
     __shared__ int feed;   // the token whose embedding the trunk after this kernel runs on
     if (threadIdx.x == 0) {
-        if (a.log_count[1]) {
+        if (stopped) {
             // stopped in an earlier replay: nothing is emitted, and the trunk recomputes the row it computed last (same token, same
             // position, same values), so replays past the stop change nothing
-            feed = a.tokens[0];
+            feed = fed_before;
         } else {
             a.out_token[0] = t;
-            const int n = a.log_count[0];
-            if (n < a.log_capacity) a.log[n] = t;
-            a.log_count[0] = n + 1;
-            if (a.eos >= 0 && a.log_count[2] && t == a.eos) {   // the stop token is emitted, not consumed (:6385-6388)
+            if (logged < a.log_capacity) a.log[logged] = t;
+            a.log_count[0] = logged + 1;
+            if (a.eos >= 0 && stop_armed && t == a.eos) {   // the stop token is emitted, not consumed (:6385-6388)
                 a.log_count[1] = 1;
-                feed = a.tokens[0];
+                feed = fed_before;
             } else {
                 a.tokens[0] = t;
-                a.pos[0] = a.visible[a.seq];
+                a.pos[0] = visible_before;
                 a.seqs[0] = a.seq;
-                a.visible[a.seq] += 1;
+                a.visible[a.seq] = visible_before + 1;
                 feed = t;
             }
         }
