@@ -651,8 +651,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_partial_kernel(const flo
     a.q = q_rows; a.k_cache = k_cache; a.v_cache = v_cache; a.pos = pos; a.seq = seq; a.head_partials = head_partials;
     a.cache_seq_stride = cache_seq_stride; a.n_head = (int)(heads & 0xFFFFu); a.n_kv_head = (int)(heads >> 16);
     constexpr int LPT = HD / 8, SLOTS = 64 / LPT, KW = KV_F16 ? 1 : 2, STRIDE = HD + 4;
-    __shared__ float wm[WAVES], wl[WAVES][SLOTS];
-    __shared__ float wacc[WAVES][SLOTS][HD];
+    __shared__ float wm[WAVES], wl[WAVES];
+    __shared__ float wacc[WAVES][HD];
     const int group = a.n_head / a.n_kv_head;
     const int kvh = blockIdx.x % a.n_kv_head, head = kvh * group + blockIdx.x / a.n_kv_head, m = blockIdx.y;
     const int split = blockIdx.z;
@@ -730,13 +730,21 @@ __global__ __launch_bounds__(WAVES * 64) void attention_partial_kernel(const flo
             mx = m_new;
         }
     }
-    // ---- every (wavefront, token slot) publishes its partial state; m is the same in all lanes ----
+    // ---- the wavefront's token slots share one m: their sums and accumulators add up across the lanes that differ in the slot
+    // index only, and the wavefront publishes one state ----
 #pragma unroll
-    for (int i = 0; i < 8; i++) wacc[wave][slot][seg + i] = acc[i];
-    if (lane % LPT == 0) wl[wave][slot] = l;
-    if (lane == 0) wm[wave] = mx;
+    for (int off = LPT; off < 64; off <<= 1) {
+        l += __shfl_xor(l, off);
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] += __shfl_xor(acc[i], off);
+    }
+    if (slot == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) wacc[wave][seg + i] = acc[i];
+    }
+    if (lane == 0) { wl[wave] = l; wm[wave] = mx; }
     __syncthreads();
-    // ---- merge over wavefronts and slots in wavefront order: thread = channel ----
+    // ---- merge over wavefronts in wavefront order: thread = channel ----
     float *ps = a.head_partials + (((size_t)m * a.n_head + head) * splits + split) * STRIDE;
     for (int dch = tid; dch < HD; dch += WAVES * 64) {
         float M = wm[0];
@@ -746,11 +754,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_partial_kernel(const flo
 #pragma unroll
         for (int w = 0; w < WAVES; w++) {
             const float f = wm[w] == -INFINITY ? 0.0f : expf(wm[w] - M);
-            float lw = 0.0f, aw = 0.0f;
-#pragma unroll
-            for (int sl = 0; sl < SLOTS; sl++) { lw += wl[w][sl]; aw += wacc[w][sl][dch]; }
-            L = __builtin_fmaf(lw, f, L);
-            A = __builtin_fmaf(aw, f, A);
+            L = __builtin_fmaf(wl[w], f, L);
+            A = __builtin_fmaf(wacc[w][dch], f, A);
         }
         ps[dch] = A;
         if (dch == 0) { ps[HD] = M; ps[HD + 1] = L; }
@@ -1203,19 +1208,33 @@ hipError_t launch_attention_prompt(const AttentionArgs &a, int rows, bool kv_f16
 
 int attention_head_splits(int) { return kAttentionHeadSplits; }
 
+template <int HD, int WAVES, int U>
+void launch_attention_partial_shape(const AttentionArgs &a, dim3 grid, bool kv_f16, unsigned heads, hipStream_t s) {
+    if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<HD, true, WAVES, U>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
+    else hipLaunchKernelGGL((attention_partial_kernel<HD, false, WAVES, U>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
+}
+
 hipError_t launch_attention_partials(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
     if (!a.head_partials || (a.head_dim != 128 && a.head_dim != 64) || a.n_head % a.n_kv_head != 0 || rows < 1 || rows > kMaxStepRows)
         return hipErrorInvalidValue;
     if (a.cache_seq_stride > 0xFFFFFFFFull || a.n_head > 0xFFFF || a.n_kv_head > 0xFFFF) return hipErrorInvalidValue;
     const unsigned heads = (unsigned)a.n_head | ((unsigned)a.n_kv_head << 16);
     dim3 grid(a.n_head, rows, attention_head_splits(a.max_seq));
-    constexpr int WAVES = 8;   // measured at head size 128: 4 wavefronts x 12 chunks 6.2 us, 8 x 6 5.0 us, 16 x 3 4.7 us but a slower step
+    // Wavefronts per workgroup x chunks in flight per wavefront.  One pass of a wavefront's loop covers splits x wavefronts x
+    // (tokens per chunk: 4 at head size 128, 8 at 64) x chunks tokens of the prefix and costs one trip to memory, with the loads of
+    // chunks past the prefix issued all the same (clamped, masked).  The shape is fixed per runtime (a captured graph replays it),
+    // so it follows the context size: the smallest that covers half of it in one pass.  Measured at head size 128, prefix 512-776:
+    // 4 x 12 6.2 us, 8 x 6 5.0 us, 16 x 3 4.7 us but a slower step.  At head size 64, prefix 16-144 of 256 (6-layer model, tok/s):
+    // 8 x 4 7.6 k, 8 x 1 7.9 k, 2 x 8 7.7 k, 1 x 8 7.8 k, 2 x 4 8.0 k, 4 x 2 8.0 k, 1 x 4 8.0 k, 2 x 2 8.1 k.
     if (a.head_dim == 128) {
-        if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<128, true, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
-        else hipLaunchKernelGGL((attention_partial_kernel<128, false, WAVES, 6>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
+        if (a.max_seq <= 256) launch_attention_partial_shape<128, 2, 4>(a, grid, kv_f16, heads, s);        // 128 tokens per pass
+        else if (a.max_seq <= 512) launch_attention_partial_shape<128, 4, 4>(a, grid, kv_f16, heads, s);   // 256
+        else launch_attention_partial_shape<128, 8, 6>(a, grid, kv_f16, heads, s);                         // 768
     } else {
-        if (kv_f16) hipLaunchKernelGGL((attention_partial_kernel<64, true, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
-        else hipLaunchKernelGGL((attention_partial_kernel<64, false, WAVES, 4>), grid, dim3(WAVES * 64), 0, s, a.q, a.k_cache, a.v_cache, a.pos, a.seq, a.head_partials, (unsigned)a.cache_seq_stride, heads);
+        if (a.max_seq <= 256) launch_attention_partial_shape<64, 2, 2>(a, grid, kv_f16, heads, s);         // 128 tokens per pass
+        else if (a.max_seq <= 512) launch_attention_partial_shape<64, 2, 4>(a, grid, kv_f16, heads, s);    // 256
+        else if (a.max_seq <= 1024) launch_attention_partial_shape<64, 4, 4>(a, grid, kv_f16, heads, s);   // 512
+        else launch_attention_partial_shape<64, 8, 4>(a, grid, kv_f16, heads, s);                          // 1024
     }
     return hipGetLastError();
 }

@@ -474,7 +474,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const uint8_t *qs, const
 #pragma unroll
         for (int b = 0; b < B; b++) acc[r][b] = wave_sum(acc[r][b]);
 
-    static_assert(R == 2, "the epilogues work on row pairs");
+    static_assert(R % 2 == 0, "the epilogues work on row pairs");
     if (a.epilogue == EPI_ARGMAX) {
         __shared__ float bv[B * kWaves];
         __shared__ int bi[B * kWaves];
@@ -484,17 +484,22 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const uint8_t *qs, const
         for (int b = 0; b < B; b++) {
             best[b] = -INFINITY;
             best_i[b] = 0x7FFFFFFF;
-            if (row0 < a.rows) argmax_take(best[b], best_i[b], acc[0][b], row0);
-            if (row0 + 1 < a.rows) argmax_take(best[b], best_i[b], acc[1][b], row0 + 1);
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                if (row0 + r < a.rows) argmax_take(best[b], best_i[b], acc[r][b], row0 + r);   // ascending rows
         }
         argmax_workgroup<B>(a, best, best_i, bv, bi);
         return;
     }
     if (lane == 0) {
-        float va[B], vb[B];
 #pragma unroll
-        for (int b = 0; b < B; b++) { va[b] = acc[0][b]; vb[b] = acc[1][b]; }
-        pair_epilogue<B>(a, row0 / 2, va, vb);
+        for (int p = 0; p < R / 2; p++) {
+            if (row0 + 2 * p >= a.rows) break;
+            float va[B], vb[B];
+#pragma unroll
+            for (int b = 0; b < B; b++) { va[b] = acc[2 * p][b]; vb[b] = acc[2 * p + 1][b]; }
+            pair_epilogue<B>(a, row0 / 2 + p, va, vb);
+        }
     }
 }
 
@@ -1699,7 +1704,12 @@ hipError_t launch_one(const KernelArgs &a, hipStream_t stream) {
 
 template <int FMT>
 hipError_t launch_fmt(const KernelArgs &a, int batch, hipStream_t stream) {
-    if (batch == 1) return launch_one<FMT, 1, 2>(a, stream);
+    if (batch == 1) {
+        // tall matrices (an output head): four rows per wavefront, so that one wave of workgroups covers the matrix (32000 x 768 Q8_0:
+        // 2000 workgroups instead of 4000, 8.8 against 10.1 us; eight rows measure the same as four)
+        if (a.rows >= 16384) return launch_one<FMT, 1, 4>(a, stream);
+        return launch_one<FMT, 1, 2>(a, stream);
+    }
     if (batch == 2) return launch_one<FMT, 2, 2>(a, stream);
     return hipErrorInvalidValue;
 }

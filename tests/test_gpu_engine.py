@@ -327,7 +327,9 @@ def test_bundle_selects_the_exact_two_token_path(E, tmp_path):
     for entry in B.REQUIRED_TOP_LEVEL_ENTRIES:
         os.makedirs(root / entry)
     full_kw, draft_kw = dict(KW, n_layer=3), dict(KW, n_layer=1)
-    seen_f = write_weight_dir(str(root / "weights"), full_kw, mu.random_weights(orc.LlamaConfig(**full_kw), 61, std=0.08))
+    # the stream is compared token for token: a seed for which the oracle's top-2 margin is at least 0.1 at each of the 20 steps
+    # (most seeds have a step below 1e-2, which the fp16 rounding of an activation can flip)
+    seen_f = write_weight_dir(str(root / "weights"), full_kw, mu.random_weights(orc.LlamaConfig(**full_kw), 80, std=0.08))
     seen_d = write_weight_dir(str(root / "weights" / "draft"), draft_kw, mu.random_weights(orc.LlamaConfig(**draft_kw), 62, std=0.08))
     (root / "weights" / "draft.json").write_text(json.dumps({"model_dir": "draft", "tokenizer_dir": None, "model_id": "d"}))
     pieces = [("▁", 0.0)] + [(chr(97 + i), 0.0) for i in range(26)] + [("▁the", 2.0), ("▁t", 1.0), ("▁th", 1.5)] + [(f"<0x{b:02X}>", 0.0) for b in range(256)]
