@@ -47,16 +47,22 @@ int hip_ok(hipError_t e, const char *what) { return e == hipSuccess ? ESP_OK : f
 // it owes after an accepted pass and the current token, or the current token twice) and proposes; the target verifies
 // (current, proposed); the accept kernel emits, keeps the hidden row and writes the next pass's rows.  No host decision, so
 // the pass replays as a captured graph.
-int enqueue_two_token_pass(LlamaRuntime &full, LlamaRuntime &draft, TwoTokenState *state, int *log, int log_capacity) {
+// draft_rows_embedded: the pass before this one left the embeddings of the draft's two rows in its hidden rows (its accept kernel
+// does); the first pass after the host set the rows has to fetch them itself.
+int enqueue_two_token_pass(LlamaRuntime &full, LlamaRuntime &draft, TwoTokenState *state, int *log, int log_capacity, bool draft_rows_embedded) {
     hipStream_t s = context().stream;
     int rc;
-    if ((rc = draft.enqueue_device_rows(2)) != ESP_OK) return rc;
+    if ((rc = draft.enqueue_device_rows(2, draft_rows_embedded)) != ESP_OK) return rc;
     if ((rc = draft.enqueue_device_head(2)) != ESP_OK) return rc;
-    ESP_HIP_TRY(launch_two_token_verify_rows(state, draft.device_head_tokens(), full.device_row_tokens(), full.device_row_positions(), s));
-    if ((rc = full.enqueue_device_rows(2)) != ESP_OK) return rc;
+    // the two small kernels between the models also fetch the embedding rows of the model that runs next: two launches fewer per pass
+    ESP_HIP_TRY(launch_two_token_verify_rows(state, draft.device_head_tokens(), full.device_row_tokens(), full.device_row_positions(),
+                                             full.device_embed_target(), s));
+    if ((rc = full.enqueue_device_rows(2, true)) != ESP_OK) return rc;
     if ((rc = full.enqueue_device_head(2)) != ESP_OK) return rc;
+    EmbedTarget draft_rows = draft.device_embed_target();
+    draft_rows.keep_row1 = draft.device_last_hidden(0);   // the draft's last output row, before the embeddings replace it
     ESP_HIP_TRY(launch_two_token_accept(state, full.device_head_tokens(), log, log_capacity, full.device_hidden_rows(), full.device_last_hidden(0),
-                                        full.config().d_model, draft.device_row_tokens(), draft.device_row_positions(), s));
+                                        full.config().d_model, draft.device_row_tokens(), draft.device_row_positions(), draft_rows, s));
     return ESP_OK;
 }
 
@@ -94,13 +100,13 @@ int run_two_token_passes_on_device(LlamaRuntime &full, LlamaRuntime &draft, TwoT
     if ((rc = hip(launch_set_rows(rows, draft.device_row_tokens(), draft.device_row_positions(), draft.device_row_sequences(), s), "rows")) != ESP_OK) return cleanup(rc);
     if ((rc = hip(launch_set_rows(rows, full.device_row_tokens(), full.device_row_positions(), full.device_row_sequences(), s), "rows")) != ESP_OK) return cleanup(rc);
     // the first pass runs as plain launches: whatever a kernel configures on its first use happens outside the capture
-    if ((rc = enqueue_two_token_pass(full, draft, d_state, d_log, capacity)) != ESP_OK) return cleanup(rc);
+    if ((rc = enqueue_two_token_pass(full, draft, d_state, d_log, capacity, false)) != ESP_OK) return cleanup(rc);
     if ((rc = fetch()) != ESP_OK) return cleanup(rc);
     while (!state->done) {
         if (!exec) {
             hipGraph_t graph = nullptr;
             if ((rc = hip(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture")) != ESP_OK) return cleanup(rc);
-            rc = enqueue_two_token_pass(full, draft, d_state, d_log, capacity);
+            rc = enqueue_two_token_pass(full, draft, d_state, d_log, capacity, true);
             const hipError_t e = hipStreamEndCapture(s, &graph);
             if (rc == ESP_OK) rc = hip(e, "hipStreamEndCapture");
             if (rc == ESP_OK) rc = hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
@@ -249,7 +255,7 @@ int generate_two_token(LlamaRuntime &full, LlamaRuntime &draft, const uint32_t *
         // both models as the host loop would have left them: the draft has consumed what the target has, less the row it owes
         if ((rc = full.set_visible(0, ds.full_pos)) != ESP_OK) return rc;
         if ((rc = draft.set_visible(0, ds.full_pos - (ds.accepted_prev ? 1 : 0))) != ESP_OK) return rc;
-        if ((rc = draft.keep_row(1, 0)) != ESP_OK) return rc;
+        // (the draft's last output row was kept by the pass's last kernel, which then put the next rows' embeddings in its place)
         if (ds.accepted_prev) {
             if ((rc = draft.advance(0, (uint32_t)ds.proposed_prev)) != ESP_OK) return rc;
             if (reference_accounting) {

@@ -115,7 +115,16 @@ struct TwoTokenState {
 };
 // After the draft's two rows went through its head: the proposal becomes row 1 of the target's verify step; the draft's
 // successor of the row it owed is compared for the reference's accepted count.
-hipError_t launch_two_token_verify_rows(TwoTokenState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, hipStream_t s);
+// `embed`: the kernel also fetches the embedding rows of the two tokens (whether it changed them or not) into the model's hidden
+// rows, so that the trunk pass after it starts without an embedding launch.
+struct EmbedTarget {
+    const void *table = nullptr;   // [vocab][d] fp16 or fp32
+    int table_is_f16 = 0, d = 0;
+    float *hidden = nullptr;       // [2][d]
+    float *keep_row1 = nullptr;    // when set: row 1 of `hidden` (the model's last output) is copied here before the rows are overwritten
+};
+hipError_t launch_two_token_verify_rows(TwoTokenState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, const EmbedTarget &embed,
+                                        hipStream_t s);
 // After the target's two rows went through its head: emits one or two tokens into log, keeps the matching hidden row of the
 // target (d floats from hidden_rows into last_hidden), advances the state and writes the draft's two rows of the next pass.
 // The same loop over up to sixteen sequences in lock step (rows 2 s and 2 s + 1 of both models belong to sequence s), and the plain
@@ -134,7 +143,7 @@ hipError_t launch_two_token_batch_accept(TwoTokenBatchState *state, int n_seq, c
 // Greedy step of n sequences: the head's tokens become the next rows at the next positions and go to log[step][n].
 hipError_t launch_batch_greedy_feed(const int *head_tokens, int n, int *tokens, int *pos, int *log, int *step, int capacity_steps, hipStream_t s);
 hipError_t launch_two_token_accept(TwoTokenState *state, const int *target_head_tokens, int *log, int log_capacity, const float *hidden_rows,
-                                   float *last_hidden, int d, int *draft_tokens, int *draft_pos, hipStream_t s);
+                                   float *last_hidden, int d, int *draft_tokens, int *draft_pos, const EmbedTarget &draft_embed, hipStream_t s);
 hipError_t launch_copy_rows(const float *src, float *dst, int rows, int d, hipStream_t s);
 
 }  // namespace esp

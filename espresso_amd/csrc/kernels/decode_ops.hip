@@ -839,10 +839,19 @@ __global__ __launch_bounds__(kBlock) void argmax_final_kernel(const float *part_
     const int m = blockIdx.x;
     float best = -INFINITY;
     int best_i = 0x7FFFFFFF;
-    for (int i = threadIdx.x; i < nblk; i += kBlock) {
-        const float v = part_value[(size_t)m * nblk + i];
-        const int idx = part_index[(size_t)m * nblk + i];
-        if (better(v, idx, best, best_i)) { best = v; best_i = idx; }
+    for (int i0 = threadIdx.x; i0 < nblk; i0 += 4 * kBlock) {   // four candidates per thread in flight; past the end the first again
+        float v[4];
+        int idx[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = i0 + u * kBlock, j = i < nblk ? i : i0;
+            v[u] = part_value[(size_t)m * nblk + j];
+            idx[u] = part_index[(size_t)m * nblk + j];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (better(v[u], idx[u], best, best_i)) { best = v[u]; best_i = idx[u]; }
     }
     argmax_block_reduce(best, best_i, bv, bi);
     if (threadIdx.x == 0) {
@@ -874,6 +883,47 @@ __global__ void greedy_feed_kernel(const int *next_token, int seq, int *visible,
     if (n < log_capacity) log[n] = t;
     *log_count = n + 1;
     visible[seq] += 1;
+}
+
+// One embedding row into `hidden` (d floats), by a whole workgroup of `threads` threads: up to four loads per thread are in flight
+// before the first store (a load after a store through an unrelated pointer would have to wait for it), eight values per load
+// where the row allows.
+__device__ __forceinline__ void embed_row(const void *table, int table_is_f16, int token, int d, float *hidden, int threads) {
+    if (table_is_f16 && d % 8 == 0) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(table) + (size_t)token * d);
+        const int groups = d / 8;
+        for (int g0 = threadIdx.x; g0 < groups; g0 += 4 * threads) {
+            uint4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = src[g0 + u * threads < groups ? g0 + u * threads : g0];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (g0 + u * threads >= groups) break;
+                const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+                float4 lo, hi;
+                lo.x = from_half_bits((uint16_t)(w[0] & 0xFFFFu)); lo.y = from_half_bits((uint16_t)(w[0] >> 16));
+                lo.z = from_half_bits((uint16_t)(w[1] & 0xFFFFu)); lo.w = from_half_bits((uint16_t)(w[1] >> 16));
+                hi.x = from_half_bits((uint16_t)(w[2] & 0xFFFFu)); hi.y = from_half_bits((uint16_t)(w[2] >> 16));
+                hi.z = from_half_bits((uint16_t)(w[3] & 0xFFFFu)); hi.w = from_half_bits((uint16_t)(w[3] >> 16));
+                float4 *dst = reinterpret_cast<float4 *>(hidden + (size_t)(g0 + u * threads) * 8);
+                dst[0] = lo;
+                dst[1] = hi;
+            }
+        }
+        return;
+    }
+    const size_t row = (size_t)token * d;
+    for (int i0 = threadIdx.x; i0 < d; i0 += 4 * threads) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = i0 + u * threads < d ? i0 + u * threads : i0;
+            v[u] = table_is_f16 ? from_half_bits(reinterpret_cast<const uint16_t *>(table)[row + i]) : reinterpret_cast<const float *>(table)[row + i];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (i0 + u * threads < d) hidden[i0 + u * threads] = v[u];
+    }
 }
 
 // The end of a greedy step in one launch: reduce the argmax slices of row 0 (argmax_final_kernel), feed the token
@@ -947,11 +997,7 @@ __global__ __launch_bounds__(kBlock) void greedy_tail_kernel(GreedyTailArgs a) {
         }
     }
     __syncthreads();
-    t = feed;
-    const size_t row = (size_t)t * a.d;
-    for (int i = threadIdx.x; i < a.d; i += kBlock)
-        a.hidden[i] = a.table_is_f16 ? from_half_bits(reinterpret_cast<const uint16_t *>(a.table)[row + i])
-                                     : reinterpret_cast<const float *>(a.table)[row + i];
+    embed_row(a.table, a.table_is_f16, feed, a.d, a.hidden, kBlock);
 }
 
 __global__ void set_ints_kernel(int *dst0, int v0, int *dst1, int v1) {
@@ -967,22 +1013,42 @@ __global__ void copy_rows_kernel(const float *src, float *dst, int d) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < d; i += gridDim.x * blockDim.x) dst[(size_t)m * d + i] = src[(size_t)m * d + i];
 }
 
-// One thread: see launch_two_token_verify_rows.
-__global__ void two_token_verify_rows_kernel(TwoTokenState *st, const int *draft_head, int *tokens, int *pos) {
-    if (threadIdx.x != 0 || blockIdx.x != 0 || st->done) return;
-    // row 0 of the draft's step was the row it owed after an accepted pass: its successor is the reference's second
-    // comparison of that pass (:6156-6163)
-    if (st->accepted_prev && st->reference_accounting && draft_head[0] == st->exact1_prev) st->reference_accepted_total += 1;
-    const int proposed = draft_head[1];
-    st->proposed = proposed;
-    tokens[0] = st->current; pos[0] = st->full_pos;
-    tokens[1] = proposed;    pos[1] = st->full_pos + 1;
+// Rows 0 and 1 of `hidden` = embedding rows of the two tokens (every thread of a 256-thread workgroup calls this).
+__device__ __forceinline__ void embed_two_rows(const EmbedTarget &e, int t0, int t1) {
+    if (e.keep_row1) {
+        for (int i = threadIdx.x; i < e.d; i += 256) e.keep_row1[i] = e.hidden[e.d + i];
+        __syncthreads();   // row 1 is read by other threads than those that overwrite it below
+    }
+    embed_row(e.table, e.table_is_f16, t0, e.d, e.hidden, 256);
+    embed_row(e.table, e.table_is_f16, t1, e.d, e.hidden + e.d, 256);
+}
+
+// Thread 0: see launch_two_token_verify_rows; then the workgroup embeds the target's two rows.
+__global__ __launch_bounds__(256) void two_token_verify_rows_kernel(TwoTokenState *st, const int *draft_head, int *tokens, int *pos, EmbedTarget embed) {
+    __shared__ int row_token[2];
+    if (threadIdx.x == 0) {
+        if (!st->done) {
+            // row 0 of the draft's step was the row it owed after an accepted pass: its successor is the reference's second
+            // comparison of that pass (:6156-6163)
+            if (st->accepted_prev && st->reference_accounting && draft_head[0] == st->exact1_prev) st->reference_accepted_total += 1;
+            const int proposed = draft_head[1];
+            st->proposed = proposed;
+            tokens[0] = st->current; pos[0] = st->full_pos;
+            tokens[1] = proposed;    pos[1] = st->full_pos + 1;
+        }
+        // after the end the rows stay what they were: the trunk then recomputes what it computed last
+        row_token[0] = tokens[0]; row_token[1] = tokens[1];
+    }
+    if (!embed.hidden) return;
+    __syncthreads();
+    embed_two_rows(embed, row_token[0], row_token[1]);
 }
 
 // Thread 0 runs one iteration of the reference loop's bookkeeping (:6109-6186), then the workgroup keeps the hidden row.
 __global__ __launch_bounds__(256) void two_token_accept_kernel(TwoTokenState *st, const int *head, int *log, int log_capacity, const float *hidden_rows,
-                                                                float *last_hidden, int d, int *draft_tokens, int *draft_pos) {
+                                                                float *last_hidden, int d, int *draft_tokens, int *draft_pos, EmbedTarget draft_embed) {
     __shared__ int keep;
+    __shared__ int draft_row_token[2];
     if (threadIdx.x == 0) {
         keep = -1;
         if (!st->done) {
@@ -1018,10 +1084,12 @@ __global__ __launch_bounds__(256) void two_token_accept_kernel(TwoTokenState *st
                 }
             }
         }
+        draft_row_token[0] = draft_tokens[0]; draft_row_token[1] = draft_tokens[1];   // changed or not: what the draft's next step runs on
     }
     __syncthreads();
     if (keep >= 0)
         for (int i = threadIdx.x; i < d; i += 256) last_hidden[i] = hidden_rows[(size_t)keep * d + i];
+    if (draft_embed.hidden) embed_two_rows(draft_embed, draft_row_token[0], draft_row_token[1]);
 }
 
 // One thread per sequence: see launch_two_token_batch_verify_rows.
@@ -1116,15 +1184,16 @@ hipError_t launch_batch_greedy_feed(const int *head_tokens, int n, int *tokens, 
     return hipGetLastError();
 }
 
-hipError_t launch_two_token_verify_rows(TwoTokenState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, hipStream_t s) {
-    hipLaunchKernelGGL(two_token_verify_rows_kernel, dim3(1), dim3(64), 0, s, state, draft_head_tokens, target_tokens, target_pos);
+hipError_t launch_two_token_verify_rows(TwoTokenState *state, const int *draft_head_tokens, int *target_tokens, int *target_pos, const EmbedTarget &embed,
+                                        hipStream_t s) {
+    hipLaunchKernelGGL(two_token_verify_rows_kernel, dim3(1), dim3(256), 0, s, state, draft_head_tokens, target_tokens, target_pos, embed);
     return hipGetLastError();
 }
 
 hipError_t launch_two_token_accept(TwoTokenState *state, const int *target_head_tokens, int *log, int log_capacity, const float *hidden_rows,
-                                   float *last_hidden, int d, int *draft_tokens, int *draft_pos, hipStream_t s) {
+                                   float *last_hidden, int d, int *draft_tokens, int *draft_pos, const EmbedTarget &draft_embed, hipStream_t s) {
     hipLaunchKernelGGL(two_token_accept_kernel, dim3(1), dim3(256), 0, s, state, target_head_tokens, log, log_capacity, hidden_rows, last_hidden, d,
-                       draft_tokens, draft_pos);
+                       draft_tokens, draft_pos, draft_embed);
     return hipGetLastError();
 }
 

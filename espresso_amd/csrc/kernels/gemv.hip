@@ -1710,7 +1710,7 @@ hipError_t launch_fmt(const KernelArgs &a, int batch, hipStream_t stream) {
         if (a.rows >= 16384) return launch_one<FMT, 1, 4>(a, stream);
         return launch_one<FMT, 1, 2>(a, stream);
     }
-    if (batch == 2) return launch_one<FMT, 2, 2>(a, stream);
+    if (batch == 2) return a.rows >= 16384 ? launch_one<FMT, 2, 4>(a, stream) : launch_one<FMT, 2, 2>(a, stream);
     return hipErrorInvalidValue;
 }
 

@@ -86,7 +86,8 @@ class LlamaRuntime {
     const int *device_head_tokens() const { return d_out_tokens_; }
     const float *device_hidden_rows() const { return hidden_; }
     float *device_last_hidden(int seq) { return last_hidden_ + (size_t)seq * c_.d_model; }
-    int enqueue_device_rows(int rows) { return enqueue_trunk(rows); }             // embedding, then every layer
+    int enqueue_device_rows(int rows, bool embedded = false) { return enqueue_trunk(rows, embedded); }   // embedding (unless the rows hold it already), then every layer
+    EmbedTarget device_embed_target() { EmbedTarget e; e.table = embedding_; e.table_is_f16 = embedding_f16_ ? 1 : 0; e.d = c_.d_model; e.hidden = hidden_; return e; }
     int enqueue_device_head(int rows) { return run_head(hidden_, rows); }         // final norm, head, first-max arg-max per row
     bool graph_replay_enabled() const { return use_graph_ && !timing_enabled_; }
 
