@@ -28,6 +28,7 @@ struct LlamaConfig {
 };
 
 constexpr int kPrefillBlockRows = 512;        // rows per MFMA prefill block
+constexpr int kStepsPerGraph = 8;             // greedy steps in the longer of the two captured step graphs
 constexpr int kMatrixPrefillMinTokens = 32;   // shorter prompts take the exact per-token path
 constexpr size_t kGemmWorkspaceFloats = (size_t)8 << 20;
 
@@ -61,7 +62,7 @@ class LlamaRuntime {
     // Keep row `row` of the most recent forward_rows() as sequence `seq`'s last hidden state.
     int keep_row(int row, int seq);
     // `steps` greedy tokens from the sequence's current state (select, then advance, per token) as
-    // replays of one captured HIP graph per token; the host synchronises once at the end.
+    // replays of captured HIP graphs (eight steps per graph while that many are left, then one); the host synchronises once at the end.
     int continue_greedy(int seq, int steps, uint32_t *out_tokens);
     // The same, ending early at the configuration's stop token: the stop token is emitted (it is the last of *produced tokens) and not
     // consumed.  The step graph notices it on the device; the host looks once per 32 replays.
@@ -123,6 +124,8 @@ class LlamaRuntime {
     bool matrix_prefill_supported() const;
     bool wo_merges_attention(const Layer &L, int rows) const;
     int capture_step_graph(int seq);
+    int capture_steps(int seq, int count, hipGraphExec_t *out);
+    int replay_steps(int seq, int steps);
     HostTensor *host_slot(int layer, int slot);
 
     LlamaConfig c_;
@@ -144,7 +147,7 @@ class LlamaRuntime {
     size_t weight_bytes_ = 0;
     // captured greedy step per sequence (head -> feed -> trunk -> keep), and its device-side state
     bool use_graph_ = true;
-    std::vector<hipGraphExec_t> step_graphs_;
+    std::vector<hipGraphExec_t> step_graphs_, multi_graphs_;   // one step, kStepsPerGraph steps
     int *d_visible_ = nullptr, *d_log_ = nullptr, *d_log_count_ = nullptr;
     ArgmaxScratch argmax_scratch_;
     int head_partial_capacity_ = 0;      // (value, index) slots per row for the head's per-workgroup candidates
