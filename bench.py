@@ -149,7 +149,7 @@ def cpu_baseline(name: str, gpu: dict) -> dict:
 # the runs and the per-kernel table are in profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt.
 MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66521607}
 # the same kernel's mean duration in the committed rocprofv3 kernel trace (a profiled run; 2-4 % slower than an unprofiled one)
-PROFILE_KERNEL_US = {("llama3-8b-q4k", "gate_up"): (13.88, "profiles/q4k_gemv_decode_llama3_8b_kernel_trace.txt")}
+PROFILE_KERNEL_US = {("llama3-8b-q4k", "gate_up"): (13.63, "profiles/q4k_gemv_decode_llama3_8b_kernel_trace.txt")}
 TRAFFIC_SOURCE = "profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload; not measured in this run)"
 
 
