@@ -241,8 +241,8 @@ int esp_llama_generate_batch(ESPLlamaRuntime *target, ESPLlamaRuntime *draft_or_
  * advance, per token (the body of the loop at RealModelInferenceEngine.swift:6365-6413 without the
  * EOS test).  Fails with ESP_ERR_OUT_OF_RANGE if the context would overflow. */
 int esp_llama_continue_greedy(ESPLlamaRuntime *runtime, int sequence, int steps, uint32_t *out_tokens);
-/* esp_llama_continue_greedy replays one captured HIP graph per token (head, argmax, trunk) and
- * synchronises once at the end; 0 switches it to one kernel launch at a time with a host read of
+/* esp_llama_continue_greedy replays captured HIP graphs (head, argmax, trunk per token; eight tokens per graph while eight
+ * are left, then one) and synchronises once at the end; 0 switches it to one kernel launch at a time with a host read of
  * every token (same results).  Default: enabled. */
 int esp_llama_set_graph_replay(ESPLlamaRuntime *runtime, int enabled);
 /* Prompts of 32 tokens or more are prefilled in blocks of up to 512 rows with every projection as one
