@@ -71,21 +71,27 @@ int enqueue_two_token_pass(LlamaRuntime &full, LlamaRuntime &draft, TwoTokenStat
 // emitted tokens at their output indices.
 int run_two_token_passes_on_device(LlamaRuntime &full, LlamaRuntime &draft, TwoTokenState *state, std::vector<int> *log) {
     hipStream_t s = context().stream;
-    TwoTokenState *d_state = nullptr;
-    int *d_log = nullptr;
-    hipGraphExec_t exec = nullptr;
+    constexpr int kPassesPerGraph = 4;   // a boundary between two graph launches costs ~3.5 us on the device
     const int capacity = state->budget + 2;
     log->assign(capacity, 0);
-    int rc = device_alloc(&d_state, (size_t)1);
-    if (rc == ESP_OK) rc = device_alloc(&d_log, (size_t)capacity);
-    auto cleanup = [&](int code) {
-        if (exec) (void)hipGraphExecDestroy(exec);
-        if (d_state) (void)hipFree(d_state);
-        if (d_log) (void)hipFree(d_log);
-        return code;
-    };
-    if (rc != ESP_OK) return cleanup(rc);
     auto hip = [&](hipError_t e, const char *what) { return e == hipSuccess ? ESP_OK : fail_hip(e, what); };
+    // State, log and the captured passes live in the target's session from call to call (a call costs neither an allocation
+    // nor a capture after the first); the session is rebuilt when the partner or either runtime's kernels changed.
+    DeviceLoopSession &ss = full.loop_session();
+    if (ss.partner_id != draft.id() || ss.epoch != full.graph_epoch() || ss.partner_epoch != draft.graph_epoch() || ss.log_capacity < capacity) {
+        full.release_loop_session();
+        TwoTokenState *fresh_state = nullptr;
+        int *fresh_log = nullptr;
+        const int log_capacity = full.config().max_seq + 2 > capacity ? full.config().max_seq + 2 : capacity;
+        int rc = device_alloc(&fresh_state, (size_t)1);
+        if (rc == ESP_OK) rc = device_alloc(&fresh_log, (size_t)log_capacity);
+        if (rc != ESP_OK) { if (fresh_state) (void)hipFree(fresh_state); return rc; }
+        ss.state = fresh_state; ss.log = fresh_log; ss.log_capacity = log_capacity;
+        ss.partner_id = draft.id(); ss.epoch = full.graph_epoch(); ss.partner_epoch = draft.graph_epoch();
+    }
+    TwoTokenState *d_state = static_cast<TwoTokenState *>(ss.state);
+    int *d_log = ss.log;
+    int rc;
     auto fetch = [&]() {
         int r = hip(hipMemcpyAsync(state, d_state, sizeof(TwoTokenState), hipMemcpyDeviceToHost, s), "two-token state");
         if (r == ESP_OK) r = hip(hipStreamSynchronize(s), "two-token pass");
@@ -96,32 +102,40 @@ int run_two_token_passes_on_device(LlamaRuntime &full, LlamaRuntime &draft, TwoT
     rows.token[0] = rows.token[1] = state->current;
     rows.pos[0] = rows.pos[1] = state->full_pos;
     rows.seq[0] = rows.seq[1] = 0;
-    if ((rc = hip(hipMemcpyAsync(d_state, state, sizeof(TwoTokenState), hipMemcpyHostToDevice, s), "two-token state")) != ESP_OK) return cleanup(rc);
-    if ((rc = hip(launch_set_rows(rows, draft.device_row_tokens(), draft.device_row_positions(), draft.device_row_sequences(), s), "rows")) != ESP_OK) return cleanup(rc);
-    if ((rc = hip(launch_set_rows(rows, full.device_row_tokens(), full.device_row_positions(), full.device_row_sequences(), s), "rows")) != ESP_OK) return cleanup(rc);
-    // the first pass runs as plain launches: whatever a kernel configures on its first use happens outside the capture
-    if ((rc = enqueue_two_token_pass(full, draft, d_state, d_log, capacity, false)) != ESP_OK) return cleanup(rc);
-    if ((rc = fetch()) != ESP_OK) return cleanup(rc);
+    if ((rc = hip(hipMemcpyAsync(d_state, state, sizeof(TwoTokenState), hipMemcpyHostToDevice, s), "two-token state")) != ESP_OK) return rc;
+    if ((rc = hip(launch_set_rows(rows, draft.device_row_tokens(), draft.device_row_positions(), draft.device_row_sequences(), s), "rows")) != ESP_OK) return rc;
+    if ((rc = hip(launch_set_rows(rows, full.device_row_tokens(), full.device_row_positions(), full.device_row_sequences(), s), "rows")) != ESP_OK) return rc;
+    // the first pass runs as plain launches: whatever a kernel configures on its first use happens outside the capture, and
+    // the draft's rows are embedded by the pass itself (later passes find them embedded by the pass before)
+    if ((rc = enqueue_two_token_pass(full, draft, d_state, d_log, ss.log_capacity, false)) != ESP_OK) return rc;
+    if ((rc = fetch()) != ESP_OK) return rc;
+    auto capture = [&](int passes, hipGraphExec_t *out) {
+        hipGraph_t graph = nullptr;
+        int r = hip(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+        if (r != ESP_OK) return r;
+        for (int p = 0; p < passes && r == ESP_OK; p++) r = enqueue_two_token_pass(full, draft, d_state, d_log, ss.log_capacity, true);
+        const hipError_t e = hipStreamEndCapture(s, &graph);
+        if (r == ESP_OK) r = hip(e, "hipStreamEndCapture");
+        if (r == ESP_OK) r = hip(hipGraphInstantiate(out, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+        if (graph) (void)hipGraphDestroy(graph);
+        return r;
+    };
     while (!state->done) {
-        if (!exec) {
-            hipGraph_t graph = nullptr;
-            if ((rc = hip(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture")) != ESP_OK) return cleanup(rc);
-            rc = enqueue_two_token_pass(full, draft, d_state, d_log, capacity, true);
-            const hipError_t e = hipStreamEndCapture(s, &graph);
-            if (rc == ESP_OK) rc = hip(e, "hipStreamEndCapture");
-            if (rc == ESP_OK) rc = hip(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
-            if (graph) (void)hipGraphDestroy(graph);
-            if (rc != ESP_OK) return cleanup(rc);
-        }
+        if (!ss.one && (rc = capture(1, &ss.one)) != ESP_OK) return rc;
         // a pass emits one or two tokens: half of what is left can never overrun, and passes after the end change nothing
         const int left = state->budget - state->emitted, chunk = left / 2 > 1 ? left / 2 : 1;
-        for (int i = 0; i < chunk; i++)
-            if ((rc = hip(hipGraphLaunch(exec, s), "hipGraphLaunch")) != ESP_OK) return cleanup(rc);
-        if ((rc = fetch()) != ESP_OK) return cleanup(rc);
+        if (!ss.many && chunk >= kPassesPerGraph && (rc = capture(kPassesPerGraph, &ss.many)) != ESP_OK) return rc;
+        int i = 0;
+        if (ss.many)
+            for (; i + kPassesPerGraph <= chunk; i += kPassesPerGraph)
+                if ((rc = hip(hipGraphLaunch(ss.many, s), "hipGraphLaunch")) != ESP_OK) return rc;
+        for (; i < chunk; i++)
+            if ((rc = hip(hipGraphLaunch(ss.one, s), "hipGraphLaunch")) != ESP_OK) return rc;
+        if ((rc = fetch()) != ESP_OK) return rc;
     }
     rc = hip(hipMemcpyAsync(log->data(), d_log, sizeof(int) * capacity, hipMemcpyDeviceToHost, s), "two-token log");
     if (rc == ESP_OK) rc = hip(hipStreamSynchronize(s), "two-token log");
-    return cleanup(rc);
+    return rc;
 }
 }  // namespace
 

@@ -1,5 +1,6 @@
 #include "llama_runtime.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -47,7 +48,9 @@ int LlamaRuntime::create(const LlamaConfig &c, LlamaRuntime **out) {
         return fail(ESP_ERR_INVALID_ARGUMENT, "llama config: max_sequences must be 1..%d", kMaxStepRows);
     int rc = ensure_init();
     if (rc != ESP_OK) return rc;
+    static std::atomic<unsigned long long> next_id{1};
     LlamaRuntime *rt = new LlamaRuntime();
+    rt->id_ = next_id.fetch_add(1);
     rt->c_ = c;
     rt->h_layers_.resize(c.n_layer);
     rt->visible_.assign(c.max_sequences, 0);
@@ -74,6 +77,7 @@ LlamaRuntime::~LlamaRuntime() {
     free_device(argmax_scratch_.part_value); free_device(argmax_scratch_.part_index);
     for (hipGraphExec_t g : step_graphs_) if (g) (void)hipGraphExecDestroy(g);
     for (hipGraphExec_t g : multi_graphs_) if (g) (void)hipGraphExecDestroy(g);
+    release_loop_session();
     for (TimedLaunch &t : timed_) { (void)hipEventDestroy(t.start); (void)hipEventDestroy(t.stop); }
     for (hipEvent_t e : event_pool_) (void)hipEventDestroy(e);
 }
@@ -539,6 +543,16 @@ void LlamaRuntime::set_merged_attention(bool enabled) {
     merged_attention_ = enabled;
     for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }   // captured with the other path
     for (auto &g : multi_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+    graph_epoch_++;
+}
+
+void LlamaRuntime::release_loop_session() {
+    DeviceLoopSession &ss = loop_session_;
+    if (ss.one) (void)hipGraphExecDestroy(ss.one);
+    if (ss.many) (void)hipGraphExecDestroy(ss.many);
+    if (ss.state) (void)hipFree(ss.state);
+    if (ss.log) (void)hipFree(ss.log);
+    ss = DeviceLoopSession{};
 }
 
 int LlamaRuntime::keep_row(int row, int seq) {

@@ -32,6 +32,18 @@ constexpr int kStepsPerGraph = 8;             // greedy steps in the longer of t
 constexpr int kMatrixPrefillMinTokens = 32;   // shorter prompts take the exact per-token path
 constexpr size_t kGemmWorkspaceFloats = (size_t)8 << 20;
 
+// What a device-resident generation loop over two runtimes (target + draft) keeps between calls, owned by the target: its state
+// and token log in device memory and the captured graphs of its passes.  The graphs hold pointers into both runtimes, so the
+// session names the partner by an identifier no later runtime can have, and both runtimes' graph epochs (which change whenever a
+// runtime's kernels for a step change): a session that does not match is rebuilt, never replayed.
+struct DeviceLoopSession {
+    unsigned long long partner_id = 0, epoch = 0, partner_epoch = 0;
+    void *state = nullptr;
+    int *log = nullptr;
+    int log_capacity = 0;
+    hipGraphExec_t one = nullptr, many = nullptr;   // one pass; several passes in a row
+};
+
 class LlamaRuntime {
   public:
     static int create(const LlamaConfig &config, LlamaRuntime **out);
@@ -91,6 +103,10 @@ class LlamaRuntime {
     EmbedTarget device_embed_target() { EmbedTarget e; e.table = embedding_; e.table_is_f16 = embedding_f16_ ? 1 : 0; e.d = c_.d_model; e.hidden = hidden_; return e; }
     int enqueue_device_head(int rows) { return run_head(hidden_, rows); }         // final norm, head, first-max arg-max per row
     bool graph_replay_enabled() const { return use_graph_ && !timing_enabled_; }
+    unsigned long long id() const { return id_; }
+    unsigned long long graph_epoch() const { return graph_epoch_; }
+    DeviceLoopSession &loop_session() { return loop_session_; }
+    void release_loop_session();   // destroys the session's graphs and frees its buffers
 
     // Per-kernel timing with HIP events on the library stream.  While enabled, every launch of the
     // kernels below is bracketed by an event pair; collect_kernel_times() synchronises and adds the
@@ -148,6 +164,8 @@ class LlamaRuntime {
     // captured greedy step per sequence (head -> feed -> trunk -> keep), and its device-side state
     bool use_graph_ = true;
     std::vector<hipGraphExec_t> step_graphs_, multi_graphs_;   // one step, kStepsPerGraph steps
+    unsigned long long id_ = 0, graph_epoch_ = 1;
+    DeviceLoopSession loop_session_;
     int *d_visible_ = nullptr, *d_log_ = nullptr, *d_log_count_ = nullptr;
     ArgmaxScratch argmax_scratch_;
     int head_partial_capacity_ = 0;      // (value, index) slots per row for the head's per-workgroup candidates
