@@ -1045,9 +1045,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
     stamp(a, 0);
     // Activations given as fp16 and K split over all wavefronts of the workgroup: a wavefront needs only its own S super-block columns
     // of them, stages those by itself and waits for no other wavefront (LDS operations of one wavefront complete in order).  Used at
-    // 14336 columns (4096 x 14336 in a train: 9.0 against 9.3 us for one row, 10.1 against 10.4 for two); at 4096 columns the common
-    // staging measures better for one row (14336 x 4096: 9.4 against 9.8 us).
-    constexpr bool PRIVATE = MODE == 0 && KS == WAVES && IPR >= 128;
+    // 14336 columns (4096 x 14336 in a train: 9.0 against 9.3 us for one row, 10.1 against 10.4 for two) and for two and more rows;
+    // at 4096 columns the common staging measures better for one row (14336 x 4096: 9.4 against 9.8 us; two rows 10.2 against 10.4-10.7).
+    constexpr bool PRIVATE = MODE == 0 && KS == WAVES && (IPR >= 128 || NB >= 2);
     constexpr int SLICE = S * 32, KW = (SLICE + 63) / 64;          // groups of eight columns in a wavefront's share
     MfmaStage<NB, IPR, THREADS, MODE> stage;
     uint4 own[PRIVATE ? NB : 1][PRIVATE ? KW : 1];
@@ -1294,17 +1294,41 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t
     };
 
     stamp(a, 0);
+    // fp16 activations and K split over all wavefronts: a wavefront stages its own S tiles' columns and waits for no other
+    // (as in gemv_q4k_mfma_kernel; 14336 columns only)
+    // (4096 x 14336: one row 8.9 against 8.7 us, so one row keeps the common staging; two rows 9.4 against 9.8, four 11.0 against 12.0)
+    constexpr bool PRIVATE = MODE == 0 && KS == WAVES && TPR >= 16 && NB >= 2;
+    constexpr int SLICE = S * 64, KW = (SLICE + 63) / 64;          // groups of eight columns in a wavefront's share
     MfmaStage<NB, IPR, THREADS, MODE, true> stage;
-    stage.issue(a);
+    uint4 own[PRIVATE ? NB : 1][PRIVATE ? KW : 1];
+    if constexpr (PRIVATE) {
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+#pragma unroll
+            for (int k = 0; k < KW; k++) own[b][k] = reinterpret_cast<const uint4 *>(a.x)[(size_t)b * GROUPS + SLICE * ks + lane + 64 * k];
+    } else {
+        stage.issue(a);
+    }
     // steps in flight, as in gemv_q4k_mfma_kernel: with fourteen wavefronts a two-step ring filled up front has 129 KB on its
     // way before the staging barrier (4096 x 14336: 10.5 / 11.4 / 13.7 us for one / two / four rows; one step ahead 8.7 / 9.8 / 12.1)
     constexpr int AHEAD = DEPTH == 2 ? 1 : DEPTH;
     Q40Item ring[DEPTH];
 #pragma unroll
     for (int d = 0; d < AHEAD; d++) ring[d] = load_step(d);
-    if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
-    stage.finish(a, xs4, xsum, misc);
-    __syncthreads();
+    if constexpr (PRIVATE) {
+        if (lane < 8) zero4[lane] = make_uint4(0, 0, 0, 0);        // every wavefront writes the same zeros
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+#pragma unroll
+            for (int k = 0; k < KW; k++) q4k_store_group_natural<true>(own[b][k], b, SLICE * ks + lane + 64 * k, cols, xs4, xsum);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
+        if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
+        stage.finish(a, xs4, xsum, misc);
+        __syncthreads();
+    }
     stamp(a, 1);
 
     // A operand: slot i = lane % 16 carries activation row i % 4 in lane group i / 4 only; group index of (tile step, j, fragment f)
