@@ -38,6 +38,7 @@ def tiled_blocks(fmt, rows, cols, seed, period=1031):
 @pytest.mark.parametrize("name,rows,cols", [
     ("q4_k", 4096, 4096), ("q4_k", 1024, 4096), ("q4_k", 14336, 4096), ("q4_k", 4096, 14336), ("q4_k", 28672, 4096),
     ("q4_0", 4096, 4096), ("q4_0", 14336, 4096), ("q4_0", 4096, 14336), ("q8_0", 32000, 768),
+    ("q8_0", 16390, 256),   # a tall matrix (four rows per wavefront) whose last workgroup is ragged
 ])
 def test_full_size_weight_gemv_matches_oracle(mods, name, rows, cols):
     ll, ops, syn = mods
