@@ -152,3 +152,27 @@ def test_lock_step_loops_on_the_device_equal_the_host_loops(llama, n_seq):
                 passes, committed, accepted = runs[(True, True)][1]
                 assert accepted == 14 * n_seq and committed == 29 * n_seq and passes == 15
         target.close(); draft.close()
+
+
+def test_device_loop_session_is_reused_and_rebuilt(llama):
+    """The target keeps the loop's device state, log and captured passes between calls: the same pair again (other budgets, long
+    enough for the four-pass graph and too short for it), another draft, the first draft again, and a pair whose kernels changed
+    (merged attention switched off and on) all give the host-driven loop's result."""
+    fmt = orc.FMT_F16
+    packed = weights(fmt, 31, 3, upper_scale=0.05)
+    other = weights(fmt, 32, 3, upper_scale=1.0)
+    target = build(llama, packed, fmt, 3, 64)
+    draft_a, draft_b = build(llama, packed, fmt, 1, 64), build(llama, other, fmt, 1, 64)
+    prompt = [7, 8, 9, 10, 11]
+    seen = []
+    for draft, budget in ((draft_a, 40), (draft_a, 9), (draft_a, 33), (draft_b, 40), (draft_a, 40), (draft_b, 5)):
+        tokens, _ = both_ways(llama, target, draft, prompt, budget)
+        seen.append(tokens)
+    assert seen[0] == seen[4] and seen[0][:9] == seen[1] and seen[3][:5] == seen[5] and seen[0] == seen[3]   # exact: the draft does not matter
+    for enabled in (False, True):
+        llama.set_merged_attention(draft_a, enabled)
+        llama.set_merged_attention(target, enabled)
+        tokens, _ = both_ways(llama, target, draft_a, prompt, 40)
+        assert tokens == seen[0]
+    for rt in (target, draft_a, draft_b):
+        rt.close()
