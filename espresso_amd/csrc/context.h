@@ -4,6 +4,7 @@
 #include <string>
 
 #include "../../include/espresso_hip.h"
+#include "../../include/espresso_hip_bench.h"
 #include "common.h"
 
 namespace esp {

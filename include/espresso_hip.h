@@ -88,12 +88,6 @@ int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y
  * GPU's array: calls that overlap on one GPU race. */
 int esp_gemv_device_noalloc(const ESPMatrix *matrix, const uint16_t *x_f16_device, int batch, float *y_device,
                             const float *residual_device_or_null);
-/* Times the GEMV kernel alone on buffers already resident in HBM: `warmup` untimed launches, then
- * `iters` launches bracketed by HIP events on the library stream.  Reports the mean and the best
- * per-launch time in microseconds.  rotate > 1 cycles through that many copies of the matrix so
- * that no launch finds its weights in the last-level cache. */
-int esp_gemv_time(const ESPMatrix *matrix, int batch, int warmup, int iters, int rotate,
-                  double *mean_us, double *best_us);
 
 /* ---- INT4 output head ---------------------------------------------------------------------------- *
  * INT4Classifier (Sources/Espresso/INT4Classifier.swift:40-160) over TensorBufferINT4
@@ -107,38 +101,6 @@ ESPInt4Classifier *esp_int4_classifier_create(const float *weights_f32, int rows
 void esp_int4_classifier_free(ESPInt4Classifier *classifier);
 int esp_int4_classifier_export(const ESPInt4Classifier *classifier, uint8_t *packed, float *scales, float *biases);
 int esp_int4_classifier_matvec_argmax(ESPInt4Classifier *classifier, const float *input, float *logits_or_null, int *index_or_null);
-
-/* Measurement aid (no counterpart in the reference): runs the Q4_K GEMV back to back over copies of the matrix that together
- * exceed the caches (at least `launches` - 1 times and once through all copies: weights from HBM, code and activations warm,
- * the state a decode step finds); every wavefront of one launch inside that train records four 100 MHz wall-clock stamps:
- * start, activations staged, first weights consumed, end.  out_stamps receives [wavefront][4]; *out_wavefronts how many
- * wavefronts wrote (at most capacity_wavefronts); *out_period_us (may be null) the time from the first wavefront start of
- * that launch to the first wavefront start of the next one: the launch's share of the train, which exceeds its last
- * wavefront's end by the time in which no wavefront of either kernel runs. */
-int esp_gemv_stamps(const ESPMatrix *matrix, int batch, int launches, uint64_t *out_stamps, int capacity_wavefronts, int *out_wavefronts,
-                    double *out_period_us);
-/* Kernel-selection switches for measurements and tests (no counterpart in the reference); the same switches are read from
- * the environment when first needed.  "q4k_mfma" (ESPRESSO_HIP_Q4K_MFMA): 1 = Q4_K GEMVs of 4096 / 14336 columns run on the
- * matrix cores (one to eight activation rows per pass over the weights), 0 = never, -1 = the library's own choice.
- * "q40_mfma" (ESPRESSO_HIP_Q40_MFMA): the same for Q4_0 (one to four rows).
- * "q4k_mfma_ks" / "q4k_mfma_waves" (ESPRESSO_HIP_Q4K_MFMA_KS / _WAVES): wavefronts that share a block of sixteen rows and
- * wavefronts per workgroup, 0 = by shape; combinations without a compiled kernel fall back to the dot-product kernels.
- * "q4k_mfma_ragged": 0 = every workgroup runs the same number of rounds.
- * "q4k_long_row_waves" (ESPRESSO_HIP_Q4K_LONG_ROW_WAVES): one activation row at 14336 columns: 0 (default) = the matrix-core
- * kernel, 8 or 4 = the dot-product kernel with that many wavefronts per workgroup (one or three workgroups per compute unit).
- * Runtimes that captured a step graph keep the kernels they captured. */
-int esp_set_tuning(const char *key, int value);
-/* Measurement aid with no counterpart in the reference: a kernel that only streams `bytes` (>= 1 MiB, a
- * multiple of 16) from HBM with 128-bit loads, `iters` times; reports GB/s.  bench.py prints it next to the
- * GEMV bandwidth so that fractions of the published peak can be read against what a plain reader gets. */
-int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s);
-/* The ceiling for ONE GEMV launch: a kernel with a persistent Q4_K GEMV's grid (`workgroups` of `wavefronts` = 4 or 8) and its
- * loads (a wavefront takes items of `pair_bytes`, a 2304-byte weight tile of the matrix-core kernel or a pair of rows of the
- * dot-product kernel, the next item's 128-bit loads in flight while the current one is consumed) that does nothing else, launched back to back `launches` times over `copies` buffers of `bytes_per_launch` in
- * turn (so that no launch finds its bytes in a cache).  Reports the mean time per launch, which includes what a dependent
- * launch costs on this machine, and the resulting GB/s. */
-int esp_hbm_read_probe_pairs(size_t bytes_per_launch, int pair_bytes, int workgroups, int wavefronts, int copies, int launches, double *mean_us,
-                             double *gb_per_s);
 
 /* ---- llama decoder state resident on the GPU -------------------------------------------- *
  * Replaces CPUExactLlamaRuntime (Sources/RealModelInference/RealModelInferenceEngine.swift:548-850):
@@ -255,34 +217,6 @@ int esp_llama_set_matrix_prefill(ESPLlamaRuntime *runtime, int enabled);
  * (head size 128, Q4_K wo of 2048 or 4096 columns).  enabled = 0 restores the split kernel plus the merge kernel
  * everywhere.  Returns 1 when the merged form is in use after the call, 0 when not, negative on error. */
 int esp_llama_set_merged_attention(ESPLlamaRuntime *runtime, int enabled);
-
-/* Per-kernel timing with HIP events on the library stream.  While enabled every launch of the GEMV
- * and attention kernels of a step is bracketed by an event pair; esp_llama_kernel_times synchronises
- * and reports, per kernel class, the summed elapsed microseconds, the launch count and the
- * algorithmic bytes of one batch-1 launch (packed weights + fp16 input + fp32 output).  Class
- * ESP_KERNEL_EVENT_PAIR brackets nothing, once per step: its mean is what an event pair itself adds to
- * every other class's mean. */
-#define ESP_KERNEL_QKV 0
-#define ESP_KERNEL_WO 1
-#define ESP_KERNEL_GATE_UP 2
-#define ESP_KERNEL_DOWN 3
-#define ESP_KERNEL_HEAD 4
-#define ESP_KERNEL_ATTENTION 5
-#define ESP_KERNEL_EVENT_PAIR 6
-#define ESP_KERNEL_CLASS_COUNT 7
-int esp_llama_set_kernel_timing(ESPLlamaRuntime *runtime, int enabled);
-int esp_llama_kernel_times(ESPLlamaRuntime *runtime, double *total_us, int64_t *launches, uint64_t *bytes_per_launch,
-                           int reset);
-/* The GEMV of one class (ESP_KERNEL_QKV .. ESP_KERNEL_HEAD) launched for every layer in turn, `iters` rounds,
- * between two HIP events: the mean duration of back-to-back dependent launches at the model's real shapes over
- * its real weights (a round moves more bytes than any cache holds).  No per-launch event overhead, so the mean
- * is directly comparable with a rocprofv3 kernel trace.  The epilogues write into live buffers: reset the
- * runtime before decoding again. */
-int esp_llama_time_kernel(ESPLlamaRuntime *runtime, int kernel_class, int iters, double *mean_us);
-/* The same launches twice: back to back between two events (back_to_back_us, as above) and then with a pair of
- * events attached to every launch, which take the kernel's own start and end (kernel_us: the mean kernel duration,
- * the figure a rocprofv3 kernel trace reports for the kernel).  Measurement only; no counterpart in the reference. */
-int esp_llama_time_kernel_dispatch(ESPLlamaRuntime *runtime, int kernel_class, int iters, double *back_to_back_us, double *kernel_us);
 
 /* ---- seeded synthetic weights ------------------------------------------------------------- *
  * Fills `out_blocks` (host memory, esp_format_bytes(format, elements) bytes) with N(0, std_dev) draws

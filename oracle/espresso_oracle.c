@@ -316,6 +316,12 @@ int orc_quantize(int format, const float *x, size_t elements, uint8_t *blocks) {
 
 /* ----------------------------------------------------------- math helpers */
 
+/* Worker threads for orc_matvec (1 = the single-threaded loop of the reference).  Timing and long walks only:
+ * results are bit-identical for every count. */
+static int g_threads = 1;
+void orc_set_threads(int threads) { g_threads = threads < 1 ? 1 : threads; }
+int orc_get_threads(void) { return g_threads; }
+
 /* Dot product in a fixed order: eight interleaved partial sums (element i goes
  * to lane i mod 8, ascending), combined pairwise.  The reference calls
  * Accelerate (vDSP_mmul / vDSP_dotpr / vDSP_svesq), whose order is not
@@ -357,6 +363,13 @@ void orc_per_head_rmsnorm(float *values, const float *weights, int heads, int he
 
 /* RealModelInferenceEngine.swift:6674-6718 — y = W x, W row-major [rows, cols]. */
 void orc_matvec(const float *matrix, int rows, int cols, const float *x, float *y) {
+    /* Rows are independent and each row's sum keeps its order, so the result does not depend on the thread count. */
+    int threads = g_threads;
+    if (threads > 1 && (size_t)rows * (size_t)cols >= ((size_t)1 << 18)) {
+#pragma omp parallel for num_threads(threads) schedule(static)
+        for (int r = 0; r < rows; r++) y[r] = dot8(matrix + (size_t)r * cols, x, cols);
+        return;
+    }
     for (int r = 0; r < rows; r++) y[r] = dot8(matrix + (size_t)r * cols, x, cols);
 }
 
@@ -620,6 +633,46 @@ int orc_llama_set_weight(orc_llama_runtime *rt, int layer, int slot, const float
     memcpy(*dst, data, sizeof(float) * count);
     return 0;
 }
+
+/* Same as orc_llama_set_weight for a matrix given as GGUF blocks: dequantised straight into the runtime's own
+ * buffer (no intermediate fp32 copy of an 8B-parameter model on the caller's side). */
+int orc_llama_set_weight_blocks(orc_llama_runtime *rt, int layer, int slot, int format, const uint8_t *blocks, size_t count) {
+    float *values = (float *)malloc(sizeof(float) * count);
+    if (!values) return -4;
+    if (orc_dequantize(format, blocks, count, values) != 0) { free(values); return -3; }
+    /* hand the buffer over instead of copying it */
+    const orc_llama_config *c = &rt->c;
+    float **dst = NULL;
+    size_t expected = 0;
+    size_t d = (size_t)c->d_model;
+    switch (slot) {
+    case ORC_W_TOKEN_EMBEDDING: dst = &rt->token_embedding; expected = (size_t)c->vocab * d; break;
+    case ORC_W_LM_HEAD: dst = &rt->lm_head; expected = (size_t)c->vocab * d; break;
+    default:
+        if (layer < 0 || layer >= c->n_layer) { free(values); return -1; }
+        {
+            orc_layer *L = &rt->layers[layer];
+            switch (slot) {
+            case ORC_W_WQ: dst = &L->wq; expected = d * attn_dim(c); break;
+            case ORC_W_WK: dst = &L->wk; expected = d * kv_dim(c); break;
+            case ORC_W_WV: dst = &L->wv; expected = d * kv_dim(c); break;
+            case ORC_W_WO: dst = &L->wo; expected = d * attn_dim(c); break;
+            case ORC_W_W1: dst = &L->w1; expected = d * c->hidden_dim; break;
+            case ORC_W_W2: dst = &L->w2; expected = d * c->hidden_dim; break;
+            case ORC_W_W3: dst = &L->w3; expected = d * c->hidden_dim; break;
+            default: free(values); return -1;
+            }
+        }
+    }
+    if (count != expected) { free(values); return -2; }
+    free(*dst);
+    *dst = values;
+    return 0;
+}
+
+/* Switches the activation mode of an existing runtime (weights stay): 0 = the reference's default, fp32 activations
+ * into every matrix product; 1 = rounded to fp16 first, as the GPU kernels take them. */
+void orc_llama_set_gemv_inputs_fp16(orc_llama_runtime *rt, int enabled) { rt->c.gemv_inputs_fp16 = enabled ? 1 : 0; }
 
 /* :616-635 */
 void orc_llama_reset(orc_llama_runtime *rt) {

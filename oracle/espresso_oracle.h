@@ -71,6 +71,9 @@ void orc_q4_k_scale_min(int j, const uint8_t *scales12, uint8_t *sc, uint8_t *m)
 void orc_rmsnorm(const float *x, const float *weight, float eps, int n, float *out);
 void orc_per_head_rmsnorm(float *values, const float *weights, int heads, int head_dim, float eps);
 void orc_matvec(const float *matrix, int rows, int cols, const float *x, float *y);
+/* Threads used by orc_matvec on large matrices (default 1; results do not depend on it). */
+void orc_set_threads(int threads);
+int orc_get_threads(void);
 void orc_rope_half_split(float *values, int heads, int head_dim, int position, float theta);
 void orc_attention_decode(const float *q, const float *k_cache, const float *v_cache, int heads,
                           int kv_heads, int head_dim, int visible, int cache_stride, float *context);
@@ -113,6 +116,9 @@ orc_llama_runtime *orc_llama_create(const orc_llama_config *config);
 void orc_llama_free(orc_llama_runtime *rt);
 /* copies `count` floats; layer ignored for the three top-level slots. 0 on success. */
 int orc_llama_set_weight(orc_llama_runtime *rt, int layer, int slot, const float *data, size_t count);
+/* A matrix slot (embedding, head, wq..w3) from GGUF blocks of `format`, `count` elements. */
+int orc_llama_set_weight_blocks(orc_llama_runtime *rt, int layer, int slot, int format, const uint8_t *blocks, size_t count);
+void orc_llama_set_gemv_inputs_fp16(orc_llama_runtime *rt, int enabled);
 void orc_llama_reset(orc_llama_runtime *rt);
 /* 0 ok; -1 empty prompt; -2 position beyond max_seq; -3 token outside vocab */
 int orc_llama_prefill(orc_llama_runtime *rt, const uint32_t *tokens, int count);

@@ -72,6 +72,10 @@ def lib():
     L.orc_llama_free.argtypes = [vp]
     L.orc_llama_set_weight.restype = C.c_int
     L.orc_llama_set_weight.argtypes = [vp, C.c_int, C.c_int, vp, C.c_size_t]
+    L.orc_llama_set_weight_blocks.restype = C.c_int
+    L.orc_llama_set_weight_blocks.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, C.c_size_t]
+    L.orc_set_threads.argtypes = [C.c_int]
+    L.orc_get_threads.restype = C.c_int
     L.orc_llama_reset.argtypes = [vp]
     L.orc_llama_prefill.restype = C.c_int; L.orc_llama_prefill.argtypes = [vp, vp, C.c_int]
     L.orc_llama_advance.restype = C.c_int; L.orc_llama_advance.argtypes = [vp, C.c_uint32]
@@ -157,6 +161,15 @@ def per_head_rmsnorm(values, weights, heads, head_dim, eps):
     w = _f32(weights)
     lib().orc_per_head_rmsnorm(_ptr(v), _ptr(w), heads, head_dim, C.c_float(eps))
     return v
+
+
+def set_threads(n: int) -> None:
+    """Threads for matvec on large matrices (rows are independent: results are bit-identical for every count)."""
+    lib().orc_set_threads(int(n))
+
+
+def get_threads() -> int:
+    return int(lib().orc_get_threads())
 
 
 def matvec(W, x):
@@ -291,6 +304,20 @@ class LlamaRuntime:
         rc = lib().orc_llama_set_weight(self._h, layer, slot, _ptr(a), a.size)
         if rc != 0:
             raise ValueError(f"set_weight(layer={layer}, slot={slot}) failed: {rc}")
+
+    def set_weight_blocks(self, layer: int, slot: int, fmt: int, blocks, elements: int):
+        """A matrix slot from GGUF blocks, dequantised inside the oracle (no fp32 copy on the Python side)."""
+        b = np.ascontiguousarray(blocks, dtype=np.uint8)
+        assert b.size == format_bytes(fmt, elements)
+        rc = lib().orc_llama_set_weight_blocks(self._h, layer, slot, fmt, _ptr(b), elements)
+        if rc != 0:
+            raise ValueError(f"set_weight_blocks(layer={layer}, slot={slot}) failed: {rc}")
+
+    def set_gemv_inputs_fp16(self, enabled: bool):
+        """Switch the activation mode in place (the weights stay loaded)."""
+        lib().orc_llama_set_gemv_inputs_fp16.argtypes = [C.c_void_p, C.c_int]
+        lib().orc_llama_set_gemv_inputs_fp16(self._h, int(enabled))
+        self.cfg.gemv_inputs_fp16 = bool(enabled)
 
     def reset(self):
         lib().orc_llama_reset(self._h)

@@ -74,15 +74,15 @@ def oracle_from_packed(cfg, packed, fmt, n_layer, kv_fp16, max_seq, gemv_inputs_
     slot = {"wq": orc.W_WQ, "wk": orc.W_WK, "wv": orc.W_WV, "wo": orc.W_WO, "w1": orc.W_W1, "w2": orc.W_W2, "w3": orc.W_W3}
     rt = orc.LlamaRuntime(ocfg)
     n = cfg.vocab * cfg.d_model
-    rt.set_weight(0, orc.W_TOKEN_EMBEDDING, orc.dequantize(orc.FMT_F16, packed["embedding"], n))
+    rt.set_weight_blocks(0, orc.W_TOKEN_EMBEDDING, orc.FMT_F16, packed["embedding"], n)
     rt.set_weight(0, orc.W_FINAL_NORM, np.ones(cfg.d_model, np.float32))
-    rt.set_weight(0, orc.W_LM_HEAD, orc.dequantize(fmt, packed["lm_head"], n))
+    rt.set_weight_blocks(0, orc.W_LM_HEAD, fmt, packed["lm_head"], n)
     for l in range(n_layer):
         rt.set_weight(l, orc.W_RMS_ATT, np.ones(cfg.d_model, np.float32))
         rt.set_weight(l, orc.W_RMS_FFN, np.ones(cfg.d_model, np.float32))
         for k, s in slot.items():
             r, c = shapes[k]
-            rt.set_weight(l, s, orc.dequantize(fmt, packed["layers"][l][k], r * c))
+            rt.set_weight_blocks(l, s, fmt, packed["layers"][l][k], r * c)
     return rt
 
 

@@ -17,13 +17,38 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def test_library_exports_every_declared_symbol():
-    header = open(os.path.join(ROOT, "include", "espresso_hip.h")).read()
-    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
-    names = set(re.findall(r"\b(esp_[a-z0-9_]+)\s*\(", header))
-    assert len(names) > 40
+    names = set()
+    for name in ("espresso_hip.h", "espresso_hip_bench.h"):
+        header = open(os.path.join(ROOT, "include", name)).read()
+        header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+        found = set(re.findall(r"\b(esp_[a-z0-9_]+)\s*\(", header))
+        assert len(found) > (40 if name == "espresso_hip.h" else 5)
+        names |= found
     L = lib.load_library()
     missing = [n for n in sorted(names) if not hasattr(L, n)]
     assert not missing, missing
+
+
+def test_headers_are_plain_c11_and_the_boundary_header_holds_no_measurement_calls():
+    """The module map hands espresso_hip.h to a C importer (Swift's clang importer reads it as C): it has to stay valid
+    C11 with no C++ or compiler extensions.  Measurement and tuning calls live in espresso_hip_bench.h, outside the
+    drop-in boundary."""
+    import shutil
+    import subprocess
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    inc = os.path.join(ROOT, "include")
+    for name in ("espresso_hip.h", "espresso_hip_bench.h"):
+        proc = subprocess.run([cc, "-x", "c", "-std=c11", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", inc,
+                               os.path.join(inc, name)], capture_output=True, text=True)
+        assert proc.returncode == 0, proc.stderr
+    boundary = open(os.path.join(inc, "espresso_hip.h")).read()
+    for name in ("esp_gemv_time", "esp_gemv_stamps", "esp_set_tuning", "esp_hbm_read_probe", "esp_llama_time_kernel",
+                 "esp_llama_set_kernel_timing", "esp_llama_kernel_times"):
+        assert name + "(" not in boundary, name
+    modulemap = open(os.path.join(inc, "module.modulemap")).read()
+    assert 'header "espresso_hip.h"' in modulemap and "espresso_hip_bench.h" not in modulemap
 
 
 def test_no_device_fails_loudly_without_cpu_fallback():
