@@ -132,5 +132,7 @@ def _declare_llama(L: C.CDLL) -> None:
     L.esp_llama_set_graph_replay.argtypes = [vp, i32]
     L.esp_llama_set_merged_attention.restype = i32
     L.esp_llama_set_merged_attention.argtypes = [vp, i32]
+    L.esp_llama_set_split_activations.restype = i32
+    L.esp_llama_set_split_activations.argtypes = [vp, i32]
     L.esp_llama_set_matrix_prefill.restype = i32
     L.esp_llama_set_matrix_prefill.argtypes = [vp, i32]

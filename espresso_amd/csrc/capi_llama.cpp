@@ -159,6 +159,12 @@ int esp_llama_set_merged_attention(ESPLlamaRuntime *runtime, int enabled) {
     return runtime->rt->merged_attention_in_use() ? 1 : 0;
 }
 
+int esp_llama_set_split_activations(ESPLlamaRuntime *runtime, int enabled) {
+    if (!runtime || !runtime->rt) return fail(ESP_ERR_INVALID_ARGUMENT, "set_split_activations: null runtime");
+    runtime->rt->set_split_activations(enabled != 0);
+    return ESP_OK;
+}
+
 int esp_llama_set_matrix_prefill(ESPLlamaRuntime *runtime, int enabled) {
     if (!runtime || !runtime->rt) return fail(ESP_ERR_INVALID_ARGUMENT, "set_matrix_prefill: null runtime");
     runtime->rt->set_matrix_prefill(enabled != 0);

@@ -392,6 +392,7 @@ int esp_gemv_stamps(const ESPMatrix *matrix, int batch, int launches, uint64_t *
         for (int k = 0; k < 4 && e == hipSuccess; k++) {
             p.w = copies[warm + k];
             p.stamps = k < 2 ? d_s + (size_t)k * words : nullptr;
+            p.stamp_capacity = capacity_wavefronts;   // wavefronts beyond it leave no stamp
             e = launch_gemv(p, c.stream);
         }
         if (e == hipSuccess) e = hipMemcpyAsync(out_stamps, d_s, words * 8, hipMemcpyDeviceToHost, c.stream);

@@ -96,8 +96,15 @@ struct GemvParams {
     int *argmax_index = nullptr;
     int argmax_capacity = 0;
     int *argmax_blocks = nullptr;
-    // measurement only: device buffer of four wall-clock stamps (100 MHz) per wavefront of the launch (persistent Q4_K kernels)
+    // split activations (gemv_splits_activations says where): `x` holds two fp16 rows per activation row, hi = fp16(v) and
+    // lo = fp16((v - hi) * 2048), [2 * batch][cols]; with norm_x or merge_partials the staging makes both from the fp32 values.
+    // The products then carry the activations to about 22 bits instead of 11.  split_out: EPI_SWIGLU_F16 writes such row pairs,
+    // out_f16 = [2 * batch][rows / 2].
+    bool split_x = false, split_out = false;
+    // measurement only: device buffer of four wall-clock stamps (100 MHz) per wavefront of the launch, room for stamp_capacity
+    // wavefronts (matrix-core Q4_K kernel, fp16 activations given, one or two rows)
     unsigned long long *stamps = nullptr;
+    int stamp_capacity = 0;
     int batch = 1;
     int epilogue = EPI_STORE_F32;
     // optional (batch <= 2): events that take the kernel's own start and end times
@@ -123,6 +130,7 @@ struct GemmParams {
 
 // kernels/gemv.hip
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
+bool gemv_splits_activations(const DeviceMatrix &w, int batch);
 // Slices of the prefix per query head that launch_attention_partials writes and the merging GEMV reads.
 #ifndef ESP_ATTENTION_HEAD_SPLITS
 #define ESP_ATTENTION_HEAD_SPLITS 4

@@ -104,13 +104,21 @@ struct KernelArgs {
     // EPI_ARGMAX: one (value, index) pair per workgroup and batch row, [batch][gridDim.x]
     float *part_value;
     int *part_index;
-    // measurement only (null otherwise): four 100 MHz wall-clock stamps per wavefront, [wavefront][4] =
-    // start, activations staged, first weights consumed, end
+    // split activations (matrix-core Q4_K kernel): x holds two fp16 rows per activation row, hi and lo (see split_group); with
+    // the fused norm or the merged attention states the staging makes both.  split_out: the SiLU(gate)*up epilogue writes such
+    // row pairs.
+    int split_x, split_out;
+    // measurement only (null otherwise; read by the stamped instantiations alone): four 100 MHz wall-clock stamps per
+    // wavefront, [wavefront][4] = start, activations staged, first weights consumed, end; stamp_capacity wavefronts have room
     unsigned long long *stamps;
+    int stamp_capacity;
 };
+template <bool STAMPS>
 __device__ __forceinline__ void stamp(const KernelArgs &a, int which) {
-    if (a.stamps && (threadIdx.x & 63) == 0)
-        a.stamps[((size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 4 + which] = wall_clock64();
+    if constexpr (STAMPS) {
+        const int w = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+        if (a.stamps && (threadIdx.x & 63) == 0 && w < a.stamp_capacity) a.stamps[(size_t)w * 4 + which] = wall_clock64();
+    }
 }
 
 // First-max rule of the reference's output head (RealModelInferenceEngine.swift:8219-8275, neon_convert.c:36-101): a larger
@@ -143,7 +151,8 @@ __device__ __forceinline__ void argmax_workgroup(const KernelArgs &a, const floa
 // The arithmetic of attention_merge_kernel: M = max m, f = exp(m - M) (0 for an empty split), L = fma(l, f, L),
 // A = fma(acc, f, A) in split order, context = A / L, rounded to fp16.  Eight channels of one query head.
 constexpr int kMergeSplits = kAttentionHeadSplits;
-__device__ __forceinline__ uint4 merge_group(const float2 (&ml)[kMergeSplits], const float4 (&a0)[kMergeSplits], const float4 (&a1)[kMergeSplits]) {
+__device__ __forceinline__ void merge_group_values(const float2 (&ml)[kMergeSplits], const float4 (&a0)[kMergeSplits], const float4 (&a1)[kMergeSplits],
+                                                   float (&c)[8]) {
     float M = ml[0].x;
 #pragma unroll
     for (int sp = 1; sp < kMergeSplits; sp++) M = fmaxf(M, ml[sp].x);
@@ -156,9 +165,12 @@ __device__ __forceinline__ uint4 merge_group(const float2 (&ml)[kMergeSplits], c
 #pragma unroll
         for (int i = 0; i < 8; i++) A[i] = __builtin_fmaf(v[i], f, A[i]);
     }
-    float c[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) c[i] = L > 0.0f ? A[i] / L : 0.0f;
+}
+__device__ __forceinline__ uint4 merge_group(const float2 (&ml)[kMergeSplits], const float4 (&a0)[kMergeSplits], const float4 (&a1)[kMergeSplits]) {
+    float c[8];
+    merge_group_values(ml, a0, a1, c);
     uint4 h;
     h.x = pack_half2(c[0], c[1]); h.y = pack_half2(c[2], c[3]); h.z = pack_half2(c[4], c[5]); h.w = pack_half2(c[6], c[7]);
     return h;
@@ -211,7 +223,15 @@ __device__ __forceinline__ void pair_epilogue(const KernelArgs &a, int pair, con
             for (int b = 0; b < B; b++) {
                 const float hg = __fmul_rn(0.5f, va[b]);
                 const float silu = __fmul_rn(hg, __fadd_rn(1.0f, tanhf(hg)));
-                a.out_f16[(size_t)b * (a.rows / 2) + pair] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(silu, vb[b]));
+                const float act = __fmul_rn(silu, vb[b]);
+                if (a.split_out) {   // hi and lo rows for a consumer that takes split activations
+                    const _Float16 hi = (_Float16)act;
+                    a.out_f16[(size_t)(2 * b) * (a.rows / 2) + pair] = __builtin_bit_cast(uint16_t, hi);
+                    a.out_f16[(size_t)(2 * b + 1) * (a.rows / 2) + pair] =
+                        __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(__fsub_rn(act, (float)hi), kSplitScale));
+                } else {
+                    a.out_f16[(size_t)b * (a.rows / 2) + pair] = __builtin_bit_cast(uint16_t, (_Float16)act);
+                }
             }
         }
         return;
@@ -753,17 +773,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_kernel(const uint8_t *qs,
     typename std::conditional<MODE == 2, Q4KMergeStage<B, MODE == 2 ? IPR : 32>, Q4KStage<B, IPR, MODE == 1, false, WAVES * 64>>::type stage;
     const int first_pair = blockIdx.x * TEAMS + wave / TEAM;
     int pair = first_pair;
-    stamp(a, 0);
     stage.issue(a);
     load_pair(pair, buf0);
     stage.finish(a, xs4, xsum, norm_red);
     __syncthreads();
-    stamp(a, 1);
     for (int j = 0; j < iters; j += 2) {
         int next = pair + n_teams;
         load_pair(next, buf1);
         process(buf0, pair, j);
-        if (j == 0) stamp(a, 2);
         pair = next;
         if (j + 1 < iters) {
             next = pair + n_teams;
@@ -772,7 +789,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_kernel(const uint8_t *qs,
             pair = next;
         }
     }
-    stamp(a, 3);
     if constexpr (TEAM == 1) {
         if (a.epilogue == EPI_ARGMAX) argmax_workgroup<B>(a, best, best_i, red, reinterpret_cast<int *>(red + B * kWaves));
     }
@@ -914,12 +930,16 @@ __device__ __forceinline__ float workgroup_sum_waves(float v, float *red) {
 
 // Activations of a row (fp16 as given, RMSNorm fused, or attention states merged) into LDS for the matrix-core kernel:
 // every load is issued before the first use, as in Q4KStage; THREADS threads take groups tid, tid + THREADS, ...
-template <int NB, int IPR, int THREADS, int MODE, bool Q40 = false>
+// SPLIT (Q4_K): the staged rows are hi / lo pairs (rows 2b and 2b + 1 of the LDS copy, see split_group); fp16 activations given
+// (MODE 0) then arrive as such pairs, 2 NB rows.
+template <int NB, int IPR, int THREADS, int MODE, bool Q40 = false, bool SPLIT = false>
 struct MfmaStage {
     static constexpr int GROUPS = IPR * 8, K = (GROUPS + THREADS - 1) / THREADS, cols = IPR * 64, WAVES = THREADS / 64;
+    static constexpr int NBX = SPLIT ? 2 * NB : NB;
     static constexpr bool FULL = GROUPS % THREADS == 0;
+    static_assert(!(Q40 && SPLIT), "split activations: Q4_K only");
     float4 v0[MODE == 1 ? NB : 1][K], v1[MODE == 1 ? NB : 1][K], g0[K], g1[K];
-    uint4 v[MODE == 0 ? NB : 1][K];
+    uint4 v[MODE == 0 ? NBX : 1][K];
     float4 a0[MODE == 2 ? K : 1][kMergeSplits], a1[MODE == 2 ? K : 1][kMergeSplits];
     float2 ml[MODE == 2 ? K : 1][kMergeSplits];
 
@@ -951,7 +971,7 @@ struct MfmaStage {
             load_merge_row(a, 0);
         } else {
 #pragma unroll
-            for (int b = 0; b < NB; b++)
+            for (int b = 0; b < NBX; b++)
 #pragma unroll
                 for (int k = 0; k < K; k++) v[b][k] = reinterpret_cast<const uint4 *>(a.x)[(size_t)b * (cols / 8) + group(k)];
         }
@@ -965,30 +985,49 @@ struct MfmaStage {
                 for (int k = 0; k < K; k++) s += sum_squares(v0[b][k], v1[b][k]);
                 const float inv = 1.0f / sqrtf(workgroup_sum_waves<WAVES>(s, red + b * WAVES) / (float)cols + a.norm_eps);
 #pragma unroll
-                for (int k = 0; k < K; k++)
-                    if (mine(k)) q4k_store_group_natural<Q40>(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, group(k), cols, xs4, xsum);
+                for (int k = 0; k < K; k++) {
+                    if (!mine(k)) continue;
+                    if constexpr (SPLIT) {
+                        float c[8];
+                        normalized_values(v0[b][k], v1[b][k], g0[k], g1[k], inv, c);
+                        q4k_store_split_natural(split_group(c), b, group(k), cols, xs4, xsum);
+                    } else {
+                        q4k_store_group_natural<Q40>(normalized_group(v0[b][k], v1[b][k], g0[k], g1[k], inv), b, group(k), cols, xs4, xsum);
+                    }
+                }
             }
         } else if constexpr (MODE == 2) {
 #pragma unroll
             for (int b = 0; b < NB; b++) {
                 if (b > 0) load_merge_row(a, b);
 #pragma unroll
-                for (int k = 0; k < K; k++)
-                    if (mine(k)) q4k_store_group_natural<Q40>(merge_group(ml[k], a0[k], a1[k]), b, group(k), cols, xs4, xsum);
+                for (int k = 0; k < K; k++) {
+                    if (!mine(k)) continue;
+                    if constexpr (SPLIT) {
+                        float c[8];
+                        merge_group_values(ml[k], a0[k], a1[k], c);
+                        q4k_store_split_natural(split_group(c), b, group(k), cols, xs4, xsum);
+                    } else {
+                        q4k_store_group_natural<Q40>(merge_group(ml[k], a0[k], a1[k]), b, group(k), cols, xs4, xsum);
+                    }
+                }
             }
         } else {
 #pragma unroll
             for (int b = 0; b < NB; b++)
 #pragma unroll
-                for (int k = 0; k < K; k++)
-                    if (mine(k)) q4k_store_group_natural<Q40>(v[b][k], b, group(k), cols, xs4, xsum);
+                for (int k = 0; k < K; k++) {
+                    if (!mine(k)) continue;
+                    if constexpr (SPLIT) q4k_store_split_natural(SplitGroup{v[2 * b][k], v[2 * b + 1][k]}, b, group(k), cols, xs4, xsum);
+                    else q4k_store_group_natural<Q40>(v[b][k], b, group(k), cols, xs4, xsum);
+                }
         }
     }
 };
 
 constexpr size_t kQ4KTileBytes = 2304;
 
-template <int NB, int IPR, int WAVES, int KS, int MODE>
+template <int NB, int IPR, int WAVES, int KS, int MODE, bool SPLIT = false, bool STAMPS = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t *tiled, const void *activations, const float *norm_w, int rows, int iters,
                                                                    int workgroups, float norm_eps, KernelArgs rest) {
     KernelArgs a = rest;
@@ -998,11 +1037,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
     else a.x = static_cast<const uint16_t *>(activations);
     constexpr int THREADS = WAVES * 64, cols = IPR * 64, NSB = IPR / 4, S = NSB / KS, RB = WAVES / KS, GROUPS = cols / 8;
     constexpr int DEPTH = S % 4 == 0 ? 4 : (S % 7 == 0 ? 7 : (S % 2 == 0 ? 2 : 1));   // divides S: a step's slot in the ring is a constant
-    constexpr int SETS = (NB + 3) / 4;   // activation rows 4 s .. 4 s + 3 ride in the slots of A operand set s; every set meets the same B operand
-    static_assert(NSB % KS == 0 && WAVES % KS == 0 && NB >= 1 && NB <= 8, "whole super-blocks per wavefront");
+    constexpr int NBX = SPLIT ? 2 * NB : NB;   // staged fp16 rows: with split activations row b is the pair (2b: hi, 2b + 1: lo)
+    constexpr int SETS = (NBX + 3) / 4;   // staged rows 4 s .. 4 s + 3 ride in the slots of A operand set s; every set meets the same B operand
+    static_assert(NSB % KS == 0 && WAVES % KS == 0 && NB >= 1 && NBX <= 8, "whole super-blocks per wavefront");
     extern __shared__ uint4 smem_raw[];
-    uint4 *xs4 = smem_raw;                                        // [NB][GROUPS] groups of eight fp16, (0,2,1,3) order inside fours
-    uint4 *zero4 = xs4 + (size_t)NB * GROUPS;                     // eight groups of zeros
+    uint4 *xs4 = smem_raw;                                        // [NBX][GROUPS] groups of eight fp16, (0,2,1,3) order inside fours
+    uint4 *zero4 = xs4 + (size_t)NBX * GROUPS;                    // eight groups of zeros
     float *xsum = reinterpret_cast<float *>(zero4 + 8);           // [NB][cols / 32]
     float *red = xsum + (size_t)NB * (cols / 32);                 // [kMfmaRounds][WAVES][NB][16]   (KS > 1)
     float *misc = red + (KS > 1 ? kMfmaRounds * WAVES * NB * 16 : 0);   // [NB][WAVES] norm sums, later [2][NB][WAVES] arg-max candidates
@@ -1042,18 +1082,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
         return it;
     };
 
-    stamp(a, 0);
+    stamp<STAMPS>(a, 0);
     // Activations given as fp16 and K split over all wavefronts of the workgroup: a wavefront needs only its own S super-block columns
     // of them, stages those by itself and waits for no other wavefront (LDS operations of one wavefront complete in order).  Used at
     // 14336 columns (4096 x 14336 in a train: 9.0 against 9.3 us for one row, 10.1 against 10.4 for two) and for two and more rows;
     // at 4096 columns the common staging measures better for one row (14336 x 4096: 9.4 against 9.8 us; two rows 10.2 against 10.4-10.7).
-    constexpr bool PRIVATE = MODE == 0 && KS == WAVES && (IPR >= 128 || NB >= 2);
+    constexpr bool PRIVATE = MODE == 0 && KS == WAVES && (IPR >= 128 || NBX >= 2);
     constexpr int SLICE = S * 32, KW = (SLICE + 63) / 64;          // groups of eight columns in a wavefront's share
-    MfmaStage<NB, IPR, THREADS, MODE> stage;
-    uint4 own[PRIVATE ? NB : 1][PRIVATE ? KW : 1];
+    MfmaStage<NB, IPR, THREADS, MODE, false, SPLIT> stage;
+    uint4 own[PRIVATE ? NBX : 1][PRIVATE ? KW : 1];
     if constexpr (PRIVATE) {
 #pragma unroll
-        for (int b = 0; b < NB; b++)
+        for (int b = 0; b < NBX; b++)
 #pragma unroll
             for (int k = 0; k < KW; k++) {
                 const int gi = lane + 64 * k;
@@ -1080,7 +1120,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
         for (int b = 0; b < NB; b++)
 #pragma unroll
             for (int k = 0; k < KW; k++)
-                if (SLICE % 64 == 0 || lane + 64 * k < SLICE) q4k_store_group_natural(own[b][k], b, SLICE * ks + lane + 64 * k, cols, xs4, xsum);
+                if (SLICE % 64 == 0 || lane + 64 * k < SLICE) {
+                    if constexpr (SPLIT) q4k_store_split_natural(SplitGroup{own[2 * b][k], own[2 * b + 1][k]}, b, SLICE * ks + lane + 64 * k, cols, xs4, xsum);
+                    else q4k_store_group_natural(own[b][k], b, SLICE * ks + lane + 64 * k, cols, xs4, xsum);
+                }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -1089,15 +1132,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
         stage.finish(a, xs4, xsum, misc);
         __syncthreads();
     }
-    stamp(a, 1);
+    stamp<STAMPS>(a, 1);
 
-    // ---- the A operand: slot i = lane % 16 carries activation row i % 4 in lane group i / 4 only ----
+    // ---- the A operand: slot i = lane % 16 carries staged row i % 4 in lane group i / 4 only ----
     const int slot = lane & 15;
     const uint4 *a_base[SETS];
     int a_stride[SETS];                                            // groups per super-block step
 #pragma unroll
     for (int set = 0; set < SETS; set++) {
-        const bool feeds = (slot >> 2) == g && 4 * set + (slot & 3) < NB;
+        const bool feeds = (slot >> 2) == g && 4 * set + (slot & 3) < NBX;
         a_base[set] = feeds ? xs4 + (size_t)(4 * set + (slot & 3)) * GROUPS + 32 * (ks * S) + 8 * g : zero4;
         a_stride[set] = feeds ? 32 : 0;
     }
@@ -1135,7 +1178,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             const float2 xsp = *reinterpret_cast<const float2 *>(xsum_base + (size_t)b * (cols >> 5) + 8 * i);
-            const float nx_lo = lo[b >> 2][b & 3] - 64.0f * xsp.x, nx_hi = hi[b >> 2][b & 3] - 4.0f * xsp.y;
+            float raw_lo, raw_hi;
+            if constexpr (SPLIT) {   // the sums over the hi and the lo row of the pair
+                const int r0 = 2 * b, r1 = 2 * b + 1;
+                raw_lo = __builtin_fmaf(lo[r1 >> 2][r1 & 3], kSplitUnscale, lo[r0 >> 2][r0 & 3]);
+                raw_hi = __builtin_fmaf(hi[r1 >> 2][r1 & 3], kSplitUnscale, hi[r0 >> 2][r0 & 3]);
+            } else {
+                raw_lo = lo[b >> 2][b & 3];
+                raw_hi = hi[b >> 2][b & 3];
+            }
+            const float nx_lo = raw_lo - 64.0f * xsp.x, nx_hi = raw_hi - 4.0f * xsp.y;
             v[b] += d16 * (sc_lo * nx_lo + sc_hi * nx_hi) - dmin * (m_lo * xsp.x + m_hi * xsp.y);
         }
     };
@@ -1169,7 +1221,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
             const Q4KItem it = ring[i % DEPTH];
             ring[(i + AHEAD) % DEPTH] = load_step(round * S + i + AHEAD);
             step_compute(it, i);
-            if (a.stamps && round == 0 && i == 0) { if (v[0] != 12345.678f) stamp(a, 2); }   // after the first weights were needed
+            if constexpr (STAMPS) { if (a.stamps && round == 0 && i == 0 && v[0] != 12345.678f) stamp<STAMPS>(a, 2); }   // after the first weights were needed
         }
 #pragma unroll
         for (int b = 0; b < NB; b++) {          // the four lane groups of a row: every lane ends up with the row's share
@@ -1207,7 +1259,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
         }
     }
 
-    stamp(a, 3);
+    stamp<STAMPS>(a, 3);
     if (a.epilogue == EPI_ARGMAX) {
         // lanes 0..15 of the finishing wavefronts hold candidates: first within the wavefront, then over the workgroup
         float *cv = misc;
@@ -1293,7 +1345,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t
         return it;
     };
 
-    stamp(a, 0);
     // fp16 activations and K split over all wavefronts: a wavefront stages its own S tiles' columns and waits for no other
     // (as in gemv_q4k_mfma_kernel; 14336 columns only)
     // (4096 x 14336: one row 8.9 against 8.7 us, so one row keeps the common staging; two rows 9.4 against 9.8, four 11.0 against 12.0)
@@ -1329,7 +1380,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t
         stage.finish(a, xs4, xsum, misc);
         __syncthreads();
     }
-    stamp(a, 1);
 
     // A operand: slot i = lane % 16 carries activation row i % 4 in lane group i / 4 only; group index of (tile step, j, fragment f)
     // = 64 step + 16 j + 4 g + f
@@ -1402,7 +1452,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t
             const Q40Item it = ring[i % DEPTH];
             ring[(i + AHEAD) % DEPTH] = load_step(round * S + i + AHEAD);
             step_compute(it, i);
-            if (a.stamps && round == 0 && i == 0) { if (v[0] != 12345.678f) stamp(a, 2); }
         }
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -1437,7 +1486,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t
             }
         }
     }
-    stamp(a, 3);
     if (a.epilogue == EPI_ARGMAX) {
         float *cv = misc;
         int *ci = reinterpret_cast<int *>(misc + NB * WAVES);
@@ -1573,14 +1621,14 @@ int q4k_mfma_waves() {
     return g_q4k_mfma_waves;
 }
 
-template <int NB, int IPR, int WAVES, int KS, int MODE>
+template <int NB, int IPR, int WAVES, int KS, int MODE, bool SPLIT = false, bool STAMPS = false>
 hipError_t launch_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
-    constexpr int RB = WAVES / KS, cols = IPR * 64, THREADS = WAVES * 64;
+    constexpr int RB = WAVES / KS, cols = IPR * 64, THREADS = WAVES * 64, NBX = SPLIT ? 2 * NB : NB;
     *launched = false;
-    const size_t lds = ((size_t)NB * (cols / 8) + 8) * 16 + (size_t)NB * (cols / 32) * 4 + (KS > 1 ? (size_t)kMfmaRounds * WAVES * NB * 16 * 4 : 0) +
+    const size_t lds = ((size_t)NBX * (cols / 8) + 8) * 16 + (size_t)NB * (cols / 32) * 4 + (KS > 1 ? (size_t)kMfmaRounds * WAVES * NB * 16 * 4 : 0) +
                        (size_t)2 * NB * WAVES * 4;
     if (lds > 160 * 1024) return hipSuccess;   // not launched
-    auto kernel = gemv_q4k_mfma_kernel<NB, IPR, WAVES, KS, MODE>;
+    auto kernel = gemv_q4k_mfma_kernel<NB, IPR, WAVES, KS, MODE, SPLIT, STAMPS>;
     static size_t configured_lds = 0;
     hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
     if (e != hipSuccess) return e;
@@ -1632,28 +1680,37 @@ hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
         }
         if (waves == 0) waves = 8;
         if (ks == 0 || ks > waves) ks = waves;
+        // split activations: one and two rows; the stamped instantiations: fp16 activations given, not split
 #define ESP_MFMA_CASE(W_, KS_)                                                                                   \
         if (waves == W_ && ks == KS_) {                                                                          \
+            if constexpr (NB <= 2) if (a.split_x) {                                                              \
+                if (mode == 0) return launch_q4k_mfma<NB, 64, W_, KS_, 0, true>(a, stream, launched);             \
+                if (mode == 1) return launch_q4k_mfma<NB, 64, W_, KS_, 1, true>(a, stream, launched);             \
+                return launch_q4k_mfma<NB, 64, W_, KS_, 2, true>(a, stream, launched);                            \
+            }                                                                                                    \
+            if (a.split_x) return hipSuccess;                                                                    \
+            if constexpr (NB <= 2) if (a.stamps && mode == 0) return launch_q4k_mfma<NB, 64, W_, KS_, 0, false, true>(a, stream, launched); \
             if (mode == 0) return launch_q4k_mfma<NB, 64, W_, KS_, 0>(a, stream, launched);                       \
             if (mode == 1) return launch_q4k_mfma<NB, 64, W_, KS_, 1>(a, stream, launched);                       \
             if constexpr (NB <= 2) return launch_q4k_mfma<NB, 64, W_, KS_, 2>(a, stream, launched);               \
         }
         ESP_MFMA_CASE(4, 1)
-        ESP_MFMA_CASE(4, 2)
-        ESP_MFMA_CASE(4, 4)
-        ESP_MFMA_CASE(8, 4)
         ESP_MFMA_CASE(8, 8)
-        ESP_MFMA_CASE(16, 8)
         ESP_MFMA_CASE(16, 16)
 #undef ESP_MFMA_CASE
         return hipSuccess;
     }
     if (a.cols == 14336 && mode == 0) {
         if (waves == 0) waves = 8;
-        if (ks == 0) ks = 8;
+        if (ks == 0) ks = waves == 16 ? 8 : waves;
+        if (waves == 8 && ks == 8) {
+            if constexpr (NB <= 2) if (a.split_x) return launch_q4k_mfma<NB, 224, 8, 8, 0, true>(a, stream, launched);
+            if (a.split_x) return hipSuccess;
+            if constexpr (NB <= 2) if (a.stamps) return launch_q4k_mfma<NB, 224, 8, 8, 0, false, true>(a, stream, launched);
+            return launch_q4k_mfma<NB, 224, 8, 8, 0>(a, stream, launched);
+        }
+        if (a.split_x) return hipSuccess;
         if (waves == 4 && ks == 4) return launch_q4k_mfma<NB, 224, 4, 4, 0>(a, stream, launched);
-        if (waves == 8 && ks == 4) return launch_q4k_mfma<NB, 224, 8, 4, 0>(a, stream, launched);
-        if (waves == 8 && ks == 8) return launch_q4k_mfma<NB, 224, 8, 8, 0>(a, stream, launched);
         if (waves == 16 && ks == 8) return launch_q4k_mfma<NB, 224, 16, 8, 0>(a, stream, launched);
         return hipSuccess;
     }
@@ -1675,6 +1732,7 @@ hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
         const hipError_t e = try_q4k_mfma<B>(a, stream, &launched);
         if (e != hipSuccess || launched) return e;
     }
+    if (a.split_x) return hipErrorInvalidValue;   // only the matrix-core kernel reads hi / lo rows
     if (a.merge_partials && a.cols == 2048) return launch_q4k_persistent<B, 32, 1, 2>(a, stream);
     if (a.merge_partials && a.cols == 4096) return launch_q4k_persistent<B, 64, 1, 2>(a, stream);
     if (!a.merge_partials) switch (a.cols) {
@@ -1857,6 +1915,16 @@ bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
     return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (w.cols == 4096 && w.rows <= 8192);
 }
 
+// Whether launch_gemv takes split activations (GemvParams::split_x) for this matrix and row count: the matrix-core Q4_K kernel
+// at one or two rows, under the same conditions as its dispatch.
+bool gemv_splits_activations(const DeviceMatrix &w, int batch) {
+    if (w.format != FMT_Q4_K || !w.tiled || batch < 1 || batch > 2 || q4k_mfma_mode() == 0) return false;
+    if (q4k_mfma_waves() != 0 || q4k_mfma_split() != 0) return false;   // tuning overrides: not every variant has a split form
+    if (w.cols == 4096) return batch >= 2 || q4k_mfma_mode() == 1 || q4k_mfma_max_rows() <= 0 || w.rows <= q4k_mfma_max_rows();
+    if (w.cols == 14336) return batch >= 2 || q4k_mfma_mode() == 1 || q4k_long_row_waves() == 0;
+    return false;
+}
+
 bool gemv_supports_argmax(const DeviceMatrix &w) {
     return !(w.format == FMT_Q4_K && (w.cols == 8192 || w.cols == 11008 || w.cols == 14336));
 }
@@ -1868,6 +1936,8 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     if ((p.epilogue == EPI_STORE_F32 || p.epilogue == EPI_ADD_RESIDUAL) && !p.y) return hipErrorInvalidValue;
     if (p.epilogue == EPI_ADD_RESIDUAL && !p.residual) return hipErrorInvalidValue;
     if (p.epilogue == EPI_SWIGLU_F16 && (!p.out_f16 || w.rows % 2 != 0)) return hipErrorInvalidValue;
+    if (p.split_x && (!gemv_splits_activations(w, p.batch) || (w.cols == 14336 && (p.norm_x || p.merge_partials)))) return hipErrorInvalidValue;
+    if (p.split_out && (p.epilogue != EPI_SWIGLU_F16 || p.batch > 2)) return hipErrorInvalidValue;
     if (p.epilogue == EPI_ARGMAX && (!p.argmax_value || !p.argmax_index || p.argmax_capacity <= 0 || p.batch > 2 || !gemv_supports_argmax(w)))
         return hipErrorInvalidValue;
     if (p.epilogue == EPI_QKV_ROPE) {
@@ -1895,7 +1965,9 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         nb = fours && p.batch - b0 == 8 ? 8 : fours && p.batch - b0 >= 4 ? 4 : p.batch - b0 >= 2 ? 2 : 1;
         KernelArgs a;
         a.qs = w.qs; a.tiled = w.tiled; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.rows = w.rows; a.cols = w.cols;
-        a.x = p.x ? p.x + (size_t)b0 * w.cols : nullptr;
+        a.x = p.x ? p.x + (size_t)b0 * w.cols * (p.split_x ? 2 : 1) : nullptr;
+        a.split_x = p.split_x ? 1 : 0;
+        a.split_out = p.split_out ? 1 : 0;
         a.merge_partials = p.merge_partials;   // batch <= 2 here: one launch
         a.merge_head_dim = p.merge_head_dim;
         a.y = p.y ? p.y + (size_t)b0 * w.rows : nullptr;
@@ -1905,6 +1977,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         a.part_value = p.argmax_value;
         a.part_index = p.argmax_index;
         a.stamps = p.stamps;
+        a.stamp_capacity = p.stamp_capacity;
         if (p.epilogue == EPI_QKV_ROPE) {
             a.qkv.pos += b0;
             a.qkv.seq += b0;

@@ -71,6 +71,35 @@ __device__ __forceinline__ uint4 normalized_group(const float4 &v0, const float4
     return h;
 }
 
+// The same eight values kept in fp32.
+__device__ __forceinline__ void normalized_values(const float4 &v0, const float4 &v1, const float4 &g0, const float4 &g1, float inv, float (&c)[8]) {
+    c[0] = __fmul_rn(__fmul_rn(v0.x, inv), g0.x); c[1] = __fmul_rn(__fmul_rn(v0.y, inv), g0.y);
+    c[2] = __fmul_rn(__fmul_rn(v0.z, inv), g0.z); c[3] = __fmul_rn(__fmul_rn(v0.w, inv), g0.w);
+    c[4] = __fmul_rn(__fmul_rn(v1.x, inv), g1.x); c[5] = __fmul_rn(__fmul_rn(v1.y, inv), g1.y);
+    c[6] = __fmul_rn(__fmul_rn(v1.z, inv), g1.z); c[7] = __fmul_rn(__fmul_rn(v1.w, inv), g1.w);
+}
+
+// Split activations: an fp32 value v travels to the matrix cores as two fp16 numbers, hi = fp16(v) and
+// lo = fp16((v - hi) * 2048), and a product with it is hi * w + (lo * w) / 2048.  The residue is scaled by 2^11 so that it
+// stays a normal fp16 number wherever hi is one; v - hi is exact in fp32, so hi + lo / 2048 carries v to about 22 bits.
+// The reference's CPU path feeds fp32 activations into every matrix product (RealModelInferenceEngine.swift:6674-6697);
+// rounding them to fp16 costs 2^-12 relative per element and, over 32 layers of the 8B shape, 3e-2 on the logits.
+constexpr float kSplitScale = 2048.0f, kSplitUnscale = 1.0f / 2048.0f;
+struct SplitGroup { uint4 hi, lo; };
+__device__ __forceinline__ void split_pair(float a, float b, u32 &hi, u32 &lo) {
+    const _Float16 ha = (_Float16)a, hb = (_Float16)b;
+    hi = (u32)__builtin_bit_cast(uint16_t, ha) | ((u32)__builtin_bit_cast(uint16_t, hb) << 16);
+    lo = pack_half2(__fmul_rn(__fsub_rn(a, (float)ha), kSplitScale), __fmul_rn(__fsub_rn(b, (float)hb), kSplitScale));
+}
+__device__ __forceinline__ SplitGroup split_group(const float (&c)[8]) {
+    SplitGroup g;
+    split_pair(c[0], c[1], g.hi.x, g.lo.x);
+    split_pair(c[2], c[3], g.hi.y, g.lo.y);
+    split_pair(c[4], c[5], g.hi.z, g.lo.z);
+    split_pair(c[6], c[7], g.hi.w, g.lo.w);
+    return g;
+}
+
 // (x0,x1,x2,x3, x4,...) -> (x0,x2,x1,x3, x4,x6,x5,x7): the order the masked nibble / byte pairs meet
 __device__ __forceinline__ uint4 swap_middle(const uint4 &v) {
     uint4 p;
@@ -182,6 +211,21 @@ __device__ __forceinline__ void q4k_store_group_natural(const uint4 &v, int b, i
     float s = ((float)as_h2(v.x).x + (float)as_h2(v.x).y) + ((float)as_h2(v.y).x + (float)as_h2(v.y).y) +
               ((float)as_h2(v.z).x + (float)as_h2(v.z).y) + ((float)as_h2(v.w).x + (float)as_h2(v.w).y);
     if constexpr (Q40) s *= (g & 2) ? 72.0f : 1032.0f;
+    s += dpp_term<0xB1, 0xF>(s);
+    s += dpp_term<0x4E, 0xF>(s);
+    if ((threadIdx.x & 3) == 0) xsum[(size_t)b * (cols >> 5) + (g >> 2)] = s;
+}
+
+__device__ __forceinline__ float sum_group(const uint4 &v) {
+    return ((float)as_h2(v.x).x + (float)as_h2(v.x).y) + ((float)as_h2(v.y).x + (float)as_h2(v.y).y) +
+           ((float)as_h2(v.z).x + (float)as_h2(v.z).y) + ((float)as_h2(v.w).x + (float)as_h2(v.w).y);
+}
+// Split activations in the matrix-core layout: logical row b occupies rows 2b (hi) and 2b + 1 (lo) of [rows][cols / 8]; the sums
+// of each 32 are those of hi + lo / 2048, one per logical row.
+__device__ __forceinline__ void q4k_store_split_natural(const SplitGroup &v, int b, int g, int cols, uint4 *xs4, float *xsum) {
+    xs4[(size_t)(2 * b) * (cols >> 3) + g] = swap_middle(v.hi);
+    xs4[(size_t)(2 * b + 1) * (cols >> 3) + g] = swap_middle(v.lo);
+    float s = __builtin_fmaf(sum_group(v.lo), kSplitUnscale, sum_group(v.hi));
     s += dpp_term<0xB1, 0xF>(s);
     s += dpp_term<0x4E, 0xF>(s);
     if ((threadIdx.x & 3) == 0) xsum[(size_t)b * (cols >> 5) + (g >> 2)] = s;

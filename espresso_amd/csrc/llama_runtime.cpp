@@ -163,6 +163,7 @@ int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us
             break;
         case K_GATE_UP:
             g.w = L->w13; g.norm_x = hidden_; g.norm_w = L->rms_ffn; g.norm_eps = c_.norm_eps; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
+            g.split_out = split_activations_ && gemv_splits_activations(L->w2, 1);
             break;
         case K_DOWN: g.w = L->w2; g.x = act_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL; break;
         default:
@@ -173,6 +174,8 @@ int LlamaRuntime::time_kernel_class(int kernel_class, int iters, double *mean_us
             }
             break;
         }
+        // what the decode step launches: split activations wherever the GEMV takes them (not for fp16 rows given unsplit)
+        g.split_x = kernel_class != K_HEAD && !(g.x == ctx_ && kernel_class == K_WO) && split_activations_ && gemv_splits_activations(g.w, 1);
         return launch_gemv(g, s);
     };
     StepRows rows{};
@@ -418,6 +421,8 @@ int LlamaRuntime::finalize() {
         prompt_attention_ = attention_prompt_supported(c_.n_head, c_.n_kv_head, c_.head_dim) && !(pa && pa[0] == '0');
         const char *fh = getenv("ESPRESSO_HIP_FUSED_HEAD_ARGMAX");   // "0": the head stores logits and separate launches pick the token
         fused_head_argmax_ = !(fh && fh[0] == '0');
+        const char *sa = getenv("ESPRESSO_HIP_SPLIT_ACTIVATIONS");   // "0": activations rounded to fp16 once
+        if (sa && sa[0] == '0') split_activations_ = false;
     }
     finalized_ = true;
     return reset();
@@ -480,6 +485,8 @@ int LlamaRuntime::enqueue_trunk(int M, bool embedded, float *final_out) {
         // both RMSNorms of the layer run inside the staging of the GEMV that consumes them
         GemvParams g;
         g.w = L.wqkv; g.norm_x = hidden_; g.norm_w = L.rms_att; g.norm_eps = c_.norm_eps; g.batch = M;
+        // Activations reach the matrix cores as hi / lo fp16 pairs wherever the GEMV has that form (GemvParams::split_x)
+        g.split_x = split_activations_ && gemv_splits_activations(L.wqkv, M);
         const size_t cache_seq_stride = (size_t)kd * c_.max_seq;
         if (L.q_norm) {
             // per-head q/k norm needs whole heads before RoPE: plain GEMV, then the post kernel
@@ -518,16 +525,22 @@ int LlamaRuntime::enqueue_trunk(int M, bool embedded, float *final_out) {
         g = GemvParams{};
         g.batch = M;
         g.w = L.wo; g.x = ctx_; g.y = hidden_; g.residual = hidden_; g.epilogue = EPI_ADD_RESIDUAL;
-        if (merge_in_wo) { g.x = nullptr; g.merge_partials = attn_scratch_; g.merge_head_dim = c_.head_dim; }
+        if (merge_in_wo) {
+            g.x = nullptr; g.merge_partials = attn_scratch_; g.merge_head_dim = c_.head_dim;
+            g.split_x = split_activations_ && gemv_splits_activations(L.wo, M);   // the merge leaves fp32 values to split
+        }
         if ((rc = time_begin(K_WO)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
         g.w = L.w13; g.x = nullptr; g.merge_partials = nullptr; g.norm_x = hidden_; g.norm_w = L.rms_ffn; g.norm_eps = c_.norm_eps;
         g.y = nullptr; g.residual = nullptr; g.out_f16 = act_; g.epilogue = EPI_SWIGLU_F16;
+        const bool split_down = split_activations_ && gemv_splits_activations(L.w2, M);   // act_ then holds hi / lo row pairs
+        g.split_x = split_activations_ && gemv_splits_activations(L.w13, M);
+        g.split_out = split_down;
         if ((rc = time_begin(K_GATE_UP)) != ESP_OK) return rc;
         ESP_HIP_TRY(launch_gemv(g, s));
         if ((rc = time_end()) != ESP_OK) return rc;
-        g.w = L.w2; g.x = act_; g.norm_x = nullptr; g.norm_w = nullptr;
+        g.w = L.w2; g.x = act_; g.norm_x = nullptr; g.norm_w = nullptr; g.split_x = split_down; g.split_out = false;
         g.y = final_out && &L == &layers_.back() ? final_out : hidden_;   // the last layer's output may go straight to its keeper
         g.residual = hidden_; g.out_f16 = nullptr; g.epilogue = EPI_ADD_RESIDUAL;
         if ((rc = time_begin(K_DOWN)) != ESP_OK) return rc;
@@ -536,6 +549,14 @@ int LlamaRuntime::enqueue_trunk(int M, bool embedded, float *final_out) {
     }
     (void)ad;
     return ESP_OK;
+}
+
+void LlamaRuntime::set_split_activations(bool enabled) {
+    if (enabled == split_activations_) return;
+    split_activations_ = enabled;
+    for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }   // captured with the other kernels
+    for (auto &g : multi_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+    graph_epoch_++;
 }
 
 void LlamaRuntime::set_merged_attention(bool enabled) {
@@ -872,10 +893,14 @@ int LlamaRuntime::continue_greedy_until_stop(int seq, int steps, uint32_t *out_t
             if ((rc = eager_step(&stopped)) != ESP_OK) return rc;
         return ESP_OK;
     }
-    if (steps > 0 && !step_graphs_[seq]) {   // one eager step first: it configures every kernel's LDS limit outside the capture
+    if (steps > 0) {
+        // The first step always runs from the host.  A replay that finds the stop token re-embeds the row that sits in
+        // d_tokens_/d_pos_/d_seq_[0] and lets the trunk recompute it, which changes nothing only when that row is the one this
+        // sequence consumed last; after a prompt block or another sequence's pass those arrays hold something else.  advance()
+        // leaves exactly that row there (and the eager step configures every kernel's LDS limit outside a capture).
         if ((rc = eager_step(&stopped)) != ESP_OK) return rc;
         if (stopped) return ESP_OK;
-        if ((rc = capture_step_graph(seq)) != ESP_OK) return rc;
+        if (!step_graphs_[seq] && (rc = capture_step_graph(seq)) != ESP_OK) return rc;
     }
     if (*produced >= steps) return ESP_OK;
     const int first = *produced, want = steps - first;

@@ -85,6 +85,10 @@ class LlamaRuntime {
     // Decode steps of one or two rows: attention as one launch that leaves partial states, merged by the wo GEMV
     // (on by default where the shapes allow); off = the split kernel plus the merge kernel.
     void set_merged_attention(bool enabled);
+    // Decode steps of one or two rows feed every layer GEMV that has the form (matrix-core Q4_K) hi / lo fp16 pairs of the fp32
+    // activations instead of their fp16 roundings (default on; ESPRESSO_HIP_SPLIT_ACTIVATIONS=0 at creation switches it off).
+    void set_split_activations(bool enabled);
+    bool split_activations() const { return split_activations_; }
     bool merged_attention_in_use() const { return !layers_.empty() && wo_merges_attention(layers_[0], 1); }
     int read_last_hidden(int seq, float *out);
     int read_logits(int seq, float *out);         // runs the head on the kept hidden state
@@ -173,6 +177,7 @@ class LlamaRuntime {
     float *attn_scratch_ = nullptr;
     bool matrix_prefill_ = true;
     bool merged_attention_ = true;
+    bool split_activations_ = true;
     bool prompt_attention_ = false;   // prompt blocks run attention on the matrix cores
     float *gemm_workspace_ = nullptr;
 

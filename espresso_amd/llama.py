@@ -190,6 +190,10 @@ def set_merged_attention(rt: LlamaRuntime, enabled: bool) -> bool:
     return bool(r)
 
 
+def set_split_activations(rt: LlamaRuntime, enabled: bool) -> None:
+    _lib.check(rt._L.esp_llama_set_split_activations(rt._h, int(enabled)))
+
+
 def set_matrix_prefill(rt: LlamaRuntime, enabled: bool) -> None:
     _lib.check(rt._L.esp_llama_set_matrix_prefill(rt._h, int(enabled)))
 

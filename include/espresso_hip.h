@@ -217,6 +217,13 @@ int esp_llama_set_matrix_prefill(ESPLlamaRuntime *runtime, int enabled);
  * (head size 128, Q4_K wo of 2048 or 4096 columns).  enabled = 0 restores the split kernel plus the merge kernel
  * everywhere.  Returns 1 when the merged form is in use after the call, 0 when not, negative on error. */
 int esp_llama_set_merged_attention(ESPLlamaRuntime *runtime, int enabled);
+/* The reference's CPU path feeds fp32 activations into every matrix product (RealModelInferenceEngine.swift:6674-6697,
+ * :6221-6347).  The matrix cores take fp16, so decode steps of one or two rows hand every layer GEMV that has the form (Q4_K
+ * matrices of 4096 or 14336 columns) each activation as two fp16 numbers, hi = fp16(v) and lo = fp16((v - hi) * 2048), and
+ * add the two products: about 22 bits of the activation instead of 11, which is what keeps a 32-layer model's logits inside
+ * 2e-2 of the CPU path.  enabled = 0 rounds activations to fp16 once (faster by the cost of staging the second row).
+ * Default: enabled. */
+int esp_llama_set_split_activations(ESPLlamaRuntime *runtime, int enabled);
 
 /* ---- seeded synthetic weights ------------------------------------------------------------- *
  * Fills `out_blocks` (host memory, esp_format_bytes(format, elements) bytes) with N(0, std_dev) draws

@@ -672,7 +672,7 @@ int orc_llama_set_weight_blocks(orc_llama_runtime *rt, int layer, int slot, int 
 
 /* Switches the activation mode of an existing runtime (weights stay): 0 = the reference's default, fp32 activations
  * into every matrix product; 1 = rounded to fp16 first, as the GPU kernels take them. */
-void orc_llama_set_gemv_inputs_fp16(orc_llama_runtime *rt, int enabled) { rt->c.gemv_inputs_fp16 = enabled ? 1 : 0; }
+void orc_llama_set_gemv_inputs_fp16(orc_llama_runtime *rt, int enabled) { rt->c.gemv_inputs_fp16 = enabled; }
 
 /* :616-635 */
 void orc_llama_reset(orc_llama_runtime *rt) {
@@ -688,8 +688,12 @@ void orc_llama_reset(orc_llama_runtime *rt) {
 static void maybe_round(const orc_llama_config *c, float *v, int n) {
     if (c->round_intermediates_fp16) orc_round_f16_vector(v, (size_t)n);
 }
-static void gemv_input(const orc_llama_config *c, float *v, int n) {
-    if (c->gemv_inputs_fp16) orc_round_f16_vector(v, (size_t)n);
+/* gemv_inputs_fp16: 0 = the reference's default (fp32 activations into every matrix product); 1 = every product's input is
+ * rounded to fp16 first; any other value is a mask of the inputs that are rounded (2 attention norm, 4 attention context,
+ * 8 FFN norm, 16 SiLU(gate)*up, 32 final norm), for measuring what each rounding contributes. */
+enum { IN_ATT_NORM = 2, IN_CONTEXT = 4, IN_FFN_NORM = 8, IN_ACT = 16, IN_FINAL_NORM = 32 };
+static void gemv_input(const orc_llama_config *c, float *v, int n, int which) {
+    if (c->gemv_inputs_fp16 == 1 || (c->gemv_inputs_fp16 & which)) orc_round_f16_vector(v, (size_t)n);
 }
 
 /* forwardToken, :686-823 (identical body at :6221-6347). */
@@ -701,7 +705,7 @@ static int forward_token(orc_llama_runtime *rt, uint32_t token, int position) {
     for (int l = 0; l < c->n_layer; l++) {
         orc_layer *L = &rt->layers[l];
         orc_rmsnorm(rt->hidden, L->rms_att, c->norm_eps, d, rt->normed);
-        gemv_input(c, rt->normed, d);
+        gemv_input(c, rt->normed, d, IN_ATT_NORM);
         orc_matvec(L->wq, ad, d, rt->normed, rt->q); maybe_round(c, rt->q, ad);
         orc_matvec(L->wk, kd, d, rt->normed, rt->k); maybe_round(c, rt->k, kd);
         orc_matvec(L->wv, kd, d, rt->normed, rt->v); maybe_round(c, rt->v, kd);
@@ -716,16 +720,16 @@ static int forward_token(orc_llama_runtime *rt, uint32_t token, int position) {
         }
         orc_attention_decode(rt->q, rt->k_cache[l], rt->v_cache[l], c->n_head, c->n_kv_head, c->head_dim,
                              position + 1, S, rt->ctx);
-        gemv_input(c, rt->ctx, ad);
+        gemv_input(c, rt->ctx, ad, IN_CONTEXT);
         orc_matvec(L->wo, d, ad, rt->ctx, rt->proj);
         for (int i = 0; i < d; i++) rt->proj[i] = rt->hidden[i] + rt->proj[i];
         maybe_round(c, rt->proj, d);
         orc_rmsnorm(rt->proj, L->rms_ffn, c->norm_eps, d, rt->normed);
-        gemv_input(c, rt->normed, d);
+        gemv_input(c, rt->normed, d, IN_FFN_NORM);
         orc_matvec(L->w1, c->hidden_dim, d, rt->normed, rt->gate);
         orc_matvec(L->w3, c->hidden_dim, d, rt->normed, rt->up);
         for (int i = 0; i < c->hidden_dim; i++) rt->act[i] = orc_silu_tanh(rt->gate[i]) * rt->up[i];
-        gemv_input(c, rt->act, c->hidden_dim);
+        gemv_input(c, rt->act, c->hidden_dim, IN_ACT);
         orc_matvec(L->w2, d, c->hidden_dim, rt->act, rt->down);
         for (int i = 0; i < d; i++) rt->hidden[i] = rt->proj[i] + rt->down[i];
         maybe_round(c, rt->hidden, d);
@@ -757,7 +761,7 @@ int orc_llama_prefill(orc_llama_runtime *rt, const uint32_t *tokens, int count) 
 
 static void final_normed(orc_llama_runtime *rt) {
     orc_rmsnorm(rt->last_hidden, rt->final_norm, rt->c.norm_eps, rt->c.d_model, rt->normed);
-    gemv_input(&rt->c, rt->normed, rt->c.d_model);
+    gemv_input(&rt->c, rt->normed, rt->c.d_model, IN_FINAL_NORM);
 }
 
 /* :663-670 + :825-849; classifierArgmaxBlockSize = 4000 */

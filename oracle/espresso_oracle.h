@@ -98,7 +98,8 @@ typedef struct {
     int eos_token;                 /* -1 = none */
     /* rounding switches */
     int round_intermediates_fp16;  /* the reference's own flag (:289-301, :682-684) */
-    int gemv_inputs_fp16;          /* round every GEMV input vector to fp16 (what the GPU path does) */
+    int gemv_inputs_fp16;          /* 1: round every GEMV input vector to fp16 (what the GPU path did before it split them);
+                                      other non-zero values: a mask of the inputs that are rounded (see gemv_input) */
     int kv_fp16;                   /* round k (post-RoPE) and v to fp16 at cache write */
 } orc_llama_config;
 

@@ -314,10 +314,11 @@ class LlamaRuntime:
             raise ValueError(f"set_weight_blocks(layer={layer}, slot={slot}) failed: {rc}")
 
     def set_gemv_inputs_fp16(self, enabled: bool):
-        """Switch the activation mode in place (the weights stay loaded)."""
+        """Switch the activation mode in place (the weights stay loaded): False, True, or a mask of the inputs that are
+        rounded to fp16 (2 attention norm, 4 attention context, 8 FFN norm, 16 SiLU(gate)*up, 32 final norm)."""
         lib().orc_llama_set_gemv_inputs_fp16.argtypes = [C.c_void_p, C.c_int]
         lib().orc_llama_set_gemv_inputs_fp16(self._h, int(enabled))
-        self.cfg.gemv_inputs_fp16 = bool(enabled)
+        self.cfg.gemv_inputs_fp16 = enabled
 
     def reset(self):
         lib().orc_llama_reset(self._h)

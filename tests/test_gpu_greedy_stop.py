@@ -64,3 +64,35 @@ def test_stop_token_inside_graph_replay(llama, fmt):
             outs.append((rt.generate(prompt, budget)[0], rt.visible()))
             rt.close()
         assert outs[0] == outs[1] and outs[0][0] == plain[:min(budget, first + 1)]
+
+
+def test_stop_token_on_a_reused_runtime_after_a_prompt_block(llama):
+    """A runtime whose step graph already exists, given a prompt long enough for the block path (its row arrays then hold the
+    block's rows, not the sequence's last row), with the stop token as the first, second or a later generated token: same tokens
+    and same state (visible count, kept hidden row, logits, the tokens that follow) as the host-driven loop."""
+    fmt = orc.FMT_Q8_0
+    ocfg = orc.LlamaConfig(gemv_inputs_fp16=True, **BASE)
+    packed = mu.pack_weights(mu.random_weights(ocfg, 43, std=0.08), fmt)[0]
+    prompt = np.random.default_rng(3).integers(0, BASE["vocab"], 40).tolist()
+    free = build(llama, packed, fmt, -1)
+    plain = free.generate(prompt, 40)[0]
+    free.close()
+    for stop_at in (0, 1, 5):
+        eos = plain[stop_at]
+        first = plain.index(eos)
+        results = []
+        for graph in (True, False):
+            rt = build(llama, packed, fmt, eos)
+            llama.set_graph_replay(rt, graph)
+            rt.generate([9, 10, 11, 12], 6)          # builds the step graphs; leaves another row in the row arrays
+            rt.reset()
+            tokens, _ = rt.generate(prompt, 40)
+            state = (tokens, rt.visible(), rt.last_hidden().tobytes(), rt.logits().tobytes())
+            rt.advance(eos)
+            more = [rt.select_greedy()]
+            rt.advance(more[0]); more.append(rt.select_greedy())
+            results.append(state + (more,))
+            rt.close()
+        assert results[0] == results[1], stop_at
+        assert results[0][0] == plain[:first + 1]
+        assert results[0][1] == len(prompt) + first
