@@ -157,6 +157,45 @@ int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y
     return e == hipSuccess ? ESP_OK : fail_hip(e, "gemv");
 }
 
+int esp_matmul_f32(const ESPMatrix *matrix, const float *x, int rows, float *y, const float *residual) {
+    if (!matrix || !x || !y) return fail(ESP_ERR_INVALID_ARGUMENT, "matmul_f32: null pointer");
+    if (rows <= 0) return fail(ESP_ERR_INVALID_ARGUMENT, "matmul_f32: rows %d", rows);
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    const DeviceMatrix &m = matrix->m;
+    if (!gemm_split_supported(m)) return fail(ESP_ERR_UNSUPPORTED, "matmul_f32: Q4_K matrices with a multiple of 256 columns");
+    const size_t nx = (size_t)rows * m.cols, ny = (size_t)rows * m.rows;
+    float *d_x = nullptr, *d_y = nullptr, *d_res = nullptr, *d_ws = nullptr;
+    SplitRowsView v;
+    auto release = [&] {
+        void *ptrs[] = {d_x, d_y, d_res, d_ws, v.hi, v.lo, v.sums};
+        for (void *p : ptrs) if (p) (void)hipFree(p);
+    };
+    if ((rc = device_alloc(&d_x, nx)) != ESP_OK || (rc = device_alloc(&d_y, ny)) != ESP_OK || (rc = device_alloc(&v.hi, nx)) != ESP_OK ||
+        (rc = device_alloc(&v.lo, nx)) != ESP_OK || (rc = device_alloc(&v.sums, nx / 16)) != ESP_OK ||
+        (residual && (rc = device_alloc(&d_res, ny)) != ESP_OK) || (rc = device_alloc(&d_ws, kGemmWorkspaceFloats)) != ESP_OK) {
+        release();
+        return rc;
+    }
+    hipError_t e = hipMemcpyAsync(d_x, x, nx * 4, hipMemcpyHostToDevice, c.stream);
+    if (e == hipSuccess && residual) e = hipMemcpyAsync(d_res, residual, ny * 4, hipMemcpyHostToDevice, c.stream);
+    if (e == hipSuccess) {
+        SplitRowsParams sp;
+        sp.x = d_x; sp.rows = rows; sp.cols = m.cols; sp.out = v;
+        e = launch_split_rows(sp, c.stream);
+    }
+    if (e == hipSuccess) {
+        GemmSplitParams g;
+        g.w = m; g.x = v; g.y = d_y; g.residual = d_res; g.rows = rows; g.workspace = d_ws; g.workspace_floats = kGemmWorkspaceFloats;
+        e = launch_gemm_split(g, c.stream);
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(y, d_y, ny * 4, hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+    release();
+    return e == hipSuccess ? ESP_OK : fail_hip(e, "matmul_f32");
+}
+
 int esp_gemv_device_noalloc(const ESPMatrix *matrix, const uint16_t *x_f16_device, int batch, float *y_device,
                             const float *residual_device_or_null) {
     if (!matrix || !x_f16_device || !y_device) return fail(ESP_ERR_INVALID_ARGUMENT, "gemv_device_noalloc: null pointer");

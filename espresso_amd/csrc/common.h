@@ -128,6 +128,43 @@ struct GemmParams {
     int *deferred_splits = nullptr;
 };
 
+// Rows of activations split for the matrix cores: v = hi + lo / 2048 with hi = fp16(v), lo = fp16((v - hi) * 2048), both
+// [rows][cols] fp16, and per (row, super-block of 256 columns) sixteen fp16 `sums`: the sums S_j of the row over the eight
+// sub-blocks of 32 columns as fp16(S_j), j = 0..7, then fp16((S_j - fp16(S_j)) * 2048).
+struct SplitRowsView {
+    uint16_t *hi = nullptr, *lo = nullptr, *sums = nullptr;
+};
+
+// y[rows][w.rows] = x * dequant(w)^T (+ residual) for a Q4_K matrix with exact weights and split activations
+// (kernels/gemm_split.hip): prompt blocks of models whose logits must stay within 2e-2 of the fp32 CPU path over many layers.
+struct GemmSplitParams {
+    DeviceMatrix w;
+    SplitRowsView x;                  // read only
+    float *y = nullptr;               // fp32 out [rows][w.rows] (unused with `swiglu`)
+    const float *residual = nullptr;  // optional, may alias y
+    int rows = 0;
+    float *workspace = nullptr;       // split-K partial sums when the grid would not fill the chip (optional)
+    size_t workspace_floats = 0;
+    SplitRowsView swiglu;             // optional: silu(y[2i]) * y[2i + 1] as split rows [rows][w.rows / 2] instead of y
+    int *deferred_splits = nullptr;   // optional: leave split-K partial sums [splits][rows][w.rows] in workspace, report the count
+};
+bool gemm_split_supported(const DeviceMatrix &w);
+hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream);
+
+// fp32 rows -> split rows, optionally summing split-K partial planes (+ residual, sums also to y) and applying RMSNorm first.
+struct SplitRowsParams {
+    const float *x = nullptr;         // [splits][rows][cols], planes `plane` floats apart
+    int splits = 1;
+    size_t plane = 0;
+    const float *residual = nullptr;
+    float *y = nullptr;
+    const float *norm_w = nullptr;    // RMSNorm weights (cols <= 8192) or null
+    float norm_eps = 0.0f;
+    int rows = 0, cols = 0;           // cols % 256 == 0
+    SplitRowsView out;
+};
+hipError_t launch_split_rows(const SplitRowsParams &p, hipStream_t stream);
+
 // kernels/gemv.hip
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
 bool gemv_splits_activations(const DeviceMatrix &w, int batch);

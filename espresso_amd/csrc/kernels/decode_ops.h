@@ -49,6 +49,9 @@ struct AttentionArgs {
     float *split_scratch;
     // partial results of attention_partial_kernel: [rows][heads][attention_head_splits][head_dim + 4] floats
     float *head_partials;
+    // launch_attention_prompt only, all three or none: the context as split rows (hi = fp16(v), lo = fp16((v - hi) * 2048),
+    // sub-block sums; SplitRowsView) instead of ctx_f16, with the queries and the softmax weights split the same way
+    uint16_t *ctx_hi, *ctx_lo, *ctx_sums;
 };
 constexpr int kAttentionMaxSplits = 32;
 // Slices of the prefix the grouped-query attention kernel works on in parallel (fixed per runtime).

@@ -484,11 +484,13 @@ __global__ __launch_bounds__(HD) void attention_merge_kernel(AttentionArgs a, in
 //     the A operand is the value tile transposed in LDS (written once per workgroup, double-buffered: one barrier per tile),
 //     read so that k slot (lane / 32, i) is key 16 j + 8 (i / 4) + 4 (lane / 32) + i % 4, the key of accumulator 8 j + i.
 // Q, K, V and the probabilities enter the matrix cores as fp16, sums are fp32.
+// SPLIT: queries and probabilities go in as hi / lo pairs (v = hi + lo / 2048: two MFMAs each against the same keys / values, which
+// the fp16 cache holds exactly), and the context comes out as split rows for the GEMM that consumes it.
 typedef _Float16 attn_half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 attn_half4 __attribute__((ext_vector_type(4)));
 typedef float attn_floatx16 __attribute__((ext_vector_type(16)));
 
-template <int HD, int G, bool KV_F16>
+template <int HD, int G, bool KV_F16, bool SPLIT>
 __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs a, int rows) {
     constexpr int THREADS = G * 64, QT = 32, KS = HD / 16, MTILES = HD / 32, LDV = 32 + 8;   // LDV: fp16 per row of V^T
     constexpr int VP = 32 * (HD / 8) / THREADS;                                            // 8-dim pieces of V per thread
@@ -508,11 +510,19 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
         return attn_half8{(_Float16)x0.x, (_Float16)x0.y, (_Float16)x0.z, (_Float16)x0.w, (_Float16)x1.x, (_Float16)x1.y, (_Float16)x1.z, (_Float16)x1.w};
     };
     // query fragments: column = query `col` (rows beyond the block repeat its last row, never stored), dims 16 ks + 8 half ..
-    attn_half8 qf[KS];
+    attn_half8 qf[KS], ql[SPLIT ? KS : 1];
     {
         const float *qp = a.q + (size_t)(m0 + (col <= last_row ? col : last_row)) * a.n_head * HD + (size_t)head * HD + 8 * half;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) qf[ks] = to_half8(*reinterpret_cast<const float4 *>(qp + 16 * ks), *reinterpret_cast<const float4 *>(qp + 16 * ks + 4));
+        for (int ks = 0; ks < KS; ks++) {
+            const float4 x0 = *reinterpret_cast<const float4 *>(qp + 16 * ks), x1 = *reinterpret_cast<const float4 *>(qp + 16 * ks + 4);
+            qf[ks] = to_half8(x0, x1);
+            if constexpr (SPLIT) {
+                const float v[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) ql[ks][e] = (_Float16)__fmul_rn(__fsub_rn(v[e], (float)qf[ks][e]), 2048.0f);
+            }
+        }
     }
     // keys beyond t_max are clamped to it: in bounds, and masked below
     auto load_k = [&](int t0, attn_half8 (&kf)[KS]) {
@@ -551,11 +561,15 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
         }
     };
 
-    attn_floatx16 o[MTILES];
+    attn_floatx16 o[MTILES], ol[SPLIT ? MTILES : 1];
 #pragma unroll
     for (int mt = 0; mt < MTILES; mt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[mt][r] = 0.0f;
+#pragma unroll
+    for (int mt = 0; mt < (SPLIT ? MTILES : 1); mt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) ol[mt][r] = 0.0f;
     float mx = -INFINITY, l = 0.0f;
     const int qpos = pos0 + col;
 
@@ -576,6 +590,15 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
         for (int r = 0; r < 16; r++) sc[r] = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], sc, 0, 0, 0);
+        if constexpr (SPLIT) {
+            attn_floatx16 sl;
+#pragma unroll
+            for (int r = 0; r < 16; r++) sl[r] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) sl = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], ql[ks], sl, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; r++) sc[r] = __builtin_fmaf(sl[r], 1.0f / 2048.0f, sc[r]);
+        }
         // accumulator r: key t0 + 8 (r / 4) + 4 half + r % 4 against query `col`
         float tile_max = -INFINITY;
 #pragma unroll
@@ -588,27 +611,38 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
         const float m_new = fmaxf(mx, tile_max);    // finite from the first tile on: key 0 is visible to every query
         const float alpha = __expf(mx - m_new);      // exp(-inf) = 0 on the first tile
         float psum = 0.0f;
-        _Float16 ph[16];
+        _Float16 ph[16], pl[SPLIT ? 16 : 1];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const float pr = __expf(sc[r] - m_new);  // masked keys: exp(-inf) = 0
             psum += pr;
             ph[r] = (_Float16)pr;
+            if constexpr (SPLIT) pl[r] = (_Float16)__fmul_rn(__fsub_rn(pr, (float)ph[r]), 2048.0f);
         }
         l = __builtin_fmaf(l, alpha, psum);
         mx = m_new;
         const attn_half8 pf[2] = {attn_half8{ph[0], ph[1], ph[2], ph[3], ph[4], ph[5], ph[6], ph[7]},
                                   attn_half8{ph[8], ph[9], ph[10], ph[11], ph[12], ph[13], ph[14], ph[15]}};
+        attn_half8 pfl[2];
+        if constexpr (SPLIT) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) { pfl[0][e] = pl[e]; pfl[1][e] = pl[8 + e]; }
+        }
 #pragma unroll
         for (int mt = 0; mt < MTILES; mt++) {
 #pragma unroll
             for (int r = 0; r < 16; r++) o[mt][r] *= alpha;
+            if constexpr (SPLIT) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) ol[mt][r] *= alpha;
+            }
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const _Float16 *vrow = vt[buf] + (32 * mt + col) * LDV + 16 * j + 4 * half;
                 const attn_half4 lo = *reinterpret_cast<const attn_half4 *>(vrow), hi = *reinterpret_cast<const attn_half4 *>(vrow + 8);
                 const attn_half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[j], o[mt], 0, 0, 0);
+                if constexpr (SPLIT) ol[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pfl[j], ol[mt], 0, 0, 0);
             }
         }
         if (more) store_v(buf ^ 1, v1);
@@ -619,6 +653,42 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
         __syncthreads();
     }
     l += __shfl_xor(l, 32);
+    if constexpr (SPLIT) {
+        // context = (o + ol / 2048) / l as split rows; dims 32 mt .. 32 mt + 31 of a head are one sub-block of the row, half of it in
+        // this lane and half in lane ^ 32
+        const float inv = 1.0f / l;
+        const size_t row = (size_t)(m0 + (col <= last_row ? col : last_row));
+        const int ad = a.n_head * HD;
+#pragma unroll
+        for (int mt = 0; mt < MTILES; mt++) {
+            float s = 0.0f;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                attn_half4 vh, vl;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float v = __fmul_rn(__builtin_fmaf(ol[mt][4 * q4 + e], 1.0f / 2048.0f, o[mt][4 * q4 + e]), inv);
+                    vh[e] = (_Float16)v;
+                    vl[e] = (_Float16)__fmul_rn(__fsub_rn(v, (float)vh[e]), 2048.0f);
+                    s += __builtin_fmaf((float)vl[e], 1.0f / 2048.0f, (float)vh[e]);
+                }
+                if (col <= last_row) {
+                    const size_t o16 = row * ad + (size_t)head * HD + 32 * mt + 8 * q4 + 4 * half;
+                    *reinterpret_cast<attn_half4 *>(a.ctx_hi + o16) = vh;
+                    *reinterpret_cast<attn_half4 *>(a.ctx_lo + o16) = vl;
+                }
+            }
+            s += __shfl_xor(s, 32);
+            if (half == 0 && col <= last_row) {
+                const int sub = head * (HD / 32) + mt;
+                uint16_t *p = a.ctx_sums + (row * (size_t)(ad / 256) + (sub >> 3)) * 16 + (sub & 7);
+                const _Float16 h = (_Float16)s;
+                p[0] = __builtin_bit_cast(uint16_t, h);
+                p[8] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(__fsub_rn(s, (float)h), 2048.0f));
+            }
+        }
+        return;
+    }
     if (col <= last_row) {
         const float inv = 1.0f / l;
         uint16_t *out = a.ctx_f16 + (size_t)(m0 + col) * a.n_head * HD + (size_t)head * HD;
@@ -1257,8 +1327,13 @@ bool attention_prompt_supported(int n_head, int n_kv_head, int head_dim) {
 template <int HD, int G>
 hipError_t launch_attention_prompt_shape(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
     dim3 grid(a.n_kv_head, (rows + 31) / 32);
-    if (kv_f16) hipLaunchKernelGGL((attention_prompt_kernel<HD, G, true>), grid, dim3(G * 64), 0, s, a, rows);
-    else hipLaunchKernelGGL((attention_prompt_kernel<HD, G, false>), grid, dim3(G * 64), 0, s, a, rows);
+    if (a.ctx_hi) {   // split rows out: fp16 caches only (they hold keys and values exactly)
+        if (!kv_f16 || !a.ctx_lo || !a.ctx_sums || (a.n_head * HD) % 256 != 0) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((attention_prompt_kernel<HD, G, true, true>), grid, dim3(G * 64), 0, s, a, rows);
+        return hipGetLastError();
+    }
+    if (kv_f16) hipLaunchKernelGGL((attention_prompt_kernel<HD, G, true, false>), grid, dim3(G * 64), 0, s, a, rows);
+    else hipLaunchKernelGGL((attention_prompt_kernel<HD, G, false, false>), grid, dim3(G * 64), 0, s, a, rows);
     return hipGetLastError();
 }
 

@@ -1,0 +1,519 @@
+// Q4_K prompt-block GEMM with exact weights and split activations:
+//     y[m][n] = sum_k x[m][k] * dequant(W)[n][k]
+// to about 22 bits of x and every bit of W, on the fp16 matrix cores with fp32 accumulation.
+//
+// The reference walks a prompt token by token with fp32 activations and fp32 dequantised weights
+// (RealModelInferenceEngine.swift:6674-6697 inside :6365-6375).  Rounding either operand to fp16 costs 2^-12
+// relative per product, which 32 layers of the 8B shape amplify to 3-4e-2 on the logits; this kernel keeps both.
+//
+//   * Weights.  A Q4_K weight is d * (sc_j * q) - dmin * m_j with a 4-bit q, 6-bit sc_j and m_j per sub-block of 32
+//     and fp16 d, dmin per super-block of 256 and row.  sc_j * q <= 945 is an integer, exact in fp16: THAT is the B operand.
+//     The sums over a super-block are then scaled by d in fp32 (one multiply-add per accumulator and super-block), and the
+//     minimum term is dmin * sum_j m_j * S_j with S_j the activations' sum over sub-block j: one more MFMA per super-block
+//     whose K is (8 x hi of S_j, 8 x lo of S_j scaled by 2048) against (m_0..m_7, m_0..m_7 / 2048).
+//   * Activations.  v = hi + lo / 2048 with hi = fp16(v), lo = fp16((v - hi) * 2048) (SplitRowsView): two A operands against
+//     the same B operand, two accumulator sets, joined in the per-super-block fold.
+//
+// Shape: a workgroup of four wavefronts (2 x 2) owns 128 activation rows x 128 weight rows, every wavefront 2 x 2 tiles of
+// v_mfma_f32_32x32x16_f16; K walks in tiles of 64 (a pair of sub-blocks) through double-buffered LDS, one barrier per tile,
+// with the packed weights and activations of the next tiles in flight in registers.  Two threads per weight row turn its 32
+// bytes of nibbles into 64 fp16 integers per tile (one v_and_or_b32 and one packed fp16 multiply-add per two weights).
+// Per 256 k a wavefront issues 128 + 4 MFMAs and about 200 fold operations.
+#include "../common.h"
+#include "decode_ops.h"
+#include <atomic>
+
+namespace esp {
+namespace {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32;
+
+constexpr int kThreads = 256;
+constexpr int KT = 64;          // k per tile
+constexpr int LDK = KT + 8;     // fp16 per LDS row
+constexpr int NT = 128, MT = 128;
+constexpr float kUnscale = 1.0f / 2048.0f, kScale = 2048.0f;
+
+struct SplitGemmArgs {
+    const uint8_t *qs;
+    size_t qs_row_bytes;
+    int N, K, M;
+    const uint16_t *xh, *xl, *xs;   // [M][K], [M][K], [M][K / 256][16]
+    float *y;
+    const float *residual;
+    float *partial;                 // [splits][M][N] when gridDim.y > 1
+    int tiles_per_split;            // a multiple of four
+    uint16_t *sw_hi, *sw_lo;        // SiLU(gate) * up as a split pair [M][N / 2] instead of y (no split-K)
+};
+
+__device__ __forceinline__ h2 as_h2(u32 v) { return __builtin_bit_cast(h2, v); }
+__device__ __forceinline__ u32 as_u32(h2 v) { return __builtin_bit_cast(u32, v); }
+__device__ __forceinline__ float half_bits_to_float(u32 bits16) { return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16); }
+__device__ __forceinline__ u32 dword_of(const uint4 &v, int k) { return k == 0 ? v.x : k == 1 ? v.y : k == 2 ? v.z : v.w; }
+__device__ __forceinline__ uint4 swap_middle(const uint4 &v) {
+    uint4 p;
+    p.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
+    p.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
+    p.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
+    p.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
+    return p;
+}
+__device__ __forceinline__ u32 scale_byte(const uint4 &hdr, int idx) {
+    const u32 word = idx < 4 ? hdr.y : idx < 8 ? hdr.z : hdr.w;
+    return (word >> ((idx & 3) * 8)) & 0xFFu;
+}
+// ggml's get_scale_min_k4, as integers
+__device__ __forceinline__ void q4k_scale_min(const uint4 &hdr, int j, u32 &sc, u32 &m) {
+    if (j < 4) {
+        sc = scale_byte(hdr, j) & 63u;
+        m = scale_byte(hdr, j + 4) & 63u;
+    } else {
+        sc = (scale_byte(hdr, j + 4) & 0xFu) | ((scale_byte(hdr, j - 4) >> 6) << 4);
+        m = (scale_byte(hdr, j + 4) >> 4) | ((scale_byte(hdr, j) >> 6) << 4);
+    }
+}
+__device__ __forceinline__ u32 pack_half2(float lo, float hi) {
+    return (u32)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((u32)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+}
+
+struct RawTile { uint4 q, hdr; };   // sixteen bytes of nibbles of (weight row, tile, half) and the super-block's header
+
+// dynamic LDS: [2] weight tiles, [2] hi tiles, [2] lo tiles, [2] minimum rows, [2] sub-block sums, [2] (d, dmin)
+constexpr size_t kTileHalfs = (size_t)128 * LDK;
+constexpr size_t kLdsBytes = 6 * kTileHalfs * 2 + 2 * 128 * 16 * 2 + 2 * 128 * 16 * 2 + 2 * 128 * 8;
+
+template <int DEPTH>
+__global__ __launch_bounds__(kThreads) void gemm_q4k_split_kernel(SplitGemmArgs a) {
+    constexpr int XV = MT * KT / 8 / kThreads;   // 128-bit pieces of a tile of one activation plane per thread (4)
+    extern __shared__ uint4 smem_raw[];
+    _Float16 *wt = reinterpret_cast<_Float16 *>(smem_raw);     // [2][128 * LDK]   sc * q, (0,2,1,3) order inside fours
+    _Float16 *xh = wt + 2 * kTileHalfs;                          // [2][128 * LDK]
+    _Float16 *xl = xh + 2 * kTileHalfs;                          // [2][128 * LDK]
+    _Float16 *ms = xl + 2 * kTileHalfs;                          // [2][128][16]     m_0..m_7, then m_0..m_7 / 2048, of the weight row's super-block
+    _Float16 *xs = ms + 2 * 128 * 16;                            // [2][128][16]     (hi of S_0..S_7, lo of S_0..S_7) of the row
+    float2 *dd = reinterpret_cast<float2 *>(xs + 2 * 128 * 16);  // [2][128]         (d, dmin)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int n0 = blockIdx.x * NT, m0 = blockIdx.z * MT;
+    const int tiles = a.K / KT;
+    const int t_begin = blockIdx.y * a.tiles_per_split;
+    const int t_end = t_begin + a.tiles_per_split < tiles ? t_begin + a.tiles_per_split : tiles;
+    const int t_last = t_end - 1;
+
+    const int wr = tid >> 1, wh = tid & 1;                       // dequantisation role: weight row, half of the tile
+    const int w_row = n0 + wr < a.N ? n0 + wr : a.N - 1;         // clamped, the result is never stored
+    const uint8_t *w_base = a.qs + (size_t)w_row * a.qs_row_bytes;
+    const int xs_row = m0 + (tid >> 1) < a.M ? m0 + (tid >> 1) : a.M - 1;
+    const int sbs = a.K / 256;
+
+    floatx16 tot[2][2], ah[2][2], al[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) tot[i][j][r] = ah[i][j][r] = al[i][j][r] = 0.0f;
+
+    auto fetch_w = [&](int tile) {
+        RawTile r;
+        const uint8_t *blk = w_base + (size_t)(tile >> 2) * 144;
+        r.hdr = *reinterpret_cast<const uint4 *>(blk);
+        r.q = *reinterpret_cast<const uint4 *>(blk + 16 + (tile & 3) * 32 + wh * 16);
+        return r;
+    };
+    auto fetch_x = [&](int tile, uint4 (&vh)[XV], uint4 (&vl)[XV]) {
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const int piece = tid + i * kThreads, row = piece >> 3, part = piece & 7;
+            const int m = m0 + row < a.M ? m0 + row : a.M - 1;   // rows beyond M repeat the last one; never stored
+            const size_t o = (size_t)m * a.K + (size_t)tile * KT;
+            vh[i] = reinterpret_cast<const uint4 *>(a.xh + o)[part];
+            vl[i] = reinterpret_cast<const uint4 *>(a.xl + o)[part];
+        }
+    };
+    auto fetch_sums = [&](int sb) {
+        return reinterpret_cast<const uint4 *>(a.xs + ((size_t)xs_row * sbs + (sb < sbs ? sb : sbs - 1)) * 16)[tid & 1];
+    };
+
+    RawTile raw[DEPTH];
+    uint4 vh[DEPTH][XV], vl[DEPTH][XV];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+        const int tile = t_begin + d < t_last ? t_begin + d : t_last;
+        raw[d] = fetch_w(tile);
+        fetch_x(tile, vh[d], vl[d]);
+    }
+    uint4 sums_next = fetch_sums(t_begin >> 2);
+    static_assert(4 % DEPTH == 0, "the main loop is unrolled by four");
+
+    // Stages tile `tile` (slot S of the registers in flight, c = tile % 4 a constant) into LDS buffer `buf`, and with the first tile
+    // of a super-block that super-block's minimums, scales and activation sums into buffer (tile / 4) % 2.
+    auto stage = [&](int S, int c, int tile, int buf) {
+        const RawTile &r = raw[S];
+        u32 sc_lo, m_lo, sc_hi, m_hi;
+        q4k_scale_min(r.hdr, 2 * c, sc_lo, m_lo);
+        q4k_scale_min(r.hdr, 2 * c + 1, sc_hi, m_hi);
+        // low nibbles under 0x6400 read 1024 + q, high nibbles under 0x5400 read 64 + q; (offset + q) * sc - offset * sc is one
+        // exact packed multiply-add: the result sc * q <= 945 is an integer
+        const _Float16 fl = (_Float16)(float)sc_lo, fh = (_Float16)(float)sc_hi;
+        const h2 s_lo = {fl, fl}, s_hi = {fh, fh};
+        const _Float16 ol = (_Float16)(-1024.0f * (float)sc_lo), oh = (_Float16)(-64.0f * (float)sc_hi);
+        const h2 o_lo = {ol, ol}, o_hi = {oh, oh};
+        u32 lo[8], hi[8];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const u32 w = dword_of(r.q, k), w8 = w >> 8;
+            lo[2 * k] = as_u32(__builtin_elementwise_fma(as_h2((w & 0x000F000Fu) | 0x64006400u), s_lo, o_lo));
+            lo[2 * k + 1] = as_u32(__builtin_elementwise_fma(as_h2((w8 & 0x000F000Fu) | 0x64006400u), s_lo, o_lo));
+            hi[2 * k] = as_u32(__builtin_elementwise_fma(as_h2((w & 0x00F000F0u) | 0x54005400u), s_hi, o_hi));
+            hi[2 * k + 1] = as_u32(__builtin_elementwise_fma(as_h2((w8 & 0x00F000F0u) | 0x54005400u), s_hi, o_hi));
+        }
+        _Float16 *wrow = wt + (size_t)buf * kTileHalfs + wr * LDK;
+        uint4 *plo = reinterpret_cast<uint4 *>(wrow + 16 * wh), *phi = reinterpret_cast<uint4 *>(wrow + 32 + 16 * wh);
+        plo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        plo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+        phi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        phi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const int piece = tid + i * kThreads, row = piece >> 3, part = piece & 7;
+            *reinterpret_cast<uint4 *>(xh + (size_t)buf * kTileHalfs + row * LDK + part * 8) = swap_middle(vh[S][i]);
+            *reinterpret_cast<uint4 *>(xl + (size_t)buf * kTileHalfs + row * LDK + part * 8) = swap_middle(vl[S][i]);
+        }
+        if (c == 0) {
+            const int sbuf = (tile >> 2) & 1;
+            u32 mm[4];
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) { u32 s_unused; q4k_scale_min(r.hdr, 4 * wh + jj, s_unused, mm[jj]); }
+            _Float16 *mrow = ms + (size_t)sbuf * 128 * 16 + wr * 16 + 4 * wh;
+            *reinterpret_cast<uint2 *>(mrow) = make_uint2(pack_half2((float)mm[0], (float)mm[1]), pack_half2((float)mm[2], (float)mm[3]));
+            *reinterpret_cast<uint2 *>(mrow + 8) = make_uint2(pack_half2((float)mm[0] * kUnscale, (float)mm[1] * kUnscale),
+                                                              pack_half2((float)mm[2] * kUnscale, (float)mm[3] * kUnscale));
+            if (wh == 0) dd[sbuf * 128 + wr] = make_float2(half_bits_to_float(r.hdr.x & 0xFFFFu), half_bits_to_float(r.hdr.x >> 16));
+            *reinterpret_cast<uint4 *>(xs + (size_t)sbuf * 128 * 16 + (tid >> 1) * 16 + 8 * (tid & 1)) = sums_next;
+            sums_next = fetch_sums((tile >> 2) + 1);
+        }
+        const int ahead = tile + DEPTH < t_last ? tile + DEPTH : t_last;
+        raw[S] = fetch_w(ahead);
+        fetch_x(ahead, vh[S], vl[S]);
+    };
+
+    stage(0, 0, t_begin, 0);   // t_begin is a multiple of four
+    __syncthreads();
+    for (int t0 = t_begin; t0 < t_end; t0 += 4) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int t = t0 + u, buf = u & 1;
+            const _Float16 *xhb = xh + (size_t)buf * kTileHalfs, *xlb = xl + (size_t)buf * kTileHalfs, *wtb = wt + (size_t)buf * kTileHalfs;
+#pragma unroll
+            for (int ks = 0; ks < KT / 16; ks++) {
+                const int kk = ks * 16 + 8 * (lane >> 5);
+                half8 fh[2], fl[2], fb[2];
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    fh[i] = *reinterpret_cast<const half8 *>(xhb + ((wm * 2 + i) * 32 + (lane & 31)) * LDK + kk);
+                    fl[i] = *reinterpret_cast<const half8 *>(xlb + ((wm * 2 + i) * 32 + (lane & 31)) * LDK + kk);
+                }
+#pragma unroll
+                for (int j = 0; j < 2; j++) fb[j] = *reinterpret_cast<const half8 *>(wtb + ((wn * 2 + j) * 32 + (lane & 31)) * LDK + kk);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        ah[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh[i], fb[j], ah[i][j], 0, 0, 0);
+                        al[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl[i], fb[j], al[i][j], 0, 0, 0);
+                    }
+            }
+            if (u == 3) {
+                // the super-block is complete: total += d * (hi sums + lo sums / 2048) - dmin * sum_j m_j S_j
+                const int sbuf = (t >> 2) & 1;
+                half8 fs[2], fm[2];
+                float2 dv[2];
+#pragma unroll
+                for (int i = 0; i < 2; i++) fs[i] = *reinterpret_cast<const half8 *>(xs + (size_t)sbuf * 128 * 16 + ((wm * 2 + i) * 32 + (lane & 31)) * 16 + 8 * (lane >> 5));
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    fm[j] = *reinterpret_cast<const half8 *>(ms + (size_t)sbuf * 128 * 16 + ((wn * 2 + j) * 32 + (lane & 31)) * 16 + 8 * (lane >> 5));
+                    dv[j] = dd[sbuf * 128 + (wn * 2 + j) * 32 + (lane & 31)];
+                }
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        floatx16 am;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) am[r] = 0.0f;
+                        am = __builtin_amdgcn_mfma_f32_32x32x16_f16(fs[i], fm[j], am, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const float main = __builtin_fmaf(al[i][j][r], kUnscale, ah[i][j][r]);
+                            tot[i][j][r] = __builtin_fmaf(-dv[j].y, am[r], __builtin_fmaf(dv[j].x, main, tot[i][j][r]));
+                            ah[i][j][r] = 0.0f;
+                            al[i][j][r] = 0.0f;
+                        }
+                    }
+            }
+            stage((u + 1) % DEPTH, (u + 1) & 3, t + 1, buf ^ 1);   // past the end: the slot holds a clamped fetch; staged into the idle buffers, never read
+            __syncthreads();
+        }
+    }
+
+    // accumulator r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of the 32 x 32 tile
+    if (a.sw_hi) {   // rows of W are (gate, up) pairs: even lanes hold gate, their right neighbours up (:6825-6827, :6337)
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int n = n0 + (wn * 2 + j) * 32 + (lane & 31);
+                const bool odd = lane & 1;
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    const float a0 = tot[i][j][2 * k], a1 = tot[i][j][2 * k + 1];
+                    const float p0 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a0), 0xB1, 0xF, 0xF, false));
+                    const float p1 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a1), 0xB1, 0xF, 0xF, false));
+                    const float g = odd ? p1 : a0, up = odd ? a1 : p0;
+                    const int r = 2 * k + (odd ? 1 : 0);
+                    const int m = m0 + (wm * 2 + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (m < a.M && (n | 1) < a.N) {
+                        const float hg = __fmul_rn(0.5f, g);
+                        const float silu = __fmul_rn(hg, __fadd_rn(1.0f, tanhf(hg)));
+                        const float act = __fmul_rn(silu, up);
+                        const _Float16 hi = (_Float16)act;
+                        const size_t o = (size_t)m * (a.N / 2) + n / 2;
+                        a.sw_hi[o] = __builtin_bit_cast(uint16_t, hi);
+                        a.sw_lo[o] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(__fsub_rn(act, (float)hi), kScale));
+                    }
+                }
+            }
+        return;
+    }
+    const bool split = gridDim.y > 1;
+    float *out = split ? a.partial + (size_t)blockIdx.y * a.M * a.N : a.y;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int n = n0 + (wn * 2 + j) * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + (wm * 2 + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < a.M && n < a.N) {
+                    const size_t o = (size_t)m * a.N + n;
+                    out[o] = (!split && a.residual) ? a.residual[o] + tot[i][j][r] : tot[i][j][r];
+                }
+            }
+        }
+}
+
+// y = (residual +) sum over splits of partial, in split order
+__global__ void split_gemm_reduce_kernel(const float *partial, int splits, size_t count, const float *residual, float *y) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float s = partial[i];
+    for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + i];
+    y[i] = residual ? residual[i] + s : s;
+}
+
+// ---- producers of split rows -------------------------------------------------------------------------------------------------
+// Eight fp32 values -> hi and lo groups; returns their sum (of hi + lo / 2048)
+__device__ __forceinline__ float split_eight(const float (&c)[8], uint4 &hi, uint4 &lo) {
+    u32 h[4], l[4];
+    float s = 0.0f;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const _Float16 ha = (_Float16)c[2 * p], hb = (_Float16)c[2 * p + 1];
+        const _Float16 la = (_Float16)__fmul_rn(__fsub_rn(c[2 * p], (float)ha), kScale), lb = (_Float16)__fmul_rn(__fsub_rn(c[2 * p + 1], (float)hb), kScale);
+        h[p] = (u32)__builtin_bit_cast(uint16_t, ha) | ((u32)__builtin_bit_cast(uint16_t, hb) << 16);
+        l[p] = (u32)__builtin_bit_cast(uint16_t, la) | ((u32)__builtin_bit_cast(uint16_t, lb) << 16);
+        s += __builtin_fmaf((float)la, kUnscale, (float)ha) + __builtin_fmaf((float)lb, kUnscale, (float)hb);
+    }
+    hi = make_uint4(h[0], h[1], h[2], h[3]);
+    lo = make_uint4(l[0], l[1], l[2], l[3]);
+    return s;
+}
+// The sum S of a sub-block (held by the first of each four lanes after the quad reduction) as the pair the GEMM's extra MFMA reads:
+// sums[(row, super-block)][j] = fp16(S), [8 + j] = fp16((S - fp16(S)) * 2048).
+__device__ __forceinline__ void store_subblock_sum(uint16_t *sums, size_t row, int cols, int group, float s) {
+    s += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0xB1, 0xF, 0xF, false));
+    s += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0x4E, 0xF, 0xF, false));
+    if ((group & 3) == 0) {
+        const int sub = group >> 2;   // sub-block of 32 columns
+        uint16_t *p = sums + (row * (size_t)(cols / 256) + (sub >> 3)) * 16 + (sub & 7);
+        const _Float16 h = (_Float16)s;
+        p[0] = __builtin_bit_cast(uint16_t, h);
+        p[8] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(__fsub_rn(s, (float)h), kScale));
+    }
+}
+
+// rows of fp32 values -> split rows; optional RMSNorm ((x * inv) * w, RealModelInferenceEngine.swift:6724-6743) and optional sum of
+// split-K partial planes (+ residual) first, in which case the sums are also written to y.  One workgroup of 256 threads per row;
+// cols % 256 == 0 and cols <= 8192 with the norm (the row is held in registers), any multiple of 256 without.
+struct SplitRowsArgs {
+    const float *x;          // [splits][rows][cols]
+    int splits;
+    size_t plane;
+    const float *residual;   // optional
+    float *y;                // optional: the summed rows
+    const float *norm_w;     // optional
+    float eps;
+    int cols;
+    uint16_t *hi, *lo, *sums;
+};
+template <bool NORM>
+__global__ __launch_bounds__(256) void split_rows_kernel(SplitRowsArgs a) {
+    __shared__ float red[4];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const int groups = a.cols / 8;   // groups of eight columns; consecutive threads take consecutive groups
+    constexpr int KV = NORM ? 4 : 1; // groups per thread held in registers with the norm
+    const size_t row = (size_t)m * a.cols;
+    auto load_group = [&](int g, float (&c)[8]) {
+        const float4 *p = reinterpret_cast<const float4 *>(a.x + row + (size_t)g * 8);
+        float4 v0 = p[0], v1 = p[1];
+        for (int sp = 1; sp < a.splits; sp++) {
+            const float4 *q = reinterpret_cast<const float4 *>(a.x + (size_t)sp * a.plane + row + (size_t)g * 8);
+            const float4 t0 = q[0], t1 = q[1];
+            v0.x += t0.x; v0.y += t0.y; v0.z += t0.z; v0.w += t0.w; v1.x += t1.x; v1.y += t1.y; v1.z += t1.z; v1.w += t1.w;
+        }
+        if (a.residual) {
+            const float4 *q = reinterpret_cast<const float4 *>(a.residual + row + (size_t)g * 8);
+            const float4 t0 = q[0], t1 = q[1];
+            v0.x = t0.x + v0.x; v0.y = t0.y + v0.y; v0.z = t0.z + v0.z; v0.w = t0.w + v0.w;
+            v1.x = t1.x + v1.x; v1.y = t1.y + v1.y; v1.z = t1.z + v1.z; v1.w = t1.w + v1.w;
+        }
+        if (a.y) {
+            float4 *o = reinterpret_cast<float4 *>(a.y + row + (size_t)g * 8);
+            o[0] = v0; o[1] = v1;
+        }
+        c[0] = v0.x; c[1] = v0.y; c[2] = v0.z; c[3] = v0.w; c[4] = v1.x; c[5] = v1.y; c[6] = v1.z; c[7] = v1.w;
+    };
+    auto emit = [&](int g, const float (&c)[8]) {
+        uint4 hi, lo;
+        const float s = split_eight(c, hi, lo);
+        reinterpret_cast<uint4 *>(a.hi + row)[g] = hi;
+        reinterpret_cast<uint4 *>(a.lo + row)[g] = lo;
+        store_subblock_sum(a.sums, (size_t)m, a.cols, g, s);
+    };
+    if constexpr (NORM) {
+        float c[KV][8];
+        float ss = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KV; k++) {
+            const int g = tid + k * 256;
+            if (g < groups) load_group(g, c[k]);
+            else
+#pragma unroll
+                for (int e = 0; e < 8; e++) c[k][e] = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) ss += c[k][e] * c[k][e];
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off);
+        if ((tid & 63) == 0) red[tid >> 6] = ss;
+        __syncthreads();
+        const float inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)a.cols + a.eps);
+#pragma unroll
+        for (int k = 0; k < KV; k++) {
+            const int g = tid + k * 256;   // whole quads of threads are in or out together: groups is a multiple of four
+            if (g < groups) {
+                const float4 *wp = reinterpret_cast<const float4 *>(a.norm_w + (size_t)g * 8);
+                const float4 w0 = wp[0], w1 = wp[1];
+                const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+                float n[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) n[e] = __fmul_rn(__fmul_rn(c[k][e], inv), w[e]);
+                emit(g, n);
+            }
+        }
+    } else {
+        for (int g = tid; g < groups; g += 256) {
+            float c[8];
+            load_group(g, c);
+            emit(g, c);
+        }
+    }
+}
+
+// sums of rows that exist as hi / lo planes already (the SiLU(gate) * up epilogue writes those)
+__global__ __launch_bounds__(256) void split_sums_kernel(const uint16_t *hi, const uint16_t *lo, int cols, uint16_t *sums) {
+    const int m = blockIdx.x;
+    const size_t row = (size_t)m * cols;
+    for (int g = threadIdx.x; g < cols / 8; g += 256) {
+        const uint4 h = reinterpret_cast<const uint4 *>(hi + row)[g], l = reinterpret_cast<const uint4 *>(lo + row)[g];
+        float s = 0.0f;
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const h2 hp = as_h2(dword_of(h, p)), lp = as_h2(dword_of(l, p));
+            s += __builtin_fmaf((float)lp.x, kUnscale, (float)hp.x) + __builtin_fmaf((float)lp.y, kUnscale, (float)hp.y);
+        }
+        store_subblock_sum(sums, (size_t)m, cols, g, s);
+    }
+}
+
+}  // namespace
+
+bool gemm_split_supported(const DeviceMatrix &w) { return w.format == FMT_Q4_K && w.qs && w.cols % 256 == 0 && w.qs_row_bytes % 16 == 0; }
+
+hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream) {
+    const DeviceMatrix &w = p.w;
+    if (!gemm_split_supported(w) || !p.x.hi || !p.x.lo || !p.x.sums || p.rows <= 0 || w.rows <= 0) return hipErrorInvalidValue;
+    const bool swiglu = p.swiglu.hi != nullptr;
+    if (swiglu ? (!p.swiglu.lo || w.rows % 2 != 0 || p.residual) : !p.y) return hipErrorInvalidValue;
+    SplitGemmArgs a{};
+    a.qs = w.qs; a.qs_row_bytes = w.qs_row_bytes; a.N = w.rows; a.K = w.cols; a.M = p.rows;
+    a.xh = p.x.hi; a.xl = p.x.lo; a.xs = p.x.sums; a.y = p.y; a.residual = p.residual; a.partial = p.workspace;
+    const int tiles = a.K / KT, blocks = ((a.N + NT - 1) / NT) * ((a.M + MT - 1) / MT);
+    // split K until the grid fills the chip (one workgroup per compute unit is resident), whole super-blocks per split
+    int splits = 1;
+    if (!swiglu && p.workspace) {
+        const int target = 256;
+        splits = blocks >= target ? 1 : (target + blocks - 1) / blocks;
+        if (splits > tiles / 16) splits = tiles / 16;
+        if (splits < 1) splits = 1;
+        while (splits > 1 && (size_t)splits * a.M * a.N > p.workspace_floats) splits--;
+    }
+    a.tiles_per_split = ((tiles + splits - 1) / splits + 3) & ~3;
+    splits = (tiles + a.tiles_per_split - 1) / a.tiles_per_split;
+    if (swiglu) { a.sw_hi = p.swiglu.hi; a.sw_lo = p.swiglu.lo; }
+    static std::atomic<uint64_t> raised{0};
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (device & 63);
+    auto kernel = gemm_q4k_split_kernel<2>;
+    if (!(raised.load(std::memory_order_acquire) & bit)) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+        if (e != hipSuccess) return e;
+        raised.fetch_or(bit, std::memory_order_release);
+    }
+    dim3 grid((a.N + NT - 1) / NT, splits, (a.M + MT - 1) / MT);
+    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kLdsBytes, stream, a);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (swiglu) {
+        hipLaunchKernelGGL(split_sums_kernel, dim3(a.M), dim3(256), 0, stream, p.swiglu.hi, p.swiglu.lo, a.N / 2, p.swiglu.sums);
+        return hipGetLastError();
+    }
+    if (splits > 1) {
+        if (p.deferred_splits) { *p.deferred_splits = splits; return hipSuccess; }
+        const size_t count = (size_t)a.M * a.N;
+        hipLaunchKernelGGL(split_gemm_reduce_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, a.partial, splits, count, a.residual, a.y);
+        return hipGetLastError();
+    }
+    if (p.deferred_splits) *p.deferred_splits = 1;
+    return hipSuccess;
+}
+
+hipError_t launch_split_rows(const SplitRowsParams &p, hipStream_t stream) {
+    if (!p.x || !p.out.hi || !p.out.lo || !p.out.sums || p.rows <= 0 || p.cols <= 0 || p.cols % 256 != 0 || p.splits < 1) return hipErrorInvalidValue;
+    if (p.norm_w && p.cols > 8192) return hipErrorInvalidValue;
+    SplitRowsArgs a{p.x, p.splits, p.plane, p.residual, p.y, p.norm_w, p.norm_eps, p.cols, p.out.hi, p.out.lo, p.out.sums};
+    if (p.norm_w) hipLaunchKernelGGL(split_rows_kernel<true>, dim3(p.rows), dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(split_rows_kernel<false>, dim3(p.rows), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace esp

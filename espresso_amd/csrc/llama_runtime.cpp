@@ -70,6 +70,7 @@ LlamaRuntime::~LlamaRuntime() {
     free_device(rope_cos_); free_device(rope_sin_);
     free_device(hidden_); free_device(qkv_); free_device(q_); free_device(gu_); free_device(logits_);
     free_device(last_hidden_); free_device(xn_); free_device(ctx_); free_device(act_);
+    free_device(xn_lo_); free_device(ctx_lo_); free_device(act_lo_); free_device(xn_sums_); free_device(ctx_sums_); free_device(act_sums_);
     free_device(d_tokens_); free_device(d_pos_); free_device(d_seq_); free_device(d_out_tokens_);
     free_device(d_visible_); free_device(d_log_); free_device(d_log_count_);
     free_device(attn_scratch_);
@@ -397,6 +398,14 @@ int LlamaRuntime::finalize() {
     if ((rc = device_alloc(&xn_, R * (size_t)(d > hd ? d : hd))) != ESP_OK) return rc;
     if ((rc = device_alloc(&ctx_, R * ad)) != ESP_OK) return rc;
     if ((rc = device_alloc(&act_, R * hd)) != ESP_OK) return rc;
+    if (d % 256 == 0 && ad % 256 == 0 && hd % 256 == 0) {   // split rows for prompt blocks (Q4_K models)
+        if ((rc = device_alloc(&xn_lo_, R * (size_t)d)) != ESP_OK) return rc;
+        if ((rc = device_alloc(&ctx_lo_, R * (size_t)ad)) != ESP_OK) return rc;
+        if ((rc = device_alloc(&act_lo_, R * (size_t)hd)) != ESP_OK) return rc;
+        if ((rc = device_alloc(&xn_sums_, R * (size_t)(d / 16))) != ESP_OK) return rc;
+        if ((rc = device_alloc(&ctx_sums_, R * (size_t)(ad / 16))) != ESP_OK) return rc;
+        if ((rc = device_alloc(&act_sums_, R * (size_t)(hd / 16))) != ESP_OK) return rc;
+    }
     if ((rc = device_alloc(&d_tokens_, R)) != ESP_OK) return rc;
     if ((rc = device_alloc(&d_pos_, R)) != ESP_OK) return rc;
     if ((rc = device_alloc(&d_seq_, R)) != ESP_OK) return rc;
@@ -653,7 +662,64 @@ int LlamaRuntime::prefill_block(int seq, const uint32_t *tokens, int rows, int b
 // The layer loop over `rows` rows whose embeddings sit in hidden_ and whose (position, sequence) sit in
 // d_pos_/d_seq_, every projection as one dequant-fused MFMA GEMM.  Rows that are one sequence at consecutive positions
 // (a prompt block) take the matrix-core attention kernel, others the single-query one.
+// Prompt blocks of Q4_K models: every projection with exact weights and split activations (launch_gemm_split), queries and softmax
+// weights split in the attention: the block then stays as close to the fp32 CPU walk as the decode steps do.
+bool LlamaRuntime::split_blocks_supported() const {
+    if (!split_activations_ || !xn_lo_ || !prompt_attention_ || c_.kv_format != FMT_F16 || c_.d_model > 8192) return false;
+    for (const Layer &L : layers_)
+        if (L.q_norm || !gemm_split_supported(L.wqkv) || !gemm_split_supported(L.wo) || !gemm_split_supported(L.w13) || !gemm_split_supported(L.w2)) return false;
+    return true;
+}
+
+int LlamaRuntime::enqueue_layers_split(int rows) {
+    hipStream_t s = context().stream;
+    const int d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
+    const size_t cache_seq_stride = (size_t)kd * c_.max_seq;
+    SplitRowsView xn{xn_, xn_lo_, xn_sums_}, ctx{ctx_, ctx_lo_, ctx_sums_}, act{act_, act_lo_, act_sums_};
+    // RMSNorm of hidden_ (or of the split-K planes a projection left, added to hidden_ first) into split rows
+    auto norm = [&](const float *w, int splits) -> hipError_t {
+        SplitRowsParams p;
+        p.rows = rows; p.cols = d; p.norm_w = w; p.norm_eps = c_.norm_eps; p.out = xn;
+        if (splits > 1) { p.x = gemm_workspace_; p.splits = splits; p.plane = (size_t)rows * d; p.residual = hidden_; p.y = hidden_; }
+        else p.x = hidden_;
+        return launch_split_rows(p, s);
+    };
+    ESP_HIP_TRY(norm(layers_.front().rms_att, 1));
+    for (size_t li = 0; li < layers_.size(); li++) {
+        Layer &L = layers_[li];
+        GemmSplitParams g;
+        g.rows = rows; g.workspace = gemm_workspace_; g.workspace_floats = kGemmWorkspaceFloats;
+        int splits = 1;
+        g.w = L.wqkv; g.x = xn; g.y = qkv_; g.deferred_splits = &splits;
+        ESP_HIP_TRY(launch_gemm_split(g, s));
+        QkvPostArgs qa{};
+        qa.qkv = splits > 1 ? gemm_workspace_ : qkv_; qa.splits = splits; qa.plane = (size_t)rows * (ad + 2 * kd);
+        qa.q_norm = nullptr; qa.k_norm = nullptr; qa.norm_eps = c_.norm_eps;
+        qa.n_head = c_.n_head; qa.n_kv_head = c_.n_kv_head; qa.head_dim = c_.head_dim; qa.max_seq = c_.max_seq;
+        qa.rope_cos = rope_cos_; qa.rope_sin = rope_sin_; qa.pos = d_pos_; qa.seq = d_seq_;
+        qa.q_out = q_; qa.k_cache = L.k_cache; qa.v_cache = L.v_cache; qa.cache_seq_stride = cache_seq_stride;
+        ESP_HIP_TRY(launch_qkv_post(qa, rows, true, s));
+        AttentionArgs aa{};
+        aa.q = q_; aa.k_cache = L.k_cache; aa.v_cache = L.v_cache; aa.cache_seq_stride = cache_seq_stride;
+        aa.n_head = c_.n_head; aa.n_kv_head = c_.n_kv_head; aa.head_dim = c_.head_dim; aa.max_seq = c_.max_seq;
+        aa.pos = d_pos_; aa.seq = d_seq_; aa.ctx_hi = ctx.hi; aa.ctx_lo = ctx.lo; aa.ctx_sums = ctx.sums;
+        ESP_HIP_TRY(launch_attention_prompt(aa, rows, true, s));
+        g.w = L.wo; g.x = ctx; g.y = hidden_; g.residual = hidden_; splits = 1;
+        ESP_HIP_TRY(launch_gemm_split(g, s));
+        ESP_HIP_TRY(norm(L.rms_ffn, splits));
+        g.w = L.w13; g.x = xn; g.y = nullptr; g.residual = nullptr; g.swiglu = act; g.deferred_splits = nullptr;
+        ESP_HIP_TRY(launch_gemm_split(g, s));
+        g.swiglu = SplitRowsView{};
+        const bool last = li + 1 == layers_.size();
+        g.w = L.w2; g.x = act; g.y = hidden_; g.residual = hidden_; splits = 1; g.deferred_splits = last ? nullptr : &splits;
+        ESP_HIP_TRY(launch_gemm_split(g, s));
+        if (!last) ESP_HIP_TRY(norm(layers_[li + 1].rms_att, splits));
+    }
+    return ESP_OK;
+}
+
 int LlamaRuntime::enqueue_layers_matrix(int rows, bool one_sequence_consecutive) {
+    if (one_sequence_consecutive && split_blocks_supported()) return enqueue_layers_split(rows);
     hipStream_t s = context().stream;
     const int d = c_.d_model, ad = c_.attention_dim(), kd = c_.kv_dim(), hd = c_.hidden_dim;
     const bool kv16 = c_.kv_format == FMT_F16;

@@ -162,6 +162,10 @@ class LlamaRuntime {
     // activations for up to kMaxStepRows rows
     float *hidden_ = nullptr, *qkv_ = nullptr, *q_ = nullptr, *gu_ = nullptr, *logits_ = nullptr, *last_hidden_ = nullptr;
     uint16_t *xn_ = nullptr, *ctx_ = nullptr, *act_ = nullptr;
+    // prompt blocks with split activations: the lo planes and sub-block sums beside xn_, ctx_ and act_ (SplitRowsView)
+    uint16_t *xn_lo_ = nullptr, *ctx_lo_ = nullptr, *act_lo_ = nullptr, *xn_sums_ = nullptr, *ctx_sums_ = nullptr, *act_sums_ = nullptr;
+    bool split_blocks_supported() const;
+    int enqueue_layers_split(int rows);
     int *d_tokens_ = nullptr, *d_pos_ = nullptr, *d_seq_ = nullptr, *d_out_tokens_ = nullptr;
     std::vector<int> visible_;
     size_t weight_bytes_ = 0;

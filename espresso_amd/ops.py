@@ -80,6 +80,17 @@ class Matrix:
         _lib.check(_lib.load_library().esp_gemv(self._h, _ptr(x), batch, _ptr(y), _ptr(res) if res is not None else None))
         return y
 
+    def matmul_f32(self, x: np.ndarray, residual: np.ndarray | None = None) -> np.ndarray:
+        """fp32 activations [rows][cols] against the matrix with no operand rounded (esp_matmul_f32; Q4_K)."""
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.cols)
+        rows = x.shape[0]
+        y = np.empty((rows, self.rows), dtype=np.float32)
+        res = None
+        if residual is not None:
+            res = np.ascontiguousarray(residual, dtype=np.float32).reshape(rows, self.rows)
+        _lib.check(_lib.load_library().esp_matmul_f32(self._h, _ptr(x), rows, _ptr(y), _ptr(res) if res is not None else None))
+        return y
+
     def time_gemv(self, batch: int = 1, warmup: int = 10, iters: int = 50, rotate: int = 1) -> dict:
         mean, best = C.c_double(0), C.c_double(0)
         _lib.check(_lib.load_library().esp_gemv_time(self._h, batch, warmup, iters, rotate, C.byref(mean), C.byref(best)))

@@ -79,6 +79,13 @@ int esp_matrix_dequantize(const ESPMatrix *matrix, float *out);
  * batch 1 and 2 run the wave-per-row-pair GEMV; batch > 2 (prompt blocks, batched verify; any count) runs
  * the dequant-fused MFMA kernel, which rounds each dequantised weight to fp16 once (the GEMV does not). */
 int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y, const float *residual);
+/* The same product for fp32 activations, as the reference's CPU path feeds them (multiplyRowMajorMatrix,
+ * RealModelInferenceEngine.swift:6674-6718, called per prompt token at :6365-6375): y[r][n] = (residual +) sum_c x[r][c] *
+ * dequant(W)[n][c] for a block of `rows` rows, x fp32 [rows][cols], y and residual fp32 [rows][matrix rows]; host pointers.
+ * Q4_K matrices with a multiple of 256 columns.  The matrix cores take fp16 operands: each activation goes in as two fp16 numbers
+ * (hi = fp16(v), lo = fp16((v - hi) * 2048)) and each weight as the exact integer sc * q of its sub-block, with d, dmin and the
+ * sub-block minimums applied in fp32, so no operand is rounded. */
+int esp_matmul_f32(const ESPMatrix *matrix, const float *x, int rows, float *y, const float *residual);
 /* esp_gemv for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  x, y and residual are DEVICE pointers
  * (fp16 [batch][cols], fp32 [batch][rows], fp32 [batch][rows] or NULL); the call makes no hipMalloc / hipFree: the
