@@ -129,7 +129,7 @@ struct GemmParams {
 };
 
 // Rows of activations split for the matrix cores: v = hi + lo / 2048 with hi = fp16(v), lo = fp16((v - hi) * 2048), both
-// [rows][cols] fp16, and per (row, super-block of 256 columns) sixteen fp16 `sums`: the sums S_j of the row over the eight
+// [rows][cols] fp16 with the middle two of every four columns exchanged (c0, c2, c1, c3: the order in which the GEMM unpacks nibbles), and per (row, super-block of 256 columns) sixteen fp16 `sums`: the sums S_j of the row over the eight
 // sub-blocks of 32 columns as fp16(S_j), j = 0..7, then fp16((S_j - fp16(S_j)) * 2048).
 struct SplitRowsView {
     uint16_t *hi = nullptr, *lo = nullptr, *sums = nullptr;

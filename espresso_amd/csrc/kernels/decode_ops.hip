@@ -672,10 +672,10 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
                     vl[e] = (_Float16)__fmul_rn(__fsub_rn(v, (float)vh[e]), 2048.0f);
                     s += __builtin_fmaf((float)vl[e], 1.0f / 2048.0f, (float)vh[e]);
                 }
-                if (col <= last_row) {
+                if (col <= last_row) {   // the planes' order inside fours: (0, 2, 1, 3)
                     const size_t o16 = row * ad + (size_t)head * HD + 32 * mt + 8 * q4 + 4 * half;
-                    *reinterpret_cast<attn_half4 *>(a.ctx_hi + o16) = vh;
-                    *reinterpret_cast<attn_half4 *>(a.ctx_lo + o16) = vl;
+                    *reinterpret_cast<attn_half4 *>(a.ctx_hi + o16) = attn_half4{vh[0], vh[2], vh[1], vh[3]};
+                    *reinterpret_cast<attn_half4 *>(a.ctx_lo + o16) = attn_half4{vl[0], vl[2], vl[1], vl[3]};
                 }
             }
             s += __shfl_xor(s, 32);

@@ -22,6 +22,8 @@
 #include "../common.h"
 #include "decode_ops.h"
 #include <atomic>
+#include <type_traits>
+#include <utility>
 
 namespace esp {
 namespace {
@@ -118,116 +120,183 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_kernel(SplitGemmArgs 
 #pragma unroll
             for (int r = 0; r < 16; r++) tot[i][j][r] = ah[i][j][r] = al[i][j][r] = 0.0f;
 
-    auto fetch_w = [&](int tile) {
+    auto fetch_w = [&](int tile) __attribute__((always_inline)) {
         RawTile r;
         const uint8_t *blk = w_base + (size_t)(tile >> 2) * 144;
         r.hdr = *reinterpret_cast<const uint4 *>(blk);
         r.q = *reinterpret_cast<const uint4 *>(blk + 16 + (tile & 3) * 32 + wh * 16);
         return r;
     };
-    auto fetch_x = [&](int tile, uint4 (&vh)[XV], uint4 (&vl)[XV]) {
-#pragma unroll
-        for (int i = 0; i < XV; i++) {
-            const int piece = tid + i * kThreads, row = piece >> 3, part = piece & 7;
-            const int m = m0 + row < a.M ? m0 + row : a.M - 1;   // rows beyond M repeat the last one; never stored
-            const size_t o = (size_t)m * a.K + (size_t)tile * KT;
-            vh[i] = reinterpret_cast<const uint4 *>(a.xh + o)[part];
-            vl[i] = reinterpret_cast<const uint4 *>(a.xl + o)[part];
-        }
+    // piece i of a thread: row (tid / 8) + 32 i of the tile, eight columns (tid % 8) * 8 .. of it; rows beyond M repeat the last
+    // one (never stored).  Element offsets fit 32 bits (the host checks M * K).
+    const unsigned x_col = (unsigned)(tid & 7) * 8;
+    auto x_row_offset = [&](int i) __attribute__((always_inline)) {
+        const int row = (tid >> 3) + 32 * i;
+        return (unsigned)(m0 + row < a.M ? m0 + row : a.M - 1) * (unsigned)a.K + x_col;
     };
-    auto fetch_sums = [&](int sb) {
+    const unsigned xo0 = x_row_offset(0), xo1 = x_row_offset(1), xo2 = x_row_offset(2), xo3 = x_row_offset(3);
+    static_assert(XV == 4, "four pieces per thread and plane");
+    struct XTile { uint4 h0, h1, h2, h3, l0, l1, l2, l3; };   // named members: the registers in flight must never look like an indexed array
+    auto fetch_x = [&](int tile) __attribute__((always_inline)) {
+        const unsigned t = (unsigned)tile * KT;
+        XTile x;
+        x.h0 = *reinterpret_cast<const uint4 *>(a.xh + (xo0 + t)); x.l0 = *reinterpret_cast<const uint4 *>(a.xl + (xo0 + t));
+        x.h1 = *reinterpret_cast<const uint4 *>(a.xh + (xo1 + t)); x.l1 = *reinterpret_cast<const uint4 *>(a.xl + (xo1 + t));
+        x.h2 = *reinterpret_cast<const uint4 *>(a.xh + (xo2 + t)); x.l2 = *reinterpret_cast<const uint4 *>(a.xl + (xo2 + t));
+        x.h3 = *reinterpret_cast<const uint4 *>(a.xh + (xo3 + t)); x.l3 = *reinterpret_cast<const uint4 *>(a.xl + (xo3 + t));
+        return x;
+    };
+    auto fetch_sums = [&](int sb) __attribute__((always_inline)) {
         return reinterpret_cast<const uint4 *>(a.xs + ((size_t)xs_row * sbs + (sb < sbs ? sb : sbs - 1)) * 16)[tid & 1];
     };
 
-    RawTile raw[DEPTH];
-    uint4 vh[DEPTH][XV], vl[DEPTH][XV];
-#pragma unroll
-    for (int d = 0; d < DEPTH; d++) {
-        const int tile = t_begin + d < t_last ? t_begin + d : t_last;
-        raw[d] = fetch_w(tile);
-        fetch_x(tile, vh[d], vl[d]);
-    }
+    static_assert(DEPTH == 2, "two tiles in flight: slots 0 and 1 below");
+    const int t_second = t_begin + 1 < t_last ? t_begin + 1 : t_last;
+    RawTile raw0 = fetch_w(t_begin), raw1 = fetch_w(t_second);
+    XTile x0 = fetch_x(t_begin), x1 = fetch_x(t_second);
     uint4 sums_next = fetch_sums(t_begin >> 2);
-    static_assert(4 % DEPTH == 0, "the main loop is unrolled by four");
 
-    // Stages tile `tile` (slot S of the registers in flight, c = tile % 4 a constant) into LDS buffer `buf`, and with the first tile
-    // of a super-block that super-block's minimums, scales and activation sums into buffer (tile / 4) % 2.
-    auto stage = [&](int S, int c, int tile, int buf) {
-        const RawTile &r = raw[S];
-        u32 sc_lo, m_lo, sc_hi, m_hi;
-        q4k_scale_min(r.hdr, 2 * c, sc_lo, m_lo);
-        q4k_scale_min(r.hdr, 2 * c + 1, sc_hi, m_hi);
+    // Staging of tile `tile` (slot S of the registers in flight, c = tile % 4) into LDS buffer `buf` - and with the first tile of a
+    // super-block that super-block's minimums, scales and activation sums into buffer (tile / 4) % 2 - cut into kPieces pieces of a few
+    // instructions each.  A wavefront is alone on its SIMD (436 registers), so nothing overlaps unless its own instruction stream
+    // interleaves: the main loop issues one piece behind every MFMA, fenced, and the piece runs while the matrix core works (counters
+    // of the plain order: MFMA busy 31 %, vector ALU 30 %, waiting 38 % of the wavefront's cycles, adding up to all of them).
+    struct StageRegs { h2 s_lo, s_hi, o_lo, o_hi; u32 lo[8], hi[8]; };
+    constexpr int kPieces = 30;
+    auto stage_piece = [&](auto piece_c, auto slot_c, auto chunk_c, int tile, int buf, StageRegs &sr) __attribute__((always_inline)) {
+        constexpr int P = decltype(piece_c)::value, S = decltype(slot_c)::value, c = decltype(chunk_c)::value;
+        RawTile &rs = S == 0 ? raw0 : raw1;
+        XTile &xr = S == 0 ? x0 : x1;
         // low nibbles under 0x6400 read 1024 + q, high nibbles under 0x5400 read 64 + q; (offset + q) * sc - offset * sc is one
         // exact packed multiply-add: the result sc * q <= 945 is an integer
-        const _Float16 fl = (_Float16)(float)sc_lo, fh = (_Float16)(float)sc_hi;
-        const h2 s_lo = {fl, fl}, s_hi = {fh, fh};
-        const _Float16 ol = (_Float16)(-1024.0f * (float)sc_lo), oh = (_Float16)(-64.0f * (float)sc_hi);
-        const h2 o_lo = {ol, ol}, o_hi = {oh, oh};
-        u32 lo[8], hi[8];
+        if constexpr (P == 0) {
+            u32 sc, m;
+            q4k_scale_min(rs.hdr, 2 * c, sc, m);
+            const _Float16 f = (_Float16)(float)sc, o = (_Float16)(-1024.0f * (float)sc);
+            sr.s_lo = h2{f, f}; sr.o_lo = h2{o, o};
+        } else if constexpr (P == 1) {
+            u32 sc, m;
+            q4k_scale_min(rs.hdr, 2 * c + 1, sc, m);
+            const _Float16 f = (_Float16)(float)sc, o = (_Float16)(-64.0f * (float)sc);
+            sr.s_hi = h2{f, f}; sr.o_hi = h2{o, o};
+        } else if constexpr (P >= 2 && P < 6) {
+            constexpr int k = P - 2;
+            const u32 w = dword_of(rs.q, k), w8 = w >> 8;
+            sr.lo[2 * k] = as_u32(__builtin_elementwise_fma(as_h2((w & 0x000F000Fu) | 0x64006400u), sr.s_lo, sr.o_lo));
+            sr.lo[2 * k + 1] = as_u32(__builtin_elementwise_fma(as_h2((w8 & 0x000F000Fu) | 0x64006400u), sr.s_lo, sr.o_lo));
+        } else if constexpr (P >= 6 && P < 10) {
+            constexpr int k = P - 6;
+            const u32 w = dword_of(rs.q, k), w8 = w >> 8;
+            sr.hi[2 * k] = as_u32(__builtin_elementwise_fma(as_h2((w & 0x00F000F0u) | 0x54005400u), sr.s_hi, sr.o_hi));
+            sr.hi[2 * k + 1] = as_u32(__builtin_elementwise_fma(as_h2((w8 & 0x00F000F0u) | 0x54005400u), sr.s_hi, sr.o_hi));
+        } else if constexpr (P >= 10 && P < 14) {
+            _Float16 *wrow = wt + buf * (int)kTileHalfs + wr * LDK;
+            if constexpr (P == 10) *reinterpret_cast<uint4 *>(wrow + 16 * wh) = make_uint4(sr.lo[0], sr.lo[1], sr.lo[2], sr.lo[3]);
+            if constexpr (P == 11) *reinterpret_cast<uint4 *>(wrow + 16 * wh + 8) = make_uint4(sr.lo[4], sr.lo[5], sr.lo[6], sr.lo[7]);
+            if constexpr (P == 12) *reinterpret_cast<uint4 *>(wrow + 32 + 16 * wh) = make_uint4(sr.hi[0], sr.hi[1], sr.hi[2], sr.hi[3]);
+            if constexpr (P == 13) *reinterpret_cast<uint4 *>(wrow + 32 + 16 * wh + 8) = make_uint4(sr.hi[4], sr.hi[5], sr.hi[6], sr.hi[7]);
+        } else if constexpr (P >= 14 && P < 22) {
+            // the planes already hold the (0,2,1,3) order the weights are unpacked in
+            const int o = buf * (int)kTileHalfs + (tid >> 3) * LDK + (tid & 7) * 8;
+            if constexpr (P == 14) *reinterpret_cast<uint4 *>(xh + o) = xr.h0;
+            if constexpr (P == 15) *reinterpret_cast<uint4 *>(xl + o) = xr.l0;
+            if constexpr (P == 16) *reinterpret_cast<uint4 *>(xh + o + 32 * LDK) = xr.h1;
+            if constexpr (P == 17) *reinterpret_cast<uint4 *>(xl + o + 32 * LDK) = xr.l1;
+            if constexpr (P == 18) *reinterpret_cast<uint4 *>(xh + o + 64 * LDK) = xr.h2;
+            if constexpr (P == 19) *reinterpret_cast<uint4 *>(xl + o + 64 * LDK) = xr.l2;
+            if constexpr (P == 20) *reinterpret_cast<uint4 *>(xh + o + 96 * LDK) = xr.h3;
+            if constexpr (P == 21) *reinterpret_cast<uint4 *>(xl + o + 96 * LDK) = xr.l3;
+        } else if constexpr (P == 22) {
+            if constexpr (c == 0) {
+                const int sbuf = (tile >> 2) & 1;
+                u32 mm[4];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const u32 w = dword_of(r.q, k), w8 = w >> 8;
-            lo[2 * k] = as_u32(__builtin_elementwise_fma(as_h2((w & 0x000F000Fu) | 0x64006400u), s_lo, o_lo));
-            lo[2 * k + 1] = as_u32(__builtin_elementwise_fma(as_h2((w8 & 0x000F000Fu) | 0x64006400u), s_lo, o_lo));
-            hi[2 * k] = as_u32(__builtin_elementwise_fma(as_h2((w & 0x00F000F0u) | 0x54005400u), s_hi, o_hi));
-            hi[2 * k + 1] = as_u32(__builtin_elementwise_fma(as_h2((w8 & 0x00F000F0u) | 0x54005400u), s_hi, o_hi));
+                for (int jj = 0; jj < 4; jj++) { u32 s_unused; q4k_scale_min(rs.hdr, 4 * wh + jj, s_unused, mm[jj]); }
+                _Float16 *mrow = ms + sbuf * 128 * 16 + wr * 16 + 4 * wh;
+                *reinterpret_cast<uint2 *>(mrow) = make_uint2(pack_half2((float)mm[0], (float)mm[1]), pack_half2((float)mm[2], (float)mm[3]));
+                *reinterpret_cast<uint2 *>(mrow + 8) = make_uint2(pack_half2((float)mm[0] * kUnscale, (float)mm[1] * kUnscale),
+                                                                  pack_half2((float)mm[2] * kUnscale, (float)mm[3] * kUnscale));
+                // both threads of a weight row write the same (d, dmin): no branch
+                dd[sbuf * 128 + wr] = make_float2(half_bits_to_float(rs.hdr.x & 0xFFFFu), half_bits_to_float(rs.hdr.x >> 16));
+                *reinterpret_cast<uint4 *>(xs + sbuf * 128 * 16 + (tid >> 1) * 16 + 8 * (tid & 1)) = sums_next;
+            }
+        } else {
+            // the slot is free: the tile DEPTH ahead goes into it (clamped past the end: fetched in bounds, never used)
+            const int ahead = tile + DEPTH < t_last ? tile + DEPTH : t_last;
+            const unsigned tk = (unsigned)ahead * KT;
+            if constexpr (P == 23) {
+                const uint8_t *blk = w_base + (size_t)(ahead >> 2) * 144;
+                rs.hdr = *reinterpret_cast<const uint4 *>(blk);
+                rs.q = *reinterpret_cast<const uint4 *>(blk + 16 + (ahead & 3) * 32 + wh * 16);
+            }
+            if constexpr (P == 24) { xr.h0 = *reinterpret_cast<const uint4 *>(a.xh + (xo0 + tk)); xr.l0 = *reinterpret_cast<const uint4 *>(a.xl + (xo0 + tk)); }
+            if constexpr (P == 25) { xr.h1 = *reinterpret_cast<const uint4 *>(a.xh + (xo1 + tk)); xr.l1 = *reinterpret_cast<const uint4 *>(a.xl + (xo1 + tk)); }
+            if constexpr (P == 26) { xr.h2 = *reinterpret_cast<const uint4 *>(a.xh + (xo2 + tk)); xr.l2 = *reinterpret_cast<const uint4 *>(a.xl + (xo2 + tk)); }
+            if constexpr (P == 27) { xr.h3 = *reinterpret_cast<const uint4 *>(a.xh + (xo3 + tk)); xr.l3 = *reinterpret_cast<const uint4 *>(a.xl + (xo3 + tk)); }
+            if constexpr (P == 28 && c == 0) sums_next = fetch_sums((tile >> 2) + 1);
         }
-        _Float16 *wrow = wt + (size_t)buf * kTileHalfs + wr * LDK;
-        uint4 *plo = reinterpret_cast<uint4 *>(wrow + 16 * wh), *phi = reinterpret_cast<uint4 *>(wrow + 32 + 16 * wh);
-        plo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        plo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-        phi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        phi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-#pragma unroll
-        for (int i = 0; i < XV; i++) {
-            const int piece = tid + i * kThreads, row = piece >> 3, part = piece & 7;
-            *reinterpret_cast<uint4 *>(xh + (size_t)buf * kTileHalfs + row * LDK + part * 8) = swap_middle(vh[S][i]);
-            *reinterpret_cast<uint4 *>(xl + (size_t)buf * kTileHalfs + row * LDK + part * 8) = swap_middle(vl[S][i]);
-        }
-        if (c == 0) {
-            const int sbuf = (tile >> 2) & 1;
-            u32 mm[4];
-#pragma unroll
-            for (int jj = 0; jj < 4; jj++) { u32 s_unused; q4k_scale_min(r.hdr, 4 * wh + jj, s_unused, mm[jj]); }
-            _Float16 *mrow = ms + (size_t)sbuf * 128 * 16 + wr * 16 + 4 * wh;
-            *reinterpret_cast<uint2 *>(mrow) = make_uint2(pack_half2((float)mm[0], (float)mm[1]), pack_half2((float)mm[2], (float)mm[3]));
-            *reinterpret_cast<uint2 *>(mrow + 8) = make_uint2(pack_half2((float)mm[0] * kUnscale, (float)mm[1] * kUnscale),
-                                                              pack_half2((float)mm[2] * kUnscale, (float)mm[3] * kUnscale));
-            if (wh == 0) dd[sbuf * 128 + wr] = make_float2(half_bits_to_float(r.hdr.x & 0xFFFFu), half_bits_to_float(r.hdr.x >> 16));
-            *reinterpret_cast<uint4 *>(xs + (size_t)sbuf * 128 * 16 + (tid >> 1) * 16 + 8 * (tid & 1)) = sums_next;
-            sums_next = fetch_sums((tile >> 2) + 1);
-        }
-        const int ahead = tile + DEPTH < t_last ? tile + DEPTH : t_last;
-        raw[S] = fetch_w(ahead);
-        fetch_x(ahead, vh[S], vl[S]);
+    };
+    auto stage_all = [&](auto slot_c, auto chunk_c, int tile, int buf) __attribute__((always_inline)) {
+        StageRegs sr;
+        auto run = [&](auto... pc) __attribute__((always_inline)) { (stage_piece(pc, slot_c, chunk_c, tile, buf, sr), ...); };
+        [&]<int... I>(std::integer_sequence<int, I...>) __attribute__((always_inline)) { run(std::integral_constant<int, I>{}...); }(std::make_integer_sequence<int, kPieces>{});
     };
 
-    stage(0, 0, t_begin, 0);   // t_begin is a multiple of four
+    stage_all(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, t_begin, 0);   // t_begin is a multiple of four
     __syncthreads();
-    for (int t0 = t_begin; t0 < t_end; t0 += 4) {
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int t = t0 + u, buf = u & 1;
+    auto tile_step = [&](auto u_c, int t) __attribute__((always_inline)) {
+            constexpr int u = decltype(u_c)::value, buf = u & 1;
             const _Float16 *xhb = xh + (size_t)buf * kTileHalfs, *xlb = xl + (size_t)buf * kTileHalfs, *wtb = wt + (size_t)buf * kTileHalfs;
-#pragma unroll
-            for (int ks = 0; ks < KT / 16; ks++) {
+            struct Frags { half8 h0, h1, l0, l1, b0, b1; };
+            auto load_frags = [&](int ks) __attribute__((always_inline)) {
                 const int kk = ks * 16 + 8 * (lane >> 5);
-                half8 fh[2], fl[2], fb[2];
-#pragma unroll
-                for (int i = 0; i < 2; i++) {
-                    fh[i] = *reinterpret_cast<const half8 *>(xhb + ((wm * 2 + i) * 32 + (lane & 31)) * LDK + kk);
-                    fl[i] = *reinterpret_cast<const half8 *>(xlb + ((wm * 2 + i) * 32 + (lane & 31)) * LDK + kk);
-                }
-#pragma unroll
-                for (int j = 0; j < 2; j++) fb[j] = *reinterpret_cast<const half8 *>(wtb + ((wn * 2 + j) * 32 + (lane & 31)) * LDK + kk);
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-#pragma unroll
-                    for (int j = 0; j < 2; j++) {
-                        ah[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh[i], fb[j], ah[i][j], 0, 0, 0);
-                        al[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl[i], fb[j], al[i][j], 0, 0, 0);
-                    }
-            }
+                const int ra = (wm * 64 + (lane & 31)) * LDK + kk, rb = (wn * 64 + (lane & 31)) * LDK + kk;
+                Frags f;
+                f.h0 = *reinterpret_cast<const half8 *>(xhb + ra);
+                f.h1 = *reinterpret_cast<const half8 *>(xhb + ra + 32 * LDK);
+                f.l0 = *reinterpret_cast<const half8 *>(xlb + ra);
+                f.l1 = *reinterpret_cast<const half8 *>(xlb + ra + 32 * LDK);
+                f.b0 = *reinterpret_cast<const half8 *>(wtb + rb);
+                f.b1 = *reinterpret_cast<const half8 *>(wtb + rb + 32 * LDK);
+                return f;
+            };
+            auto mfma_one = [&](const Frags &f, auto m_c) __attribute__((always_inline)) {
+                constexpr int m = decltype(m_c)::value;
+                if constexpr (m == 0) ah[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.h0, f.b0, ah[0][0], 0, 0, 0);
+                if constexpr (m == 1) al[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.l0, f.b0, al[0][0], 0, 0, 0);
+                if constexpr (m == 2) ah[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.h0, f.b1, ah[0][1], 0, 0, 0);
+                if constexpr (m == 3) al[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.l0, f.b1, al[0][1], 0, 0, 0);
+                if constexpr (m == 4) ah[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.h1, f.b0, ah[1][0], 0, 0, 0);
+                if constexpr (m == 5) al[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.l1, f.b0, al[1][0], 0, 0, 0);
+                if constexpr (m == 6) ah[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.h1, f.b1, ah[1][1], 0, 0, 0);
+                if constexpr (m == 7) al[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.l1, f.b1, al[1][1], 0, 0, 0);
+            };
+            // the tile being staged behind the MFMAs: t + 1, from slot (u + 1) % 2 into the other LDS buffer
+            constexpr int S = (u + 1) % DEPTH, c = (u + 1) & 3;
+            StageRegs sr;
+            // eight MFMAs of k step `ks` (fragments f), piece first + m behind MFMA m
+            auto k_step = [&](const Frags &f, auto first_c) __attribute__((always_inline)) {
+                constexpr int first = decltype(first_c)::value;
+                [&]<int... M>(std::integer_sequence<int, M...>) __attribute__((always_inline)) {
+                    ((mfma_one(f, std::integral_constant<int, M>{}),
+                      stage_piece(std::integral_constant<int, (first + M < kPieces ? first + M : kPieces)>{}, std::integral_constant<int, S>{},
+                                  std::integral_constant<int, c>{}, t + 1, buf ^ 1, sr),
+                      __builtin_amdgcn_sched_barrier(0)), ...);
+                }(std::make_integer_sequence<int, 8>{});
+            };
+            const Frags f0 = load_frags(0);
+            stage_piece(std::integral_constant<int, 0>{}, std::integral_constant<int, S>{}, std::integral_constant<int, c>{}, t + 1, buf ^ 1, sr);
+            stage_piece(std::integral_constant<int, 1>{}, std::integral_constant<int, S>{}, std::integral_constant<int, c>{}, t + 1, buf ^ 1, sr);
+            const Frags f1 = load_frags(1);
+            __builtin_amdgcn_sched_barrier(0);
+            k_step(f0, std::integral_constant<int, 2>{});
+            const Frags f2 = load_frags(2);
+            __builtin_amdgcn_sched_barrier(0);
+            k_step(f1, std::integral_constant<int, 10>{});
+            const Frags f3 = load_frags(3);
+            __builtin_amdgcn_sched_barrier(0);
+            k_step(f2, std::integral_constant<int, 18>{});
+            k_step(f3, std::integral_constant<int, 26>{});
             if (u == 3) {
                 // the super-block is complete: total += d * (hi sums + lo sums / 2048) - dmin * sum_j m_j S_j
                 const int sbuf = (t >> 2) & 1;
@@ -252,14 +321,18 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_kernel(SplitGemmArgs 
                         for (int r = 0; r < 16; r++) {
                             const float main = __builtin_fmaf(al[i][j][r], kUnscale, ah[i][j][r]);
                             tot[i][j][r] = __builtin_fmaf(-dv[j].y, am[r], __builtin_fmaf(dv[j].x, main, tot[i][j][r]));
-                            ah[i][j][r] = 0.0f;
-                            al[i][j][r] = 0.0f;
                         }
+                        ah[i][j] = floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                        al[i][j] = ah[i][j];
                     }
             }
-            stage((u + 1) % DEPTH, (u + 1) & 3, t + 1, buf ^ 1);   // past the end: the slot holds a clamped fetch; staged into the idle buffers, never read
             __syncthreads();
-        }
+    };
+    for (int t0 = t_begin; t0 < t_end; t0 += 4) {
+        tile_step(std::integral_constant<int, 0>{}, t0);
+        tile_step(std::integral_constant<int, 1>{}, t0 + 1);
+        tile_step(std::integral_constant<int, 2>{}, t0 + 2);
+        tile_step(std::integral_constant<int, 3>{}, t0 + 3);
     }
 
     // accumulator r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of the 32 x 32 tile
@@ -283,7 +356,8 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_kernel(SplitGemmArgs 
                         const float silu = __fmul_rn(hg, __fadd_rn(1.0f, tanhf(hg)));
                         const float act = __fmul_rn(silu, up);
                         const _Float16 hi = (_Float16)act;
-                        const size_t o = (size_t)m * (a.N / 2) + n / 2;
+                        const int unit = n / 2, slot = unit & 3;   // the planes' order inside fours: (0, 2, 1, 3)
+                        const size_t o = (size_t)m * (a.N / 2) + (unit & ~3) + (slot == 1 ? 2 : slot == 2 ? 1 : slot);
                         a.sw_hi[o] = __builtin_bit_cast(uint16_t, hi);
                         a.sw_lo[o] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(__fsub_rn(act, (float)hi), kScale));
                     }
@@ -325,8 +399,10 @@ __device__ __forceinline__ float split_eight(const float (&c)[8], uint4 &hi, uin
     float s = 0.0f;
 #pragma unroll
     for (int p = 0; p < 4; p++) {
-        const _Float16 ha = (_Float16)c[2 * p], hb = (_Float16)c[2 * p + 1];
-        const _Float16 la = (_Float16)__fmul_rn(__fsub_rn(c[2 * p], (float)ha), kScale), lb = (_Float16)__fmul_rn(__fsub_rn(c[2 * p + 1], (float)hb), kScale);
+        // pairs (c0, c2), (c1, c3), (c4, c6), (c5, c7): the planes' order inside fours
+        const int ia = 4 * (p >> 1) + (p & 1), ib = ia + 2;
+        const _Float16 ha = (_Float16)c[ia], hb = (_Float16)c[ib];
+        const _Float16 la = (_Float16)__fmul_rn(__fsub_rn(c[ia], (float)ha), kScale), lb = (_Float16)__fmul_rn(__fsub_rn(c[ib], (float)hb), kScale);
         h[p] = (u32)__builtin_bit_cast(uint16_t, ha) | ((u32)__builtin_bit_cast(uint16_t, hb) << 16);
         l[p] = (u32)__builtin_bit_cast(uint16_t, la) | ((u32)__builtin_bit_cast(uint16_t, lb) << 16);
         s += __builtin_fmaf((float)la, kUnscale, (float)ha) + __builtin_fmaf((float)lb, kUnscale, (float)hb);
@@ -460,6 +536,7 @@ bool gemm_split_supported(const DeviceMatrix &w) { return w.format == FMT_Q4_K &
 hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream) {
     const DeviceMatrix &w = p.w;
     if (!gemm_split_supported(w) || !p.x.hi || !p.x.lo || !p.x.sums || p.rows <= 0 || w.rows <= 0) return hipErrorInvalidValue;
+    if ((uint64_t)p.rows * (uint64_t)w.cols >= (1ull << 32)) return hipErrorInvalidValue;   // the kernel's activation offsets are 32-bit
     const bool swiglu = p.swiglu.hi != nullptr;
     if (swiglu ? (!p.swiglu.lo || w.rows % 2 != 0 || p.residual) : !p.y) return hipErrorInvalidValue;
     SplitGemmArgs a{};
