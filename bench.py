@@ -83,81 +83,98 @@ def run_gpu(name: str, steps: int, warmup: int, graph: bool = True):
     rt.prefill(prompt)
     rt.last_hidden()
     prefill_again_s = time.perf_counter() - t0
-    return dict(kernel_us=own, cfg=cfg, rt=rt, packed=packed, prompt=prompt, tokens=warm_tokens + tokens, elapsed=elapsed,
+    # and with every operand rounded to fp16 once (the faster, less exact block path)
+    ll.set_split_activations(rt, False)
+    rt.reset()
+    rt.last_hidden()
+    t0 = time.perf_counter()
+    rt.prefill(prompt)
+    rt.last_hidden()
+    prefill_fp16_s = time.perf_counter() - t0
+    ll.set_split_activations(rt, True)
+    return dict(prefill_fp16_s=prefill_fp16_s, kernel_us=own, cfg=cfg, rt=rt, packed=packed, prompt=prompt, tokens=warm_tokens + tokens, elapsed=elapsed,
                 build_s=build_s, prefill_s=prefill_s, prefill_again_s=prefill_again_s, kernel_times=kt, b2b_us=b2b, weight_bytes=rt.weight_bytes)
 
 
 def cpu_baseline(name: str, gpu: dict) -> dict:
-    """Times the CPU oracle (the C restatement of the reference's CPU-exact path, single thread) on a bounded
-    sample of the same model: same packed bytes, dequantised to fp32 as the reference holds them."""
+    """Times the CPU oracle (the C restatement of the reference's CPU-exact path) in the reference's default arithmetic - fp32
+    activations into every matrix product - on a bounded sample of the same model: same packed bytes, dequantised to fp32 as the
+    reference holds them.  The 6-layer model runs whole on one thread; the 8B model runs whole (all 32 layers, 32 GB of fp32
+    weights) with the matrix-vector rows spread over the host cores this process may use, on a short prompt."""
     from oracle import oracle as orc
-    import espresso_amd.llama as ll
     from espresso_amd import _lib
     w = WORKLOADS[name]
     cfg, packed = gpu["cfg"], gpu["packed"]
     fmt = _lib.FORMAT_NAMES[w["fmt"]]
-    shapes = {"wq": (cfg.attention_dim, cfg.d_model), "wk": (cfg.kv_dim, cfg.d_model), "wv": (cfg.kv_dim, cfg.d_model),
-              "wo": (cfg.d_model, cfg.attention_dim), "w1": (cfg.hidden_dim, cfg.d_model),
-              "w3": (cfg.hidden_dim, cfg.d_model), "w2": (cfg.d_model, cfg.hidden_dim)}
-    slot = {"rms_att": orc.W_RMS_ATT, "wq": orc.W_WQ, "wk": orc.W_WK, "wv": orc.W_WV, "wo": orc.W_WO,
-            "rms_ffn": orc.W_RMS_FFN, "w1": orc.W_W1, "w2": orc.W_W2, "w3": orc.W_W3}
+    host_cores = os.cpu_count() or 1
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = host_cores
     full = name == "stories-6l-q8_0"
-    n_layer = cfg.n_layer if full else 1
-    ocfg = orc.LlamaConfig(n_layer=n_layer, n_head=cfg.n_head, n_kv_head=cfg.n_kv_head, d_model=cfg.d_model,
-                           head_dim=cfg.head_dim, hidden_dim=cfg.hidden_dim, vocab=cfg.vocab, max_seq=len(gpu["prompt"]) + 16 if not full else cfg.max_seq,
-                           norm_eps=cfg.norm_eps, rope_theta=cfg.rope_theta, gemv_inputs_fp16=True, kv_fp16=w["kv"] == "f16")
-    rt = orc.LlamaRuntime(ocfg)
-    n = cfg.vocab * cfg.d_model
-    rt.set_weight(0, orc.W_TOKEN_EMBEDDING, orc.dequantize(orc.FMT_F16, packed["embedding"], n))
-    rt.set_weight(0, orc.W_FINAL_NORM, np.ones(cfg.d_model, np.float32))
-    rt.set_weight(0, orc.W_LM_HEAD, orc.dequantize(fmt, packed["lm_head"], n))
-    for l in range(n_layer):
-        for k, s in slot.items():
-            if k in shapes:
-                r, c = shapes[k]
-                rt.set_weight(l, s, orc.dequantize(fmt, packed["layers"][l][k], r * c))
-            else:
-                rt.set_weight(l, s, np.ones(cfg.d_model, np.float32))
+    threads = 1 if full else max(1, min(16, usable))
     prompt = gpu["prompt"]
-    if full:
+    n_prompt = len(prompt) if full else 32
+    before = orc.get_threads()
+    orc.set_threads(threads)
+    try:
         t0 = time.perf_counter()
-        rt.prefill(prompt.tolist())
-        n_tok = 32
+        rt = orc.runtime_from_packed(cfg, packed, fmt, cfg.n_layer, w["kv"] == "f16", cfg.max_seq if full else n_prompt + 24, gemv_inputs_fp16=False)
+        t_load = time.perf_counter() - t0
         t0 = time.perf_counter()
+        rt.prefill(prompt[:n_prompt].tolist())
+        t_prefill = time.perf_counter() - t0
+        n_tok = 32 if full else 16
         toks = []
+        t0 = time.perf_counter()
         for _ in range(n_tok):
             t = rt.select_greedy(); toks.append(t); rt.advance(t)
         dt = time.perf_counter() - t0
+        rt.close()
+    finally:
+        orc.set_threads(before)
+    out = {"value": n_tok / dt, "unit": "tok/s", "cores": threads, "host_cores": host_cores, "usable_cores": usable, "kind": "port",
+           "arithmetic": "reference default: fp32 activations, fp32 dequantised weights, fp32 sums"}
+    if full:
         same = toks == gpu["tokens"][:n_tok]
-        return {"value": n_tok / dt, "unit": "tok/s", "cores": 1, "kind": "port",
-                "sample": f"whole model, {n_tok} greedy tokens after the same {len(prompt)}-token prompt; "
-                          f"tokens identical to the GPU run: {same}"}
-    # bounded sample of the 8B shape: layer 0 alone plus the LM head, at the benchmark's context (the prompt is walked through
-    # the one layer first, so the timed tokens attend over 512+ cached positions as the GPU's do)
-    ctx = len(prompt)
-    t0 = time.perf_counter()
-    rt.prefill(prompt.tolist())
-    t_prefill = time.perf_counter() - t0
-    n_tok = 6
-    t_layer = t_head = 0.0
-    for i in range(n_tok):
-        t0 = time.perf_counter(); tok = rt.select_greedy(); t_head += time.perf_counter() - t0
-        t0 = time.perf_counter(); rt.advance(tok); t_layer += time.perf_counter() - t0
-    t_layer /= n_tok; t_head /= n_tok
-    est = 1.0 / (cfg.n_layer * t_layer + t_head)
-    return {"value": est, "unit": "tok/s", "cores": 1, "kind": "port",
-            "sample": f"layer 0 of {cfg.n_layer} ({t_layer * 1e3:.0f} ms/token incl. attention over {ctx}+ cached tokens) and the LM head "
-                      f"({t_head * 1e3:.0f} ms/token), {n_tok} decode tokens after the {ctx}-token prompt was walked through that layer "
-                      f"({t_prefill:.1f} s), extrapolated to {cfg.n_layer} layers"}
+        out["sample"] = (f"whole model, {n_tok} greedy tokens after the same {n_prompt}-token prompt on one thread; "
+                         f"tokens identical to the GPU run: {same}")
+    else:
+        out["sample"] = (f"whole model (all {cfg.n_layer} layers, fp32 weights dequantised in {t_load:.1f} s), {n_tok} greedy tokens after the "
+                         f"first {n_prompt} tokens of the prompt were walked ({t_prefill:.1f} s, {n_prompt / t_prefill:.1f} tok/s); matrix-vector "
+                         f"rows over {threads} threads (the order of every row's sum is the single-threaded one)")
+    return out
 
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # workload (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors kernels of known size in the same runs gave);
 # the runs and the per-kernel table are in profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt.
-MEASURED_TRAFFIC = {("llama3-8b-q4k", "gate_up"): 66521607}
-# the same kernel's mean duration in the committed rocprofv3 kernel trace (a profiled run; 2-4 % slower than an unprofiled one)
-PROFILE_KERNEL_US = {("llama3-8b-q4k", "gate_up"): (13.63, "profiles/q4k_gemv_decode_llama3_8b_kernel_trace.txt")}
-TRAFFIC_SOURCE = "profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload; not measured in this run)"
+TRAFFIC_FILE = "profiles/q4k_gemv_decode_llama3_8b_pmc_traffic.txt"
+# the same kernel's mean duration in the committed rocprofv3 kernel trace (a profiled run with eager launches)
+TRACE_FILE = "profiles/q4k_gemv_decode_llama3_8b_kernel_trace.txt"
+TRAFFIC_SOURCE = TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload; not measured in this run)"
+
+
+def profile_figure(path: str, key: str):
+    """A figure the committed profile summaries carry on a line of their own, `key = value`; None when the file or the line is absent."""
+    try:
+        with open(os.path.join(ROOT, path)) as f:
+            for line in f:
+                parts = line.split("=")
+                if len(parts) == 2 and parts[0].strip() == key:
+                    return float(parts[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
+def measured_traffic(workload: str, kernel: str):
+    v = profile_figure(TRAFFIC_FILE, f"{workload}.{kernel}.hbm_bytes_per_launch")
+    return int(v) if v is not None else None
+
+
+def profile_kernel_us(workload: str, kernel: str):
+    return profile_figure(TRACE_FILE, f"{workload}.{kernel}.mean_us")
 
 
 # BASELINE.json configs[2]: weight-GEMV microbenchmark at the Llama-3-8B layer shapes
@@ -423,12 +440,12 @@ def main() -> None:
                    "weight_bytes_per_token": gpu["weight_bytes"],
                    "token_bytes_over_hbm_peak_tok_s": HBM_PEAK_GBPS * 1e9 / gpu["weight_bytes"]},
         "roofline": {"bound": "hbm", "kernel": f"dequant-GEMV {dominant}", "achieved": d["gbps"], "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": d["gbps"] / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get((args.workload, dominant)),
-                     "traffic_source": TRAFFIC_SOURCE if (args.workload, dominant) in MEASURED_TRAFFIC else None,
-                     "profile": ({"mean_launch_us": PROFILE_KERNEL_US[(args.workload, dominant)][0],
-                                  "frac": d["bytes_per_launch"] / PROFILE_KERNEL_US[(args.workload, dominant)][0] / 1e3 / HBM_PEAK_GBPS,
-                                  "source": PROFILE_KERNEL_US[(args.workload, dominant)][1] + " (rocprofv3 --kernel-trace of the same command; not measured in this run)"}
-                                 if (args.workload, dominant) in PROFILE_KERNEL_US else None),
+                     "unit": "GB/s", "frac": d["gbps"] / HBM_PEAK_GBPS, "traffic": measured_traffic(args.workload, dominant),
+                     "traffic_source": TRAFFIC_SOURCE if measured_traffic(args.workload, dominant) is not None else None,
+                     "profile": ({"mean_launch_us": profile_kernel_us(args.workload, dominant),
+                                  "frac": d["bytes_per_launch"] / profile_kernel_us(args.workload, dominant) / 1e3 / HBM_PEAK_GBPS,
+                                  "source": TRACE_FILE + " (rocprofv3 --kernel-trace of this command with --no-graph; not measured in this run)"}
+                                 if profile_kernel_us(args.workload, dominant) else None),
                      "bytes_per_launch": d["bytes_per_launch"], "mean_launch_us": d["kernel_us"], "launches_timed": 8 * (1 if dominant == "head" else n_layer),
                      "all_gemv_gbps": gemv_bytes / gemv_us / 1e3 if gemv_us else 0.0,
                      "all_gemv_frac": gemv_bytes / gemv_us / 1e3 / HBM_PEAK_GBPS if gemv_us else 0.0,
@@ -452,9 +469,13 @@ def main() -> None:
         "model_build_s": round(gpu["build_s"], 1), "prefill_s": round(gpu["prefill_s"], 3),
         "prefill": {"tokens": w["prompt"], "tok_s": w["prompt"] / gpu["prefill_s"], "second_walk_s": round(gpu["prefill_again_s"], 4),
                     "second_walk_tok_s": w["prompt"] / gpu["prefill_again_s"],
-                    "note": "tok_s: the first walk of the prompt in the process (kernels' first launches included); second_walk: the same prompt again after a reset",
-                    "path": "blocks of up to 512 rows through the dequant-fused MFMA GEMM" if w["prompt"] >= 32
-                            else "token by token (prompts under 32 tokens)"},
+                    "second_walk_fp16_operands_s": round(gpu["prefill_fp16_s"], 4),
+                    "second_walk_fp16_operands_tok_s": w["prompt"] / gpu["prefill_fp16_s"],
+                    "note": "tok_s: the first walk of the prompt in the process (kernels' first launches included); second_walk: the same prompt "
+                            "again after a reset; fp16_operands: the same with esp_llama_set_split_activations(0), every operand rounded to fp16 once",
+                    "path": ("blocks of up to 512 rows; Q4_K: MFMA GEMM with exact integer weights and activations as hi/lo fp16 pairs (twice the "
+                             "MFMA work of the fp16-operand GEMM, logits within 2e-2 of the fp32 CPU walk at 32 layers); other formats: "
+                             "dequant-fused fp16 MFMA GEMM") if w["prompt"] >= 32 else "token by token (prompts under 32 tokens)"},
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, gpu)

@@ -132,6 +132,10 @@ def _declare_llama(L: C.CDLL) -> None:
     L.esp_llama_set_graph_replay.argtypes = [vp, i32]
     L.esp_llama_set_merged_attention.restype = i32
     L.esp_llama_set_merged_attention.argtypes = [vp, i32]
+    L.esp_matrix_resident_bytes.restype = C.c_size_t
+    L.esp_matrix_resident_bytes.argtypes = [vp]
+    L.esp_llama_resident_weight_bytes.restype = C.c_size_t
+    L.esp_llama_resident_weight_bytes.argtypes = [vp]
     L.esp_matmul_f32.restype = i32
     L.esp_matmul_f32.argtypes = [vp, vp, i32, vp, vp]
     L.esp_llama_set_split_activations.restype = i32

@@ -564,8 +564,9 @@ bool esp_interop_rope_decode(ESPSurfaceRef q, ESPSurfaceRef k, int n_heads, int 
         return false;
     const hipError_t e = launch_surface_rope(reinterpret_cast<uint16_t *>(q->device), reinterpret_cast<uint16_t *>(k->device), n_heads, n_kv_heads, head_dim,
                                              position, theta, lane_spatial, context().stream);
+    if (!finish(e, "rope_decode")) return false;   // a launch that failed wrote nothing: the surfaces keep their valid copies
     written_on_device(q); written_on_device(k);
-    return finish(e, "rope_decode");
+    return true;
 }
 
 bool esp_interop_kv_cache_scatter(ESPSurfaceRef k_src, ESPSurfaceRef v_src, ESPSurfaceRef k_cache, ESPSurfaceRef v_cache, int kv_dim, int token_index,
@@ -576,8 +577,9 @@ bool esp_interop_kv_cache_scatter(ESPSurfaceRef k_src, ESPSurfaceRef v_src, ESPS
     const hipError_t e = launch_surface_kv_scatter(reinterpret_cast<const uint16_t *>(k_src->device), reinterpret_cast<const uint16_t *>(v_src->device),
                                                    reinterpret_cast<uint16_t *>(k_cache->device), reinterpret_cast<uint16_t *>(v_cache->device), kv_dim,
                                                    token_index, cache_stride, lane_spatial, context().stream);
+    if (!finish(e, "kv_cache_scatter")) return false;
     written_on_device(k_cache); written_on_device(v_cache);
-    return finish(e, "kv_cache_scatter");
+    return true;
 }
 
 bool esp_interop_decode_sdpa(ESPSurfaceRef q, ESPSurfaceRef k_cache, ESPSurfaceRef v_cache, ESPSurfaceRef context_surface, int heads, int kv_heads, int head_dim,
@@ -590,8 +592,9 @@ bool esp_interop_decode_sdpa(ESPSurfaceRef q, ESPSurfaceRef k_cache, ESPSurfaceR
     const hipError_t e = launch_surface_sdpa(reinterpret_cast<const uint16_t *>(q->device), reinterpret_cast<const uint16_t *>(k_cache->device),
                                              reinterpret_cast<const uint16_t *>(v_cache->device), reinterpret_cast<uint16_t *>(context_surface->device), heads,
                                              kv_heads, head_dim, visible_tokens, token_base, cache_stride, lane_spatial, context().stream);
+    if (!finish(e, "decode_sdpa")) return false;
     written_on_device(context_surface);
-    return finish(e, "decode_sdpa");
+    return true;
 }
 
 // ---- the remaining surface I/O variants of ane_interop.h ----

@@ -43,6 +43,7 @@ int esp_llama_set_weight(ESPLlamaRuntime *runtime, int layer, int slot, int form
 }
 int esp_llama_finalize(ESPLlamaRuntime *runtime) { return runtime ? runtime->rt->finalize() : bad_handle(); }
 size_t esp_llama_weight_bytes(const ESPLlamaRuntime *runtime) { return runtime ? runtime->rt->weight_bytes_per_token() : 0; }
+size_t esp_llama_resident_weight_bytes(const ESPLlamaRuntime *runtime) { return runtime ? runtime->rt->resident_weight_bytes() : 0; }
 int esp_llama_reset(ESPLlamaRuntime *runtime) { return runtime ? runtime->rt->reset() : bad_handle(); }
 int esp_llama_prefill(ESPLlamaRuntime *runtime, int sequence, const uint32_t *tokens, int count) {
     if (!runtime) return bad_handle();

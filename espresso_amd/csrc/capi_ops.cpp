@@ -95,6 +95,7 @@ void esp_matrix_free(ESPMatrix *matrix) {
 }
 
 size_t esp_matrix_bytes(const ESPMatrix *matrix) { return matrix ? matrix->m.bytes() : 0; }
+size_t esp_matrix_resident_bytes(const ESPMatrix *matrix) { return matrix ? matrix->m.resident_bytes() : 0; }
 
 int esp_matrix_dequantize(const ESPMatrix *matrix, float *out) {
     if (!matrix || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "matrix_dequantize: null pointer");
@@ -114,7 +115,9 @@ int esp_matrix_dequantize(const ESPMatrix *matrix, float *out) {
 namespace {
 // More than two rows of activations go to the matrix-core kernel (fp32 matrices stay on the GEMV path).
 bool use_gemm(const DeviceMatrix &m, int batch) { return batch > 2 && m.format != FMT_F32 && m.cols % 64 == 0 && !gemv_takes_rows(m, batch); }
-constexpr size_t kGemmWorkspaceFloats = (size_t)8 << 20;   // 32 MiB of split-K partial sums
+// 16 MiB of split-K partial sums: the size of the fixed scratch of esp_gemv_device_noalloc, so that both entry points always pick
+// the same split count and add in the same order
+constexpr size_t kGemmWorkspaceFloats = kNoAllocScratchFloats;
 
 hipError_t run_matvec(const DeviceMatrix &m, const uint16_t *d_x, int batch, float *d_y, const float *d_res, float *workspace, hipStream_t s) {
     if (use_gemm(m, batch)) {

@@ -51,6 +51,7 @@ struct DeviceMatrix {
     size_t bytes() const {  // algorithmic bytes: what one GEMV must read
         return (size_t)rows * qs_row_bytes + (scales ? (size_t)rows * (cols / 32) * 2 : 0);
     }
+    size_t resident_bytes() const { return bytes() + tiled_bytes(); }   // what the matrix holds in HBM
 };
 
 // GEMV epilogues (what happens to the fp32 row sums)
@@ -168,6 +169,7 @@ hipError_t launch_split_rows(const SplitRowsParams &p, hipStream_t stream);
 // kernels/gemv.hip
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
 bool gemv_splits_activations(const DeviceMatrix &w, int batch);
+bool gemv_wants_tiled_copy(int format, int cols);
 // Slices of the prefix per query head that launch_attention_partials writes and the merging GEMV reads.
 #ifndef ESP_ATTENTION_HEAD_SPLITS
 #define ESP_ATTENTION_HEAD_SPLITS 4

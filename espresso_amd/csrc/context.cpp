@@ -90,7 +90,7 @@ int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, Devic
         e = hipMemcpyAsync(staging, gguf_blocks, src_bytes, hipMemcpyHostToDevice, c.stream);
         if (e == hipSuccess) e = launch_repack(format, staging, rows, cols, m, c.stream);
         // Q4_0 matrices of the widths the matrix-core GEMV is built for also get the tiled copy it reads
-        if (e == hipSuccess && format == FMT_Q4_0 && (cols == 4096 || cols == 14336)) {
+        if (e == hipSuccess && format == FMT_Q4_0 && gemv_wants_tiled_copy(format, cols)) {
             const size_t tiled_bytes = (size_t)((rows + 15) / 16) * (cols / 512) * 4608;
             if ((rc = device_alloc(&m.tiled, tiled_bytes)) != ESP_OK) { (void)hipFree(staging); matrix_release(&m); return rc; }
             e = launch_q40_tile(m.qs, m.scales, rows, cols, m.tiled, c.stream);
@@ -100,7 +100,7 @@ int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, Devic
     } else {
         e = hipMemcpyAsync(m.qs, gguf_blocks, src_bytes, hipMemcpyHostToDevice, c.stream);
         // Q4_K matrices of the widths the matrix-core GEMV is built for also get the tiled copy it reads
-        if (e == hipSuccess && format == FMT_Q4_K && (cols == 4096 || cols == 14336)) {
+        if (e == hipSuccess && format == FMT_Q4_K && gemv_wants_tiled_copy(format, cols)) {
             const size_t tiled_bytes = (size_t)((rows + 15) / 16) * (cols / 256) * 2304;
             if ((rc = device_alloc(&m.tiled, tiled_bytes)) != ESP_OK) { matrix_release(&m); return rc; }
             e = launch_q4k_tile(m.qs, rows, cols, m.tiled, c.stream);

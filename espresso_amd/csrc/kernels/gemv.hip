@@ -1624,6 +1624,9 @@ int q4k_mfma_waves() {
     return g_q4k_mfma_waves;
 }
 
+// widths beside 4096 and 14336 that have matrix-core instantiations (one and two activation rows)
+inline bool q4k_registry_width(int cols) { return cols == 1024 || cols == 2048 || cols == 3072 || cols == 8192; }
+
 template <int NB, int IPR, int WAVES, int KS, int MODE, bool SPLIT = false, bool STAMPS = false>
 hipError_t launch_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
     constexpr int RB = WAVES / KS, cols = IPR * 64, THREADS = WAVES * 64, NBX = SPLIT ? 2 * NB : NB;
@@ -1717,6 +1720,31 @@ hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
         if (waves == 16 && ks == 8) return launch_q4k_mfma<NB, 224, 16, 8, 0>(a, stream, launched);
         return hipSuccess;
     }
+    // The other widths of the reference's model registry (Sources/ModelSupport/ModelRegistry.swift:59-107: llama3.2-1B d 2048, llama3.2-3B
+    // d 3072, both FFN 8192; Qwen3-0.6B d 1024, FFN 3072), one and two activation rows: a wavefront takes one super-block column per step
+    // at the model widths (all wavefronts of a workgroup share a row block), two at 8192 columns.  No tuning variants.
+    if constexpr (NB <= 2) {
+        if (waves != 0 || ks != 0) return hipSuccess;
+#define ESP_MFMA_WIDTH(COLS_, W_)                                                                                   \
+        if (a.cols == COLS_) {                                                                                     \
+            if (a.split_x) {                                                                                       \
+                if (mode == 0) return launch_q4k_mfma<NB, COLS_ / 64, W_, W_, 0, true>(a, stream, launched);       \
+                if (mode == 1) return launch_q4k_mfma<NB, COLS_ / 64, W_, W_, 1, true>(a, stream, launched);       \
+                return launch_q4k_mfma<NB, COLS_ / 64, W_, W_, 2, true>(a, stream, launched);                      \
+            }                                                                                                      \
+            if (mode == 0) return launch_q4k_mfma<NB, COLS_ / 64, W_, W_, 0>(a, stream, launched);                 \
+            if (mode == 1) return launch_q4k_mfma<NB, COLS_ / 64, W_, W_, 1>(a, stream, launched);                 \
+            return launch_q4k_mfma<NB, COLS_ / 64, W_, W_, 2>(a, stream, launched);                                \
+        }
+        ESP_MFMA_WIDTH(1024, 4)
+        ESP_MFMA_WIDTH(2048, 8)
+        ESP_MFMA_WIDTH(3072, 12)
+#undef ESP_MFMA_WIDTH
+        if (a.cols == 8192 && mode == 0) {
+            if (a.split_x) return launch_q4k_mfma<NB, 128, 16, 16, 0, true>(a, stream, launched);
+            return launch_q4k_mfma<NB, 128, 16, 16, 0>(a, stream, launched);
+        }
+    }
     return hipSuccess;
 }
 
@@ -1729,7 +1757,7 @@ hipError_t launch_q4k(const KernelArgs &a, hipStream_t stream) {
     // columns, 4096 rows, one row, in the 8B decode step: 8.3 us on the matrix cores with three steps in flight, 9.3 us on the
     // eight-wavefront dot-product kernel below, which "q4k_long_row_waves" = 8 or 4 selects).
     const bool one_row_on_the_matrix_cores = (a.cols == 4096 && (q4k_mfma_max_rows() <= 0 || a.rows <= q4k_mfma_max_rows())) ||
-                                             (a.cols == 14336 && q4k_long_row_waves() == 0);
+                                             (a.cols == 14336 && q4k_long_row_waves() == 0) || q4k_registry_width(a.cols);
     if (q4k_mfma_mode() == 1 || (q4k_mfma_mode() < 0 && (B >= 2 || one_row_on_the_matrix_cores))) {
         bool launched = false;
         const hipError_t e = try_q4k_mfma<B>(a, stream, &launched);
@@ -1925,6 +1953,16 @@ bool gemv_splits_activations(const DeviceMatrix &w, int batch) {
     if (q4k_mfma_waves() != 0 || q4k_mfma_split() != 0) return false;   // tuning overrides: not every variant has a split form
     if (w.cols == 4096) return batch >= 2 || q4k_mfma_mode() == 1 || q4k_mfma_max_rows() <= 0 || w.rows <= q4k_mfma_max_rows();
     if (w.cols == 14336) return batch >= 2 || q4k_mfma_mode() == 1 || q4k_long_row_waves() == 0;
+    return q4k_registry_width(w.cols) && w.rows <= 32768;   // taller matrices would need more rounds than the kernel's LDS slots
+}
+
+// Which matrices get the tiled copy the matrix-core GEMVs read, at upload (ESPRESSO_HIP_TILED_COPIES=0: none, the dot-product
+// kernels run everywhere and resident weight memory is the packed size).
+bool gemv_wants_tiled_copy(int format, int cols) {
+    static const int enabled = env_int("ESPRESSO_HIP_TILED_COPIES", 1);
+    if (!enabled) return false;
+    if (format == FMT_Q4_K) return cols == 4096 || cols == 14336 || q4k_registry_width(cols);
+    if (format == FMT_Q4_0) return cols == 4096 || cols == 14336;
     return false;
 }
 
@@ -1939,7 +1977,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     if ((p.epilogue == EPI_STORE_F32 || p.epilogue == EPI_ADD_RESIDUAL) && !p.y) return hipErrorInvalidValue;
     if (p.epilogue == EPI_ADD_RESIDUAL && !p.residual) return hipErrorInvalidValue;
     if (p.epilogue == EPI_SWIGLU_F16 && (!p.out_f16 || w.rows % 2 != 0)) return hipErrorInvalidValue;
-    if (p.split_x && (!gemv_splits_activations(w, p.batch) || (w.cols == 14336 && (p.norm_x || p.merge_partials)))) return hipErrorInvalidValue;
+    if (p.split_x && (!gemv_splits_activations(w, p.batch) || ((w.cols == 14336 || w.cols == 8192) && (p.norm_x || p.merge_partials)))) return hipErrorInvalidValue;
     if (p.split_out && (p.epilogue != EPI_SWIGLU_F16 || p.batch > 2)) return hipErrorInvalidValue;
     if (p.epilogue == EPI_ARGMAX && (!p.argmax_value || !p.argmax_index || p.argmax_capacity <= 0 || p.batch > 2 || !gemv_supports_argmax(w)))
         return hipErrorInvalidValue;

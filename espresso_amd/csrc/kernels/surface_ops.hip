@@ -136,8 +136,9 @@ hipError_t launch_surface_kv_scatter(const uint16_t *k_src, const uint16_t *v_sr
 }
 hipError_t launch_surface_sdpa(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *context, int heads, int kv_heads, int head_dim,
                                int visible_tokens, int token_base, int cache_stride, int lane_stride, hipStream_t s) {
+    // one score per visible token in LDS: up to 48 KB without raising the kernel's limit, i.e. 12032 tokens
     const size_t lds = ((size_t)visible_tokens + 256) * 4;
-    if (lds > 64 * 1024) return hipErrorInvalidValue;
+    if (lds > 48 * 1024) return hipErrorInvalidValue;
     hipLaunchKernelGGL(surface_sdpa_kernel, dim3(heads), dim3(256), lds, s, q, k_cache, v_cache, context, heads, kv_heads, head_dim, visible_tokens, token_base,
                        cache_stride, lane_stride);
     return hipGetLastError();

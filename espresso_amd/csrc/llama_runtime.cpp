@@ -309,6 +309,7 @@ int LlamaRuntime::finalize() {
     if (h_lm_head_.format < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "finalize: missing lm_head");
     if ((rc = matrix_upload(h_lm_head_.format, h_lm_head_.bytes.data(), c_.vocab, d, &lm_head_)) != ESP_OK) return rc;
     weight_bytes_ = lm_head_.bytes();
+    resident_weight_bytes_ = lm_head_.resident_bytes() + h_embedding_.bytes.size();
 
     // ---- layers ----
     layers_.resize(c_.n_layer);
@@ -362,6 +363,7 @@ int LlamaRuntime::finalize() {
         if ((rc = matrix_upload(H.wo.format, H.wo.bytes.data(), d, ad, &L.wo)) != ESP_OK) return rc;
         if ((rc = matrix_upload(H.w2.format, H.w2.bytes.data(), d, hd, &L.w2)) != ESP_OK) return rc;
         weight_bytes_ += L.wqkv.bytes() + L.wo.bytes() + L.w13.bytes() + L.w2.bytes();
+        resident_weight_bytes_ += L.wqkv.resident_bytes() + L.wo.resident_bytes() + L.w13.resident_bytes() + L.w2.resident_bytes();
         uint8_t *kc = nullptr, *vc = nullptr;
         if ((rc = device_alloc(&kc, cache_bytes)) != ESP_OK) return rc;
         L.k_cache = kc;

@@ -94,6 +94,8 @@ class LlamaRuntime {
     int read_logits(int seq, float *out);         // runs the head on the kept hidden state
 
     size_t weight_bytes_per_token() const { return weight_bytes_; }
+    // what the weights hold in HBM: the packed matrices, the tiled copies the matrix-core GEMVs read beside them, the embedding table
+    size_t resident_weight_bytes() const { return resident_weight_bytes_; }
 
     // Steps whose rows (token, position, sequence) already sit in the device arrays below: generation loops that keep
     // their decisions on the device enqueue these, also under stream capture.  Nothing here synchronises.
@@ -168,7 +170,7 @@ class LlamaRuntime {
     int enqueue_layers_split(int rows);
     int *d_tokens_ = nullptr, *d_pos_ = nullptr, *d_seq_ = nullptr, *d_out_tokens_ = nullptr;
     std::vector<int> visible_;
-    size_t weight_bytes_ = 0;
+    size_t weight_bytes_ = 0, resident_weight_bytes_ = 0;
     // captured greedy step per sequence (head -> feed -> trunk -> keep), and its device-side state
     bool use_graph_ = true;
     std::vector<hipGraphExec_t> step_graphs_, multi_graphs_;   // one step, kStepsPerGraph steps

@@ -79,6 +79,10 @@ class LlamaRuntime:
     def weight_bytes(self) -> int:
         return int(self._L.esp_llama_weight_bytes(self._h))
 
+    @property
+    def resident_weight_bytes(self) -> int:
+        return int(self._L.esp_llama_resident_weight_bytes(self._h))
+
     def reset(self) -> None:
         _lib.check(self._L.esp_llama_reset(self._h))
 

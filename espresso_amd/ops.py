@@ -65,6 +65,10 @@ class Matrix:
     def bytes(self) -> int:
         return int(_lib.load_library().esp_matrix_bytes(self._h))
 
+    @property
+    def resident_bytes(self) -> int:
+        return int(_lib.load_library().esp_matrix_resident_bytes(self._h))
+
     def dequantize(self) -> np.ndarray:
         out = np.empty(self.rows * self.cols, dtype=np.float32)
         _lib.check(_lib.load_library().esp_matrix_dequantize(self._h, _ptr(out)))

@@ -69,6 +69,10 @@ ESPMatrix *esp_matrix_create(int format, const void *gguf_blocks, int rows, int 
 void esp_matrix_free(ESPMatrix *matrix);
 /* Bytes one GEMV must read from HBM for this matrix (packed weights incl. scales). */
 size_t esp_matrix_bytes(const ESPMatrix *matrix);
+/* Bytes the matrix holds in HBM: the packed weights plus, for the Q4_K / Q4_0 widths the matrix-core GEMVs are built for (Q4_K:
+ * 1024, 2048, 3072, 4096, 8192, 14336 columns; Q4_0: 4096, 14336), a second copy tiled for those kernels (about as large again).
+ * ESPRESSO_HIP_TILED_COPIES=0 in the environment keeps matrices at their packed size; the dot-product GEMVs then run everywhere. */
+size_t esp_matrix_resident_bytes(const ESPMatrix *matrix);
 /* Decode the resident copy back to fp32 [rows*cols] (checks the HBM layout carries the same bits). */
 int esp_matrix_dequantize(const ESPMatrix *matrix, float *out);
 
@@ -86,12 +90,14 @@ int esp_gemv(const ESPMatrix *matrix, const uint16_t *x_f16, int batch, float *y
  * (hi = fp16(v), lo = fp16((v - hi) * 2048)) and each weight as the exact integer sc * q of its sub-block, with d, dmin and the
  * sub-block minimums applied in fp32, so no operand is rounded. */
 int esp_matmul_f32(const ESPMatrix *matrix, const float *x, int rows, float *y, const float *residual);
-/* esp_gemv for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc).  No counterpart in the reference.  x, y and residual are DEVICE pointers
+/* esp_gemv for callers that cannot allocate device memory (tight serving loops, harnesses that forbid hipMalloc, code that runs
+ * between the captures of its own HIP graphs).  No counterpart in the reference.  x, y and residual are DEVICE pointers
  * (fp16 [batch][cols], fp32 [batch][rows], fp32 [batch][rows] or NULL); the call makes no hipMalloc / hipFree: the
  * split-K partial sums of the matrix-core kernels (batch > 2) live in a fixed 16 MiB array inside the library, one
- * copy per GPU, held until the process ends.  Limits: batch 1..64 and, for batch > 2, 2 * batch * rows <= 4 Mi floats;
- * beyond them the call fails with ESP_ERR_OUT_OF_RANGE.  Synchronous like esp_gemv.  All calls on a GPU share that
+ * copy per GPU, held until the process ends.  Limits: batch 1..64 and, for batch > 2, 2 * batch * rows <= 4 Mi floats
+ * (whether or not the kernel ends up splitting K); beyond them the call fails with ESP_ERR_OUT_OF_RANGE.  It runs on the
+ * library's stream and returns when the result is there, like esp_gemv, so it cannot itself sit inside a caller's stream
+ * capture.  esp_gemv sizes its own workspace the same, so the two return the same bits.  All calls on a GPU share that
  * GPU's array: calls that overlap on one GPU race. */
 int esp_gemv_device_noalloc(const ESPMatrix *matrix, const uint16_t *x_f16_device, int batch, float *y_device,
                             const float *residual_device_or_null);
@@ -156,6 +162,8 @@ int esp_llama_set_weight(ESPLlamaRuntime *runtime, int layer, int slot, int form
 int esp_llama_finalize(ESPLlamaRuntime *runtime);
 /* Packed weight bytes one decoded token reads (all projections plus lm_head). */
 size_t esp_llama_weight_bytes(const ESPLlamaRuntime *runtime);
+/* Bytes the weights hold in HBM (packed matrices, their tiled copies, the embedding table): see esp_matrix_resident_bytes. */
+size_t esp_llama_resident_weight_bytes(const ESPLlamaRuntime *runtime);
 int esp_llama_reset(ESPLlamaRuntime *runtime);
 int esp_llama_prefill(ESPLlamaRuntime *runtime, int sequence, const uint32_t *tokens, int count);
 int esp_llama_advance(ESPLlamaRuntime *runtime, int sequence, uint32_t token);
@@ -591,7 +599,11 @@ bool esp_interop_rebind_input(ESPHandle *handle, int index, ESPSurfaceRef new_su
  *   rope_decode       :1756-1795  half-split RoPE in place on lane 0 of q [heads*D, S] and k [kvHeads*D, S]
  *   kv_cache_scatter  :1805-1820  lane 0 of k / v into column token_index of the caches [kvDim, cacheStride]
  *   decode_sdpa       :1824-1886  fused_decode_sdpa: softmax(q K / sqrt(D)) V over columns token_base .. +visible of the caches into
- *                                 lane 0 of the context surface [heads*D, S] (fp16; kvHead = head / (heads / kvHeads)) */
+ *                                 lane 0 of the context surface [heads*D, S] (fp16; kvHead = head / (heads / kvHeads), the
+ *                                 reference's groupedContiguous mapping, :146-153; its moduloInterleaved mapping is not offered;
+ *                                 at most 12032 visible tokens; the reference keeps this context in an fp32 buffer, there is no
+ *                                 vector of it in the reference's tests to compare the fp16 rounding with)
+ * A call that fails leaves every surface as it was. */
 bool esp_interop_rope_decode(ESPSurfaceRef q, ESPSurfaceRef k, int n_heads, int n_kv_heads, int head_dim, int position, float theta, int lane_spatial);
 bool esp_interop_kv_cache_scatter(ESPSurfaceRef k_src, ESPSurfaceRef v_src, ESPSurfaceRef k_cache, ESPSurfaceRef v_cache, int kv_dim, int token_index,
                                   int cache_stride, int lane_spatial);

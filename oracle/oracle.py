@@ -383,3 +383,28 @@ def generate_two_token(full: LlamaRuntime, draft: LlamaRuntime, prompt, max_toke
         raise RuntimeError(f"oracle two-token generate failed: {n}")
     return out[:n].tolist(), {"passes": st.passes, "committed_total": st.committed_total,
                               "accepted_total": st.accepted_total}
+
+
+def runtime_from_packed(cfg, packed, fmt, n_layer, kv_fp16, max_seq, gemv_inputs_fp16=True):
+    """An oracle runtime over a model given as GGUF blocks (the dict espresso_amd.synthetic.build_runtime(keep_packed=True) returns:
+    embedding fp16, lm_head and per-layer wq..w3 in `fmt`; norm weights one), dequantised inside the oracle.  `cfg` carries the
+    shape (n_head, n_kv_head, d_model, head_dim, hidden_dim, vocab, norm_eps, rope_theta and the derived attention_dim, kv_dim)."""
+    ocfg = LlamaConfig(n_layer=n_layer, n_head=cfg.n_head, n_kv_head=cfg.n_kv_head, d_model=cfg.d_model, head_dim=cfg.head_dim,
+                       hidden_dim=cfg.hidden_dim, vocab=cfg.vocab, max_seq=max_seq, norm_eps=cfg.norm_eps, rope_theta=cfg.rope_theta,
+                       gemv_inputs_fp16=gemv_inputs_fp16, kv_fp16=kv_fp16)
+    shapes = {"wq": (cfg.attention_dim, cfg.d_model), "wk": (cfg.kv_dim, cfg.d_model), "wv": (cfg.kv_dim, cfg.d_model),
+              "wo": (cfg.d_model, cfg.attention_dim), "w1": (cfg.hidden_dim, cfg.d_model), "w3": (cfg.hidden_dim, cfg.d_model),
+              "w2": (cfg.d_model, cfg.hidden_dim)}
+    slot = {"wq": W_WQ, "wk": W_WK, "wv": W_WV, "wo": W_WO, "w1": W_W1, "w2": W_W2, "w3": W_W3}
+    rt = LlamaRuntime(ocfg)
+    n = cfg.vocab * cfg.d_model
+    rt.set_weight_blocks(0, W_TOKEN_EMBEDDING, FMT_F16, packed["embedding"], n)
+    rt.set_weight(0, W_FINAL_NORM, np.ones(cfg.d_model, np.float32))
+    rt.set_weight_blocks(0, W_LM_HEAD, fmt, packed["lm_head"], n)
+    for l in range(n_layer):
+        rt.set_weight(l, W_RMS_ATT, np.ones(cfg.d_model, np.float32))
+        rt.set_weight(l, W_RMS_FFN, np.ones(cfg.d_model, np.float32))
+        for k, sl in slot.items():
+            r, c = shapes[k]
+            rt.set_weight_blocks(l, sl, fmt, packed["layers"][l][k], r * c)
+    return rt

@@ -64,26 +64,7 @@ def test_full_size_weight_gemv_matches_oracle(mods, name, rows, cols):
     mat.close()
 
 
-def oracle_from_packed(cfg, packed, fmt, n_layer, kv_fp16, max_seq, gemv_inputs_fp16=True):
-    ocfg = orc.LlamaConfig(n_layer=n_layer, n_head=cfg.n_head, n_kv_head=cfg.n_kv_head, d_model=cfg.d_model, head_dim=cfg.head_dim,
-                           hidden_dim=cfg.hidden_dim, vocab=cfg.vocab, max_seq=max_seq, norm_eps=cfg.norm_eps, rope_theta=cfg.rope_theta,
-                           gemv_inputs_fp16=gemv_inputs_fp16, kv_fp16=kv_fp16)
-    shapes = {"wq": (cfg.attention_dim, cfg.d_model), "wk": (cfg.kv_dim, cfg.d_model), "wv": (cfg.kv_dim, cfg.d_model),
-              "wo": (cfg.d_model, cfg.attention_dim), "w1": (cfg.hidden_dim, cfg.d_model), "w3": (cfg.hidden_dim, cfg.d_model),
-              "w2": (cfg.d_model, cfg.hidden_dim)}
-    slot = {"wq": orc.W_WQ, "wk": orc.W_WK, "wv": orc.W_WV, "wo": orc.W_WO, "w1": orc.W_W1, "w2": orc.W_W2, "w3": orc.W_W3}
-    rt = orc.LlamaRuntime(ocfg)
-    n = cfg.vocab * cfg.d_model
-    rt.set_weight_blocks(0, orc.W_TOKEN_EMBEDDING, orc.FMT_F16, packed["embedding"], n)
-    rt.set_weight(0, orc.W_FINAL_NORM, np.ones(cfg.d_model, np.float32))
-    rt.set_weight_blocks(0, orc.W_LM_HEAD, fmt, packed["lm_head"], n)
-    for l in range(n_layer):
-        rt.set_weight(l, orc.W_RMS_ATT, np.ones(cfg.d_model, np.float32))
-        rt.set_weight(l, orc.W_RMS_FFN, np.ones(cfg.d_model, np.float32))
-        for k, s in slot.items():
-            r, c = shapes[k]
-            rt.set_weight_blocks(l, s, fmt, packed["layers"][l][k], r * c)
-    return rt
+oracle_from_packed = orc.runtime_from_packed
 
 
 def test_8b_shaped_layer_and_head_match_oracle(mods):

@@ -20,7 +20,10 @@ def llama():
 
 
 def make_pair(ll, cfg_kw, fmt, seed, std=0.02, kv_fp16=False, norm_jitter=0.0, qk_norm=False):
-    ocfg = orc.LlamaConfig(gemv_inputs_fp16=True, kv_fp16=kv_fp16, **cfg_kw)
+    # Q4_K models at the widths the matrix-core GEMV is built for feed their activations as hi / lo fp16 pairs: their oracle is the
+    # reference's default arithmetic (fp32 activations); every other kernel rounds activations to fp16 once, as the oracle's other mode does
+    split = fmt == orc.FMT_Q4_K and cfg_kw["d_model"] in (1024, 2048, 3072, 4096)
+    ocfg = orc.LlamaConfig(gemv_inputs_fp16=not split, kv_fp16=kv_fp16, **cfg_kw)
     w = mu.random_weights(ocfg, seed, std=std, norm_jitter=norm_jitter)
     if qk_norm:
         rng = np.random.default_rng(seed + 1)

@@ -63,6 +63,71 @@ def test_matches_oracle_and_dot_product_kernels(mods, rows, cols):
     mat.close()
 
 
+# the other widths of the reference's model registry (ModelRegistry.swift:59-107): llama3.2-1B d 2048 / FFN 8192, llama3.2-3B d 3072,
+# Qwen3-0.6B d 1024 / FFN 3072; ragged row counts included
+@pytest.mark.parametrize("rows,cols", [(2048, 1024), (1000, 1024), (6144, 1024), (2048, 2048), (16384, 2048), (3072, 3072), (1024, 3072),
+                                       (2048, 8192), (3072, 8192), (40, 8192)])
+def test_registry_widths_on_the_matrix_cores(mods, rows, cols):
+    ll, ops, syn = mods
+    mat, deq = q4k_matrix(ops, rows, cols, rows + cols)
+    assert mat.resident_bytes > mat.bytes            # the tiled copy exists: these widths run on the matrix cores
+    rng = np.random.default_rng(rows + 1)
+    scale = np.abs(deq).max() * np.sqrt(cols)
+    for batch in (1, 2):
+        x = rng.normal(0, 1, (batch, cols)).astype(np.float16)
+        res = rng.normal(0, 1, (batch, rows)).astype(np.float32)
+        want = np.stack([orc.matvec(deq, x[b].astype(np.float32)) for b in range(batch)])
+        ops.set_tuning("q4k_mfma", 0)
+        base = mat.gemv(x)
+        ops.set_tuning("q4k_mfma", -1)
+        y = mat.gemv(x)
+        assert np.abs(y - want).max() <= 2e-5 * scale + 1e-6, (batch, np.abs(y - want).max())
+        assert np.abs(y - base).max() <= 2e-5 * scale + 1e-6
+        assert np.array_equal(mat.gemv(x).view(np.uint32), y.view(np.uint32))
+        assert np.abs(mat.gemv(x, res) - (want + res)).max() <= 2e-5 * scale + 1e-5
+    for j in (0, 31, 255, 256, cols - 1):
+        x = np.zeros((2, cols), np.float16)
+        x[0, j] = 1.0; x[1, cols - 1 - j] = -2.0
+        y = mat.gemv(x)
+        assert np.abs(y[0] - deq[:, j]).max() <= 1e-6 * max(1.0, np.abs(deq[:, j]).max()) + 1e-7
+        assert np.abs(y[1] + 2.0 * deq[:, cols - 1 - j]).max() <= 2e-6 * max(1.0, np.abs(deq[:, j]).max()) + 1e-7
+    mat.close()
+
+
+@pytest.mark.parametrize("name,shape", [
+    ("llama3.2-1b width", dict(n_head=32, n_kv_head=8, d_model=2048, head_dim=64, hidden_dim=8192)),
+    ("llama3.2-3b width", dict(n_head=24, n_kv_head=8, d_model=3072, head_dim=128, hidden_dim=8192)),
+    ("qwen3-0.6b width", dict(n_head=16, n_kv_head=8, d_model=1024, head_dim=128, hidden_dim=3072)),
+])
+def test_registry_width_decoders_match_oracle(mods, name, shape):
+    """Two layers at each registry width, Q4_K, fp16 KV: fused-norm, merge and SwiGLU forms of the matrix-core GEMV with split
+    activations against the oracle in the reference's default arithmetic, then graph replay against the eager steps."""
+    from test_gpu_full_size import oracle_from_packed
+    ll, ops, syn = mods
+    cfg = ll.MultiModelConfig(**dict(shape, n_layer=2, vocab=4096, max_seq=64, norm_eps=1e-5, rope_theta=500000.0, name=name))
+    g, packed = syn.build_runtime(cfg, orc.FMT_Q4_K, seed=31, kv_format=orc.FMT_F16, keep_packed=True)
+    assert g.resident_weight_bytes > g.weight_bytes
+    o = oracle_from_packed(cfg, packed, orc.FMT_Q4_K, 2, True, 64, gemv_inputs_fp16=False)
+    prompt = [1, 4000, 777, 2048, 5, 902, 3133, 2]
+    o.prefill(prompt)
+    g.prefill(np.asarray(prompt, np.uint32))
+    worst = 0.0
+    for step in range(6):
+        ho, hg = o.last_hidden(), g.last_hidden()
+        assert np.abs(ho - hg).max() <= 1e-3 * max(1.0, np.abs(ho).max())
+        worst = max(worst, float(np.abs(o.logits() - g.logits()).max()))
+        tok = o.select_greedy()
+        if o.top2_margin() > 1e-3:
+            assert g.select_greedy() == tok
+        o.advance(tok); g.advance(tok)
+    print(f"{name}: worst logit difference over 6 steps {worst:.3e}")
+    assert worst <= 2e-3
+    plain = g.generate(prompt, 20)[0]
+    ll.set_graph_replay(g, False)
+    assert g.generate(prompt, 20)[0] == plain
+    g.close()
+
+
 @pytest.mark.parametrize("waves,ks", [(0, 0), (4, 1), (16, 16)])
 def test_decoder_with_matrix_core_gemvs_matches_oracle(mods, waves, ks):
     """One layer of the 8B shape: fused RMSNorm staging, RoPE / KV-write, SwiGLU and residual epilogues, attention states merged
