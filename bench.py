@@ -200,7 +200,7 @@ def run_microbench(shapes=None, formats=("q4_k", "q4_0"), batches=(1, 2, 4, 8), 
                                  "gbps": round(nbytes / t["mean_us"] / 1e3, 1), "frac_hbm_peak": round(nbytes / t["mean_us"] / 1e3 / HBM_PEAK_GBPS, 3),
                                  "bytes": nbytes})
             m.close()
-    return {"metric": "dequant-GEMV HBM GB/s (Llama-3-8B layer shapes)", "unit": "GB/s", "n_gpus": 1, "data": "synthetic",
+    return {"metric": "dequant-GEMV HBM GB/s", "unit": "GB/s", "n_gpus": 1, "data": "synthetic",
             "how": f"mean of {launches} back-to-back launches between two HIP events after 10 warm-up launches; weights rotate "
                    "through copies totalling > 600 MB so every launch reads HBM; each mean includes the ~4 us a dependent launch costs",
             "results": rows_out}
@@ -501,6 +501,10 @@ def main() -> None:
             secondary[other] = sec
         # BASELINE.json configs[2] (the two largest shapes; --microbench prints all four) and configs[4]
         secondary["gemv_microbench"] = run_microbench(shapes=[(14336, 4096), (4096, 14336)], launches=50)
+        # BASELINE.json configs[1]: the 6-layer model's isolated Q8_0 shapes at batch 1 and 2 (the small ones fit the memory-side cache
+        # even when rotated, and are launch-bound: about 3 us per dependent launch whatever they read)
+        secondary["gemv_microbench_q8_0"] = run_microbench(shapes=[(768, 768), (2048, 768), (768, 2048), (32000, 768)], formats=("q8_0",),
+                                                           batches=(1, 2), launches=50)
         secondary["two_token"] = run_two_token(240)
         secondary["two_token_8b"] = run_two_token_8b(240)
         result["secondary"] = secondary

@@ -45,6 +45,7 @@ struct DeviceMatrix {
     uint8_t *tiled = nullptr;
     size_t tiled_bytes() const {
         if (!tiled) return 0;
+        if (format == FMT_Q8_0) return (size_t)((rows + 15) / 16) * (cols / 256) * 4352;
         return format == FMT_Q4_K ? (size_t)((rows + 15) / 16) * (cols / 256) * 2304 : (size_t)((rows + 15) / 16) * (cols / 512) * 4608;
     }
     size_t qs_row_bytes = 0;
@@ -170,6 +171,7 @@ hipError_t launch_split_rows(const SplitRowsParams &p, hipStream_t stream);
 hipError_t launch_gemv(const GemvParams &p, hipStream_t stream);
 bool gemv_splits_activations(const DeviceMatrix &w, int batch);
 bool gemv_wants_tiled_copy(int format, int cols);
+unsigned gemv_tuning_epoch();   // bumped by every gemv_set_tuning call
 // Slices of the prefix per query head that launch_attention_partials writes and the merging GEMV reads.
 #ifndef ESP_ATTENTION_HEAD_SPLITS
 #define ESP_ATTENTION_HEAD_SPLITS 4
@@ -196,6 +198,8 @@ hipError_t launch_repack(int format, const uint8_t *blocks, int rows, int cols, 
 hipError_t launch_q4k_tile(const uint8_t *blocks, int rows, int cols, uint8_t *tiled, hipStream_t stream);
 // Q4_0 planes -> the tiled copy ((rows + 15) / 16 * cols / 512 tiles of 4608 bytes)
 hipError_t launch_q40_tile(const uint8_t *qs, const uint16_t *scales, int rows, int cols, uint8_t *tiled, hipStream_t stream);
+// Q8_0 planes -> the tiled copy ((rows + 15) / 16 * cols / 256 tiles of 4352 bytes)
+hipError_t launch_q80_tile(const uint8_t *qs, const uint16_t *scales, int rows, int cols, uint8_t *tiled, hipStream_t stream);
 // DeviceMatrix -> fp32 [rows][cols] (used to check the planes carry the same bits)
 hipError_t launch_dequant_matrix(const DeviceMatrix &m, float *out, hipStream_t stream);
 

@@ -95,6 +95,11 @@ int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, Devic
             if ((rc = device_alloc(&m.tiled, tiled_bytes)) != ESP_OK) { (void)hipFree(staging); matrix_release(&m); return rc; }
             e = launch_q40_tile(m.qs, m.scales, rows, cols, m.tiled, c.stream);
         }
+        if (e == hipSuccess && format == FMT_Q8_0 && gemv_wants_tiled_copy(format, cols)) {
+            const size_t tiled_bytes = (size_t)((rows + 15) / 16) * (cols / 256) * 4352;
+            if ((rc = device_alloc(&m.tiled, tiled_bytes)) != ESP_OK) { (void)hipFree(staging); matrix_release(&m); return rc; }
+            e = launch_q80_tile(m.qs, m.scales, rows, cols, m.tiled, c.stream);
+        }
         if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
         (void)hipFree(staging);
     } else {

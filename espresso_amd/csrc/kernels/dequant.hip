@@ -154,6 +154,33 @@ __global__ void q40_tile_kernel(const uint8_t *qs, const uint16_t *scales, int r
     }
 }
 
+// Q8_0 planes -> the tiled copy of the matrix-core GEMV: tile (rb, t) = sixteen rows x 256 columns = [j][half][lane] 16 bytes of
+// quants (lane (n, g) = g * 16 + n owns block 8 t + 4 j + g of row n; half = its first or last sixteen bytes), then [lane][j] fp16
+// scales.  320 threads per tile; rows past the matrix are zero blocks with zero scales.
+__global__ void q80_tile_kernel(const uint8_t *qs, const uint16_t *scales, int rows, int tpr, size_t tiles, uint8_t *tiled) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t tile = i / 320;
+    if (tile >= tiles) return;
+    const int p = (int)(i - tile * 320);
+    const int rb = (int)(tile / tpr), t = (int)(tile - (size_t)rb * tpr);
+    uint8_t *dst = tiled + tile * 4352;
+    const int blocks_per_row = tpr * 8;
+    if (p < 256) {
+        const int j = p >> 7, half = (p >> 6) & 1, lane = p & 63, g = lane >> 4, n = lane & 15, row = rb * 16 + n;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (row < rows) v = *reinterpret_cast<const uint4 *>(qs + ((size_t)row * blocks_per_row + 8 * t + 4 * j + g) * 32 + 16 * half);
+        *reinterpret_cast<uint4 *>(dst + 1024 * (2 * j + half) + 16 * lane) = v;
+    } else {
+        const int lane = p - 256, g = lane >> 4, n = lane & 15, row = rb * 16 + n;
+        unsigned d0 = 0, d1 = 0;
+        if (row < rows) {
+            d0 = scales[(size_t)row * blocks_per_row + 8 * t + g];
+            d1 = scales[(size_t)row * blocks_per_row + 8 * t + 4 + g];
+        }
+        *reinterpret_cast<unsigned *>(dst + 4096 + 4 * lane) = d0 | (d1 << 16);
+    }
+}
+
 inline dim3 grid_for(size_t n, int threads) { return dim3((unsigned)((n + threads - 1) / threads)); }
 
 }  // namespace
@@ -211,6 +238,14 @@ hipError_t launch_q40_tile(const uint8_t *qs, const uint16_t *scales, int rows, 
     const int tpr = cols / 512;
     const size_t tiles = (size_t)((rows + 15) / 16) * tpr;
     hipLaunchKernelGGL(q40_tile_kernel, grid_for(tiles * 320, 320), dim3(320), 0, stream, qs, scales, rows, tpr, tiles, tiled);
+    return hipGetLastError();
+}
+
+hipError_t launch_q80_tile(const uint8_t *qs, const uint16_t *scales, int rows, int cols, uint8_t *tiled, hipStream_t stream) {
+    if (!qs || !scales || !tiled || rows <= 0 || cols <= 0 || cols % 256 != 0) return hipErrorInvalidValue;
+    const int tpr = cols / 256;
+    const size_t tiles = (size_t)((rows + 15) / 16) * tpr;
+    hipLaunchKernelGGL(q80_tile_kernel, grid_for(tiles * 320, 320), dim3(320), 0, stream, qs, scales, rows, tpr, tiles, tiled);
     return hipGetLastError();
 }
 

@@ -1515,6 +1515,186 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t
     }
 }
 
+// ---- Q8_0 on the matrix cores ---------------------------------------------------------------------------------------------------
+// The same scheme for Q8_0's 32-byte blocks with one fp16 scale.  The tiled copy holds, per (sixteen rows, 256 columns), four
+// kilobytes of quants as [j][half][lane] 16 bytes (lane (n, g) owns blocks 4 j + g, j = 0, 1, of row n; half = its first or last
+// sixteen bytes) and then [lane][j] fp16 scales: four contiguous 1 KB loads and one of 256 bytes per wavefront and tile.  A signed
+// byte b becomes the fp16 number 1152 + b without arithmetic (v_perm puts b ^ 0x80 under the exponent byte 0x64: 1024 + 128 + b,
+// exact), two bytes per v_perm; the four MFMAs of a block share its scale and one accumulator, and w = d b folds as
+// d (acc - 1152 Sx) with Sx the sum of the block's activations, staged beside them.  Exact products, fp32 sums.
+constexpr size_t kQ80TileBytes = 4352;
+constexpr int kQ80Rounds = 8;   // rounds whose partial sums have an LDS slot of their own (KS > 1)
+struct Q80Item { uint4 q[4]; u32 d; };
+
+template <int NB, int TPR, int WAVES, int KS, int MODE>
+__global__ __launch_bounds__(WAVES * 64) void gemv_q80_mfma_kernel(const uint8_t *tiled, const void *activations, const float *norm_w, int rows, int iters,
+                                                                   int workgroups, float norm_eps, KernelArgs rest) {
+    KernelArgs a = rest;
+    a.rows = rows;
+    if constexpr (MODE == 1) { a.norm_x = static_cast<const float *>(activations); a.norm_w = norm_w; a.norm_eps = norm_eps; }
+    else if constexpr (MODE == 2) a.merge_partials = static_cast<const float *>(activations);
+    else a.x = static_cast<const uint16_t *>(activations);
+    constexpr int THREADS = WAVES * 64, cols = TPR * 256, IPR = cols / 64, S = TPR / KS, RB = WAVES / KS, GROUPS = cols / 8;
+    constexpr int DEPTH = S % 4 == 0 ? 4 : (S % 2 == 0 ? 2 : 1);   // divides S: a step's slot in the ring is a constant
+    static_assert(TPR % KS == 0 && WAVES % KS == 0 && NB >= 1 && NB <= 4, "whole tiles per wavefront, one set of A slots");
+    extern __shared__ uint4 smem_raw[];
+    uint4 *xs4 = smem_raw;                                        // [NB][GROUPS] groups of eight fp16, (0,2,1,3) order inside fours
+    uint4 *zero4 = xs4 + (size_t)NB * GROUPS;                     // eight groups of zeros
+    float *xsum = reinterpret_cast<float *>(zero4 + 8);           // [NB][cols / 32]: the sum of every block's activations
+    float *red = xsum + (size_t)NB * (cols / 32);                 // [kQ80Rounds][WAVES][NB][16]   (KS > 1)
+    float *misc = red + (KS > 1 ? kQ80Rounds * WAVES * NB * 16 : 0);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = lane >> 4, ks = wave % KS, team = wave / KS;
+    const int row_blocks = (a.rows + 15) >> 4;
+    {
+        const int units = (row_blocks + RB - 1) / RB;
+        iters = (units - (int)blockIdx.x + workgroups - 1) / workgroups;   // ragged last round for the lowest workgroups
+        if (iters < 0) iters = 0;
+    }
+    const int total_steps = iters * S;
+    auto block_of = [&](int round) { return (round * workgroups + (int)blockIdx.x) * RB + team; };
+    auto load_step = [&](int f) {   // unconditional: steps past the end read bytes that every lane shares
+        Q80Item it;
+        const bool real = f < total_steps;
+        const int round = f / S, step = f - round * S;
+        const int rb = block_of(round) < row_blocks ? block_of(round) : row_blocks - 1;
+        const uint8_t *tp = real ? tiled + ((size_t)rb * TPR + (ks * S + step)) * kQ80TileBytes : tiled;
+        const int spread = real ? 16 : 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) it.q[j] = *reinterpret_cast<const uint4 *>(tp + (real ? 1024 * j : 0) + spread * lane);
+        it.d = *reinterpret_cast<const u32 *>(tp + (real ? 4096 : 0) + (real ? 4 : 0) * lane);
+        return it;
+    };
+
+    MfmaStage<NB, IPR, THREADS, MODE> stage;
+    stage.issue(a);
+    constexpr int AHEAD = DEPTH == 2 ? 1 : DEPTH;
+    Q80Item ring[DEPTH];
+#pragma unroll
+    for (int d = 0; d < AHEAD; d++) ring[d] = load_step(d);
+    if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
+    stage.finish(a, xs4, xsum, misc);
+    __syncthreads();
+
+    // A operand: slot i = lane % 16 carries activation row i % 4 in lane group i / 4 only; group index of (tile step, j, fragment m)
+    // = 32 step + 16 j + 4 g + m
+    const int slot = lane & 15;
+    const bool feeds = (slot >> 2) == g && (slot & 3) < NB;
+    const uint4 *a_base = feeds ? xs4 + (size_t)(slot & 3) * GROUPS + 32 * (ks * S) + 4 * g : zero4;
+    const int a_stride = feeds ? 32 : 0, a_jstride = feeds ? 16 : 0;
+    const float *xsum_base = xsum + 8 * (ks * S) + g;
+
+    float v[NB];
+    auto step_compute = [&](const Q80Item &it, int i) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            const uint4 *ap = a_base + i * a_stride + j * a_jstride;
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                const uint4 &q = it.q[2 * j + (m >> 1)];
+                const u32 t0 = ((m & 1) ? q.z : q.x) ^ 0x80808080u, t1 = ((m & 1) ? q.w : q.y) ^ 0x80808080u;   // signed -> biased
+                const uint4 p = make_uint4(__builtin_amdgcn_perm(0x64646464u, t0, 0x04020400u), __builtin_amdgcn_perm(0x64646464u, t0, 0x04030401u),
+                                           __builtin_amdgcn_perm(0x64646464u, t1, 0x04020400u), __builtin_amdgcn_perm(0x64646464u, t1, 0x04030401u));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[m]), __builtin_bit_cast(half8, p), acc, 0, 0, 0);
+            }
+            const float d = half_bits_to_float((it.d >> (16 * j)) & 0xFFFFu);
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                const float sx = xsum_base[(size_t)b * (cols >> 5) + 8 * i + 4 * j];
+                v[b] += d * (acc[b] - 1152.0f * sx);
+            }
+        }
+    };
+
+    float best[NB];
+    int best_i[NB];
+#pragma unroll
+    for (int b = 0; b < NB; b++) { best[b] = -INFINITY; best_i[b] = 0x7FFFFFFF; }
+    auto finish_block = [&](int rb, float (&sum)[NB]) {
+        if (a.epilogue == EPI_ARGMAX) {
+            const int row = rb * 16 + lane;
+            if (lane < 16 && row < a.rows) {
+#pragma unroll
+                for (int b = 0; b < NB; b++) argmax_take(best[b], best_i[b], sum[b], row);
+            }
+            return;
+        }
+        float other[NB];
+#pragma unroll
+        for (int b = 0; b < NB; b++) other[b] = dpp_term<0xB1, 0xF>(sum[b]);
+        if (lane < 16 && (lane & 1) == 0 && rb < row_blocks) pair_epilogue<NB>(a, rb * 8 + (lane >> 1), sum, other);
+    };
+
+    for (int round = 0; round < iters; round++) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) v[b] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < S; i++) {
+            const Q80Item it = ring[i % DEPTH];
+            ring[(i + AHEAD) % DEPTH] = load_step(round * S + i + AHEAD);
+            step_compute(it, i);
+            if constexpr (S >= 3) __builtin_amdgcn_sched_barrier(0);   // rounds of several steps: keep the unrolled steps apart (registers)
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            v[b] += __shfl_xor(v[b], 16);
+            v[b] += __shfl_xor(v[b], 32);
+        }
+        if constexpr (KS == 1) {
+            finish_block(block_of(round), v);
+        } else {
+            float *slot_base = red + ((size_t)(round % kQ80Rounds) * WAVES + wave) * NB * 16;
+            if (lane < 16) {
+#pragma unroll
+                for (int b = 0; b < NB; b++) slot_base[b * 16 + lane] = v[b];
+            }
+        }
+    }
+    if constexpr (KS > 1) {
+        __syncthreads();
+        if (ks == 0) {   // the team's shares in wavefront order, then the epilogue
+            for (int round = 0; round < iters; round++) {
+                float sum[NB];
+#pragma unroll
+                for (int b = 0; b < NB; b++) {
+                    float t = 0.0f;
+                    if (lane < 16) {
+#pragma unroll
+                        for (int w = 0; w < KS; w++) t += red[((size_t)(round % kQ80Rounds) * WAVES + wave + w) * NB * 16 + b * 16 + lane];
+                    }
+                    sum[b] = t;
+                }
+                finish_block(block_of(round), sum);
+            }
+        }
+    }
+    if (a.epilogue == EPI_ARGMAX) {
+        float *cv = misc;
+        int *ci = reinterpret_cast<int *>(misc + NB * WAVES);
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+#pragma unroll
+            for (int off = 8; off >= 1; off >>= 1) {
+                const float ov = __shfl_xor(best[b], off);
+                const int oi = __shfl_xor(best_i[b], off);
+                argmax_take(best[b], best_i[b], ov, oi);
+            }
+            if (lane == 0) { cv[b * WAVES + wave] = ks == 0 ? best[b] : -INFINITY; ci[b * WAVES + wave] = ks == 0 ? best_i[b] : 0x7FFFFFFF; }
+        }
+        __syncthreads();
+        if (tid < NB) {
+            float bv = cv[tid * WAVES];
+            int bi = ci[tid * WAVES];
+#pragma unroll
+            for (int w = 1; w < WAVES; w++) argmax_take(bv, bi, cv[tid * WAVES + w], ci[tid * WAVES + w]);
+            a.part_value[(size_t)tid * gridDim.x + blockIdx.x] = bv;
+            a.part_index[(size_t)tid * gridDim.x + blockIdx.x] = bi;
+        }
+    }
+}
+
 // Launch through the extension entry point when the caller gave the launch a pair of events of its own: they
 // take the kernel's own start and end times (what a kernel trace reports), without the gaps between launches.
 static thread_local hipEvent_t tl_start_event = nullptr, tl_stop_event = nullptr;
@@ -1905,6 +2085,83 @@ hipError_t try_q40_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
     return hipSuccess;
 }
 
+template <int NB, int TPR, int WAVES, int KS, int MODE>
+hipError_t launch_q80_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
+    constexpr int RB = WAVES / KS, cols = TPR * 256, THREADS = WAVES * 64;
+    *launched = false;
+    const size_t lds = ((size_t)NB * (cols / 8) + 8) * 16 + (size_t)NB * (cols / 32) * 4 + (KS > 1 ? (size_t)kQ80Rounds * WAVES * NB * 16 * 4 : 0) +
+                       (size_t)2 * NB * WAVES * 4;
+    auto kernel = gemv_q80_mfma_kernel<NB, TPR, WAVES, KS, MODE>;
+    static size_t configured_lds = 0;
+    hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
+    if (e != hipSuccess) return e;
+    static int resident_per_cu = 0;
+    if (resident_per_cu == 0) {
+        int n = 0;
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, THREADS, lds);
+        if (e != hipSuccess) return e;
+        const int by_waves = WAVES >= 16 ? 1 : 16 / WAVES;   // sixteen wavefronts per compute unit, as for the other formats
+        resident_per_cu = n < 1 ? 1 : (n > by_waves ? by_waves : n);
+    }
+    const int row_blocks = (a.rows + 15) / 16;
+    const int want = (row_blocks + RB - 1) / RB;
+    const int cap = compute_units() * resident_per_cu;
+    const int grid = want < cap ? want : cap;
+    const int iters = (want + grid - 1) / grid;
+    if (KS > 1 && iters > kQ80Rounds) return hipSuccess;   // not launched: the caller takes the other kernel
+    const void *activations = MODE == 1 ? static_cast<const void *>(a.norm_x) : MODE == 2 ? static_cast<const void *>(a.merge_partials) : static_cast<const void *>(a.x);
+    launch_kernel(kernel, dim3(grid), dim3(THREADS), lds, stream, a.tiled, activations, a.norm_w, a.rows, iters, grid, a.norm_eps, a);
+    *launched = true;
+    return hipGetLastError();
+}
+
+// "q80_mfma" (ESPRESSO_HIP_Q80_MFMA): 0 never, 1 wherever an instantiation exists (768, 2048 and 4096 columns, one and two activation
+// rows), -1 the default (see launch_q80).  Tall matrices (an output head) take four wavefronts that each walk whole rows; the others split a row
+// block's columns over the wavefronts of a workgroup.
+int g_q80_mfma_mode = -2;
+int q80_mfma_mode() {
+    if (g_q80_mfma_mode == -2) g_q80_mfma_mode = env_int("ESPRESSO_HIP_Q80_MFMA", -1);
+    return g_q80_mfma_mode;
+}
+inline bool q80_mfma_width(int cols) { return cols == 768 || cols == 2048 || cols == 4096; }
+
+template <int NB>
+hipError_t try_q80_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
+    *launched = false;
+    if (!a.tiled || q80_mfma_mode() == 0) return hipSuccess;
+    const int mode = a.merge_partials ? 2 : a.norm_x ? 1 : 0;
+    const bool tall = a.rows > 8192;
+#define ESP_Q80_WIDTH(COLS_, W_)                                                                                       \
+    if (a.cols == COLS_) {                                                                                            \
+        if (tall) {                                                                                                   \
+            if (mode == 0) return launch_q80_mfma<NB, COLS_ / 256, 4, 1, 0>(a, stream, launched);                     \
+            if (mode == 1) return launch_q80_mfma<NB, COLS_ / 256, 4, 1, 1>(a, stream, launched);                     \
+            return hipSuccess;                                                                                        \
+        }                                                                                                             \
+        if (mode == 0) return launch_q80_mfma<NB, COLS_ / 256, W_, W_, 0>(a, stream, launched);                       \
+        if (mode == 1) return launch_q80_mfma<NB, COLS_ / 256, W_, W_, 1>(a, stream, launched);                       \
+        return launch_q80_mfma<NB, COLS_ / 256, W_, W_, 2>(a, stream, launched);                                      \
+    }
+    ESP_Q80_WIDTH(768, 3)
+    ESP_Q80_WIDTH(2048, 8)
+    ESP_Q80_WIDTH(4096, 8)
+#undef ESP_Q80_WIDTH
+    return hipSuccess;
+}
+
+template <int B>
+hipError_t launch_q80(const KernelArgs &a, hipStream_t stream) {
+    // measured (us, dot-product / matrix cores): one row 2304 x 768 2.74 / 2.96, 4096 x 768 3.08 / 3.22, 768 x 2048 3.01 / 3.00, 4096 x 4096
+    // 6.36 / 5.52, 32000 x 768 9.26 / 6.76, 32000 x 4096 31.5 / 26.9; two rows 3.36 / 3.17, 3.77 / 3.31, 3.47 / 3.36, 7.23 / 5.69, 12.1 / 6.8, 32.8 / 27.6:
+    // two rows always, one row where the matrix is tall or wide ("q80_mfma" = 1: wherever an instantiation exists)
+    if (q80_mfma_mode() == 1 || (q80_mfma_mode() < 0 && (B >= 2 || a.rows > 8192 || a.cols >= 4096))) {
+        bool launched = false;
+        const hipError_t e = try_q80_mfma<B>(a, stream, &launched);
+        if (e != hipSuccess || launched) return e;
+    }
+    return launch_fmt<FMT_Q8_0>(a, B, stream);
+}
+
 template <int B>
 hipError_t launch_q40(const KernelArgs &a, hipStream_t stream) {
     if (q40_mfma_mode() == 1 || (q40_mfma_mode() < 0 && (B >= 2 || a.rows >= 2048))) {
@@ -1923,13 +2180,18 @@ bool gemv_merges_attention_partials(const DeviceMatrix &w, int batch, int head_d
     return true;
 }
 
+static unsigned g_tuning_epoch = 0;
+unsigned gemv_tuning_epoch() { return g_tuning_epoch; }
+
 bool gemv_set_tuning(const char *key, int value) {
     const std::string k = key ? key : "";
+    g_tuning_epoch++;   // runtimes drop the graphs they captured under the old selection
     if (k == "q4k_mfma") { g_q4k_mfma_mode = value; return true; }
     if (k == "q4k_mfma_ks") { g_q4k_mfma_split = value; return true; }
     if (k == "q4k_mfma_waves") { g_q4k_mfma_waves = value; return true; }
     if (k == "q4k_mfma_ragged") { g_q4k_mfma_ragged = value; return true; }
     if (k == "q40_mfma") { g_q40_mfma_mode = value; return true; }
+    if (k == "q80_mfma") { g_q80_mfma_mode = value; return true; }
     if (k == "q4k_mfma_max_rows") { g_q4k_mfma_max_rows = value; return true; }
     if (k == "q4k_long_row_waves") { g_q4k_long_row_waves = value; return true; }
     return false;
@@ -1963,6 +2225,7 @@ bool gemv_wants_tiled_copy(int format, int cols) {
     if (!enabled) return false;
     if (format == FMT_Q4_K) return cols == 4096 || cols == 14336 || q4k_registry_width(cols);
     if (format == FMT_Q4_0) return cols == 4096 || cols == 14336;
+    if (format == FMT_Q8_0) return q80_mfma_width(cols);
     return false;
 }
 
@@ -2044,7 +2307,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
                 if (e == hipSuccess && !launched) { nb = 2; e = launch_q40<2>(a, stream); }
             } else e = nb == 1 ? launch_q40<1>(a, stream) : launch_q40<2>(a, stream);
             break;
-        case FMT_Q8_0: e = launch_fmt<FMT_Q8_0>(a, nb, stream); break;
+        case FMT_Q8_0: e = nb == 1 ? launch_q80<1>(a, stream) : launch_q80<2>(a, stream); break;
         case FMT_F16: e = launch_fmt<FMT_F16>(a, nb, stream); break;
         case FMT_F32: e = launch_fmt<FMT_F32>(a, nb, stream); break;
         default: e = hipErrorInvalidValue;

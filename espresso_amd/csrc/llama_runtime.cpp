@@ -562,20 +562,30 @@ int LlamaRuntime::enqueue_trunk(int M, bool embedded, float *final_out) {
     return ESP_OK;
 }
 
+void LlamaRuntime::drop_captured_graphs() {
+    for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+    for (auto &g : multi_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+    graph_epoch_++;
+}
+
+// esp_set_tuning changes which kernels launch_gemv picks: graphs captured before it would keep replaying the old ones.
+void LlamaRuntime::sync_tuning() {
+    const unsigned e = gemv_tuning_epoch();
+    if (e == tuning_epoch_) return;
+    tuning_epoch_ = e;
+    drop_captured_graphs();
+}
+
 void LlamaRuntime::set_split_activations(bool enabled) {
     if (enabled == split_activations_) return;
     split_activations_ = enabled;
-    for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }   // captured with the other kernels
-    for (auto &g : multi_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
-    graph_epoch_++;
+    drop_captured_graphs();   // captured with the other kernels
 }
 
 void LlamaRuntime::set_merged_attention(bool enabled) {
     if (enabled == merged_attention_) return;
     merged_attention_ = enabled;
-    for (auto &g : step_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }   // captured with the other path
-    for (auto &g : multi_graphs_) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
-    graph_epoch_++;
+    drop_captured_graphs();   // captured with the other path
 }
 
 void LlamaRuntime::release_loop_session() {
@@ -897,6 +907,7 @@ int LlamaRuntime::capture_steps(int seq, int count, hipGraphExec_t *out) {
 
 int LlamaRuntime::continue_greedy(int seq, int steps, uint32_t *out_tokens) {
     if (!finalized_) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
+    sync_tuning();
     if (seq < 0 || seq >= c_.max_sequences) return fail(ESP_ERR_OUT_OF_RANGE, "sequence %d of %d", seq, c_.max_sequences);
     if (steps < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "steps must be >= 0");
     if (visible_[seq] + steps > c_.max_seq)
@@ -941,6 +952,7 @@ int LlamaRuntime::continue_greedy_until_stop(int seq, int steps, uint32_t *out_t
     if (!finalized_) return fail(ESP_ERR_INVALID_ARGUMENT, "runtime is not finalized");
     if (seq < 0 || seq >= c_.max_sequences || !out_tokens || !produced) return fail(ESP_ERR_OUT_OF_RANGE, "continue_greedy_until_stop(seq %d)", seq);
     *produced = 0;
+    sync_tuning();
     if (steps < 0) return fail(ESP_ERR_INVALID_ARGUMENT, "steps must be >= 0");
     if (visible_[seq] + steps > c_.max_seq)
         return fail(ESP_ERR_OUT_OF_RANGE, "runtime position %d + %d steps exceeds context %d", visible_[seq], steps, c_.max_seq);

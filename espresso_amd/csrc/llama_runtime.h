@@ -110,7 +110,9 @@ class LlamaRuntime {
     int enqueue_device_head(int rows) { return run_head(hidden_, rows); }         // final norm, head, first-max arg-max per row
     bool graph_replay_enabled() const { return use_graph_ && !timing_enabled_; }
     unsigned long long id() const { return id_; }
-    unsigned long long graph_epoch() const { return graph_epoch_; }
+    // changes whenever the kernels a captured graph would hold have changed (switches of this runtime, esp_set_tuning): holders
+    // of captured passes compare it before they replay
+    unsigned long long graph_epoch() { sync_tuning(); return graph_epoch_; }
     DeviceLoopSession &loop_session() { return loop_session_; }
     void release_loop_session();   // destroys the session's graphs and frees its buffers
 
@@ -175,6 +177,9 @@ class LlamaRuntime {
     bool use_graph_ = true;
     std::vector<hipGraphExec_t> step_graphs_, multi_graphs_;   // one step, kStepsPerGraph steps
     unsigned long long id_ = 0, graph_epoch_ = 1;
+    unsigned tuning_epoch_ = 0;   // the kernel-selection epoch (gemv_tuning_epoch) this runtime's captured graphs were made under
+    void drop_captured_graphs();
+    void sync_tuning();
     DeviceLoopSession loop_session_;
     int *d_visible_ = nullptr, *d_log_ = nullptr, *d_log_count_ = nullptr;
     ArgmaxScratch argmax_scratch_;
