@@ -46,6 +46,7 @@ struct DeviceMatrix {
     size_t tiled_bytes() const {
         if (!tiled) return 0;
         if (format == FMT_Q8_0) return (size_t)((rows + 15) / 16) * (cols / 256) * 4352;
+        if (format == FMT_F16) return (size_t)((rows + 15) / 16) * (cols / 256) * 8192;
         return format == FMT_Q4_K ? (size_t)((rows + 15) / 16) * (cols / 256) * 2304 : (size_t)((rows + 15) / 16) * (cols / 512) * 4608;
     }
     size_t qs_row_bytes = 0;
@@ -200,6 +201,8 @@ hipError_t launch_q4k_tile(const uint8_t *blocks, int rows, int cols, uint8_t *t
 hipError_t launch_q40_tile(const uint8_t *qs, const uint16_t *scales, int rows, int cols, uint8_t *tiled, hipStream_t stream);
 // Q8_0 planes -> the tiled copy ((rows + 15) / 16 * cols / 256 tiles of 4352 bytes)
 hipError_t launch_q80_tile(const uint8_t *qs, const uint16_t *scales, int rows, int cols, uint8_t *tiled, hipStream_t stream);
+// fp16 weights -> the tiled copy ((rows + 15) / 16 * cols / 256 tiles of 8192 bytes)
+hipError_t launch_f16_tile(const uint8_t *weights, int rows, int cols, uint8_t *tiled, hipStream_t stream);
 // DeviceMatrix -> fp32 [rows][cols] (used to check the planes carry the same bits)
 hipError_t launch_dequant_matrix(const DeviceMatrix &m, float *out, hipStream_t stream);
 

@@ -110,6 +110,11 @@ int matrix_upload(int format, const void *gguf_blocks, int rows, int cols, Devic
             if ((rc = device_alloc(&m.tiled, tiled_bytes)) != ESP_OK) { matrix_release(&m); return rc; }
             e = launch_q4k_tile(m.qs, rows, cols, m.tiled, c.stream);
         }
+        if (e == hipSuccess && format == FMT_F16 && gemv_wants_tiled_copy(format, cols)) {
+            const size_t tiled_bytes = (size_t)((rows + 15) / 16) * (cols / 256) * 8192;
+            if ((rc = device_alloc(&m.tiled, tiled_bytes)) != ESP_OK) { matrix_release(&m); return rc; }
+            e = launch_f16_tile(m.qs, rows, cols, m.tiled, c.stream);
+        }
         if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
     }
     if (e != hipSuccess) { matrix_release(&m); return fail_hip(e, "matrix upload"); }

@@ -181,6 +181,24 @@ __global__ void q80_tile_kernel(const uint8_t *qs, const uint16_t *scales, int r
     }
 }
 
+// fp16 weights -> the tiled copy of the matrix-core GEMV: tile (rb, t) = sixteen rows x 256 columns = [j][m][lane] 16 bytes (lane
+// (n, g) = g * 16 + n owns columns 32 (4 j + g) .. + 31 of the tile, row n; m = which eight of them), the middle two of every four
+// weights exchanged (the order in which the kernels stage activations).  512 threads per tile; rows past the matrix are zeros.
+__global__ void f16_tile_kernel(const uint16_t *w, int rows, int cols, size_t tiles, uint8_t *tiled) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t tile = i / 512;
+    if (tile >= tiles) return;
+    const int p = (int)(i - tile * 512), tpr = cols / 256;
+    const int rb = (int)(tile / tpr), t = (int)(tile - (size_t)rb * tpr);
+    const int j = p >> 8, m = (p >> 6) & 3, lane = p & 63, g = lane >> 4, n = lane & 15, row = rb * 16 + n;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (row < rows) v = *reinterpret_cast<const uint4 *>(w + (size_t)row * cols + 256 * t + 32 * (4 * j + g) + 8 * m);
+    uint4 s;
+    s.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u); s.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
+    s.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u); s.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
+    *reinterpret_cast<uint4 *>(tiled + tile * 8192 + 1024 * (4 * j + m) + 16 * lane) = s;
+}
+
 inline dim3 grid_for(size_t n, int threads) { return dim3((unsigned)((n + threads - 1) / threads)); }
 
 }  // namespace
@@ -246,6 +264,13 @@ hipError_t launch_q80_tile(const uint8_t *qs, const uint16_t *scales, int rows, 
     const int tpr = cols / 256;
     const size_t tiles = (size_t)((rows + 15) / 16) * tpr;
     hipLaunchKernelGGL(q80_tile_kernel, grid_for(tiles * 320, 320), dim3(320), 0, stream, qs, scales, rows, tpr, tiles, tiled);
+    return hipGetLastError();
+}
+
+hipError_t launch_f16_tile(const uint8_t *weights, int rows, int cols, uint8_t *tiled, hipStream_t stream) {
+    if (!weights || !tiled || rows <= 0 || cols <= 0 || cols % 256 != 0) return hipErrorInvalidValue;
+    const size_t tiles = (size_t)((rows + 15) / 16) * (cols / 256);
+    hipLaunchKernelGGL(f16_tile_kernel, grid_for(tiles * 512, 512), dim3(512), 0, stream, reinterpret_cast<const uint16_t *>(weights), rows, cols, tiles, tiled);
     return hipGetLastError();
 }
 

@@ -1522,11 +1522,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q40_mfma_kernel(const uint8_t
 // byte b becomes the fp16 number 1152 + b without arithmetic (v_perm puts b ^ 0x80 under the exponent byte 0x64: 1024 + 128 + b,
 // exact), two bytes per v_perm; the four MFMAs of a block share its scale and one accumulator, and w = d b folds as
 // d (acc - 1152 Sx) with Sx the sum of the block's activations, staged beside them.  Exact products, fp32 sums.
-constexpr size_t kQ80TileBytes = 4352;
+// F16 = true: the same kernel for fp16 weights.  Their tiled copy holds the weights themselves, [j][m][lane] 16 bytes per (sixteen
+// rows, 256 columns) = eight 1 KB loads per wavefront and tile, already in the order the activations are staged in: a lane's sixteen
+// bytes ARE its B operand, and one accumulator runs over the whole round.
+constexpr size_t kQ80TileBytes = 4352, kF16TileBytes = 8192;
 constexpr int kQ80Rounds = 8;   // rounds whose partial sums have an LDS slot of their own (KS > 1)
-struct Q80Item { uint4 q[4]; u32 d; };
+template <bool F16> struct Q80Item { uint4 q[F16 ? 8 : 4]; u32 d; };
 
-template <int NB, int TPR, int WAVES, int KS, int MODE>
+template <int NB, int TPR, int WAVES, int KS, int MODE, bool F16 = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_q80_mfma_kernel(const uint8_t *tiled, const void *activations, const float *norm_w, int rows, int iters,
                                                                    int workgroups, float norm_eps, KernelArgs rest) {
     KernelArgs a = rest;
@@ -1554,22 +1557,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q80_mfma_kernel(const uint8_t
     const int total_steps = iters * S;
     auto block_of = [&](int round) { return (round * workgroups + (int)blockIdx.x) * RB + team; };
     auto load_step = [&](int f) {   // unconditional: steps past the end read bytes that every lane shares
-        Q80Item it;
+        Q80Item<F16> it;
         const bool real = f < total_steps;
         const int round = f / S, step = f - round * S;
         const int rb = block_of(round) < row_blocks ? block_of(round) : row_blocks - 1;
-        const uint8_t *tp = real ? tiled + ((size_t)rb * TPR + (ks * S + step)) * kQ80TileBytes : tiled;
+        const uint8_t *tp = real ? tiled + ((size_t)rb * TPR + (ks * S + step)) * (F16 ? kF16TileBytes : kQ80TileBytes) : tiled;
         const int spread = real ? 16 : 0;
 #pragma unroll
-        for (int j = 0; j < 4; j++) it.q[j] = *reinterpret_cast<const uint4 *>(tp + (real ? 1024 * j : 0) + spread * lane);
-        it.d = *reinterpret_cast<const u32 *>(tp + (real ? 4096 : 0) + (real ? 4 : 0) * lane);
+        for (int j = 0; j < (F16 ? 8 : 4); j++) it.q[j] = *reinterpret_cast<const uint4 *>(tp + (real ? 1024 * j : 0) + spread * lane);
+        if constexpr (F16) it.d = 0;
+        else it.d = *reinterpret_cast<const u32 *>(tp + (real ? 4096 : 0) + (real ? 4 : 0) * lane);
         return it;
     };
 
     MfmaStage<NB, IPR, THREADS, MODE> stage;
     stage.issue(a);
     constexpr int AHEAD = DEPTH == 2 ? 1 : DEPTH;
-    Q80Item ring[DEPTH];
+    Q80Item<F16> ring[DEPTH];
 #pragma unroll
     for (int d = 0; d < AHEAD; d++) ring[d] = load_step(d);
     if (tid < 8) zero4[tid] = make_uint4(0, 0, 0, 0);
@@ -1585,14 +1589,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q80_mfma_kernel(const uint8_t
     const float *xsum_base = xsum + 8 * (ks * S) + g;
 
     float v[NB];
-    auto step_compute = [&](const Q80Item &it, int i) {
+    floatx4 run = floatx4{0.0f, 0.0f, 0.0f, 0.0f};   // fp16 weights: the round's sums (no scale stands between the blocks)
+    auto step_compute = [&](const Q80Item<F16> &it, int i) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
             const uint4 *ap = a_base + i * a_stride + j * a_jstride;
+            if constexpr (F16) {
+#pragma unroll
+                for (int m = 0; m < 4; m++)
+                    run = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, ap[m]), __builtin_bit_cast(half8, it.q[4 * j + m]), run, 0, 0, 0);
+                continue;
+            }
+            floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int m = 0; m < 4; m++) {
-                const uint4 &q = it.q[2 * j + (m >> 1)];
+                if constexpr (F16) continue;
+                const uint4 &q = it.q[F16 ? 0 : 2 * j + (m >> 1)];
                 const u32 t0 = ((m & 1) ? q.z : q.x) ^ 0x80808080u, t1 = ((m & 1) ? q.w : q.y) ^ 0x80808080u;   // signed -> biased
                 const uint4 p = make_uint4(__builtin_amdgcn_perm(0x64646464u, t0, 0x04020400u), __builtin_amdgcn_perm(0x64646464u, t0, 0x04030401u),
                                            __builtin_amdgcn_perm(0x64646464u, t1, 0x04020400u), __builtin_amdgcn_perm(0x64646464u, t1, 0x04030401u));
@@ -1631,10 +1643,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q80_mfma_kernel(const uint8_t
         for (int b = 0; b < NB; b++) v[b] = 0.0f;
 #pragma unroll
         for (int i = 0; i < S; i++) {
-            const Q80Item it = ring[i % DEPTH];
+            const Q80Item<F16> it = ring[i % DEPTH];
             ring[(i + AHEAD) % DEPTH] = load_step(round * S + i + AHEAD);
             step_compute(it, i);
             if constexpr (S >= 3) __builtin_amdgcn_sched_barrier(0);   // rounds of several steps: keep the unrolled steps apart (registers)
+        }
+        if constexpr (F16) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) v[b] = run[b];
+            run = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
         }
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -2085,13 +2102,13 @@ hipError_t try_q40_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
     return hipSuccess;
 }
 
-template <int NB, int TPR, int WAVES, int KS, int MODE>
+template <int NB, int TPR, int WAVES, int KS, int MODE, bool F16 = false>
 hipError_t launch_q80_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
     constexpr int RB = WAVES / KS, cols = TPR * 256, THREADS = WAVES * 64;
     *launched = false;
     const size_t lds = ((size_t)NB * (cols / 8) + 8) * 16 + (size_t)NB * (cols / 32) * 4 + (KS > 1 ? (size_t)kQ80Rounds * WAVES * NB * 16 * 4 : 0) +
                        (size_t)2 * NB * WAVES * 4;
-    auto kernel = gemv_q80_mfma_kernel<NB, TPR, WAVES, KS, MODE>;
+    auto kernel = gemv_q80_mfma_kernel<NB, TPR, WAVES, KS, MODE, F16>;
     static size_t configured_lds = 0;
     hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
     if (e != hipSuccess) return e;
@@ -2125,7 +2142,7 @@ int q80_mfma_mode() {
 }
 inline bool q80_mfma_width(int cols) { return cols == 768 || cols == 2048 || cols == 4096; }
 
-template <int NB>
+template <int NB, bool F16 = false>
 hipError_t try_q80_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
     *launched = false;
     if (!a.tiled || q80_mfma_mode() == 0) return hipSuccess;
@@ -2134,19 +2151,30 @@ hipError_t try_q80_mfma(const KernelArgs &a, hipStream_t stream, bool *launched)
 #define ESP_Q80_WIDTH(COLS_, W_)                                                                                       \
     if (a.cols == COLS_) {                                                                                            \
         if (tall) {                                                                                                   \
-            if (mode == 0) return launch_q80_mfma<NB, COLS_ / 256, 4, 1, 0>(a, stream, launched);                     \
-            if (mode == 1) return launch_q80_mfma<NB, COLS_ / 256, 4, 1, 1>(a, stream, launched);                     \
+            if (mode == 0) return launch_q80_mfma<NB, COLS_ / 256, 4, 1, 0, F16>(a, stream, launched);                \
+            if (mode == 1) return launch_q80_mfma<NB, COLS_ / 256, 4, 1, 1, F16>(a, stream, launched);                \
             return hipSuccess;                                                                                        \
         }                                                                                                             \
-        if (mode == 0) return launch_q80_mfma<NB, COLS_ / 256, W_, W_, 0>(a, stream, launched);                       \
-        if (mode == 1) return launch_q80_mfma<NB, COLS_ / 256, W_, W_, 1>(a, stream, launched);                       \
-        return launch_q80_mfma<NB, COLS_ / 256, W_, W_, 2>(a, stream, launched);                                      \
+        if (mode == 0) return launch_q80_mfma<NB, COLS_ / 256, W_, W_, 0, F16>(a, stream, launched);                  \
+        if (mode == 1) return launch_q80_mfma<NB, COLS_ / 256, W_, W_, 1, F16>(a, stream, launched);                  \
+        return launch_q80_mfma<NB, COLS_ / 256, W_, W_, 2, F16>(a, stream, launched);                                 \
     }
     ESP_Q80_WIDTH(768, 3)
     ESP_Q80_WIDTH(2048, 8)
-    ESP_Q80_WIDTH(4096, 8)
+    if constexpr (!F16) { ESP_Q80_WIDTH(4096, 8) }
 #undef ESP_Q80_WIDTH
     return hipSuccess;
+}
+
+// fp16 weights (768 and 2048 columns): the same rule
+template <int B>
+hipError_t launch_f16(const KernelArgs &a, hipStream_t stream) {
+    if (q80_mfma_mode() == 1 || (q80_mfma_mode() < 0 && (B >= 2 || a.rows > 8192))) {
+        bool launched = false;
+        const hipError_t e = try_q80_mfma<B, true>(a, stream, &launched);
+        if (e != hipSuccess || launched) return e;
+    }
+    return launch_fmt<FMT_F16>(a, B, stream);
 }
 
 template <int B>
@@ -2226,6 +2254,7 @@ bool gemv_wants_tiled_copy(int format, int cols) {
     if (format == FMT_Q4_K) return cols == 4096 || cols == 14336 || q4k_registry_width(cols);
     if (format == FMT_Q4_0) return cols == 4096 || cols == 14336;
     if (format == FMT_Q8_0) return q80_mfma_width(cols);
+    if (format == FMT_F16) return cols == 768 || cols == 2048;
     return false;
 }
 
@@ -2308,7 +2337,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
             } else e = nb == 1 ? launch_q40<1>(a, stream) : launch_q40<2>(a, stream);
             break;
         case FMT_Q8_0: e = nb == 1 ? launch_q80<1>(a, stream) : launch_q80<2>(a, stream); break;
-        case FMT_F16: e = launch_fmt<FMT_F16>(a, nb, stream); break;
+        case FMT_F16: e = nb == 1 ? launch_f16<1>(a, stream) : launch_f16<2>(a, stream); break;
         case FMT_F32: e = launch_fmt<FMT_F32>(a, nb, stream); break;
         default: e = hipErrorInvalidValue;
         }

@@ -92,3 +92,36 @@ def test_stories_shape_decoder_on_the_matrix_cores(mods):
     ops.set_tuning("q80_mfma", -1)
     for r in (g, twin, ref):
         r.close()
+
+
+# the same kernel with fp16 weights as its B operand (BASELINE configs[0] and [4]: the 6-layer model with fp16 weights)
+@pytest.mark.parametrize("rows,cols", [(768, 768), (2048, 768), (768, 2048), (32000, 768), (1000, 768), (30, 2048)])
+def test_fp16_weights_on_the_matrix_cores(mods, rows, cols):
+    ll, ops, syn = mods
+    w = np.random.default_rng(rows + cols).normal(0, 0.02, (rows, cols)).astype(np.float32)
+    blocks = orc.quantize(orc.FMT_F16, w)
+    deq = orc.dequantize(orc.FMT_F16, blocks, rows * cols).reshape(rows, cols)
+    mat = ops.Matrix(orc.FMT_F16, blocks, rows, cols)
+    assert mat.resident_bytes > mat.bytes
+    rng = np.random.default_rng(cols)
+    scale = np.abs(deq).max() * np.sqrt(cols)
+    for batch in (1, 2):
+        x = rng.normal(0, 1, (batch, cols)).astype(np.float16)
+        res = rng.normal(0, 1, (batch, rows)).astype(np.float32)
+        want = np.stack([orc.matvec(deq, x[b].astype(np.float32)) for b in range(batch)])
+        ops.set_tuning("q80_mfma", 0)
+        base = mat.gemv(x)
+        ops.set_tuning("q80_mfma", 1)
+        y = mat.gemv(x)
+        assert np.abs(y - want).max() <= 2e-6 * scale + 1e-6, (batch, float(np.abs(y - want).max()))   # exact products, fp32 sums
+        assert np.abs(y - base).max() <= 2e-6 * scale + 1e-6
+        assert np.array_equal(mat.gemv(x).view(np.uint32), y.view(np.uint32))
+        assert np.abs(mat.gemv(x, res) - (want + res)).max() <= 2e-6 * scale + 1e-5
+    for j in (0, 1, 2, 3, 7, 8, 31, 32, 255, 256, cols - 1):
+        x = np.zeros((2, cols), np.float16)
+        x[0, j] = 1.0; x[1, cols - 1 - j] = -2.0
+        y = mat.gemv(x)
+        assert np.array_equal(y[0], deq[:, j]), j
+        assert np.array_equal(y[1], -2.0 * deq[:, cols - 1 - j]), j
+    ops.set_tuning("q80_mfma", -1)
+    mat.close()
