@@ -1805,6 +1805,12 @@ int q4k_mfma_split() {
     if (g_q4k_mfma_split == -2) g_q4k_mfma_split = env_int("ESPRESSO_HIP_Q4K_MFMA_KS", 0);
     return g_q4k_mfma_split;
 }
+// five to eight activation rows: matrices with more weight rows stay on the nibble-B GEMM kernel
+int g_q4k_mfma_rows8_max = -2;
+int q4k_mfma_rows8_max() {
+    if (g_q4k_mfma_rows8_max == -2) g_q4k_mfma_rows8_max = env_int("ESPRESSO_HIP_Q4K_MFMA_ROWS8_MAX", 8192);
+    return g_q4k_mfma_rows8_max;
+}
 int g_q4k_mfma_max_rows = -2;   // single activation rows: matrices with more rows stay on the dot-product kernel (0: no limit)
 int q4k_mfma_max_rows() {
     if (g_q4k_mfma_max_rows == -2) g_q4k_mfma_max_rows = env_int("ESPRESSO_HIP_Q4K_MFMA_MAX_ROWS", 0);
@@ -2221,6 +2227,7 @@ bool gemv_set_tuning(const char *key, int value) {
     if (k == "q40_mfma") { g_q40_mfma_mode = value; return true; }
     if (k == "q80_mfma") { g_q80_mfma_mode = value; return true; }
     if (k == "q4k_mfma_max_rows") { g_q4k_mfma_max_rows = value; return true; }
+    if (k == "q4k_mfma_rows8_max") { g_q4k_mfma_rows8_max = value; return true; }
     if (k == "q4k_long_row_waves") { g_q4k_long_row_waves = value; return true; }
     return false;
 }
@@ -2233,7 +2240,7 @@ bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
         // (five to eight rows: up to 8192 x 4096 8.7 against 10.7 us on the nibble-B kernel, at 14336 rows 18.9 against 17.1)
         return w.tiled && q40_mfma_mode() != 0 && (batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (batch <= 8 && w.cols == 4096 && w.rows <= 8192));
     if (w.format != FMT_Q4_K || !w.tiled || q4k_mfma_mode() == 0 || batch > 8) return false;
-    return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (w.cols == 4096 && w.rows <= 8192);
+    return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (w.cols == 4096 && w.rows <= q4k_mfma_rows8_max());
 }
 
 // Whether launch_gemv takes split activations (GemvParams::split_x) for this matrix and row count: the matrix-core Q4_K kernel
