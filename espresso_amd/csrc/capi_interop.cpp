@@ -730,6 +730,79 @@ bool esp_interop_fused_expansion_argmax_fp16(ESPSurfaceRef proj_surface, int pro
     return true;
 }
 
+// The factored head resident in HBM (MetalExpansionArgmax.swift:966-1088): weights uploaded once, candidates and results in buffers the
+// object keeps, one kernel over (vocab, lane) and a final pick per lane.
+struct ESPExpansionHead {
+    uint16_t *w = nullptr;
+    int bottleneck = 0, groups = 0, vocab = 0, blocks = 0, lanes = 0;
+    float *cand_v = nullptr, *out_v = nullptr;
+    int *cand_i = nullptr, *out_i = nullptr;
+};
+
+namespace {
+void release_expansion_buffers(ESPExpansionHead *h) {
+    for (void *p : {(void *)h->cand_v, (void *)h->out_v, (void *)h->cand_i, (void *)h->out_i}) if (p) (void)hipFree(p);
+    h->cand_v = h->out_v = nullptr;
+    h->cand_i = h->out_i = nullptr;
+    h->lanes = 0;
+}
+bool reserve_expansion_lanes(ESPExpansionHead *h, int lanes) {
+    if (lanes <= h->lanes) return true;
+    release_expansion_buffers(h);
+    const size_t cand = (size_t)lanes * h->blocks;
+    if (hipMalloc((void **)&h->cand_v, cand * sizeof(float)) != hipSuccess || hipMalloc((void **)&h->cand_i, cand * sizeof(int)) != hipSuccess ||
+        hipMalloc((void **)&h->out_v, (size_t)lanes * sizeof(float)) != hipSuccess || hipMalloc((void **)&h->out_i, (size_t)lanes * sizeof(int)) != hipSuccess) {
+        release_expansion_buffers(h);
+        return false;
+    }
+    h->lanes = lanes;
+    return true;
+}
+}  // namespace
+
+ESPExpansionHeadRef esp_interop_expansion_head_create(const void *expansion_weights_fp16, int bottleneck, int groups, int vocab_size) {
+    if (!expansion_weights_fp16 || bottleneck <= 0 || groups <= 0 || vocab_size <= 0 || vocab_size > 65535 || bottleneck % groups != 0 ||
+        vocab_size % groups != 0 || bottleneck > 24 * 1024) {
+        fail(ESP_ERR_INVALID_ARGUMENT, "expansion_head_create: vocab <= 65535, bottleneck and vocab multiples of groups");
+        return nullptr;
+    }
+    if (ensure_init() != ESP_OK) return nullptr;
+    ESPExpansionHead *h = new ESPExpansionHead();
+    h->bottleneck = bottleneck; h->groups = groups; h->vocab = vocab_size;
+    h->blocks = (vocab_size + 255) / 256 < 256 ? (vocab_size + 255) / 256 : 256;
+    const size_t bytes = (size_t)vocab_size * (bottleneck / groups) * 2;
+    hipError_t e = hipMalloc((void **)&h->w, bytes);
+    if (e == hipSuccess) e = hipMemcpy(h->w, expansion_weights_fp16, bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        fail_hip(e, "expansion_head_create");
+        if (h->w) (void)hipFree(h->w);
+        delete h;
+        return nullptr;
+    }
+    return h;
+}
+
+bool esp_interop_expansion_head_argmax(ESPExpansionHeadRef head, ESPSurfaceRef proj_surface, int proj_ch_off, int spatial, int stream_count, int fp32_sums,
+                                       int *out_indices, float *out_values) {
+    if (!head || !proj_surface || !out_indices || !out_values) return false;
+    if (proj_ch_off < 0 || spatial <= 0 || stream_count <= 0 || stream_count > spatial || spatial > 32768 || spatial % 8 != 0) return false;
+    if (!region_ok(proj_surface, proj_ch_off, head->bottleneck, spatial) || !surfaces_on_device({proj_surface})) return false;
+    if (!reserve_expansion_lanes(head, stream_count)) { fail(ESP_ERR_OUT_OF_MEMORY, "expansion_head_argmax: candidate buffers"); return false; }
+    const uint16_t *proj = reinterpret_cast<const uint16_t *>(proj_surface->device) + (size_t)proj_ch_off * spatial;
+    hipError_t e = launch_expansion_argmax(proj, spatial, stream_count, head->w, head->bottleneck, head->groups, head->vocab, fp32_sums != 0, head->blocks,
+                                           head->cand_v, head->cand_i, head->out_i, head->out_v, context().stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(out_indices, head->out_i, (size_t)stream_count * sizeof(int), hipMemcpyDeviceToHost, context().stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(out_values, head->out_v, (size_t)stream_count * sizeof(float), hipMemcpyDeviceToHost, context().stream);
+    return finish(e, "expansion_head_argmax");
+}
+
+void esp_interop_expansion_head_free(ESPExpansionHeadRef head) {
+    if (!head) return;
+    release_expansion_buffers(head);
+    if (head->w) (void)hipFree(head->w);
+    delete head;
+}
+
 bool esp_interop_io_lock_write(ESPSurfaceRef s) { if (!s || !surface_to_host(s)) return false; s->write_locks++; return true; }
 bool esp_interop_io_unlock_write(ESPSurfaceRef s) { if (!s || s->write_locks <= 0) return false; s->write_locks--; s->device_valid = false; return true; }
 bool esp_interop_io_lock_read(ESPSurfaceRef s) { if (!s || !surface_to_host(s)) return false; s->read_locks++; return true; }

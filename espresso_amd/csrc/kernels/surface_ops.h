@@ -17,5 +17,9 @@ hipError_t launch_surface_kv_scatter(const uint16_t *k_src, const uint16_t *v_sr
 // (MetalAttentionKernel.swift:1824-1886, fused_decode_sdpa; CPU twin DecodeForwardPass.swift:683-756).
 hipError_t launch_surface_sdpa(const uint16_t *q, const uint16_t *k_cache, const uint16_t *v_cache, uint16_t *context, int heads, int kv_heads, int head_dim,
                                int visible_tokens, int token_base, int cache_stride, int lane_stride, hipStream_t s);
+// Factored output head: expansion of the projected surface [bottleneck, spatial] (lanes 0 .. lanes - 1) by w [vocab][bottleneck / groups] fused with the
+// arg-max (surface_io.c:1438-1700 with fp16 sums, MetalExpansionArgmax.swift:966-1186 with fp32 sums); `blocks` candidates per lane go through cand_v / cand_i.
+hipError_t launch_expansion_argmax(const uint16_t *proj, int spatial, int lanes, const uint16_t *w, int bottleneck, int groups, int vocab, bool fp32_sums,
+                                   int blocks, float *cand_v, int *cand_i, int *out_i, float *out_v, hipStream_t s);
 hipError_t launch_row_max(const float *in, int channels, int spatial, int lanes, uint16_t *surface, hipStream_t s);
 }  // namespace esp

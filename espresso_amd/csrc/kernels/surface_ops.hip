@@ -109,6 +109,92 @@ __global__ __launch_bounds__(256) void row_max_kernel(const float *in, int chann
     (void)spatial;
 }
 
+
+// ---- factored output head: expansion [bottleneck -> vocab] fused with the arg-max ----
+// logit[c] = sum_k proj[g * cpg + k][lane] * w[c][k], g = c / (vocab / groups), one fused multiply-add per term in k order, in fp16
+// (the arithmetic of surface_io.c:1521-1700) or in fp32 (MetalExpansionArgmax.swift:1104-1140); no logit is stored.  A thread owns
+// whole channels, so a channel's chain is sequential whatever the grid; candidates compare by (value, lowest channel).
+template <bool FP32>
+__device__ __forceinline__ void expansion_take(float &best, int &best_i, float v, int i) {
+    if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+}
+
+template <bool FP32, bool VEC>
+__global__ __launch_bounds__(256) void expansion_argmax_kernel(const uint16_t *proj, int spatial, const uint16_t *w, int cpg, int ch_per_group, int vocab,
+                                                               int bottleneck, float *cand_v, int *cand_i) {
+    extern __shared__ uint16_t proj_lds[];                         // [bottleneck] of this lane
+    const int lane_col = blockIdx.y, tid = threadIdx.x;
+    for (int j = tid; j < bottleneck; j += 256) proj_lds[j] = proj[(size_t)j * spatial + lane_col];
+    __syncthreads();
+    // the running first maximum starts where the reference's does: fp16's most negative finite value (fp32: -inf) at channel 0
+    float best = FP32 ? -INFINITY : -65504.0f;
+    int best_i = 0;
+    for (int c = blockIdx.x * 256 + tid; c < vocab; c += gridDim.x * 256) {
+        const uint16_t *wr = w + (size_t)c * cpg;
+        const uint16_t *pg = proj_lds + (c / ch_per_group) * cpg;
+        float value;
+        if constexpr (FP32) {
+            float acc = 0.0f;
+            if constexpr (VEC) {
+                for (int k = 0; k < cpg; k += 8) {
+                    const uint4 q = *reinterpret_cast<const uint4 *>(wr + k);
+                    const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        acc = __builtin_fmaf(h2f(pg[k + 2 * t]), h2f((uint16_t)(qw[t] & 0xFFFFu)), acc);
+                        acc = __builtin_fmaf(h2f(pg[k + 2 * t + 1]), h2f((uint16_t)(qw[t] >> 16)), acc);
+                    }
+                }
+            } else {
+                for (int k = 0; k < cpg; k++) acc = __builtin_fmaf(h2f(pg[k]), h2f(wr[k]), acc);
+            }
+            value = acc;
+        } else {
+            _Float16 acc = (_Float16)0.0f;
+            if constexpr (VEC) {
+                for (int k = 0; k < cpg; k += 8) {
+                    const uint4 q = *reinterpret_cast<const uint4 *>(wr + k);
+                    const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        acc = __builtin_fmaf16(__builtin_bit_cast(_Float16, (uint16_t)(qw[t] & 0xFFFFu)), __builtin_bit_cast(_Float16, pg[k + 2 * t]), acc);
+                        acc = __builtin_fmaf16(__builtin_bit_cast(_Float16, (uint16_t)(qw[t] >> 16)), __builtin_bit_cast(_Float16, pg[k + 2 * t + 1]), acc);
+                    }
+                }
+            } else {
+                for (int k = 0; k < cpg; k++) acc = __builtin_fmaf16(__builtin_bit_cast(_Float16, wr[k]), __builtin_bit_cast(_Float16, pg[k]), acc);
+            }
+            value = (float)acc;
+        }
+        if (value > best) { best = value; best_i = c; }            // a thread's channels only grow: strict > keeps the first maximum
+    }
+    __shared__ float sv[256];
+    __shared__ int si[256];
+    sv[tid] = best; si[tid] = best_i;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if (tid < off) expansion_take<FP32>(sv[tid], si[tid], sv[tid + off], si[tid + off]);
+        __syncthreads();
+    }
+    if (tid == 0) {
+        cand_v[(size_t)lane_col * gridDim.x + blockIdx.x] = sv[0];
+        cand_i[(size_t)lane_col * gridDim.x + blockIdx.x] = si[0];
+    }
+}
+
+__global__ __launch_bounds__(64) void expansion_argmax_final_kernel(const float *cand_v, const int *cand_i, int blocks, int *out_i, float *out_v) {
+    const int lane_col = blockIdx.x, tid = threadIdx.x;
+    float best = cand_v[(size_t)lane_col * blocks];
+    int best_i = cand_i[(size_t)lane_col * blocks];
+    for (int b = tid; b < blocks; b += 64) expansion_take<true>(best, best_i, cand_v[(size_t)lane_col * blocks + b], cand_i[(size_t)lane_col * blocks + b]);
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off);
+        const int oi = __shfl_xor(best_i, off);
+        expansion_take<true>(best, best_i, ov, oi);
+    }
+    if (tid == 0) { out_i[lane_col] = best_i; out_v[lane_col] = best; }
+}
+
 }  // namespace
 
 hipError_t launch_gather_columns(const uint16_t *surface, int channels, int spatial, int lanes, uint16_t *out16, float *out32, hipStream_t s) {
@@ -145,6 +231,26 @@ hipError_t launch_surface_sdpa(const uint16_t *q, const uint16_t *k_cache, const
 }
 hipError_t launch_row_max(const float *in, int channels, int spatial, int lanes, uint16_t *surface, hipStream_t s) {
     hipLaunchKernelGGL(row_max_kernel, dim3(lanes), dim3(256), 0, s, in, channels, spatial, surface);
+    return hipGetLastError();
+}
+
+hipError_t launch_expansion_argmax(const uint16_t *proj, int spatial, int lanes, const uint16_t *w, int bottleneck, int groups, int vocab, bool fp32_sums,
+                                   int blocks, float *cand_v, int *cand_i, int *out_i, float *out_v, hipStream_t s) {
+    const int cpg = bottleneck / groups, ch_per_group = vocab / groups;
+    const size_t lds = (size_t)bottleneck * 2;
+    if (lds > 48 * 1024 || blocks <= 0) return hipErrorInvalidValue;
+    const dim3 grid(blocks, lanes);
+    const bool vec = cpg % 8 == 0;
+    if (fp32_sums) {
+        if (vec) hipLaunchKernelGGL((expansion_argmax_kernel<true, true>), grid, dim3(256), lds, s, proj, spatial, w, cpg, ch_per_group, vocab, bottleneck, cand_v, cand_i);
+        else hipLaunchKernelGGL((expansion_argmax_kernel<true, false>), grid, dim3(256), lds, s, proj, spatial, w, cpg, ch_per_group, vocab, bottleneck, cand_v, cand_i);
+    } else {
+        if (vec) hipLaunchKernelGGL((expansion_argmax_kernel<false, true>), grid, dim3(256), lds, s, proj, spatial, w, cpg, ch_per_group, vocab, bottleneck, cand_v, cand_i);
+        else hipLaunchKernelGGL((expansion_argmax_kernel<false, false>), grid, dim3(256), lds, s, proj, spatial, w, cpg, ch_per_group, vocab, bottleneck, cand_v, cand_i);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(expansion_argmax_final_kernel, dim3(lanes), dim3(64), 0, s, cand_v, cand_i, blocks, out_i, out_v);
     return hipGetLastError();
 }
 

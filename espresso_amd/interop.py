@@ -65,6 +65,9 @@ def _L() -> C.CDLL:
         "esp_interop_io_argmax_batch_fp16_spatial_parallel": (b, [vp, i32, i32, i32, i32, ip, fp, i32]),
         "esp_interop_io_argmax_batch_fp16_spatial_nolock": (b, [vp, i32, i32, i32, i32, ip, fp, i32]),
         "esp_interop_fused_expansion_argmax_fp16": (b, [vp, i32, i32, i32, i32, vp, i32, i32, ip, fp, i32]),
+        "esp_interop_expansion_head_create": (vp, [vp, i32, i32, i32]),
+        "esp_interop_expansion_head_argmax": (b, [vp, vp, i32, i32, i32, i32, ip, fp]),
+        "esp_interop_expansion_head_free": (None, [vp]),
         "esp_interop_gather_f16_to_f32": (None, [vp, vp, i32, i32]),
         "esp_interop_scatter_f32_to_f16": (None, [vp, vp, i32, i32]),
         "esp_interop_rope_decode": (b, [vp, vp, i32, i32, i32, i32, C.c_float, i32]),
@@ -281,6 +284,41 @@ class SurfaceIO:
         _ok(_L().esp_interop_fused_expansion_argmax_fp16(projSurface.ref, projChannelOffset, spatial, bottleneck, groups, _ptr(w), vocabSize, streamCount,
                                                          idx, val, nBlocks), "fusedExpansionArgmax")
         return list(idx[:streamCount]), list(val[:streamCount])
+
+
+class FusedExpansionArgmax:
+    """MetalExpansionArgmax.swift:966-1088: the factored head's expansion weights resident on the GPU; run() returns one token per lane.
+    expansionWeights: fp16 bits [vocab, bottleneck / groups]."""
+
+    def __init__(self, expansionWeights, bottleneck: int, vocabSize: int, spatial: int, groups: int = 1):
+        w = np.ascontiguousarray(expansionWeights, dtype=np.uint16)
+        if bottleneck <= 0 or vocabSize <= 0 or spatial <= 0:
+            raise SurfaceIOError("all dimensions must be > 0")
+        if groups <= 0 or bottleneck % groups != 0 or w.size < vocabSize * (bottleneck // groups):
+            raise SurfaceIOError("wExpand too small")
+        self.bottleneck, self.vocabSize, self.spatial, self.groups = bottleneck, vocabSize, spatial, groups
+        self.ref = _L().esp_interop_expansion_head_create(_ptr(w), bottleneck, groups, vocabSize)
+        if not self.ref:
+            raise SurfaceIOError("FusedExpansionArgmax: " + _lib.last_error())
+
+    def run(self, projectedSurface: Surface, streamCount: int = None, channelOffset: int = 0, fp32Sums: bool = False, withValues: bool = False):
+        n = self.spatial if streamCount is None else streamCount
+        idx = (C.c_int * max(n, 1))()
+        val = (C.c_float * max(n, 1))()
+        _ok(_L().esp_interop_expansion_head_argmax(self.ref, projectedSurface.ref, channelOffset, self.spatial, n, 1 if fp32Sums else 0, idx, val),
+            "FusedExpansionArgmax.run")
+        return (list(idx[:n]), list(val[:n])) if withValues else list(idx[:n])
+
+    def close(self):
+        if self.ref:
+            _L().esp_interop_expansion_head_free(self.ref)
+            self.ref = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 def gather_f16_to_f32(bits, count: int, stride: int) -> np.ndarray:

@@ -661,6 +661,18 @@ bool esp_interop_io_argmax_batch_fp16_spatial_nolock(ESPSurfaceRef surface, int 
 bool esp_interop_fused_expansion_argmax_fp16(ESPSurfaceRef proj_surface, int proj_ch_off, int spatial, int bottleneck, int groups,
                                              const void *expansion_weights_fp16, int vocab_size, int stream_count, int *out_indices,
                                              float *out_values, int n_blocks);
+/* The same head resident on the GPU, in the shape of the reference's Metal twin (Sources/Espresso/MetalExpansionArgmax.swift:966-1186,
+ * FusedExpansionArgmax: init(wExpand:bottleneck:vocabSize:spatial:) uploads the expansion weights once, run(projectedSurface:) returns one
+ * token per spatial lane, no logits are stored).  create copies vocab_size x (bottleneck / groups) fp16 weights into HBM (groups = 1 is the
+ * Metal twin's dense expansion; grouped weights as in surface_io.c).  argmax reads lanes 0 .. stream_count - 1 of the projected surface
+ * where it lives on the device and runs one kernel over (vocab, lane): every logit is one chain of fused multiply-adds in k order, in fp16
+ * (fp32_sums = 0: bit-identical to esp_interop_fused_expansion_argmax_fp16, including its argument checks) or in fp32 (fp32_sums = 1: the
+ * Metal shader's arithmetic, first maximum on ties where the shader's reduction order is unspecified). */
+typedef struct ESPExpansionHead *ESPExpansionHeadRef;
+ESPExpansionHeadRef esp_interop_expansion_head_create(const void *expansion_weights_fp16, int bottleneck, int groups, int vocab_size);
+bool esp_interop_expansion_head_argmax(ESPExpansionHeadRef head, ESPSurfaceRef proj_surface, int proj_ch_off, int spatial, int stream_count,
+                                       int fp32_sums, int *out_indices, float *out_values);
+void esp_interop_expansion_head_free(ESPExpansionHeadRef head);
 bool esp_interop_io_lock_write(ESPSurfaceRef surface);                                                                     /* :335 */
 bool esp_interop_io_unlock_write(ESPSurfaceRef surface);
 bool esp_interop_io_lock_read(ESPSurfaceRef surface);

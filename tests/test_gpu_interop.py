@@ -278,3 +278,50 @@ def test_one_layer_handle_by_handle_matches_the_runtime(io, name, shape):
     for kernel in (qkv, proj, ffn):
         kernel.free()
     rt.close()
+
+
+@pytest.mark.parametrize("bottleneck,groups,vocab,spatial,streams", [(128, 1, 32000, 8, 3), (128, 4, 4096, 16, 16), (36, 3, 1002, 8, 1), (256, 1, 65535, 8, 2)])
+def test_factored_head_resident_on_the_gpu(io, bottleneck, groups, vocab, spatial, streams):
+    """The expansion + arg-max of the factored output head with its weights resident in HBM (MetalExpansionArgmax.swift:966-1186)
+    against the host routine (surface_io.c:1438-1700 restated; itself held to exact fp16 arithmetic in test_interop_surfaces.py):
+    bit-identical values and the same first maximum with fp16 sums; with fp32 sums against a sequential fp32 chain in numpy."""
+    cpg, per = bottleneck // groups, vocab // groups
+    rng = np.random.default_rng(vocab + bottleneck)
+    proj = rng.normal(0, 1, (bottleneck, spatial)).astype(np.float16)
+    w = rng.normal(0, 0.3, (vocab, cpg)).astype(np.float16)
+    w[per // 2 + 1] = w[per // 2]                     # two rows of one group tie exactly
+    s = io.Surface.create((bottleneck + 3) * spatial * 2)
+    io.SurfaceIO.writeFP16At(s, 3, proj.astype(np.float32), bottleneck, spatial)
+    head = io.FusedExpansionArgmax(w.view(np.uint16), bottleneck, vocab, spatial, groups)
+    want_i, want_v = io.SurfaceIO.fusedExpansionArgmax(s, 3, spatial, bottleneck, groups, w.view(np.uint16), vocab, streams)
+    got_i, got_v = head.run(s, streams, channelOffset=3, withValues=True)
+    assert got_i == want_i and got_v == want_v
+    assert head.run(s, streams, channelOffset=3) == want_i                       # a second call reuses the object's buffers
+    # fp32 sums: one fused multiply-add per term in k order (the Metal shader's loop), first maximum
+    got_i, got_v = head.run(s, streams, channelOffset=3, fp32Sums=True, withValues=True)
+    wf = w.astype(np.float64)
+    for lane in range(streams):
+        acc = np.zeros(vocab, np.float32)
+        pl = proj[:, lane].astype(np.float64).reshape(groups, cpg)
+        for k in range(cpg):
+            pk = np.repeat(pl[:, k], per)
+            acc = (pk * wf[:, k] + acc.astype(np.float64)).astype(np.float32)    # exact product, one rounding: a fused multiply-add
+        assert got_i[lane] == int(np.argmax(acc)) and got_v[lane] == float(acc.max())
+    # the tie: a projection that is one-hot in the tied rows' group makes rows per/2 and per/2 + 1 lead when their weight is the column's largest
+    col = int(np.argmax(w[per // 2].astype(np.float32)))
+    onehot = np.zeros((bottleneck, spatial), np.float32); onehot[col, 0] = 1.0
+    io.SurfaceIO.writeFP16At(s, 3, onehot, bottleneck, spatial)
+    column = w[:per, col].astype(np.float32)
+    i, v = head.run(s, 1, channelOffset=3, withValues=True)
+    assert i == [int(np.argmax(column))] and v == [float(column.max())]
+    if int(np.argmax(column)) == per // 2:
+        assert column[per // 2 + 1] == column[per // 2]
+    # argument checks of the host routine
+    import ctypes as C
+    idx, val = (C.c_int * 16)(), (C.c_float * 16)()
+    L = io._L()
+    assert not L.esp_interop_expansion_head_argmax(head.ref, s.ref, 3, 12, 1, 0, idx, val)                 # spatial not a multiple of 8
+    assert not L.esp_interop_expansion_head_argmax(head.ref, s.ref, 3, spatial, spatial + 1, 0, idx, val)   # more streams than lanes
+    assert not L.esp_interop_expansion_head_argmax(head.ref, s.ref, 4, spatial, 1, 0, idx, val)             # region past the surface
+    assert not L.esp_interop_expansion_head_create(w.ctypes.data_as(C.c_void_p), bottleneck, groups, 65536 + groups)
+    head.close()
