@@ -1291,6 +1291,194 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
 }
 
 
+// ---- Q4_K, five to eight activation rows in one pass over the tiled copy ----------------------------------------------------------
+// The slot trick above spends three quarters of the A operand on keeping lane groups apart, so that each lane can fold its own
+// sub-block's scale after the MFMA: four rows per MFMA set, and the fold's vector work grows with the rows (eight rows: 18.7 us at
+// 14336 x 4096 where four take 10.5).  Here the scale is folded into the B operand instead: the nibble becomes the exact integer
+// sc * q (at most 63 * 15, exact in fp16) with one v_and_or_b32 and one packed fused multiply-add per two weights
+// ((1024 + q) * sc - 1024 * sc for low nibbles, (64 + q) * sc - 64 * sc for high ones), the rows of A carry activation rows, one
+// accumulator runs over the whole super-block and d is applied to it once.  The minimum term d_min * sum_k x_k * m_sub(k) comes from
+// a second MFMA chain over the same A fragments whose B operand is the lane's own sub-block minimum, repeated (the k values a lane
+// feeds all belong to its chunk's two sub-blocks).  Products are exact and sums fp32, as in the kernels above; the vector work per
+// tile does not depend on the number of rows.  Lane (i, g) of the A operand needs the 64 columns of chunk g of activation row i,
+// each group of four in the order in which nibbles unpack (0, 2, 1, 3).  Read straight from memory those are sixteen-byte pieces
+// 128 bytes apart within an instruction, and the cache-line accesses, not the bytes, bound the kernel (15-18 us at eight rows); so
+// the activations go through LDS, in one of two ways:
+//   XMODE 1 (4096 columns, tall matrices): the workgroup stages all rows once (eight rows: 64 KB; rows 16 bytes apart in the banks,
+//           so that the reads of a lane group do not collide) and every round reuses them;
+//   XMODE 2 (any width): the wavefront fetches its tile's 8 x 256 activations with four fully coalesced loads (two rows of 512 bytes
+//           per instruction, one step ahead like the weights), writes them to four kilobytes of LDS of its own and reads the fragments
+//           from there: no workgroup barrier, nothing resident beyond the tile.
+// Rows of A past the batch repeat live rows; their products land in accumulator rows that are never stored.
+constexpr int kWideRounds = 4;            // rounds whose partial sums have an LDS slot of their own
+constexpr int kWideRowBytes = 512 + 16;   // XMODE 2: a row of the wavefront's tile of activations in LDS
+
+template <int XMODE>
+struct Q4KWideItem {
+    uint4 q0, q1, hdr;
+    uint4 xa[XMODE == 2 ? 4 : 1];   // XMODE 2: sixteen bytes of row 2 j + lane / 32 at 16 (lane % 32), j = 0..3
+};
+
+template <int IPR, int WAVES, int KS, int XMODE>
+__global__ __launch_bounds__(WAVES * 64, 4) void gemv_q4k_wide_kernel(const uint8_t *tiled, const uint16_t *x, int rows, int batch, int workgroups,
+                                                                      KernelArgs rest) {
+    KernelArgs a = rest;
+    a.rows = rows;
+    constexpr int cols = IPR * 64, NSB = IPR / 4, S = NSB / KS, RB = WAVES / KS, THREADS = WAVES * 64;
+    constexpr int XROW = cols * 2 + 16;                             // XMODE 1: bytes between staged rows
+    static_assert(NSB % KS == 0 && WAVES % KS == 0 && (XMODE == 1 || XMODE == 2), "whole super-blocks per wavefront");
+    extern __shared__ float4 wide_red[];                            // [kWideRounds][WAVES][64] partial sums (four rows per lane)
+    // XMODE 1: [8 rows][XROW]; XMODE 2: [WAVES][8 rows][kWideRowBytes]
+    uint8_t *xs = reinterpret_cast<uint8_t *>(wide_red + (size_t)kWideRounds * WAVES * 64);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, g = lane >> 4, ks = wave % KS, team = wave / KS;
+    const int row_blocks = (a.rows + 15) >> 4;
+    const Q4KLane L = q4k_chunk_constants(g);
+    u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+    asm volatile("" : "+s"(mask_lo), "+s"(mask_hi));
+    asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
+
+    const int units = (row_blocks + RB - 1) / RB;
+    int iters = (units - (int)blockIdx.x + workgroups - 1) / workgroups;
+    if (iters < 0) iters = 0;
+    const int total_steps = iters * S;
+    auto block_of = [&](int round) { return (round * workgroups + (int)blockIdx.x) * RB + team; };
+    // XMODE 2: rows 2 j + lane / 32 of the batch (rows past it repeat the last one)
+    const uint8_t *xtile = reinterpret_cast<const uint8_t *>(x) + (size_t)ks * S * 512 + 16 * (lane & 31);
+    size_t xrow2[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int r = 2 * j + (lane >> 5);
+        xrow2[j] = (size_t)(r < batch ? r : batch - 1) * cols * 2;
+    }
+    uint8_t *xw = xs + (size_t)wave * 8 * kWideRowBytes;            // XMODE 2: this wavefront's tile
+    auto load_step = [&](int f) {                                   // every load unconditional, addresses clamped (as above)
+        Q4KWideItem<XMODE> it;
+        const bool real = f < total_steps;
+        const int round = f / S, step = f - round * S;
+        const int rb = block_of(round) < row_blocks ? block_of(round) : row_blocks - 1;
+        const uint8_t *tp = real ? tiled + ((size_t)rb * NSB + (ks * S + step)) * kQ4KTileBytes : tiled;
+        const int spread = real ? 16 : 0;
+        it.hdr = *reinterpret_cast<const uint4 *>(tp + spread * n);
+        it.q0 = *reinterpret_cast<const uint4 *>(tp + (real ? 256 : 0) + spread * lane);
+        it.q1 = *reinterpret_cast<const uint4 *>(tp + (real ? 1280 : 0) + spread * lane);
+        if constexpr (XMODE == 2) {
+            const uint8_t *xp = xtile + (real ? step * 512 : 0);
+#pragma unroll
+            for (int j = 0; j < 4; j++) it.xa[j] = *reinterpret_cast<const uint4 *>(xp + xrow2[j]);
+        }
+        return it;
+    };
+
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto nibble_order = [](const uint4 &t) {                        // (x0 x1)(x2 x3)(x4 x5)(x6 x7) -> (x0 x2)(x1 x3)(x4 x6)(x5 x7)
+        uint4 r;
+        r.x = __builtin_amdgcn_perm(t.y, t.x, 0x05040100u);
+        r.y = __builtin_amdgcn_perm(t.y, t.x, 0x07060302u);
+        r.z = __builtin_amdgcn_perm(t.w, t.z, 0x05040100u);
+        r.w = __builtin_amdgcn_perm(t.w, t.z, 0x07060302u);
+        return r;
+    };
+    // lane (i = n, g) of the A operand: chunk g of row i % 8.  XMODE 1: of the staged rows, by super-block column; XMODE 2: of the tile
+    const uint8_t *xl = XMODE == 1 ? xs + (n & 7) * XROW + 128 * g + ks * S * 512 : xw + (n & 7) * kWideRowBytes + 128 * g;
+    auto step_compute = [&](const Q4KWideItem<XMODE> &it, int f) {
+        const int round = f / S, step = f - round * S;
+        if constexpr (XMODE == 2) {
+            // LDS operations of one wavefront complete in order: the reads of the previous step are done before these writes land
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                *reinterpret_cast<uint4 *>(xw + (2 * j + (lane >> 5)) * kWideRowBytes + 16 * (lane & 31)) = nibble_order(it.xa[j]);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        const uint8_t *xp = XMODE == 1 ? xl + step * 512 : xl;
+        const u32 src_sc = L.upper ? it.hdr.w : it.hdr.y, src_min = L.upper ? it.hdr.w : it.hdr.z;
+        const u32 scp = ((src_sc >> L.sh_sc) & L.mask_low) | ((it.hdr.y >> L.sh_top) & L.mask_top);
+        const u32 mp = ((src_min >> L.sh_min) & L.mask_low) | ((it.hdr.z >> L.sh_top) & L.mask_top);
+        const _Float16 s0 = (_Float16)(unsigned short)(scp & 0xFFu), s1 = (_Float16)(unsigned short)((scp >> 8) & 0xFFu);
+        const _Float16 m0 = (_Float16)(unsigned short)(mp & 0xFFu), m1 = (_Float16)(unsigned short)((mp >> 8) & 0xFFu);
+        const h2 s_lo = {s0, s0}, s_hi = {s1, s1};
+        const h2 o_lo = s_lo * (h2){(_Float16)-1024.0f, (_Float16)-1024.0f}, o_hi = s_hi * (h2){(_Float16)-64.0f, (_Float16)-64.0f};
+        const u32 mm0 = __builtin_bit_cast(u32, (h2){m0, m0}), mm1 = __builtin_bit_cast(u32, (h2){m1, m1});
+        const uint4 bm_lo = make_uint4(mm0, mm0, mm0, mm0), bm_hi = make_uint4(mm1, mm1, mm1, mm1);
+        floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f}, accm = {0.0f, 0.0f, 0.0f, 0.0f};
+        const u32 qd[8] = {it.q0.x, it.q0.y, it.q0.z, it.q0.w, it.q1.x, it.q1.y, it.q1.z, it.q1.w};
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const u32 w0 = qd[2 * jj], w1 = qd[2 * jj + 1];
+            uint4 pl, ph;
+            pl.x = __builtin_bit_cast(u32, __builtin_elementwise_fma(as_h2((w0 & mask_lo) | magic_lo), s_lo, o_lo));
+            pl.y = __builtin_bit_cast(u32, __builtin_elementwise_fma(as_h2(((w0 >> 8) & mask_lo) | magic_lo), s_lo, o_lo));
+            pl.z = __builtin_bit_cast(u32, __builtin_elementwise_fma(as_h2((w1 & mask_lo) | magic_lo), s_lo, o_lo));
+            pl.w = __builtin_bit_cast(u32, __builtin_elementwise_fma(as_h2(((w1 >> 8) & mask_lo) | magic_lo), s_lo, o_lo));
+            ph.x = __builtin_bit_cast(u32, __builtin_elementwise_fma(as_h2((w0 & mask_hi) | magic_hi), s_hi, o_hi));
+            ph.y = __builtin_bit_cast(u32, __builtin_elementwise_fma(as_h2(((w0 >> 8) & mask_hi) | magic_hi), s_hi, o_hi));
+            ph.z = __builtin_bit_cast(u32, __builtin_elementwise_fma(as_h2((w1 & mask_hi) | magic_hi), s_hi, o_hi));
+            ph.w = __builtin_bit_cast(u32, __builtin_elementwise_fma(as_h2(((w1 >> 8) & mask_hi) | magic_hi), s_hi, o_hi));
+            // low nibbles of the chunk: columns 8 jj .. 8 jj + 7 of its first half, high nibbles: of its second half
+            const half8 a_lo = *reinterpret_cast<const half8 *>(xp + 16 * jj), a_hi = *reinterpret_cast<const half8 *>(xp + 64 + 16 * jj);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_lo, __builtin_bit_cast(half8, pl), acc, 0, 0, 0);
+            accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_lo, __builtin_bit_cast(half8, bm_lo), accm, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, __builtin_bit_cast(half8, ph), acc, 0, 0, 0);
+            accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, __builtin_bit_cast(half8, bm_hi), accm, 0, 0, 0);
+        }
+        const float d = half_bits_to_float(it.hdr.x & 0xFFFFu), dmin = half_bits_to_float(it.hdr.x >> 16);
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] += d * acc[r] - dmin * accm[r];
+        if (step == S - 1) {                                        // the round's last step: this wavefront's share of sixteen rows x sixteen
+            wide_red[((size_t)(round % kWideRounds) * WAVES + wave) * 64 + lane] = make_float4(v[0], v[1], v[2], v[3]);
+            v[0] = v[1] = v[2] = v[3] = 0.0f;
+        }
+    };
+
+    // two slots, each filled while the other is consumed
+    Q4KWideItem<XMODE> even = load_step(0);
+    if constexpr (XMODE == 1) {
+        // the first weights are on their way; every thread stages its share of the batch's rows, in nibble order
+        constexpr int GROUPS = cols / 8;
+        for (int idx = tid; idx < 8 * GROUPS; idx += THREADS) {
+            const int row = idx / GROUPS, grp = idx - row * GROUPS;
+            const uint4 t = reinterpret_cast<const uint4 *>(x)[(size_t)(row < batch ? row : batch - 1) * GROUPS + grp];
+            *reinterpret_cast<uint4 *>(xs + row * XROW + 16 * grp) = nibble_order(t);
+        }
+        __syncthreads();
+    }
+    for (int f = 0; f < total_steps; f += 2) {
+        Q4KWideItem<XMODE> odd = load_step(f + 1);
+        step_compute(even, f);
+        even = load_step(f + 2);
+        if (f + 1 < total_steps) step_compute(odd, f + 1);
+    }
+    __syncthreads();
+    // wavefront ks == 0 of each team adds the team's shares in wavefront order and stores: lane (n, g) holds weight row n of the
+    // block for activation rows 4 g .. 4 g + 3
+    if (ks == 0) {
+        for (int round = 0; round < iters; round++) {
+            const int rb = block_of(round);
+            float4 t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+            for (int w = 0; w < KS; w++) {
+                const float4 p = wide_red[((size_t)(round % kWideRounds) * WAVES + wave + w) * 64 + lane];
+                t.x += p.x; t.y += p.y; t.z += p.z; t.w += p.w;
+            }
+            const int row = rb * 16 + n;
+            if (rb < row_blocks && row < a.rows) {
+                const float out[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int b = 4 * g + r;
+                    if (b < batch) {
+                        const size_t o = (size_t)b * a.rows + row;
+                        a.y[o] = a.epilogue == EPI_ADD_RESIDUAL ? a.residual[o] + out[r] : out[r];
+                    }
+                }
+            }
+        }
+    }
+}
+
+
 // ---- Q4_0 on the matrix cores ---------------------------------------------------------------------------------------------------
 // The same scheme as gemv_q4k_mfma_kernel for Q4_0's 32-weight blocks.  The tiled copy holds, per (sixteen rows, 512 columns),
 // four kilobytes of nibbles as [j][lane] 16 bytes (lane (n, g) owns blocks 4 j + g, j = 0..3, of row n) and then [lane][j] fp16
@@ -1868,6 +2056,54 @@ hipError_t launch_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launch
     return hipGetLastError();
 }
 
+// Five to eight rows (gemv_q4k_wide_kernel): fp16 activations given, store / residual epilogues, 4096 and 14336 columns.
+int g_q4k_wide_mode = -2;
+int q4k_wide_mode() {
+    if (g_q4k_wide_mode == -2) g_q4k_wide_mode = env_int("ESPRESSO_HIP_Q4K_WIDE", 1);
+    return g_q4k_wide_mode;
+}
+template <int IPR, int WAVES, int KS, int XMODE>
+hipError_t launch_q4k_wide(const KernelArgs &a, int batch, hipStream_t stream, bool *launched) {
+    constexpr int RB = WAVES / KS, THREADS = WAVES * 64;
+    *launched = false;
+    const size_t lds = (size_t)kWideRounds * WAVES * 64 * sizeof(float4) + (XMODE == 1 ? (size_t)8 * (IPR * 128 + 16) : (size_t)WAVES * 8 * kWideRowBytes);
+    auto kernel = gemv_q4k_wide_kernel<IPR, WAVES, KS, XMODE>;
+    static size_t configured_lds = 0;
+    hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
+    if (e != hipSuccess) return e;
+    static int resident_per_cu = 0;
+    if (resident_per_cu == 0) {
+        int n = 0;
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, THREADS, lds);
+        if (e != hipSuccess) return e;
+        const int by_waves = WAVES >= 16 ? 1 : 16 / WAVES;
+        resident_per_cu = n < 1 ? 1 : (n > by_waves ? by_waves : n);
+    }
+    const int row_blocks = (a.rows + 15) / 16;
+    const int want = (row_blocks + RB - 1) / RB;
+    const int cap = compute_units() * resident_per_cu;
+    const int grid = want < cap ? want : cap;
+    const int iters = (want + grid - 1) / grid;
+    if (iters > kWideRounds) return hipSuccess;   // not launched
+    launch_kernel(kernel, dim3(grid), dim3(THREADS), lds, stream, a.tiled, a.x, a.rows, batch, grid, a);
+    *launched = true;
+    return hipGetLastError();
+}
+// Measured (us, eight rows; nibble-B GEMM kernel in brackets): 14336 x 4096 staged rows 11.3, own tiles 12.75 (15.5); 28672 x 4096 18.7,
+// 21.05 (27.4); 4096 x 4096 7.0, 5.9 (7.6); 4096 x 14336 own tiles 12.0 (22.3).  Tuning key "q4k_wide": 0 off, 1 this table, 2 / 3 own tiles / staged rows wherever both exist.
+hipError_t try_q4k_wide(const KernelArgs &a, int batch, hipStream_t stream, bool *launched) {
+    *launched = false;
+    if (!a.tiled || !a.x || a.norm_x || a.merge_partials || a.split_x || batch < 5 || batch > 8) return hipSuccess;
+    if (a.epilogue != EPI_STORE_F32 && a.epilogue != EPI_ADD_RESIDUAL) return hipSuccess;
+    const int form = q4k_wide_mode();
+    if (a.cols == 4096) {
+        if (form == 2 || (form != 3 && a.rows <= 8192)) return launch_q4k_wide<64, 8, 8, 2>(a, batch, stream, launched);
+        return launch_q4k_wide<64, 16, 8, 1>(a, batch, stream, launched);
+    }
+    if (a.cols == 14336) return launch_q4k_wide<224, 8, 8, 2>(a, batch, stream, launched);
+    return hipSuccess;
+}
+
 // Picks the instantiation; *launched stays false when there is none for this shape.
 template <int NB>
 hipError_t try_q4k_mfma(const KernelArgs &a, hipStream_t stream, bool *launched) {
@@ -2229,8 +2465,12 @@ bool gemv_set_tuning(const char *key, int value) {
     if (k == "q4k_mfma_max_rows") { g_q4k_mfma_max_rows = value; return true; }
     if (k == "q4k_mfma_rows8_max") { g_q4k_mfma_rows8_max = value; return true; }
     if (k == "q4k_long_row_waves") { g_q4k_long_row_waves = value; return true; }
+    if (k == "q4k_wide") { g_q4k_wide_mode = value; return true; }
     return false;
 }
+
+// The wide kernel keeps kWideRounds rounds of partial sums in LDS: row blocks / (compute units x workgroups per unit) may not exceed that.
+static int q4k_wide_max_rows() { return compute_units() * 2 * 16 * kWideRounds; }
 
 bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
     if (batch <= 2) return true;
@@ -2239,7 +2479,9 @@ bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
     if (w.format == FMT_Q4_0)
         // (five to eight rows: up to 8192 x 4096 8.7 against 10.7 us on the nibble-B kernel, at 14336 rows 18.9 against 17.1)
         return w.tiled && q40_mfma_mode() != 0 && (batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (batch <= 8 && w.cols == 4096 && w.rows <= 8192));
-    if (w.format != FMT_Q4_K || !w.tiled || q4k_mfma_mode() == 0 || batch > 8) return false;
+    if (w.format != FMT_Q4_K || !w.tiled || q4k_mfma_mode() == 0) return false;
+    if (batch >= 5 && batch <= 8 && q4k_wide_mode() != 0 && (w.cols == 4096 || w.cols == 14336) && w.rows <= q4k_wide_max_rows()) return true;
+    if (batch > 8) return false;
     return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (w.cols == 4096 && w.rows <= q4k_mfma_rows8_max());
 }
 
@@ -2302,7 +2544,9 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     // batches beyond 2 run as successive pairs (each pair re-reads the weights); the matrix-core Q4_K kernel takes four rows at once
     const bool fours = p.batch > 2 && gemv_takes_rows(w, p.batch) && !p.merge_partials;
     for (int b0 = 0, nb = 0; b0 < p.batch; b0 += nb) {
-        nb = fours && p.batch - b0 == 8 ? 8 : fours && p.batch - b0 >= 4 ? 4 : p.batch - b0 >= 2 ? 2 : 1;
+        const bool wide = fours && w.format == FMT_Q4_K && p.batch - b0 >= 5 && p.batch - b0 <= 8 && q4k_wide_mode() != 0 && w.rows <= q4k_wide_max_rows() &&
+                          (p.epilogue == EPI_STORE_F32 || p.epilogue == EPI_ADD_RESIDUAL) && p.x && !p.split_x;
+        nb = wide ? p.batch - b0 : fours && p.batch - b0 == 8 ? 8 : fours && p.batch - b0 >= 4 ? 4 : p.batch - b0 >= 2 ? 2 : 1;
         KernelArgs a;
         a.qs = w.qs; a.tiled = w.tiled; a.scales = w.scales; a.qs_row_bytes = w.qs_row_bytes; a.rows = w.rows; a.cols = w.cols;
         a.x = p.x ? p.x + (size_t)b0 * w.cols * (p.split_x ? 2 : 1) : nullptr;
@@ -2330,7 +2574,11 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
         hipError_t e;
         switch (w.format) {
         case FMT_Q4_K:
-            if (nb == 8) {   // only the matrix-core kernel takes eight rows
+            if (nb >= 5 && wide) {
+                bool launched = false;
+                e = try_q4k_wide(a, nb, stream, &launched);
+                if (e == hipSuccess && !launched) e = hipErrorInvalidValue;
+            } else if (nb == 8) {   // only the matrix-core kernel takes eight rows
                 bool launched = false;
                 e = try_q4k_mfma<8>(a, stream, &launched);
                 if (e == hipSuccess && !launched) e = hipErrorInvalidValue;

@@ -18,6 +18,7 @@ def mods():
     ops.set_tuning("q4k_mfma", -1)
     ops.set_tuning("q4k_mfma_waves", 0)
     ops.set_tuning("q4k_mfma_ks", 0)
+    ops.set_tuning("q4k_wide", 1)
 
 
 def q4k_matrix(ops, rows, cols, seed):
@@ -60,6 +61,41 @@ def test_matches_oracle_and_dot_product_kernels(mods, rows, cols):
         y = mat.gemv(x)
         for b, (col, f) in enumerate([(j, 1.0), ((j + 1) % cols, 1.0), ((j + 33) % cols, 2.0), (cols - 1 - j, -1.0)]):
             assert np.abs(y[b] - f * deq[:, col]).max() <= 1e-6 * max(1.0, np.abs(deq[:, col]).max()) + 1e-7, (j, b)
+    mat.close()
+
+
+@pytest.mark.parametrize("rows,cols", [(16, 4096), (1000, 4096), (14336, 4096), (28672, 4096), (130, 14336), (4096, 14336)])
+def test_five_to_eight_rows_in_one_pass(mods, rows, cols):
+    """Five to eight activation rows on the kernel that folds the sub-block scales into the B operand (exact integer sc * q, a second
+    MFMA chain for the minimums), activations staged per workgroup or per wavefront tile: against the oracle's matvec, against the
+    nibble-B GEMM kernel it replaces, residual form, determinism, one-hot columns in every row."""
+    ll, ops, syn = mods
+    mat, deq = q4k_matrix(ops, rows, cols, rows + cols + 1)
+    rng = np.random.default_rng(rows + 5)
+    scale = np.abs(deq).max() * np.sqrt(cols)
+    for batch in (5, 6, 7, 8):
+        x = rng.normal(0, 1, (batch, cols)).astype(np.float16)
+        res = rng.normal(0, 1, (batch, rows)).astype(np.float32)
+        want = x.astype(np.float64) @ deq.astype(np.float64).T
+        ops.set_tuning("q4k_wide", 0)
+        base = mat.gemv(x)
+        assert np.abs(base - want).max() <= 2e-5 * scale + 1e-6
+        for form in ((1, 2, 3) if cols == 4096 else (1,)):
+            ops.set_tuning("q4k_wide", form)
+            y = mat.gemv(x)
+            # exact products, fp32 sums over 256 columns at a time inside the matrix core
+            assert np.abs(y - want).max() <= 2e-6 * scale + 1e-6, (batch, form, np.abs(y - want).max() / scale)
+            assert np.array_equal(mat.gemv(x).view(np.uint32), y.view(np.uint32))
+            assert np.abs(mat.gemv(x, res) - (want + res)).max() <= 2e-6 * scale + 1e-5
+    ops.set_tuning("q4k_wide", 1)
+    for j in (0, 7, 31, 32, 63, 64, 255, 256, cols - 1):
+        x = np.zeros((8, cols), np.float16)
+        picks = [(j + 37 * b) % cols for b in range(8)]
+        for b, c in enumerate(picks):
+            x[b, c] = 1.0 + b
+        y = mat.gemv(x)
+        for b, c in enumerate(picks):
+            assert np.abs(y[b] - (1.0 + b) * deq[:, c]).max() <= 1e-6 * (1.0 + b) * max(1.0, np.abs(deq[:, c]).max()) + 1e-7, (j, b)
     mat.close()
 
 
