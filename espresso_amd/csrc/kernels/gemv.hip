@@ -1310,22 +1310,53 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_mfma_kernel(const uint8_t
 //           per instruction, one step ahead like the weights), writes them to four kilobytes of LDS of its own and reads the fragments
 //           from there: no workgroup barrier, nothing resident beyond the tile.
 // Rows of A past the batch repeat live rows; their products land in accumulator rows that are never stored.
+//
+// Q40: the same kernel for Q4_0 (tiled copy of sixteen rows x 512 columns, see gemv_q40_mfma_kernel below; a step here is half a
+// tile).  A block's one scale is an arbitrary fp16 number and cannot go into the B operand exactly, so every MFMA contracts exactly
+// one 32-weight block for all sixteen weight rows: lane (n, g) needs dword g of each of the half tile's eight blocks of row n, which it
+// gets from the whole blocks the four lane groups loaded by a transpose in registers (v_permlane32_swap / v_permlane16_swap; as
+// four-byte loads the same bytes cost sixteen memory instructions per step instead of seven and the kernel 15.4 / 16.5 us instead of
+// 11.4 / 12.3 at 14336 x 4096 / 4096 x 14336, eight rows); B is the exact integer q - 8 ((1024 + q) - 1032,
+// (64 + q) - 72: one v_and_or_b32 and one packed add per two weights), and the block's scale multiplies the four accumulator
+// registers afterwards.  A lane's eight k values are weights 4 g .. 4 g + 3 and 16 + 4 g .. 16 + 4 g + 3 of the block: two eight-byte
+// reads of the staged activations.
 constexpr int kWideRounds = 4;            // rounds whose partial sums have an LDS slot of their own
-constexpr int kWideRowBytes = 512 + 16;   // XMODE 2: a row of the wavefront's tile of activations in LDS
+constexpr size_t kQ40TileBytes = 4608;
+// XMODE 2: bytes between the rows of a wavefront's tile of activations in LDS; the pad spreads the eight rows over the banks for
+// sixteen-byte (Q4_K) and eight-byte (Q4_0) reads
+constexpr int wide_row_bytes(bool q40) { return 512 + (q40 ? 32 : 16); }
+
+// v_permlane32_swap exchanges the upper 32 lanes of its first operand with the lower 32 of its second, v_permlane16_swap the odd
+// sixteen-lane rows of the first with the even rows of the second: two of each transpose four registers over the four lane groups.
+__device__ __forceinline__ uint4 transpose_lane_groups(const uint4 &q) {
+    const auto a = __builtin_amdgcn_permlane32_swap(q.x, q.z, false, false);
+    const auto b = __builtin_amdgcn_permlane32_swap(q.y, q.w, false, false);
+    const auto c = __builtin_amdgcn_permlane16_swap(a[0], b[0], false, false);
+    const auto d = __builtin_amdgcn_permlane16_swap(a[1], b[1], false, false);
+    return make_uint4(c[0], c[1], d[0], d[1]);
+}
+// .x .. .w = the value that lane groups 0 .. 3 hold in the same lane % 16
+__device__ __forceinline__ uint4 gather_lane_groups(u32 v) {
+    const auto a = __builtin_amdgcn_permlane32_swap(v, v, false, false);      // rows (v0 v1 v0 v1), (v2 v3 v2 v3)
+    const auto c = __builtin_amdgcn_permlane16_swap(a[0], a[0], false, false);
+    const auto d = __builtin_amdgcn_permlane16_swap(a[1], a[1], false, false);
+    return make_uint4(c[0], c[1], d[0], d[1]);
+}
 
 template <int XMODE>
 struct Q4KWideItem {
-    uint4 q0, q1, hdr;
+    uint4 q0, q1, hdr;              // Q4_0: q0, q1 = the lane's two blocks of the half tile, hdr.x = their scales
     uint4 xa[XMODE == 2 ? 4 : 1];   // XMODE 2: sixteen bytes of row 2 j + lane / 32 at 16 (lane % 32), j = 0..3
 };
 
-template <int IPR, int WAVES, int KS, int XMODE>
+template <int IPR, int WAVES, int KS, int XMODE, bool Q40 = false>
 __global__ __launch_bounds__(WAVES * 64, 4) void gemv_q4k_wide_kernel(const uint8_t *tiled, const uint16_t *x, int rows, int batch, int workgroups,
                                                                       KernelArgs rest) {
     KernelArgs a = rest;
     a.rows = rows;
     constexpr int cols = IPR * 64, NSB = IPR / 4, S = NSB / KS, RB = WAVES / KS, THREADS = WAVES * 64;
-    constexpr int XROW = cols * 2 + 16;                             // XMODE 1: bytes between staged rows
+    constexpr int XROW = cols * 2 + (Q40 ? 32 : 16);                // XMODE 1: bytes between staged rows
+    constexpr int kWideRowBytes = wide_row_bytes(Q40);
     static_assert(NSB % KS == 0 && WAVES % KS == 0 && (XMODE == 1 || XMODE == 2), "whole super-blocks per wavefront");
     extern __shared__ float4 wide_red[];                            // [kWideRounds][WAVES][64] partial sums (four rows per lane)
     // XMODE 1: [8 rows][XROW]; XMODE 2: [WAVES][8 rows][kWideRowBytes]
@@ -1357,11 +1388,21 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_q4k_wide_kernel(const uint
         const bool real = f < total_steps;
         const int round = f / S, step = f - round * S;
         const int rb = block_of(round) < row_blocks ? block_of(round) : row_blocks - 1;
-        const uint8_t *tp = real ? tiled + ((size_t)rb * NSB + (ks * S + step)) * kQ4KTileBytes : tiled;
-        const int spread = real ? 16 : 0;
-        it.hdr = *reinterpret_cast<const uint4 *>(tp + spread * n);
-        it.q0 = *reinterpret_cast<const uint4 *>(tp + (real ? 256 : 0) + spread * lane);
-        it.q1 = *reinterpret_cast<const uint4 *>(tp + (real ? 1280 : 0) + spread * lane);
+        if constexpr (Q40) {
+            // whole blocks as the tile holds them: lane (n, g) gets blocks (2 half, g) and (2 half + 1, g) of row n and their two scales
+            const int unit = ks * S + step, half = unit & 1;
+            const uint8_t *tp = real ? tiled + ((size_t)rb * (NSB / 2) + (unit >> 1)) * kQ40TileBytes + 2048 * half : tiled;
+            const int spread = real ? 16 : 0;
+            it.q0 = *reinterpret_cast<const uint4 *>(tp + spread * lane);
+            it.q1 = *reinterpret_cast<const uint4 *>(tp + (real ? 1024 : 0) + spread * lane);
+            it.hdr.x = *reinterpret_cast<const u32 *>(tp + (real ? 4096 - 2048 * half + 4 * half : 0) + (real ? 8 : 0) * lane);
+        } else {
+            const uint8_t *tp = real ? tiled + ((size_t)rb * NSB + (ks * S + step)) * kQ4KTileBytes : tiled;
+            const int spread = real ? 16 : 0;
+            it.hdr = *reinterpret_cast<const uint4 *>(tp + spread * n);
+            it.q0 = *reinterpret_cast<const uint4 *>(tp + (real ? 256 : 0) + spread * lane);
+            it.q1 = *reinterpret_cast<const uint4 *>(tp + (real ? 1280 : 0) + spread * lane);
+        }
         if constexpr (XMODE == 2) {
             const uint8_t *xp = xtile + (real ? step * 512 : 0);
 #pragma unroll
@@ -1380,7 +1421,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_q4k_wide_kernel(const uint
         return r;
     };
     // lane (i = n, g) of the A operand: chunk g of row i % 8.  XMODE 1: of the staged rows, by super-block column; XMODE 2: of the tile
-    const uint8_t *xl = XMODE == 1 ? xs + (n & 7) * XROW + 128 * g + ks * S * 512 : xw + (n & 7) * kWideRowBytes + 128 * g;
+    const int xg = Q40 ? 8 * g : 128 * g;
+    const uint8_t *xl = XMODE == 1 ? xs + (n & 7) * XROW + xg + ks * S * 512 : xw + (n & 7) * kWideRowBytes + xg;
     auto step_compute = [&](const Q4KWideItem<XMODE> &it, int f) {
         const int round = f / S, step = f - round * S;
         if constexpr (XMODE == 2) {
@@ -1393,6 +1435,32 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_q4k_wide_kernel(const uint
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
         const uint8_t *xp = XMODE == 1 ? xl + step * 512 : xl;
+        if constexpr (Q40) {
+            // dword g of every block of the half tile, and every block's scale, from the lanes that loaded them: a 4 x 4 transpose
+            // over the four lane groups (register r of group g <-> register g of group r) and an all-gather of the scale dword
+            const uint4 t0 = transpose_lane_groups(it.q0), t1 = transpose_lane_groups(it.q1);
+            const u32 qd[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+            const uint4 ds4 = gather_lane_groups(it.hdr.x);
+            const u32 dsc[4] = {ds4.x, ds4.y, ds4.z, ds4.w};
+            const h2 c_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f}, c_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                const u32 w = qd[b];
+                uint4 pb;
+                pb.x = __builtin_bit_cast(u32, as_h2((w & mask_lo) | magic_lo) + c_lo);           // weights 4 g, 4 g + 2
+                pb.y = __builtin_bit_cast(u32, as_h2(((w >> 8) & mask_lo) | magic_lo) + c_lo);    // 4 g + 1, 4 g + 3
+                pb.z = __builtin_bit_cast(u32, as_h2((w & mask_hi) | magic_hi) + c_hi);           // 16 + 4 g, 16 + 4 g + 2
+                pb.w = __builtin_bit_cast(u32, as_h2(((w >> 8) & mask_hi) | magic_hi) + c_hi);    // 16 + 4 g + 1, 16 + 4 g + 3
+                const uint2 x_lo = *reinterpret_cast<const uint2 *>(xp + 64 * b), x_hi = *reinterpret_cast<const uint2 *>(xp + 64 * b + 32);
+                const uint4 pa = make_uint4(x_lo.x, x_lo.y, x_hi.x, x_hi.y);
+                const floatx4 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, pa), __builtin_bit_cast(half8, pb),
+                                                                           floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+                const float d = half_bits_to_float(b < 4 ? dsc[b] & 0xFFFFu : dsc[b - 4] >> 16);
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[r] = __builtin_fmaf(d, acc[r], v[r]);
+            }
+        } else {
+        const u32 qd[8] = {it.q0.x, it.q0.y, it.q0.z, it.q0.w, it.q1.x, it.q1.y, it.q1.z, it.q1.w};
         const u32 src_sc = L.upper ? it.hdr.w : it.hdr.y, src_min = L.upper ? it.hdr.w : it.hdr.z;
         const u32 scp = ((src_sc >> L.sh_sc) & L.mask_low) | ((it.hdr.y >> L.sh_top) & L.mask_top);
         const u32 mp = ((src_min >> L.sh_min) & L.mask_low) | ((it.hdr.z >> L.sh_top) & L.mask_top);
@@ -1403,7 +1471,6 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_q4k_wide_kernel(const uint
         const u32 mm0 = __builtin_bit_cast(u32, (h2){m0, m0}), mm1 = __builtin_bit_cast(u32, (h2){m1, m1});
         const uint4 bm_lo = make_uint4(mm0, mm0, mm0, mm0), bm_hi = make_uint4(mm1, mm1, mm1, mm1);
         floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f}, accm = {0.0f, 0.0f, 0.0f, 0.0f};
-        const u32 qd[8] = {it.q0.x, it.q0.y, it.q0.z, it.q0.w, it.q1.x, it.q1.y, it.q1.z, it.q1.w};
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
             const u32 w0 = qd[2 * jj], w1 = qd[2 * jj + 1];
@@ -1426,6 +1493,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_q4k_wide_kernel(const uint
         const float d = half_bits_to_float(it.hdr.x & 0xFFFFu), dmin = half_bits_to_float(it.hdr.x >> 16);
 #pragma unroll
         for (int r = 0; r < 4; r++) v[r] += d * acc[r] - dmin * accm[r];
+        }
         if (step == S - 1) {                                        // the round's last step: this wavefront's share of sixteen rows x sixteen
             wide_red[((size_t)(round % kWideRounds) * WAVES + wave) * 64 + lane] = make_float4(v[0], v[1], v[2], v[3]);
             v[0] = v[1] = v[2] = v[3] = 0.0f;
@@ -1485,7 +1553,6 @@ __global__ __launch_bounds__(WAVES * 64, 4) void gemv_q4k_wide_kernel(const uint
 // scales: four contiguous 1 KB loads and one of 512 bytes per wavefront and tile.  The four MFMAs of a block (low and high nibbles
 // of its two byte halves) share the block's one scale and hence one accumulator: w = d (n - 8) = d (16 acc - 1032 Sx_first16 -
 // 72 Sx_last16) with the low nibbles read as 64 + n / 16 and the high ones as 4 + n / 16 (staged beside the activations per block).
-constexpr size_t kQ40TileBytes = 4608;
 // rounds whose partial sums have an LDS slot of their own (KS > 1): sixteen at 4096 columns (a 128256-row head needs eleven), eight
 // at 14336 columns, where four activation rows leave no room for more
 constexpr int q40_rounds(int tpr) { return tpr >= 28 ? 8 : 16; }
@@ -2062,12 +2129,13 @@ int q4k_wide_mode() {
     if (g_q4k_wide_mode == -2) g_q4k_wide_mode = env_int("ESPRESSO_HIP_Q4K_WIDE", 1);
     return g_q4k_wide_mode;
 }
-template <int IPR, int WAVES, int KS, int XMODE>
+template <int IPR, int WAVES, int KS, int XMODE, bool Q40 = false>
 hipError_t launch_q4k_wide(const KernelArgs &a, int batch, hipStream_t stream, bool *launched) {
     constexpr int RB = WAVES / KS, THREADS = WAVES * 64;
     *launched = false;
-    const size_t lds = (size_t)kWideRounds * WAVES * 64 * sizeof(float4) + (XMODE == 1 ? (size_t)8 * (IPR * 128 + 16) : (size_t)WAVES * 8 * kWideRowBytes);
-    auto kernel = gemv_q4k_wide_kernel<IPR, WAVES, KS, XMODE>;
+    const size_t lds = (size_t)kWideRounds * WAVES * 64 * sizeof(float4) +
+                       (XMODE == 1 ? (size_t)8 * (IPR * 128 + (Q40 ? 32 : 16)) : (size_t)WAVES * 8 * wide_row_bytes(Q40));
+    auto kernel = gemv_q4k_wide_kernel<IPR, WAVES, KS, XMODE, Q40>;
     static size_t configured_lds = 0;
     hipError_t e = ensure_lds(reinterpret_cast<const void *>(kernel), lds, &configured_lds);
     if (e != hipSuccess) return e;
@@ -2090,7 +2158,7 @@ hipError_t launch_q4k_wide(const KernelArgs &a, int batch, hipStream_t stream, b
     return hipGetLastError();
 }
 // Measured (us, eight rows; nibble-B GEMM kernel in brackets): 14336 x 4096 staged rows 11.3, own tiles 12.75 (15.5); 28672 x 4096 18.7,
-// 21.05 (27.4); 4096 x 4096 7.0, 5.9 (7.6); 4096 x 14336 own tiles 12.0 (22.3).  Tuning key "q4k_wide": 0 off, 1 this table, 2 / 3 own tiles / staged rows wherever both exist.
+// 21.05 (27.4); 4096 x 4096 7.0, 5.9 (7.6); 4096 x 14336 own tiles 12.0 (22.3).  Q4_0: 11.3, 12.8 (17.1); 18.9, 21.5 (29.6); 7.2, 5.8 (8.3); 12.3 (24.0).  Tuning key "q4k_wide": 0 off, 1 this table, 2 / 3 own tiles / staged rows wherever both exist.
 hipError_t try_q4k_wide(const KernelArgs &a, int batch, hipStream_t stream, bool *launched) {
     *launched = false;
     if (!a.tiled || !a.x || a.norm_x || a.merge_partials || a.split_x || batch < 5 || batch > 8) return hipSuccess;
@@ -2101,6 +2169,18 @@ hipError_t try_q4k_wide(const KernelArgs &a, int batch, hipStream_t stream, bool
         return launch_q4k_wide<64, 16, 8, 1>(a, batch, stream, launched);
     }
     if (a.cols == 14336) return launch_q4k_wide<224, 8, 8, 2>(a, batch, stream, launched);
+    return hipSuccess;
+}
+hipError_t try_q40_wide(const KernelArgs &a, int batch, hipStream_t stream, bool *launched) {
+    *launched = false;
+    if (!a.tiled || !a.x || a.norm_x || a.merge_partials || a.split_x || batch < 5 || batch > 8) return hipSuccess;
+    if (a.epilogue != EPI_STORE_F32 && a.epilogue != EPI_ADD_RESIDUAL) return hipSuccess;
+    const int form = q4k_wide_mode();
+    if (a.cols == 4096) {
+        if (form == 2 || (form != 3 && a.rows <= 8192)) return launch_q4k_wide<64, 8, 8, 2, true>(a, batch, stream, launched);
+        return launch_q4k_wide<64, 16, 8, 1, true>(a, batch, stream, launched);
+    }
+    if (a.cols == 14336) return launch_q4k_wide<224, 8, 8, 2, true>(a, batch, stream, launched);
     return hipSuccess;
 }
 
@@ -2476,9 +2556,12 @@ bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
     if (batch <= 2) return true;
     // (eight rows of 14336 columns do not fit the kernel's LDS staging in one pass and stay on the nibble-B GEMM kernel)
     // and so do five to eight rows of the long 4096-column matrices, where that kernel measures faster: 15.3 against 17.1 us at 14336 rows)
-    if (w.format == FMT_Q4_0)
-        // (five to eight rows: up to 8192 x 4096 8.7 against 10.7 us on the nibble-B kernel, at 14336 rows 18.9 against 17.1)
-        return w.tiled && q40_mfma_mode() != 0 && (batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (batch <= 8 && w.cols == 4096 && w.rows <= 8192));
+    if (w.format == FMT_Q4_0) {
+        if (!w.tiled || q40_mfma_mode() == 0) return false;
+        if (batch >= 5 && batch <= 8 && q4k_wide_mode() != 0 && (w.cols == 4096 || w.cols == 14336) && w.rows <= q4k_wide_max_rows()) return true;
+        // (five to eight rows without the wide kernel: up to 8192 x 4096 8.7 against 10.7 us on the nibble-B kernel, at 14336 rows 18.9 against 17.1)
+        return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (batch <= 8 && w.cols == 4096 && w.rows <= 8192);
+    }
     if (w.format != FMT_Q4_K || !w.tiled || q4k_mfma_mode() == 0) return false;
     if (batch >= 5 && batch <= 8 && q4k_wide_mode() != 0 && (w.cols == 4096 || w.cols == 14336) && w.rows <= q4k_wide_max_rows()) return true;
     if (batch > 8) return false;
@@ -2544,7 +2627,7 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
     // batches beyond 2 run as successive pairs (each pair re-reads the weights); the matrix-core Q4_K kernel takes four rows at once
     const bool fours = p.batch > 2 && gemv_takes_rows(w, p.batch) && !p.merge_partials;
     for (int b0 = 0, nb = 0; b0 < p.batch; b0 += nb) {
-        const bool wide = fours && w.format == FMT_Q4_K && p.batch - b0 >= 5 && p.batch - b0 <= 8 && q4k_wide_mode() != 0 && w.rows <= q4k_wide_max_rows() &&
+        const bool wide = fours && (w.format == FMT_Q4_K || w.format == FMT_Q4_0) && p.batch - b0 >= 5 && p.batch - b0 <= 8 && q4k_wide_mode() != 0 && w.rows <= q4k_wide_max_rows() &&
                           (p.epilogue == EPI_STORE_F32 || p.epilogue == EPI_ADD_RESIDUAL) && p.x && !p.split_x;
         nb = wide ? p.batch - b0 : fours && p.batch - b0 == 8 ? 8 : fours && p.batch - b0 >= 4 ? 4 : p.batch - b0 >= 2 ? 2 : 1;
         KernelArgs a;
@@ -2585,7 +2668,11 @@ hipError_t launch_gemv(const GemvParams &p, hipStream_t stream) {
             } else e = nb == 1 ? launch_q4k<1>(a, stream) : nb == 2 ? launch_q4k<2>(a, stream) : launch_q4k<4>(a, stream);
             break;
         case FMT_Q4_0:
-            if (nb >= 4) {   // four and eight rows only on the matrix cores; where that kernel declines the shape, two rows at a time
+            if (nb >= 5 && wide) {
+                bool launched = false;
+                e = try_q40_wide(a, nb, stream, &launched);
+                if (e == hipSuccess && !launched) e = hipErrorInvalidValue;
+            } else if (nb >= 4) {   // four and eight rows only on the matrix cores; where that kernel declines the shape, two rows at a time
                 bool launched = false;
                 e = nb == 8 ? try_q40_mfma<8>(a, stream, &launched) : try_q40_mfma<4>(a, stream, &launched);
                 if (e == hipSuccess && !launched) { nb = 2; e = launch_q40<2>(a, stream); }

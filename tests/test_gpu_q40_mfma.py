@@ -16,7 +16,7 @@ def mods():
     import espresso_amd.synthetic as syn
     ops.init()
     yield ll, ops, syn
-    for key, value in (("q40_mfma", -1), ("q4k_mfma_waves", 0), ("q4k_mfma_ks", 0)):
+    for key, value in (("q40_mfma", -1), ("q4k_mfma_waves", 0), ("q4k_mfma_ks", 0), ("q4k_wide", 1)):
         ops.set_tuning(key, value)
 
 
@@ -99,3 +99,39 @@ def test_decoder_with_matrix_core_q4_0_gemvs_matches_oracle(mods, mode):
         assert plain == want
     for r in (g, twin, reference_kernels):
         r.close()
+
+
+@pytest.mark.parametrize("rows,cols", [(16, 4096), (1000, 4096), (14336, 4096), (28672, 4096), (130, 14336), (4096, 14336)])
+def test_five_to_eight_rows_in_one_pass(mods, rows, cols):
+    """Five to eight activation rows on the kernel whose every MFMA contracts one 32-weight block for sixteen weight rows (B = the exact
+    integer q - 8, the block's scale applied to the accumulator): against the oracle's matvec and the kernels it replaces, both ways of
+    staging the activations, residual form, determinism, one-hot columns in every row."""
+    ll, ops, syn = mods
+    for key, value in (("q40_mfma", -1), ("q4k_mfma_waves", 0), ("q4k_mfma_ks", 0)):
+        ops.set_tuning(key, value)
+    mat, deq = q40_matrix(ops, rows, cols, rows + cols + 1)
+    rng = np.random.default_rng(rows + 5)
+    scale = np.abs(deq).max() * np.sqrt(cols)
+    for batch in (5, 6, 7, 8):
+        x = rng.normal(0, 1, (batch, cols)).astype(np.float16)
+        res = rng.normal(0, 1, (batch, rows)).astype(np.float32)
+        want = x.astype(np.float64) @ deq.astype(np.float64).T
+        ops.set_tuning("q4k_wide", 0)
+        base = mat.gemv(x)
+        assert np.abs(base - want).max() <= 3e-4 * scale + 1e-6
+        for form in ((1, 2, 3) if cols == 4096 else (1,)):
+            ops.set_tuning("q4k_wide", form)
+            y = mat.gemv(x)
+            assert np.abs(y - want).max() <= 2e-6 * scale + 1e-6, (batch, form, np.abs(y - want).max() / scale)
+            assert np.array_equal(mat.gemv(x).view(np.uint32), y.view(np.uint32))
+            assert np.abs(mat.gemv(x, res) - (want + res)).max() <= 2e-6 * scale + 1e-5
+    ops.set_tuning("q4k_wide", 1)
+    for j in (0, 3, 4, 15, 16, 31, 32, 255, 256, 511, 512, cols - 1):
+        x = np.zeros((8, cols), np.float16)
+        picks = [(j + 37 * b) % cols for b in range(8)]
+        for b, c in enumerate(picks):
+            x[b, c] = 1.0 + b
+        y = mat.gemv(x)
+        for b, c in enumerate(picks):
+            assert np.abs(y[b] - (1.0 + b) * deq[:, c]).max() <= 1e-6 * (1.0 + b) * max(1.0, np.abs(deq[:, c]).max()) + 1e-7, (j, b)
+    mat.close()

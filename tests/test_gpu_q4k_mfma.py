@@ -70,6 +70,8 @@ def test_five_to_eight_rows_in_one_pass(mods, rows, cols):
     MFMA chain for the minimums), activations staged per workgroup or per wavefront tile: against the oracle's matvec, against the
     nibble-B GEMM kernel it replaces, residual form, determinism, one-hot columns in every row."""
     ll, ops, syn = mods
+    for key, value in (("q4k_mfma", -1), ("q4k_mfma_waves", 0), ("q4k_mfma_ks", 0)):
+        ops.set_tuning(key, value)
     mat, deq = q4k_matrix(ops, rows, cols, rows + cols + 1)
     rng = np.random.default_rng(rows + 5)
     scale = np.abs(deq).max() * np.sqrt(cols)
