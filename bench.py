@@ -182,7 +182,7 @@ MICRO_SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
 
 
 def run_microbench(shapes=None, formats=("q4_k", "q4_0"), batches=(1, 2, 4, 8), launches=100) -> dict:
-    """Isolated dequant-GEMV (batch 1, 2: wave-per-row-pair kernel; batch 8: MFMA kernel) for Q4_K and Q4_0, weights
+    """Isolated dequant-GEMV (matrix-core GEMV kernels: one to four rows, and five to eight rows in one pass) for Q4_K and Q4_0, weights
     rotated through enough copies that no launch finds them in the last-level cache."""
     import espresso_amd.ops as ops
     from espresso_amd import _lib
