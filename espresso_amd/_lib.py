@@ -133,6 +133,8 @@ def _declare_llama(L: C.CDLL) -> None:
     L.esp_llama_set_merged_attention.restype = i32
     L.esp_llama_set_merged_attention.argtypes = [vp, i32]
     L.esp_matrix_resident_bytes.restype = C.c_size_t
+    L.esp_matrix_read_tiled.restype = C.c_longlong
+    L.esp_matrix_read_tiled.argtypes = [vp, vp, C.c_size_t]
     L.esp_matrix_resident_bytes.argtypes = [vp]
     L.esp_llama_resident_weight_bytes.restype = C.c_size_t
     L.esp_llama_resident_weight_bytes.argtypes = [vp]

@@ -97,6 +97,18 @@ void esp_matrix_free(ESPMatrix *matrix) {
 size_t esp_matrix_bytes(const ESPMatrix *matrix) { return matrix ? matrix->m.bytes() : 0; }
 size_t esp_matrix_resident_bytes(const ESPMatrix *matrix) { return matrix ? matrix->m.resident_bytes() : 0; }
 
+long long esp_matrix_read_tiled(const ESPMatrix *matrix, void *out, size_t capacity) {
+    if (!matrix || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "matrix_read_tiled: null pointer");
+    const size_t bytes = matrix->m.tiled ? matrix->m.tiled_bytes() : 0;
+    if (bytes == 0) return 0;
+    if (capacity < bytes) return fail(ESP_ERR_OUT_OF_RANGE, "matrix_read_tiled: %zu bytes needed", bytes);
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    const hipError_t e = hipMemcpy(out, matrix->m.tiled, bytes, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return fail_hip(e, "matrix_read_tiled");
+    return (long long)bytes;
+}
+
 int esp_matrix_dequantize(const ESPMatrix *matrix, float *out) {
     if (!matrix || !out) return fail(ESP_ERR_INVALID_ARGUMENT, "matrix_dequantize: null pointer");
     int rc = ensure_init();

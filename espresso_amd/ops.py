@@ -69,6 +69,15 @@ class Matrix:
     def resident_bytes(self) -> int:
         return int(_lib.load_library().esp_matrix_resident_bytes(self._h))
 
+    def read_tiled(self) -> np.ndarray:
+        """The tiled copy the matrix-core GEMVs read, as bytes (empty when the matrix keeps none)."""
+        n = self.resident_bytes - self.bytes
+        out = np.empty(max(n, 1), dtype=np.uint8)
+        got = _lib.load_library().esp_matrix_read_tiled(self._h, _ptr(out), out.size)
+        if got < 0:
+            _lib.check(int(got))
+        return out[:got]
+
     def dequantize(self) -> np.ndarray:
         out = np.empty(self.rows * self.cols, dtype=np.float32)
         _lib.check(_lib.load_library().esp_matrix_dequantize(self._h, _ptr(out)))

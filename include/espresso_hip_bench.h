@@ -44,6 +44,10 @@ int esp_set_tuning(const char *key, int value);
 /* Measurement aid with no counterpart in the reference: a kernel that only streams `bytes` (>= 1 MiB, a
  * multiple of 16) from HBM with 128-bit loads, `iters` times; reports GB/s.  bench.py prints it next to the
  * GEMV bandwidth so that fractions of the published peak can be read against what a plain reader gets. */
+/* Diagnostic: copies the matrix's tiled copy (the second resident format, read by the matrix-core GEMVs) to `out`; returns the number of
+ * bytes (esp_matrix_resident_bytes - esp_matrix_bytes; 0 when the matrix keeps none) or a negative ESP_ERR_* code.  tests/ rebuild the tiles
+ * from the GGUF blocks with numpy and compare byte for byte. */
+long long esp_matrix_read_tiled(const ESPMatrix *matrix, void *out, size_t capacity);
 int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s);
 /* The ceiling for ONE GEMV launch: a kernel with a persistent Q4_K GEMV's grid (`workgroups` of `wavefronts` = 4 or 8) and its
  * loads (a wavefront takes items of `pair_bytes`, a 2304-byte weight tile of the matrix-core kernel or a pair of rows of the
