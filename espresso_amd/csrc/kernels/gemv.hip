@@ -2169,6 +2169,11 @@ hipError_t try_q4k_wide(const KernelArgs &a, int batch, hipStream_t stream, bool
         return launch_q4k_wide<64, 16, 8, 1>(a, batch, stream, launched);
     }
     if (a.cols == 14336) return launch_q4k_wide<224, 8, 8, 2>(a, batch, stream, launched);
+    // the registry's other widths (see try_q4k_mfma): own tiles, the K split that leaves whole super-blocks per wavefront
+    if (a.cols == 1024) return launch_q4k_wide<16, 8, 4, 2>(a, batch, stream, launched);
+    if (a.cols == 2048) return launch_q4k_wide<32, 8, 8, 2>(a, batch, stream, launched);
+    if (a.cols == 3072) return launch_q4k_wide<48, 8, 4, 2>(a, batch, stream, launched);
+    if (a.cols == 8192) return launch_q4k_wide<128, 8, 8, 2>(a, batch, stream, launched);
     return hipSuccess;
 }
 hipError_t try_q40_wide(const KernelArgs &a, int batch, hipStream_t stream, bool *launched) {
@@ -2563,7 +2568,8 @@ bool gemv_takes_rows(const DeviceMatrix &w, int batch) {
         return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (batch <= 8 && w.cols == 4096 && w.rows <= 8192);
     }
     if (w.format != FMT_Q4_K || !w.tiled || q4k_mfma_mode() == 0) return false;
-    if (batch >= 5 && batch <= 8 && q4k_wide_mode() != 0 && (w.cols == 4096 || w.cols == 14336) && w.rows <= q4k_wide_max_rows()) return true;
+    if (batch >= 5 && batch <= 8 && q4k_wide_mode() != 0 && (w.cols == 4096 || w.cols == 14336 || q4k_registry_width(w.cols)) && w.rows <= q4k_wide_max_rows())
+        return true;
     if (batch > 8) return false;
     return batch <= 4 ? (w.cols == 4096 || w.cols == 14336) : (w.cols == 4096 && w.rows <= q4k_mfma_rows8_max());
 }

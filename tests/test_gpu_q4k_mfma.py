@@ -64,7 +64,8 @@ def test_matches_oracle_and_dot_product_kernels(mods, rows, cols):
     mat.close()
 
 
-@pytest.mark.parametrize("rows,cols", [(16, 4096), (1000, 4096), (14336, 4096), (28672, 4096), (130, 14336), (4096, 14336)])
+@pytest.mark.parametrize("rows,cols", [(16, 4096), (1000, 4096), (14336, 4096), (28672, 4096), (130, 14336), (4096, 14336),
+                                       (2048, 1024), (100, 2048), (3072, 3072), (2050, 8192)])
 def test_five_to_eight_rows_in_one_pass(mods, rows, cols):
     """Five to eight activation rows on the kernel that folds the sub-block scales into the B operand (exact integer sc * q, a second
     MFMA chain for the minimums), activations staged per workgroup or per wavefront tile: against the oracle's matvec, against the
