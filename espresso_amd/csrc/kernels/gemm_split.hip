@@ -22,6 +22,7 @@
 #include "../common.h"
 #include "decode_ops.h"
 #include <atomic>
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -50,6 +51,7 @@ struct SplitGemmArgs {
     float *partial;                 // [splits][M][N] when gridDim.y > 1
     int tiles_per_split;            // a multiple of four
     uint16_t *sw_hi, *sw_lo;        // SiLU(gate) * up as a split pair [M][N / 2] instead of y (no split-K)
+    const uint8_t *tiled;           // the matrix-core GEMV's tiled copy (gemm_q4k_split_regb_kernel reads its weights there)
 };
 
 __device__ __forceinline__ h2 as_h2(u32 v) { return __builtin_bit_cast(h2, v); }
@@ -383,6 +385,282 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_kernel(SplitGemmArgs 
         }
 }
 
+// ---- the same product with the weights kept out of LDS -------------------------------------------------------------------------
+// Counters and timing-only builds of the kernel above say where its time goes: the 64 x 64 tile of a wavefront reads 6 KB of
+// fragments per eight MFMAs (LDS busier than the matrix cores), a quarter of the time is the weights' way through LDS (dequantise,
+// write, barrier, read back) and a sixth is the barrier itself.  Here a wavefront builds its B fragments in registers, straight from
+// the tiled copy the GEMV reads (lane (n, kg) of a 32-column block fetches bytes 8 kg .. 8 kg + 7 of the first and of the second half
+// of its row's 32-byte chunk: eight-byte loads that cover whole 256-byte runs of the tile), so only the activations go through LDS
+// and a wavefront can own 64 activation rows x 128 weight rows: four A fragments per sixteen MFMAs.  The lo plane accumulates into
+// the same registers as the hi plane, against the B operand scaled by 2^-11 (sc * q / 2048 is exact in fp16 too), so one accumulator
+// set of 128 registers and one of totals suffice.  Workgroup = 2 x 2 wavefronts = 128 activation rows x 256 weight rows.
+constexpr int NT2 = 256;
+constexpr size_t kLdsBytesRegB = 4 * kTileHalfs * 2 + 2 * 128 * 16 * 2;
+
+__global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemmArgs a) {
+    constexpr int RB = 2, THREADS = kThreads, XP = 1024 / THREADS;   // 32-row blocks per wavefront; sixteen-byte pieces of a plane's tile per thread
+    extern __shared__ uint4 smem_raw[];
+    _Float16 *xh = reinterpret_cast<_Float16 *>(smem_raw);     // [2][128 * LDK]
+    _Float16 *xl = xh + 2 * kTileHalfs;                          // [2][128 * LDK]
+    _Float16 *xs = xl + 2 * kTileHalfs;                          // [2][128][16]   (hi of S_0..S_7, lo of S_0..S_7) of the row
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;             // wm: which 32 RB rows of the tile
+    const int n0 = blockIdx.x * NT2, m0 = blockIdx.z * MT;
+    const int tiles = a.K / KT, sbs = a.K / 256;
+    const int t_begin = blockIdx.y * a.tiles_per_split;
+    const int t_end = t_begin + a.tiles_per_split < tiles ? t_begin + a.tiles_per_split : tiles;
+    const int t_last = t_end - 1;
+    const int bn = lane & 31, kg = lane >> 5;
+
+    // weights: column block cb of this wavefront = weight rows n0 + 128 wn + 32 cb + (0..31); this lane's row of it, clamped (never stored)
+    const uint8_t *wrow[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; cb++) {
+        const int row = n0 + 128 * wn + 32 * cb + bn < a.N ? n0 + 128 * wn + 32 * cb + bn : a.N - 1;
+        wrow[cb] = a.tiled + (size_t)(row >> 4) * sbs * 2304 + 16 * (row & 15);
+    }
+    struct WRaw { uint2 a0, a1, a2, a3, b0, b1, b2, b3; };   // per column block: eight bytes of the chunk's first / second sixteen
+    auto fetch_w = [&](int tile) __attribute__((always_inline)) {
+        WRaw r;
+        const size_t o = (size_t)(tile >> 2) * 2304 + 256 + 256 * (tile & 3) + 8 * kg;
+        r.a0 = *reinterpret_cast<const uint2 *>(wrow[0] + o); r.b0 = *reinterpret_cast<const uint2 *>(wrow[0] + o + 1024);
+        r.a1 = *reinterpret_cast<const uint2 *>(wrow[1] + o); r.b1 = *reinterpret_cast<const uint2 *>(wrow[1] + o + 1024);
+        r.a2 = *reinterpret_cast<const uint2 *>(wrow[2] + o); r.b2 = *reinterpret_cast<const uint2 *>(wrow[2] + o + 1024);
+        r.a3 = *reinterpret_cast<const uint2 *>(wrow[3] + o); r.b3 = *reinterpret_cast<const uint2 *>(wrow[3] + o + 1024);
+        return r;
+    };
+    struct Hdrs { uint4 h0, h1, h2, h3; };
+    auto fetch_hdr = [&](int sb) __attribute__((always_inline)) {
+        Hdrs h;
+        const size_t o = (size_t)(sb < sbs ? sb : sbs - 1) * 2304;
+        h.h0 = *reinterpret_cast<const uint4 *>(wrow[0] + o); h.h1 = *reinterpret_cast<const uint4 *>(wrow[1] + o);
+        h.h2 = *reinterpret_cast<const uint4 *>(wrow[2] + o); h.h3 = *reinterpret_cast<const uint4 *>(wrow[3] + o);
+        return h;
+    };
+
+    // activations: piece i of a thread = row (tid / 8) + 32 i of the tile, eight columns (tid % 8) * 8 .. of it (as in the kernel above)
+    const unsigned x_col = (unsigned)(tid & 7) * 8;
+    constexpr int XSTEP = THREADS / 8;   // rows between a thread's pieces
+    auto x_row_offset = [&](int i) __attribute__((always_inline)) {
+        const int row = (tid >> 3) + XSTEP * i;
+        return (unsigned)(m0 + row < a.M ? m0 + row : a.M - 1) * (unsigned)a.K + x_col;
+    };
+    const unsigned xo0 = x_row_offset(0), xo1 = x_row_offset(1), xo2 = x_row_offset(XP > 2 ? 2 : 0), xo3 = x_row_offset(XP > 2 ? 3 : 0);
+    struct XTile { uint4 h0, h1, h2, h3, l0, l1, l2, l3; };
+    auto fetch_x = [&](int tile) __attribute__((always_inline)) {
+        const unsigned t = (unsigned)tile * KT;
+        XTile x;
+        x.h0 = *reinterpret_cast<const uint4 *>(a.xh + (xo0 + t)); x.l0 = *reinterpret_cast<const uint4 *>(a.xl + (xo0 + t));
+        x.h1 = *reinterpret_cast<const uint4 *>(a.xh + (xo1 + t)); x.l1 = *reinterpret_cast<const uint4 *>(a.xl + (xo1 + t));
+        if constexpr (XP > 2) {
+            x.h2 = *reinterpret_cast<const uint4 *>(a.xh + (xo2 + t)); x.l2 = *reinterpret_cast<const uint4 *>(a.xl + (xo2 + t));
+            x.h3 = *reinterpret_cast<const uint4 *>(a.xh + (xo3 + t)); x.l3 = *reinterpret_cast<const uint4 *>(a.xl + (xo3 + t));
+        }
+        return x;
+    };
+    const int xs_row = m0 + ((tid & 255) >> 1) < a.M ? m0 + ((tid & 255) >> 1) : a.M - 1;
+    auto fetch_sums = [&](int sb) __attribute__((always_inline)) {
+        return reinterpret_cast<const uint4 *>(a.xs + ((size_t)xs_row * sbs + (sb < sbs ? sb : sbs - 1)) * 16)[tid & 1];
+    };
+    auto store_x = [&](const XTile &x, int buf) __attribute__((always_inline)) {
+        const int o = buf * (int)kTileHalfs + (tid >> 3) * LDK + (tid & 7) * 8;
+        *reinterpret_cast<uint4 *>(xh + o) = x.h0; *reinterpret_cast<uint4 *>(xl + o) = x.l0;
+        *reinterpret_cast<uint4 *>(xh + o + XSTEP * LDK) = x.h1; *reinterpret_cast<uint4 *>(xl + o + XSTEP * LDK) = x.l1;
+        if constexpr (XP > 2) {
+            *reinterpret_cast<uint4 *>(xh + o + 64 * LDK) = x.h2; *reinterpret_cast<uint4 *>(xl + o + 64 * LDK) = x.l2;
+            *reinterpret_cast<uint4 *>(xh + o + 96 * LDK) = x.h3; *reinterpret_cast<uint4 *>(xl + o + 96 * LDK) = x.l3;
+        }
+    };
+    auto store_sums = [&](const uint4 &v, int sb) __attribute__((always_inline)) {   // with 512 threads both halves write the same values
+        *reinterpret_cast<uint4 *>(xs + (sb & 1) * 128 * 16 + ((tid & 255) >> 1) * 16 + 8 * (tid & 1)) = v;
+    };
+
+    floatx16 tot[RB][4], acc[RB][4];   // acc starts every super-block from the zero C operand of its first MFMAs
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) tot[i][j][r] = 0.0f;
+    const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // constants of the nibble trick, hidden from the optimiser so that (w & mask) | magic stays one v_and_or_b32
+    u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+    asm volatile("" : "+s"(mask_lo), "+s"(mask_hi));
+    asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
+
+    // prologue: tile t_begin staged, t_begin + 1 in registers, weights of both in registers
+    const int t_second = t_begin + 1 < t_last ? t_begin + 1 : t_last;
+    WRaw w0 = fetch_w(t_begin), w1 = fetch_w(t_second);
+    Hdrs hdr = fetch_hdr(t_begin >> 2);
+    {
+        const XTile xfirst = fetch_x(t_begin);
+        store_sums(fetch_sums(t_begin >> 2), t_begin >> 2);
+        store_x(xfirst, 0);
+    }
+    XTile xn = fetch_x(t_second);
+    uint4 sums_next = fetch_sums((t_begin >> 2) + 1);
+    Hdrs hdr_next = fetch_hdr((t_begin >> 2) + 1);
+    __syncthreads();
+
+    const h2 kTwoM11 = {(_Float16)kUnscale, (_Float16)kUnscale};
+    auto tile_step = [&](auto u_c, int t) __attribute__((always_inline)) {
+        constexpr int u = decltype(u_c)::value, buf = u & 1;
+        const _Float16 *xhb = xh + (size_t)buf * kTileHalfs, *xlb = xl + (size_t)buf * kTileHalfs;
+        WRaw &w = buf == 0 ? w0 : w1;
+        const uint4 hd[4] = {hdr.h0, hdr.h1, hdr.h2, hdr.h3};
+        const uint2 wa[4] = {w.a0, w.a1, w.a2, w.a3}, wb[4] = {w.b0, w.b1, w.b2, w.b3};
+        // scale constants of the tile's two sub-blocks per column block: (offset + q) * sc - offset * sc, and the same / 2048
+        h2 s_lo[4], o_lo[4], s_hi[4], o_hi[4];
+#pragma unroll
+        for (int cb = 0; cb < 4; cb++) {
+            u32 sc, m;
+            q4k_scale_min(hd[cb], 2 * u, sc, m);
+            const _Float16 f0 = (_Float16)(unsigned short)sc;
+            s_lo[cb] = h2{f0, f0}; o_lo[cb] = s_lo[cb] * h2{(_Float16)-1024.0f, (_Float16)-1024.0f};
+            q4k_scale_min(hd[cb], 2 * u + 1, sc, m);
+            const _Float16 f1 = (_Float16)(unsigned short)sc;
+            s_hi[cb] = h2{f1, f1}; o_hi[cb] = s_hi[cb] * h2{(_Float16)-64.0f, (_Float16)-64.0f};
+        }
+        // the next tile goes to the other LDS buffer (its activations were fetched during the previous tile), then its successor is fetched
+        store_x(xn, buf ^ 1);
+        if (u == 3) store_sums(sums_next, (t >> 2) + 1);
+        {
+            const int ahead = t + 2 < t_last ? t + 2 : t_last;
+            xn = fetch_x(ahead);
+            if (u == 3) sums_next = fetch_sums((t >> 2) + 2);
+        }
+        struct Frags { half8 h0, h1, l0, l1; };
+        auto load_frags = [&](int ks) __attribute__((always_inline)) {
+            const int ra = (wm * 32 * RB + bn) * LDK + ks * 16 + 8 * kg;
+            Frags f;
+            f.h0 = *reinterpret_cast<const half8 *>(xhb + ra); f.l0 = *reinterpret_cast<const half8 *>(xlb + ra);
+            if constexpr (RB == 2) { f.h1 = *reinterpret_cast<const half8 *>(xhb + ra + 32 * LDK); f.l1 = *reinterpret_cast<const half8 *>(xlb + ra + 32 * LDK); }
+            else { f.h1 = f.h0; f.l1 = f.l0; }
+            return f;
+        };
+        // the super-block's fold, per column block, right behind that block's last MFMAs (the other blocks' MFMAs run meanwhile):
+        // total += d * sums - dmin * sum_j m_j S_j (one MFMA: K = (8 x hi of S_j, 8 x lo of S_j * 2048) against (m_0..m_7, m_0..m_7 / 2048))
+        half8 fs[RB];
+        if (u == 3) {
+            const int sbuf = (t >> 2) & 1;
+#pragma unroll
+            for (int i = 0; i < RB; i++) fs[i] = *reinterpret_cast<const half8 *>(xs + (size_t)sbuf * 128 * 16 + ((wm * RB + i) * 32 + bn) * 16 + 8 * kg);
+        }
+        auto fold = [&](int cb) __attribute__((always_inline)) {
+            const float mscale = kg ? kUnscale : 1.0f;
+            float mv[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) { u32 sc, m; q4k_scale_min(hd[cb], j, sc, m); mv[j] = (float)m * mscale; }
+            const uint4 mq = make_uint4(pack_half2(mv[0], mv[1]), pack_half2(mv[2], mv[3]), pack_half2(mv[4], mv[5]), pack_half2(mv[6], mv[7]));
+            const float d = half_bits_to_float(hd[cb].x & 0xFFFFu), dmin = half_bits_to_float(hd[cb].x >> 16);
+#pragma unroll
+            for (int i = 0; i < RB; i++) {
+                const floatx16 am = __builtin_amdgcn_mfma_f32_32x32x16_f16(fs[i], __builtin_bit_cast(half8, mq), zero16, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; r++) tot[i][cb][r] = __builtin_fmaf(-dmin, am[r], __builtin_fmaf(d, acc[i][cb][r], tot[i][cb][r]));
+            }
+        };
+        Frags fnext = load_frags(0);
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const Frags f = fnext;
+            if (ks < 3) fnext = load_frags(ks + 1);
+            const half8 fh0 = f.h0, fh1 = f.h1, fl0 = f.l0, fl1 = f.l1;
+#pragma unroll
+            for (int cb = 0; cb < 4; cb++) {
+                const uint2 q = (ks & 1) ? wb[cb] : wa[cb];   // k 0..15 and 32..47 of the tile: the chunk's first sixteen bytes; 16..31, 48..63: its second
+                const u32 x0 = q.x, x1 = q.y, x08 = x0 >> 8, x18 = x1 >> 8;
+                uint4 bq, bs;
+                if (ks < 2) {
+                    const h2 v0 = as_h2((x0 & mask_lo) | magic_lo), v1 = as_h2((x08 & mask_lo) | magic_lo);
+                    const h2 v2 = as_h2((x1 & mask_lo) | magic_lo), v3 = as_h2((x18 & mask_lo) | magic_lo);
+                    const h2 p0 = __builtin_elementwise_fma(v0, s_lo[cb], o_lo[cb]), p1 = __builtin_elementwise_fma(v1, s_lo[cb], o_lo[cb]);
+                    const h2 p2 = __builtin_elementwise_fma(v2, s_lo[cb], o_lo[cb]), p3 = __builtin_elementwise_fma(v3, s_lo[cb], o_lo[cb]);
+                    bq = make_uint4(as_u32(p0), as_u32(p1), as_u32(p2), as_u32(p3));
+                    bs = make_uint4(as_u32(p0 * kTwoM11), as_u32(p1 * kTwoM11), as_u32(p2 * kTwoM11), as_u32(p3 * kTwoM11));
+                } else {
+                    const h2 v0 = as_h2((x0 & mask_hi) | magic_hi), v1 = as_h2((x08 & mask_hi) | magic_hi);
+                    const h2 v2 = as_h2((x1 & mask_hi) | magic_hi), v3 = as_h2((x18 & mask_hi) | magic_hi);
+                    const h2 p0 = __builtin_elementwise_fma(v0, s_hi[cb], o_hi[cb]), p1 = __builtin_elementwise_fma(v1, s_hi[cb], o_hi[cb]);
+                    const h2 p2 = __builtin_elementwise_fma(v2, s_hi[cb], o_hi[cb]), p3 = __builtin_elementwise_fma(v3, s_hi[cb], o_hi[cb]);
+                    bq = make_uint4(as_u32(p0), as_u32(p1), as_u32(p2), as_u32(p3));
+                    bs = make_uint4(as_u32(p0 * kTwoM11), as_u32(p1 * kTwoM11), as_u32(p2 * kTwoM11), as_u32(p3 * kTwoM11));
+                }
+                const half8 fb = __builtin_bit_cast(half8, bq), fbs = __builtin_bit_cast(half8, bs);
+                acc[0][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh0, fb, (u == 0 && ks == 0) ? zero16 : acc[0][cb], 0, 0, 0);
+                if constexpr (RB == 2) acc[1][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh1, fb, (u == 0 && ks == 0) ? zero16 : acc[1][cb], 0, 0, 0);
+                acc[0][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl0, fbs, acc[0][cb], 0, 0, 0);
+                if constexpr (RB == 2) acc[1][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl1, fbs, acc[1][cb], 0, 0, 0);
+                if (u == 3 && ks == 3 && cb > 0) fold(cb - 1);
+            }
+        }
+        if (u == 3) fold(3);
+        // this slot's weights are used up: the tile two ahead goes into it
+        {
+            const int ahead = t + 2 < t_last ? t + 2 : t_last;
+            w = fetch_w(ahead);
+        }
+        if (u == 3) {
+            hdr = hdr_next;
+            hdr_next = fetch_hdr((t >> 2) + 2);
+        }
+        __syncthreads();
+    };
+    for (int t0 = t_begin; t0 < t_end; t0 += 4) {
+        tile_step(std::integral_constant<int, 0>{}, t0);
+        tile_step(std::integral_constant<int, 1>{}, t0 + 1);
+        tile_step(std::integral_constant<int, 2>{}, t0 + 2);
+        tile_step(std::integral_constant<int, 3>{}, t0 + 3);
+    }
+
+    // accumulator r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of the 32 x 32 tile
+    if (a.sw_hi) {
+#pragma unroll
+        for (int i = 0; i < RB; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int n = n0 + 128 * wn + 32 * j + bn;
+                const bool odd = lane & 1;
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    const float a0 = tot[i][j][2 * k], a1 = tot[i][j][2 * k + 1];
+                    const float p0 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a0), 0xB1, 0xF, 0xF, false));
+                    const float p1 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a1), 0xB1, 0xF, 0xF, false));
+                    const float g = odd ? p1 : a0, up = odd ? a1 : p0;
+                    const int r = 2 * k + (odd ? 1 : 0);
+                    const int m = m0 + (wm * RB + i) * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
+                    if (m < a.M && (n | 1) < a.N) {
+                        const float hg = __fmul_rn(0.5f, g);
+                        const float silu = __fmul_rn(hg, __fadd_rn(1.0f, tanhf(hg)));
+                        const float act = __fmul_rn(silu, up);
+                        const _Float16 hi = (_Float16)act;
+                        const int unit = n / 2, slot = unit & 3;   // the planes' order inside fours: (0, 2, 1, 3)
+                        const size_t o = (size_t)m * (a.N / 2) + (unit & ~3) + (slot == 1 ? 2 : slot == 2 ? 1 : slot);
+                        a.sw_hi[o] = __builtin_bit_cast(uint16_t, hi);
+                        a.sw_lo[o] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(__fsub_rn(act, (float)hi), kScale));
+                    }
+                }
+            }
+        return;
+    }
+    const bool split = gridDim.y > 1;
+    float *out = split ? a.partial + (size_t)blockIdx.y * a.M * a.N : a.y;
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int n = n0 + 128 * wn + 32 * j + bn;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + (wm * RB + i) * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
+                if (m < a.M && n < a.N) {
+                    const size_t o = (size_t)m * a.N + n;
+                    out[o] = (!split && a.residual) ? a.residual[o] + tot[i][j][r] : tot[i][j][r];
+                }
+            }
+        }
+}
+
 // y = (residual +) sum over splits of partial, in split order
 __global__ void split_gemm_reduce_kernel(const float *partial, int splits, size_t count, const float *residual, float *y) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -542,7 +820,13 @@ hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream) {
     SplitGemmArgs a{};
     a.qs = w.qs; a.qs_row_bytes = w.qs_row_bytes; a.N = w.rows; a.K = w.cols; a.M = p.rows;
     a.xh = p.x.hi; a.xl = p.x.lo; a.xs = p.x.sums; a.y = p.y; a.residual = p.residual; a.partial = p.workspace;
-    const int tiles = a.K / KT, blocks = ((a.N + NT - 1) / NT) * ((a.M + MT - 1) / MT);
+    a.tiled = w.tiled;
+    // weights in registers (workgroups of 128 x 256) wherever the matrix keeps the tiled copy; ESPRESSO_HIP_SPLIT_GEMM_LDS_WEIGHTS=1
+    // restores the kernel that stages them
+    static const bool lds_weights = [] { const char *e = getenv("ESPRESSO_HIP_SPLIT_GEMM_LDS_WEIGHTS"); return e && atoi(e) != 0; }();
+    const bool regb = w.tiled != nullptr && !lds_weights;
+    const int nt = regb ? NT2 : NT;
+    const int tiles = a.K / KT, blocks = ((a.N + nt - 1) / nt) * ((a.M + MT - 1) / MT);
     // split K until the grid fills the chip (one workgroup per compute unit is resident), whole super-blocks per split
     int splits = 1;
     if (!swiglu && p.workspace) {
@@ -560,14 +844,16 @@ hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream) {
     hipError_t e = hipGetDevice(&device);
     if (e != hipSuccess) return e;
     const uint64_t bit = 1ull << (device & 63);
-    auto kernel = gemm_q4k_split_kernel<2>;
     if (!(raised.load(std::memory_order_acquire) & bit)) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_regb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytesRegB);
         if (e != hipSuccess) return e;
         raised.fetch_or(bit, std::memory_order_release);
     }
-    dim3 grid((a.N + NT - 1) / NT, splits, (a.M + MT - 1) / MT);
-    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kLdsBytes, stream, a);
+    dim3 grid((a.N + nt - 1) / nt, splits, (a.M + MT - 1) / MT);
+    if (regb) hipLaunchKernelGGL(gemm_q4k_split_regb_kernel, grid, dim3(kThreads), kLdsBytesRegB, stream, a);
+    else hipLaunchKernelGGL(gemm_q4k_split_kernel<2>, grid, dim3(kThreads), kLdsBytes, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (swiglu) {
