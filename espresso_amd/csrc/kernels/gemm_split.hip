@@ -393,18 +393,26 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_kernel(SplitGemmArgs 
 // of its row's 32-byte chunk: eight-byte loads that cover whole 256-byte runs of the tile), so only the activations go through LDS
 // and a wavefront can own 64 activation rows x 128 weight rows: four A fragments per sixteen MFMAs.  The lo plane accumulates into
 // the same registers as the hi plane, against the B operand scaled by 2^-11 (sc * q / 2048 is exact in fp16 too), so one accumulator
-// set of 128 registers and one of totals suffice.  Workgroup = 2 x 2 wavefronts = 128 activation rows x 256 weight rows.
+// set of 128 registers and one of totals suffice.  Workgroup = four wavefronts = 128 activation rows x 256 weight rows.
+// Counters of this kernel: a wavefront's vector-ALU instructions and its MFMAs take turns (39 % + 44 % of its cycles; forcing an MFMA /
+// vector interleave in the instruction order changes nothing, a second wavefront per SIMD with half the tile is slower), so what counts
+// is the vector work per MFMA: with every wavefront on all 128 rows and 64 weight rows (RB x CB = 4 x 2) a B fragment serves eight
+// MFMAs instead of four: gate|up of a 512-row block 356 -> 324 us (the kernel above: 421 on the same boxes).
 constexpr int NT2 = 256;
 constexpr size_t kLdsBytesRegB = 4 * kTileHalfs * 2 + 2 * 128 * 16 * 2;
 
+// RB x CB = 32-row blocks of activations x 32-row blocks of weights per wavefront (eight in all: 128 accumulator registers).
+template <int RB, int CB>
 __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemmArgs a) {
-    constexpr int RB = 2, THREADS = kThreads, XP = 1024 / THREADS;   // 32-row blocks per wavefront; sixteen-byte pieces of a plane's tile per thread
+    static_assert(RB * CB == 8 && (RB == 2 || RB == 4), "a wavefront owns eight 32 x 32 tiles");
+    constexpr int THREADS = kThreads, XP = 1024 / THREADS;   // sixteen-byte pieces of a plane's tile per thread
+    constexpr int NW = 8 / CB;                               // wavefronts along the weight rows
     extern __shared__ uint4 smem_raw[];
     _Float16 *xh = reinterpret_cast<_Float16 *>(smem_raw);     // [2][128 * LDK]
     _Float16 *xl = xh + 2 * kTileHalfs;                          // [2][128 * LDK]
     _Float16 *xs = xl + 2 * kTileHalfs;                          // [2][128][16]   (hi of S_0..S_7, lo of S_0..S_7) of the row
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;             // wm: which 32 RB rows of the tile
+    const int wm = wave / NW, wn = wave % NW;            // wm: which 32 RB activation rows of the tile, wn: which 32 CB weight rows
     const int n0 = blockIdx.x * NT2, m0 = blockIdx.z * MT;
     const int tiles = a.K / KT, sbs = a.K / 256;
     const int t_begin = blockIdx.y * a.tiles_per_split;
@@ -412,11 +420,12 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
     const int t_last = t_end - 1;
     const int bn = lane & 31, kg = lane >> 5;
 
-    // weights: column block cb of this wavefront = weight rows n0 + 128 wn + 32 cb + (0..31); this lane's row of it, clamped (never stored)
+    // weights: column block cb of this wavefront = weight rows n0 + 32 CB wn + 32 cb + (0..31); this lane's row of it, clamped (never stored)
     const uint8_t *wrow[4];
 #pragma unroll
     for (int cb = 0; cb < 4; cb++) {
-        const int row = n0 + 128 * wn + 32 * cb + bn < a.N ? n0 + 128 * wn + 32 * cb + bn : a.N - 1;
+        const int want = n0 + 32 * CB * wn + 32 * (cb < CB ? cb : 0) + bn;
+        const int row = want < a.N ? want : a.N - 1;
         wrow[cb] = a.tiled + (size_t)(row >> 4) * sbs * 2304 + 16 * (row & 15);
     }
     struct WRaw { uint2 a0, a1, a2, a3, b0, b1, b2, b3; };   // per column block: eight bytes of the chunk's first / second sixteen
@@ -425,8 +434,10 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
         const size_t o = (size_t)(tile >> 2) * 2304 + 256 + 256 * (tile & 3) + 8 * kg;
         r.a0 = *reinterpret_cast<const uint2 *>(wrow[0] + o); r.b0 = *reinterpret_cast<const uint2 *>(wrow[0] + o + 1024);
         r.a1 = *reinterpret_cast<const uint2 *>(wrow[1] + o); r.b1 = *reinterpret_cast<const uint2 *>(wrow[1] + o + 1024);
-        r.a2 = *reinterpret_cast<const uint2 *>(wrow[2] + o); r.b2 = *reinterpret_cast<const uint2 *>(wrow[2] + o + 1024);
-        r.a3 = *reinterpret_cast<const uint2 *>(wrow[3] + o); r.b3 = *reinterpret_cast<const uint2 *>(wrow[3] + o + 1024);
+        if constexpr (CB > 2) {
+            r.a2 = *reinterpret_cast<const uint2 *>(wrow[2] + o); r.b2 = *reinterpret_cast<const uint2 *>(wrow[2] + o + 1024);
+            r.a3 = *reinterpret_cast<const uint2 *>(wrow[3] + o); r.b3 = *reinterpret_cast<const uint2 *>(wrow[3] + o + 1024);
+        } else { r.a2 = r.a3 = r.a0; r.b2 = r.b3 = r.b0; }
         return r;
     };
     struct Hdrs { uint4 h0, h1, h2, h3; };
@@ -434,7 +445,8 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
         Hdrs h;
         const size_t o = (size_t)(sb < sbs ? sb : sbs - 1) * 2304;
         h.h0 = *reinterpret_cast<const uint4 *>(wrow[0] + o); h.h1 = *reinterpret_cast<const uint4 *>(wrow[1] + o);
-        h.h2 = *reinterpret_cast<const uint4 *>(wrow[2] + o); h.h3 = *reinterpret_cast<const uint4 *>(wrow[3] + o);
+        if constexpr (CB > 2) { h.h2 = *reinterpret_cast<const uint4 *>(wrow[2] + o); h.h3 = *reinterpret_cast<const uint4 *>(wrow[3] + o); }
+        else { h.h2 = h.h3 = h.h0; }
         return h;
     };
 
@@ -475,11 +487,11 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
         *reinterpret_cast<uint4 *>(xs + (sb & 1) * 128 * 16 + ((tid & 255) >> 1) * 16 + 8 * (tid & 1)) = v;
     };
 
-    floatx16 tot[RB][4], acc[RB][4];   // acc starts every super-block from the zero C operand of its first MFMAs
+    floatx16 tot[RB][CB], acc[RB][CB];   // acc starts every super-block from the zero C operand of its first MFMAs
 #pragma unroll
     for (int i = 0; i < RB; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < CB; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) tot[i][j][r] = 0.0f;
     const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -510,9 +522,9 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
         const uint4 hd[4] = {hdr.h0, hdr.h1, hdr.h2, hdr.h3};
         const uint2 wa[4] = {w.a0, w.a1, w.a2, w.a3}, wb[4] = {w.b0, w.b1, w.b2, w.b3};
         // scale constants of the tile's two sub-blocks per column block: (offset + q) * sc - offset * sc, and the same / 2048
-        h2 s_lo[4], o_lo[4], s_hi[4], o_hi[4];
+        h2 s_lo[CB], o_lo[CB], s_hi[CB], o_hi[CB];
 #pragma unroll
-        for (int cb = 0; cb < 4; cb++) {
+        for (int cb = 0; cb < CB; cb++) {
             u32 sc, m;
             q4k_scale_min(hd[cb], 2 * u, sc, m);
             const _Float16 f0 = (_Float16)(unsigned short)sc;
@@ -529,13 +541,15 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
             xn = fetch_x(ahead);
             if (u == 3) sums_next = fetch_sums((t >> 2) + 2);
         }
-        struct Frags { half8 h0, h1, l0, l1; };
+        struct Frags { half8 h[RB], l[RB]; };
         auto load_frags = [&](int ks) __attribute__((always_inline)) {
             const int ra = (wm * 32 * RB + bn) * LDK + ks * 16 + 8 * kg;
             Frags f;
-            f.h0 = *reinterpret_cast<const half8 *>(xhb + ra); f.l0 = *reinterpret_cast<const half8 *>(xlb + ra);
-            if constexpr (RB == 2) { f.h1 = *reinterpret_cast<const half8 *>(xhb + ra + 32 * LDK); f.l1 = *reinterpret_cast<const half8 *>(xlb + ra + 32 * LDK); }
-            else { f.h1 = f.h0; f.l1 = f.l0; }
+#pragma unroll
+            for (int i = 0; i < RB; i++) {
+                f.h[i] = *reinterpret_cast<const half8 *>(xhb + ra + 32 * i * LDK);
+                f.l[i] = *reinterpret_cast<const half8 *>(xlb + ra + 32 * i * LDK);
+            }
             return f;
         };
         // the super-block's fold, per column block, right behind that block's last MFMAs (the other blocks' MFMAs run meanwhile):
@@ -565,9 +579,8 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
         for (int ks = 0; ks < 4; ks++) {
             const Frags f = fnext;
             if (ks < 3) fnext = load_frags(ks + 1);
-            const half8 fh0 = f.h0, fh1 = f.h1, fl0 = f.l0, fl1 = f.l1;
 #pragma unroll
-            for (int cb = 0; cb < 4; cb++) {
+            for (int cb = 0; cb < CB; cb++) {
                 const uint2 q = (ks & 1) ? wb[cb] : wa[cb];   // k 0..15 and 32..47 of the tile: the chunk's first sixteen bytes; 16..31, 48..63: its second
                 const u32 x0 = q.x, x1 = q.y, x08 = x0 >> 8, x18 = x1 >> 8;
                 uint4 bq, bs;
@@ -587,14 +600,15 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
                     bs = make_uint4(as_u32(p0 * kTwoM11), as_u32(p1 * kTwoM11), as_u32(p2 * kTwoM11), as_u32(p3 * kTwoM11));
                 }
                 const half8 fb = __builtin_bit_cast(half8, bq), fbs = __builtin_bit_cast(half8, bs);
-                acc[0][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh0, fb, (u == 0 && ks == 0) ? zero16 : acc[0][cb], 0, 0, 0);
-                if constexpr (RB == 2) acc[1][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh1, fb, (u == 0 && ks == 0) ? zero16 : acc[1][cb], 0, 0, 0);
-                acc[0][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl0, fbs, acc[0][cb], 0, 0, 0);
-                if constexpr (RB == 2) acc[1][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl1, fbs, acc[1][cb], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < RB; i++)
+                    acc[i][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.h[i], fb, (u == 0 && ks == 0) ? zero16 : acc[i][cb], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < RB; i++) acc[i][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.l[i], fbs, acc[i][cb], 0, 0, 0);
                 if (u == 3 && ks == 3 && cb > 0) fold(cb - 1);
             }
         }
-        if (u == 3) fold(3);
+        if (u == 3) fold(CB - 1);
         // this slot's weights are used up: the tile two ahead goes into it
         {
             const int ahead = t + 2 < t_last ? t + 2 : t_last;
@@ -618,8 +632,8 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
 #pragma unroll
         for (int i = 0; i < RB; i++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int n = n0 + 128 * wn + 32 * j + bn;
+            for (int j = 0; j < CB; j++) {
+                const int n = n0 + 32 * CB * wn + 32 * j + bn;
                 const bool odd = lane & 1;
 #pragma unroll
                 for (int k = 0; k < 8; k++) {
@@ -648,8 +662,8 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
 #pragma unroll
     for (int i = 0; i < RB; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int n = n0 + 128 * wn + 32 * j + bn;
+        for (int j = 0; j < CB; j++) {
+            const int n = n0 + 32 * CB * wn + 32 * j + bn;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int m = m0 + (wm * RB + i) * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
@@ -847,12 +861,16 @@ hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream) {
     if (!(raised.load(std::memory_order_acquire) & bit)) {
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
         if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_regb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytesRegB);
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_regb_kernel<2, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytesRegB);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_regb_kernel<4, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytesRegB);
         if (e != hipSuccess) return e;
         raised.fetch_or(bit, std::memory_order_release);
     }
     dim3 grid((a.N + nt - 1) / nt, splits, (a.M + MT - 1) / MT);
-    if (regb) hipLaunchKernelGGL(gemm_q4k_split_regb_kernel, grid, dim3(kThreads), kLdsBytesRegB, stream, a);
+    static const int regb_shape = [] { const char *e = getenv("ESPRESSO_HIP_SPLIT_GEMM_SHAPE"); return e ? atoi(e) : 4; }();
+    if (regb && regb_shape == 4) hipLaunchKernelGGL((gemm_q4k_split_regb_kernel<4, 2>), grid, dim3(kThreads), kLdsBytesRegB, stream, a);
+    else if (regb) hipLaunchKernelGGL((gemm_q4k_split_regb_kernel<2, 4>), grid, dim3(kThreads), kLdsBytesRegB, stream, a);
     else hipLaunchKernelGGL(gemm_q4k_split_kernel<2>, grid, dim3(kThreads), kLdsBytes, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
