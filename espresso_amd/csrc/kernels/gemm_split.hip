@@ -397,9 +397,11 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_kernel(SplitGemmArgs 
 // Counters of this kernel: a wavefront's vector-ALU instructions and its MFMAs take turns (39 % + 44 % of its cycles; forcing an MFMA /
 // vector interleave in the instruction order changes nothing, a second wavefront per SIMD with half the tile is slower), so what counts
 // is the vector work per MFMA: with every wavefront on all 128 rows and 64 weight rows (RB x CB = 4 x 2) a B fragment serves eight
-// MFMAs instead of four: gate|up of a 512-row block 356 -> 324 us (the kernel above: 421 on the same boxes).
+// MFMAs instead of four: gate|up of a 512-row block 356 -> 324 us (the kernel above: 421 on the same boxes).  The activation tiles
+// rotate through four LDS buffers so that one barrier serves two tiles (318 -> 313 us, old and new alternating on one box).
 constexpr int NT2 = 256;
-constexpr size_t kLdsBytesRegB = 4 * kTileHalfs * 2 + 2 * 128 * 16 * 2;
+constexpr int kRegBBufs = 4;   // activation tiles in LDS: with four, one barrier serves two tiles
+constexpr size_t kLdsBytesRegB = 2 * kRegBBufs * kTileHalfs * 2 + 2 * 128 * 16 * 2;
 
 // RB x CB = 32-row blocks of activations x 32-row blocks of weights per wavefront (eight in all: 128 accumulator registers).
 template <int RB, int CB>
@@ -408,9 +410,9 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
     constexpr int THREADS = kThreads, XP = 1024 / THREADS;   // sixteen-byte pieces of a plane's tile per thread
     constexpr int NW = 8 / CB;                               // wavefronts along the weight rows
     extern __shared__ uint4 smem_raw[];
-    _Float16 *xh = reinterpret_cast<_Float16 *>(smem_raw);     // [2][128 * LDK]
-    _Float16 *xl = xh + 2 * kTileHalfs;                          // [2][128 * LDK]
-    _Float16 *xs = xl + 2 * kTileHalfs;                          // [2][128][16]   (hi of S_0..S_7, lo of S_0..S_7) of the row
+    _Float16 *xh = reinterpret_cast<_Float16 *>(smem_raw);     // [kRegBBufs][128 * LDK]
+    _Float16 *xl = xh + kRegBBufs * kTileHalfs;                  // [kRegBBufs][128 * LDK]
+    _Float16 *xs = xl + kRegBBufs * kTileHalfs;                        // [2][128][16]   (hi of S_0..S_7, lo of S_0..S_7) of the row
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / NW, wn = wave % NW;            // wm: which 32 RB activation rows of the tile, wn: which 32 CB weight rows
     const int n0 = blockIdx.x * NT2, m0 = blockIdx.z * MT;
@@ -500,7 +502,7 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
     asm volatile("" : "+s"(mask_lo), "+s"(mask_hi));
     asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
 
-    // prologue: tile t_begin staged, t_begin + 1 in registers, weights of both in registers
+    // prologue: tiles t_begin and t_begin + 1 staged, t_begin + 2 in registers, weights of the first two in registers
     const int t_second = t_begin + 1 < t_last ? t_begin + 1 : t_last;
     WRaw w0 = fetch_w(t_begin), w1 = fetch_w(t_second);
     Hdrs hdr = fetch_hdr(t_begin >> 2);
@@ -508,17 +510,19 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
         const XTile xfirst = fetch_x(t_begin);
         store_sums(fetch_sums(t_begin >> 2), t_begin >> 2);
         store_x(xfirst, 0);
+        const XTile xsecond = fetch_x(t_second);
+        store_x(xsecond, 1);
     }
-    XTile xn = fetch_x(t_second);
+    XTile xn = fetch_x(t_begin + 2 < t_last ? t_begin + 2 : t_last);
     uint4 sums_next = fetch_sums((t_begin >> 2) + 1);
     Hdrs hdr_next = fetch_hdr((t_begin >> 2) + 1);
     __syncthreads();
 
     const h2 kTwoM11 = {(_Float16)kUnscale, (_Float16)kUnscale};
     auto tile_step = [&](auto u_c, int t) __attribute__((always_inline)) {
-        constexpr int u = decltype(u_c)::value, buf = u & 1;
-        const _Float16 *xhb = xh + (size_t)buf * kTileHalfs, *xlb = xl + (size_t)buf * kTileHalfs;
-        WRaw &w = buf == 0 ? w0 : w1;
+        constexpr int u = decltype(u_c)::value;
+        const _Float16 *xhb = xh + (size_t)u * kTileHalfs, *xlb = xl + (size_t)u * kTileHalfs;
+        WRaw &w = (u & 1) == 0 ? w0 : w1;
         const uint4 hd[4] = {hdr.h0, hdr.h1, hdr.h2, hdr.h3};
         const uint2 wa[4] = {w.a0, w.a1, w.a2, w.a3}, wb[4] = {w.b0, w.b1, w.b2, w.b3};
         // scale constants of the tile's two sub-blocks per column block: (offset + q) * sc - offset * sc, and the same / 2048
@@ -533,11 +537,12 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
             const _Float16 f1 = (_Float16)(unsigned short)sc;
             s_hi[cb] = h2{f1, f1}; o_hi[cb] = s_hi[cb] * h2{(_Float16)-64.0f, (_Float16)-64.0f};
         }
-        // the next tile goes to the other LDS buffer (its activations were fetched during the previous tile), then its successor is fetched
-        store_x(xn, buf ^ 1);
+        // the tile two ahead goes to its LDS buffer (fetched during the previous tile), then its successor is fetched.  A tile's buffer
+        // was last read two tiles ago and is read again two tiles on, and a barrier closes every odd tile: one lies in between either way.
+        store_x(xn, (u + 2) & 3);
         if (u == 3) store_sums(sums_next, (t >> 2) + 1);
         {
-            const int ahead = t + 2 < t_last ? t + 2 : t_last;
+            const int ahead = t + 3 < t_last ? t + 3 : t_last;
             xn = fetch_x(ahead);
             if (u == 3) sums_next = fetch_sums((t >> 2) + 2);
         }
@@ -618,7 +623,7 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
             hdr = hdr_next;
             hdr_next = fetch_hdr((t >> 2) + 2);
         }
-        __syncthreads();
+        if (u & 1) __syncthreads();
     };
     for (int t0 = t_begin; t0 < t_end; t0 += 4) {
         tile_step(std::integral_constant<int, 0>{}, t0);
