@@ -140,6 +140,8 @@ def _declare_llama(L: C.CDLL) -> None:
     L.esp_llama_resident_weight_bytes.argtypes = [vp]
     L.esp_matmul_f32.restype = i32
     L.esp_matmul_f32.argtypes = [vp, vp, i32, vp, vp]
+    L.esp_matmul_f32_swiglu.restype = i32
+    L.esp_matmul_f32_swiglu.argtypes = [vp, vp, i32, vp]
     L.esp_llama_set_split_activations.restype = i32
     L.esp_llama_set_split_activations.argtypes = [vp, i32]
     L.esp_llama_set_matrix_prefill.restype = i32

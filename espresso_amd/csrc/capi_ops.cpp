@@ -6,6 +6,7 @@
 #include <cstring>
 
 #include "context.h"
+#include "host/model_support.h"
 #include "kernels/decode_ops.h"
 
 using namespace esp;
@@ -209,6 +210,57 @@ int esp_matmul_f32(const ESPMatrix *matrix, const float *x, int rows, float *y, 
     if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
     release();
     return e == hipSuccess ? ESP_OK : fail_hip(e, "matmul_f32");
+}
+
+int esp_matmul_f32_swiglu(const ESPMatrix *matrix, const float *x, int rows, float *act) {
+    if (!matrix || !x || !act) return fail(ESP_ERR_INVALID_ARGUMENT, "matmul_f32_swiglu: null pointer");
+    if (rows <= 0) return fail(ESP_ERR_INVALID_ARGUMENT, "matmul_f32_swiglu: rows %d", rows);
+    int rc = ensure_init();
+    if (rc != ESP_OK) return rc;
+    Context &c = context();
+    const DeviceMatrix &m = matrix->m;
+    if (!gemm_split_supported(m) || m.rows % 8 != 0) return fail(ESP_ERR_UNSUPPORTED, "matmul_f32_swiglu: Q4_K matrices with a multiple of 256 columns and of 8 rows");
+    const size_t nx = (size_t)rows * m.cols, units = (size_t)m.rows / 2, na = (size_t)rows * units;
+    float *d_x = nullptr;
+    GemmSplitSharedK pool;
+    SplitRowsView v, out;
+    auto release = [&] {
+        void *ptrs[] = {d_x, v.hi, v.lo, v.sums, out.hi, out.lo, out.sums};
+        for (void *p : ptrs) if (p) (void)hipFree(p);
+    };
+    if ((rc = device_alloc(&d_x, nx)) != ESP_OK || (rc = device_alloc(&v.hi, nx)) != ESP_OK || (rc = device_alloc(&v.lo, nx)) != ESP_OK ||
+        (rc = device_alloc(&v.sums, nx / 16)) != ESP_OK || (rc = device_alloc(&out.hi, na)) != ESP_OK || (rc = device_alloc(&out.lo, na)) != ESP_OK ||
+        (rc = device_alloc(&out.sums, na / 16 + 16)) != ESP_OK) {
+        release();
+        return rc;
+    }
+    std::vector<uint16_t> hi(na), lo(na);
+    hipError_t e = hipMemcpyAsync(d_x, x, nx * 4, hipMemcpyHostToDevice, c.stream);
+    if (e == hipSuccess) e = gemm_split_shared_k_pool(&pool);
+    if (e == hipSuccess) {
+        SplitRowsParams sp;
+        sp.x = d_x; sp.rows = rows; sp.cols = m.cols; sp.out = v;
+        e = launch_split_rows(sp, c.stream);
+    }
+    // twice: the second launch runs under the next launch number and finds the first one's flags in place
+    for (int pass = 0; pass < 2 && e == hipSuccess; pass++) {
+        GemmSplitParams g;
+        g.w = m; g.x = v; g.rows = rows; g.swiglu = out; g.shared_k = &pool;
+        if (pass == 1) e = hipMemsetAsync(out.hi, 0xff, na * 2, c.stream);
+        if (e == hipSuccess) e = launch_gemm_split(g, c.stream);
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(hi.data(), out.hi, na * 2, hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(lo.data(), out.lo, na * 2, hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+    release();
+    if (e != hipSuccess) return fail_hip(e, "matmul_f32_swiglu");
+    // the planes keep the units of every four in the order (0, 2, 1, 3)
+    for (int r = 0; r < rows; r++)
+        for (size_t u = 0; u < units; u++) {
+            const size_t slot = u & 3, o = (size_t)r * units + (u & ~(size_t)3) + (slot == 1 ? 2 : slot == 2 ? 1 : slot);
+            act[(size_t)r * units + u] = half_to_float(hi[o]) + half_to_float(lo[o]) * (1.0f / 2048.0f);
+        }
+    return ESP_OK;
 }
 
 int esp_gemv_device_noalloc(const ESPMatrix *matrix, const uint16_t *x_f16_device, int batch, float *y_device,

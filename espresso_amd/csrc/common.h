@@ -150,7 +150,18 @@ struct GemmSplitParams {
     size_t workspace_floats = 0;
     SplitRowsView swiglu;             // optional: silu(y[2i]) * y[2i + 1] as split rows [rows][w.rows / 2] instead of y
     int *deferred_splits = nullptr;   // optional: leave split-K partial sums [splits][rows][w.rows] in workspace, report the count
+    // optional, with `swiglu`: the device's hand-over pool (gemm_split_shared_k_pool).  Given it, a launch whose output tiles do not
+    // fill whole rounds of the chip runs one workgroup per compute unit with equal shares of K tiles; workgroups that share an output
+    // tile hand partial totals over through the pool.  One launch at a time per device.
+    const struct GemmSplitSharedK *shared_k = nullptr;
 };
+struct GemmSplitSharedK {
+    unsigned *flags = nullptr;
+    float *partial = nullptr;
+    size_t partial_floats = 0;
+};
+hipError_t gemm_split_shared_k_pool(GemmSplitSharedK *out);   // allocated on first use, kept until the process ends; not during a capture
+void gemm_split_set_shared_k(int mode);   // 0 off, 1 on (default), 2 on with the finisher never waiting (tests)
 bool gemm_split_supported(const DeviceMatrix &w);
 hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream);
 

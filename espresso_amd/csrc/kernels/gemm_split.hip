@@ -22,6 +22,7 @@
 #include "../common.h"
 #include "decode_ops.h"
 #include <atomic>
+#include <mutex>
 #include <cstdlib>
 #include <type_traits>
 #include <utility>
@@ -52,7 +53,15 @@ struct SplitGemmArgs {
     int tiles_per_split;            // a multiple of four
     uint16_t *sw_hi, *sw_lo;        // SiLU(gate) * up as a split pair [M][N / 2] instead of y (no split-K)
     const uint8_t *tiled;           // the matrix-core GEMV's tiled copy (gemm_q4k_split_regb_kernel reads its weights there)
+    // shared K ranges (gemm_q4k_split_regb_kernel<.., true>): workgroup i owns K tiles [i * sk_units, (i + 1) * sk_units) of the
+    // sequence (output tile 0: K tiles 0 .. K / 64 - 1, output tile 1: ...), output tile t = (t % sk_tiles_n, t / sk_tiles_n)
+    int sk_units, sk_tiles_n;
+    unsigned *sk_flags;             // [kStreamKFlags]: one word per workgroup + the launch counter, zero before the first launch
+    unsigned sk_spin_limit;
+    float *sk_partial;              // [workgroups][128 accumulators][256 threads]
 };
+constexpr int kStreamKFlags = 1024, kStreamKEpochSlot = kStreamKFlags - 1, kStreamKMaxWorkgroups = 256;
+constexpr unsigned kStreamKSpinLimit = 1u << 22;   // polls of the finisher (each at least a trip to memory) before it computes the rest itself
 
 __device__ __forceinline__ h2 as_h2(u32 v) { return __builtin_bit_cast(h2, v); }
 __device__ __forceinline__ u32 as_u32(h2 v) { return __builtin_bit_cast(u32, v); }
@@ -404,23 +413,57 @@ constexpr int kRegBBufs = 4;   // activation tiles in LDS: with four, one barrie
 constexpr size_t kLdsBytesRegB = 2 * kRegBBufs * kTileHalfs * 2 + 2 * 128 * 16 * 2;
 
 // RB x CB = 32-row blocks of activations x 32-row blocks of weights per wavefront (eight in all: 128 accumulator registers).
-template <int RB, int CB>
+//
+// SK (shared K ranges): the SiLU(gate) * up launch of a 512-row block is 448 output tiles on 256 compute units, a full round and one
+// that is three quarters full.  With SK the grid is one workgroup per compute unit and workgroup i takes K tiles [i u, (i + 1) u) of
+// the sequence "all K tiles of output tile 0, then of output tile 1, ..." (u = all K tiles / workgroups, at least one output tile's
+// worth, a multiple of four): the rest of the output tile its predecessor began, whole output tiles, and the beginning of one more.
+// A workgroup that ends inside an output tile finishes it: its successor, whose first piece that tile's rest is, leaves its 128
+// totals per lane in `sk_partial` and then writes the launch's number into its flag word; the finisher adds them and runs the
+// epilogue.  The successor's piece is the first thing it does and waits for nothing, so whatever the order in which workgroups
+// become resident the finisher's wait ends; it is bounded all the same (sk_spin_limit polls), and a finisher whose wait runs out
+// computes the rest of the tile itself.  The launch number lives in device memory (the kernel that follows every such launch
+// increments it), so a captured launch replays correctly and a flag of an earlier launch is never taken for this one's.
+// `sk_partial` and `sk_flags` are uncached device memory: with ordinary memory the hand-over needs a release that writes the die's
+// L2 back (10 us per workgroup, measured) and an acquire that invalidates the finisher's.
+// Measured on gate|up of a 512-row block, workgroup by workgroup (wall-clock stamps): 2.2 us per K tile, 4.7 us per epilogue, 3.7 us to
+// hand the totals over, 6.3 us to take them; the launch 295 against 310 us for the plain grid on the same box.
+template <int RB, int CB, bool SK = false>
 __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemmArgs a) {
     static_assert(RB * CB == 8 && (RB == 2 || RB == 4), "a wavefront owns eight 32 x 32 tiles");
+    __shared__ int sk_flag_seen;
     constexpr int THREADS = kThreads, XP = 1024 / THREADS;   // sixteen-byte pieces of a plane's tile per thread
     constexpr int NW = 8 / CB;                               // wavefronts along the weight rows
     extern __shared__ uint4 smem_raw[];
     _Float16 *xh = reinterpret_cast<_Float16 *>(smem_raw);     // [kRegBBufs][128 * LDK]
     _Float16 *xl = xh + kRegBBufs * kTileHalfs;                  // [kRegBBufs][128 * LDK]
     _Float16 *xs = xl + kRegBBufs * kTileHalfs;                        // [2][128][16]   (hi of S_0..S_7, lo of S_0..S_7) of the row
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / NW, wn = wave % NW;            // wm: which 32 RB activation rows of the tile, wn: which 32 CB weight rows
-    const int n0 = blockIdx.x * NT2, m0 = blockIdx.z * MT;
     const int tiles = a.K / KT, sbs = a.K / 256;
-    const int t_begin = blockIdx.y * a.tiles_per_split;
-    const int t_end = t_begin + a.tiles_per_split < tiles ? t_begin + a.tiles_per_split : tiles;
-    const int t_last = t_end - 1;
+    floatx16 tot[RB][CB], acc[RB][CB];   // acc starts every super-block from the zero C operand of its first MFMAs
+    int sk_unit = SK ? (int)blockIdx.x * a.sk_units : 0;
+    const int sk_unit_end = sk_unit + a.sk_units;
+    const unsigned sk_launch = SK ? a.sk_flags[kStreamKEpochSlot] + 1u : 0u;
+    int sk_resume_from = 0;   // > 0: the previous pass ended at this K tile of the same output tile and the totals stay
+  for (;;) {   // one pass per piece of an output tile with SK, a single pass otherwise (the body keeps a function body's indentation)
+    // The thread's coordinates are formed anew for every output tile piece: taken from outside the loop, every LDS and row offset
+    // derived from them would be kept in registers across the pieces, and the kernel has none to spare.
+    int tid = threadIdx.x;
+    if constexpr (SK) asm volatile("" : "+v"(tid));
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / NW, wn = wave % NW;            // wm: which 32 RB activation rows of the tile, wn: which 32 CB weight rows
     const int bn = lane & 31, kg = lane >> 5;
+    int n0, m0, t_begin, t_end;
+    if constexpr (SK) {
+        const int out_tile = sk_unit / tiles, first = sk_resume_from ? sk_resume_from : sk_unit % tiles;
+        const int room = sk_resume_from ? tiles - first : sk_unit_end - sk_unit;
+        n0 = (out_tile % a.sk_tiles_n) * NT2; m0 = (out_tile / a.sk_tiles_n) * MT;
+        t_begin = first; t_end = first + room < tiles ? first + room : tiles;
+    } else {
+        n0 = blockIdx.x * NT2; m0 = blockIdx.z * MT;
+        t_begin = blockIdx.y * a.tiles_per_split;
+        t_end = t_begin + a.tiles_per_split < tiles ? t_begin + a.tiles_per_split : tiles;
+    }
+    const int t_last = t_end - 1;
 
     // weights: column block cb of this wavefront = weight rows n0 + 32 CB wn + 32 cb + (0..31); this lane's row of it, clamped (never stored)
     const uint8_t *wrow[4];
@@ -489,13 +532,14 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
         *reinterpret_cast<uint4 *>(xs + (sb & 1) * 128 * 16 + ((tid & 255) >> 1) * 16 + 8 * (tid & 1)) = v;
     };
 
-    floatx16 tot[RB][CB], acc[RB][CB];   // acc starts every super-block from the zero C operand of its first MFMAs
+    if (!SK || !sk_resume_from) {
 #pragma unroll
-    for (int i = 0; i < RB; i++)
+        for (int i = 0; i < RB; i++)
 #pragma unroll
-        for (int j = 0; j < CB; j++)
+            for (int j = 0; j < CB; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) tot[i][j][r] = 0.0f;
+                for (int r = 0; r < 16; r++) tot[i][j][r] = 0.0f;
+    }
     const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     // constants of the nibble trick, hidden from the optimiser so that (w & mask) | magic stays one v_and_or_b32
     u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
@@ -632,34 +676,114 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
         tile_step(std::integral_constant<int, 3>{}, t0 + 3);
     }
 
+    if constexpr (SK) {
+        const bool resumed = sk_resume_from != 0;
+        if (!resumed) sk_unit += t_end - t_begin;
+        sk_resume_from = 0;
+        if (!resumed && t_begin > 0) {
+            // the rest of an output tile that the previous workgroup began: hand the totals over and go on
+            // (uncached memory: once the stores are acknowledged and the wavefronts have met, the flag may follow)
+            float4 *slot = reinterpret_cast<float4 *>(a.sk_partial + (size_t)blockIdx.x * 128 * THREADS) + tid;
+            asm volatile("" : "+v"(slot));   // formed here, not ahead of the loop: 32 addresses kept in registers would spill
+#pragma unroll
+            for (int i = 0; i < RB; i++)
+#pragma unroll
+                for (int j = 0; j < CB; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        slot[(size_t)((i * CB + j) * 4 + q) * THREADS] = make_float4(tot[i][j][4 * q], tot[i][j][4 * q + 1], tot[i][j][4 * q + 2], tot[i][j][4 * q + 3]);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // every store of this wavefront acknowledged
+            __syncthreads();
+            if (tid == 0) __hip_atomic_store(a.sk_flags + blockIdx.x, sk_launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (sk_unit >= sk_unit_end) return;
+            continue;
+        }
+        if (t_end < tiles) {
+            // this workgroup began the output tile: the next one has (or will have) the rest
+            if (tid == 0) {
+                int seen = 0;
+                for (unsigned polls = 0; polls < a.sk_spin_limit; polls++) {
+                    if (__hip_atomic_load(a.sk_flags + blockIdx.x + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == sk_launch) { seen = 1; break; }
+                    __builtin_amdgcn_s_sleep(8);
+                }
+                sk_flag_seen = seen;
+            }
+            __syncthreads();
+            const bool seen = sk_flag_seen != 0;
+            __syncthreads();
+            if (!seen) { sk_resume_from = t_end; continue; }
+            // (issued behind the barrier that follows thread 0's sight of the flag)
+            const float4 *slot = reinterpret_cast<const float4 *>(a.sk_partial + (size_t)(blockIdx.x + 1) * 128 * THREADS) + tid;
+            asm volatile("" : "+v"(slot));
+            // all loads in flight at once, into the accumulators (free between two super-blocks), then one pass of additions
+#pragma unroll
+            for (int i = 0; i < RB; i++)
+#pragma unroll
+                for (int j = 0; j < CB; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const float4 v = slot[(size_t)((i * CB + j) * 4 + q) * THREADS];
+                        acc[i][j][4 * q] = v.x; acc[i][j][4 * q + 1] = v.y; acc[i][j][4 * q + 2] = v.z; acc[i][j][4 * q + 3] = v.w;
+                    }
+#pragma unroll
+            for (int i = 0; i < RB; i++)
+#pragma unroll
+                for (int j = 0; j < CB; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) tot[i][j][r] += acc[i][j][r];
+        }
+    }
     // accumulator r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of the 32 x 32 tile
     if (a.sw_hi) {
+        // SiLU(gate) * up of the workgroup's 128 x 128 units as the two fp16 planes, through LDS (free now) so that the planes leave
+        // in whole 16-byte pieces of a row: [plane][128 rows][kActLd].  SiLU as g / (1 + exp(-g)): the same function as the
+        // 0.5 g (1 + tanh(0.5 g)) of the single-row kernels, a fifth of the instructions (this epilogue measured 10 us per
+        // output tile with tanhf and two-byte stores, a fifteenth of the tile's time).
+        constexpr int kActLd = 144;   // halfs per staged row: consecutive rows eight LDS banks apart
+        uint16_t *act_hi = reinterpret_cast<uint16_t *>(smem_raw), *act_lo = act_hi + 128 * kActLd;
+        const bool odd = lane & 1;
 #pragma unroll
         for (int i = 0; i < RB; i++)
 #pragma unroll
             for (int j = 0; j < CB; j++) {
-                const int n = n0 + 32 * CB * wn + 32 * j + bn;
-                const bool odd = lane & 1;
+                const int unit = (32 * CB * wn + 32 * j + bn) >> 1, slot = unit & 3;   // the planes' order inside fours: (0, 2, 1, 3)
+                const int col = (unit & ~3) + (slot == 1 ? 2 : slot == 2 ? 1 : slot);
+                const int row0 = (wm * RB + i) * 32 + 4 * kg + (odd ? 1 : 0);
 #pragma unroll
                 for (int k = 0; k < 8; k++) {
                     const float a0 = tot[i][j][2 * k], a1 = tot[i][j][2 * k + 1];
                     const float p0 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a0), 0xB1, 0xF, 0xF, false));
                     const float p1 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, a1), 0xB1, 0xF, 0xF, false));
                     const float g = odd ? p1 : a0, up = odd ? a1 : p0;
-                    const int r = 2 * k + (odd ? 1 : 0);
-                    const int m = m0 + (wm * RB + i) * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
-                    if (m < a.M && (n | 1) < a.N) {
-                        const float hg = __fmul_rn(0.5f, g);
-                        const float silu = __fmul_rn(hg, __fadd_rn(1.0f, tanhf(hg)));
-                        const float act = __fmul_rn(silu, up);
-                        const _Float16 hi = (_Float16)act;
-                        const int unit = n / 2, slot = unit & 3;   // the planes' order inside fours: (0, 2, 1, 3)
-                        const size_t o = (size_t)m * (a.N / 2) + (unit & ~3) + (slot == 1 ? 2 : slot == 2 ? 1 : slot);
-                        a.sw_hi[o] = __builtin_bit_cast(uint16_t, hi);
-                        a.sw_lo[o] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(__fsub_rn(act, (float)hi), kScale));
-                    }
+                    const float silu = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+                    const float act = __fmul_rn(silu, up);
+                    const _Float16 hi = (_Float16)act;
+                    const int o = (row0 + 8 * (k >> 1) + 2 * (k & 1)) * kActLd + col;   // row 8 (r / 4) + r % 4 of the block, r = 2 k (+ 1)
+                    act_hi[o] = __builtin_bit_cast(uint16_t, hi);
+                    act_lo[o] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(__fsub_rn(act, (float)hi), kScale));
                 }
             }
+        __syncthreads();
+        const int units_n = a.N / 2, unit0 = n0 / 2;
+        const bool whole_pieces = units_n % 8 == 0;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const int piece = q * THREADS + tid, row = piece >> 4, c8 = (piece & 15) * 8;
+            const int m = m0 + row;
+            if (m >= a.M || unit0 + c8 >= units_n) continue;
+            const size_t o = (size_t)m * units_n + unit0 + c8;
+            if (whole_pieces) {   // units_n and unit0 + c8 are multiples of eight: the piece is whole and 16-byte aligned
+                *reinterpret_cast<uint4 *>(a.sw_hi + o) = *reinterpret_cast<const uint4 *>(act_hi + row * kActLd + c8);
+                *reinterpret_cast<uint4 *>(a.sw_lo + o) = *reinterpret_cast<const uint4 *>(act_lo + row * kActLd + c8);
+            } else {
+                for (int e = 0; e < 8 && unit0 + c8 + e < units_n; e++) {
+                    a.sw_hi[o + e] = act_hi[row * kActLd + c8 + e];
+                    a.sw_lo[o + e] = act_lo[row * kActLd + c8 + e];
+                }
+            }
+        }
+        __syncthreads();   // the next output tile's prologue writes the same LDS
+        if (SK && sk_unit < sk_unit_end) continue;
         return;
     }
     const bool split = gridDim.y > 1;
@@ -678,6 +802,9 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
                 }
             }
         }
+    if (SK && sk_unit < sk_unit_end) continue;
+    return;
+  }
 }
 
 // y = (residual +) sum over splits of partial, in split order
@@ -811,8 +938,9 @@ __global__ __launch_bounds__(256) void split_rows_kernel(SplitRowsArgs a) {
 }
 
 // sums of rows that exist as hi / lo planes already (the SiLU(gate) * up epilogue writes those)
-__global__ __launch_bounds__(256) void split_sums_kernel(const uint16_t *hi, const uint16_t *lo, int cols, uint16_t *sums) {
+__global__ __launch_bounds__(256) void split_sums_kernel(const uint16_t *hi, const uint16_t *lo, int cols, uint16_t *sums, unsigned *launch_counter) {
     const int m = blockIdx.x;
+    if (launch_counter && m == 0 && threadIdx.x == 0) *launch_counter += 1u;   // the GEMM before this kernel shared K ranges under this number
     const size_t row = (size_t)m * cols;
     for (int g = threadIdx.x; g < cols / 8; g += 256) {
         const uint4 h = reinterpret_cast<const uint4 *>(hi + row)[g], l = reinterpret_cast<const uint4 *>(lo + row)[g];
@@ -827,6 +955,42 @@ __global__ __launch_bounds__(256) void split_sums_kernel(const uint16_t *hi, con
 }
 
 }  // namespace
+
+// 1 (default): shared K ranges where they apply; 0: never; 2: as 1, but a finishing workgroup does not wait for its successor's
+// totals and always computes the rest of its output tile itself (the path a wait that runs out takes; for tests).
+// Initial value from ESPRESSO_HIP_SPLIT_GEMM_SHARED_K.
+static int g_shared_k_mode = -1;
+static int shared_k_mode() {
+    if (g_shared_k_mode < 0) { const char *e = getenv("ESPRESSO_HIP_SPLIT_GEMM_SHARED_K"); g_shared_k_mode = e ? atoi(e) : 1; }
+    return g_shared_k_mode;
+}
+// One pool per device for the process's lifetime (uncached device memory is never given back once a kernel has read it).
+hipError_t gemm_split_shared_k_pool(GemmSplitSharedK *out) {
+    static std::atomic<void *> pools[64];
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return e;
+    const size_t partial_floats = (size_t)kStreamKMaxWorkgroups * 128 * kThreads, bytes = partial_floats * 4 + kStreamKFlags * 4;
+    void *p = pools[device & 63].load(std::memory_order_acquire);
+    if (!p) {
+        static std::mutex m;
+        std::lock_guard<std::mutex> lock(m);
+        p = pools[device & 63].load(std::memory_order_acquire);
+        if (!p) {
+            e = hipExtMallocWithFlags(&p, bytes, hipDeviceMallocUncached);
+            if (e != hipSuccess) return e;
+            e = hipMemset(p, 0, bytes);
+            if (e == hipSuccess) e = hipDeviceSynchronize();
+            if (e != hipSuccess) return e;   // (the allocation stays: see above)
+            pools[device & 63].store(p, std::memory_order_release);
+        }
+    }
+    out->partial = static_cast<float *>(p);
+    out->partial_floats = partial_floats;
+    out->flags = reinterpret_cast<unsigned *>(static_cast<float *>(p) + partial_floats);
+    return hipSuccess;
+}
+void gemm_split_set_shared_k(int mode) { g_shared_k_mode = mode < 0 ? 1 : mode; }
 
 bool gemm_split_supported(const DeviceMatrix &w) { return w.format == FMT_Q4_K && w.qs && w.cols % 256 == 0 && w.qs_row_bytes % 16 == 0; }
 
@@ -863,24 +1027,49 @@ hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream) {
     hipError_t e = hipGetDevice(&device);
     if (e != hipSuccess) return e;
     const uint64_t bit = 1ull << (device & 63);
+    static const int regb_shape = [] { const char *e = getenv("ESPRESSO_HIP_SPLIT_GEMM_SHAPE"); return e ? atoi(e) : 4; }();
+    // Shared K ranges for the SiLU(gate) * up launch when its output tiles do not fill whole rounds of the chip: one workgroup
+    // per compute unit, each with the same number of K tiles.
+    const int shared_k = shared_k_mode();
+    int shared_k_workgroups = 0;
+    if (swiglu && regb && regb_shape == 4 && shared_k != 0 && p.shared_k && p.shared_k->flags && p.shared_k->partial) {
+        static std::atomic<int> cus[64];
+        int n = cus[device & 63].load(std::memory_order_relaxed);
+        if (n == 0) {
+            e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device);
+            if (e != hipSuccess) return e;
+            cus[device & 63].store(n, std::memory_order_relaxed);
+        }
+        const long long units = (long long)blocks * tiles;
+        if (n > 0 && n <= kStreamKMaxWorkgroups && blocks > n && blocks % n != 0 && units % n == 0 && (units / n) % 4 == 0 && units / n >= tiles &&
+            (size_t)n * 128 * kThreads <= p.shared_k->partial_floats) {
+            shared_k_workgroups = n;
+            a.sk_units = (int)(units / n); a.sk_tiles_n = (a.N + nt - 1) / nt;
+            a.sk_flags = p.shared_k->flags; a.sk_partial = p.shared_k->partial;
+            a.sk_spin_limit = shared_k == 2 ? 0u : kStreamKSpinLimit;
+        }
+    }
     if (!(raised.load(std::memory_order_acquire) & bit)) {
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_regb_kernel<2, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytesRegB);
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_regb_kernel<4, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytesRegB);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_split_regb_kernel<4, 2, true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytesRegB);
         if (e != hipSuccess) return e;
         raised.fetch_or(bit, std::memory_order_release);
     }
     dim3 grid((a.N + nt - 1) / nt, splits, (a.M + MT - 1) / MT);
-    static const int regb_shape = [] { const char *e = getenv("ESPRESSO_HIP_SPLIT_GEMM_SHAPE"); return e ? atoi(e) : 4; }();
-    if (regb && regb_shape == 4) hipLaunchKernelGGL((gemm_q4k_split_regb_kernel<4, 2>), grid, dim3(kThreads), kLdsBytesRegB, stream, a);
+    if (shared_k_workgroups) hipLaunchKernelGGL((gemm_q4k_split_regb_kernel<4, 2, true>), dim3(shared_k_workgroups), dim3(kThreads), kLdsBytesRegB, stream, a);
+    else if (regb && regb_shape == 4) hipLaunchKernelGGL((gemm_q4k_split_regb_kernel<4, 2>), grid, dim3(kThreads), kLdsBytesRegB, stream, a);
     else if (regb) hipLaunchKernelGGL((gemm_q4k_split_regb_kernel<2, 4>), grid, dim3(kThreads), kLdsBytesRegB, stream, a);
     else hipLaunchKernelGGL(gemm_q4k_split_kernel<2>, grid, dim3(kThreads), kLdsBytes, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (swiglu) {
-        hipLaunchKernelGGL(split_sums_kernel, dim3(a.M), dim3(256), 0, stream, p.swiglu.hi, p.swiglu.lo, a.N / 2, p.swiglu.sums);
+        hipLaunchKernelGGL(split_sums_kernel, dim3(a.M), dim3(256), 0, stream, p.swiglu.hi, p.swiglu.lo, a.N / 2, p.swiglu.sums,
+                           shared_k_workgroups ? a.sk_flags + kStreamKEpochSlot : nullptr);
         return hipGetLastError();
     }
     if (splits > 1) {

@@ -2551,6 +2551,7 @@ bool gemv_set_tuning(const char *key, int value) {
     if (k == "q4k_mfma_rows8_max") { g_q4k_mfma_rows8_max = value; return true; }
     if (k == "q4k_long_row_waves") { g_q4k_long_row_waves = value; return true; }
     if (k == "q4k_wide") { g_q4k_wide_mode = value; return true; }
+    if (k == "split_gemm_shared_k") { gemm_split_set_shared_k(value); return true; }
     return false;
 }
 

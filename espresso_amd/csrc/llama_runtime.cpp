@@ -427,6 +427,7 @@ int LlamaRuntime::finalize() {
         if ((rc = device_alloc(&attn_scratch_, R * per_row)) != ESP_OK) return rc;
     }
     if ((rc = device_alloc(&gemm_workspace_, kGemmWorkspaceFloats)) != ESP_OK) return rc;
+    ESP_HIP_TRY(gemm_split_shared_k_pool(&gemm_shared_k_));
     {
         const char *pa = getenv("ESPRESSO_HIP_PROMPT_ATTENTION");   // "0": prompt blocks keep the single-query attention kernel
         prompt_attention_ = attention_prompt_supported(c_.n_head, c_.n_kv_head, c_.head_dim) && !(pa && pa[0] == '0');
@@ -720,8 +721,9 @@ int LlamaRuntime::enqueue_layers_split(int rows) {
         ESP_HIP_TRY(launch_gemm_split(g, s));
         ESP_HIP_TRY(norm(L.rms_ffn, splits));
         g.w = L.w13; g.x = xn; g.y = nullptr; g.residual = nullptr; g.swiglu = act; g.deferred_splits = nullptr;
+        g.shared_k = &gemm_shared_k_;
         ESP_HIP_TRY(launch_gemm_split(g, s));
-        g.swiglu = SplitRowsView{};
+        g.swiglu = SplitRowsView{}; g.shared_k = nullptr;
         const bool last = li + 1 == layers_.size();
         g.w = L.w2; g.x = act; g.y = hidden_; g.residual = hidden_; splits = 1; g.deferred_splits = last ? nullptr : &splits;
         ESP_HIP_TRY(launch_gemm_split(g, s));

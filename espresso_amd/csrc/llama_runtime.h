@@ -191,6 +191,7 @@ class LlamaRuntime {
     bool split_activations_ = true;
     bool prompt_attention_ = false;   // prompt blocks run attention on the matrix cores
     float *gemm_workspace_ = nullptr;
+    GemmSplitSharedK gemm_shared_k_;   // the device's pool for launch_gemm_split's hand-over between workgroups (not owned)
 
     struct TimedLaunch { int kernel_class; hipEvent_t start, stop; };
     bool timing_enabled_ = false;

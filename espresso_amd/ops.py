@@ -104,6 +104,13 @@ class Matrix:
         _lib.check(_lib.load_library().esp_matmul_f32(self._h, _ptr(x), rows, _ptr(y), _ptr(res) if res is not None else None))
         return y
 
+    def matmul_f32_swiglu(self, x: np.ndarray) -> np.ndarray:
+        """SiLU(gate) * up of the exact Q4_K product for a matrix of interleaved gate / up rows (esp_matmul_f32_swiglu; test aid)."""
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.cols)
+        act = np.empty((x.shape[0], self.rows // 2), dtype=np.float32)
+        _lib.check(_lib.load_library().esp_matmul_f32_swiglu(self._h, _ptr(x), x.shape[0], _ptr(act)))
+        return act
+
     def time_gemv(self, batch: int = 1, warmup: int = 10, iters: int = 50, rotate: int = 1) -> dict:
         mean, best = C.c_double(0), C.c_double(0)
         _lib.check(_lib.load_library().esp_gemv_time(self._h, batch, warmup, iters, rotate, C.byref(mean), C.byref(best)))

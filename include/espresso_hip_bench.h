@@ -48,6 +48,12 @@ int esp_set_tuning(const char *key, int value);
  * bytes (esp_matrix_resident_bytes - esp_matrix_bytes; 0 when the matrix keeps none) or a negative ESP_ERR_* code.  tests/ rebuild the tiles
  * from the GGUF blocks with numpy and compare byte for byte. */
 long long esp_matrix_read_tiled(const ESPMatrix *matrix, void *out, size_t capacity);
+/* Test aid: the exact Q4_K product of esp_matmul_f32 with the epilogue the feed-forward block uses.  The matrix holds gate and up rows
+ * interleaved (row 2i = gate_i, 2i + 1 = up_i; `matrix rows` a multiple of 8); act[r][i] = SiLU(x[r] . gate_i) * (x[r] . up_i) as the pair of
+ * fp16 planes the kernel writes, added back together (hi + lo / 2048), fp32 [rows][matrix rows / 2]; host pointers.  The launch is made
+ * twice on the same flag words, so the second one runs under the next launch number; tuning key split_gemm_shared_k selects how
+ * workgroups share an output tile's K range (0 never, 1 where it applies, 2 as 1 with the finishing workgroup never waiting). */
+int esp_matmul_f32_swiglu(const ESPMatrix *matrix, const float *x, int rows, float *act);
 int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s);
 /* The ceiling for ONE GEMV launch: a kernel with a persistent Q4_K GEMV's grid (`workgroups` of `wavefronts` = 4 or 8) and its
  * loads (a wavefront takes items of `pair_bytes`, a 2304-byte weight tile of the matrix-core kernel or a pair of rows of the

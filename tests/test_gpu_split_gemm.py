@@ -69,6 +69,46 @@ def test_matmul_f32_reads_single_weights_and_small_activations_back(ops):
     mat.close()
 
 
+# (weight rows = 2 x feed-forward units, columns, activation rows, does the launch share K ranges between workgroups on a chip of 256
+# compute units): the 8B gate|up at a full 512-row block (448 output tiles: 112 K tiles per workgroup, 1.75 output tiles) and at 384
+# rows (84 K tiles), a 16-K-tile matrix (28 per workgroup), 320 output tiles of 32 K tiles (40 per workgroup), and shapes the
+# plain grid keeps (fewer output tiles than compute units; a whole number of rounds; ragged rows)
+SWIGLU_SHAPES = [(28672, 4096, 512, True), (28672, 4096, 384, True), (28672, 1024, 512, True), (10240, 2048, 1024, True),
+                 (28672, 4096, 256, False), (16384, 1024, 512, False), (1000, 512, 130, False)]
+
+
+@pytest.mark.parametrize("rows,cols,m,shared", SWIGLU_SHAPES)
+def test_swiglu_epilogue_with_and_without_shared_k_ranges(ops, rows, cols, m, shared):
+    """SiLU(gate) * up in the exact GEMM's epilogue against float64, with the workgroups sharing output tiles' K ranges (mode 1), on
+    the plain grid (mode 0), and with every finishing workgroup computing the rest of its tile itself instead of taking its
+    successor's totals (mode 2: the path a wait that runs out takes).  Mode 2 adds in the plain grid's order: bit-identical to mode 0."""
+    mat, deq = q4k(ops, rows, cols, rows + cols + m)
+    x = np.random.default_rng(m + 1).normal(0, 1, (m, cols)).astype(np.float32)
+    y = x.astype(np.float64) @ deq.astype(np.float64).T
+    gate, up = y[:, 0::2], y[:, 1::2]
+    want = gate / (1.0 + np.exp(-gate)) * up
+    scale, ystd = float(want.std()), float(y.std())
+    got = {}
+    try:
+        for mode in (0, 1, 2, 1):
+            ops.set_tuning("split_gemm_shared_k", mode)
+            act = mat.matmul_f32_swiglu(x)
+            err = np.abs(act - want)
+            print(f"{rows}x{cols}, {m} rows, mode {mode}: max {err.max():.2e} rms {np.sqrt((err ** 2).mean()):.2e} (scale {scale:.3f})", flush=True)
+            # gate and up carry the product's few 1e-6 (relative to its spread); d(SiLU(g) u) = SiLU'(g) u dg + SiLU(g) du
+            assert (err <= 5e-6 * ystd * (np.abs(up) + np.abs(gate) + 1.0)).all() and np.sqrt((err ** 2).mean()) <= 1.5e-6 * scale, (mode, err.max(), scale)
+            if mode in got:
+                assert np.array_equal(got[mode].view(np.uint32), act.view(np.uint32)), mode    # deterministic across launches
+            got[mode] = act
+    finally:
+        ops.set_tuning("split_gemm_shared_k", 1)
+    assert np.array_equal(got[0].view(np.uint32), got[2].view(np.uint32))
+    same = np.array_equal(got[0].view(np.uint32), got[1].view(np.uint32))
+    if ops.device_info()["compute_units"] == 256:
+        assert same != shared, "shared K ranges add an output tile's two parts in another order; the plain grid does not"
+    mat.close()
+
+
 def test_matmul_f32_refuses_other_formats(ops):
     w = np.random.default_rng(1).normal(0, 0.02, (64, 256)).astype(np.float32)
     mat = ops.Matrix(orc.FMT_Q8_0, orc.quantize(orc.FMT_Q8_0, w), 64, 256)
