@@ -161,7 +161,8 @@ struct GemmSplitSharedK {
     size_t partial_floats = 0;
 };
 hipError_t gemm_split_shared_k_pool(GemmSplitSharedK *out);   // allocated on first use, kept until the process ends; not during a capture
-void gemm_split_set_shared_k(int mode);   // 0 off, 1 on (default), 2 on with the finisher never waiting (tests)
+void gemm_split_set_shared_k(int mode);
+void attention_prompt_set_key_sets(int sets);   // prompt attention: 0 = sets of wavefronts by block size (default), 1 or 2 = always that many   // 0 off, 1 on (default), 2 on with the finisher never waiting (tests)
 bool gemm_split_supported(const DeviceMatrix &w);
 hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream);
 

@@ -475,8 +475,8 @@ __global__ __launch_bounds__(HD) void attention_merge_kernel(AttentionArgs a, in
 // sequence at consecutive positions (pos[m0 + i] = pos[m0] + i), which is what a prompt block is.  Replaces the per-row
 // loop of the reference's attention (:6774-6823) over a block: the single-query kernels above read a row's whole prefix
 // once per row, this one reads a key tile once per 32 rows.
-// grid (KV heads, tiles of 32 rows); wavefront g of a workgroup serves query head kvh * G + g, so the G heads that share
-// a KV head share the value tiles.  Per tile of 32 keys:
+// grid (KV heads, tiles of 32 rows, sets of G query heads); wavefront g of a workgroup serves query head kvh * group + G z + g,
+// so G heads that share a KV head share the value tiles.  Per tile of 32 keys:
 //   * S^T = K Q^T: keys are the A rows (a lane loads eight consecutive dims of its key straight from the cache, two
 //     tiles ahead), queries the B columns (fragments kept in registers); a lane's 16 accumulators are
 //     16 keys of ONE query, so the row maximum and sum of the online softmax are in-lane plus one exchange with lane ^ 32;
@@ -490,15 +490,21 @@ typedef _Float16 attn_half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 attn_half4 __attribute__((ext_vector_type(4)));
 typedef float attn_floatx16 __attribute__((ext_vector_type(16)));
 
-template <int HD, int G, bool KV_F16, bool SPLIT>
-__global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs a, int rows) {
-    constexpr int THREADS = G * 64, QT = 32, KS = HD / 16, MTILES = HD / 32, LDV = 32 + 8;   // LDV: fp16 per row of V^T
+// KP = 2: the workgroup has two sets of G wavefronts; set p takes the key tiles p, p + 2, ... with value tiles of its own, and the two
+// (maximum, sum, context) states of a head are merged through LDS at the end.  A workgroup's time is the length of its chain of key
+// tiles (a tile of arithmetic is shorter than the trip to memory behind it), and the last row tile of a 512-row block has sixteen.
+template <int HD, int G, bool KV_F16, bool SPLIT, int KP>
+__global__ __launch_bounds__(G * KP * 64) void attention_prompt_kernel(AttentionArgs a, int rows) {
+    constexpr int THREADS = G * 64, QT = 32, KS = HD / 16, MTILES = HD / 32, LDV = 32 + 8;   // THREADS: of one set; LDV: fp16 per row of V^T
     constexpr int VP = 32 * (HD / 8) / THREADS;                                            // 8-dim pieces of V per thread
-    static_assert(VP >= 1 && 32 * (HD / 8) % THREADS == 0, "value tile divides over the workgroup");
-    __shared__ _Float16 vt[2][HD * LDV];
+    static_assert(VP >= 1 && 32 * (HD / 8) % THREADS == 0, "value tile divides over a set of wavefronts");
+    static_assert(KP == 1 || KP == 2, "one or two sets");
+    __shared__ _Float16 vt_all[KP][2][HD * LDV];
     const int kvh = blockIdx.x, m0 = blockIdx.y * QT;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
-    const int head = kvh * G + wave;
+    const int phase = KP == 1 ? 0 : (int)threadIdx.x / THREADS;
+    const int tid = (int)threadIdx.x - phase * THREADS, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+    _Float16 (*vt)[HD * LDV] = vt_all[phase];
+    const int head = kvh * (a.n_head / a.n_kv_head) + (int)blockIdx.z * G + wave;   // grid z: sets of G query heads of the KV head
     const int pos0 = a.pos[m0];
     const int last_row = rows - 1 - m0 < QT - 1 ? rows - 1 - m0 : QT - 1;
     const int t_max = pos0 + last_row;             // last key any row of the tile sees
@@ -574,17 +580,19 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
     const int qpos = pos0 + col;
 
     // Keys and values are fetched two tiles ahead: one tile of arithmetic is shorter than a trip to memory.
+    constexpr int STEP = 32 * KP;   // keys between a set's tiles
     attn_half8 kf[KS], k1[KS], k2[KS], v1[VP], v2[VP];
-    load_k(0, kf);
-    load_v(0, v1);
+    load_k(32 * phase, kf);
+    load_v(32 * phase, v1);
     store_v(0, v1);
-    load_k(32, k1);      // tiles beyond t_max are clamped to it, in bounds and never used
-    load_v(32, v1);
+    load_k(32 * phase + STEP, k1);      // tiles beyond t_max are clamped to it, in bounds and masked
+    load_v(32 * phase + STEP, v1);
     __syncthreads();
-    for (int t0 = 0, buf = 0; t0 <= t_max; t0 += 32, buf ^= 1) {
-        const bool more = t0 + 32 <= t_max;
-        load_k(t0 + 64, k2);
-        load_v(t0 + 64, v2);
+    for (int base = 0, buf = 0; base <= t_max; base += STEP, buf ^= 1) {   // the same number of rounds for both sets
+        const int t0 = base + 32 * phase;
+        const bool more = base + STEP <= t_max;
+        load_k(t0 + 2 * STEP, k2);
+        load_v(t0 + 2 * STEP, v2);
         attn_floatx16 sc;
 #pragma unroll
         for (int r = 0; r < 16; r++) sc[r] = 0.0f;
@@ -608,13 +616,16 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
             tile_max = fmaxf(tile_max, sc[r]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
-        const float m_new = fmaxf(mx, tile_max);    // finite from the first tile on: key 0 is visible to every query
-        const float alpha = __expf(mx - m_new);      // exp(-inf) = 0 on the first tile
+        // finite from the first tile on in set 0 (key 0 is visible to every query); set 1 may see only masked keys for a while:
+        // its state then stays (-inf, 0, 0) (exponents taken against 0 instead of -inf)
+        const float m_new = fmaxf(mx, tile_max);
+        const float m_ref = (KP > 1 && m_new == -INFINITY) ? 0.0f : m_new;
+        const float alpha = __expf(mx - m_ref);      // exp(-inf) = 0 on the first tile
         float psum = 0.0f;
         _Float16 ph[16], pl[SPLIT ? 16 : 1];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const float pr = __expf(sc[r] - m_new);  // masked keys: exp(-inf) = 0
+            const float pr = __expf(sc[r] - m_ref);  // masked keys: exp(-inf) = 0
             psum += pr;
             ph[r] = (_Float16)pr;
             if constexpr (SPLIT) pl[r] = (_Float16)__fmul_rn(__fsub_rn(pr, (float)ph[r]), 2048.0f);
@@ -651,6 +662,40 @@ __global__ __launch_bounds__(G * 64) void attention_prompt_kernel(AttentionArgs 
 #pragma unroll
         for (int i = 0; i < VP; i++) v1[i] = v2[i];
         __syncthreads();
+    }
+    if constexpr (KP == 2) {
+        // set 1 hands (maximum, sum, context) to set 0 through the value tiles' LDS, 32 dims at a time: [wave][value][lane]
+        float *mb = reinterpret_cast<float *>(&vt_all[0][0][0]);
+        constexpr int kPerWave = (SPLIT ? 32 : 16) * 64, kStateBase = G * kPerWave;
+        static_assert((size_t)(kStateBase + G * 2 * 64) * 4 <= sizeof(vt_all), "the merge fits the value tiles");
+        float f0 = 1.0f, f1 = 0.0f;
+        if (phase == 1) { mb[kStateBase + (wave * 2) * 64 + lane] = mx; mb[kStateBase + (wave * 2 + 1) * 64 + lane] = l; }
+#pragma unroll
+        for (int mt = 0; mt < MTILES; mt++) {
+            if (phase == 1) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    mb[wave * kPerWave + r * 64 + lane] = o[mt][r];
+                    if constexpr (SPLIT) mb[wave * kPerWave + (16 + r) * 64 + lane] = ol[mt][r];
+                }
+            }
+            __syncthreads();
+            if (phase == 0) {
+                if (mt == 0) {
+                    const float m1 = mb[kStateBase + (wave * 2) * 64 + lane], l1 = mb[kStateBase + (wave * 2 + 1) * 64 + lane];
+                    const float m_all = fmaxf(mx, m1);   // finite: set 0 saw key 0
+                    f0 = __expf(mx - m_all); f1 = __expf(m1 - m_all);
+                    l = __builtin_fmaf(l, f0, __fmul_rn(l1, f1));
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    o[mt][r] = __builtin_fmaf(o[mt][r], f0, __fmul_rn(mb[wave * kPerWave + r * 64 + lane], f1));
+                    if constexpr (SPLIT) ol[mt][r] = __builtin_fmaf(ol[mt][r], f0, __fmul_rn(mb[wave * kPerWave + (16 + r) * 64 + lane], f1));
+                }
+            }
+            __syncthreads();
+        }
+        if (phase == 1) return;
     }
     l += __shfl_xor(l, 32);
     if constexpr (SPLIT) {
@@ -1325,29 +1370,51 @@ bool attention_prompt_supported(int n_head, int n_kv_head, int head_dim) {
 }
 
 template <int HD, int G>
-hipError_t launch_attention_prompt_shape(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
+hipError_t launch_attention_prompt_shape(const AttentionArgs &a, int rows, bool kv_f16, int key_sets, hipStream_t s) {
     dim3 grid(a.n_kv_head, (rows + 31) / 32);
+    // Two sets of wavefronts per workgroup (alternate key tiles) for 128-dim heads: the workgroup keeps its size (the kernel needs more
+    // than 256 registers, one wavefront per SIMD), so half of the KV head's query heads go to a second workgroup (grid z).
+    constexpr bool kTwoSets = HD == 128;
+    constexpr int GS = G >= 2 ? G / 2 : 1;
+    dim3 grid2(a.n_kv_head, (rows + 31) / 32, G / GS);
     if (a.ctx_hi) {   // split rows out: fp16 caches only (they hold keys and values exactly)
         if (!kv_f16 || !a.ctx_lo || !a.ctx_sums || (a.n_head * HD) % 256 != 0) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((attention_prompt_kernel<HD, G, true, true>), grid, dim3(G * 64), 0, s, a, rows);
+        if constexpr (kTwoSets) {
+            if (key_sets == 2) {
+                hipLaunchKernelGGL((attention_prompt_kernel<HD, GS, true, true, 2>), grid2, dim3(GS * 128), 0, s, a, rows);
+                return hipGetLastError();
+            }
+        }
+        hipLaunchKernelGGL((attention_prompt_kernel<HD, G, true, true, 1>), grid, dim3(G * 64), 0, s, a, rows);
         return hipGetLastError();
     }
-    if (kv_f16) hipLaunchKernelGGL((attention_prompt_kernel<HD, G, true, false>), grid, dim3(G * 64), 0, s, a, rows);
-    else hipLaunchKernelGGL((attention_prompt_kernel<HD, G, false, false>), grid, dim3(G * 64), 0, s, a, rows);
+    if constexpr (kTwoSets) {
+        if (key_sets == 2 && kv_f16) {
+            hipLaunchKernelGGL((attention_prompt_kernel<HD, GS, true, false, 2>), grid2, dim3(GS * 128), 0, s, a, rows);
+            return hipGetLastError();
+        }
+    }
+    if (kv_f16) hipLaunchKernelGGL((attention_prompt_kernel<HD, G, true, false, 1>), grid, dim3(G * 64), 0, s, a, rows);
+    else hipLaunchKernelGGL((attention_prompt_kernel<HD, G, false, false, 1>), grid, dim3(G * 64), 0, s, a, rows);
     return hipGetLastError();
 }
+
+// 0 (default): two sets of wavefronts for blocks of more than 64 rows; 1 / 2: always that many (tests, measurements)
+static int g_prompt_attention_key_sets = 0;
+void attention_prompt_set_key_sets(int sets) { g_prompt_attention_key_sets = sets == 1 || sets == 2 ? sets : 0; }
 
 hipError_t launch_attention_prompt(const AttentionArgs &a, int rows, bool kv_f16, hipStream_t s) {
     if (rows <= 0 || !attention_prompt_supported(a.n_head, a.n_kv_head, a.head_dim)) return hipErrorInvalidValue;
     const int group = a.n_head / a.n_kv_head;
+    const int sets = g_prompt_attention_key_sets ? g_prompt_attention_key_sets : (rows > 64 ? 2 : 1);
     if (a.head_dim == 128) {
-        if (group == 1) return launch_attention_prompt_shape<128, 1>(a, rows, kv_f16, s);
-        if (group == 2) return launch_attention_prompt_shape<128, 2>(a, rows, kv_f16, s);
-        return launch_attention_prompt_shape<128, 4>(a, rows, kv_f16, s);
+        if (group == 1) return launch_attention_prompt_shape<128, 1>(a, rows, kv_f16, sets, s);
+        if (group == 2) return launch_attention_prompt_shape<128, 2>(a, rows, kv_f16, sets, s);
+        return launch_attention_prompt_shape<128, 4>(a, rows, kv_f16, sets, s);
     }
-    if (group == 1) return launch_attention_prompt_shape<64, 1>(a, rows, kv_f16, s);
-    if (group == 2) return launch_attention_prompt_shape<64, 2>(a, rows, kv_f16, s);
-    return launch_attention_prompt_shape<64, 4>(a, rows, kv_f16, s);
+    if (group == 1) return launch_attention_prompt_shape<64, 1>(a, rows, kv_f16, sets, s);
+    if (group == 2) return launch_attention_prompt_shape<64, 2>(a, rows, kv_f16, sets, s);
+    return launch_attention_prompt_shape<64, 4>(a, rows, kv_f16, sets, s);
 }
 
 int attention_head_splits(int) { return kAttentionHeadSplits; }

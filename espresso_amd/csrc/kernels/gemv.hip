@@ -2552,6 +2552,7 @@ bool gemv_set_tuning(const char *key, int value) {
     if (k == "q4k_long_row_waves") { g_q4k_long_row_waves = value; return true; }
     if (k == "q4k_wide") { g_q4k_wide_mode = value; return true; }
     if (k == "split_gemm_shared_k") { gemm_split_set_shared_k(value); return true; }
+    if (k == "prompt_attention_key_sets") { attention_prompt_set_key_sets(value); return true; }
     return false;
 }
 

@@ -247,19 +247,31 @@ def test_matrix_prefill_matches_oracle_and_per_token_path(llama, fmt, count, kv_
         assert np.abs(o.logits() - g.logits()).max() <= LOGIT_TOL
 
 
-@pytest.mark.parametrize("heads,kv_heads,head_dim,kv_fp16,count", [
-    (2, 2, 128, True, 75), (4, 1, 128, False, 530), (4, 1, 128, True, 97), (4, 2, 128, False, 40), (4, 4, 64, False, 64),
-    (4, 1, 64, True, 33),
+@pytest.mark.parametrize("heads,kv_heads,head_dim,kv_fp16,count,fmt,key_sets", [
+    (2, 2, 128, True, 75, orc.FMT_Q8_0, 0), (4, 1, 128, False, 530, orc.FMT_Q8_0, 0), (4, 1, 128, True, 97, orc.FMT_Q8_0, 0),
+    (4, 2, 128, False, 40, orc.FMT_Q8_0, 0), (4, 4, 64, False, 64, orc.FMT_Q8_0, 0), (4, 1, 64, True, 33, orc.FMT_Q8_0, 0),
+    # both forms of the 128-dim kernel forced: one set of wavefronts per workgroup, and two sets on alternate key tiles (four, two and one
+    # query heads per KV head; a block whose second set sees only masked keys in its first tiles; Q4_K = queries and probabilities as pairs)
+    (4, 1, 128, True, 200, orc.FMT_Q8_0, 1), (4, 1, 128, True, 200, orc.FMT_Q8_0, 2), (4, 2, 128, True, 33, orc.FMT_Q8_0, 2),
+    (2, 2, 128, True, 130, orc.FMT_Q8_0, 2), (8, 2, 128, True, 300, orc.FMT_Q4_K, 1), (8, 2, 128, True, 300, orc.FMT_Q4_K, 2),
+    (8, 4, 128, True, 70, orc.FMT_Q4_K, 2), (8, 8, 128, True, 530, orc.FMT_Q4_K, 0),
 ])
-def test_prompt_block_attention_on_the_matrix_cores(llama, heads, kv_heads, head_dim, kv_fp16, count):
+def test_prompt_block_attention_on_the_matrix_cores(llama, heads, kv_heads, head_dim, kv_fp16, count, fmt, key_sets):
     """Prompt blocks run causal attention as MFMA tiles (32 rows x 32 keys) for head sizes 64 / 128 and 1, 2 or 4 query
     heads per KV head: ragged last tiles, a prompt longer than one 512-row block, both cache types.  The state it leaves
     agrees with the oracle's token-by-token walk and with the per-token GPU path."""
+    import espresso_amd.ops as ops
     cfg = dict(TINY, n_head=heads, n_kv_head=kv_heads, head_dim=head_dim, max_seq=count + 8, vocab=512)
-    o, g = make_pair(llama, cfg, orc.FMT_Q8_0, seed=900 + count, std=0.08, kv_fp16=kv_fp16, norm_jitter=0.05)
+    if fmt == orc.FMT_Q4_K:   # a width at which Q4_K runs on split pairs, the prompt attention included
+        cfg.update(d_model=1024, hidden_dim=1024)
+    o, g = make_pair(llama, cfg, fmt, seed=900 + count, std=0.08 if fmt != orc.FMT_Q4_K else 0.04, kv_fp16=kv_fp16, norm_jitter=0.05)
     prompt = np.random.default_rng(count).integers(0, 512, count).tolist()
     o.prefill(prompt)
-    g.prefill(prompt)
+    ops.set_tuning("prompt_attention_key_sets", key_sets)
+    try:
+        g.prefill(prompt)
+    finally:
+        ops.set_tuning("prompt_attention_key_sets", 0)
     ho, hg = o.last_hidden(), g.last_hidden()
     scale = max(1.0, np.abs(ho).max())
     assert np.abs(ho - hg).max() <= 4e-3 * scale, np.abs(ho - hg).max()
