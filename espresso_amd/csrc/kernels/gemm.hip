@@ -319,8 +319,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs a) {
                     const int r = 2 * k + (odd ? 1 : 0);
                     const int m = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                     if (m < a.M && (n | 1) < a.N) {
-                        const float hg = __fmul_rn(0.5f, g);
-                        const float silu = __fmul_rn(hg, __fadd_rn(1.0f, tanhf(hg)));
+                        const float silu = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g));   // = 0.5 g (1 + tanh(0.5 g)), a fifth of tanhf's instructions
                         a.swiglu_out[(size_t)m * (a.N / 2) + n / 2] = __builtin_bit_cast(uint16_t, (_Float16)__fmul_rn(silu, u));
                     }
                 }

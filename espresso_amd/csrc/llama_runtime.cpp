@@ -427,7 +427,10 @@ int LlamaRuntime::finalize() {
         if ((rc = device_alloc(&attn_scratch_, R * per_row)) != ESP_OK) return rc;
     }
     if ((rc = device_alloc(&gemm_workspace_, kGemmWorkspaceFloats)) != ESP_OK) return rc;
-    ESP_HIP_TRY(gemm_split_shared_k_pool(&gemm_shared_k_));
+    if (gemm_split_shared_k_pool(&gemm_shared_k_) != hipSuccess) {   // without the pool the prompt GEMM keeps its plain grid
+        (void)hipGetLastError();
+        gemm_shared_k_ = GemmSplitSharedK{};
+    }
     {
         const char *pa = getenv("ESPRESSO_HIP_PROMPT_ATTENTION");   // "0": prompt blocks keep the single-query attention kernel
         prompt_attention_ = attention_prompt_supported(c_.n_head, c_.n_kv_head, c_.head_dim) && !(pa && pa[0] == '0');
