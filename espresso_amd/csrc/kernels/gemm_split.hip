@@ -735,8 +735,8 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
     // accumulator r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of the 32 x 32 tile
     if (a.sw_hi) {
         // SiLU(gate) * up of the workgroup's 128 x 128 units as the two fp16 planes, through LDS (free now) so that the planes leave
-        // in whole 16-byte pieces of a row: [plane][128 rows][kActLd].  SiLU as g / (1 + exp(-g)): the same function as the
-        // 0.5 g (1 + tanh(0.5 g)) of the single-row kernels, a fifth of the instructions (this epilogue measured 10 us per
+        // in whole 16-byte pieces of a row: [plane][128 rows][kActLd].  SiLU as g / (1 + exp(-g)) (the form of Sources/CPUOps/SiLU.swift:5-8):
+        // the same function as the 0.5 g (1 + tanh(0.5 g)) of RealModelInferenceEngine.swift:6825-6827 that the single-row kernels keep, a fifth of the instructions (this epilogue measured 10 us per
         // output tile with tanhf and two-byte stores, a fifteenth of the tile's time).
         constexpr int kActLd = 144;   // halfs per staged row: consecutive rows eight LDS banks apart
         uint16_t *act_hi = reinterpret_cast<uint16_t *>(smem_raw), *act_lo = act_hi + 128 * kActLd;
