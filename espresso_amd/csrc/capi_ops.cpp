@@ -251,9 +251,22 @@ int esp_matmul_f32_swiglu(const ESPMatrix *matrix, const float *x, int rows, flo
     }
     if (e == hipSuccess) e = hipMemcpyAsync(hi.data(), out.hi, na * 2, hipMemcpyDeviceToHost, c.stream);
     if (e == hipSuccess) e = hipMemcpyAsync(lo.data(), out.lo, na * 2, hipMemcpyDeviceToHost, c.stream);
+    std::vector<uint16_t> sums(na / 16);
+    if (e == hipSuccess) e = hipMemcpyAsync(sums.data(), out.sums, sums.size() * 2, hipMemcpyDeviceToHost, c.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
     release();
     if (e != hipSuccess) return fail_hip(e, "matmul_f32_swiglu");
+    // the sub-block sums that accompany the planes ([row][super-block][hi of S_0..7, lo of S_0..7]) must be the planes' own, to rounding
+    // (checked where the units fill whole super-blocks of the next matrix, as a model's do)
+    for (int r = 0; r < rows && units % 256 == 0; r++)
+        for (size_t sub = 0; sub < units / 32; sub++) {
+            double want = 0.0;
+            for (size_t k = 0; k < 32; k++) want += (double)half_to_float(hi[(size_t)r * units + 32 * sub + k]) + (double)half_to_float(lo[(size_t)r * units + 32 * sub + k]) / 2048.0;
+            const uint16_t *p = sums.data() + ((size_t)r * (units / 256) + (sub >> 3)) * 16 + (sub & 7);
+            const double got = (double)half_to_float(p[0]) + (double)half_to_float(p[8]) / 2048.0;
+            if (std::fabs(got - want) > 1e-5 * (1.0 + std::fabs(want)))
+                return fail(ESP_ERR_LAUNCH_FAILED, "matmul_f32_swiglu: sub-block sum of row %d, sub-block %zu is %.9g, the planes give %.9g", r, sub, got, want);
+        }
     // the planes keep the units of every four in the order (0, 2, 1, 3)
     for (int r = 0; r < rows; r++)
         for (size_t u = 0; u < units; u++) {

@@ -52,15 +52,17 @@ struct SplitGemmArgs {
     float *partial;                 // [splits][M][N] when gridDim.y > 1
     int tiles_per_split;            // a multiple of four
     uint16_t *sw_hi, *sw_lo;        // SiLU(gate) * up as a split pair [M][N / 2] instead of y (no split-K)
+    uint16_t *sw_sums;              // optional (gemm_q4k_split_regb_kernel, N / 2 a multiple of 32): the pair's sub-block sums, else split_sums_kernel follows
     const uint8_t *tiled;           // the matrix-core GEMV's tiled copy (gemm_q4k_split_regb_kernel reads its weights there)
     // shared K ranges (gemm_q4k_split_regb_kernel<.., true>): workgroup i owns K tiles [i * sk_units, (i + 1) * sk_units) of the
     // sequence (output tile 0: K tiles 0 .. K / 64 - 1, output tile 1: ...), output tile t = (t % sk_tiles_n, t / sk_tiles_n)
     int sk_units, sk_tiles_n;
-    unsigned *sk_flags;             // [kStreamKFlags]: one word per workgroup + the launch counter, zero before the first launch
+    unsigned *sk_flags;             // [kStreamKFlags]: one word per workgroup, zero between launches
     unsigned sk_spin_limit;
     float *sk_partial;              // [workgroups][128 accumulators][256 threads]
 };
-constexpr int kStreamKFlags = 1024, kStreamKEpochSlot = kStreamKFlags - 1, kStreamKMaxWorkgroups = 256;
+constexpr int kStreamKFlags = 1024, kStreamKMaxWorkgroups = 256;
+constexpr unsigned kStreamKReady = 1, kStreamKCancelled = 2;   // a flag word's states besides 0
 constexpr unsigned kStreamKSpinLimit = 1u << 22;   // polls of the finisher (each at least a trip to memory) before it computes the rest itself
 
 __device__ __forceinline__ h2 as_h2(u32 v) { return __builtin_bit_cast(h2, v); }
@@ -407,6 +409,7 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_kernel(SplitGemmArgs 
 // is the vector work per MFMA: with every wavefront on all 128 rows and 64 weight rows (RB x CB = 4 x 2) a B fragment serves eight
 // MFMAs instead of four: gate|up of a 512-row block 356 -> 324 us (the kernel above: 421 on the same boxes).  The activation tiles
 // rotate through four LDS buffers so that one barrier serves two tiles (318 -> 313 us, old and new alternating on one box).
+__device__ __forceinline__ void store_subblock_sum(uint16_t *sums, size_t row, int cols, int group, float s);
 constexpr int NT2 = 256;
 constexpr int kRegBBufs = 4;   // activation tiles in LDS: with four, one barrier serves two tiles
 constexpr size_t kLdsBytesRegB = 2 * kRegBBufs * kTileHalfs * 2 + 2 * 128 * 16 * 2;
@@ -421,8 +424,9 @@ constexpr size_t kLdsBytesRegB = 2 * kRegBBufs * kTileHalfs * 2 + 2 * 128 * 16 *
 // totals per lane in `sk_partial` and then writes the launch's number into its flag word; the finisher adds them and runs the
 // epilogue.  The successor's piece is the first thing it does and waits for nothing, so whatever the order in which workgroups
 // become resident the finisher's wait ends; it is bounded all the same (sk_spin_limit polls), and a finisher whose wait runs out
-// computes the rest of the tile itself.  The launch number lives in device memory (the kernel that follows every such launch
-// increments it), so a captured launch replays correctly and a flag of an earlier launch is never taken for this one's.
+// computes the rest of the tile itself.  A flag word is 0 between launches: the successor moves it 0 -> ready, the finisher back to 0 once
+// it has the totals; a finisher that gives up moves it 0 -> cancelled and the successor, finding that, back to 0 (both by compare-and-swap,
+// so whichever comes first the word ends at 0 and the totals are taken at most once): a replay under a captured graph starts clean.
 // `sk_partial` and `sk_flags` are uncached device memory: with ordinary memory the hand-over needs a release that writes the die's
 // L2 back (10 us per workgroup, measured) and an acquire that invalidates the finisher's.
 // Measured on gate|up of a 512-row block, workgroup by workgroup (wall-clock stamps): 2.2 us per K tile, 4.7 us per epilogue, 3.7 us to
@@ -441,7 +445,6 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
     floatx16 tot[RB][CB], acc[RB][CB];   // acc starts every super-block from the zero C operand of its first MFMAs
     int sk_unit = SK ? (int)blockIdx.x * a.sk_units : 0;
     const int sk_unit_end = sk_unit + a.sk_units;
-    const unsigned sk_launch = SK ? a.sk_flags[kStreamKEpochSlot] + 1u : 0u;
     int sk_resume_from = 0;   // > 0: the previous pass ended at this K tile of the same output tile and the totals stay
   for (;;) {   // one pass per piece of an output tile with SK, a single pass otherwise (the body keeps a function body's indentation)
     // The thread's coordinates are formed anew for every output tile piece: taken from outside the loop, every LDS and row offset
@@ -693,17 +696,29 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
                         slot[(size_t)((i * CB + j) * 4 + q) * THREADS] = make_float4(tot[i][j][4 * q], tot[i][j][4 * q + 1], tot[i][j][4 * q + 2], tot[i][j][4 * q + 3]);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // every store of this wavefront acknowledged
             __syncthreads();
-            if (tid == 0) __hip_atomic_store(a.sk_flags + blockIdx.x, sk_launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tid == 0) {   // 0 -> ready; a finisher that gave up left "cancelled": nobody will take the totals, back to 0
+                unsigned expected = 0;
+                if (!__hip_atomic_compare_exchange_strong(a.sk_flags + blockIdx.x, &expected, kStreamKReady, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                    __hip_atomic_store(a.sk_flags + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             if (sk_unit >= sk_unit_end) return;
             continue;
         }
         if (t_end < tiles) {
             // this workgroup began the output tile: the next one has (or will have) the rest
             if (tid == 0) {
+                unsigned *flag = a.sk_flags + blockIdx.x + 1;
                 int seen = 0;
                 for (unsigned polls = 0; polls < a.sk_spin_limit; polls++) {
-                    if (__hip_atomic_load(a.sk_flags + blockIdx.x + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == sk_launch) { seen = 1; break; }
+                    if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == kStreamKReady) { seen = 1; break; }
                     __builtin_amdgcn_s_sleep(8);
+                }
+                if (!seen && a.sk_spin_limit != 0) {   // give up: 0 -> cancelled, unless the successor got there first
+                    unsigned expected = 0;
+                    if (!__hip_atomic_compare_exchange_strong(flag, &expected, kStreamKCancelled, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) seen = 1;
+                } else if (!seen) {                    // no polls at all (tests): never take the totals, even if they are there
+                    if (__hip_atomic_exchange(flag, kStreamKCancelled, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == kStreamKReady)
+                        __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
                 sk_flag_seen = seen;
             }
@@ -730,6 +745,8 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
                 for (int j = 0; j < CB; j++)
 #pragma unroll
                     for (int r = 0; r < 16; r++) tot[i][j][r] += acc[i][j][r];
+            __syncthreads();   // every wavefront has its share of the totals
+            if (tid == 0) __hip_atomic_store(a.sk_flags + blockIdx.x + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     // accumulator r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of the 32 x 32 tile
@@ -772,8 +789,18 @@ __global__ __launch_bounds__(kThreads) void gemm_q4k_split_regb_kernel(SplitGemm
             if (m >= a.M || unit0 + c8 >= units_n) continue;
             const size_t o = (size_t)m * units_n + unit0 + c8;
             if (whole_pieces) {   // units_n and unit0 + c8 are multiples of eight: the piece is whole and 16-byte aligned
-                *reinterpret_cast<uint4 *>(a.sw_hi + o) = *reinterpret_cast<const uint4 *>(act_hi + row * kActLd + c8);
-                *reinterpret_cast<uint4 *>(a.sw_lo + o) = *reinterpret_cast<const uint4 *>(act_lo + row * kActLd + c8);
+                const uint4 h = *reinterpret_cast<const uint4 *>(act_hi + row * kActLd + c8), l = *reinterpret_cast<const uint4 *>(act_lo + row * kActLd + c8);
+                *reinterpret_cast<uint4 *>(a.sw_hi + o) = h;
+                *reinterpret_cast<uint4 *>(a.sw_lo + o) = l;
+                if (a.sw_sums) {   // the sums split_sums_kernel would form, in its order; four consecutive lanes hold one sub-block of a row
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int pp = 0; pp < 4; pp++) {
+                        const h2 hp = as_h2(dword_of(h, pp)), lp = as_h2(dword_of(l, pp));
+                        sum += __builtin_fmaf((float)lp.x, kUnscale, (float)hp.x) + __builtin_fmaf((float)lp.y, kUnscale, (float)hp.y);
+                    }
+                    store_subblock_sum(a.sw_sums, (size_t)m, units_n, (unit0 + c8) >> 3, sum);
+                }
             } else {
                 for (int e = 0; e < 8 && unit0 + c8 + e < units_n; e++) {
                     a.sw_hi[o + e] = act_hi[row * kActLd + c8 + e];
@@ -937,9 +964,8 @@ __global__ __launch_bounds__(256) void split_rows_kernel(SplitRowsArgs a) {
 }
 
 // sums of rows that exist as hi / lo planes already (the SiLU(gate) * up epilogue writes those)
-__global__ __launch_bounds__(256) void split_sums_kernel(const uint16_t *hi, const uint16_t *lo, int cols, uint16_t *sums, unsigned *launch_counter) {
+__global__ __launch_bounds__(256) void split_sums_kernel(const uint16_t *hi, const uint16_t *lo, int cols, uint16_t *sums) {
     const int m = blockIdx.x;
-    if (launch_counter && m == 0 && threadIdx.x == 0) *launch_counter += 1u;   // the GEMM before this kernel shared K ranges under this number
     const size_t row = (size_t)m * cols;
     for (int g = threadIdx.x; g < cols / 8; g += 256) {
         const uint4 h = reinterpret_cast<const uint4 *>(hi + row)[g], l = reinterpret_cast<const uint4 *>(lo + row)[g];
@@ -1020,7 +1046,7 @@ hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream) {
     }
     a.tiles_per_split = ((tiles + splits - 1) / splits + 3) & ~3;
     splits = (tiles + a.tiles_per_split - 1) / a.tiles_per_split;
-    if (swiglu) { a.sw_hi = p.swiglu.hi; a.sw_lo = p.swiglu.lo; }
+    if (swiglu) { a.sw_hi = p.swiglu.hi; a.sw_lo = p.swiglu.lo; a.sw_sums = regb && (a.N / 2) % 32 == 0 ? p.swiglu.sums : nullptr; }
     static std::atomic<uint64_t> raised{0};
     int device = 0;
     hipError_t e = hipGetDevice(&device);
@@ -1067,8 +1093,8 @@ hipError_t launch_gemm_split(const GemmSplitParams &p, hipStream_t stream) {
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (swiglu) {
-        hipLaunchKernelGGL(split_sums_kernel, dim3(a.M), dim3(256), 0, stream, p.swiglu.hi, p.swiglu.lo, a.N / 2, p.swiglu.sums,
-                           shared_k_workgroups ? a.sk_flags + kStreamKEpochSlot : nullptr);
+        if (a.sw_sums) return hipSuccess;   // the GEMM's epilogue wrote the sums
+        hipLaunchKernelGGL(split_sums_kernel, dim3(a.M), dim3(256), 0, stream, p.swiglu.hi, p.swiglu.lo, a.N / 2, p.swiglu.sums);
         return hipGetLastError();
     }
     if (splits > 1) {

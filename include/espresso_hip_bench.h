@@ -51,7 +51,8 @@ long long esp_matrix_read_tiled(const ESPMatrix *matrix, void *out, size_t capac
 /* Test aid: the exact Q4_K product of esp_matmul_f32 with the epilogue the feed-forward block uses.  The matrix holds gate and up rows
  * interleaved (row 2i = gate_i, 2i + 1 = up_i; `matrix rows` a multiple of 8); act[r][i] = SiLU(x[r] . gate_i) * (x[r] . up_i) as the pair of
  * fp16 planes the kernel writes, added back together (hi + lo / 2048), fp32 [rows][matrix rows / 2]; host pointers.  The launch is made
- * twice on the same flag words, so the second one runs under the next launch number; tuning key split_gemm_shared_k selects how
+ * twice on the same flag words; the sub-block sums the kernel writes beside the planes are checked against the planes on the host
+ * (a mismatch fails the call); tuning key split_gemm_shared_k selects how
  * workgroups share an output tile's K range (0 never, 1 where it applies, 2 as 1 with the finishing workgroup never waiting). */
 int esp_matmul_f32_swiglu(const ESPMatrix *matrix, const float *x, int rows, float *act);
 int esp_hbm_read_probe(size_t bytes, int iters, double *gb_per_s);
